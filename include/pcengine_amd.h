@@ -1,0 +1,170 @@
+/* pcengine_amd — C ABI of the MI355X (gfx950) sparse-convolution hot path.
+ *
+ * Plain pointers and sizes only; every pointer named "device" is HIP device memory owned by the
+ * caller.  The library keeps no state between calls, allocates no device memory, and launches all
+ * work on the stream it is given.  Functions return PCE_OK (0) or an error code; the text of the
+ * last error on the calling thread is returned by pce_last_error().
+ *
+ * These entry points are what the reference's five pybind functions
+ * (backend/pybind_cuda.cpp:8-14) decompose into:
+ *
+ *   mapping_d2_cuda  = HashMapD2  (backend/hash.h:37-58,  backend/hash.cu:258-435)
+ *       -> pce_outcoords_build/_emit (strided only) + pce_kmap_build
+ *   mapping_d1_cuda  = HashMapD1  (backend/hash.h:11-34,  backend/hash.cu:20-255)
+ *       -> the same, with the CSR outputs of pce_kmap_build requested
+ *   conv_fwd_d2_cuda = ConvolutionForwardD2 (backend/spconv.h:28-40, backend/spconv.cu:224-398)
+ *       -> pce_conv_fwd_fod
+ *   conv_fwd_d1_cuda = ConvolutionForwardD1 (backend/spconv.h:11-25, backend/spconv.cu:24-222)
+ *       -> pce_conv_fwd_gms
+ *   conv_bwd_d1_cuda = ConvolutionBackwardD1 (backend/spconv.h:43-58): training, not provided.
+ */
+#ifndef PCENGINE_AMD_H
+#define PCENGINE_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *pce_stream_t; /* hipStream_t */
+
+enum {
+  PCE_OK = 0,
+  PCE_EINVAL = 1,     /* bad argument (shape mismatch, null pointer, unsupported size) */
+  PCE_ECAPACITY = 2,  /* a documented capacity limit would be exceeded */
+  PCE_EHIP = 3,       /* a HIP runtime call or kernel launch failed */
+  PCE_EWORKSPACE = 4, /* workspace too small */
+  PCE_ECOORD = 5      /* a coordinate is outside the representable range */
+};
+
+enum { PCE_F16 = 0, PCE_F32 = 1 };
+
+/* dataflows of the forward convolution */
+enum {
+  PCE_DATAFLOW_FOD = 0, /* fetch-on-demand fused gather-matmul-scatter (reference "D2") */
+  PCE_DATAFLOW_GMS = 1, /* gather - grouped GEMM - scatter over a staging buffer (reference "D1") */
+  PCE_DATAFLOW_OS = 2   /* output-stationary fetch-on-demand: no atomics, no staging buffer */
+};
+
+#define PCE_QUANTUM 128        /* rows per tile of the pair list; qkpos granularity (backend/hash.cu:203-205) */
+#define PCE_CSR_CODE 1186111   /* CSR entry code = kp * PCE_CSR_CODE + rank (backend/hash.cuh:7-9) */
+#define PCE_COORD_BOUND 3259   /* spatial coordinates of a strided conv's output must be < this (backend/hash.cuh:503) */
+#define PCE_COORD_LIMIT 32000  /* |coordinate| limit of the packed 64-bit hash key */
+
+/* Geometry of one convolution; what the reference passes as four packed codes plus bounds
+ * (backend/hash.cu:57-76, script/spconv.py:354-367). */
+typedef struct pce_geom {
+  int32_t ks[3];      /* kernel size */
+  int32_t stride[3];  /* layer stride */
+  int32_t pad[3];     /* padding */
+  int32_t cmin[3];    /* lower bound of output coordinates */
+  int32_t cmax[3];    /* upper bound of output coordinates, already reduced for strided layers */
+  int32_t subm;       /* 1: submanifold (out coords = in coords, centre offset handled densely) */
+} pce_geom_t;
+
+int pce_version(void);
+const char *pce_last_error(void);
+
+/* ---- coordinate hash table: open addressing on the packed (b,x,y,z) 64-bit key ------------- */
+
+/* Slot count for n keys: 2 * 2^ceil(log2 n), the reference's load factor (backend/hash.cu:46). */
+int64_t pce_hash_slots(int64_t n);
+/* Bytes of a table with that many slots (16 bytes per slot: key + row). */
+int64_t pce_hash_table_bytes(int64_t n);
+/* Insert rows 0..n-1 of coords[n,4] (replaces insertHash + insertVal, backend/hash.cuh:55-91).
+ * status (device int32[2]) receives [0] = 1 if a coordinate was out of range,
+ * [1] = 1 if probing exhausted the table; the caller zeroes it first. */
+int pce_hash_build(void *table_dev, int64_t slots, const int32_t *coords_dev, int64_t n,
+                   int32_t *status_dev, pce_stream_t stream);
+/* rows_dev[q] = row of qcoords[q] in the table, or -1 (probe loop of backend/hash.cuh:154-161). */
+int pce_hash_query(const void *table_dev, int64_t slots, const int32_t *qcoords_dev, int64_t nq,
+                   int32_t *rows_dev, pce_stream_t stream);
+
+/* ---- output coordinates of a strided convolution -------------------------------------------- *
+ * Replaces coordsDownsampleExpand + remove + sort + unique + coordsGenerator
+ * (backend/hash.cuh:535-641, backend/hash.cu:141-173).  Always the generic rule; the reference's
+ * stride==kernel shortcut is not reproduced because it disagrees with its own query kernels. */
+int64_t pce_outcoords_workspace_bytes(int64_t n_in, const pce_geom_t *g);
+/* Builds the sorted unique output codes inside the workspace and returns their number in
+ * *n_out_host.  Synchronises the stream once (the count has to reach the host). */
+int pce_outcoords_build(const int32_t *in_coords_dev, int64_t n_in, const pce_geom_t *g,
+                        void *ws_dev, int64_t ws_bytes, int64_t *n_out_host, pce_stream_t stream);
+/* Decodes them into out_coords_dev[n_out,4] (same workspace, untouched since _build). */
+int pce_outcoords_emit(const void *ws_dev, int64_t n_in, const pce_geom_t *g, int64_t n_out,
+                       int32_t *out_coords_dev, pce_stream_t stream);
+
+/* ---- kernel map ------------------------------------------------------------------------------ *
+ * Replaces the four _queryhash_* kernels, exclusive_scan_for_kernel_quantified, mapping_counter and
+ * the thrust remove/scan calls (backend/hash.cuh:97-497, backend/hash.cu:180-243) and the
+ * nonzero-compaction done in Python (script/spconv.py:370-372).
+ *
+ * Outputs (device, caller-allocated; nothing needs pre-initialising):
+ *   imap, omap   int32[kv*n_in] capacity; the first M = kpos[kv] entries are the (input row,
+ *                output row) pairs ordered by (offset, input row)
+ *   knnz[kv], kpos[kv+1], qkpos[kv+1]
+ *   optional (pass NULL to skip), all four or none:
+ *     icsr[n_in+1], icode[kv*n_in cap], ocsr[n_out+1], ocode[kv*n_in cap]: CSR-coded map,
+ *     entry = kp*PCE_CSR_CODE + rank, ascending kp inside a row, rank = position inside the offset
+ *   optional nbr_out int32[kv*n_out]: output-major table nbr[kp*n_out + o] = input row or -1
+ *     (centre offset of a submanifold layer = the row itself)
+ *   optional nbr_in int32[kv*n_in]: input-major table nbr[kp*n_in + i] = output row or -1, the
+ *     layout of the reference's dense fetch-on-demand map (backend/hash.cuh:331,417); it is the
+ *     output-major table of the transposed layer
+ *   status int32[4]: [0] coordinate out of range, [1] table exhausted, [2] an offset holds
+ *     >= PCE_CSR_CODE pairs (CSR code would overflow).  Caller zeroes it; read it after a sync. */
+int64_t pce_kmap_workspace_bytes(int64_t n_in, int64_t n_out, int32_t kv, int32_t want_csr);
+int pce_kmap_build(const int32_t *in_coords_dev, int64_t n_in, const int32_t *out_coords_dev,
+                   int64_t n_out, const pce_geom_t *g, void *ws_dev, int64_t ws_bytes,
+                   int32_t *imap_dev, int32_t *omap_dev, int32_t *knnz_dev, int32_t *kpos_dev,
+                   int32_t *qkpos_dev, int32_t *icsr_dev, int32_t *icode_dev, int32_t *ocsr_dev,
+                   int32_t *ocode_dev, int32_t *nbr_out_dev, int32_t *nbr_in_dev,
+                   int32_t *status_dev, pce_stream_t stream);
+
+/* ---- forward convolution --------------------------------------------------------------------- *
+ * Common arguments: in_feats[n_in,c_in], weight[kv,c_in,c_out], out_feats[n_out,c_out], all of
+ * `dtype` (PCE_F16: fp16 storage, fp32 accumulate; PCE_F32), row-major, device.
+ * mid >= 0 selects the submanifold centre offset handled as a dense GEMM over identical rows
+ * (requires n_in == n_out); mid < 0 for strided / transposed layers.
+ * For a transposed layer pass the map with the roles swapped (imap<->omap, icsr<->ocsr), as the
+ * reference front end does (script/spconv.py:142-151, 236-244). */
+
+/* Fetch-on-demand: pairs (imap, omap, kpos, qkpos) and qsum = qkpos[kv] on the host.
+ * fp16 needs an fp32 accumulation scratch of pce_conv_fod_workspace_bytes(); fp32 needs none. */
+int64_t pce_conv_fod_workspace_bytes(int64_t n_out, int32_t c_out, int32_t dtype);
+int pce_conv_fwd_fod(const void *in_feats, const void *weight, void *out_feats, int32_t dtype,
+                     int64_t n_in, int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv,
+                     int32_t mid, const int32_t *imap_dev, const int32_t *omap_dev,
+                     const int32_t *kpos_dev, const int32_t *qkpos_dev, int64_t qsum,
+                     void *ws_dev, int64_t ws_bytes, pce_stream_t stream);
+
+/* Gather - GEMM - scatter: CSR-coded map; `buffer` holds qsum*(c_in+c_out) elements of dtype
+ * (first qsum*c_in gathered inputs, then the GEMM outputs; backend/spconv.cu:121). */
+int pce_conv_fwd_gms(const void *in_feats, const void *weight, void *out_feats, int32_t dtype,
+                     int64_t n_in, int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv,
+                     int32_t mid, const int32_t *icsr_dev, const int32_t *icode_dev,
+                     const int32_t *ocsr_dev, const int32_t *ocode_dev, const int32_t *kpos_dev,
+                     const int32_t *qkpos_dev, int64_t qsum, void *buffer_dev,
+                     int64_t buffer_elems, pce_stream_t stream);
+
+/* Output-stationary: nbr[kv*n_out] from pce_kmap_build (for a transposed layer, a table built
+ * with the roles swapped).  One kernel, one store per output row.  No counterpart in the
+ * reference: it is the same fetch-on-demand computation with the scatter-add replaced by
+ * register accumulation. */
+int pce_conv_fwd_os(const void *in_feats, const void *weight, void *out_feats, int32_t dtype,
+                    int64_t n_in, int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv,
+                    const int32_t *nbr_dev, pce_stream_t stream);
+
+/* out[n,c_out] = in[n,c_in] * weight[c_in,c_out]: the 1x1 stride-1 shortcut of the front end
+ * (script/spconv.py:297-304), on the same MFMA tile kernel. */
+int pce_conv_fwd_dense(const void *in_feats, const void *weight, void *out_feats, int32_t dtype,
+                       int64_t n, int32_t c_in, int32_t c_out, pce_stream_t stream);
+
+/* Per-layer dataflow choice from map density (pairs per output row) and channel widths. */
+int pce_select_dataflow(int64_t n_in, int64_t n_out, int64_t n_pairs, int32_t c_in, int32_t c_out,
+                        int32_t kv, int32_t dtype);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PCENGINE_AMD_H */

@@ -1,0 +1,98 @@
+"""ctypes binding of libpcengine_amd.so (the C ABI declared in include/pcengine_amd.h).
+
+The library is the only compute path: if it is missing, loading raises and every operator of
+the package fails with that error.  There is no CPU fallback.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_int32, c_int64, c_void_p, c_char_p, POINTER, Structure
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libpcengine_amd.so")
+
+PCE_OK, PCE_EINVAL, PCE_ECAPACITY, PCE_EHIP, PCE_EWORKSPACE, PCE_ECOORD = range(6)
+PCE_F16, PCE_F32 = 0, 1
+DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS = 0, 1, 2
+QUANTUM = 128
+CSR_CODE = 1186111
+
+
+class Geom(Structure):
+    _fields_ = [("ks", c_int32 * 3), ("stride", c_int32 * 3), ("pad", c_int32 * 3),
+                ("cmin", c_int32 * 3), ("cmax", c_int32 * 3), ("subm", c_int32)]
+
+    @classmethod
+    def make(cls, ks, stride, pad, cmin, cmax, subm):
+        g = cls()
+        for name, v in (("ks", ks), ("stride", stride), ("pad", pad), ("cmin", cmin), ("cmax", cmax)):
+            arr = getattr(g, name)
+            for a in range(3):
+                arr[a] = int(v[a])
+        g.subm = int(bool(subm))
+        return g
+
+
+class PCEError(RuntimeError):
+    pass
+
+
+_SIGNATURES = {
+    "pce_version": (c_int32, []),
+    "pce_last_error": (c_char_p, []),
+    "pce_hash_slots": (c_int64, [c_int64]),
+    "pce_hash_table_bytes": (c_int64, [c_int64]),
+    "pce_hash_build": (c_int32, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p]),
+    "pce_hash_query": (c_int32, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p]),
+    "pce_outcoords_workspace_bytes": (c_int64, [c_int64, POINTER(Geom)]),
+    "pce_outcoords_build": (c_int32, [c_void_p, c_int64, POINTER(Geom), c_void_p, c_int64, POINTER(c_int64), c_void_p]),
+    "pce_outcoords_emit": (c_int32, [c_void_p, c_int64, POINTER(Geom), c_int64, c_void_p, c_void_p]),
+    "pce_kmap_workspace_bytes": (c_int64, [c_int64, c_int64, c_int32, c_int32]),
+    "pce_kmap_build": (c_int32, [c_void_p, c_int64, c_void_p, c_int64, POINTER(Geom), c_void_p, c_int64] + [c_void_p] * 12 + [c_void_p]),
+    "pce_conv_fod_workspace_bytes": (c_int64, [c_int64, c_int32, c_int32]),
+    "pce_conv_fwd_fod": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32,
+                                   c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
+    "pce_conv_fwd_gms": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32,
+                                   c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
+    "pce_conv_fwd_os": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
+    "pce_conv_fwd_dense": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32, c_void_p]),
+    "pce_select_dataflow": (c_int32, [c_int64, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32]),
+}
+
+_lib = None
+
+
+def exported_names():
+    return sorted(_SIGNATURES)
+
+
+def load() -> ctypes.CDLL:
+    """Load the shared library (once) and attach the argument types."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise PCEError(
+            f"{LIB_PATH} is missing: build it with `python -m pcengine_amd.build` "
+            "(hipcc, --offload-arch=gfx950).  pcengine_amd has no other compute path.")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in _SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(rc: int) -> None:
+    """Turn a status code into the exception class the reference's pybind layer would raise
+    (std::invalid_argument -> ValueError, std::runtime_error -> RuntimeError)."""
+    if rc == PCE_OK:
+        return
+    msg = load().pce_last_error().decode("utf-8", "replace")
+    if rc == PCE_EINVAL:
+        raise ValueError(msg)
+    if rc == PCE_ECAPACITY:
+        raise OverflowError(msg)
+    raise PCEError(f"[pce status {rc}] {msg}")

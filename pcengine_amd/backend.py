@@ -1,0 +1,367 @@
+"""Torch-facing wrappers over the C ABI.
+
+Two layers live here:
+
+* ``build_kernel_map`` / ``conv_forward`` / ``dense_forward`` — what this package's own front
+  end (spconv.py) calls: one native call per map, one per convolution.
+* ``mapping_d1_cuda``, ``mapping_d2_cuda``, ``conv_fwd_d1_cuda``, ``conv_fwd_d2_cuda``,
+  ``conv_bwd_d1_cuda`` — the five names of the reference's pybind module
+  (backend/pybind_cuda.cpp:8-14) with the reference's argument order, so that code written
+  against ``PCEngine.backend`` keeps working.
+
+Torch is used for device memory and the current stream only.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import Geom, DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS, PCE_F16, PCE_F32, QUANTUM, CSR_CODE
+
+CODE_A, CODE_B = 94273, 311  # packed 3-vectors, script/utils.py:233-242
+
+
+def decode3(code: int) -> Tuple[int, int, int]:
+    x = code // CODE_A
+    y = (code - x * CODE_A) // CODE_B
+    return (x, y, code - x * CODE_A - y * CODE_B)
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _stream(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _require_cuda(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on the GPU: pcengine_amd has no CPU compute path")
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.float16:
+        return PCE_F16
+    if t.dtype == torch.float32:
+        return PCE_F32
+    raise TypeError(f"features must be float16 or float32, got {t.dtype}")
+
+
+def _mid(ks: Sequence[int]) -> int:
+    return (ks[0] - 1) // 2 * ks[1] * ks[2] + (ks[1] - 1) // 2 * ks[2] + (ks[2] - 1) // 2
+
+
+@dataclass
+class KernelMap:
+    """Kernel map of one (kernel size, tensor stride, layer stride) key.
+
+    Pair lists are in (offset, input row) order.  Indexing and ``len`` reproduce the list the
+    reference stores in ``spTensor.kmaps`` (script/spconv.py:382, 431): six entries for the
+    fetch-on-demand map, eight when the CSR view has been built.
+    """
+    ks: Tuple[int, int, int]
+    stride: Tuple[int, int, int]
+    pad: Tuple[int, int, int]
+    subm: bool
+    n_in: int
+    n_out: int
+    kv: int
+    M: int
+    qsum: int
+    imap: torch.Tensor
+    omap: torch.Tensor
+    knnz: torch.Tensor
+    kpos: torch.Tensor
+    qkpos: torch.Tensor
+    out_coords: torch.Tensor
+    nbr_out: Optional[torch.Tensor] = None
+    nbr_in: Optional[torch.Tensor] = None
+    icsr: Optional[torch.Tensor] = None
+    icode: Optional[torch.Tensor] = None
+    ocsr: Optional[torch.Tensor] = None
+    ocode: Optional[torch.Tensor] = None
+    tag: str = "auto"           # 'D1' / 'D2' when the reference's init_tag protocol fixed it
+    in_coords: Optional[torch.Tensor] = None
+    geom: Optional[Geom] = None
+    knnz_host: list = field(default_factory=list)
+
+    @property
+    def has_csr(self) -> bool:
+        return self.icsr is not None
+
+    def _as_list(self):
+        if self.tag == "D1" and self.has_csr:
+            return [self.icode, self.ocode, self.icsr, self.ocsr, self.kpos, self.qkpos, self.qsum, (self.n_in, self.n_out)]
+        return [self.imap, self.omap, self.kpos, self.qkpos, self.qsum, (self.n_in, self.n_out)]
+
+    def __len__(self):
+        return len(self._as_list())
+
+    def __getitem__(self, i):
+        return self._as_list()[i]
+
+
+def strided_coords_max(cmax, ks, stride, pad):
+    """script/spconv.py:358-360."""
+    return [(int(cmax[a]) + 2 * pad[a] - (ks[a] - 1)) // stride[a] for a in range(3)]
+
+
+def build_out_coords(in_coords: torch.Tensor, geom: Geom) -> torch.Tensor:
+    """Sorted unique output coordinates of a strided layer (one host sync for the count)."""
+    lib = _lib.load()
+    _require_cuda(in_coords, "coords")
+    n_in = in_coords.shape[0]
+    ws_bytes = lib.pce_outcoords_workspace_bytes(n_in, geom)
+    if ws_bytes < 0:
+        _lib.check(_lib.PCE_EINVAL)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=in_coords.device)
+    n_out = _lib.c_int64(0)
+    s = _stream(in_coords.device)
+    _lib.check(lib.pce_outcoords_build(in_coords.data_ptr(), n_in, geom, ws.data_ptr(), ws_bytes, n_out, s))
+    out = torch.empty((n_out.value, 4), dtype=torch.int32, device=in_coords.device)
+    _lib.check(lib.pce_outcoords_emit(ws.data_ptr(), n_in, geom, n_out.value, _ptr(out), s))
+    return out
+
+
+def build_kernel_map(in_coords: torch.Tensor, ks, stride, pad, cmin, cmax_out, subm: bool,
+                     want_csr: bool = False, want_nbr_out: bool = True, want_nbr_in: bool = False,
+                     out_coords: Optional[torch.Tensor] = None) -> KernelMap:
+    """Hash the output coordinates, probe every (input row, offset) and emit the canonical map.
+
+    ``cmax_out`` is the bound on output coordinates (already reduced for strided layers)."""
+    lib = _lib.load()
+    _require_cuda(in_coords, "coords")
+    if in_coords.dtype != torch.int32 or in_coords.dim() != 2 or in_coords.shape[1] != 4:
+        raise ValueError("coords must be int32 [N, 4] = (b, x, y, z)")
+    in_coords = in_coords.contiguous()
+    dev = in_coords.device
+    n_in = in_coords.shape[0]
+    kv = int(ks[0]) * int(ks[1]) * int(ks[2])
+    geom = Geom.make(ks, stride, pad, cmin, cmax_out, subm)
+    if subm:
+        out_coords = in_coords
+    elif out_coords is None:
+        out_coords = build_out_coords(in_coords, geom)
+    n_out = out_coords.shape[0]
+    if n_in == 0 or n_out == 0:
+        raise ValueError(f"empty sparse tensor (n_in={n_in}, n_out={n_out})")
+    s = _stream(dev)
+    ws_bytes = lib.pce_kmap_workspace_bytes(n_in, n_out, kv, int(want_csr))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    pairs = torch.empty((2, kv * n_in), dtype=torch.int32, device=dev)
+    # knnz | kpos | qkpos | status in one tensor: a single device->host copy reads all of them
+    meta = torch.zeros(kv + 2 * (kv + 1) + 4, dtype=torch.int32, device=dev)
+    knnz, kpos, qkpos = meta[:kv], meta[kv:2 * kv + 1], meta[2 * kv + 1:3 * kv + 2]
+    status = meta[3 * kv + 2:]
+    nbr_out = torch.empty(kv * n_out, dtype=torch.int32, device=dev) if want_nbr_out else None
+    nbr_in = torch.empty(kv * n_in, dtype=torch.int32, device=dev) if want_nbr_in else None
+    if want_csr:
+        icsr = torch.empty(n_in + 1, dtype=torch.int32, device=dev)
+        ocsr = torch.empty(n_out + 1, dtype=torch.int32, device=dev)
+        codes = torch.empty((2, kv * n_in), dtype=torch.int32, device=dev)
+        icode, ocode = codes[0], codes[1]
+    else:
+        icsr = ocsr = icode = ocode = None
+    _lib.check(lib.pce_kmap_build(in_coords.data_ptr(), n_in, out_coords.data_ptr(), n_out, geom, ws.data_ptr(), ws_bytes,
+                                  pairs[0].data_ptr(), pairs[1].data_ptr(), knnz.data_ptr(), kpos.data_ptr(),
+                                  qkpos.data_ptr(), _ptr(icsr), _ptr(icode), _ptr(ocsr), _ptr(ocode), _ptr(nbr_out),
+                                  _ptr(nbr_in), status.data_ptr(), s))
+    host = meta.cpu().tolist()   # the one synchronisation of a map build
+    st = host[3 * kv + 2:]
+    if st[0]:
+        raise ValueError(f"a coordinate is outside the supported range (|c| < {32000}, batch < 32768)")
+    if st[1]:
+        raise _lib.PCEError("hash table exhausted while building the kernel map")
+    if want_csr and st[2]:
+        raise OverflowError(f"an offset holds >= {CSR_CODE} pairs: the CSR code of the gather-GEMM-scatter map overflows")
+    M, qsum = host[2 * kv], host[3 * kv + 1]
+    km = KernelMap(ks=tuple(ks), stride=tuple(stride), pad=tuple(pad), subm=bool(subm), n_in=n_in, n_out=n_out, kv=kv,
+                   M=M, qsum=qsum, imap=pairs[0, :M], omap=pairs[1, :M], knnz=knnz, kpos=kpos, qkpos=qkpos,
+                   out_coords=out_coords, nbr_out=nbr_out, nbr_in=nbr_in, icsr=icsr, ocsr=ocsr,
+                   icode=None if icode is None else icode[:M], ocode=None if ocode is None else ocode[:M],
+                   in_coords=in_coords, geom=geom, knnz_host=host[:kv])
+    km._cmin, km._cmax = list(cmin), list(cmax_out)
+    return km
+
+
+def ensure_csr(km: KernelMap) -> None:
+    """Build the CSR-coded view of an existing map (first use of gather-GEMM-scatter on it)."""
+    if km.has_csr:
+        return
+    full = build_kernel_map(km.in_coords, km.ks, km.stride, km.pad, km._cmin, km._cmax, km.subm, want_csr=True,
+                            want_nbr_out=False, out_coords=km.out_coords)
+    km.icsr, km.icode, km.ocsr, km.ocode = full.icsr, full.icode, full.ocsr, full.ocode
+
+
+def ensure_nbr(km: KernelMap, transposed: bool) -> None:
+    if (km.nbr_in if transposed else km.nbr_out) is not None:
+        return
+    full = build_kernel_map(km.in_coords, km.ks, km.stride, km.pad, km._cmin, km._cmax, km.subm, want_csr=False,
+                            want_nbr_out=True, want_nbr_in=True, out_coords=km.out_coords)
+    km.nbr_out, km.nbr_in = full.nbr_out, full.nbr_in
+
+
+def select_dataflow(km: KernelMap, c_in: int, c_out: int, dtype: torch.dtype, transposed: bool = False) -> int:
+    lib = _lib.load()
+    n_out = km.n_in if transposed else km.n_out
+    n_in = km.n_out if transposed else km.n_in
+    return lib.pce_select_dataflow(n_in, n_out, km.M, c_in, c_out, km.kv, PCE_F16 if dtype == torch.float16 else PCE_F32)
+
+
+def dense_forward(feats: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """feats @ weight for the 1x1 stride-1 layer (script/spconv.py:297-304)."""
+    lib = _lib.load()
+    _require_cuda(feats, "feats")
+    feats = feats.contiguous()
+    weight = weight.contiguous()
+    if feats.shape[1] != weight.shape[0]:
+        raise ValueError("Input feature size and kernel size mismatch")
+    out = torch.empty((feats.shape[0], weight.shape[1]), dtype=feats.dtype, device=feats.device)
+    _lib.check(lib.pce_conv_fwd_dense(feats.data_ptr(), weight.data_ptr(), out.data_ptr(), _dtype_code(feats),
+                                      feats.shape[0], feats.shape[1], weight.shape[1], _stream(feats.device)))
+    return out
+
+
+def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataflow: int, transposed: bool = False,
+                 buffer: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One forward convolution over an existing map with the chosen dataflow."""
+    lib = _lib.load()
+    _require_cuda(feats, "feats")
+    feats = feats.contiguous()
+    weight = weight.contiguous()
+    if weight.dim() == 2:
+        weight = weight.unsqueeze(0)
+    if feats.dtype != weight.dtype:
+        raise TypeError(f"features are {feats.dtype} but the kernel is {weight.dtype}")
+    kv, c_in, c_out = weight.shape
+    if feats.shape[1] != c_in:
+        raise ValueError("Input feature size and kernel size mismatch")   # backend/spconv.cu:38-40
+    if kv != km.kv:
+        raise ValueError(f"kernel volume {kv} does not match the map ({km.kv})")
+    n_in, n_out = (km.n_out, km.n_in) if transposed else (km.n_in, km.n_out)
+    if feats.shape[0] != n_in:
+        raise ValueError(f"features have {feats.shape[0]} rows, the map expects {n_in}")
+    dt = _dtype_code(feats)
+    dev = feats.device
+    s = _stream(dev)
+    mid = _mid(km.ks) if km.subm else -1
+    out = torch.empty((n_out, c_out), dtype=feats.dtype, device=dev)
+    if dataflow == DATAFLOW_FOD:
+        imap, omap = (km.omap, km.imap) if transposed else (km.imap, km.omap)
+        ws_bytes = lib.pce_conv_fod_workspace_bytes(n_out, c_out, dt)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+        _lib.check(lib.pce_conv_fwd_fod(feats.data_ptr(), weight.data_ptr(), out.data_ptr(), dt, n_in, n_out, c_in, c_out,
+                                        kv, mid, imap.data_ptr(), omap.data_ptr(), km.kpos.data_ptr(), km.qkpos.data_ptr(),
+                                        km.qsum, _ptr(ws), ws_bytes, s))
+    elif dataflow == DATAFLOW_GMS:
+        ensure_csr(km)
+        need = km.qsum * (c_in + c_out)
+        if buffer is None or buffer.numel() < need or buffer.dtype != feats.dtype or buffer.device != dev:
+            buffer = torch.empty(max(need, 1), dtype=feats.dtype, device=dev)
+        icsr, icode, ocsr, ocode = (km.ocsr, km.ocode, km.icsr, km.icode) if transposed else (km.icsr, km.icode, km.ocsr, km.ocode)
+        _lib.check(lib.pce_conv_fwd_gms(feats.data_ptr(), weight.data_ptr(), out.data_ptr(), dt, n_in, n_out, c_in, c_out,
+                                        kv, mid, icsr.data_ptr(), icode.data_ptr(), ocsr.data_ptr(), ocode.data_ptr(),
+                                        km.kpos.data_ptr(), km.qkpos.data_ptr(), km.qsum, buffer.data_ptr(), buffer.numel(), s))
+    elif dataflow == DATAFLOW_OS:
+        ensure_nbr(km, transposed)
+        nbr = km.nbr_in if transposed else km.nbr_out
+        _lib.check(lib.pce_conv_fwd_os(feats.data_ptr(), weight.data_ptr(), out.data_ptr(), dt, n_in, n_out, c_in, c_out,
+                                       kv, nbr.data_ptr(), s))
+    else:
+        raise NotImplementedError(f"unknown dataflow {dataflow}")
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# The reference's pybind names (backend/pybind_cuda.cpp:8-14), same argument order.
+# ---------------------------------------------------------------------------------------------
+def _geom_from_codes(k_size_code, l_stride_code, padding_code, mins, maxs, separate_mid):
+    return decode3(k_size_code), decode3(l_stride_code), decode3(padding_code), list(mins), list(maxs), bool(separate_mid)
+
+
+def mapping_d2_cuda(in_coords, batch_size, k_size_code, k_vol, c_in, c_out, l_stride_code, t_stride_code, padding_code,
+                    min_x, min_y, min_z, max_x, max_y, max_z, map, kernel_nnz, kernel_kpos, kernel_qkpos, separate_mid):
+    """HashMapD2 (backend/hash.h:37-58): fills the dense map ``map[kp*N_in + i] = o`` (caller
+    pre-fills -1), the per-offset counts and both scans; returns the output coordinates (the
+    input tensor itself for a submanifold layer)."""
+    ks, stride, pad, cmin, cmax, subm = _geom_from_codes(k_size_code, l_stride_code, padding_code,
+                                                         (min_x, min_y, min_z), (max_x, max_y, max_z), separate_mid)
+    km = build_kernel_map(in_coords, ks, stride, pad, cmin, cmax, subm, want_nbr_out=False, want_nbr_in=True)
+    map.view(-1)[:km.kv * km.n_in].copy_(km.nbr_in)
+    kernel_nnz[:km.kv].copy_(km.knnz)
+    kernel_kpos[:km.kv + 1].copy_(km.kpos)
+    kernel_qkpos[:km.kv + 1].copy_(km.qkpos)
+    return in_coords if subm else km.out_coords
+
+
+def mapping_d1_cuda(in_coords, k_size_code, k_vol, c_in, c_out, l_stride_code, t_stride_code, padding_code,
+                    min_x, min_y, min_z, max_x, max_y, max_z, imap, omap, icsr, ocsr, kernel_nnz, kernel_kpos,
+                    kernel_qkpos, separate_mid):
+    """HashMapD1 (backend/hash.h:11-34): compacted CSR codes at the front of ``imap`` / ``omap``,
+    row pointers in ``icsr`` / ``ocsr``, counts and scans.  ``kernel_kpos`` may have the
+    reference's kv entries (script/spconv.py:396) or kv+1; only what fits is written."""
+    ks, stride, pad, cmin, cmax, subm = _geom_from_codes(k_size_code, l_stride_code, padding_code,
+                                                         (min_x, min_y, min_z), (max_x, max_y, max_z), separate_mid)
+    km = build_kernel_map(in_coords, ks, stride, pad, cmin, cmax, subm, want_csr=True, want_nbr_out=False)
+    if omap.numel() < km.M or ocsr.numel() < km.n_out + 1:
+        raise OverflowError("omap / ocsr are too small for this map")
+    imap.view(-1)[:km.M].copy_(km.icode)
+    omap.view(-1)[:km.M].copy_(km.ocode)
+    icsr[:km.n_in + 1].copy_(km.icsr)
+    ocsr[:km.n_out + 1].copy_(km.ocsr)
+    kernel_nnz[:km.kv].copy_(km.knnz)
+    n = min(kernel_kpos.numel(), km.kv + 1)
+    kernel_kpos[:n].copy_(km.kpos[:n])
+    kernel_qkpos[:km.kv + 1].copy_(km.qkpos)
+    return in_coords if subm else km.out_coords
+
+
+def _ksize_mid(ksize_code: int, separate_mid: bool) -> int:
+    return _mid(decode3(ksize_code)) if separate_mid else -1
+
+
+def conv_fwd_d2_cuda(in_feats, kernel, ksize_code, sum_nnz, out_feats, kpos, qkpos, in_map, out_map, separate_mid, tf32):
+    """ConvolutionForwardD2 (backend/spconv.h:28-40); ``sum_nnz`` is qkpos[-1] as in the reference."""
+    lib = _lib.load()
+    _require_cuda(in_feats, "in_feats")
+    if in_feats.shape[1] != kernel.shape[1]:
+        raise ValueError("Input feature size and kernel size mismatch")
+    kv, c_in, c_out = kernel.shape
+    dt = _dtype_code(in_feats)
+    n_in, n_out = in_feats.shape[0], out_feats.shape[0]
+    ws_bytes = lib.pce_conv_fod_workspace_bytes(n_out, c_out, dt)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=in_feats.device) if ws_bytes else None
+    _lib.check(lib.pce_conv_fwd_fod(in_feats.data_ptr(), kernel.data_ptr(), out_feats.data_ptr(), dt, n_in, n_out, c_in,
+                                    c_out, kv, _ksize_mid(ksize_code, separate_mid), in_map.data_ptr(), out_map.data_ptr(),
+                                    kpos.data_ptr(), qkpos.data_ptr(), int(sum_nnz), _ptr(ws), ws_bytes,
+                                    _stream(in_feats.device)))
+
+
+def conv_fwd_d1_cuda(in_feats, kernel, ksize_code, qsum_nnz, out_feats, kpos, qkpos, in_map, out_map, in_csr, out_csr,
+                     buffer, separate_mid, tensorcore):
+    """ConvolutionForwardD1 (backend/spconv.h:11-25)."""
+    lib = _lib.load()
+    _require_cuda(in_feats, "in_feats")
+    if in_feats.shape[1] != kernel.shape[1]:
+        raise ValueError("Input feature size and kernel size mismatch")
+    kv, c_in, c_out = kernel.shape
+    dt = _dtype_code(in_feats)
+    if buffer.dtype != in_feats.dtype:
+        raise TypeError("the staging buffer must have the dtype of the features")
+    if kpos.numel() < kv + 1:
+        # the reference front end allocates kv entries (script/spconv.py:396); the total is the last row pointer
+        kpos = torch.cat([kpos[:kv], in_csr[in_feats.shape[0]:in_feats.shape[0] + 1]])
+    _lib.check(lib.pce_conv_fwd_gms(in_feats.data_ptr(), kernel.data_ptr(), out_feats.data_ptr(), dt, in_feats.shape[0],
+                                    out_feats.shape[0], c_in, c_out, kv, _ksize_mid(ksize_code, separate_mid),
+                                    in_csr.data_ptr(), in_map.data_ptr(), out_csr.data_ptr(), out_map.data_ptr(),
+                                    kpos.data_ptr(), qkpos.data_ptr(), int(qsum_nnz), buffer.data_ptr(), buffer.numel(),
+                                    _stream(in_feats.device)))
+
+
+def conv_bwd_d1_cuda(*args, **kwargs):
+    """ConvolutionBackwardD1 (backend/spconv.h:43-58) belongs to training; this engine is forward-only."""
+    raise NotImplementedError("pcengine_amd is an inference engine: the backward pass is not provided")

@@ -1,0 +1,752 @@
+// Coordinate hash table, output-coordinate generation and kernel-map construction for gfx950.
+//
+// All kernels are integer / byte work bound by HBM and L2 traffic: one lane per voxel row, row
+// indices contiguous across a wavefront so that every table of the form t[kp * n + row] is read and
+// written with full 256-byte wave transactions; per-offset ranks come from wave ballots, so the
+// (offset, input row) order of the pair list is fixed by construction and needs no atomics.
+#include <stdarg.h>
+#include <string.h>
+
+#include "pce_common.h"
+
+// ------------------------------------------------------------------------------------------------
+// host-side error text
+// ------------------------------------------------------------------------------------------------
+static thread_local char g_err[512] = "";
+
+void pce_set_error(const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+extern "C" const char *pce_last_error(void) { return g_err; }
+extern "C" int pce_version(void) { return 100; }
+
+// ------------------------------------------------------------------------------------------------
+// small device helpers
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ unsigned long long lanemask_lt() {
+  unsigned lane = __lane_id();
+  return lane == 0 ? 0ull : (~0ull >> (64 - lane));
+}
+
+__global__ void fill_u32_kernel(unsigned *p, long long n, unsigned v) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  long long step = (long long)gridDim.x * blockDim.x;
+  for (; i < n; i += step) p[i] = v;
+}
+
+static int fill_u32(void *p, int64_t n_words, unsigned v, hipStream_t s) {
+  if (n_words <= 0) return PCE_OK;
+  int64_t blocks = pce_div_up(n_words, 256 * 8);
+  if (blocks > 65535 * 16) blocks = 65535 * 16;
+  hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (unsigned *)p,
+                     (long long)n_words, v);
+  PCE_LAUNCH_CHECK("fill_u32");
+  return PCE_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// hash table
+// ------------------------------------------------------------------------------------------------
+// Insert key -> row.  Equal keys keep the smallest row, so the table content does not depend on
+// the order in which lanes arrive.  The probe loop is bounded by the slot count.
+__device__ __forceinline__ bool table_insert(pce_slot_t *table, unsigned long long slots,
+                                             unsigned long long key, unsigned row, bool *was_new) {
+  unsigned long long s = pce_home_slot(key, slots);
+  for (unsigned long long it = 0; it < slots; ++it) {
+    unsigned long long prev = atomicCAS(&table[s].key, PCE_EMPTY_KEY, key);
+    if (prev == PCE_EMPTY_KEY || prev == key) {
+      atomicMin(&table[s].row, row);
+      if (was_new) *was_new = (prev == PCE_EMPTY_KEY);
+      return true;
+    }
+    s = (s + 1) & (slots - 1);
+  }
+  return false;
+}
+
+__device__ __forceinline__ int table_find(const pce_slot_t *__restrict__ table,
+                                          unsigned long long slots, unsigned long long key) {
+  unsigned long long s = pce_home_slot(key, slots);
+  for (unsigned long long it = 0; it < slots; ++it) {
+    // one 16-byte load returns key and row together
+    const uint4 e = *reinterpret_cast<const uint4 *>(&table[s]);
+    unsigned long long k = ((unsigned long long)e.y << 32) | e.x;
+    if (k == key) return (int)e.z;
+    if (k == PCE_EMPTY_KEY) return -1;
+    s = (s + 1) & (slots - 1);
+  }
+  return -1;
+}
+
+__global__ void __launch_bounds__(256) hash_insert_kernel(pce_slot_t *table, unsigned long long slots,
+                                                          const int4 *__restrict__ coords,
+                                                          long long n, int *status) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  int4 c = coords[i];
+  if (!pce_coord_ok(c.x, c.y, c.z, c.w)) {
+    status[0] = 1;
+    return;
+  }
+  if (!table_insert(table, slots, pce_pack_key(c.x, c.y, c.z, c.w), (unsigned)i, nullptr)) status[1] = 1;
+}
+
+__global__ void __launch_bounds__(256) hash_query_kernel(const pce_slot_t *__restrict__ table,
+                                                         unsigned long long slots,
+                                                         const int4 *__restrict__ q, long long nq,
+                                                         int *__restrict__ rows) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= nq) return;
+  int4 c = q[i];
+  rows[i] = pce_coord_ok(c.x, c.y, c.z, c.w) ? table_find(table, slots, pce_pack_key(c.x, c.y, c.z, c.w)) : -1;
+}
+
+extern "C" int64_t pce_hash_slots(int64_t n) {
+  int64_t p = 1;
+  while (p < n) p <<= 1;
+  int64_t s = 2 * p;
+  return s < 8 ? 8 : s;
+}
+
+extern "C" int64_t pce_hash_table_bytes(int64_t n) { return pce_hash_slots(n) * (int64_t)sizeof(pce_slot_t); }
+
+static int table_clear(void *table, int64_t slots, hipStream_t s) {
+  return fill_u32(table, slots * 4, 0xFFFFFFFFu, s);
+}
+
+extern "C" int pce_hash_build(void *table, int64_t slots, const int32_t *coords, int64_t n,
+                              int32_t *status, pce_stream_t stream) {
+  hipStream_t s = (hipStream_t)stream;
+  if (!table || !status || (n > 0 && !coords)) PCE_FAIL(PCE_EINVAL, "pce_hash_build: null pointer");
+  if (slots < 8 || (slots & (slots - 1)) || slots < 2 * n)
+    PCE_FAIL(PCE_EINVAL, "pce_hash_build: slots=%lld must be a power of two >= 2*n", (long long)slots);
+  if (n >= (1ll << 31)) PCE_FAIL(PCE_ECAPACITY, "pce_hash_build: n=%lld exceeds int32 rows", (long long)n);
+  int rc = table_clear(table, slots, s);
+  if (rc) return rc;
+  if (n == 0) return PCE_OK;
+  hipLaunchKernelGGL(hash_insert_kernel, dim3((unsigned)pce_div_up(n, 256)), dim3(256), 0, s,
+                     (pce_slot_t *)table, (unsigned long long)slots, (const int4 *)coords, (long long)n, status);
+  PCE_LAUNCH_CHECK("hash_insert");
+  return PCE_OK;
+}
+
+extern "C" int pce_hash_query(const void *table, int64_t slots, const int32_t *q, int64_t nq,
+                              int32_t *rows, pce_stream_t stream) {
+  if (!table || (nq > 0 && (!q || !rows))) PCE_FAIL(PCE_EINVAL, "pce_hash_query: null pointer");
+  if (slots < 8 || (slots & (slots - 1))) PCE_FAIL(PCE_EINVAL, "pce_hash_query: slots must be a power of two");
+  if (nq == 0) return PCE_OK;
+  hipLaunchKernelGGL(hash_query_kernel, dim3((unsigned)pce_div_up(nq, 256)), dim3(256), 0, (hipStream_t)stream,
+                     (const pce_slot_t *)table, (unsigned long long)slots, (const int4 *)q, (long long)nq, rows);
+  PCE_LAUNCH_CHECK("hash_query");
+  return PCE_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// exclusive scan of int32 in place (three launches, any length)
+// ------------------------------------------------------------------------------------------------
+#define SCAN_ITEMS 8
+#define SCAN_TILE (256 * SCAN_ITEMS)
+
+__device__ __forceinline__ int wave_inclusive_scan(int v) {
+#pragma unroll
+  for (int d = 1; d < PCE_WAVE; d <<= 1) {
+    int t = __shfl_up(v, d, PCE_WAVE);
+    if ((int)__lane_id() >= d) v += t;
+  }
+  return v;
+}
+
+// exclusive prefix of v over the 256 threads of the block; *total = block sum
+__device__ __forceinline__ int block_exclusive_scan(int v, int *total) {
+  __shared__ int wsum[4];
+  int inc = wave_inclusive_scan(v);
+  int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 63) wsum[wave] = inc;
+  __syncthreads();
+  int base = 0;
+  for (int w = 0; w < wave; ++w) base += wsum[w];
+  *total = wsum[0] + wsum[1] + wsum[2] + wsum[3];
+  __syncthreads();
+  return base + inc - v;
+}
+
+__global__ void __launch_bounds__(256) scan_reduce_kernel(const int *__restrict__ data, long long n,
+                                                          int *__restrict__ sums) {
+  long long base = (long long)blockIdx.x * SCAN_TILE + (long long)threadIdx.x * SCAN_ITEMS;
+  int acc = 0;
+#pragma unroll
+  for (int j = 0; j < SCAN_ITEMS; ++j)
+    if (base + j < n) acc += data[base + j];
+  int total;
+  block_exclusive_scan(acc, &total);
+  if (threadIdx.x == 0) sums[blockIdx.x] = total;
+}
+
+__global__ void __launch_bounds__(256) scan_sums_kernel(int *sums, long long nb) {
+  int carry = 0;
+  for (long long base = 0; base < nb; base += 256) {
+    long long i = base + threadIdx.x;
+    int v = i < nb ? sums[i] : 0;
+    int total;
+    int ex = block_exclusive_scan(v, &total);
+    if (i < nb) sums[i] = carry + ex;
+    carry += total;
+  }
+}
+
+__global__ void __launch_bounds__(256) scan_apply_kernel(int *data, long long n, const int *__restrict__ sums) {
+  long long base = (long long)blockIdx.x * SCAN_TILE + (long long)threadIdx.x * SCAN_ITEMS;
+  int v[SCAN_ITEMS];
+  int acc = 0;
+#pragma unroll
+  for (int j = 0; j < SCAN_ITEMS; ++j) {
+    v[j] = (base + j < n) ? data[base + j] : 0;
+    acc += v[j];
+  }
+  int total;
+  int run = block_exclusive_scan(acc, &total) + sums[blockIdx.x];
+#pragma unroll
+  for (int j = 0; j < SCAN_ITEMS; ++j) {
+    if (base + j < n) data[base + j] = run;
+    run += v[j];
+  }
+}
+
+static int64_t scan_tmp_ints(int64_t n) { return pce_div_up(n, SCAN_TILE) + 1; }
+
+static int scan_exclusive(int *data, int64_t n, int *tmp, hipStream_t s) {
+  if (n <= 0) return PCE_OK;
+  int64_t nb = pce_div_up(n, SCAN_TILE);
+  hipLaunchKernelGGL(scan_reduce_kernel, dim3((unsigned)nb), dim3(256), 0, s, (const int *)data, (long long)n, tmp);
+  PCE_LAUNCH_CHECK("scan_reduce");
+  hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(256), 0, s, tmp, (long long)nb);
+  PCE_LAUNCH_CHECK("scan_sums");
+  hipLaunchKernelGGL(scan_apply_kernel, dim3((unsigned)nb), dim3(256), 0, s, data, (long long)n, (const int *)tmp);
+  PCE_LAUNCH_CHECK("scan_apply");
+  return PCE_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// geometry
+// ------------------------------------------------------------------------------------------------
+struct GeomDev {
+  int ks[3], stride[3], pad[3], cmin[3], cmax[3];
+  int bump[3];  // +1 on odd kernel sizes > 1 for strided layers (backend/hash.cuh:235-237)
+  int half[3];  // (ks-1)/2
+  int subm, kv, mid;
+};
+
+static int make_geom(const pce_geom_t *g, GeomDev *d) {
+  if (!g) PCE_FAIL(PCE_EINVAL, "geometry is null");
+  int64_t kv = 1;
+  for (int a = 0; a < 3; ++a) {
+    if (g->ks[a] < 1 || g->stride[a] < 1 || g->pad[a] < 0)
+      PCE_FAIL(PCE_EINVAL, "geometry: kernel size and stride must be >= 1, padding >= 0");
+    d->ks[a] = g->ks[a];
+    d->stride[a] = g->stride[a];
+    d->pad[a] = g->pad[a];
+    d->cmin[a] = g->cmin[a];
+    d->cmax[a] = g->cmax[a];
+    d->half[a] = (g->ks[a] - 1) / 2;
+    d->bump[a] = (!g->subm && g->ks[a] % 2 == 1 && g->ks[a] > 1) ? 1 : 0;
+    kv *= g->ks[a];
+  }
+  if (kv > 1024) PCE_FAIL(PCE_ECAPACITY, "kernel volume %lld exceeds 1024", (long long)kv);
+  d->subm = g->subm ? 1 : 0;
+  d->kv = (int)kv;
+  d->mid = d->half[0] * g->ks[1] * g->ks[2] + d->half[1] * g->ks[2] + d->half[2];
+  if (g->subm && (g->stride[0] != 1 || g->stride[1] != 1 || g->stride[2] != 1))
+    PCE_FAIL(PCE_EINVAL, "a submanifold layer has stride 1");
+  return PCE_OK;
+}
+
+// offset index (ix,iy,iz) -> d(kp), advanced incrementally by the callers
+struct OffsetIter {
+  int ix, iy, iz;
+  __device__ __forceinline__ void init() { ix = iy = iz = 0; }
+  __device__ __forceinline__ void next(const GeomDev &g) {
+    if (++iz == g.ks[2]) {
+      iz = 0;
+      if (++iy == g.ks[1]) {
+        iy = 0;
+        ++ix;
+      }
+    }
+  }
+  __device__ __forceinline__ int dx(const GeomDev &g) const { return ix - g.half[0] + g.bump[0]; }
+  __device__ __forceinline__ int dy(const GeomDev &g) const { return iy - g.half[1] + g.bump[1]; }
+  __device__ __forceinline__ int dz(const GeomDev &g) const { return iz - g.half[2] + g.bump[2]; }
+};
+
+// Output coordinate reached from input coordinate c through offset d on one axis of a strided
+// layer: (c - d + pad) / stride when it divides and lies in [cmin, cmax]  (backend/hash.cuh:596-605).
+__device__ __forceinline__ bool strided_axis(int c, int d, int pad, int stride, int lo, int hi, int *o) {
+  int cand = c - d + pad;
+  int q = cand / stride;
+  *o = q;
+  return (cand % stride == 0) && q >= lo && q <= hi;
+}
+
+// ------------------------------------------------------------------------------------------------
+// output coordinates of a strided layer
+// ------------------------------------------------------------------------------------------------
+struct OutCoordLayout {
+  int64_t upper;       // bound on the number of candidates that survive
+  int64_t slots;       // de-duplication table
+  int64_t off_table, off_codes_a, off_codes_b, off_hist, off_scan, off_counters, total;
+  int64_t sort_blocks;
+};
+
+#define SORT_KEYS_PER_BLOCK 1024  // one wavefront per block, 16 rounds of 64 keys
+
+static void outcoord_layout(int64_t n_in, const GeomDev &g, OutCoordLayout *L) {
+  int64_t per = 1;
+  for (int a = 0; a < 3; ++a) per *= pce_div_up(g.ks[a], g.stride[a]);
+  L->upper = n_in * per;
+  if (L->upper < 1) L->upper = 1;
+  L->slots = pce_hash_slots(L->upper);
+  L->sort_blocks = pce_div_up(L->upper, SORT_KEYS_PER_BLOCK);
+  int64_t o = 0;
+  L->off_table = o;
+  o += pce_align_up(L->slots * 16, 256);
+  L->off_codes_a = o;
+  o += pce_align_up(L->upper * 8, 256);
+  L->off_codes_b = o;
+  o += pce_align_up(L->upper * 8, 256);
+  L->off_hist = o;
+  o += pce_align_up((256 * L->sort_blocks + 1) * 4, 256);
+  L->off_scan = o;
+  o += pce_align_up(scan_tmp_ints(256 * L->sort_blocks + 1) * 4, 256);
+  L->off_counters = o;
+  o += 256;
+  L->total = o;
+}
+
+// counters[0] = number of unique candidates, counters[1] = largest code
+__global__ void __launch_bounds__(256) outcoord_candidates_kernel(const int4 *__restrict__ coords, long long n_in,
+                                                                  GeomDev g, pce_slot_t *table,
+                                                                  unsigned long long slots,
+                                                                  unsigned long long *__restrict__ codes,
+                                                                  unsigned long long *counters, int *status) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  bool live = i < n_in;
+  int4 c = live ? coords[i] : make_int4(0, 0, 0, 0);
+  if (live && !pce_coord_ok(c.x, c.y, c.z, c.w)) {
+    status[0] = 1;
+    live = false;
+  }
+  OffsetIter it;
+  it.init();
+  unsigned long long my_max = 0;
+  for (int kp = 0; kp < g.kv; ++kp, it.next(g)) {
+    bool fresh = false;
+    unsigned long long code = 0;
+    if (live) {
+      int ox, oy, oz;
+      bool ok = strided_axis(c.y, it.dx(g), g.pad[0], g.stride[0], g.cmin[0], g.cmax[0], &ox);
+      ok &= strided_axis(c.z, it.dy(g), g.pad[1], g.stride[1], g.cmin[1], g.cmax[1], &oy);
+      ok &= strided_axis(c.w, it.dz(g), g.pad[2], g.stride[2], g.cmin[2], g.cmax[2], &oz);
+      if (ok) {
+        if (ox < 0 || oy < 0 || oz < 0 || ox >= PCE_COORD_BOUND || oy >= PCE_COORD_BOUND || oz >= PCE_COORD_BOUND) {
+          status[0] = 1;
+        } else {
+          if (!table_insert(table, slots, pce_pack_key(c.x, ox, oy, oz), 0u, &fresh)) status[1] = 1;
+          // base-3259 code whose ascending order is (b,x,y,z) order (backend/hash.cuh:607-608)
+          code = (((unsigned long long)c.x * PCE_COORD_BOUND + ox) * PCE_COORD_BOUND + oy) * PCE_COORD_BOUND + oz;
+        }
+      }
+    }
+    unsigned long long bal = __ballot(fresh);
+    if (bal) {
+      unsigned long long base = 0;
+      int leader = __ffsll((long long)bal) - 1;
+      if ((int)__lane_id() == leader) base = atomicAdd(&counters[0], (unsigned long long)__popcll(bal));
+      base = __shfl(base, leader, PCE_WAVE);
+      if (fresh) {
+        codes[base + __popcll(bal & lanemask_lt())] = code;
+        my_max = code > my_max ? code : my_max;
+      }
+    }
+  }
+  // wave max, one atomic per wave
+  for (int d = 32; d >= 1; d >>= 1) {
+    unsigned long long o = __shfl_xor(my_max, d, PCE_WAVE);
+    my_max = o > my_max ? o : my_max;
+  }
+  if (__lane_id() == 0 && my_max) atomicMax(&counters[1], my_max);
+}
+
+// --- stable LSD radix sort on 64-bit codes, 8 bits per pass, one wavefront per block -------------
+__global__ void __launch_bounds__(64) sort_hist_kernel(const unsigned long long *__restrict__ keys, long long n,
+                                                       int shift, int *__restrict__ hist, int nblocks) {
+  __shared__ int bins[256];
+  for (int j = threadIdx.x; j < 256; j += 64) bins[j] = 0;
+  __syncthreads();
+  long long base = (long long)blockIdx.x * SORT_KEYS_PER_BLOCK;
+  for (int r = 0; r < SORT_KEYS_PER_BLOCK / 64; ++r) {
+    long long i = base + r * 64 + threadIdx.x;
+    if (i < n) atomicAdd(&bins[(keys[i] >> shift) & 255], 1);
+  }
+  __syncthreads();
+  for (int j = threadIdx.x; j < 256; j += 64) hist[(long long)j * nblocks + blockIdx.x] = bins[j];
+}
+
+__global__ void __launch_bounds__(64) sort_scatter_kernel(const unsigned long long *__restrict__ src,
+                                                          unsigned long long *__restrict__ dst, long long n,
+                                                          int shift, const int *__restrict__ offs, int nblocks) {
+  __shared__ int run[256];  // keys of each digit already placed by this block
+  for (int j = threadIdx.x; j < 256; j += 64) run[j] = 0;
+  __syncthreads();
+  long long base = (long long)blockIdx.x * SORT_KEYS_PER_BLOCK;
+  for (int r = 0; r < SORT_KEYS_PER_BLOCK / 64; ++r) {
+    long long i = base + r * 64 + threadIdx.x;
+    bool live = i < n;
+    unsigned long long key = live ? src[i] : 0;
+    int d = (int)((key >> shift) & 255);
+    // lanes holding the same digit
+    unsigned long long peers = __ballot(live);
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+      unsigned long long bal = __ballot((d >> b) & 1);
+      peers &= ((d >> b) & 1) ? bal : ~bal;
+    }
+    int before = 0, old = 0;
+    if (live) {
+      before = __popcll(peers & lanemask_lt());
+      int leader = __ffsll((long long)peers) - 1;
+      if (before == 0) {
+        old = run[d];
+        run[d] = old + __popcll(peers);
+      }
+      old = __shfl(old, leader, PCE_WAVE);
+      dst[(long long)offs[(long long)d * nblocks + blockIdx.x] + old + before] = key;
+    }
+    __syncthreads();
+  }
+}
+
+__global__ void decode_codes_kernel(const unsigned long long *__restrict__ codes, long long n, int4 *__restrict__ out) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  unsigned long long c = codes[i];
+  int4 o;
+  o.w = (int)(c % PCE_COORD_BOUND);
+  c /= PCE_COORD_BOUND;
+  o.z = (int)(c % PCE_COORD_BOUND);
+  c /= PCE_COORD_BOUND;
+  o.y = (int)(c % PCE_COORD_BOUND);
+  c /= PCE_COORD_BOUND;
+  o.x = (int)c;
+  out[i] = o;
+}
+
+extern "C" int64_t pce_outcoords_workspace_bytes(int64_t n_in, const pce_geom_t *g) {
+  GeomDev gd;
+  if (make_geom(g, &gd)) return -1;
+  OutCoordLayout L;
+  outcoord_layout(n_in, gd, &L);
+  return L.total;
+}
+
+extern "C" int pce_outcoords_build(const int32_t *in_coords, int64_t n_in, const pce_geom_t *g, void *ws,
+                                   int64_t ws_bytes, int64_t *n_out_host, pce_stream_t stream) {
+  hipStream_t s = (hipStream_t)stream;
+  GeomDev gd;
+  int rc = make_geom(g, &gd);
+  if (rc) return rc;
+  if (!in_coords || !ws || !n_out_host) PCE_FAIL(PCE_EINVAL, "pce_outcoords_build: null pointer");
+  if (n_in <= 0 || n_in >= (1ll << 31)) PCE_FAIL(PCE_EINVAL, "pce_outcoords_build: n_in=%lld", (long long)n_in);
+  OutCoordLayout L;
+  outcoord_layout(n_in, gd, &L);
+  if (ws_bytes < L.total) PCE_FAIL(PCE_EWORKSPACE, "pce_outcoords_build: workspace %lld < %lld", (long long)ws_bytes, (long long)L.total);
+  if (L.upper >= (1ll << 31)) PCE_FAIL(PCE_ECAPACITY, "pce_outcoords_build: candidate bound %lld exceeds int32", (long long)L.upper);
+  char *w = (char *)ws;
+  pce_slot_t *table = (pce_slot_t *)(w + L.off_table);
+  unsigned long long *ca = (unsigned long long *)(w + L.off_codes_a);
+  unsigned long long *cb = (unsigned long long *)(w + L.off_codes_b);
+  int *hist = (int *)(w + L.off_hist);
+  int *scan_tmp = (int *)(w + L.off_scan);
+  unsigned long long *counters = (unsigned long long *)(w + L.off_counters);
+  if ((rc = table_clear(table, L.slots, s))) return rc;
+  if ((rc = fill_u32(counters, 64, 0u, s))) return rc;  // counters[0..1] and status at counters[4..]
+  int *status = (int *)(counters + 4);
+  hipLaunchKernelGGL(outcoord_candidates_kernel, dim3((unsigned)pce_div_up(n_in, 256)), dim3(256), 0, s,
+                     (const int4 *)in_coords, (long long)n_in, gd, table, (unsigned long long)L.slots, ca, counters, status);
+  PCE_LAUNCH_CHECK("outcoord_candidates");
+  unsigned long long host[6];
+  PCE_HIP(hipMemcpyAsync(host, counters, sizeof(host), hipMemcpyDeviceToHost, s));
+  PCE_HIP(hipStreamSynchronize(s));
+  int hstatus[2];
+  memcpy(hstatus, &host[4], sizeof(hstatus));
+  if (hstatus[0]) PCE_FAIL(PCE_ECOORD, "pce_outcoords_build: coordinate outside [0,%d) or batch index out of range", PCE_COORD_BOUND);
+  if (hstatus[1]) PCE_FAIL(PCE_ECAPACITY, "pce_outcoords_build: de-duplication table exhausted");
+  int64_t n = (int64_t)host[0];
+  *n_out_host = n;
+  if (n == 0) return PCE_OK;
+  int bits = 0;
+  while (bits < 64 && (host[1] >> bits)) ++bits;
+  int passes = (bits + 7) / 8;
+  if (passes < 1) passes = 1;
+  int nblocks = (int)pce_div_up(n, SORT_KEYS_PER_BLOCK);
+  unsigned long long *src = ca, *dst = cb;
+  for (int p = 0; p < passes; ++p) {
+    hipLaunchKernelGGL(sort_hist_kernel, dim3(nblocks), dim3(64), 0, s, (const unsigned long long *)src, (long long)n,
+                       8 * p, hist, nblocks);
+    PCE_LAUNCH_CHECK("sort_hist");
+    if ((rc = scan_exclusive(hist, 256ll * nblocks, scan_tmp, s))) return rc;
+    hipLaunchKernelGGL(sort_scatter_kernel, dim3(nblocks), dim3(64), 0, s, (const unsigned long long *)src, dst,
+                       (long long)n, 8 * p, (const int *)hist, nblocks);
+    PCE_LAUNCH_CHECK("sort_scatter");
+    unsigned long long *t = src;
+    src = dst;
+    dst = t;
+  }
+  if (src != ca) PCE_HIP(hipMemcpyAsync(ca, src, (size_t)n * 8, hipMemcpyDeviceToDevice, s));
+  return PCE_OK;
+}
+
+extern "C" int pce_outcoords_emit(const void *ws, int64_t n_in, const pce_geom_t *g, int64_t n_out,
+                                  int32_t *out_coords, pce_stream_t stream) {
+  GeomDev gd;
+  int rc = make_geom(g, &gd);
+  if (rc) return rc;
+  if (!ws || (n_out > 0 && !out_coords)) PCE_FAIL(PCE_EINVAL, "pce_outcoords_emit: null pointer");
+  OutCoordLayout L;
+  outcoord_layout(n_in, gd, &L);
+  if (n_out < 0 || n_out > L.upper) PCE_FAIL(PCE_EINVAL, "pce_outcoords_emit: n_out=%lld out of range", (long long)n_out);
+  if (n_out == 0) return PCE_OK;
+  const unsigned long long *ca = (const unsigned long long *)((const char *)ws + L.off_codes_a);
+  hipLaunchKernelGGL(decode_codes_kernel, dim3((unsigned)pce_div_up(n_out, 256)), dim3(256), 0, (hipStream_t)stream, ca,
+                     (long long)n_out, (int4 *)out_coords);
+  PCE_LAUNCH_CHECK("decode_codes");
+  return PCE_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// kernel map
+// ------------------------------------------------------------------------------------------------
+struct KmapLayout {
+  int64_t slots, nseg, scan_len;
+  int64_t off_table, off_dense, off_seg, off_scan, off_orank, off_irank, total;
+};
+
+static void kmap_layout(int64_t n_in, int64_t n_out, int kv, int want_csr, KmapLayout *L) {
+  L->slots = pce_hash_slots(n_out);
+  L->nseg = pce_div_up(n_in, PCE_WAVE);
+  L->scan_len = (int64_t)kv * L->nseg + 1;
+  int64_t longest = L->scan_len;
+  if (n_in + 1 > longest) longest = n_in + 1;
+  if (n_out + 1 > longest) longest = n_out + 1;
+  int64_t o = 0;
+  L->off_table = o;
+  o += pce_align_up(L->slots * 16, 256);
+  L->off_dense = o;
+  o += pce_align_up((int64_t)kv * n_in * 4, 256);
+  L->off_seg = o;
+  o += pce_align_up(L->scan_len * 4, 256);
+  L->off_scan = o;
+  o += pce_align_up(scan_tmp_ints(longest) * 4, 256);
+  L->off_orank = o;
+  if (want_csr) o += pce_align_up((int64_t)kv * n_out * 4, 256);
+  L->off_irank = o;
+  if (want_csr) o += pce_align_up((int64_t)kv * n_in * 4, 256);
+  L->total = o;
+}
+
+// One lane per input row.  For every offset kp the lane asks which output row the input reaches:
+//   submanifold: out = in - d(kp)          (pair (i,o,kp) <=> coords[i] == coords[o] + d(kp))
+//   strided:     out = (in - d(kp) + pad) / stride when it divides
+// dense[kp*n_in + i] = output row or -1; segcnt[kp*nseg + seg] = hits among the 64 rows of a wave.
+__global__ void __launch_bounds__(256) kmap_query_kernel(const int4 *__restrict__ in_coords, long long n_in,
+                                                         long long n_out, GeomDev g,
+                                                         const pce_slot_t *__restrict__ table,
+                                                         unsigned long long slots, int *__restrict__ dense,
+                                                         int *__restrict__ segcnt, long long nseg,
+                                                         int *__restrict__ nbr_out, int *status) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  long long seg = i >> 6;
+  bool live = i < n_in;
+  int4 c = live ? in_coords[i] : make_int4(0, 0, 0, 0);
+  if (live && !pce_coord_ok(c.x, c.y, c.z, c.w)) {
+    status[0] = 1;
+    live = false;
+  }
+  OffsetIter it;
+  it.init();
+  for (int kp = 0; kp < g.kv; ++kp, it.next(g)) {
+    int res = -1;
+    if (g.subm && kp == g.mid) {
+      if (nbr_out && live) nbr_out[(long long)kp * n_out + i] = (int)i;
+    } else if (live) {
+      int ox, oy, oz;
+      bool ok = true;
+      if (g.subm) {
+        ox = c.y - it.dx(g);
+        oy = c.z - it.dy(g);
+        oz = c.w - it.dz(g);
+      } else {
+        ok = strided_axis(c.y, it.dx(g), g.pad[0], g.stride[0], g.cmin[0], g.cmax[0], &ox);
+        ok &= strided_axis(c.z, it.dy(g), g.pad[1], g.stride[1], g.cmin[1], g.cmax[1], &oy);
+        ok &= strided_axis(c.w, it.dz(g), g.pad[2], g.stride[2], g.cmin[2], g.cmax[2], &oz);
+      }
+      if (ok) res = table_find(table, slots, pce_pack_key(c.x, ox, oy, oz));
+    }
+    if (i < n_in) dense[(long long)kp * n_in + i] = res;
+    unsigned long long bal = __ballot(res >= 0);
+    if (__lane_id() == 0 && seg < nseg) segcnt[(long long)kp * nseg + seg] = __popcll(bal);
+  }
+}
+
+// segoff = exclusive scan of segcnt in (kp, segment) order = position of the segment's first pair.
+__global__ void __launch_bounds__(256) kmap_fill_kernel(long long n_in, long long n_out, int kv,
+                                                        const int *__restrict__ dense, const int *__restrict__ segoff,
+                                                        long long nseg, int *__restrict__ imap,
+                                                        int *__restrict__ omap, int *__restrict__ irank,
+                                                        int *__restrict__ orank, int *__restrict__ nbr_out,
+                                                        int want_csr, int *status) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  long long seg = i >> 6;
+  bool live = i < n_in;
+  for (int kp = 0; kp < kv; ++kp) {
+    int v = live ? dense[(long long)kp * n_in + i] : -1;
+    unsigned long long bal = __ballot(v >= 0);
+    int rank = -1;
+    if (v >= 0) {
+      int p = segoff[(long long)kp * nseg + seg] + __popcll(bal & lanemask_lt());
+      imap[p] = (int)i;
+      omap[p] = v;
+      if (nbr_out) nbr_out[(long long)kp * n_out + v] = (int)i;
+      if (want_csr) {
+        rank = p - segoff[(long long)kp * nseg];
+        if (rank >= PCE_CSR_CODE) status[2] = 1;
+        orank[(long long)kp * n_out + v] = rank;
+      }
+    }
+    if (want_csr && live) irank[(long long)kp * n_in + i] = rank;
+  }
+}
+
+__global__ void kmap_offsets_kernel(const int *__restrict__ segoff, long long nseg, int kv, int *knnz, int *kpos,
+                                    int *qkpos) {
+  // kpos[kp] = first pair of offset kp; then the scan of counts rounded up to the tile height
+  // (backend/hash.cuh:478-497)
+  for (int kp = threadIdx.x; kp <= kv; kp += blockDim.x) {
+    int a = segoff[(long long)kp * nseg];
+    kpos[kp] = a;
+    if (kp < kv) knnz[kp] = segoff[(long long)(kp + 1) * nseg] - a;
+  }
+  if (threadIdx.x == 0) {
+    int q = 0;
+    qkpos[0] = 0;
+    for (int kp = 0; kp < kv; ++kp) {
+      int c = segoff[(long long)(kp + 1) * nseg] - segoff[(long long)kp * nseg];
+      q += (c + PCE_QUANTUM - 1) / PCE_QUANTUM * PCE_QUANTUM;
+      qkpos[kp + 1] = q;
+    }
+  }
+}
+
+// rank[kp*n + r] >= 0 marks an entry of row r; count them (mapping_counter, backend/hash.cuh:422-437)
+__global__ void __launch_bounds__(256) csr_count_kernel(const int *__restrict__ rank, long long n, int kv,
+                                                        int *__restrict__ cnt) {
+  long long r = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (r > n) return;
+  int c = 0;
+  if (r < n)
+    for (int kp = 0; kp < kv; ++kp) c += rank[(long long)kp * n + r] >= 0;
+  cnt[r] = c;  // cnt[n] = 0 receives the total after the scan
+}
+
+__global__ void __launch_bounds__(256) csr_fill_kernel(const int *__restrict__ rank, long long n, int kv,
+                                                       const int *__restrict__ csr, int *__restrict__ code) {
+  long long r = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= n) return;
+  int pos = csr[r];
+  for (int kp = 0; kp < kv; ++kp) {
+    int rk = rank[(long long)kp * n + r];
+    if (rk >= 0) code[pos++] = kp * PCE_CSR_CODE + rk;
+  }
+}
+
+extern "C" int64_t pce_kmap_workspace_bytes(int64_t n_in, int64_t n_out, int32_t kv, int32_t want_csr) {
+  KmapLayout L;
+  kmap_layout(n_in, n_out, kv, want_csr, &L);
+  return L.total;
+}
+
+extern "C" int pce_kmap_build(const int32_t *in_coords, int64_t n_in, const int32_t *out_coords, int64_t n_out,
+                              const pce_geom_t *g, void *ws, int64_t ws_bytes, int32_t *imap, int32_t *omap,
+                              int32_t *knnz, int32_t *kpos, int32_t *qkpos, int32_t *icsr, int32_t *icode,
+                              int32_t *ocsr, int32_t *ocode, int32_t *nbr_out, int32_t *nbr_in, int32_t *status,
+                              pce_stream_t stream) {
+  hipStream_t s = (hipStream_t)stream;
+  GeomDev gd;
+  int rc = make_geom(g, &gd);
+  if (rc) return rc;
+  if (!in_coords || !out_coords || !ws || !imap || !omap || !knnz || !kpos || !qkpos || !status)
+    PCE_FAIL(PCE_EINVAL, "pce_kmap_build: null pointer");
+  int ncsr = (icsr != nullptr) + (icode != nullptr) + (ocsr != nullptr) + (ocode != nullptr);
+  if (ncsr != 0 && ncsr != 4) PCE_FAIL(PCE_EINVAL, "pce_kmap_build: pass all four CSR outputs or none");
+  int want_csr = ncsr == 4;
+  if (n_in <= 0 || n_out <= 0) PCE_FAIL(PCE_EINVAL, "pce_kmap_build: empty tensor (n_in=%lld, n_out=%lld)", (long long)n_in, (long long)n_out);
+  if (gd.subm && n_in != n_out) PCE_FAIL(PCE_EINVAL, "pce_kmap_build: submanifold layer needs n_in == n_out");
+  if ((int64_t)gd.kv * n_in >= (1ll << 31) || (int64_t)gd.kv * n_out >= (1ll << 31))
+    PCE_FAIL(PCE_ECAPACITY, "pce_kmap_build: kv*n exceeds int32 pair indexing");
+  KmapLayout L;
+  kmap_layout(n_in, n_out, gd.kv, want_csr, &L);
+  if (ws_bytes < L.total) PCE_FAIL(PCE_EWORKSPACE, "pce_kmap_build: workspace %lld < %lld", (long long)ws_bytes, (long long)L.total);
+  char *w = (char *)ws;
+  pce_slot_t *table = (pce_slot_t *)(w + L.off_table);
+  int *dense = nbr_in ? nbr_in : (int *)(w + L.off_dense);  // the input-major table is the probe result itself
+  int *irank = want_csr ? (int *)(w + L.off_irank) : nullptr;
+  int *seg = (int *)(w + L.off_seg);
+  int *scan_tmp = (int *)(w + L.off_scan);
+  int *orank = want_csr ? (int *)(w + L.off_orank) : nullptr;
+
+  // 1. table over the output coordinates (for a submanifold layer these are the input coordinates)
+  if ((rc = table_clear(table, L.slots, s))) return rc;
+  hipLaunchKernelGGL(hash_insert_kernel, dim3((unsigned)pce_div_up(n_out, 256)), dim3(256), 0, s, table,
+                     (unsigned long long)L.slots, (const int4 *)out_coords, (long long)n_out, status);
+  PCE_LAUNCH_CHECK("hash_insert");
+  if (nbr_out && (rc = fill_u32(nbr_out, (int64_t)gd.kv * n_out, 0xFFFFFFFFu, s))) return rc;
+  if (want_csr && (rc = fill_u32(orank, (int64_t)gd.kv * n_out, 0xFFFFFFFFu, s))) return rc;
+  // 2. probe, per-wave counts
+  unsigned blocks = (unsigned)pce_div_up(n_in, 256);
+  hipLaunchKernelGGL(kmap_query_kernel, dim3(blocks), dim3(256), 0, s, (const int4 *)in_coords, (long long)n_in,
+                     (long long)n_out, gd, (const pce_slot_t *)table, (unsigned long long)L.slots, dense, seg,
+                     (long long)L.nseg, nbr_out, status);
+  PCE_LAUNCH_CHECK("kmap_query");
+  // 3. positions
+  if ((rc = fill_u32(seg + (L.scan_len - 1), 1, 0u, s))) return rc;
+  if ((rc = scan_exclusive(seg, L.scan_len, scan_tmp, s))) return rc;
+  hipLaunchKernelGGL(kmap_offsets_kernel, dim3(1), dim3(128), 0, s, (const int *)seg, (long long)L.nseg, gd.kv, knnz,
+                     kpos, qkpos);
+  PCE_LAUNCH_CHECK("kmap_offsets");
+  // 4. pair lists in (offset, input row) order
+  hipLaunchKernelGGL(kmap_fill_kernel, dim3(blocks), dim3(256), 0, s, (long long)n_in, (long long)n_out, gd.kv,
+                     (const int *)dense, (const int *)seg, (long long)L.nseg, imap, omap, irank, orank, nbr_out, want_csr,
+                     status);
+  PCE_LAUNCH_CHECK("kmap_fill");
+  // 5. CSR-coded view
+  if (want_csr) {
+    hipLaunchKernelGGL(csr_count_kernel, dim3((unsigned)pce_div_up(n_in + 1, 256)), dim3(256), 0, s, (const int *)irank,
+                       (long long)n_in, gd.kv, icsr);
+    PCE_LAUNCH_CHECK("csr_count(in)");
+    if ((rc = scan_exclusive(icsr, n_in + 1, scan_tmp, s))) return rc;
+    hipLaunchKernelGGL(csr_fill_kernel, dim3((unsigned)pce_div_up(n_in, 256)), dim3(256), 0, s, (const int *)irank,
+                       (long long)n_in, gd.kv, (const int *)icsr, icode);
+    PCE_LAUNCH_CHECK("csr_fill(in)");
+    hipLaunchKernelGGL(csr_count_kernel, dim3((unsigned)pce_div_up(n_out + 1, 256)), dim3(256), 0, s, (const int *)orank,
+                       (long long)n_out, gd.kv, ocsr);
+    PCE_LAUNCH_CHECK("csr_count(out)");
+    if ((rc = scan_exclusive(ocsr, n_out + 1, scan_tmp, s))) return rc;
+    hipLaunchKernelGGL(csr_fill_kernel, dim3((unsigned)pce_div_up(n_out, 256)), dim3(256), 0, s, (const int *)orank,
+                       (long long)n_out, gd.kv, (const int *)ocsr, ocode);
+    PCE_LAUNCH_CHECK("csr_fill(out)");
+  }
+  return PCE_OK;
+}

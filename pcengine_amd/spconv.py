@@ -1,0 +1,175 @@
+"""conv3d: sparse 3-D convolution with the reference's module interface
+(script/spconv.py:15-106) over the MI355X backend.
+
+Differences a user can see, all supersets of the reference:
+* ``dataflow='auto'|'fod'|'gms'|'os'`` constructor argument (and the PCENGINE_DATAFLOW
+  environment variable) on top of the reference's ``init_tag`` list.  A tensor whose
+  ``init_tag`` starts with 'D1' / 'D2' pins the next newly built map to gather-GEMM-scatter /
+  fetch-on-demand exactly as in the reference (script/spconv.py:343, 388); the default tag
+  ('end') lets the selector decide per layer.
+* every strided layer uses the generic output-coordinate rule, also when stride == kernel size.
+* forward only.
+"""
+from __future__ import annotations
+
+import math
+import os
+from typing import List, Optional, Union
+
+import numpy as np
+import torch
+import torch.nn as nn
+
+from . import backend
+from .backend import DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS
+from .sptensor import spTensor
+from .utils import conv_info_decoder, conv_info_encoder, output_stride_compute
+
+_UNIT = conv_info_encoder([1, 1, 1])
+_DATAFLOWS = {"fod": DATAFLOW_FOD, "d2": DATAFLOW_FOD, "gms": DATAFLOW_GMS, "d1": DATAFLOW_GMS, "os": DATAFLOW_OS}
+
+# one record per executed layer when enabled: (N_in, N_out, M, C_in, C_out, dataflow)
+layer_log: Optional[list] = None
+
+
+def _triple(v, what: str) -> List[int]:
+    if isinstance(v, int):
+        return [v, v, v]
+    if isinstance(v, list):
+        return v
+    raise NotImplementedError(f"{what} must be an int or a list of three ints")
+
+
+class conv3d(nn.Module):
+
+    def __init__(self, in_channels: int = 16, out_channels: int = 32, kernel_size: Union[int, List[int]] = 3,
+                 stride: Union[int, List[int]] = 1, padding: Union[int, List[int]] = 0, bias: bool = False,
+                 transposed: bool = False, tc_mode: bool = True, dataflow: str = "auto") -> None:
+        super().__init__()
+        self.in_channels = in_channels
+        self.out_channels = out_channels
+        self.transposed = transposed
+        self.kernel_size = _triple(kernel_size, "kernel_size")
+        self.kernel_size_code = conv_info_encoder(self.kernel_size)
+        self.kernel_volume = int(np.prod(self.kernel_size, dtype=int))
+        self.stride = _triple(stride, "stride")
+        self.stride_code = conv_info_encoder(self.stride)
+        self.padding = _triple(padding, "padding")
+        self.padding_code = conv_info_encoder(self.padding)
+        self.tensorcore = tc_mode
+        if dataflow != "auto" and dataflow.lower() not in _DATAFLOWS:
+            raise NotImplementedError(f"unknown dataflow {dataflow!r}")
+        self.dataflow = dataflow.lower()
+        shape = (self.kernel_volume, in_channels, out_channels) if self.kernel_volume > 1 else (in_channels, out_channels)
+        self.kernel = nn.Parameter(torch.zeros(shape))
+        self.bias = nn.Parameter(torch.zeros((out_channels,))) if bias else None
+        self.reset_parameters()
+
+    def extra_repr(self) -> str:
+        s = f"{self.in_channels}, {self.out_channels}, kernel_size={self.kernel_size}"
+        if self.stride_code != _UNIT:
+            s += f", stride={self.stride}"
+        if self.bias is None:
+            s += ", bias=False"
+        if self.transposed:
+            s += ", transposed=True"
+        return s
+
+    def reset_parameters(self) -> None:
+        # U(-1/sqrt(C_out*kv), +1/sqrt(C_out*kv)) for kernel and bias (script/spconv.py:101-106)
+        bound = 1.0 / math.sqrt(self.out_channels * self.kernel_volume)
+        with torch.no_grad():
+            self.kernel.uniform_(-bound, bound)
+            if self.bias is not None:
+                self.bias.uniform_(-bound, bound)
+
+    def forward(self, input: spTensor) -> spTensor:
+        return conv_func(input=input, in_channel=self.in_channels, out_channel=self.out_channels, kernel=self.kernel,
+                         kernel_size_code=self.kernel_size_code, stride_code=self.stride_code,
+                         padding_code=self.padding_code, bias=self.bias, transposed=self.transposed,
+                         tensorcore=self.tensorcore, dataflow=self.dataflow)
+
+
+def _pick_dataflow(km: backend.KernelMap, requested: str, c_in: int, c_out: int, dtype, transposed: bool) -> int:
+    env = os.environ.get("PCENGINE_DATAFLOW", "").lower()
+    if env in _DATAFLOWS:
+        return _DATAFLOWS[env]
+    if requested in _DATAFLOWS:
+        return _DATAFLOWS[requested]
+    if km.tag == "D1":
+        return DATAFLOW_GMS
+    if km.tag == "D2":
+        return DATAFLOW_FOD
+    return backend.select_dataflow(km, c_in, c_out, dtype, transposed)
+
+
+def _run(input: spTensor, km: backend.KernelMap, kernel, in_channel, out_channel, transposed, dataflow) -> torch.Tensor:
+    feats = input.feats
+    if kernel.dtype != feats.dtype:
+        kernel = kernel.to(feats.dtype)
+    df = _pick_dataflow(km, dataflow, in_channel, out_channel, feats.dtype, transposed)
+    out = backend.conv_forward(feats, kernel.detach(), km, df, transposed=transposed, buffer=input.buffer)
+    if layer_log is not None:
+        layer_log.append((feats.shape[0], out.shape[0], km.M, in_channel, out_channel, df))
+    return out
+
+
+def conv_func(input: spTensor, in_channel, out_channel, kernel, kernel_size_code, stride_code, padding_code, bias,
+              transposed, tensorcore, dataflow: str = "auto") -> spTensor:
+    """Map cache lookup / build, dataflow dispatch, bias, metadata propagation
+    (script/spconv.py:291-464)."""
+    if kernel_size_code == _UNIT and stride_code == _UNIT:
+        # 1x1 stride 1: plain matrix product, coordinates unchanged, no map (script/spconv.py:297-304)
+        w = kernel if kernel.dtype == input.feats.dtype else kernel.to(input.feats.dtype)
+        out_feats = backend.dense_forward(input.feats, w.detach())
+        if bias is not None:
+            out_feats += bias.to(out_feats.dtype)
+        return input._like(out_feats)
+
+    if transposed:
+        # replay the cached strided map backwards (script/spconv.py:306-329)
+        output_stride = output_stride_compute(stride_code, input.stride, 1)
+        km = input.kmaps.get((kernel_size_code, output_stride, stride_code))
+        if km is None:
+            raise KeyError("transposed conv3d found no cached map for this (kernel, stride): "
+                           "the matching strided conv3d must run first on the same tensor family")
+        out_coords = input.cbook[output_stride]
+        out_feats = _run(input, km, kernel, in_channel, out_channel, True, dataflow)
+        if bias is not None:
+            out_feats += bias.to(out_feats.dtype)
+        output = spTensor(feats=out_feats, coords=out_coords, buffer=input.buffer, batchsize=input.batchsize,
+                          stride=output_stride, init_tag=input.init_tag, coords_max=input.coords_max,
+                          coords_min=input.coords_min)
+        output.kmaps, output.cbook = input.kmaps, input.cbook
+        return output
+
+    output_stride = output_stride_compute(stride_code, input.stride, 0)
+    key = (kernel_size_code, input.stride, stride_code)
+    km = input.kmaps.get(key)
+    subm = stride_code == _UNIT
+    coords_max = list(input.coords_max[:3])
+    coords_min = list(input.coords_min[:3])
+    ks = conv_info_decoder(kernel_size_code)
+    stride = conv_info_decoder(stride_code)
+    pad = conv_info_decoder(padding_code)
+    if not subm:
+        coords_max = backend.strided_coords_max(input.coords_max, ks, stride, pad)   # script/spconv.py:358-360
+    if km is None:
+        tag = input.init_tag[0] if input.init_tag else 'end'
+        if tag not in ('D1', 'D2', 'end', 'auto'):
+            raise NotImplementedError(f"unknown init_tag entry {tag!r}")
+        km = backend.build_kernel_map(input.coords, ks, stride, pad, coords_min, coords_max, subm,
+                                      want_csr=(tag == 'D1'), want_nbr_out=(tag in ('end', 'auto')))
+        km.tag = tag if tag in ('D1', 'D2') else 'auto'
+        input.kmaps[key] = km
+        input.cbook[output_stride] = km.out_coords
+        if tag in ('D1', 'D2'):
+            input.init_tag = input.init_tag[1:]
+    input.cbook.setdefault(input.stride, input.coords)
+    out_feats = _run(input, km, kernel, in_channel, out_channel, False, dataflow)
+    if bias is not None:
+        out_feats += bias.to(out_feats.dtype)
+    output = spTensor(feats=out_feats, coords=km.out_coords, buffer=input.buffer, batchsize=input.batchsize,
+                      stride=output_stride, init_tag=input.init_tag, coords_max=coords_max, coords_min=coords_min)
+    output.kmaps, output.cbook = input.kmaps, input.cbook
+    return output

@@ -1,0 +1,140 @@
+"""Forward-value parity of the three HIP dataflows with the float64 oracle, through the C ABI.
+Bars: rel-L2 <= 1e-3 for fp16 storage (fp32 accumulate), <= 1e-5 for fp32."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+from pcengine_amd import backend, synth
+from pcengine_amd.backend import DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS
+from tests.util import DEV, TOL, gpu_map, rounded
+
+pytestmark = pytest.mark.gpu
+
+FLOWS = [DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS]
+CHANNELS = [(16, 16), (64, 64), (4, 32), (32, 20), (96, 96), (5, 7), (64, 160), (130, 40)]
+
+
+def _case(coords, ks, stride, pad, c_in, c_out, dtype, seed=0):
+    kv = ks[0] * ks[1] * ks[2]
+    f = synth.features(seed, len(coords), c_in)
+    w = synth.weights(seed, kv, c_in, c_out)
+    ref_map = orc.kernel_map(coords, ks, stride, pad)
+    want = orc.conv_forward(rounded(f, dtype), rounded(w, dtype), ref_map, ks)
+    fd = torch.as_tensor(f, device=DEV).to(dtype)
+    wd = torch.as_tensor(w, device=DEV).to(dtype)
+    return fd, wd, ref_map, want
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("c_in,c_out", CHANNELS)
+def test_submanifold_all_dataflows(c_in, c_out, dtype):
+    coords = synth.random_cloud(seed=41, n=9000, extent=22, batches=2)
+    fd, wd, ref_map, want = _case(coords, (3, 3, 3), (1, 1, 1), (0, 0, 0), c_in, c_out, dtype)
+    km = gpu_map(coords, (3, 3, 3), want_csr=True, want_nbr_in=True)
+    for flow in FLOWS:
+        out = backend.conv_forward(fd, wd, km, flow)
+        err = orc.rel_l2(out.double().cpu().numpy(), want)
+        assert err <= TOL[dtype], (flow, err)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("ks,stride,pad", [((2, 2, 2), (2, 2, 2), (0, 0, 0)), ((3, 3, 3), (2, 2, 2), (1, 1, 1)),
+                                           ((2, 3, 1), (2, 1, 1), (0, 1, 0))])
+def test_strided_then_transposed_all_dataflows(ks, stride, pad, dtype):
+    coords = synth.random_cloud(seed=42, n=7000, extent=20, batches=2)
+    c_in, c_out = 64, 128
+    fd, wd, ref_map, want = _case(coords, ks, stride, pad, c_in, c_out, dtype)
+    km = gpu_map(coords, ks, stride, pad, want_csr=True, want_nbr_in=True)
+    kv = km.kv
+    wt = synth.weights(9, kv, c_out, c_in)
+    wtd = torch.as_tensor(wt, device=DEV).to(dtype)
+    for flow in FLOWS:
+        out = backend.conv_forward(fd, wd, km, flow)
+        assert orc.rel_l2(out.double().cpu().numpy(), want) <= TOL[dtype], flow
+        # transposed layer back onto the input coordinates, fed with the GPU's own output
+        back = backend.conv_forward(out, wtd, km, flow, transposed=True)
+        want_t = orc.conv_forward(out.double().cpu().numpy(), rounded(wt, dtype), ref_map, ks, transposed=True)
+        assert back.shape == (len(coords), c_in)
+        assert orc.rel_l2(back.double().cpu().numpy(), want_t) <= TOL[dtype], flow
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_dense_1x1(dtype):
+    f = synth.features(3, 5001, 96)
+    w = synth.weights(3, 1, 96, 20)[0]
+    out = backend.dense_forward(torch.as_tensor(f, device=DEV).to(dtype), torch.as_tensor(w, device=DEV).to(dtype))
+    want = rounded(f, dtype) @ rounded(w, dtype)
+    assert orc.rel_l2(out.double().cpu().numpy(), want) <= TOL[dtype]
+
+
+def test_config1_fp32_c16():
+    coords = synth.sphere_plane_cloud()
+    fd, wd, ref_map, want = _case(coords, (3, 3, 3), (1, 1, 1), (0, 0, 0), 16, 16, torch.float32, seed=1)
+    km = gpu_map(coords, (3, 3, 3), want_csr=True)
+    for flow in FLOWS:
+        out = backend.conv_forward(fd, wd, km, flow)
+        assert orc.rel_l2(out.double().cpu().numpy(), want) <= 1e-5, flow
+
+
+def test_config2_fp16_c64_full_size():
+    coords = synth.lidar_cloud()
+    fd, wd, ref_map, want = _case(coords, (3, 3, 3), (1, 1, 1), (0, 0, 0), 64, 64, torch.float16, seed=2)
+    km = gpu_map(coords, (3, 3, 3), want_csr=True)
+    outs = [backend.conv_forward(fd, wd, km, flow) for flow in FLOWS]
+    for flow, out in zip(FLOWS, outs):
+        assert orc.rel_l2(out.double().cpu().numpy(), want) <= 1e-3, flow
+    # linearity in the features holds at any size: conv(2x) == 2 conv(x) exactly in fp16 storage
+    twice = backend.conv_forward(fd * 2, wd, km, DATAFLOW_OS)
+    assert torch.equal(twice, outs[2] * 2)
+
+
+def test_reference_named_entry_points_d2_and_d1():
+    """Drive the five pybind names the way the reference front end does (script/spconv.py:343-431)."""
+    coords = synth.random_cloud(seed=44, n=6000, extent=18)
+    n = len(coords)
+    kv, ci, co = 27, 32, 48
+    enc = lambda v: 94273 * v[0] + 311 * v[1] + v[2]
+    c = torch.as_tensor(coords, device=DEV)
+    f = synth.features(4, n, ci)
+    w = synth.weights(4, kv, ci, co)
+    fd = torch.as_tensor(f, device=DEV).half()
+    wd = torch.as_tensor(w, device=DEV).half()
+    ref_map = orc.kernel_map(coords, (3, 3, 3))
+    want = orc.conv_forward(rounded(f, torch.float16), rounded(w, torch.float16), ref_map, (3, 3, 3))
+    cmax = coords[:, 1:].max(0).tolist()
+    # fetch-on-demand protocol
+    imap = -torch.ones(kv * n, dtype=torch.int, device=DEV)
+    knnz = torch.zeros(kv, dtype=torch.int, device=DEV)
+    kpos = torch.zeros(kv + 1, dtype=torch.int, device=DEV)
+    qkpos = torch.zeros(kv + 1, dtype=torch.int, device=DEV)
+    oc = backend.mapping_d2_cuda(c, 1, enc([3, 3, 3]), kv, ci, co, enc([1, 1, 1]), enc([1, 1, 1]), enc([0, 0, 0]),
+                                 0, 0, 0, *cmax, imap, knnz, kpos, qkpos, True)
+    assert oc is c
+    nz = torch.nonzero(imap != -1)
+    omap = imap[nz]
+    imap2 = (nz % n).int()
+    assert np.array_equal(imap2.flatten().cpu().numpy(), ref_map.imap) and np.array_equal(omap.flatten().cpu().numpy(), ref_map.omap)
+    qsum = int(qkpos[-1].cpu())
+    out = torch.zeros((n, co), dtype=torch.half, device=DEV)
+    backend.conv_fwd_d2_cuda(fd, wd, enc([3, 3, 3]), qsum, out, kpos, qkpos, imap2.contiguous(), omap.contiguous(), True, False)
+    assert orc.rel_l2(out.double().cpu().numpy(), want) <= 1e-3
+    # gather-GEMM-scatter protocol, with the reference's allocation sizes (kpos has kv entries)
+    imap = -torch.ones(n * kv, dtype=torch.int, device=DEV)
+    omap = -torch.ones(n * kv * 8, dtype=torch.int, device=DEV)
+    knnz = torch.zeros(kv, dtype=torch.int, device=DEV)
+    kpos = torch.zeros(kv, dtype=torch.int, device=DEV)
+    qkpos = torch.zeros(kv + 1, dtype=torch.int, device=DEV)
+    icsr = torch.zeros(n + 2, dtype=torch.int, device=DEV)
+    ocsr = torch.zeros((n + 2) * 8, dtype=torch.int, device=DEV)
+    backend.mapping_d1_cuda(c, enc([3, 3, 3]), kv, ci, co, enc([1, 1, 1]), enc([1, 1, 1]), enc([0, 0, 0]), 0, 0, 0, *cmax,
+                            imap, omap, icsr, ocsr, knnz, kpos, qkpos, True)
+    qsum = int(qkpos[-1].cpu())
+    buffer = torch.empty(qsum * (ci + co), dtype=torch.half, device=DEV)
+    out = torch.zeros((n, co), dtype=torch.half, device=DEV)
+    backend.conv_fwd_d1_cuda(fd, wd, enc([3, 3, 3]), qsum, out, kpos, qkpos, imap, omap, icsr, ocsr, buffer, True, 1)
+    assert orc.rel_l2(out.double().cpu().numpy(), want) <= 1e-3
+    with pytest.raises(ValueError):     # backend/spconv.cu:38-40
+        backend.conv_fwd_d2_cuda(fd[:, :16].contiguous(), wd, enc([3, 3, 3]), qsum, out, kpos, qkpos, imap, omap, True, False)
+    with pytest.raises(NotImplementedError):
+        backend.conv_bwd_d1_cuda()

@@ -1,0 +1,127 @@
+"""CPU-side checks: the C-ABI library loads and exports what include/pcengine_amd.h declares,
+the host logic of the front end, and the loud failure without a GPU.  No compute calls."""
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import pcengine_amd as pe
+from pcengine_amd import _lib, backend
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "pcengine_amd.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(pce_[a-z0-9_]+)\s*\(", header))
+    assert declared, "no declarations found"
+    lib = _lib.load()
+    for name in sorted(declared):
+        assert hasattr(lib, name), f"{name} is declared but not exported"
+    assert declared == set(_lib.exported_names())
+    assert lib.pce_version() >= 100
+
+
+def test_pure_host_entry_points():
+    lib = _lib.load()
+    assert lib.pce_hash_slots(1) == 8 and lib.pce_hash_slots(20000) == 65536 and lib.pce_hash_slots(150000) == 524288
+    assert lib.pce_hash_table_bytes(150000) == 524288 * 16
+    g = _lib.Geom.make((2, 2, 2), (2, 2, 2), (0, 0, 0), (0, 0, 0), (10, 10, 10), False)
+    assert lib.pce_outcoords_workspace_bytes(1000, g) > 0
+    bad = _lib.Geom.make((0, 2, 2), (2, 2, 2), (0, 0, 0), (0, 0, 0), (10, 10, 10), False)
+    assert lib.pce_outcoords_workspace_bytes(1000, bad) == -1
+    assert lib.pce_kmap_workspace_bytes(1000, 1000, 27, 1) > lib.pce_kmap_workspace_bytes(1000, 1000, 27, 0)
+    assert lib.pce_conv_fod_workspace_bytes(1000, 64, _lib.PCE_F16) == 1000 * 64 * 4
+    assert lib.pce_conv_fod_workspace_bytes(1000, 64, _lib.PCE_F32) == 0
+
+
+def test_argument_validation_needs_no_gpu():
+    lib = _lib.load()
+    assert lib.pce_conv_fwd_fod(None, None, None, 0, 1, 1, 1, 1, 1, -1, None, None, None, None, 0, None, 0, None) == _lib.PCE_EINVAL
+    with pytest.raises(ValueError):
+        _lib.check(_lib.PCE_EINVAL)
+    one = 1
+    assert lib.pce_conv_fwd_fod(one, one, one, 0, 10, 10, 4, 4, 27, 13, one, one, one, one, 100, one, 1 << 20, None) == _lib.PCE_EINVAL  # qsum % 128
+    assert lib.pce_conv_fwd_fod(one, one, one, 0, 10, 12, 4, 4, 27, 13, one, one, one, one, 128, one, 1 << 20, None) == _lib.PCE_EINVAL  # centre needs n_in == n_out
+    assert lib.pce_conv_fwd_fod(one, one, one, 0, 10, 10, 4, 4, 27, 13, one, one, one, one, 128, one, 16, None) == _lib.PCE_EWORKSPACE
+    assert lib.pce_conv_fwd_gms(one, one, one, 0, 10, 10, 4, 4, 27, 13, one, one, one, one, one, one, 128, one, 10, None) == _lib.PCE_EWORKSPACE
+    assert lib.pce_conv_fwd_os(one, one, one, 7, 10, 10, 4, 4, 27, one, None) == _lib.PCE_EINVAL      # dtype
+
+
+def test_selector_is_monotone_in_density():
+    lib = _lib.load()
+    n = 100000
+    picks = [lib.pce_select_dataflow(n, n, int(rho * n), 64, 64, 27, 0) for rho in (0.1, 0.5, 1.0, 3.0, 8.0, 20.0)]
+    assert picks[0] == _lib.DATAFLOW_FOD and picks[-1] == _lib.DATAFLOW_OS
+    order = {_lib.DATAFLOW_FOD: 0, _lib.DATAFLOW_GMS: 1, _lib.DATAFLOW_OS: 2}
+    ranks = [order[p] for p in picks]
+    assert ranks == sorted(ranks)
+
+
+def test_codes_and_strides():
+    assert pe.conv_info_encoder([1, 1, 1]) == 94585
+    for v in [(1, 1, 1), (2, 2, 2), (3, 1, 5), (8, 8, 8)]:
+        assert pe.conv_info_decoder(pe.conv_info_encoder(list(v))) == v
+        assert backend.decode3(pe.conv_info_encoder(list(v))) == v
+    assert pe.output_stride_compute(pe.conv_info_encoder([2, 2, 2]), pe.conv_info_encoder([2, 2, 2])) == pe.conv_info_encoder([4, 4, 4])
+    assert pe.output_stride_compute(pe.conv_info_encoder([2, 2, 2]), pe.conv_info_encoder([4, 4, 4]), True) == pe.conv_info_encoder([2, 2, 2])
+
+
+def test_quantize_and_collate():
+    rng = np.random.default_rng(0)
+    pts = rng.uniform(0, 1, size=(2000, 3))
+    q, idx, inv = pe.sparse_quantize(pts, 0.1, return_index=True, return_inverse=True)
+    assert q.dtype == np.int32 and len(np.unique(q, axis=0)) == len(q)
+    assert np.array_equal(q[inv], np.floor(pts / 0.1).astype(np.int32))
+    assert np.array_equal(np.floor(pts[idx] / 0.1).astype(np.int32), q)
+    assert (np.diff(pe.ravel_hash(q).astype(np.int64)) > 0).all()     # sorted by the mixed-radix code
+    a = pe.spTensor(torch.ones(len(q), 3), torch.as_tensor(q), None, [0, 0, 0], q.max(0).tolist())
+    b = pe.spTensor(torch.ones(5, 3), torch.as_tensor(q[:5]), None, [0, 0, 0], q.max(0).tolist())
+    x = pe.sparse_collate([a, b])
+    assert x.coords.shape == (len(q) + 5, 4) and x.coords.dtype == torch.int32 and x.batchsize == 2
+    assert x.coords[-1, 0] == 1 and x.coords_min == [0, 0, 0] and x.coords_max == q.max(0).tolist()
+    y = pe.cat([x, x])
+    assert y.feats.shape[1] == 6 and y.kmaps is x.kmaps and y.cbook is x.cbook
+    z = x + x
+    assert torch.equal(z.feats, x.feats * 2) and z.kmaps is x.kmaps
+    assert x.F is x.feats and x.C is x.coords and x.stride == 94585
+
+
+def test_module_construction_and_errors():
+    c = pe.conv3d(4, 8, 3)
+    assert tuple(c.kernel.shape) == (27, 4, 8) and c.bias is None
+    bound = 1 / np.sqrt(8 * 27)
+    assert float(c.kernel.abs().max()) <= bound
+    assert tuple(pe.conv3d(4, 8, 1).kernel.shape) == (4, 8)
+    assert "stride=[2, 2, 2]" in repr(pe.conv3d(4, 8, 2, 2, transposed=True)) and "transposed=True" in repr(pe.conv3d(4, 8, 2, 2, transposed=True))
+    assert set(pe.conv3d(4, 8, 3, bias=True).state_dict()) == {"kernel", "bias"}
+    for kw in ({"kernel_size": (3, 3, 3)}, {"stride": 1.5}, {"padding": "same"}):
+        with pytest.raises(NotImplementedError):
+            pe.conv3d(4, 8, **kw)
+    with pytest.raises(NotImplementedError):
+        pe.conv3d(4, 8, dataflow="magic")
+
+
+def test_no_cpu_compute_path():
+    x = pe.spTensor(torch.zeros(3, 4), torch.zeros(3, 4, dtype=torch.int32), None, [0, 0, 0], [0, 0, 0])
+    with pytest.raises(RuntimeError, match="no CPU compute path"):
+        pe.conv3d(4, 8, 3)(x)
+    with pytest.raises(RuntimeError, match="no CPU compute path"):
+        pe.conv3d(4, 8, 1)(x)
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libpcengine_amd.so")
+    with pytest.raises(_lib.PCEError, match="no other compute path"):
+        _lib.load()
+
+
+def test_scheduler_hint_and_buffer_size():
+    assert pe.init_layer_scheduler({"stride": [1, 1, 2], "in": [4, 32, 32], "out": [32, 32, 64]}) == "simple"
+    assert pe.init_layer_scheduler({"stride": [1, 1, 2], "in": [4, 64, 64], "out": [64, 64, 64]}) == "whole"
+    buf = pe.build_conv_buffer({"in": [4, 8], "out": [8, 16], "kernel": [3, 2]}, 10, torch.float16, "cpu")
+    assert buf.numel() == (8 + 16) * 10 * 16 and buf.dtype == torch.float16
