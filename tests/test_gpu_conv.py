@@ -84,9 +84,10 @@ def test_config2_fp16_c64_full_size():
     outs = [backend.conv_forward(fd, wd, km, flow) for flow in FLOWS]
     for flow, out in zip(FLOWS, outs):
         assert orc.rel_l2(out.double().cpu().numpy(), want) <= 1e-3, flow
-    # linearity in the features holds at any size: conv(2x) == 2 conv(x) exactly in fp16 storage
+    # linearity in the features holds at any size: conv(2x) == 2 conv(x); scaling by two is exact in
+    # fp16 except for results in the subnormal range, whose spacing is 2^-24
     twice = backend.conv_forward(fd * 2, wd, km, DATAFLOW_OS)
-    assert torch.equal(twice, outs[2] * 2)
+    assert torch.allclose(twice.float(), outs[2].float() * 2, rtol=0, atol=2.0 ** -23)
 
 
 def test_reference_named_entry_points_d2_and_d1():
