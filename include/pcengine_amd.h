@@ -44,7 +44,9 @@ enum { PCE_F16 = 0, PCE_F32 = 1 };
 enum {
   PCE_DATAFLOW_FOD = 0, /* fetch-on-demand fused gather-matmul-scatter (reference "D2") */
   PCE_DATAFLOW_GMS = 1, /* gather - grouped GEMM - scatter over a staging buffer (reference "D1") */
-  PCE_DATAFLOW_OS = 2   /* output-stationary fetch-on-demand: no atomics, no staging buffer */
+  PCE_DATAFLOW_OS = 2,  /* output-stationary fetch-on-demand: no atomics, no staging buffer */
+  PCE_DATAFLOW_FDS = 3  /* fetch-on-demand with deferred scatter: pair tiles write partial rows to a
+                           staging buffer, the centre GEMM's epilogue sums them per output row */
 };
 
 #define PCE_QUANTUM 128        /* rows per tile of the pair list; qkpos granularity (backend/hash.cu:203-205) */
@@ -65,6 +67,11 @@ typedef struct pce_geom {
 
 int pce_version(void);
 const char *pce_last_error(void);
+
+/* Measurement aid: bit i of the mask enables stage i of the forward entry points below
+ * (0: centre GEMM or zero-fill, 1: pair / tile kernel, 2: convert or scatter, 3: gather), so a
+ * benchmark can time one kernel of a dataflow alone.  Default: all stages.  Process-wide. */
+void pce_set_stage_mask(uint32_t mask);
 
 /* ---- coordinate hash table: open addressing on the packed (b,x,y,z) 64-bit key ------------- */
 
@@ -129,10 +136,18 @@ int pce_kmap_build(const int32_t *in_coords_dev, int64_t n_in, const int32_t *ou
  * For a transposed layer pass the map with the roles swapped (imap<->omap, icsr<->ocsr), as the
  * reference front end does (script/spconv.py:142-151, 236-244). */
 
+/* fp16 weights can be handed over a second time in the order the kernels stage them into LDS
+ * (pce_pack_weights, once per weight tensor); every forward entry point takes that copy as
+ * `weight_packed`, or NULL to stage from the row-major tensor.  fp32 has no packed form. */
+int64_t pce_packed_weight_bytes(int32_t dtype, int32_t kv, int32_t c_in, int32_t c_out);
+int pce_pack_weights(const void *weight, int32_t dtype, int32_t kv, int32_t c_in, int32_t c_out,
+                     void *packed_dev, pce_stream_t stream);
+
 /* Fetch-on-demand: pairs (imap, omap, kpos, qkpos) and qsum = qkpos[kv] on the host.
  * fp16 needs an fp32 accumulation scratch of pce_conv_fod_workspace_bytes(); fp32 needs none. */
 int64_t pce_conv_fod_workspace_bytes(int64_t n_out, int32_t c_out, int32_t dtype);
-int pce_conv_fwd_fod(const void *in_feats, const void *weight, void *out_feats, int32_t dtype,
+int pce_conv_fwd_fod(const void *in_feats, const void *weight, const void *weight_packed,
+                     void *out_feats, int32_t dtype,
                      int64_t n_in, int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv,
                      int32_t mid, const int32_t *imap_dev, const int32_t *omap_dev,
                      const int32_t *kpos_dev, const int32_t *qkpos_dev, int64_t qsum,
@@ -140,24 +155,41 @@ int pce_conv_fwd_fod(const void *in_feats, const void *weight, void *out_feats, 
 
 /* Gather - GEMM - scatter: CSR-coded map; `buffer` holds qsum*(c_in+c_out) elements of dtype
  * (first qsum*c_in gathered inputs, then the GEMM outputs; backend/spconv.cu:121). */
-int pce_conv_fwd_gms(const void *in_feats, const void *weight, void *out_feats, int32_t dtype,
+int pce_conv_fwd_gms(const void *in_feats, const void *weight, const void *weight_packed,
+                     void *out_feats, int32_t dtype,
                      int64_t n_in, int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv,
                      int32_t mid, const int32_t *icsr_dev, const int32_t *icode_dev,
                      const int32_t *ocsr_dev, const int32_t *ocode_dev, const int32_t *kpos_dev,
                      const int32_t *qkpos_dev, int64_t qsum, void *buffer_dev,
                      int64_t buffer_elems, pce_stream_t stream);
 
+/* Fetch-on-demand with deferred scatter: the pair list gives the gather side (imap), the
+ * CSR-coded list of the output rows (ocsr, ocode) gives the scatter side; `buffer` holds
+ * qsum*c_out elements of dtype.  kpos_host / qkpos_host are optional host copies of kpos / qkpos
+ * (kv+1 entries); with them the kernels take the offsets from their arguments instead of loading
+ * them.  No counterpart in the reference: it is ConvolutionForwardD2 with the atomic scatter-add
+ * replaced by the output-stationary sum of ConvolutionForwardD1 (backend/spconv.cu:149-161),
+ * fused with the centre GEMM. */
+int pce_conv_fwd_fds(const void *in_feats, const void *weight, const void *weight_packed,
+                     void *out_feats, int32_t dtype, int64_t n_in, int64_t n_out, int32_t c_in,
+                     int32_t c_out, int32_t kv, int32_t mid, const int32_t *imap_dev,
+                     const int32_t *kpos_dev, const int32_t *qkpos_dev, const int32_t *kpos_host,
+                     const int32_t *qkpos_host, const int32_t *ocsr_dev, const int32_t *ocode_dev,
+                     int64_t qsum, void *buffer_dev, int64_t buffer_elems, pce_stream_t stream);
+
 /* Output-stationary: nbr[kv*n_out] from pce_kmap_build (for a transposed layer, a table built
  * with the roles swapped).  One kernel, one store per output row.  No counterpart in the
  * reference: it is the same fetch-on-demand computation with the scatter-add replaced by
  * register accumulation. */
-int pce_conv_fwd_os(const void *in_feats, const void *weight, void *out_feats, int32_t dtype,
+int pce_conv_fwd_os(const void *in_feats, const void *weight, const void *weight_packed,
+                    void *out_feats, int32_t dtype,
                     int64_t n_in, int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv,
                     const int32_t *nbr_dev, pce_stream_t stream);
 
 /* out[n,c_out] = in[n,c_in] * weight[c_in,c_out]: the 1x1 stride-1 shortcut of the front end
  * (script/spconv.py:297-304), on the same MFMA tile kernel. */
-int pce_conv_fwd_dense(const void *in_feats, const void *weight, void *out_feats, int32_t dtype,
+int pce_conv_fwd_dense(const void *in_feats, const void *weight, const void *weight_packed,
+                       void *out_feats, int32_t dtype,
                        int64_t n, int32_t c_in, int32_t c_out, pce_stream_t stream);
 
 /* Per-layer dataflow choice from map density (pairs per output row) and channel widths. */

@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libpcengine_amd.so")
 
 PCE_OK, PCE_EINVAL, PCE_ECAPACITY, PCE_EHIP, PCE_EWORKSPACE, PCE_ECOORD = range(6)
 PCE_F16, PCE_F32 = 0, 1
-DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS = 0, 1, 2
+DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS, DATAFLOW_FDS = 0, 1, 2, 3
 QUANTUM = 128
 CSR_CODE = 1186111
 
@@ -41,6 +41,7 @@ class PCEError(RuntimeError):
 _SIGNATURES = {
     "pce_version": (c_int32, []),
     "pce_last_error": (c_char_p, []),
+    "pce_set_stage_mask": (None, [ctypes.c_uint32]),
     "pce_hash_slots": (c_int64, [c_int64]),
     "pce_hash_table_bytes": (c_int64, [c_int64]),
     "pce_hash_build": (c_int32, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p]),
@@ -51,12 +52,17 @@ _SIGNATURES = {
     "pce_kmap_workspace_bytes": (c_int64, [c_int64, c_int64, c_int32, c_int32]),
     "pce_kmap_build": (c_int32, [c_void_p, c_int64, c_void_p, c_int64, POINTER(Geom), c_void_p, c_int64] + [c_void_p] * 12 + [c_void_p]),
     "pce_conv_fod_workspace_bytes": (c_int64, [c_int64, c_int32, c_int32]),
-    "pce_conv_fwd_fod": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32,
+    "pce_packed_weight_bytes": (c_int64, [c_int32, c_int32, c_int32, c_int32]),
+    "pce_pack_weights": (c_int32, [c_void_p, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
+    "pce_conv_fwd_fds": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32,
+                                   c_void_p, c_void_p, c_void_p, POINTER(c_int32), POINTER(c_int32), c_void_p, c_void_p, c_int64,
+                                   c_void_p, c_int64, c_void_p]),
+    "pce_conv_fwd_fod": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32,
                                    c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
-    "pce_conv_fwd_gms": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32,
+    "pce_conv_fwd_gms": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32,
                                    c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
-    "pce_conv_fwd_os": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
-    "pce_conv_fwd_dense": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32, c_void_p]),
+    "pce_conv_fwd_os": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
+    "pce_conv_fwd_dense": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32, c_void_p]),
     "pce_select_dataflow": (c_int32, [c_int64, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32]),
 }
 

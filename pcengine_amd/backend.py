@@ -19,7 +19,7 @@ from typing import Optional, Sequence, Tuple
 import torch
 
 from . import _lib
-from ._lib import Geom, DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS, PCE_F16, PCE_F32, QUANTUM, CSR_CODE
+from ._lib import Geom, DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS, DATAFLOW_FDS, PCE_F16, PCE_F32, QUANTUM, CSR_CODE
 
 CODE_A, CODE_B = 94273, 311  # packed 3-vectors, script/utils.py:233-242
 
@@ -88,6 +88,8 @@ class KernelMap:
     in_coords: Optional[torch.Tensor] = None
     geom: Optional[Geom] = None
     knnz_host: list = field(default_factory=list)
+    kpos_host: object = None     # ctypes int32 arrays (kv+1) mirrored on the host by the map build's one read-back
+    qkpos_host: object = None
 
     @property
     def has_csr(self) -> bool:
@@ -185,6 +187,8 @@ def build_kernel_map(in_coords: torch.Tensor, ks, stride, pad, cmin, cmax_out, s
                    icode=None if icode is None else icode[:M], ocode=None if ocode is None else ocode[:M],
                    in_coords=in_coords, geom=geom, knnz_host=host[:kv])
     km._cmin, km._cmax = list(cmin), list(cmax_out)
+    km.kpos_host = (_lib.c_int32 * (kv + 1))(*host[kv:2 * kv + 1])
+    km.qkpos_host = (_lib.c_int32 * (kv + 1))(*host[2 * kv + 1:3 * kv + 2])
     return km
 
 
@@ -212,7 +216,24 @@ def select_dataflow(km: KernelMap, c_in: int, c_out: int, dtype: torch.dtype, tr
     return lib.pce_select_dataflow(n_in, n_out, km.M, c_in, c_out, km.kv, PCE_F16 if dtype == torch.float16 else PCE_F32)
 
 
-def dense_forward(feats: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+def pack_weights(weight: torch.Tensor) -> Optional[torch.Tensor]:
+    """fp16 weights [kv, c_in, c_out] in the order the kernels stage them into LDS (None for fp32).
+    Weights are constants of an inference engine: callers pack once and pass the copy along."""
+    lib = _lib.load()
+    if weight.dtype != torch.float16:
+        return None
+    _require_cuda(weight, "weight")
+    weight = weight.contiguous()
+    if weight.dim() == 2:
+        weight = weight.unsqueeze(0)
+    kv, c_in, c_out = weight.shape
+    nbytes = lib.pce_packed_weight_bytes(PCE_F16, kv, c_in, c_out)
+    packed = torch.empty(nbytes, dtype=torch.uint8, device=weight.device)
+    _lib.check(lib.pce_pack_weights(weight.data_ptr(), PCE_F16, kv, c_in, c_out, packed.data_ptr(), _stream(weight.device)))
+    return packed
+
+
+def dense_forward(feats: torch.Tensor, weight: torch.Tensor, packed: Optional[torch.Tensor] = None) -> torch.Tensor:
     """feats @ weight for the 1x1 stride-1 layer (script/spconv.py:297-304)."""
     lib = _lib.load()
     _require_cuda(feats, "feats")
@@ -221,13 +242,13 @@ def dense_forward(feats: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     if feats.shape[1] != weight.shape[0]:
         raise ValueError("Input feature size and kernel size mismatch")
     out = torch.empty((feats.shape[0], weight.shape[1]), dtype=feats.dtype, device=feats.device)
-    _lib.check(lib.pce_conv_fwd_dense(feats.data_ptr(), weight.data_ptr(), out.data_ptr(), _dtype_code(feats),
+    _lib.check(lib.pce_conv_fwd_dense(feats.data_ptr(), weight.data_ptr(), _ptr(packed), out.data_ptr(), _dtype_code(feats),
                                       feats.shape[0], feats.shape[1], weight.shape[1], _stream(feats.device)))
     return out
 
 
 def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataflow: int, transposed: bool = False,
-                 buffer: Optional[torch.Tensor] = None) -> torch.Tensor:
+                 buffer: Optional[torch.Tensor] = None, packed: Optional[torch.Tensor] = None) -> torch.Tensor:
     """One forward convolution over an existing map with the chosen dataflow."""
     lib = _lib.load()
     _require_cuda(feats, "feats")
@@ -254,23 +275,34 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
         imap, omap = (km.omap, km.imap) if transposed else (km.imap, km.omap)
         ws_bytes = lib.pce_conv_fod_workspace_bytes(n_out, c_out, dt)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
-        _lib.check(lib.pce_conv_fwd_fod(feats.data_ptr(), weight.data_ptr(), out.data_ptr(), dt, n_in, n_out, c_in, c_out,
-                                        kv, mid, imap.data_ptr(), omap.data_ptr(), km.kpos.data_ptr(), km.qkpos.data_ptr(),
-                                        km.qsum, _ptr(ws), ws_bytes, s))
+        _lib.check(lib.pce_conv_fwd_fod(feats.data_ptr(), weight.data_ptr(), _ptr(packed), out.data_ptr(), dt, n_in, n_out,
+                                        c_in, c_out, kv, mid, imap.data_ptr(), omap.data_ptr(), km.kpos.data_ptr(),
+                                        km.qkpos.data_ptr(), km.qsum, _ptr(ws), ws_bytes, s))
+    elif dataflow == DATAFLOW_FDS:
+        ensure_csr(km)
+        need = km.qsum * c_out
+        if buffer is None or buffer.numel() < need or buffer.dtype != feats.dtype or buffer.device != dev:
+            buffer = torch.empty(max(need, 1), dtype=feats.dtype, device=dev)
+        imap = km.omap if transposed else km.imap
+        ocsr, ocode = (km.icsr, km.icode) if transposed else (km.ocsr, km.ocode)
+        _lib.check(lib.pce_conv_fwd_fds(feats.data_ptr(), weight.data_ptr(), _ptr(packed), out.data_ptr(), dt, n_in, n_out,
+                                        c_in, c_out, kv, mid, imap.data_ptr(), km.kpos.data_ptr(), km.qkpos.data_ptr(),
+                                        km.kpos_host, km.qkpos_host, ocsr.data_ptr(), ocode.data_ptr(), km.qsum,
+                                        buffer.data_ptr(), buffer.numel(), s))
     elif dataflow == DATAFLOW_GMS:
         ensure_csr(km)
         need = km.qsum * (c_in + c_out)
         if buffer is None or buffer.numel() < need or buffer.dtype != feats.dtype or buffer.device != dev:
             buffer = torch.empty(max(need, 1), dtype=feats.dtype, device=dev)
         icsr, icode, ocsr, ocode = (km.ocsr, km.ocode, km.icsr, km.icode) if transposed else (km.icsr, km.icode, km.ocsr, km.ocode)
-        _lib.check(lib.pce_conv_fwd_gms(feats.data_ptr(), weight.data_ptr(), out.data_ptr(), dt, n_in, n_out, c_in, c_out,
-                                        kv, mid, icsr.data_ptr(), icode.data_ptr(), ocsr.data_ptr(), ocode.data_ptr(),
+        _lib.check(lib.pce_conv_fwd_gms(feats.data_ptr(), weight.data_ptr(), _ptr(packed), out.data_ptr(), dt, n_in, n_out,
+                                        c_in, c_out, kv, mid, icsr.data_ptr(), icode.data_ptr(), ocsr.data_ptr(), ocode.data_ptr(),
                                         km.kpos.data_ptr(), km.qkpos.data_ptr(), km.qsum, buffer.data_ptr(), buffer.numel(), s))
     elif dataflow == DATAFLOW_OS:
         ensure_nbr(km, transposed)
         nbr = km.nbr_in if transposed else km.nbr_out
-        _lib.check(lib.pce_conv_fwd_os(feats.data_ptr(), weight.data_ptr(), out.data_ptr(), dt, n_in, n_out, c_in, c_out,
-                                       kv, nbr.data_ptr(), s))
+        _lib.check(lib.pce_conv_fwd_os(feats.data_ptr(), weight.data_ptr(), _ptr(packed), out.data_ptr(), dt, n_in, n_out,
+                                       c_in, c_out, kv, nbr.data_ptr(), s))
     else:
         raise NotImplementedError(f"unknown dataflow {dataflow}")
     return out
@@ -335,7 +367,7 @@ def conv_fwd_d2_cuda(in_feats, kernel, ksize_code, sum_nnz, out_feats, kpos, qkp
     n_in, n_out = in_feats.shape[0], out_feats.shape[0]
     ws_bytes = lib.pce_conv_fod_workspace_bytes(n_out, c_out, dt)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=in_feats.device) if ws_bytes else None
-    _lib.check(lib.pce_conv_fwd_fod(in_feats.data_ptr(), kernel.data_ptr(), out_feats.data_ptr(), dt, n_in, n_out, c_in,
+    _lib.check(lib.pce_conv_fwd_fod(in_feats.data_ptr(), kernel.data_ptr(), None, out_feats.data_ptr(), dt, n_in, n_out, c_in,
                                     c_out, kv, _ksize_mid(ksize_code, separate_mid), in_map.data_ptr(), out_map.data_ptr(),
                                     kpos.data_ptr(), qkpos.data_ptr(), int(sum_nnz), _ptr(ws), ws_bytes,
                                     _stream(in_feats.device)))
@@ -355,7 +387,7 @@ def conv_fwd_d1_cuda(in_feats, kernel, ksize_code, qsum_nnz, out_feats, kpos, qk
     if kpos.numel() < kv + 1:
         # the reference front end allocates kv entries (script/spconv.py:396); the total is the last row pointer
         kpos = torch.cat([kpos[:kv], in_csr[in_feats.shape[0]:in_feats.shape[0] + 1]])
-    _lib.check(lib.pce_conv_fwd_gms(in_feats.data_ptr(), kernel.data_ptr(), out_feats.data_ptr(), dt, in_feats.shape[0],
+    _lib.check(lib.pce_conv_fwd_gms(in_feats.data_ptr(), kernel.data_ptr(), None, out_feats.data_ptr(), dt, in_feats.shape[0],
                                     out_feats.shape[0], c_in, c_out, kv, _ksize_mid(ksize_code, separate_mid),
                                     in_csr.data_ptr(), in_map.data_ptr(), out_csr.data_ptr(), out_map.data_ptr(),
                                     kpos.data_ptr(), qkpos.data_ptr(), int(qsum_nnz), buffer.data_ptr(), buffer.numel(),

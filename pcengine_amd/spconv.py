@@ -2,7 +2,7 @@
 (script/spconv.py:15-106) over the MI355X backend.
 
 Differences a user can see, all supersets of the reference:
-* ``dataflow='auto'|'fod'|'gms'|'os'`` constructor argument (and the PCENGINE_DATAFLOW
+* ``dataflow='auto'|'fod'|'gms'|'os'|'fds'`` constructor argument (and the PCENGINE_DATAFLOW
   environment variable) on top of the reference's ``init_tag`` list.  A tensor whose
   ``init_tag`` starts with 'D1' / 'D2' pins the next newly built map to gather-GEMM-scatter /
   fetch-on-demand exactly as in the reference (script/spconv.py:343, 388); the default tag
@@ -21,12 +21,13 @@ import torch
 import torch.nn as nn
 
 from . import backend
-from .backend import DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS
+from .backend import DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS, DATAFLOW_FDS
 from .sptensor import spTensor
 from .utils import conv_info_decoder, conv_info_encoder, output_stride_compute
 
 _UNIT = conv_info_encoder([1, 1, 1])
-_DATAFLOWS = {"fod": DATAFLOW_FOD, "d2": DATAFLOW_FOD, "gms": DATAFLOW_GMS, "d1": DATAFLOW_GMS, "os": DATAFLOW_OS}
+_DATAFLOWS = {"fod": DATAFLOW_FOD, "d2": DATAFLOW_FOD, "gms": DATAFLOW_GMS, "d1": DATAFLOW_GMS, "os": DATAFLOW_OS,
+              "fds": DATAFLOW_FDS}
 
 # one record per executed layer when enabled: (N_in, N_out, M, C_in, C_out, dataflow)
 layer_log: Optional[list] = None
@@ -83,11 +84,24 @@ class conv3d(nn.Module):
             if self.bias is not None:
                 self.bias.uniform_(-bound, bound)
 
+    def _weights_for(self, dtype):
+        """Kernel in the feature dtype plus its packed fp16 copy, rebuilt only when the parameter changes."""
+        k = self.kernel
+        key = (k.data_ptr(), k._version, dtype, k.device)
+        if getattr(self, "_wcache_key", None) != key:
+            w = k.detach()
+            w = w if w.dtype == dtype else w.to(dtype)
+            w = w.contiguous()
+            self._wcache = (w, backend.pack_weights(w) if w.is_cuda else None)
+            self._wcache_key = key
+        return self._wcache
+
     def forward(self, input: spTensor) -> spTensor:
-        return conv_func(input=input, in_channel=self.in_channels, out_channel=self.out_channels, kernel=self.kernel,
+        w, packed = self._weights_for(input.feats.dtype)
+        return conv_func(input=input, in_channel=self.in_channels, out_channel=self.out_channels, kernel=w,
                          kernel_size_code=self.kernel_size_code, stride_code=self.stride_code,
                          padding_code=self.padding_code, bias=self.bias, transposed=self.transposed,
-                         tensorcore=self.tensorcore, dataflow=self.dataflow)
+                         tensorcore=self.tensorcore, dataflow=self.dataflow, packed=packed)
 
 
 def _pick_dataflow(km: backend.KernelMap, requested: str, c_in: int, c_out: int, dtype, transposed: bool) -> int:
@@ -103,25 +117,26 @@ def _pick_dataflow(km: backend.KernelMap, requested: str, c_in: int, c_out: int,
     return backend.select_dataflow(km, c_in, c_out, dtype, transposed)
 
 
-def _run(input: spTensor, km: backend.KernelMap, kernel, in_channel, out_channel, transposed, dataflow) -> torch.Tensor:
+def _run(input: spTensor, km: backend.KernelMap, kernel, in_channel, out_channel, transposed, dataflow, packed) -> torch.Tensor:
     feats = input.feats
     if kernel.dtype != feats.dtype:
-        kernel = kernel.to(feats.dtype)
+        kernel, packed = kernel.to(feats.dtype), None
     df = _pick_dataflow(km, dataflow, in_channel, out_channel, feats.dtype, transposed)
-    out = backend.conv_forward(feats, kernel.detach(), km, df, transposed=transposed, buffer=input.buffer)
+    out = backend.conv_forward(feats, kernel.detach(), km, df, transposed=transposed, buffer=input.buffer, packed=packed)
     if layer_log is not None:
         layer_log.append((feats.shape[0], out.shape[0], km.M, in_channel, out_channel, df))
     return out
 
 
 def conv_func(input: spTensor, in_channel, out_channel, kernel, kernel_size_code, stride_code, padding_code, bias,
-              transposed, tensorcore, dataflow: str = "auto") -> spTensor:
+              transposed, tensorcore, dataflow: str = "auto", packed=None) -> spTensor:
     """Map cache lookup / build, dataflow dispatch, bias, metadata propagation
     (script/spconv.py:291-464)."""
     if kernel_size_code == _UNIT and stride_code == _UNIT:
         # 1x1 stride 1: plain matrix product, coordinates unchanged, no map (script/spconv.py:297-304)
-        w = kernel if kernel.dtype == input.feats.dtype else kernel.to(input.feats.dtype)
-        out_feats = backend.dense_forward(input.feats, w.detach())
+        if kernel.dtype != input.feats.dtype:
+            kernel, packed = kernel.to(input.feats.dtype), None
+        out_feats = backend.dense_forward(input.feats, kernel.detach(), packed)
         if bias is not None:
             out_feats += bias.to(out_feats.dtype)
         return input._like(out_feats)
@@ -134,7 +149,7 @@ def conv_func(input: spTensor, in_channel, out_channel, kernel, kernel_size_code
             raise KeyError("transposed conv3d found no cached map for this (kernel, stride): "
                            "the matching strided conv3d must run first on the same tensor family")
         out_coords = input.cbook[output_stride]
-        out_feats = _run(input, km, kernel, in_channel, out_channel, True, dataflow)
+        out_feats = _run(input, km, kernel, in_channel, out_channel, True, dataflow, packed)
         if bias is not None:
             out_feats += bias.to(out_feats.dtype)
         output = spTensor(feats=out_feats, coords=out_coords, buffer=input.buffer, batchsize=input.batchsize,
@@ -158,15 +173,16 @@ def conv_func(input: spTensor, in_channel, out_channel, kernel, kernel_size_code
         tag = input.init_tag[0] if input.init_tag else 'end'
         if tag not in ('D1', 'D2', 'end', 'auto'):
             raise NotImplementedError(f"unknown init_tag entry {tag!r}")
+        auto = tag in ('end', 'auto')
         km = backend.build_kernel_map(input.coords, ks, stride, pad, coords_min, coords_max, subm,
-                                      want_csr=(tag == 'D1'), want_nbr_out=(tag in ('end', 'auto')))
+                                      want_csr=(tag == 'D1' or auto), want_nbr_out=auto, want_nbr_in=auto and not subm)
         km.tag = tag if tag in ('D1', 'D2') else 'auto'
         input.kmaps[key] = km
         input.cbook[output_stride] = km.out_coords
         if tag in ('D1', 'D2'):
             input.init_tag = input.init_tag[1:]
     input.cbook.setdefault(input.stride, input.coords)
-    out_feats = _run(input, km, kernel, in_channel, out_channel, False, dataflow)
+    out_feats = _run(input, km, kernel, in_channel, out_channel, False, dataflow, packed)
     if bias is not None:
         out_feats += bias.to(out_feats.dtype)
     output = spTensor(feats=out_feats, coords=km.out_coords, buffer=input.buffer, batchsize=input.batchsize,

@@ -26,7 +26,7 @@ def voxelize(points: np.ndarray, voxel: float, batch: int = 0) -> np.ndarray:
     return np.concatenate([b, q], axis=1).astype(np.int32)
 
 
-def sphere_plane_cloud(seed: int = 1, n_sphere: int = 26000, n_plane: int = 9000,
+def sphere_plane_cloud(seed: int = 1, n_sphere: int = 21000, n_plane: int = 7300,
                        voxel: float = 0.02) -> np.ndarray:
     """Config 1: unit-sphere surface samples plus a z=0 patch over [-1,1]^2."""
     rng = np.random.default_rng(seed)
@@ -38,7 +38,7 @@ def sphere_plane_cloud(seed: int = 1, n_sphere: int = 26000, n_plane: int = 9000
 
 
 def lidar_cloud(seed: int = 2, rings: int = 64, azimuths: int = 2048,
-                n_ground: int = 24000, voxel: float = 0.1,
+                n_ground: int = 19500, voxel: float = 0.1,
                 half_extent: float = 50.0) -> np.ndarray:
     """Config 2: 64 elevation rings (-25..+3 deg) x 2048 azimuth steps with
     per-ray range U(2, 50) m, plus ground-plane samples at z = -1.7 m."""
@@ -56,7 +56,7 @@ def lidar_cloud(seed: int = 2, rings: int = 64, azimuths: int = 2048,
 
 def lidar_cloud_100k(seed: int = 2) -> np.ndarray:
     """Config 4 input: the config-2 generator with counts tuned to ~100k voxels."""
-    return lidar_cloud(seed=seed, rings=64, azimuths=1344, n_ground=16000)
+    return lidar_cloud(seed=seed, rings=64, azimuths=1344, n_ground=14000)
 
 
 def _box_surface(rng, lo, hi, n):
@@ -74,7 +74,7 @@ def _box_surface(rng, lo, hi, n):
     return pts
 
 
-def indoor_scene(rng, n_room: int = 260000, n_box: int = 4000) -> np.ndarray:
+def indoor_scene(rng, n_room: int = 120000, n_box: int = 2500) -> np.ndarray:
     """One 8 x 8 x 3 m room (four walls + floor) plus 20 axis-aligned boxes."""
     room = _box_surface(rng, (0, 0, 0), (8, 8, 3), n_room)
     room = room[room[:, 2] < 3.0 - 1e-9]  # no ceiling
@@ -87,7 +87,7 @@ def indoor_scene(rng, n_room: int = 260000, n_box: int = 4000) -> np.ndarray:
 
 
 def indoor_batch(seed: int = 5, scenes: int = 8, voxel: float = 0.02,
-                 n_room: int = 260000, n_box: int = 4000) -> np.ndarray:
+                 n_room: int = 120000, n_box: int = 2500) -> np.ndarray:
     """Config 5: ``scenes`` rooms collated with the batch index in column 0."""
     rng = np.random.default_rng(seed)
     out = [voxelize(indoor_scene(rng, n_room, n_box), voxel, batch=b) for b in range(scenes)]

@@ -6,12 +6,12 @@ import torch
 
 from oracle import oracle as orc
 from pcengine_amd import backend, synth
-from pcengine_amd.backend import DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS
+from pcengine_amd.backend import DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS, DATAFLOW_FDS
 from tests.util import DEV, TOL, gpu_map, rounded
 
 pytestmark = pytest.mark.gpu
 
-FLOWS = [DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS]
+FLOWS = [DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS, DATAFLOW_FDS]
 CHANNELS = [(16, 16), (64, 64), (4, 32), (32, 20), (96, 96), (5, 7), (64, 160), (130, 40)]
 
 
@@ -32,10 +32,13 @@ def test_submanifold_all_dataflows(c_in, c_out, dtype):
     coords = synth.random_cloud(seed=41, n=9000, extent=22, batches=2)
     fd, wd, ref_map, want = _case(coords, (3, 3, 3), (1, 1, 1), (0, 0, 0), c_in, c_out, dtype)
     km = gpu_map(coords, (3, 3, 3), want_csr=True, want_nbr_in=True)
+    packed = backend.pack_weights(wd)
+    assert (packed is None) == (dtype == torch.float32)
     for flow in FLOWS:
-        out = backend.conv_forward(fd, wd, km, flow)
-        err = orc.rel_l2(out.double().cpu().numpy(), want)
-        assert err <= TOL[dtype], (flow, err)
+        for pk in (None, packed):
+            out = backend.conv_forward(fd, wd, km, flow, packed=pk)
+            err = orc.rel_l2(out.double().cpu().numpy(), want)
+            assert err <= TOL[dtype], (flow, pk is not None, err)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
@@ -49,11 +52,12 @@ def test_strided_then_transposed_all_dataflows(ks, stride, pad, dtype):
     kv = km.kv
     wt = synth.weights(9, kv, c_out, c_in)
     wtd = torch.as_tensor(wt, device=DEV).to(dtype)
+    pk, pkt = backend.pack_weights(wd), backend.pack_weights(wtd)
     for flow in FLOWS:
-        out = backend.conv_forward(fd, wd, km, flow)
+        out = backend.conv_forward(fd, wd, km, flow, packed=pk)
         assert orc.rel_l2(out.double().cpu().numpy(), want) <= TOL[dtype], flow
         # transposed layer back onto the input coordinates, fed with the GPU's own output
-        back = backend.conv_forward(out, wtd, km, flow, transposed=True)
+        back = backend.conv_forward(out, wtd, km, flow, transposed=True, packed=pkt)
         want_t = orc.conv_forward(out.double().cpu().numpy(), rounded(wt, dtype), ref_map, ks, transposed=True)
         assert back.shape == (len(coords), c_in)
         assert orc.rel_l2(back.double().cpu().numpy(), want_t) <= TOL[dtype], flow
@@ -63,9 +67,11 @@ def test_strided_then_transposed_all_dataflows(ks, stride, pad, dtype):
 def test_dense_1x1(dtype):
     f = synth.features(3, 5001, 96)
     w = synth.weights(3, 1, 96, 20)[0]
-    out = backend.dense_forward(torch.as_tensor(f, device=DEV).to(dtype), torch.as_tensor(w, device=DEV).to(dtype))
+    fd, wd = torch.as_tensor(f, device=DEV).to(dtype), torch.as_tensor(w, device=DEV).to(dtype)
     want = rounded(f, dtype) @ rounded(w, dtype)
-    assert orc.rel_l2(out.double().cpu().numpy(), want) <= TOL[dtype]
+    for pk in (None, backend.pack_weights(wd)):
+        out = backend.dense_forward(fd, wd, pk)
+        assert orc.rel_l2(out.double().cpu().numpy(), want) <= TOL[dtype]
 
 
 def test_config1_fp32_c16():
@@ -86,8 +92,8 @@ def test_config2_fp16_c64_full_size():
         assert orc.rel_l2(out.double().cpu().numpy(), want) <= 1e-3, flow
     # linearity in the features holds at any size: conv(2x) == 2 conv(x); scaling by two is exact in
     # fp16 except for results in the subnormal range, whose spacing is 2^-24
-    twice = backend.conv_forward(fd * 2, wd, km, DATAFLOW_OS)
-    assert torch.allclose(twice.float(), outs[2].float() * 2, rtol=0, atol=2.0 ** -23)
+    twice = backend.conv_forward(fd * 2, wd, km, DATAFLOW_FDS, packed=backend.pack_weights(wd))
+    assert torch.allclose(twice.float(), outs[3].float() * 2, rtol=0, atol=2.0 ** -23)
 
 
 def test_reference_named_entry_points_d2_and_d1():

@@ -23,7 +23,7 @@ def _weights(layer, dtype):
     return w
 
 
-@pytest.mark.parametrize("flow,tags", [("auto", None), ("fod", None), ("gms", None), ("os", None), ("auto", ["D1", "D2", "end"]),
+@pytest.mark.parametrize("flow,tags", [("auto", None), ("fod", None), ("gms", None), ("os", None), ("fds", None), ("auto", ["D1", "D2", "end"]),
                                        ("auto", ["D2", "D1", "end"])])
 def test_down_up_block_matches_oracle(flow, tags):
     dtype = torch.float16

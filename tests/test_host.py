@@ -40,23 +40,28 @@ def test_pure_host_entry_points():
 
 def test_argument_validation_needs_no_gpu():
     lib = _lib.load()
-    assert lib.pce_conv_fwd_fod(None, None, None, 0, 1, 1, 1, 1, 1, -1, None, None, None, None, 0, None, 0, None) == _lib.PCE_EINVAL
+    assert lib.pce_conv_fwd_fod(None, None, None, None, 0, 1, 1, 1, 1, 1, -1, None, None, None, None, 0, None, 0, None) == _lib.PCE_EINVAL
     with pytest.raises(ValueError):
         _lib.check(_lib.PCE_EINVAL)
     one = 1
-    assert lib.pce_conv_fwd_fod(one, one, one, 0, 10, 10, 4, 4, 27, 13, one, one, one, one, 100, one, 1 << 20, None) == _lib.PCE_EINVAL  # qsum % 128
-    assert lib.pce_conv_fwd_fod(one, one, one, 0, 10, 12, 4, 4, 27, 13, one, one, one, one, 128, one, 1 << 20, None) == _lib.PCE_EINVAL  # centre needs n_in == n_out
-    assert lib.pce_conv_fwd_fod(one, one, one, 0, 10, 10, 4, 4, 27, 13, one, one, one, one, 128, one, 16, None) == _lib.PCE_EWORKSPACE
-    assert lib.pce_conv_fwd_gms(one, one, one, 0, 10, 10, 4, 4, 27, 13, one, one, one, one, one, one, 128, one, 10, None) == _lib.PCE_EWORKSPACE
-    assert lib.pce_conv_fwd_os(one, one, one, 7, 10, 10, 4, 4, 27, one, None) == _lib.PCE_EINVAL      # dtype
+    fod = lambda n_in, n_out, qsum, ws: lib.pce_conv_fwd_fod(one, one, None, one, 0, n_in, n_out, 4, 4, 27, 13, one, one, one, one, qsum, one, ws, None)
+    assert fod(10, 10, 100, 1 << 20) == _lib.PCE_EINVAL        # qsum % 128
+    assert fod(10, 12, 128, 1 << 20) == _lib.PCE_EINVAL        # a centre offset needs n_in == n_out
+    assert fod(10, 10, 128, 16) == _lib.PCE_EWORKSPACE
+    assert lib.pce_conv_fwd_gms(one, one, None, one, 0, 10, 10, 4, 4, 27, 13, one, one, one, one, one, one, 128, one, 10, None) == _lib.PCE_EWORKSPACE
+    assert lib.pce_conv_fwd_fds(one, one, None, one, 0, 10, 10, 4, 4, 27, 13, one, one, one, None, None, one, one, 128, one, 10, None) == _lib.PCE_EWORKSPACE
+    assert lib.pce_conv_fwd_os(one, one, None, one, 7, 10, 10, 4, 4, 27, one, None) == _lib.PCE_EINVAL      # dtype
+    assert lib.pce_packed_weight_bytes(_lib.PCE_F16, 27, 64, 64) == 27 * 8 * 64 * 16
+    assert lib.pce_packed_weight_bytes(_lib.PCE_F16, 27, 4, 20) == 27 * 1 * 32 * 16
+    assert lib.pce_packed_weight_bytes(_lib.PCE_F32, 27, 64, 64) == 0
 
 
 def test_selector_is_monotone_in_density():
     lib = _lib.load()
     n = 100000
     picks = [lib.pce_select_dataflow(n, n, int(rho * n), 64, 64, 27, 0) for rho in (0.1, 0.5, 1.0, 3.0, 8.0, 20.0)]
-    assert picks[0] == _lib.DATAFLOW_FOD and picks[-1] == _lib.DATAFLOW_OS
-    order = {_lib.DATAFLOW_FOD: 0, _lib.DATAFLOW_GMS: 1, _lib.DATAFLOW_OS: 2}
+    assert picks[0] == _lib.DATAFLOW_FDS and picks[-1] == _lib.DATAFLOW_OS
+    order = {_lib.DATAFLOW_FDS: 0, _lib.DATAFLOW_FOD: 0, _lib.DATAFLOW_GMS: 1, _lib.DATAFLOW_OS: 2}
     ranks = [order[p] for p in picks]
     assert ranks == sorted(ranks)
 
