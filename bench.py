@@ -34,7 +34,7 @@ def main() -> int:
     import numpy as np
     import torch
     from pcengine_amd import _lib, backend, synth
-    from pcengine_amd.backend import DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS
+    from pcengine_amd.backend import DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS, DATAFLOW_FDS
 
     lib = _lib.load()
     dev = "cuda:0"
@@ -72,13 +72,14 @@ def main() -> int:
     map_ms = (time.perf_counter() - t0) / 5 * 1e3
     M = km.M
 
-    names = {DATAFLOW_FOD: "fod", DATAFLOW_GMS: "gms", DATAFLOW_OS: "os"}
+    names = {DATAFLOW_FOD: "fod", DATAFLOW_GMS: "gms", DATAFLOW_OS: "os", DATAFLOW_FDS: "fds"}
+    packed = backend.pack_weights(wd)     # weights are constants: packed once, outside the timed region
     if args.dataflow == "auto":
         flow = backend.select_dataflow(km, c_in, c_out, torch.float16)
     else:
         flow = {v: k for k, v in names.items()}[args.dataflow]
     buffer = torch.empty(max(km.qsum * (c_in + c_out), 1), dtype=torch.float16, device=dev)
-    step = lambda f=flow: backend.conv_forward(fd, wd, km, f, buffer=buffer)
+    step = lambda f=flow: backend.conv_forward(fd, wd, km, f, buffer=buffer, packed=packed)
 
     # ---- timed region ---------------------------------------------------------------------------
     for _ in range(args.warmup):
@@ -99,6 +100,7 @@ def main() -> int:
     stages = {}
     stage_names = {DATAFLOW_FOD: {0: "centre_gemm", 1: "fod_pairs", 2: "convert"},
                    DATAFLOW_GMS: {3: "gather", 1: "grouped_gemm", 0: "centre_gemm", 2: "scatter"},
+                   DATAFLOW_FDS: {1: "fod_pairs_to_buffer", 2: "centre_gemm_csr_sum"},
                    DATAFLOW_OS: {1: "os_tile"}}[flow]
     if flow != DATAFLOW_OS:
         for bit, name in stage_names.items():
@@ -107,7 +109,7 @@ def main() -> int:
         lib.pce_set_stage_mask(0xFFFFFFFF)
     else:
         stages["os_tile"] = ms
-    others = {names[f]: ev_ms(lambda f=f: backend.conv_forward(fd, wd, km, f, buffer=buffer), max(20, args.steps // 4), 5)
+    others = {names[f]: ev_ms(lambda f=f: backend.conv_forward(fd, wd, km, f, buffer=buffer, packed=packed), max(20, args.steps // 4), 5)
               for f in names if f != flow}
 
     # algorithmic bytes of the layer: every tensor once + the pair list
@@ -123,6 +125,8 @@ def main() -> int:
         "grouped_gemm": M * (c_in + c_out) * e + 26 * c_in * c_out * e,
         "scatter": M * c_out * e + 2 * n * c_out * e + 4 * M + 4 * (n + 1),
         "os_tile": b_conv - 8 * M + 4 * 27 * n,
+        "fod_pairs_to_buffer": M * (c_in + c_out) * e + 4 * M + 26 * c_in * c_out * e,
+        "centre_gemm_csr_sum": n * c_in * e + n * c_out * e + c_in * c_out * e + M * c_out * e + 4 * M + 4 * (n + 1),
     }[dom]
     achieved = dom_bytes / (stages[dom] * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",

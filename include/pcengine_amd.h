@@ -113,6 +113,8 @@ int pce_outcoords_emit(const void *ws_dev, int64_t n_in, const pce_geom_t *g, in
  *   optional (pass NULL to skip), all four or none:
  *     icsr[n_in+1], icode[kv*n_in cap], ocsr[n_out+1], ocode[kv*n_in cap]: CSR-coded map,
  *     entry = kp*PCE_CSR_CODE + rank, ascending kp inside a row, rank = position inside the offset
+ *   optional, with the CSR outputs: islot, oslot int32[kv*n_in cap]: for pair p, the position of
+ *     its entry in icode / ocode (the inverse permutation of the CSR orders)
  *   optional nbr_out int32[kv*n_out]: output-major table nbr[kp*n_out + o] = input row or -1
  *     (centre offset of a submanifold layer = the row itself)
  *   optional nbr_in int32[kv*n_in]: input-major table nbr[kp*n_in + i] = output row or -1, the
@@ -125,8 +127,8 @@ int pce_kmap_build(const int32_t *in_coords_dev, int64_t n_in, const int32_t *ou
                    int64_t n_out, const pce_geom_t *g, void *ws_dev, int64_t ws_bytes,
                    int32_t *imap_dev, int32_t *omap_dev, int32_t *knnz_dev, int32_t *kpos_dev,
                    int32_t *qkpos_dev, int32_t *icsr_dev, int32_t *icode_dev, int32_t *ocsr_dev,
-                   int32_t *ocode_dev, int32_t *nbr_out_dev, int32_t *nbr_in_dev,
-                   int32_t *status_dev, pce_stream_t stream);
+                   int32_t *ocode_dev, int32_t *islot_dev, int32_t *oslot_dev, int32_t *nbr_out_dev,
+                   int32_t *nbr_in_dev, int32_t *status_dev, pce_stream_t stream);
 
 /* ---- forward convolution --------------------------------------------------------------------- *
  * Common arguments: in_feats[n_in,c_in], weight[kv,c_in,c_out], out_feats[n_out,c_out], all of
@@ -163,19 +165,23 @@ int pce_conv_fwd_gms(const void *in_feats, const void *weight, const void *weigh
                      const int32_t *qkpos_dev, int64_t qsum, void *buffer_dev,
                      int64_t buffer_elems, pce_stream_t stream);
 
-/* Fetch-on-demand with deferred scatter: the pair list gives the gather side (imap), the
- * CSR-coded list of the output rows (ocsr, ocode) gives the scatter side; `buffer` holds
- * qsum*c_out elements of dtype.  kpos_host / qkpos_host are optional host copies of kpos / qkpos
- * (kv+1 entries); with them the kernels take the offsets from their arguments instead of loading
- * them.  No counterpart in the reference: it is ConvolutionForwardD2 with the atomic scatter-add
- * replaced by the output-stationary sum of ConvolutionForwardD1 (backend/spconv.cu:149-161),
- * fused with the centre GEMM. */
+/* Fetch-on-demand with deferred scatter.  Gather side: the pair list (imap, kpos, qkpos).  Scatter
+ * side: oslot[p] = position of pair p among the entries of its output row in CSR order, and the
+ * row pointers ocsr.  Pair tiles store their partial row at buffer[oslot[p]]; the epilogue of the
+ * centre GEMM (or a row-sum kernel when there is no centre offset) adds rows
+ * buffer[ocsr[o] .. ocsr[o+1]) in fp32 and stores output row o once.  `buffer` holds
+ * n_pairs*c_out elements of dtype.  kpos_host / qkpos_host are optional host copies of kpos / qkpos
+ * (kv+1 entries): with them the kernels take the offsets from their arguments.
+ * No counterpart in the reference: it is ConvolutionForwardD2 with the atomic scatter-add replaced
+ * by the output-stationary sum of ConvolutionForwardD1 (backend/spconv.cu:149-161), fused with
+ * the centre GEMM. */
 int pce_conv_fwd_fds(const void *in_feats, const void *weight, const void *weight_packed,
                      void *out_feats, int32_t dtype, int64_t n_in, int64_t n_out, int32_t c_in,
                      int32_t c_out, int32_t kv, int32_t mid, const int32_t *imap_dev,
-                     const int32_t *kpos_dev, const int32_t *qkpos_dev, const int32_t *kpos_host,
-                     const int32_t *qkpos_host, const int32_t *ocsr_dev, const int32_t *ocode_dev,
-                     int64_t qsum, void *buffer_dev, int64_t buffer_elems, pce_stream_t stream);
+                     const int32_t *oslot_dev, const int32_t *kpos_dev, const int32_t *qkpos_dev,
+                     const int32_t *kpos_host, const int32_t *qkpos_host, const int32_t *ocsr_dev,
+                     int64_t n_pairs, int64_t qsum, void *buffer_dev, int64_t buffer_elems,
+                     pce_stream_t stream);
 
 /* Output-stationary: nbr[kv*n_out] from pce_kmap_build (for a transposed layer, a table built
  * with the roles swapped).  One kernel, one store per output row.  No counterpart in the

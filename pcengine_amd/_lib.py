@@ -50,13 +50,13 @@ _SIGNATURES = {
     "pce_outcoords_build": (c_int32, [c_void_p, c_int64, POINTER(Geom), c_void_p, c_int64, POINTER(c_int64), c_void_p]),
     "pce_outcoords_emit": (c_int32, [c_void_p, c_int64, POINTER(Geom), c_int64, c_void_p, c_void_p]),
     "pce_kmap_workspace_bytes": (c_int64, [c_int64, c_int64, c_int32, c_int32]),
-    "pce_kmap_build": (c_int32, [c_void_p, c_int64, c_void_p, c_int64, POINTER(Geom), c_void_p, c_int64] + [c_void_p] * 12 + [c_void_p]),
+    "pce_kmap_build": (c_int32, [c_void_p, c_int64, c_void_p, c_int64, POINTER(Geom), c_void_p, c_int64] + [c_void_p] * 14 + [c_void_p]),
     "pce_conv_fod_workspace_bytes": (c_int64, [c_int64, c_int32, c_int32]),
     "pce_packed_weight_bytes": (c_int64, [c_int32, c_int32, c_int32, c_int32]),
     "pce_pack_weights": (c_int32, [c_void_p, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
     "pce_conv_fwd_fds": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32,
-                                   c_void_p, c_void_p, c_void_p, POINTER(c_int32), POINTER(c_int32), c_void_p, c_void_p, c_int64,
-                                   c_void_p, c_int64, c_void_p]),
+                                   c_void_p, c_void_p, c_void_p, c_void_p, POINTER(c_int32), POINTER(c_int32), c_void_p, c_int64,
+                                   c_int64, c_void_p, c_int64, c_void_p]),
     "pce_conv_fwd_fod": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32,
                                    c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
     "pce_conv_fwd_gms": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32,

@@ -84,6 +84,8 @@ class KernelMap:
     icode: Optional[torch.Tensor] = None
     ocsr: Optional[torch.Tensor] = None
     ocode: Optional[torch.Tensor] = None
+    islot: Optional[torch.Tensor] = None   # pair -> position of its entry in icode / ocode
+    oslot: Optional[torch.Tensor] = None
     tag: str = "auto"           # 'D1' / 'D2' when the reference's init_tag protocol fixed it
     in_coords: Optional[torch.Tensor] = None
     geom: Optional[Geom] = None
@@ -164,14 +166,14 @@ def build_kernel_map(in_coords: torch.Tensor, ks, stride, pad, cmin, cmax_out, s
     if want_csr:
         icsr = torch.empty(n_in + 1, dtype=torch.int32, device=dev)
         ocsr = torch.empty(n_out + 1, dtype=torch.int32, device=dev)
-        codes = torch.empty((2, kv * n_in), dtype=torch.int32, device=dev)
-        icode, ocode = codes[0], codes[1]
+        codes = torch.empty((4, kv * n_in), dtype=torch.int32, device=dev)
+        icode, ocode, islot, oslot = codes[0], codes[1], codes[2], codes[3]
     else:
-        icsr = ocsr = icode = ocode = None
+        icsr = ocsr = icode = ocode = islot = oslot = None
     _lib.check(lib.pce_kmap_build(in_coords.data_ptr(), n_in, out_coords.data_ptr(), n_out, geom, ws.data_ptr(), ws_bytes,
                                   pairs[0].data_ptr(), pairs[1].data_ptr(), knnz.data_ptr(), kpos.data_ptr(),
-                                  qkpos.data_ptr(), _ptr(icsr), _ptr(icode), _ptr(ocsr), _ptr(ocode), _ptr(nbr_out),
-                                  _ptr(nbr_in), status.data_ptr(), s))
+                                  qkpos.data_ptr(), _ptr(icsr), _ptr(icode), _ptr(ocsr), _ptr(ocode), _ptr(islot),
+                                  _ptr(oslot), _ptr(nbr_out), _ptr(nbr_in), status.data_ptr(), s))
     host = meta.cpu().tolist()   # the one synchronisation of a map build
     st = host[3 * kv + 2:]
     if st[0]:
@@ -185,6 +187,7 @@ def build_kernel_map(in_coords: torch.Tensor, ks, stride, pad, cmin, cmax_out, s
                    M=M, qsum=qsum, imap=pairs[0, :M], omap=pairs[1, :M], knnz=knnz, kpos=kpos, qkpos=qkpos,
                    out_coords=out_coords, nbr_out=nbr_out, nbr_in=nbr_in, icsr=icsr, ocsr=ocsr,
                    icode=None if icode is None else icode[:M], ocode=None if ocode is None else ocode[:M],
+                   islot=None if islot is None else islot[:M], oslot=None if oslot is None else oslot[:M],
                    in_coords=in_coords, geom=geom, knnz_host=host[:kv])
     km._cmin, km._cmax = list(cmin), list(cmax_out)
     km.kpos_host = (_lib.c_int32 * (kv + 1))(*host[kv:2 * kv + 1])
@@ -199,6 +202,7 @@ def ensure_csr(km: KernelMap) -> None:
     full = build_kernel_map(km.in_coords, km.ks, km.stride, km.pad, km._cmin, km._cmax, km.subm, want_csr=True,
                             want_nbr_out=False, out_coords=km.out_coords)
     km.icsr, km.icode, km.ocsr, km.ocode = full.icsr, full.icode, full.ocsr, full.ocode
+    km.islot, km.oslot = full.islot, full.oslot
 
 
 def ensure_nbr(km: KernelMap, transposed: bool) -> None:
@@ -280,14 +284,14 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
                                         km.qkpos.data_ptr(), km.qsum, _ptr(ws), ws_bytes, s))
     elif dataflow == DATAFLOW_FDS:
         ensure_csr(km)
-        need = km.qsum * c_out
+        need = km.M * c_out
         if buffer is None or buffer.numel() < need or buffer.dtype != feats.dtype or buffer.device != dev:
             buffer = torch.empty(max(need, 1), dtype=feats.dtype, device=dev)
         imap = km.omap if transposed else km.imap
-        ocsr, ocode = (km.icsr, km.icode) if transposed else (km.ocsr, km.ocode)
+        ocsr, oslot = (km.icsr, km.islot) if transposed else (km.ocsr, km.oslot)
         _lib.check(lib.pce_conv_fwd_fds(feats.data_ptr(), weight.data_ptr(), _ptr(packed), out.data_ptr(), dt, n_in, n_out,
-                                        c_in, c_out, kv, mid, imap.data_ptr(), km.kpos.data_ptr(), km.qkpos.data_ptr(),
-                                        km.kpos_host, km.qkpos_host, ocsr.data_ptr(), ocode.data_ptr(), km.qsum,
+                                        c_in, c_out, kv, mid, imap.data_ptr(), oslot.data_ptr(), km.kpos.data_ptr(),
+                                        km.qkpos.data_ptr(), km.kpos_host, km.qkpos_host, ocsr.data_ptr(), km.M, km.qsum,
                                         buffer.data_ptr(), buffer.numel(), s))
     elif dataflow == DATAFLOW_GMS:
         ensure_csr(km)

@@ -14,18 +14,27 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
+template <typename T, int N>
+struct VecOfC;
+template <>
+struct VecOfC<half_t, 8> { typedef half8 type; };
+template <>
+struct VecOfC<float, 4> { typedef f32x4 type; };
+template <>
+struct VecOfC<half_t, 4> { typedef _Float16 type __attribute__((ext_vector_type(4))); };
+
 enum {
   MODE_FOD = 0,      // A row = imap[pair], out row = omap[pair]
   MODE_BUF = 1,      // A row = out row = quantised pair row (staging buffer)
   MODE_DENSE = 2,    // A row = out row = tile row, one fixed weight
   MODE_OS = 3,       // out row = tile row, A row = nbr[kp][row], loop over all offsets
-  MODE_FOD_BUF = 4   // A row = imap[pair], out row = quantised pair row (staging buffer)
+  MODE_FOD_BUF = 4   // A row = imap[pair], out row = oslot[pair] (partial-row buffer in output-CSR order)
 };
 enum {
   EPI_ATOMIC_F32 = 0,  // fp32 atomic add, one column per lane
   EPI_ROWS = 1,        // store T, 16 bytes per lane along the row
   EPI_ROWS_F32 = 2,    // store fp32 (accumulator of the atomic dataflow), 16 bytes per lane
-  EPI_ROWS_CSR = 3     // EPI_ROWS plus the sum of the row's staging-buffer rows (CSR-coded list)
+  EPI_ROWS_CSR = 3     // EPI_ROWS plus the sum of partial rows buf[ocsr[row] .. ocsr[row+1])
 };
 
 #define MAX_KV_ARGS 32  // kpos / qkpos travel in the kernel arguments up to this kernel volume
@@ -41,7 +50,7 @@ struct TileArgs {
   const int *qkpos;
   const int *nbr;
   const int *ocsr;
-  const int *ocode;
+  const int *oslot;
   const void *buf;
   long long n_rows;  // MODE_DENSE / MODE_OS: rows of the output
   int kv, c_in, c_out;
@@ -86,38 +95,71 @@ __global__ void __launch_bounds__(256) pack_weights_kernel(const half_t *__restr
   *reinterpret_cast<half8 *>(&P[e * 8]) = v;
 }
 
-// ---- weight chunk -> LDS -----------------------------------------------------------------------
-// fp16 LDS layout: Wl[k/8][n][k%8]
+// Workgroup barrier that orders LDS accesses only.  __syncthreads() also waits for every outstanding
+// global load; here loads for later use (feature rows, partial rows) stay in flight across the
+// barrier and are waited for where their registers are first read.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// ---- weight chunk: global -> registers -> LDS --------------------------------------------------
+// The global loads are issued together with the feature-row loads, before the first barrier of a
+// chunk, so that both latencies overlap; the registers are written to LDS after that barrier.
+// fp16 LDS layout: Wl[k/8][n][k%8];  fp32 LDS layout: Wl[k][n].
+template <typename T, int NT>
+struct WRegs;
 template <int NT>
-__device__ __forceinline__ void stage_weights(half_t *Wl, const half_t *__restrict__ Wk, const half_t *__restrict__ Pk,
-                                              int k0, int n0, const TileArgs &a) {
-  constexpr int KC = Cfg<half_t>::KC;
-  for (int e = threadIdx.x; e < (KC / 8) * NT; e += 256) {
+struct WRegs<half_t, NT> {
+  static constexpr int N = (Cfg<half_t>::KC / 8) * NT / 256;
+  half8 v[N];
+};
+template <int NT>
+struct WRegs<float, NT> {
+  static constexpr int N = Cfg<float>::KC * NT / 4 / 256;
+  f32x4 v[N];
+};
+
+template <int NT, bool FAST>
+__device__ __forceinline__ void load_weights(WRegs<half_t, NT> &r, const half_t *__restrict__ Wk,
+                                             const half_t *__restrict__ Pk, int k0, int n0, const TileArgs &a) {
+#pragma unroll
+  for (int i = 0; i < WRegs<half_t, NT>::N; ++i) {
+    int e = threadIdx.x + i * 256;
     int n = e % NT, k8 = e / NT;
     int gn = n0 + n, gk = k0 + k8 * 8;
     half8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (Pk) {
+    if (FAST || Pk) {
       if (gk / 8 < a.k8_total && gn < a.n_pad) v = *reinterpret_cast<const half8 *>(&Pk[((long long)(gk / 8) * a.n_pad + gn) * 8]);
     } else {
 #pragma unroll
       for (int j = 0; j < 8; ++j)
         if (gn < a.c_out && gk + j < a.c_in) v[j] = Wk[(long long)(gk + j) * a.c_out + gn];
     }
-    *reinterpret_cast<half8 *>(&Wl[(k8 * NT + n) * 8]) = v;
+    r.v[i] = v;
   }
 }
 
-// fp32 LDS layout: Wl[k][n]
 template <int NT>
-__device__ __forceinline__ void stage_weights(float *Wl, const float *__restrict__ Wk, const float * /*Pk*/, int k0,
-                                              int n0, const TileArgs &a) {
-  constexpr int KC = Cfg<float>::KC;
-  for (int e = threadIdx.x; e < KC * NT / 4; e += 256) {
+__device__ __forceinline__ void store_weights(half_t *Wl, const WRegs<half_t, NT> &r) {
+#pragma unroll
+  for (int i = 0; i < WRegs<half_t, NT>::N; ++i) {
+    int e = threadIdx.x + i * 256;
+    int n = e % NT, k8 = e / NT;
+    *reinterpret_cast<half8 *>(&Wl[(k8 * NT + n) * 8]) = r.v[i];
+  }
+}
+
+template <int NT, bool FAST>
+__device__ __forceinline__ void load_weights(WRegs<float, NT> &r, const float *__restrict__ Wk, const float * /*Pk*/,
+                                             int k0, int n0, const TileArgs &a) {
+#pragma unroll
+  for (int i = 0; i < WRegs<float, NT>::N; ++i) {
+    int e = threadIdx.x + i * 256;
     int n = (e % (NT / 4)) * 4, k = e / (NT / 4);
     int gn = n0 + n, gk = k0 + k;
     f32x4 v = {0.f, 0.f, 0.f, 0.f};
     if (gk < a.c_in) {
-      if (a.w_vec && gn + 4 <= a.c_out) {
+      if (FAST) {
+        if (gn < a.c_out) v = *reinterpret_cast<const f32x4 *>(&Wk[(long long)gk * a.c_out + gn]);
+      } else if (a.w_vec && gn + 4 <= a.c_out) {
         v = *reinterpret_cast<const f32x4 *>(&Wk[(long long)gk * a.c_out + gn]);
       } else {
 #pragma unroll
@@ -125,25 +167,44 @@ __device__ __forceinline__ void stage_weights(float *Wl, const float *__restrict
           if (gn + j < a.c_out) v[j] = Wk[(long long)gk * a.c_out + gn + j];
       }
     }
-    *reinterpret_cast<f32x4 *>(&Wl[k * NT + n]) = v;
+    r.v[i] = v;
   }
 }
 
-// ---- one K chunk of MFMA work for a wavefront ---------------------------------------------------
-template <int NB>
-__device__ __forceinline__ void mma_chunk(f32x16 (&acc)[NB], const half_t *Wl, const half_t *__restrict__ A,
-                                          int arow, int k0, int klen, int c_in, int a_vec, int l32, int g) {
-  constexpr int NT = NB * 32;
-  constexpr int KC = Cfg<half_t>::KC;
-  half8 a[KC / 16];
-  // issue every row load of the chunk before the first MFMA
+template <int NT>
+__device__ __forceinline__ void store_weights(float *Wl, const WRegs<float, NT> &r) {
 #pragma unroll
-  for (int s = 0; s < KC / 16; ++s) {
+  for (int i = 0; i < WRegs<float, NT>::N; ++i) {
+    int e = threadIdx.x + i * 256;
+    int n = (e % (NT / 4)) * 4, k = e / (NT / 4);
+    *reinterpret_cast<f32x4 *>(&Wl[k * NT + n]) = r.v[i];
+  }
+}
+
+// ---- feature rows of one K chunk: global -> registers in MFMA operand order -------------------
+template <typename T>
+struct AFrag;
+template <>
+struct AFrag<half_t> {
+  half8 v[Cfg<half_t>::KC / 16];
+};
+template <>
+struct AFrag<float> {
+  f32x4 v[Cfg<float>::KC / 8];
+};
+
+template <bool FAST>
+__device__ __forceinline__ void load_rows(AFrag<half_t> &f, const half_t *__restrict__ A, int arow, int k0, int klen,
+                                          int c_in, int a_vec, int g) {
+#pragma unroll
+  for (int s = 0; s < Cfg<half_t>::KC / 16; ++s) {
     int k = k0 + s * 16 + g * 8;
     half8 v = {0, 0, 0, 0, 0, 0, 0, 0};
     if (arow >= 0 && s * 16 < klen) {
       const half_t *p = A + (long long)arow * c_in + k;
-      if (a_vec && k + 8 <= c_in) {
+      if (FAST) {
+        if (k < c_in) v = *reinterpret_cast<const half8 *>(p);
+      } else if (a_vec && k + 8 <= c_in) {
         v = *reinterpret_cast<const half8 *>(p);
       } else {
 #pragma unroll
@@ -151,33 +212,22 @@ __device__ __forceinline__ void mma_chunk(f32x16 (&acc)[NB], const half_t *Wl, c
           if (k + j < c_in) v[j] = p[j];
       }
     }
-    a[s] = v;
-  }
-#pragma unroll
-  for (int s = 0; s < KC / 16; ++s) {
-    if (s * 16 < klen) {
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        half8 b = *reinterpret_cast<const half8 *>(&Wl[((s * 2 + g) * NT + nb * 32 + l32) * 8]);
-        acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[s], b, acc[nb], 0, 0, 0);
-      }
-    }
+    f.v[s] = v;
   }
 }
 
-template <int NB>
-__device__ __forceinline__ void mma_chunk(f32x16 (&acc)[NB], const float *Wl, const float *__restrict__ A, int arow,
-                                          int k0, int klen, int c_in, int a_vec, int l32, int g) {
-  constexpr int NT = NB * 32;
-  constexpr int KC = Cfg<float>::KC;
-  f32x4 a[KC / 8];
+template <bool FAST>
+__device__ __forceinline__ void load_rows(AFrag<float> &f, const float *__restrict__ A, int arow, int k0, int klen,
+                                          int c_in, int a_vec, int g) {
 #pragma unroll
-  for (int s = 0; s < KC / 8; ++s) {
+  for (int s = 0; s < Cfg<float>::KC / 8; ++s) {
     int k = k0 + s * 8 + g * 4;
     f32x4 v = {0.f, 0.f, 0.f, 0.f};
     if (arow >= 0 && s * 8 < klen) {
       const float *p = A + (long long)arow * c_in + k;
-      if (a_vec && k + 4 <= c_in) {
+      if (FAST) {
+        if (k < c_in) v = *reinterpret_cast<const f32x4 *>(p);
+      } else if (a_vec && k + 4 <= c_in) {
         v = *reinterpret_cast<const f32x4 *>(p);
       } else {
 #pragma unroll
@@ -185,10 +235,40 @@ __device__ __forceinline__ void mma_chunk(f32x16 (&acc)[NB], const float *Wl, co
           if (k + j < c_in) v[j] = p[j];
       }
     }
-    a[s] = v;
+    f.v[s] = v;
   }
+}
+
+// ---- one K chunk of MFMA work for a wavefront ---------------------------------------------------
+// ROWMAJOR = false: D[row][col], lane (l32, g) holds column l32 of rows 8*(j/4) + 4*g + j%4 (one
+//   column per lane: what the atomic epilogue wants).
+// ROWMAJOR = true: the operands are exchanged, D'[col][row]: lane (l32, g) holds, for ITS OWN row
+//   l32, columns 8*(j/4) + 4*g + j%4 of every 32-column block (what the row epilogue wants).
+template <int NB, bool ROWMAJOR>
+__device__ __forceinline__ void mma_chunk(f32x16 (&acc)[NB], const half_t *Wl, const AFrag<half_t> &f, int klen,
+                                          int l32, int g) {
+  constexpr int NT = NB * 32;
 #pragma unroll
-  for (int s = 0; s < KC / 8; ++s) {
+  for (int s = 0; s < Cfg<half_t>::KC / 16; ++s) {
+    if (s * 16 < klen) {
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        half8 b = *reinterpret_cast<const half8 *>(&Wl[((s * 2 + g) * NT + nb * 32 + l32) * 8]);
+        if (ROWMAJOR)
+          acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b, f.v[s], acc[nb], 0, 0, 0);
+        else
+          acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.v[s], b, acc[nb], 0, 0, 0);
+      }
+    }
+  }
+}
+
+template <int NB, bool ROWMAJOR>
+__device__ __forceinline__ void mma_chunk(f32x16 (&acc)[NB], const float *Wl, const AFrag<float> &f, int klen,
+                                          int l32, int g) {
+  constexpr int NT = NB * 32;
+#pragma unroll
+  for (int s = 0; s < Cfg<float>::KC / 8; ++s) {
     if (s * 8 < klen) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -197,7 +277,10 @@ __device__ __forceinline__ void mma_chunk(f32x16 (&acc)[NB], const float *Wl, co
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
           float b = Wl[kk * NT + nb * 32 + l32];
-          acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s][e], b, acc[nb], 0, 0, 0);
+          if (ROWMAJOR)
+            acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(b, f.v[s][e], acc[nb], 0, 0, 0);
+          else
+            acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.v[s][e], b, acc[nb], 0, 0, 0);
         }
       }
     }
@@ -205,7 +288,6 @@ __device__ __forceinline__ void mma_chunk(f32x16 (&acc)[NB], const float *Wl, co
 }
 
 // ---- epilogues ---------------------------------------------------------------------------------
-// MFMA layout: lane (l32, g) holds column l32 of rows 8*(j/4) + 4*g + j%4, j = 0..15.
 template <int NB>
 __device__ __forceinline__ void epilogue_atomic(const f32x16 (&acc)[NB], int orow, const TileArgs &a, int n0, int l32,
                                                 int g) {
@@ -222,108 +304,211 @@ __device__ __forceinline__ void epilogue_atomic(const f32x16 (&acc)[NB], int oro
   }
 }
 
-template <typename TB, int CPL>
-__device__ __forceinline__ void add_buf_row(float (&v)[CPL], const TB *__restrict__ p, int ncol, int vec_ok);
-
-template <>
-__device__ __forceinline__ void add_buf_row<half_t, 8>(float (&v)[8], const half_t *__restrict__ p, int ncol, int vec_ok) {
-  if (vec_ok && ncol >= 8) {
-    half8 b = *reinterpret_cast<const half8 *>(p);
+// Row epilogue, first step: the two lanes of a row (g = 0, 1) exchange 4-column pieces so that each
+// ends with 8 consecutive columns per 16-column group: lane g owns columns 16*h + 8*g + 0..7,
+// h = 0, 1, of every 32-column block.
+template <int NB>
+__device__ __forceinline__ void gather_row_pieces(const f32x16 (&acc)[NB], float (&V)[NB][2][8], int g) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] += (float)b[j];
-  } else {
-    for (int j = 0; j < 8 && j < ncol; ++j) v[j] += (float)p[j];
-  }
-}
-template <>
-__device__ __forceinline__ void add_buf_row<float, 4>(float (&v)[4], const float *__restrict__ p, int ncol, int vec_ok) {
-  if (vec_ok && ncol >= 4) {
-    f32x4 b = *reinterpret_cast<const f32x4 *>(p);
+  for (int nb = 0; nb < NB; ++nb) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) v[j] += b[j];
-  } else {
-    for (int j = 0; j < 4 && j < ncol; ++j) v[j] += p[j];
-  }
-}
-template <>
-__device__ __forceinline__ void add_buf_row<half_t, 4>(float (&)[4], const half_t *__restrict__, int, int) {}
-
-// Row-wise epilogue.  The wavefront transposes its 32 x NT accumulator through LDS, 16 rows at a
-// time, so that a lane owns CPL consecutive columns of one row: stores (and the staging-buffer
-// rows added in EPI_ROWS_CSR) are 16-byte accesses along the row.
-template <typename T, int NB, bool F32OUT>
-__device__ __forceinline__ void epilogue_rows(const f32x16 (&acc)[NB], float *El, int orow, int e0, int e1,
-                                              const TileArgs &a, int n0, int lane, int l32, int g) {
-  constexpr int NT = NB * 32, LD = NT + 8;
-  constexpr int CPL = (F32OUT || sizeof(T) == 4) ? 4 : 8;
-  constexpr int LPR = NT / CPL;
-  const bool csr = a.epi == EPI_ROWS_CSR;
+    for (int h = 0; h < 2; ++h) {
+      const int qa = 2 * h, qb = 2 * h + 1;  // lane g=0 keeps piece qa, lane g=1 keeps piece qb
 #pragma unroll
-  for (int half = 0; half < 2; ++half) {
-#pragma unroll
-    for (int jj = 0; jj < 8; ++jj) {
-      int lr = 8 * (jj >> 2) + 4 * g + (jj & 3);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) El[lr * LD + nb * 32 + l32] = acc[nb][8 * half + jj];
-    }
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    for (int idx = lane; idx < 16 * LPR; idx += 64) {  // 16 * LPR is a multiple of 64
-      int lr = idx / LPR, ch = idx - lr * LPR;
-      int r = 16 * half + lr;
-      int dst = __shfl(orow, r, PCE_WAVE);
-      int s0 = __shfl(e0, r, PCE_WAVE), s1 = __shfl(e1, r, PCE_WAVE);
-      int col = n0 + ch * CPL;
-      int ncol = a.c_out - col;
-      if (dst < 0 || ncol <= 0) continue;
-      float v[CPL];
-#pragma unroll
-      for (int q4 = 0; q4 < CPL / 4; ++q4) {
-        f32x4 x = *reinterpret_cast<const f32x4 *>(&El[lr * LD + ch * CPL + q4 * 4]);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) v[q4 * 4 + j] = x[j];
-      }
-      if (csr) {
-        const T *buf = (const T *)a.buf;
-        for (int e = s0; e < s1; ++e) {
-          int code = a.ocode[e];
-          int kq = code / PCE_CSR_CODE;
-          long long q = (long long)(a.host_pos ? a.qkpos_h[kq] : a.qkpos[kq]) + (code - kq * PCE_CSR_CODE);
-          add_buf_row<T, CPL>(v, buf + q * a.c_out + col, ncol, a.b_vec);
-        }
-      }
-      long long off = (long long)dst * a.c_out + col;
-      if (F32OUT || sizeof(T) == 4) {
-        float *o = (float *)a.out + off;
-        if (a.o_vec && ncol >= 4) {
-          f32x4 y = {v[0], v[1], v[2], v[3]};
-          *reinterpret_cast<f32x4 *>(o) = y;
-        } else {
-          for (int j = 0; j < 4 && j < ncol; ++j) o[j] = v[j];
-        }
-      } else {
-        half_t *o = (half_t *)a.out + off;
-        if (a.o_vec && ncol >= 8) {
-          half8 y;
-#pragma unroll
-          for (int j = 0; j < CPL; ++j) y[j] = (half_t)v[j];
-          *reinterpret_cast<half8 *>(o) = y;
-        } else {
-          for (int j = 0; j < CPL && j < ncol; ++j) o[j] = (half_t)v[j];
-        }
+      for (int i = 0; i < 4; ++i) {
+        float lo = acc[nb][4 * qa + i], hi = acc[nb][4 * qb + i];
+        float recv = __shfl_xor(g == 0 ? hi : lo, 32, PCE_WAVE);
+        V[nb][h][i] = g == 0 ? lo : recv;
+        V[nb][h][4 + i] = g == 0 ? recv : hi;
       }
     }
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    __builtin_amdgcn_wave_barrier();
   }
 }
+
+// Per-wavefront LDS region, in 16-byte pieces: big enough for 16 fp32 rows or 32 fp16 rows of the
+// output tile with 8 elements of padding per row.  It first stages partial rows, then the finished
+// rows on their way to memory.
+template <int NB>
+struct WaveLds {
+  static constexpr int NT = NB * 32;
+  static constexpr int PIECES = 4 * (NT + 8);
+};
+
+// Partial rows of a tile's 128 output rows are one contiguous range [tb, te) of the buffer.  The
+// workgroup copies it through LDS CH rows at a time with coalesced 16-byte loads (PARTIAL_LOADS per
+// thread, all in flight together; the first round is requested at kernel start), and every lane
+// adds the rows [e0, e1) of its own output row.  Sharing the rounds among the four wavefronts keeps
+// a tile inside a dense cluster from serialising many small rounds in one wavefront.
+#define PARTIAL_LOADS 4  // 16-byte pieces per thread and round
 
 template <typename T, int NB>
-__global__ void __launch_bounds__(256) tile_gemm_kernel(TileArgs a) {
+struct Partials {
+  static constexpr int NT = NB * 32;
+  static constexpr int CPL = 16 / sizeof(T);  // elements per 16-byte piece
+  static constexpr int PPR = NT / CPL;        // pieces per partial row (of this column slab)
+  static constexpr int LOADS = PARTIAL_LOADS;
+  static constexpr int CAP = LOADS * 256 < 4 * WaveLds<NB>::PIECES ? LOADS * 256 : 4 * WaveLds<NB>::PIECES;
+  static constexpr int CH = CAP / PPR;        // partial rows per round
+  typedef typename VecOfC<T, CPL>::type PV;
+};
+
+template <typename T, int NB, typename PV>
+__device__ __forceinline__ void load_partial_chunk(PV (&r)[PARTIAL_LOADS], int cb, int te, const TileArgs &a, int n0) {
+  typedef Partials<T, NB> P;
+  const T *buf = (const T *)a.buf;
+#pragma unroll
+  for (int i = 0; i < P::LOADS; ++i) {
+    int pc = threadIdx.x + 256 * i;
+    int ent = pc / P::PPR, piece = pc - ent * P::PPR;
+    int e = cb + ent;
+    int col = n0 + piece * P::CPL;
+    PV v;
+#pragma unroll
+    for (int j = 0; j < P::CPL; ++j) v[j] = (T)0;
+    if (ent < P::CH && e < te && col < a.c_out) v = *reinterpret_cast<const PV *>(buf + (long long)e * a.c_out + col);
+    r[i] = v;
+  }
+}
+
+template <typename T, int NB, typename PV>
+__device__ __forceinline__ void add_partials(float (&V)[NB][2][8], PV *Pl, PV (&first)[PARTIAL_LOADS], int e0, int e1,
+                                             int tb, int te, const TileArgs &a, int n0, int g) {
+  typedef Partials<T, NB> P;
+  for (int cb = tb; cb < te; cb += P::CH) {  // tb, te are uniform over the workgroup
+    if (cb > tb) load_partial_chunk<T, NB, PV>(first, cb, te, a, n0);
+#pragma unroll
+    for (int i = 0; i < P::LOADS; ++i)
+      if (threadIdx.x + 256 * i < P::CH * P::PPR) Pl[threadIdx.x + 256 * i] = first[i];
+    lds_barrier();
+    int lo = e0 > cb ? e0 : cb, hi = e1 < cb + P::CH ? e1 : cb + P::CH;
+    for (int e = lo; e < hi; ++e) {
+      const PV *rowp = Pl + (e - cb) * P::PPR;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          if (sizeof(T) == 2) {
+            PV x = rowp[nb * 4 + 2 * h + g];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) V[nb][h][j] += (float)x[j % P::CPL];
+          } else {
+            PV x0 = rowp[nb * 8 + 4 * h + 2 * g], x1 = rowp[nb * 8 + 4 * h + 2 * g + 1];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              V[nb][h][j] += (float)x0[j];
+              V[nb][h][4 + j] += (float)x1[j];
+            }
+          }
+        }
+      }
+    }
+    lds_barrier();  // the region is rewritten by the next round or by the store phase
+  }
+}
+
+// element-wise partial-row sum for rows that are not 16-byte multiples
+template <typename T, int NB>
+__device__ __forceinline__ void add_partials_slow(float (&V)[NB][2][8], int e0, int e1, const TileArgs &a, int n0,
+                                                  int g) {
+  const T *buf = (const T *)a.buf;
+  for (int e = e0; e < e1; ++e) {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          int col = n0 + nb * 32 + 16 * h + 8 * g + j;
+          if (col < a.c_out) V[nb][h][j] += (float)buf[(long long)e * a.c_out + col];
+        }
+  }
+}
+
+// element-wise stores straight from the row pieces (rows that are not 16-byte multiples)
+template <typename TO, int NB>
+__device__ __forceinline__ void store_row_pieces_slow(const float (&V)[NB][2][8], TO *out, int orow, const TileArgs &a,
+                                                      int n0, int g) {
+  if (orow < 0) return;
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        int col = n0 + nb * 32 + 16 * h + 8 * g + j;
+        if (col < a.c_out) out[(long long)orow * a.c_out + col] = (TO)V[nb][h][j];
+      }
+}
+
+// Finished rows -> memory through the wavefront's LDS region: the lane that owns (row, 8 columns)
+// writes its pieces; then 16 bytes per lane are read back along the rows, so that NT*sizeof(TO)/16
+// consecutive lanes store one full row segment (whole 128-byte lines at 64 fp16 channels).
+template <typename TO, int NB>
+__device__ __forceinline__ void store_rows_via_lds(const float (&V)[NB][2][8], void *region, TO *out, int orow,
+                                                   const TileArgs &a, int n0, int lane, int l32, int g) {
+  constexpr int NT = NB * 32;
+  constexpr int EPP = 16 / sizeof(TO);              // elements per piece
+  constexpr int LDP = (NT + 8) / EPP;               // row stride in pieces
+  constexpr int ROWS = sizeof(TO) == 2 ? 32 : 16;   // rows per pass
+  constexpr int PPR = NT / EPP;                     // pieces per row
+  constexpr int ITS = ROWS * PPR / 64;
+  typedef typename VecOfC<TO, EPP>::type OV;
+  OV *R = (OV *)region;
+#pragma unroll
+  for (int pass = 0; pass < 32 / ROWS; ++pass) {
+    if (ROWS == 32 || (l32 / 16) == pass) {
+      int lr = l32 % ROWS;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          int c0 = nb * 32 + 16 * h + 8 * g;  // first of this lane's 8 columns
+          if (sizeof(TO) == 2) {
+            OV y;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) y[j % EPP] = (TO)V[nb][h][j];
+            R[lr * LDP + c0 / EPP] = y;
+          } else {
+            OV y0, y1;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              y0[j] = (TO)V[nb][h][j];
+              y1[j] = (TO)V[nb][h][4 + j];
+            }
+            R[lr * LDP + c0 / EPP] = y0;
+            R[lr * LDP + c0 / EPP + 1] = y1;
+          }
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int it = 0; it < ITS; ++it) {
+      int idx = it * 64 + lane;
+      int lr = idx / PPR, ch = idx - lr * PPR;
+      int dst = __shfl(orow, pass * ROWS + lr, PCE_WAVE);
+      int col = n0 + ch * EPP;
+      OV y = R[lr * LDP + ch];
+      if (dst >= 0 && col < a.c_out) *reinterpret_cast<OV *>(out + (long long)dst * a.c_out + col) = y;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+// FAST: every row (features, weights or packed weights, output, partial buffer) is a multiple of
+// 16 bytes and 16-byte aligned, fp16 weights are packed: no element-wise access path is compiled.
+// TMODE / TEPI >= 0 fix the mode and the epilogue at compile time (the hot combinations); -1 reads
+// them from the arguments.
+template <typename T, int NB, bool FAST, int TMODE, int TEPI>
+__global__ void __launch_bounds__(256, ((TMODE >= 0 && sizeof(T) == 2 && NB <= 2) ? 5 : 1)) tile_gemm_kernel(TileArgs a) {
+  const int mode = TMODE >= 0 ? TMODE : a.mode;
+  const int epi = TEPI >= 0 ? TEPI : a.epi;
   constexpr int NT = NB * 32;
   constexpr int KC = Cfg<T>::KC;
+  typedef Partials<T, NB> P;
   __shared__ __attribute__((aligned(16))) T Wl[KC * NT];
-  __shared__ __attribute__((aligned(16))) float El[4][16 * (NT + 8)];
+  __shared__ __attribute__((aligned(16))) typename P::PV Pl[4][WaveLds<NB>::PIECES];
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int l32 = lane & 31, g = lane >> 5;
@@ -336,12 +521,12 @@ __global__ void __launch_bounds__(256) tile_gemm_kernel(TileArgs a) {
   int arow = -1, orow = -1;
   int w_begin, w_end;
   long long row = tile * 128 + wave * 32 + l32;
-  if (a.mode == MODE_DENSE || a.mode == MODE_OS) {
+  if (mode == MODE_DENSE || mode == MODE_OS) {
     bool ok = row < a.n_rows;
     orow = ok ? (int)row : -1;
-    arow = (a.mode == MODE_DENSE) ? orow : -1;
-    w_begin = (a.mode == MODE_DENSE) ? a.w_fixed : 0;
-    w_end = (a.mode == MODE_DENSE) ? a.w_fixed + 1 : a.kv;
+    arow = (mode == MODE_DENSE) ? orow : -1;
+    w_begin = (mode == MODE_DENSE) ? a.w_fixed : 0;
+    w_end = (mode == MODE_DENSE) ? a.w_fixed + 1 : a.kv;
   } else {
     // indicator: which offset owns this tile = number of segment ends at or before its first row
     long long q0 = tile * 128;
@@ -366,17 +551,40 @@ __global__ void __launch_bounds__(256) tile_gemm_kernel(TileArgs a) {
       ok = p < (long long)a.kpos[widx + 1];
     }
     if (ok) {
-      arow = (a.mode == MODE_BUF) ? (int)row : a.imap[p];
-      orow = (a.mode == MODE_FOD) ? a.omap[p] : (int)row;
+      arow = (mode == MODE_BUF) ? (int)row : a.imap[p];
+      orow = (mode == MODE_FOD) ? a.omap[p] : (mode == MODE_FOD_BUF ? a.oslot[p] : (int)row);
     }
     w_begin = widx;
     w_end = widx + 1;
   }
-  // CSR range of this lane's row, fetched early: the epilogue needs it last
-  int e0 = 0, e1 = 0;
-  if (a.epi == EPI_ROWS_CSR && orow >= 0) {
-    e0 = a.ocsr[orow];
-    e1 = a.ocsr[orow + 1];
+  // MODE_DENSE and the pair modes use one offset: issue its first chunk of loads now, ahead of the
+  // partial-row metadata, so that nothing delays them
+  const int klen0 = a.c_in < KC ? a.c_in : KC;
+  WRegs<T, NT> wr;
+  AFrag<T> af;
+  if (mode != MODE_OS) {
+    load_weights<NT, FAST>(wr, W + (long long)w_begin * a.c_in * a.c_out,
+                           Wp ? Wp + (long long)w_begin * a.k8_total * a.n_pad * 8 : nullptr, 0, n0, a);
+    load_rows<FAST>(af, A, arow, 0, klen0, a.c_in, a.a_vec, g);
+  }
+  // Partial rows: the tile's contiguous range [tb, te) comes from two scalar loads (uniform index),
+  // so the first round of partial rows is requested together with the feature rows; the per-lane
+  // bounds [e0, e1) of the lane's own row are only needed in the epilogue.
+  int e0 = 0, e1 = 0, tb = 0, te = 0;
+  typename P::PV first[P::LOADS];
+  const bool csr_fast = (epi == EPI_ROWS_CSR) && (FAST || a.b_vec);
+  if (epi == EPI_ROWS_CSR) {
+    long long r0 = tile * 128;
+    if (r0 < a.n_rows) {
+      long long r1 = r0 + 128 < a.n_rows ? r0 + 128 : a.n_rows;
+      tb = a.ocsr[r0];
+      te = a.ocsr[r1];
+    }
+    if (csr_fast) load_partial_chunk<T, NB, typename P::PV>(first, tb, te, a, n0);
+    if (orow >= 0) {
+      e0 = a.ocsr[orow];
+      e1 = a.ocsr[orow + 1];
+    }
   }
 
   f32x16 acc[NB];
@@ -385,8 +593,10 @@ __global__ void __launch_bounds__(256) tile_gemm_kernel(TileArgs a) {
 #pragma unroll
     for (int j = 0; j < 16; ++j) acc[nb][j] = 0.f;
 
+  const bool rowmajor = epi != EPI_ATOMIC_F32;
+  bool lds_used = false;
   for (int w = w_begin; w < w_end; ++w) {
-    if (a.mode == MODE_OS) {
+    if (mode == MODE_OS) {
       arow = orow >= 0 ? a.nbr[(long long)w * a.n_rows + orow] : -1;
       if (!__syncthreads_or(arow >= 0)) continue;
     }
@@ -394,20 +604,62 @@ __global__ void __launch_bounds__(256) tile_gemm_kernel(TileArgs a) {
     const T *Wk = W + (long long)w * a.c_in * a.c_out;
     const T *Pk = Wp ? Wp + (long long)w * a.k8_total * a.n_pad * 8 : nullptr;
     for (int k0 = 0; k0 < a.c_in; k0 += KC) {
-      __syncthreads();
-      stage_weights<NT>(Wl, Wk, Pk, k0, n0, a);
-      __syncthreads();
       int klen = a.c_in - k0 < KC ? a.c_in - k0 : KC;
-      if (wave_has) mma_chunk<NB>(acc, Wl, A, arow, k0, klen, a.c_in, a.a_vec, l32, g);
+      if (mode == MODE_OS || k0 > 0) {
+        load_weights<NT, FAST>(wr, Wk, Pk, k0, n0, a);
+        load_rows<FAST>(af, A, arow, k0, klen, a.c_in, a.a_vec, g);
+      }
+      if (lds_used) lds_barrier();  // the previous chunk's LDS reads are complete
+      store_weights<NT>(Wl, wr);
+      lds_barrier();
+      lds_used = true;
+      if (wave_has) {
+        if (rowmajor)
+          mma_chunk<NB, true>(acc, Wl, af, klen, l32, g);
+        else
+          mma_chunk<NB, false>(acc, Wl, af, klen, l32, g);
+      }
     }
   }
 
-  if (a.epi == EPI_ATOMIC_F32) {
+  if (!rowmajor) {
     epilogue_atomic<NB>(acc, orow, a, n0, l32, g);
-  } else if (a.epi == EPI_ROWS_F32) {
-    epilogue_rows<T, NB, true>(acc, El[wave], orow, e0, e1, a, n0, lane, l32, g);
+    return;
+  }
+  float V[NB][2][8];
+  gather_row_pieces<NB>(acc, V, g);
+  if (epi == EPI_ROWS_CSR) {
+    if (csr_fast)
+      add_partials<T, NB, typename P::PV>(V, &Pl[0][0], first, e0, e1, tb, te, a, n0, g);
+    else
+      add_partials_slow<T, NB>(V, e0, e1, a, n0, g);
+  }
+  const bool f32out = (epi == EPI_ROWS_F32) || sizeof(T) == 4;
+  if (FAST || a.o_vec) {
+    if (f32out)
+      store_rows_via_lds<float, NB>(V, Pl[wave], (float *)a.out, orow, a, n0, lane, l32, g);
+    else
+      store_rows_via_lds<half_t, NB>(V, Pl[wave], (half_t *)a.out, orow, a, n0, lane, l32, g);
   } else {
-    epilogue_rows<T, NB, false>(acc, El[wave], orow, e0, e1, a, n0, lane, l32, g);
+    if (f32out)
+      store_row_pieces_slow<float, NB>(V, (float *)a.out, orow, a, n0, g);
+    else
+      store_row_pieces_slow<half_t, NB>(V, (half_t *)a.out, orow, a, n0, g);
+  }
+}
+
+template <typename T, bool FAST, int TMODE, int TEPI>
+static void launch_tile_nb(const TileArgs &a, long long tiles, hipStream_t s) {
+  int nb = (a.c_out + 31) / 32;
+  if (nb >= 4) {
+    dim3 grid((unsigned)tiles, (unsigned)((a.c_out + 127) / 128));
+    hipLaunchKernelGGL((tile_gemm_kernel<T, 4, FAST, TMODE, TEPI>), grid, dim3(256), 0, s, a);
+  } else if (nb == 3) {
+    hipLaunchKernelGGL((tile_gemm_kernel<T, 3, FAST, TMODE, TEPI>), dim3((unsigned)tiles, 1), dim3(256), 0, s, a);
+  } else if (nb == 2) {
+    hipLaunchKernelGGL((tile_gemm_kernel<T, 2, FAST, TMODE, TEPI>), dim3((unsigned)tiles, 1), dim3(256), 0, s, a);
+  } else {
+    hipLaunchKernelGGL((tile_gemm_kernel<T, 1, FAST, TMODE, TEPI>), dim3((unsigned)tiles, 1), dim3(256), 0, s, a);
   }
 }
 
@@ -415,17 +667,26 @@ template <typename T>
 static int launch_tile(const TileArgs &a, long long tiles, hipStream_t s) {
   if (tiles <= 0) return PCE_OK;
   if (tiles >= (1ll << 31)) PCE_FAIL(PCE_ECAPACITY, "tile count %lld exceeds the grid limit", tiles);
-  int nb = (a.c_out + 31) / 32;
-  if (nb >= 4) {
-    dim3 grid((unsigned)tiles, (unsigned)((a.c_out + 127) / 128));
-    hipLaunchKernelGGL((tile_gemm_kernel<T, 4>), grid, dim3(256), 0, s, a);
-  } else if (nb == 3) {
-    hipLaunchKernelGGL((tile_gemm_kernel<T, 3>), dim3((unsigned)tiles, 1), dim3(256), 0, s, a);
-  } else if (nb == 2) {
-    hipLaunchKernelGGL((tile_gemm_kernel<T, 2>), dim3((unsigned)tiles, 1), dim3(256), 0, s, a);
-  } else {
-    hipLaunchKernelGGL((tile_gemm_kernel<T, 1>), dim3((unsigned)tiles, 1), dim3(256), 0, s, a);
-  }
+  bool fast = a.a_vec && a.o_vec && (sizeof(T) == 2 ? a.Wp != nullptr : a.w_vec != 0) &&
+              (a.epi != EPI_ROWS_CSR || a.b_vec);
+  if (!fast)
+    launch_tile_nb<T, false, -1, -1>(a, tiles, s);
+  else if (a.mode == MODE_DENSE && a.epi == EPI_ROWS_CSR)
+    launch_tile_nb<T, true, MODE_DENSE, EPI_ROWS_CSR>(a, tiles, s);
+  else if (a.mode == MODE_DENSE && a.epi == EPI_ROWS)
+    launch_tile_nb<T, true, MODE_DENSE, EPI_ROWS>(a, tiles, s);
+  else if (a.mode == MODE_FOD_BUF && a.epi == EPI_ROWS)
+    launch_tile_nb<T, true, MODE_FOD_BUF, EPI_ROWS>(a, tiles, s);
+  else if (a.mode == MODE_OS && a.epi == EPI_ROWS)
+    launch_tile_nb<T, true, MODE_OS, EPI_ROWS>(a, tiles, s);
+  else if (a.mode == MODE_FOD && a.epi == EPI_ATOMIC_F32)
+    launch_tile_nb<T, true, MODE_FOD, EPI_ATOMIC_F32>(a, tiles, s);
+  else if (a.mode == MODE_BUF && a.epi == EPI_ROWS)
+    launch_tile_nb<T, true, MODE_BUF, EPI_ROWS>(a, tiles, s);
+  else if (a.mode == MODE_DENSE && a.epi == EPI_ROWS_F32)
+    launch_tile_nb<T, true, MODE_DENSE, EPI_ROWS_F32>(a, tiles, s);
+  else
+    launch_tile_nb<T, true, -1, -1>(a, tiles, s);
   PCE_LAUNCH_CHECK("tile_gemm");
   return PCE_OK;
 }
@@ -491,6 +752,33 @@ __global__ void __launch_bounds__(256) scatter_rows_kernel(const T *__restrict__
       int code = ocode[e];
       long long q = (long long)qkpos[code / PCE_CSR_CODE] + code % PCE_CSR_CODE;
       V x = *reinterpret_cast<const V *>(&buf[q * c_out + (long long)v * VEC]);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) acc[j] += (float)(reinterpret_cast<const T *>(&x)[j]);
+    }
+    V y;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) reinterpret_cast<T *>(&y)[j] = (T)acc[j];
+    *reinterpret_cast<V *>(&out[row * c_out + (long long)v * VEC]) = y;
+  }
+}
+
+// out[row] = sum of the contiguous partial rows buf[csr[row] .. csr[row+1]), fp32 accumulate
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256) rowsum_kernel(const T *__restrict__ buf, long long n_out, int c_out, int G,
+                                                     const int *__restrict__ csr, T *__restrict__ out) {
+  typedef typename VecOf<T, VEC>::type V;
+  int rows_per_block = 256 / G;
+  long long row = (long long)blockIdx.x * rows_per_block + threadIdx.x / G;
+  int sub = threadIdx.x % G;
+  if (row >= n_out) return;
+  int e0 = csr[row], e1 = csr[row + 1];
+  int row_vecs = c_out / VEC;
+  for (int v = sub; v < row_vecs; v += G) {
+    float acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
+    for (int e = e0; e < e1; ++e) {
+      V x = *reinterpret_cast<const V *>(&buf[(long long)e * c_out + (long long)v * VEC]);
 #pragma unroll
       for (int j = 0; j < VEC; ++j) acc[j] += (float)(reinterpret_cast<const T *>(&x)[j]);
     }
@@ -578,10 +866,10 @@ static TileArgs base_args(const void *in, const void *w, const void *wp, int kv,
 }
 
 template <typename T>
-static void set_out(TileArgs *a, void *out, bool f32out) {
-  int vec = (f32out || sizeof(T) == 4) ? 4 : 8;
+static void set_out(TileArgs *a, void *out, bool /*f32out*/) {
+  // a lane of the row epilogue owns 8 consecutive columns, whatever the element type
   a->out = out;
-  a->o_vec = (a->c_out % vec == 0) && aligned16(out);
+  a->o_vec = (a->c_out % 8 == 0) && aligned16(out);
 }
 
 static void set_host_pos(TileArgs *a, const int32_t *kpos_host, const int32_t *qkpos_host) {
@@ -757,20 +1045,22 @@ extern "C" int pce_conv_fwd_gms(const void *in, const void *w, const void *wp, v
   return gms_impl<float>(in, w, wp, out, n_in, n_out, c_in, c_out, kv, mid, icsr, icode, ocsr, ocode, kpos, qkpos, qsum, (float *)buffer, s);
 }
 
-// Fetch-on-demand with deferred scatter: pair tiles gather their input rows, multiply and store
-// the partial rows to the staging buffer (no atomics); the scatter is the epilogue of the centre
-// GEMM, which adds each output row's staging rows in fp32 and stores the row once.
+// Fetch-on-demand with deferred scatter: pair tiles gather their input rows, multiply and store the
+// partial row at its slot in output-CSR order (no atomics); the scatter is the epilogue of the
+// centre GEMM, which adds each output row's contiguous partial rows in fp32 and stores the row once.
 template <typename T>
 static int fds_impl(const void *in, const void *w, const void *wp, void *out, int64_t n_out, int c_in, int c_out, int kv,
-                    int mid, const int *imap, const int *kpos, const int *qkpos, const int32_t *kpos_host,
-                    const int32_t *qkpos_host, const int *ocsr, const int *ocode, int64_t qsum, T *buffer,
+                    int mid, const int *imap, const int *oslot, const int *kpos, const int *qkpos,
+                    const int32_t *kpos_host, const int32_t *qkpos_host, const int *ocsr, int64_t qsum, T *buffer,
                     hipStream_t s) {
+  constexpr int VEC = sizeof(T) == 2 ? 8 : 4;
   int rc;
   if (qsum > 0 && stage_on(1)) {
     TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
     set_out<T>(&a, buffer, false);
     set_host_pos(&a, kpos_host, qkpos_host);
     a.imap = imap;
+    a.oslot = oslot;
     a.kpos = kpos;
     a.qkpos = qkpos;
     a.mode = MODE_FOD_BUF;
@@ -781,35 +1071,46 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
   if (mid >= 0) {
     TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
     set_out<T>(&a, out, false);
-    set_host_pos(&a, kpos_host, qkpos_host);
-    a.qkpos = qkpos;
     a.mode = MODE_DENSE;
     a.epi = EPI_ROWS_CSR;
     a.w_fixed = mid;
     a.n_rows = n_out;
     a.ocsr = ocsr;
-    a.ocode = ocode;
     a.buf = buffer;
-    a.b_vec = a.o_vec && aligned16(buffer);
+    a.b_vec = (c_out % 8 == 0) && aligned16(buffer);
     return launch_tile<T>(a, pce_div_up(n_out, 128), s);
   }
-  return launch_scatter<T>(buffer, (T *)out, n_out, c_out, ocsr, ocode, qkpos, 0, s);
+  bool vec = (c_out % VEC == 0) && aligned16(out) && aligned16(buffer);
+  if (vec) {
+    int G = pow2_at_least(c_out / VEC);
+    if (G > 64) G = 64;
+    hipLaunchKernelGGL((rowsum_kernel<T, VEC>), dim3((unsigned)pce_div_up(n_out, 256 / G)), dim3(256), 0, s,
+                       (const T *)buffer, (long long)n_out, c_out, G, ocsr, (T *)out);
+  } else {
+    int G = pow2_at_least(c_out);
+    if (G > 64) G = 64;
+    hipLaunchKernelGGL((rowsum_kernel<T, 1>), dim3((unsigned)pce_div_up(n_out, 256 / G)), dim3(256), 0, s,
+                       (const T *)buffer, (long long)n_out, c_out, G, ocsr, (T *)out);
+  }
+  PCE_LAUNCH_CHECK("rowsum");
+  return PCE_OK;
 }
 
 extern "C" int pce_conv_fwd_fds(const void *in, const void *w, const void *wp, void *out, int32_t dtype, int64_t n_in,
                                 int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv, int32_t mid, const int32_t *imap,
-                                const int32_t *kpos, const int32_t *qkpos, const int32_t *kpos_host,
-                                const int32_t *qkpos_host, const int32_t *ocsr, const int32_t *ocode, int64_t qsum,
-                                void *buffer, int64_t buffer_elems, pce_stream_t stream) {
+                                const int32_t *oslot, const int32_t *kpos, const int32_t *qkpos,
+                                const int32_t *kpos_host, const int32_t *qkpos_host, const int32_t *ocsr,
+                                int64_t n_pairs, int64_t qsum, void *buffer, int64_t buffer_elems, pce_stream_t stream) {
   int rc = check_common("pce_conv_fwd_fds", in, w, out, dtype, n_in, n_out, c_in, c_out, kv, mid);
   if (rc || (rc = check_qsum("pce_conv_fwd_fds", qsum))) return rc;
-  if (!ocsr || !kpos || !qkpos || (qsum > 0 && (!imap || !ocode))) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_fds: null map pointer");
-  if (qsum > 0 && (!buffer || buffer_elems < qsum * (int64_t)c_out))
-    PCE_FAIL(PCE_EWORKSPACE, "pce_conv_fwd_fds: buffer holds %lld elements, needs %lld", (long long)buffer_elems, (long long)(qsum * (int64_t)c_out));
+  if (!ocsr || !kpos || !qkpos || (qsum > 0 && (!imap || !oslot))) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_fds: null map pointer");
+  if (n_pairs < 0 || n_pairs > qsum) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_fds: n_pairs=%lld outside [0, qsum]", (long long)n_pairs);
+  if (n_pairs > 0 && (!buffer || buffer_elems < n_pairs * (int64_t)c_out))
+    PCE_FAIL(PCE_EWORKSPACE, "pce_conv_fwd_fds: buffer holds %lld elements, needs %lld", (long long)buffer_elems, (long long)(n_pairs * (int64_t)c_out));
   hipStream_t s = (hipStream_t)stream;
   if (dtype == PCE_F16)
-    return fds_impl<half_t>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, kpos, qkpos, kpos_host, qkpos_host, ocsr, ocode, qsum, (half_t *)buffer, s);
-  return fds_impl<float>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, kpos, qkpos, kpos_host, qkpos_host, ocsr, ocode, qsum, (float *)buffer, s);
+    return fds_impl<half_t>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, oslot, kpos, qkpos, kpos_host, qkpos_host, ocsr, qsum, (half_t *)buffer, s);
+  return fds_impl<float>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, oslot, kpos, qkpos, kpos_host, qkpos_host, ocsr, qsum, (float *)buffer, s);
 }
 
 extern "C" int pce_conv_fwd_os(const void *in, const void *w, const void *wp, void *out, int32_t dtype, int64_t n_in,

@@ -661,14 +661,21 @@ __global__ void __launch_bounds__(256) csr_count_kernel(const int *__restrict__ 
   cnt[r] = c;  // cnt[n] = 0 receives the total after the scan
 }
 
+// Also records, for every pair (offset kp, rank rk), the slot of its entry in this CSR order:
+// slot_of_pair[kpos[kp] + rk] = position in `code`.
 __global__ void __launch_bounds__(256) csr_fill_kernel(const int *__restrict__ rank, long long n, int kv,
-                                                       const int *__restrict__ csr, int *__restrict__ code) {
+                                                       const int *__restrict__ csr, int *__restrict__ code,
+                                                       const int *__restrict__ kpos, int *__restrict__ slot_of_pair) {
   long long r = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (r >= n) return;
   int pos = csr[r];
   for (int kp = 0; kp < kv; ++kp) {
     int rk = rank[(long long)kp * n + r];
-    if (rk >= 0) code[pos++] = kp * PCE_CSR_CODE + rk;
+    if (rk >= 0) {
+      code[pos] = kp * PCE_CSR_CODE + rk;
+      if (slot_of_pair) slot_of_pair[kpos[kp] + rk] = pos;
+      ++pos;
+    }
   }
 }
 
@@ -681,8 +688,8 @@ extern "C" int64_t pce_kmap_workspace_bytes(int64_t n_in, int64_t n_out, int32_t
 extern "C" int pce_kmap_build(const int32_t *in_coords, int64_t n_in, const int32_t *out_coords, int64_t n_out,
                               const pce_geom_t *g, void *ws, int64_t ws_bytes, int32_t *imap, int32_t *omap,
                               int32_t *knnz, int32_t *kpos, int32_t *qkpos, int32_t *icsr, int32_t *icode,
-                              int32_t *ocsr, int32_t *ocode, int32_t *nbr_out, int32_t *nbr_in, int32_t *status,
-                              pce_stream_t stream) {
+                              int32_t *ocsr, int32_t *ocode, int32_t *islot, int32_t *oslot, int32_t *nbr_out,
+                              int32_t *nbr_in, int32_t *status, pce_stream_t stream) {
   hipStream_t s = (hipStream_t)stream;
   GeomDev gd;
   int rc = make_geom(g, &gd);
@@ -692,6 +699,7 @@ extern "C" int pce_kmap_build(const int32_t *in_coords, int64_t n_in, const int3
   int ncsr = (icsr != nullptr) + (icode != nullptr) + (ocsr != nullptr) + (ocode != nullptr);
   if (ncsr != 0 && ncsr != 4) PCE_FAIL(PCE_EINVAL, "pce_kmap_build: pass all four CSR outputs or none");
   int want_csr = ncsr == 4;
+  if (!want_csr && (islot || oslot)) PCE_FAIL(PCE_EINVAL, "pce_kmap_build: slot outputs need the CSR outputs");
   if (n_in <= 0 || n_out <= 0) PCE_FAIL(PCE_EINVAL, "pce_kmap_build: empty tensor (n_in=%lld, n_out=%lld)", (long long)n_in, (long long)n_out);
   if (gd.subm && n_in != n_out) PCE_FAIL(PCE_EINVAL, "pce_kmap_build: submanifold layer needs n_in == n_out");
   if ((int64_t)gd.kv * n_in >= (1ll << 31) || (int64_t)gd.kv * n_out >= (1ll << 31))
@@ -738,14 +746,14 @@ extern "C" int pce_kmap_build(const int32_t *in_coords, int64_t n_in, const int3
     PCE_LAUNCH_CHECK("csr_count(in)");
     if ((rc = scan_exclusive(icsr, n_in + 1, scan_tmp, s))) return rc;
     hipLaunchKernelGGL(csr_fill_kernel, dim3((unsigned)pce_div_up(n_in, 256)), dim3(256), 0, s, (const int *)irank,
-                       (long long)n_in, gd.kv, (const int *)icsr, icode);
+                       (long long)n_in, gd.kv, (const int *)icsr, icode, (const int *)kpos, islot);
     PCE_LAUNCH_CHECK("csr_fill(in)");
     hipLaunchKernelGGL(csr_count_kernel, dim3((unsigned)pce_div_up(n_out + 1, 256)), dim3(256), 0, s, (const int *)orank,
                        (long long)n_out, gd.kv, ocsr);
     PCE_LAUNCH_CHECK("csr_count(out)");
     if ((rc = scan_exclusive(ocsr, n_out + 1, scan_tmp, s))) return rc;
     hipLaunchKernelGGL(csr_fill_kernel, dim3((unsigned)pce_div_up(n_out, 256)), dim3(256), 0, s, (const int *)orank,
-                       (long long)n_out, gd.kv, (const int *)ocsr, ocode);
+                       (long long)n_out, gd.kv, (const int *)ocsr, ocode, (const int *)kpos, oslot);
     PCE_LAUNCH_CHECK("csr_fill(out)");
   }
   return PCE_OK;

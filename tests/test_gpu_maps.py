@@ -122,5 +122,5 @@ def test_error_paths():
         backend.build_kernel_map(torch.zeros((4, 4), dtype=torch.int32), (3, 3, 3), (1, 1, 1), (0, 0, 0), [0, 0, 0],
                                  [1, 1, 1], True)
     lib = _lib.load()
-    rc = lib.pce_kmap_build(None, 1, None, 1, None, None, 0, *([None] * 12), None)
+    rc = lib.pce_kmap_build(None, 1, None, 1, None, None, 0, *([None] * 14), None)
     assert rc == _lib.PCE_EINVAL and b"null" in lib.pce_last_error()

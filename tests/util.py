@@ -45,6 +45,12 @@ def assert_map_equal(km: backend.KernelMap, ref: orc.KernelMap, csr: bool = Fals
         assert np.array_equal(km.ocsr.cpu().numpy(), ocsr)
         assert np.array_equal(km.icode.cpu().numpy(), icode)
         assert np.array_equal(km.ocode.cpu().numpy(), ocode)
+        # slot arrays are the inverse permutations of the CSR orders: entry slot[p] of the coded list is pair p
+        kp_of = np.repeat(np.arange(ref.kv), ref.knnz.astype(np.int64))
+        pair_code = (kp_of * orc.CSR_CODE + (np.arange(ref.M) - ref.kpos[:-1].astype(np.int64)[kp_of])).astype(np.int32)
+        for slot, code in ((km.islot, icode), (km.oslot, ocode)):
+            sl = slot.cpu().numpy()
+            assert np.array_equal(np.sort(sl), np.arange(ref.M)) and np.array_equal(code[sl], pair_code)
 
 
 def rounded(a: np.ndarray, dtype: torch.dtype) -> np.ndarray:
