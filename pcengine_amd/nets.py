@@ -1,0 +1,111 @@
+"""MinkUNet-style sparse residual U-Net composed from this package's front-end modules.
+
+The reference ships no network; this is the composition its primitives are meant for
+(conv3d, BatchNorm, ReLU, cat, spTensor.__add__; script/spconv.py, script/utils.py:152-164,
+script/sptensor.py:80-91): a stem, four encoder stages (k2s2 down-sampling + two residual
+blocks), four decoder stages (transposed k2s2 + skip concatenation + two residual blocks) and a
+1x1 head.  ``fuse_bn()`` folds every BatchNorm into the preceding convolution (inference mode).
+"""
+from __future__ import annotations
+
+from typing import List, Sequence
+
+import torch
+from torch import nn
+
+from .activation import ReLU
+from .batchnorm import BatchNorm
+from .spconv import conv3d
+from .sptensor import spTensor
+from .utils import cat
+
+
+class ConvBN(nn.Module):
+    """conv3d followed by BatchNorm and an optional ReLU; the norm can be folded into the conv."""
+
+    def __init__(self, cin, cout, ks=3, stride=1, transposed=False, relu=True, dataflow="auto"):
+        super().__init__()
+        self.conv = conv3d(cin, cout, ks, stride, transposed=transposed, dataflow=dataflow)
+        self.bn = BatchNorm(cout)
+        self.relu = ReLU(True) if relu else None
+
+    def fuse(self) -> None:
+        if self.bn is None:
+            return
+        bn = self.bn
+        scale = bn.weight.detach() / torch.sqrt(bn.running_var + bn.eps)
+        shift = bn.bias.detach() - bn.running_mean * scale
+        with torch.no_grad():
+            self.conv.kernel.mul_(scale.to(self.conv.kernel.dtype))
+            b = shift.to(self.conv.kernel.dtype)
+            if self.conv.bias is not None:
+                b = b + self.conv.bias * scale.to(self.conv.kernel.dtype)
+            self.conv.bias = nn.Parameter(b)
+        self.bn = None
+
+    def forward(self, x: spTensor) -> spTensor:
+        x = self.conv(x)
+        if self.bn is not None:
+            x = self.bn(x)
+        return self.relu(x) if self.relu is not None else x
+
+
+class ResidualBlock(nn.Module):
+    def __init__(self, cin, cout, dataflow="auto"):
+        super().__init__()
+        self.a = ConvBN(cin, cout, 3, dataflow=dataflow)
+        self.b = ConvBN(cout, cout, 3, relu=False, dataflow=dataflow)
+        self.shortcut = None if cin == cout else ConvBN(cin, cout, 1, relu=False)
+        self.relu = ReLU(True)
+
+    def forward(self, x: spTensor) -> spTensor:
+        y = self.b(self.a(x))
+        s = x if self.shortcut is None else self.shortcut(x)
+        return self.relu(y + s)
+
+
+class SparseResUNet(nn.Module):
+    """enc = channels of the four encoder stages, dec = channels of the four decoder stages."""
+
+    def __init__(self, in_channels: int = 4, num_classes: int = 20, stem: int = 32,
+                 enc: Sequence[int] = (32, 64, 128, 256), dec: Sequence[int] = (256, 128, 96, 96),
+                 dataflow: str = "auto"):
+        super().__init__()
+        df = dataflow
+        self.stem = nn.Sequential(ConvBN(in_channels, stem, 3, dataflow=df), ConvBN(stem, stem, 3, dataflow=df))
+        self.down = nn.ModuleList()
+        self.enc = nn.ModuleList()
+        c = stem
+        skips: List[int] = [stem]
+        for ce in enc:
+            self.down.append(ConvBN(c, c, 2, 2, dataflow=df))
+            self.enc.append(nn.Sequential(ResidualBlock(c, ce, df), ResidualBlock(ce, ce, df)))
+            c = ce
+            skips.append(c)
+        skips.pop()                       # the deepest output is not a skip
+        self.up = nn.ModuleList()
+        self.dec = nn.ModuleList()
+        for cd in dec:
+            self.up.append(ConvBN(c, cd, 2, 2, transposed=True, dataflow=df))
+            cs = skips.pop()
+            self.dec.append(nn.Sequential(ResidualBlock(cd + cs, cd, df), ResidualBlock(cd, cd, df)))
+            c = cd
+        self.head = conv3d(c, num_classes, 1, bias=True)
+
+    def fuse_bn(self) -> "SparseResUNet":
+        for m in self.modules():
+            if isinstance(m, ConvBN):
+                m.fuse()
+        return self
+
+    def forward(self, x: spTensor) -> spTensor:
+        x = self.stem(x)
+        feats = [x]
+        for down, enc in zip(self.down, self.enc):
+            x = enc(down(x))
+            feats.append(x)
+        feats.pop()
+        for up, dec in zip(self.up, self.dec):
+            x = up(x)
+            x = dec(cat([x, feats.pop()]))
+        return self.head(x)
