@@ -26,6 +26,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--dataflow", default="auto")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-net", action="store_true", help="skip the MinkUNet-style forward (configuration 4)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this engine has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -95,6 +96,11 @@ def main() -> int:
     wall_ms = (time.perf_counter() - t_wall) * 1e3 / args.steps
     ms = start.elapsed_time(stop) / args.steps
 
+    # calibration for hardware counters: a plain copy of known size (2 x 19.2 MB) runs three times, so
+    # that a counter run can scale FETCH_SIZE / WRITE_SIZE by what they read for it
+    for _ in range(3):
+        fd.clone()
+
     # ---- per-stage durations of the chosen dataflow (stage mask), and the other dataflows -------
     e = 2
     stages = {}
@@ -148,6 +154,37 @@ def main() -> int:
                   "stage_ms": {k: round(v, 5) for k, v in stages.items()},
                   "other_dataflows_ms": {k: round(v, 5) for k, v in others.items()}},
     }
+
+    # ---- configuration 4: MinkUNet-style forward, ~100k voxels, fp16, BN folded --------------------
+    if not args.no_net:
+        import pcengine_amd as pe
+        from pcengine_amd import nets
+        c4 = synth.lidar_cloud_100k()
+        f4 = torch.as_tensor(synth.features(4, len(c4), 4), device=dev).half()
+        c4d = torch.as_tensor(c4, device=dev)
+        torch.manual_seed(4)
+        model = nets.SparseResUNet(4, 20).to(dev).eval().fuse_bn().half()
+        cmax4 = c4[:, 1:].max(0).tolist()
+
+        def forward(keep=None):
+            x = pe.spTensor(f4, c4d, None, [0, 0, 0], cmax4)
+            if keep is not None:          # reuse the kernel maps of an earlier pass
+                x.kmaps, x.cbook = keep.kmaps, keep.cbook
+            with torch.no_grad():
+                return model(x)
+        net = {}
+        for name in ("auto", "fod", "gms"):
+            if name == "auto":
+                os.environ.pop("PCENGINE_DATAFLOW", None)
+            else:
+                os.environ["PCENGINE_DATAFLOW"] = name
+            y0 = forward()
+            full = ev_ms(forward, 10, 2)
+            cached = ev_ms(lambda: forward(y0), 20, 3)
+            net[name] = {"forward_ms_with_map_build": round(full, 4), "forward_ms_cached_maps": round(cached, 4)}
+        os.environ.pop("PCENGINE_DATAFLOW", None)
+        result["extra"]["cfg4_minkunet"] = {"voxels": int(len(c4)), "dtype": "f16", "selector": net["auto"],
+                                            "all_fetch_on_demand": net["fod"], "all_gather_gemm_scatter": net["gms"]}
 
     # ---- CPU baseline: the oracle's torch path on this box's host cores, same workload ---------
     if not args.no_cpu:
