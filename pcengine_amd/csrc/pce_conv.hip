@@ -53,6 +53,8 @@ struct TileArgs {
   const int *oslot;
   const void *buf;
   long long n_rows;  // MODE_DENSE / MODE_OS: rows of the output
+  long long items;   // (tile, column slab) work items of the launch
+  int slabs;         // column slabs per tile
   int kv, c_in, c_out;
   int w_fixed;
   int mode, epi;
@@ -93,6 +95,21 @@ __global__ void __launch_bounds__(256) pack_weights_kernel(const half_t *__restr
     v[j] = (n < c_out && k < c_in) ? W[((long long)kp * c_in + k) * c_out + n] : (half_t)0;
   }
   *reinterpret_cast<half8 *>(&P[e * 8]) = v;
+}
+
+// XCD-aware work mapping.  Workgroups are dealt to the 8 XCDs round-robin in launch order and each
+// XCD has its own L2.  Neighbouring tiles read overlapping feature rows, so every XCD gets one
+// contiguous range of the (tile, column slab) items instead of every eighth one.  The launch is one-
+// dimensional with ceil8(items) workgroups; returns false for the padding workgroups.
+#define PCE_XCDS 8
+__device__ __forceinline__ bool xcd_item(long long items, int slabs, bool remap, long long *tile, int *slab) {
+  long long lid = blockIdx.x;
+  long long per = (items + PCE_XCDS - 1) / PCE_XCDS;
+  long long item = remap ? (lid % PCE_XCDS) * per + lid / PCE_XCDS : lid;
+  if ((remap && lid / PCE_XCDS >= per) || item >= items) return false;
+  *tile = item / slabs;
+  *slab = (int)(item % slabs);
+  return true;
 }
 
 // Workgroup barrier that orders LDS accesses only.  __syncthreads() also waits for every outstanding
@@ -443,20 +460,19 @@ __device__ __forceinline__ void store_row_pieces_slow(const float (&V)[NB][2][8]
 // Finished rows -> memory through the wavefront's LDS region: the lane that owns (row, 8 columns)
 // writes its pieces; then 16 bytes per lane are read back along the rows, so that NT*sizeof(TO)/16
 // consecutive lanes store one full row segment (whole 128-byte lines at 64 fp16 channels).
-template <typename TO, int NB>
+template <typename TO, int NB, int ROWS = (sizeof(TO) == 2 ? 32 : 16)>
 __device__ __forceinline__ void store_rows_via_lds(const float (&V)[NB][2][8], void *region, TO *out, int orow,
                                                    const TileArgs &a, int n0, int lane, int l32, int g) {
   constexpr int NT = NB * 32;
   constexpr int EPP = 16 / sizeof(TO);              // elements per piece
-  constexpr int LDP = (NT + 8) / EPP;               // row stride in pieces
-  constexpr int ROWS = sizeof(TO) == 2 ? 32 : 16;   // rows per pass
+  constexpr int LDP = (NT + 8) / EPP;               // row stride in pieces; ROWS rows per pass
   constexpr int PPR = NT / EPP;                     // pieces per row
   constexpr int ITS = ROWS * PPR / 64;
   typedef typename VecOfC<TO, EPP>::type OV;
   OV *R = (OV *)region;
 #pragma unroll
   for (int pass = 0; pass < 32 / ROWS; ++pass) {
-    if (ROWS == 32 || (l32 / 16) == pass) {
+    if ((l32 / ROWS) == pass) {
       int lr = l32 % ROWS;
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
@@ -512,8 +528,11 @@ __global__ void __launch_bounds__(256, ((TMODE >= 0 && sizeof(T) == 2 && NB <= 2
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int l32 = lane & 31, g = lane >> 5;
-  const int n0 = blockIdx.y * NT;
-  const long long tile = blockIdx.x;
+  long long tile;
+  int slab;
+  // only the output-stationary mode re-reads rows across tiles; streaming modes keep launch order
+  if (!xcd_item(a.items, a.slabs, mode == MODE_OS, &tile, &slab)) return;
+  const int n0 = slab * NT;
   const T *A = (const T *)a.A;
   const T *W = (const T *)a.W;
   const T *Wp = (const T *)a.Wp;
@@ -648,25 +667,34 @@ __global__ void __launch_bounds__(256, ((TMODE >= 0 && sizeof(T) == 2 && NB <= 2
   }
 }
 
+static unsigned xcd_grid(TileArgs *a, long long tiles, int slabs) {
+  a->slabs = slabs;
+  a->items = tiles * slabs;
+  return (unsigned)(pce_div_up(a->items, PCE_XCDS) * PCE_XCDS);
+}
+
 template <typename T, bool FAST, int TMODE, int TEPI>
-static void launch_tile_nb(const TileArgs &a, long long tiles, hipStream_t s) {
+static void launch_tile_nb(TileArgs a, long long tiles, hipStream_t s) {
   int nb = (a.c_out + 31) / 32;
   if (nb >= 4) {
-    dim3 grid((unsigned)tiles, (unsigned)((a.c_out + 127) / 128));
-    hipLaunchKernelGGL((tile_gemm_kernel<T, 4, FAST, TMODE, TEPI>), grid, dim3(256), 0, s, a);
+    unsigned grid = xcd_grid(&a, tiles, (a.c_out + 127) / 128);
+    hipLaunchKernelGGL((tile_gemm_kernel<T, 4, FAST, TMODE, TEPI>), dim3(grid), dim3(256), 0, s, a);
   } else if (nb == 3) {
-    hipLaunchKernelGGL((tile_gemm_kernel<T, 3, FAST, TMODE, TEPI>), dim3((unsigned)tiles, 1), dim3(256), 0, s, a);
+    unsigned grid = xcd_grid(&a, tiles, 1);
+    hipLaunchKernelGGL((tile_gemm_kernel<T, 3, FAST, TMODE, TEPI>), dim3(grid), dim3(256), 0, s, a);
   } else if (nb == 2) {
-    hipLaunchKernelGGL((tile_gemm_kernel<T, 2, FAST, TMODE, TEPI>), dim3((unsigned)tiles, 1), dim3(256), 0, s, a);
+    unsigned grid = xcd_grid(&a, tiles, 1);
+    hipLaunchKernelGGL((tile_gemm_kernel<T, 2, FAST, TMODE, TEPI>), dim3(grid), dim3(256), 0, s, a);
   } else {
-    hipLaunchKernelGGL((tile_gemm_kernel<T, 1, FAST, TMODE, TEPI>), dim3((unsigned)tiles, 1), dim3(256), 0, s, a);
+    unsigned grid = xcd_grid(&a, tiles, 1);
+    hipLaunchKernelGGL((tile_gemm_kernel<T, 1, FAST, TMODE, TEPI>), dim3(grid), dim3(256), 0, s, a);
   }
 }
 
 template <typename T>
 static int launch_tile(const TileArgs &a, long long tiles, hipStream_t s) {
   if (tiles <= 0) return PCE_OK;
-  if (tiles >= (1ll << 31)) PCE_FAIL(PCE_ECAPACITY, "tile count %lld exceeds the grid limit", tiles);
+  if (tiles * ((a.c_out + 127) / 128) >= (1ll << 31) - 8) PCE_FAIL(PCE_ECAPACITY, "tile count %lld exceeds the grid limit", tiles);
   bool fast = a.a_vec && a.o_vec && (sizeof(T) == 2 ? a.Wp != nullptr : a.w_vec != 0) &&
               (a.epi != EPI_ROWS_CSR || a.b_vec);
   if (!fast)

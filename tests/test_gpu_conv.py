@@ -63,6 +63,27 @@ def test_strided_then_transposed_all_dataflows(ks, stride, pad, dtype):
         assert orc.rel_l2(back.double().cpu().numpy(), want_t) <= TOL[dtype], flow
 
 
+@pytest.mark.parametrize("c_in,c_out", [(128, 256), (256, 128), (96, 96), (384, 256), (40, 200)])
+def test_wide_channels_dense_map(c_in, c_out):
+    """Deep-layer shapes (dense map, wide channels): the pipelined output-stationary kernel and the others."""
+    coords = synth.random_cloud(seed=43, n=5000, extent=14, batches=2)       # ~17 neighbours per voxel
+    fd, wd, ref_map, want = _case(coords, (3, 3, 3), (1, 1, 1), (0, 0, 0), c_in, c_out, torch.float16)
+    km = gpu_map(coords, (3, 3, 3), want_csr=True)
+    packed = backend.pack_weights(wd)
+    for flow in FLOWS:
+        out = backend.conv_forward(fd, wd, km, flow, packed=packed)
+        assert orc.rel_l2(out.double().cpu().numpy(), want) <= 1e-3, flow
+    # k2s2 down and transposed up at wide channels through the same kernels
+    fd2, wd2, ref2, want2 = _case(coords, (2, 2, 2), (2, 2, 2), (0, 0, 0), c_in, c_out, torch.float16)
+    km2 = gpu_map(coords, (2, 2, 2), (2, 2, 2), want_csr=True, want_nbr_in=True)
+    out2 = backend.conv_forward(fd2, wd2, km2, DATAFLOW_OS, packed=backend.pack_weights(wd2))
+    assert orc.rel_l2(out2.double().cpu().numpy(), want2) <= 1e-3
+    wt = torch.as_tensor(synth.weights(5, 8, c_out, c_in), device=DEV).half()
+    back = backend.conv_forward(out2, wt, km2, DATAFLOW_OS, transposed=True, packed=backend.pack_weights(wt))
+    want_t = orc.conv_forward(out2.double().cpu().numpy(), wt.double().cpu().numpy(), ref2, (2, 2, 2), transposed=True)
+    assert orc.rel_l2(back.double().cpu().numpy(), want_t) <= 1e-3
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 def test_dense_1x1(dtype):
     f = synth.features(3, 5001, 96)
