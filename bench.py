@@ -25,6 +25,8 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--dataflow", default="auto")
+    ap.add_argument("--workload", default="cfg2", choices=["cfg2", "deep"],
+                    help="cfg2: the headline layer; deep: a decoder-like layer (dense map, C 256->256) for the MFMA roofline")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-net", action="store_true", help="skip the MinkUNet-style forward (configuration 4)")
     args = ap.parse_args()
@@ -41,8 +43,17 @@ def main() -> int:
     dev = "cuda:0"
     torch.cuda.set_device(0)
     ks = (3, 3, 3)
-    c_in = c_out = 64
-    coords = synth.lidar_cloud()
+    if args.workload == "cfg2":
+        c_in = c_out = 64
+        coords = synth.lidar_cloud()
+        what = "cfg2: submanifold 3x3x3 conv, fp16 storage / fp32 accumulate, C 64->64, batch 1, N={n} voxels " \
+               "(64x2048 LiDAR-like rays + ground plane @0.1 m), M={M} pairs, cached kernel map"
+    else:
+        c_in = c_out = 256
+        coords = synth.random_cloud(seed=7, n=90000, extent=58)
+        args.no_net = True
+        what = "deep: submanifold 3x3x3 conv, fp16 storage / fp32 accumulate, C 256->256, batch 1, N={n} voxels of a " \
+               "dense random cloud (the pair density of the decoder layers of configuration 4), M={M} pairs, cached kernel map"
     n = len(coords)
     feats = synth.features(2, n, c_in)
     weight = synth.weights(2, 27, c_in, c_out)
@@ -135,20 +146,28 @@ def main() -> int:
         "centre_gemm_csr_sum": n * c_in * e + n * c_out * e + c_in * c_out * e + M * c_out * e + 4 * M + 4 * (n + 1),
     }[dom]
     achieved = dom_bytes / (stages[dom] * 1e-3) / 1e9
-    roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                "algorithmic_bytes": dom_bytes, "kernel_ms": round(stages[dom], 5),
-                "layer_bytes": b_conv, "layer_GBs": round(b_conv / (ms * 1e-3) / 1e9, 1),
-                "layer_frac": round(b_conv / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                "layer_TFLOPs": round(flops / (ms * 1e-3) / 1e12, 2)}
+    # HBM bytes per launch of that kernel from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
+    # profiles/pmc_traffic_cfg2.md (scaled by the copy-kernel calibration); counters cannot be read here
+    measured_traffic = {("cfg2", "centre_gemm_csr_sum"): 43.46e6}
+    if args.workload == "cfg2":
+        roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic.get((args.workload, dom)),
+                    "algorithmic_bytes": dom_bytes, "kernel_ms": round(stages[dom], 5),
+                    "layer_bytes": b_conv, "layer_GBs": round(b_conv / (ms * 1e-3) / 1e9, 1),
+                    "layer_frac": round(b_conv / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                    "layer_TFLOPs": round(flops / (ms * 1e-3) / 1e12, 2)}
+    else:
+        tf = flops / (stages[dom] * 1e-3) / 1e12
+        roofline = {"bound": "mfma", "kernel": dom, "achieved": round(tf, 1), "peak": 2500.0, "unit": "TFLOP/s",
+                    "frac": round(tf / 2500.0, 4), "traffic": None, "algorithmic_flops": flops,
+                    "kernel_ms": round(stages[dom], 5),
+                    "executed_TFLOPs_output_stationary": round(2.0 * 27 * n * c_in * c_out / (stages[dom] * 1e-3) / 1e12, 1)}
 
     result = {
         "metric": "subm3_conv_layer_ms", "value": round(ms, 5), "unit": "ms", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": False, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
-        "config": {"workload": "cfg2: submanifold 3x3x3 conv, fp16 storage / fp32 accumulate, C 64->64, batch 1, "
-                               f"N={n} voxels (64x2048 LiDAR-like rays + ground plane @0.1 m), M={M} pairs, cached kernel map",
-                   "dataflow": names[flow], "selector": args.dataflow == "auto"},
+        "config": {"workload": what.format(n=n, M=M), "dataflow": names[flow], "selector": args.dataflow == "auto"},
         "roofline": roofline,
         "extra": {"wall_ms_per_step": round(wall_ms, 5), "map_build_ms": round(map_ms, 4),
                   "stage_ms": {k: round(v, 5) for k, v in stages.items()},
@@ -196,7 +215,7 @@ def main() -> int:
         cpu_map_ms, cpu_conv_ms, cpu_out, _ = cpu_path.time_layer(coords, f16, w16, ks, warmup=2, runs=5)
         gpu_out = step().float().cpu().numpy()
         result["cpu_baseline"] = {"value": round(cpu_conv_ms, 3), "unit": "ms", "cores": cores, "kind": "port",
-                                  "sample": "the full cfg2 layer (same N, M, C), fp32 on fp16-rounded inputs, "
+                                  "sample": f"the full {args.workload} layer (same N, M, C), fp32 on fp16-rounded inputs, "
                                             "median of 5 runs after 2 warm-ups; map build timed separately",
                                   "map_build_ms": round(cpu_map_ms, 3)}
         result["extra"]["rel_l2_vs_cpu"] = float(orc.rel_l2(gpu_out, cpu_out))
