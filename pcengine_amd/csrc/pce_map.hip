@@ -174,32 +174,35 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int *total) {
   return base + inc - v;
 }
 
-__global__ void __launch_bounds__(256) scan_reduce_kernel(const int *__restrict__ data, long long n,
-                                                          int *__restrict__ sums) {
-  long long base = (long long)blockIdx.x * SCAN_TILE + (long long)threadIdx.x * SCAN_ITEMS;
-  int acc = 0;
-#pragma unroll
-  for (int j = 0; j < SCAN_ITEMS; ++j)
-    if (base + j < n) acc += data[base + j];
-  int total;
-  block_exclusive_scan(acc, &total);
-  if (threadIdx.x == 0) sums[blockIdx.x] = total;
-}
+// Two launches for up to two arrays at once: (1) every block scans its SCAN_TILE items in place
+// (exclusive) and records its total; (2) every block adds the totals of the blocks before it in
+// the same array.  Blocks [0, nbA) belong to array A, the rest to array B.
+struct ScanPair {
+  int *a;
+  long long na;
+  int *b;
+  long long nb;
+  int blocks_a;
+};
 
-__global__ void __launch_bounds__(256) scan_sums_kernel(int *sums, long long nb) {
-  int carry = 0;
-  for (long long base = 0; base < nb; base += 256) {
-    long long i = base + threadIdx.x;
-    int v = i < nb ? sums[i] : 0;
-    int total;
-    int ex = block_exclusive_scan(v, &total);
-    if (i < nb) sums[i] = carry + ex;
-    carry += total;
+__device__ __forceinline__ void scan_pick(const ScanPair &p, int *&data, long long &n, int &blk) {
+  if ((int)blockIdx.x < p.blocks_a) {
+    data = p.a;
+    n = p.na;
+    blk = blockIdx.x;
+  } else {
+    data = p.b;
+    n = p.nb;
+    blk = blockIdx.x - p.blocks_a;
   }
 }
 
-__global__ void __launch_bounds__(256) scan_apply_kernel(int *data, long long n, const int *__restrict__ sums) {
-  long long base = (long long)blockIdx.x * SCAN_TILE + (long long)threadIdx.x * SCAN_ITEMS;
+__global__ void __launch_bounds__(256) scan_local_kernel(ScanPair p, int *__restrict__ sums) {
+  int *data;
+  long long n;
+  int blk;
+  scan_pick(p, data, n, blk);
+  long long base = (long long)blk * SCAN_TILE + (long long)threadIdx.x * SCAN_ITEMS;
   int v[SCAN_ITEMS];
   int acc = 0;
 #pragma unroll
@@ -208,26 +211,55 @@ __global__ void __launch_bounds__(256) scan_apply_kernel(int *data, long long n,
     acc += v[j];
   }
   int total;
-  int run = block_exclusive_scan(acc, &total) + sums[blockIdx.x];
+  int run = block_exclusive_scan(acc, &total);
 #pragma unroll
   for (int j = 0; j < SCAN_ITEMS; ++j) {
     if (base + j < n) data[base + j] = run;
     run += v[j];
   }
+  if (threadIdx.x == 0) sums[blockIdx.x] = total;
+}
+
+__global__ void __launch_bounds__(256) scan_add_kernel(ScanPair p, const int *__restrict__ sums) {
+  int *data;
+  long long n;
+  int blk;
+  scan_pick(p, data, n, blk);
+  if (blk == 0) return;
+  int first = (int)blockIdx.x - blk;  // first block of this array
+  int acc = 0;
+  for (int j = threadIdx.x; j < blk; j += 256) acc += sums[first + j];
+  int total;
+  block_exclusive_scan(acc, &total);
+  long long base = (long long)blk * SCAN_TILE + (long long)threadIdx.x * SCAN_ITEMS;
+#pragma unroll
+  for (int j = 0; j < SCAN_ITEMS; ++j)
+    if (base + j < n) data[base + j] += total;
 }
 
 static int64_t scan_tmp_ints(int64_t n) { return pce_div_up(n, SCAN_TILE) + 1; }
 
-static int scan_exclusive(int *data, int64_t n, int *tmp, hipStream_t s) {
-  if (n <= 0) return PCE_OK;
-  int64_t nb = pce_div_up(n, SCAN_TILE);
-  hipLaunchKernelGGL(scan_reduce_kernel, dim3((unsigned)nb), dim3(256), 0, s, (const int *)data, (long long)n, tmp);
-  PCE_LAUNCH_CHECK("scan_reduce");
-  hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(256), 0, s, tmp, (long long)nb);
-  PCE_LAUNCH_CHECK("scan_sums");
-  hipLaunchKernelGGL(scan_apply_kernel, dim3((unsigned)nb), dim3(256), 0, s, data, (long long)n, (const int *)tmp);
-  PCE_LAUNCH_CHECK("scan_apply");
+// exclusive scans of a[0..na) and b[0..nb) in place (b may be null); tmp holds one int per block
+static int scan_exclusive2(int *a, int64_t na, int *b, int64_t nb, int *tmp, hipStream_t s) {
+  ScanPair p;
+  p.a = a;
+  p.na = na;
+  p.b = b;
+  p.nb = b ? nb : 0;
+  p.blocks_a = (int)pce_div_up(na, SCAN_TILE);
+  int blocks = p.blocks_a + (int)pce_div_up(p.nb, SCAN_TILE);
+  if (blocks <= 0) return PCE_OK;
+  hipLaunchKernelGGL(scan_local_kernel, dim3(blocks), dim3(256), 0, s, p, tmp);
+  PCE_LAUNCH_CHECK("scan_local");
+  if (p.blocks_a > 1 || blocks - p.blocks_a > 1) {
+    hipLaunchKernelGGL(scan_add_kernel, dim3(blocks), dim3(256), 0, s, p, (const int *)tmp);
+    PCE_LAUNCH_CHECK("scan_add");
+  }
   return PCE_OK;
+}
+
+static int scan_exclusive(int *data, int64_t n, int *tmp, hipStream_t s) {
+  return scan_exclusive2(data, n, nullptr, 0, tmp, s);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -534,13 +566,10 @@ struct KmapLayout {
   int64_t off_table, off_dense, off_seg, off_scan, off_orank, off_irank, total;
 };
 
-static void kmap_layout(int64_t n_in, int64_t n_out, int kv, int want_csr, KmapLayout *L) {
+static void kmap_layout(int64_t n_in, int64_t n_out, int kv, int want_csr, int subm, KmapLayout *L) {
   L->slots = pce_hash_slots(n_out);
   L->nseg = pce_div_up(n_in, PCE_WAVE);
   L->scan_len = (int64_t)kv * L->nseg + 1;
-  int64_t longest = L->scan_len;
-  if (n_in + 1 > longest) longest = n_in + 1;
-  if (n_out + 1 > longest) longest = n_out + 1;
   int64_t o = 0;
   L->off_table = o;
   o += pce_align_up(L->slots * 16, 256);
@@ -549,84 +578,170 @@ static void kmap_layout(int64_t n_in, int64_t n_out, int kv, int want_csr, KmapL
   L->off_seg = o;
   o += pce_align_up(L->scan_len * 4, 256);
   L->off_scan = o;
-  o += pce_align_up(scan_tmp_ints(longest) * 4, 256);
+  o += pce_align_up((scan_tmp_ints(L->scan_len) + scan_tmp_ints(n_in + 1) + scan_tmp_ints(n_out + 1)) * 4, 256);
   L->off_orank = o;
-  if (want_csr) o += pce_align_up((int64_t)kv * n_out * 4, 256);
+  if (want_csr && !subm) o += pce_align_up((int64_t)kv * n_out * 4, 256);
   L->off_irank = o;
   if (want_csr) o += pce_align_up((int64_t)kv * n_in * 4, 256);
   L->total = o;
 }
 
+// Probe batches: the first-probe loads of PROBE_BATCH offsets are issued together, then resolved;
+// only a probe that lands on another key continues along the chain.  (One dependent probe loop per
+// offset kept a lane waiting on 26 load latencies in a row.)
+#define PROBE_BATCH 7
+
 // One lane per input row.  For every offset kp the lane asks which output row the input reaches:
 //   submanifold: out = in - d(kp)          (pair (i,o,kp) <=> coords[i] == coords[o] + d(kp))
 //   strided:     out = (in - d(kp) + pad) / stride when it divides
-// dense[kp*n_in + i] = output row or -1; segcnt[kp*nseg + seg] = hits among the 64 rows of a wave.
-__global__ void __launch_bounds__(256) kmap_query_kernel(const int4 *__restrict__ in_coords, long long n_in,
-                                                         long long n_out, GeomDev g,
+// dense[kp*n_in + i] = output row or -1.
+// A submanifold map is symmetric: pair (i,o,kp) <=> pair (o,i,kv-1-kp).  Only the offsets below the
+// centre are probed; a hit also writes the mirrored entry dense[(kv-1-kp)*n + o] = i.  The caller
+// pre-fills the rows of dense from the centre upwards with -1.
+__global__ void __launch_bounds__(256) kmap_query_kernel(const int4 *__restrict__ in_coords, long long n_in, GeomDev g,
                                                          const pce_slot_t *__restrict__ table,
                                                          unsigned long long slots, int *__restrict__ dense,
-                                                         int *__restrict__ segcnt, long long nseg,
-                                                         int *__restrict__ nbr_out, int *status) {
+                                                         int *status) {
   long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  long long seg = i >> 6;
   bool live = i < n_in;
   int4 c = live ? in_coords[i] : make_int4(0, 0, 0, 0);
   if (live && !pce_coord_ok(c.x, c.y, c.z, c.w)) {
     status[0] = 1;
     live = false;
   }
+  const int kend = g.subm ? g.mid : g.kv;
   OffsetIter it;
   it.init();
-  for (int kp = 0; kp < g.kv; ++kp, it.next(g)) {
-    int res = -1;
-    if (g.subm && kp == g.mid) {
-      if (nbr_out && live) nbr_out[(long long)kp * n_out + i] = (int)i;
-    } else if (live) {
-      int ox, oy, oz;
-      bool ok = true;
-      if (g.subm) {
-        ox = c.y - it.dx(g);
-        oy = c.z - it.dy(g);
-        oz = c.w - it.dz(g);
-      } else {
-        ok = strided_axis(c.y, it.dx(g), g.pad[0], g.stride[0], g.cmin[0], g.cmax[0], &ox);
-        ok &= strided_axis(c.z, it.dy(g), g.pad[1], g.stride[1], g.cmin[1], g.cmax[1], &oy);
-        ok &= strided_axis(c.w, it.dz(g), g.pad[2], g.stride[2], g.cmin[2], g.cmax[2], &oz);
+  for (int kp0 = 0; kp0 < kend; kp0 += PROBE_BATCH) {
+    unsigned long long key[PROBE_BATCH], slot[PROBE_BATCH];
+    uint4 e[PROBE_BATCH];
+    bool ok[PROBE_BATCH];
+#pragma unroll
+    for (int j = 0; j < PROBE_BATCH; ++j) {
+      ok[j] = live && kp0 + j < kend;
+      int ox = 0, oy = 0, oz = 0;
+      if (ok[j]) {
+        if (g.subm) {
+          ox = c.y - it.dx(g);
+          oy = c.z - it.dy(g);
+          oz = c.w - it.dz(g);
+        } else {
+          bool v = strided_axis(c.y, it.dx(g), g.pad[0], g.stride[0], g.cmin[0], g.cmax[0], &ox);
+          v &= strided_axis(c.z, it.dy(g), g.pad[1], g.stride[1], g.cmin[1], g.cmax[1], &oy);
+          v &= strided_axis(c.w, it.dz(g), g.pad[2], g.stride[2], g.cmin[2], g.cmax[2], &oz);
+          ok[j] = v;
+        }
       }
-      if (ok) res = table_find(table, slots, pce_pack_key(c.x, ox, oy, oz));
+      key[j] = pce_pack_key(c.x, ox, oy, oz);
+      slot[j] = pce_home_slot(key[j], slots);
+      e[j] = make_uint4(0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu, 0u);
+      if (ok[j]) e[j] = *reinterpret_cast<const uint4 *>(&table[slot[j]]);
+      if (kp0 + j < kend) it.next(g);
     }
-    if (i < n_in) dense[(long long)kp * n_in + i] = res;
-    unsigned long long bal = __ballot(res >= 0);
-    if (__lane_id() == 0 && seg < nseg) segcnt[(long long)kp * nseg + seg] = __popcll(bal);
+#pragma unroll
+    for (int j = 0; j < PROBE_BATCH; ++j) {
+      int kp = kp0 + j;
+      if (kp >= kend) break;
+      int res = -1;
+      if (ok[j]) {
+        unsigned long long k = ((unsigned long long)e[j].y << 32) | e[j].x;
+        if (k == key[j]) {
+          res = (int)e[j].z;
+        } else if (k != PCE_EMPTY_KEY) {
+          unsigned long long sl = (slot[j] + 1) & (slots - 1);
+          for (unsigned long long t = 1; t < slots; ++t) {
+            const uint4 f = *reinterpret_cast<const uint4 *>(&table[sl]);
+            unsigned long long k2 = ((unsigned long long)f.y << 32) | f.x;
+            if (k2 == key[j]) {
+              res = (int)f.z;
+              break;
+            }
+            if (k2 == PCE_EMPTY_KEY) break;
+            sl = (sl + 1) & (slots - 1);
+          }
+        }
+      }
+      if (i < n_in) {
+        dense[(long long)kp * n_in + i] = res;
+        if (g.subm && res >= 0) dense[(long long)(g.kv - 1 - kp) * n_in + res] = (int)i;
+      }
+    }
   }
 }
 
+// The per-row loops over the offsets below load ROW_BATCH table entries before using any of them.
+#define ROW_BATCH 9
+
+// One pass over the probe results: hits per (offset, 64-row segment) from wave ballots, and hits per
+// row (the row lengths of the CSR view, mapping_counter of backend/hash.cuh:422-437).
+__global__ void __launch_bounds__(256) kmap_count_kernel(long long n_in, int kv, const int *__restrict__ dense,
+                                                         int *__restrict__ segcnt, long long nseg,
+                                                         int *__restrict__ rowcnt) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  long long seg = i >> 6;
+  bool live = i < n_in;
+  int c = 0;
+  for (int kp0 = 0; kp0 < kv; kp0 += ROW_BATCH) {
+    int v[ROW_BATCH];
+#pragma unroll
+    for (int j = 0; j < ROW_BATCH; ++j) v[j] = (live && kp0 + j < kv) ? dense[(long long)(kp0 + j) * n_in + i] : -1;
+#pragma unroll
+    for (int j = 0; j < ROW_BATCH; ++j) {
+      if (kp0 + j >= kv) break;
+      bool hit = v[j] >= 0;
+      c += hit;
+      unsigned long long bal = __ballot(hit);
+      if (__lane_id() == 0 && seg < nseg) segcnt[(long long)(kp0 + j) * nseg + seg] = __popcll(bal);
+    }
+  }
+  if (rowcnt && i <= n_in) rowcnt[i] = live ? c : 0;  // rowcnt[n_in] = 0 receives the total after the scan
+  if (i == 0) segcnt[(long long)kv * nseg] = 0;
+}
+
 // segoff = exclusive scan of segcnt in (kp, segment) order = position of the segment's first pair.
-__global__ void __launch_bounds__(256) kmap_fill_kernel(long long n_in, long long n_out, int kv,
+// Emits the pair lists in (offset, input row) order from ballot ranks, the rank of every pair inside
+// its offset (irank, and orank scattered by output row for strided layers), and the output-major
+// neighbour table: scattered for strided layers, read off the mirrored row for submanifold ones.
+__global__ void __launch_bounds__(256) kmap_fill_kernel(long long n_in, long long n_out, int kv, int subm, int mid,
                                                         const int *__restrict__ dense, const int *__restrict__ segoff,
                                                         long long nseg, int *__restrict__ imap,
                                                         int *__restrict__ omap, int *__restrict__ irank,
                                                         int *__restrict__ orank, int *__restrict__ nbr_out,
-                                                        int want_csr, int *status) {
+                                                        int *status) {
   long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   long long seg = i >> 6;
   bool live = i < n_in;
-  for (int kp = 0; kp < kv; ++kp) {
-    int v = live ? dense[(long long)kp * n_in + i] : -1;
-    unsigned long long bal = __ballot(v >= 0);
-    int rank = -1;
-    if (v >= 0) {
-      int p = segoff[(long long)kp * nseg + seg] + __popcll(bal & lanemask_lt());
-      imap[p] = (int)i;
-      omap[p] = v;
-      if (nbr_out) nbr_out[(long long)kp * n_out + v] = (int)i;
-      if (want_csr) {
-        rank = p - segoff[(long long)kp * nseg];
-        if (rank >= PCE_CSR_CODE) status[2] = 1;
-        orank[(long long)kp * n_out + v] = rank;
-      }
+  for (int kp0 = 0; kp0 < kv; kp0 += ROW_BATCH) {
+    int vv[ROW_BATCH], mm[ROW_BATCH], base[ROW_BATCH], first[ROW_BATCH];
+#pragma unroll
+    for (int j = 0; j < ROW_BATCH; ++j) {
+      int kp = kp0 + j;
+      bool in = kp < kv;
+      vv[j] = (live && in) ? dense[(long long)kp * n_in + i] : -1;
+      mm[j] = (live && in && nbr_out && subm && kp != mid) ? dense[(long long)(kv - 1 - kp) * n_in + i] : -1;
+      base[j] = (in && seg < nseg) ? segoff[(long long)kp * nseg + seg] : 0;
+      first[j] = in ? segoff[(long long)kp * nseg] : 0;
     }
-    if (want_csr && live) irank[(long long)kp * n_in + i] = rank;
+#pragma unroll
+    for (int j = 0; j < ROW_BATCH; ++j) {
+      int kp = kp0 + j;
+      if (kp >= kv) break;
+      int v = vv[j];
+      unsigned long long bal = __ballot(v >= 0);
+      int rank = -1;
+      if (v >= 0) {
+        int p = base[j] + __popcll(bal & lanemask_lt());
+        imap[p] = (int)i;
+        omap[p] = v;
+        if (nbr_out && !subm) nbr_out[(long long)kp * n_out + v] = (int)i;
+        rank = p - first[j];
+        if (irank && rank >= PCE_CSR_CODE) status[2] = 1;
+        if (orank) orank[(long long)kp * n_out + v] = rank;
+      }
+      if (irank && live) irank[(long long)kp * n_in + i] = rank;
+      if (nbr_out && subm && live)  // nbr_out[kp][o] = input of the pair whose output is o = mirrored probe result
+        nbr_out[(long long)kp * n_out + i] = kp == mid ? (int)i : mm[j];
+    }
   }
 }
 
@@ -661,8 +776,8 @@ __global__ void __launch_bounds__(256) csr_count_kernel(const int *__restrict__ 
   cnt[r] = c;  // cnt[n] = 0 receives the total after the scan
 }
 
-// Also records, for every pair (offset kp, rank rk), the slot of its entry in this CSR order:
-// slot_of_pair[kpos[kp] + rk] = position in `code`.
+// CSR-coded entries of every row in ascending offset order, plus, for every pair (offset kp, rank rk),
+// the slot of its entry in this order: slot_of_pair[kpos[kp] + rk] = position in `code`.
 __global__ void __launch_bounds__(256) csr_fill_kernel(const int *__restrict__ rank, long long n, int kv,
                                                        const int *__restrict__ csr, int *__restrict__ code,
                                                        const int *__restrict__ kpos, int *__restrict__ slot_of_pair) {
@@ -679,9 +794,54 @@ __global__ void __launch_bounds__(256) csr_fill_kernel(const int *__restrict__ r
   }
 }
 
+// Submanifold map: both CSR views in one pass.  The input-side entry of row r at offset kp is the
+// pair (r, dense[kp][r], kp); the output-side entry is the pair (dense[kv-1-kp][r], r, kp), whose
+// rank is read from the rank table at its input row.  Both views have the same row pointers.
+__global__ void __launch_bounds__(256) csr_fill_subm_kernel(const int *__restrict__ dense, const int *__restrict__ irank,
+                                                            long long n, int kv, const int *__restrict__ csr,
+                                                            const int *__restrict__ kpos, int *__restrict__ icode,
+                                                            int *__restrict__ ocode, int *__restrict__ islot,
+                                                            int *__restrict__ oslot, int *__restrict__ ocsr) {
+  long long r = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (r > n) return;
+  if (r == n) {
+    ocsr[n] = csr[n];
+    return;
+  }
+  int pi = csr[r], po = pi;
+  ocsr[r] = pi;
+  for (int kp0 = 0; kp0 < kv; kp0 += ROW_BATCH) {
+    int rk[ROW_BATCH], src[ROW_BATCH], rk2[ROW_BATCH], kb[ROW_BATCH];
+#pragma unroll
+    for (int j = 0; j < ROW_BATCH; ++j) {
+      int kp = kp0 + j;
+      bool in = kp < kv;
+      rk[j] = in ? irank[(long long)kp * n + r] : -1;
+      src[j] = in ? dense[(long long)(kv - 1 - kp) * n + r] : -1;
+      kb[j] = in ? kpos[kp] : 0;
+    }
+#pragma unroll
+    for (int j = 0; j < ROW_BATCH; ++j) rk2[j] = src[j] >= 0 ? irank[(long long)(kp0 + j) * n + src[j]] : -1;
+#pragma unroll
+    for (int j = 0; j < ROW_BATCH; ++j) {
+      int kp = kp0 + j;
+      if (rk[j] >= 0) {
+        icode[pi] = kp * PCE_CSR_CODE + rk[j];
+        if (islot) islot[kb[j] + rk[j]] = pi;
+        ++pi;
+      }
+      if (src[j] >= 0) {
+        ocode[po] = kp * PCE_CSR_CODE + rk2[j];
+        if (oslot) oslot[kb[j] + rk2[j]] = po;
+        ++po;
+      }
+    }
+  }
+}
+
 extern "C" int64_t pce_kmap_workspace_bytes(int64_t n_in, int64_t n_out, int32_t kv, int32_t want_csr) {
   KmapLayout L;
-  kmap_layout(n_in, n_out, kv, want_csr, &L);
+  kmap_layout(n_in, n_out, kv, want_csr, 0, &L);  // the strided layout is the larger one
   return L.total;
 }
 
@@ -705,7 +865,7 @@ extern "C" int pce_kmap_build(const int32_t *in_coords, int64_t n_in, const int3
   if ((int64_t)gd.kv * n_in >= (1ll << 31) || (int64_t)gd.kv * n_out >= (1ll << 31))
     PCE_FAIL(PCE_ECAPACITY, "pce_kmap_build: kv*n exceeds int32 pair indexing");
   KmapLayout L;
-  kmap_layout(n_in, n_out, gd.kv, want_csr, &L);
+  kmap_layout(n_in, n_out, gd.kv, want_csr, gd.subm, &L);
   if (ws_bytes < L.total) PCE_FAIL(PCE_EWORKSPACE, "pce_kmap_build: workspace %lld < %lld", (long long)ws_bytes, (long long)L.total);
   char *w = (char *)ws;
   pce_slot_t *table = (pce_slot_t *)(w + L.off_table);
@@ -713,38 +873,45 @@ extern "C" int pce_kmap_build(const int32_t *in_coords, int64_t n_in, const int3
   int *irank = want_csr ? (int *)(w + L.off_irank) : nullptr;
   int *seg = (int *)(w + L.off_seg);
   int *scan_tmp = (int *)(w + L.off_scan);
-  int *orank = want_csr ? (int *)(w + L.off_orank) : nullptr;
+  int *orank = (want_csr && !gd.subm) ? (int *)(w + L.off_orank) : nullptr;
 
   // 1. table over the output coordinates (for a submanifold layer these are the input coordinates)
   if ((rc = table_clear(table, L.slots, s))) return rc;
   hipLaunchKernelGGL(hash_insert_kernel, dim3((unsigned)pce_div_up(n_out, 256)), dim3(256), 0, s, table,
                      (unsigned long long)L.slots, (const int4 *)out_coords, (long long)n_out, status);
   PCE_LAUNCH_CHECK("hash_insert");
-  if (nbr_out && (rc = fill_u32(nbr_out, (int64_t)gd.kv * n_out, 0xFFFFFFFFu, s))) return rc;
-  if (want_csr && (rc = fill_u32(orank, (int64_t)gd.kv * n_out, 0xFFFFFFFFu, s))) return rc;
-  // 2. probe, per-wave counts
+  if (gd.subm) {
+    // rows of the probe table that the mirrored writes only touch on a hit (and the centre row)
+    if ((rc = fill_u32(dense + (int64_t)gd.mid * n_in, (int64_t)(gd.kv - gd.mid) * n_in, 0xFFFFFFFFu, s))) return rc;
+  } else {
+    if (nbr_out && (rc = fill_u32(nbr_out, (int64_t)gd.kv * n_out, 0xFFFFFFFFu, s))) return rc;
+    if (orank && (rc = fill_u32(orank, (int64_t)gd.kv * n_out, 0xFFFFFFFFu, s))) return rc;
+  }
+  // 2. probe, then count per (offset, segment) and per row
   unsigned blocks = (unsigned)pce_div_up(n_in, 256);
-  hipLaunchKernelGGL(kmap_query_kernel, dim3(blocks), dim3(256), 0, s, (const int4 *)in_coords, (long long)n_in,
-                     (long long)n_out, gd, (const pce_slot_t *)table, (unsigned long long)L.slots, dense, seg,
-                     (long long)L.nseg, nbr_out, status);
+  hipLaunchKernelGGL(kmap_query_kernel, dim3(blocks), dim3(256), 0, s, (const int4 *)in_coords, (long long)n_in, gd,
+                     (const pce_slot_t *)table, (unsigned long long)L.slots, dense, status);
   PCE_LAUNCH_CHECK("kmap_query");
-  // 3. positions
-  if ((rc = fill_u32(seg + (L.scan_len - 1), 1, 0u, s))) return rc;
-  if ((rc = scan_exclusive(seg, L.scan_len, scan_tmp, s))) return rc;
+  hipLaunchKernelGGL(kmap_count_kernel, dim3((unsigned)pce_div_up(n_in + 1, 256)), dim3(256), 0, s, (long long)n_in, gd.kv,
+                     (const int *)dense, seg, (long long)L.nseg, want_csr ? icsr : nullptr);
+  PCE_LAUNCH_CHECK("kmap_count");
+  // 3. positions: scan of the segment counts and, in the same launches, of the input row lengths
+  if ((rc = scan_exclusive2(seg, L.scan_len, want_csr ? icsr : nullptr, n_in + 1, scan_tmp, s))) return rc;
   hipLaunchKernelGGL(kmap_offsets_kernel, dim3(1), dim3(128), 0, s, (const int *)seg, (long long)L.nseg, gd.kv, knnz,
                      kpos, qkpos);
   PCE_LAUNCH_CHECK("kmap_offsets");
   // 4. pair lists in (offset, input row) order
-  hipLaunchKernelGGL(kmap_fill_kernel, dim3(blocks), dim3(256), 0, s, (long long)n_in, (long long)n_out, gd.kv,
-                     (const int *)dense, (const int *)seg, (long long)L.nseg, imap, omap, irank, orank, nbr_out, want_csr,
+  hipLaunchKernelGGL(kmap_fill_kernel, dim3(blocks), dim3(256), 0, s, (long long)n_in, (long long)n_out, gd.kv, gd.subm,
+                     gd.mid, (const int *)dense, (const int *)seg, (long long)L.nseg, imap, omap, irank, orank, nbr_out,
                      status);
   PCE_LAUNCH_CHECK("kmap_fill");
   // 5. CSR-coded view
-  if (want_csr) {
-    hipLaunchKernelGGL(csr_count_kernel, dim3((unsigned)pce_div_up(n_in + 1, 256)), dim3(256), 0, s, (const int *)irank,
-                       (long long)n_in, gd.kv, icsr);
-    PCE_LAUNCH_CHECK("csr_count(in)");
-    if ((rc = scan_exclusive(icsr, n_in + 1, scan_tmp, s))) return rc;
+  if (want_csr && gd.subm) {
+    hipLaunchKernelGGL(csr_fill_subm_kernel, dim3((unsigned)pce_div_up(n_in + 1, 256)), dim3(256), 0, s,
+                       (const int *)dense, (const int *)irank, (long long)n_in, gd.kv, (const int *)icsr,
+                       (const int *)kpos, icode, ocode, islot, oslot, ocsr);
+    PCE_LAUNCH_CHECK("csr_fill_subm");
+  } else if (want_csr) {
     hipLaunchKernelGGL(csr_fill_kernel, dim3((unsigned)pce_div_up(n_in, 256)), dim3(256), 0, s, (const int *)irank,
                        (long long)n_in, gd.kv, (const int *)icsr, icode, (const int *)kpos, islot);
     PCE_LAUNCH_CHECK("csr_fill(in)");
