@@ -91,14 +91,22 @@ int pce_hash_query(const void *table_dev, int64_t slots, const int32_t *qcoords_
 /* ---- output coordinates of a strided convolution -------------------------------------------- *
  * Replaces coordsDownsampleExpand + remove + sort + unique + coordsGenerator
  * (backend/hash.cuh:535-641, backend/hash.cu:141-173).  Always the generic rule; the reference's
- * stride==kernel shortcut is not reproduced because it disagrees with its own query kernels. */
-int64_t pce_outcoords_workspace_bytes(int64_t n_in, const pce_geom_t *g);
-/* Builds the sorted unique output codes inside the workspace and returns their number in
+ * stride==kernel shortcut is not reproduced because it disagrees with its own query kernels.
+ *
+ * n_batch is the batch count the reference carries as spTensor.batchsize and hands to its mapping
+ * call (script/spconv.py:363).  With n_batch > 0 and a modest output bounding box (geometry cmin /
+ * cmax) the candidates are marked in an occupancy bitmap in (b,x,y,z) order and a popcount scan
+ * de-duplicates, sorts and counts them at once; a batch index >= n_batch is then PCE_EINVAL.
+ * With n_batch <= 0, or a box too large or too empty for a bitmap, candidates go through a hash
+ * table and a radix sort of their codes instead.  Both give the same coordinates.  The three calls
+ * of one build take the same (n_in, g, n_batch). */
+int64_t pce_outcoords_workspace_bytes(int64_t n_in, const pce_geom_t *g, int32_t n_batch);
+/* Builds the sorted unique output set inside the workspace and returns its size in
  * *n_out_host.  Synchronises the stream once (the count has to reach the host). */
-int pce_outcoords_build(const int32_t *in_coords_dev, int64_t n_in, const pce_geom_t *g,
+int pce_outcoords_build(const int32_t *in_coords_dev, int64_t n_in, const pce_geom_t *g, int32_t n_batch,
                         void *ws_dev, int64_t ws_bytes, int64_t *n_out_host, pce_stream_t stream);
-/* Decodes them into out_coords_dev[n_out,4] (same workspace, untouched since _build). */
-int pce_outcoords_emit(const void *ws_dev, int64_t n_in, const pce_geom_t *g, int64_t n_out,
+/* Decodes it into out_coords_dev[n_out,4] (same workspace, untouched since _build). */
+int pce_outcoords_emit(const void *ws_dev, int64_t n_in, const pce_geom_t *g, int32_t n_batch, int64_t n_out,
                        int32_t *out_coords_dev, pce_stream_t stream);
 
 /* ---- kernel map ------------------------------------------------------------------------------ *

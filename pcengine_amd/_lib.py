@@ -46,9 +46,9 @@ _SIGNATURES = {
     "pce_hash_table_bytes": (c_int64, [c_int64]),
     "pce_hash_build": (c_int32, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p]),
     "pce_hash_query": (c_int32, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p]),
-    "pce_outcoords_workspace_bytes": (c_int64, [c_int64, POINTER(Geom)]),
-    "pce_outcoords_build": (c_int32, [c_void_p, c_int64, POINTER(Geom), c_void_p, c_int64, POINTER(c_int64), c_void_p]),
-    "pce_outcoords_emit": (c_int32, [c_void_p, c_int64, POINTER(Geom), c_int64, c_void_p, c_void_p]),
+    "pce_outcoords_workspace_bytes": (c_int64, [c_int64, POINTER(Geom), c_int32]),
+    "pce_outcoords_build": (c_int32, [c_void_p, c_int64, POINTER(Geom), c_int32, c_void_p, c_int64, POINTER(c_int64), c_void_p]),
+    "pce_outcoords_emit": (c_int32, [c_void_p, c_int64, POINTER(Geom), c_int32, c_int64, c_void_p, c_void_p]),
     "pce_kmap_workspace_bytes": (c_int64, [c_int64, c_int64, c_int32, c_int32]),
     "pce_kmap_build": (c_int32, [c_void_p, c_int64, c_void_p, c_int64, POINTER(Geom), c_void_p, c_int64] + [c_void_p] * 14 + [c_void_p]),
     "pce_conv_fod_workspace_bytes": (c_int64, [c_int64, c_int32, c_int32]),

@@ -114,26 +114,33 @@ def strided_coords_max(cmax, ks, stride, pad):
     return [(int(cmax[a]) + 2 * pad[a] - (ks[a] - 1)) // stride[a] for a in range(3)]
 
 
-def build_out_coords(in_coords: torch.Tensor, geom: Geom) -> torch.Tensor:
-    """Sorted unique output coordinates of a strided layer (one host sync for the count)."""
+def build_out_coords(in_coords: torch.Tensor, geom: Geom, batchsize: int = 0) -> torch.Tensor:
+    """Sorted unique output coordinates of a strided layer (one host sync for the count).
+
+    ``batchsize`` > 0 bounds the batch indices and lets the library use its occupancy-bitmap path;
+    a cloud that holds a larger batch index than announced is redone without the bound."""
     lib = _lib.load()
     _require_cuda(in_coords, "coords")
     n_in = in_coords.shape[0]
-    ws_bytes = lib.pce_outcoords_workspace_bytes(n_in, geom)
-    if ws_bytes < 0:
-        _lib.check(_lib.PCE_EINVAL)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=in_coords.device)
-    n_out = _lib.c_int64(0)
     s = _stream(in_coords.device)
-    _lib.check(lib.pce_outcoords_build(in_coords.data_ptr(), n_in, geom, ws.data_ptr(), ws_bytes, n_out, s))
-    out = torch.empty((n_out.value, 4), dtype=torch.int32, device=in_coords.device)
-    _lib.check(lib.pce_outcoords_emit(ws.data_ptr(), n_in, geom, n_out.value, _ptr(out), s))
-    return out
+    for n_batch in ((int(batchsize), 0) if batchsize > 0 else (0,)):
+        ws_bytes = lib.pce_outcoords_workspace_bytes(n_in, geom, n_batch)
+        if ws_bytes < 0:
+            _lib.check(_lib.PCE_EINVAL)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=in_coords.device)
+        n_out = _lib.c_int64(0)
+        rc = lib.pce_outcoords_build(in_coords.data_ptr(), n_in, geom, n_batch, ws.data_ptr(), ws_bytes, n_out, s)
+        if rc == _lib.PCE_EINVAL and n_batch > 0 and b"n_batch" in lib.pce_last_error():
+            continue
+        _lib.check(rc)
+        out = torch.empty((n_out.value, 4), dtype=torch.int32, device=in_coords.device)
+        _lib.check(lib.pce_outcoords_emit(ws.data_ptr(), n_in, geom, n_batch, n_out.value, _ptr(out), s))
+        return out
 
 
 def build_kernel_map(in_coords: torch.Tensor, ks, stride, pad, cmin, cmax_out, subm: bool,
                      want_csr: bool = False, want_nbr_out: bool = True, want_nbr_in: bool = False,
-                     out_coords: Optional[torch.Tensor] = None) -> KernelMap:
+                     out_coords: Optional[torch.Tensor] = None, batchsize: int = 0) -> KernelMap:
     """Hash the output coordinates, probe every (input row, offset) and emit the canonical map.
 
     ``cmax_out`` is the bound on output coordinates (already reduced for strided layers)."""
@@ -149,7 +156,7 @@ def build_kernel_map(in_coords: torch.Tensor, ks, stride, pad, cmin, cmax_out, s
     if subm:
         out_coords = in_coords
     elif out_coords is None:
-        out_coords = build_out_coords(in_coords, geom)
+        out_coords = build_out_coords(in_coords, geom, batchsize)
     n_out = out_coords.shape[0]
     if n_in == 0 or n_out == 0:
         raise ValueError(f"empty sparse tensor (n_in={n_in}, n_out={n_out})")
@@ -326,7 +333,8 @@ def mapping_d2_cuda(in_coords, batch_size, k_size_code, k_vol, c_in, c_out, l_st
     input tensor itself for a submanifold layer)."""
     ks, stride, pad, cmin, cmax, subm = _geom_from_codes(k_size_code, l_stride_code, padding_code,
                                                          (min_x, min_y, min_z), (max_x, max_y, max_z), separate_mid)
-    km = build_kernel_map(in_coords, ks, stride, pad, cmin, cmax, subm, want_nbr_out=False, want_nbr_in=True)
+    km = build_kernel_map(in_coords, ks, stride, pad, cmin, cmax, subm, want_nbr_out=False, want_nbr_in=True,
+                          batchsize=int(batch_size))
     map.view(-1)[:km.kv * km.n_in].copy_(km.nbr_in)
     kernel_nnz[:km.kv].copy_(km.knnz)
     kernel_kpos[:km.kv + 1].copy_(km.kpos)

@@ -183,6 +183,7 @@ struct ScanPair {
   int *b;
   long long nb;
   int blocks_a;
+  const unsigned *popc_a;  // when set, the input of array A is popcount(popc_a[i]) instead of a[i]
 };
 
 __device__ __forceinline__ void scan_pick(const ScanPair &p, int *&data, long long &n, int &blk) {
@@ -205,9 +206,11 @@ __global__ void __launch_bounds__(256) scan_local_kernel(ScanPair p, int *__rest
   long long base = (long long)blk * SCAN_TILE + (long long)threadIdx.x * SCAN_ITEMS;
   int v[SCAN_ITEMS];
   int acc = 0;
+  const bool popc = p.popc_a && (int)blockIdx.x < p.blocks_a;
 #pragma unroll
   for (int j = 0; j < SCAN_ITEMS; ++j) {
-    v[j] = (base + j < n) ? data[base + j] : 0;
+    v[j] = 0;
+    if (base + j < n) v[j] = popc ? __popc(p.popc_a[base + j]) : data[base + j];
     acc += v[j];
   }
   int total;
@@ -240,8 +243,10 @@ __global__ void __launch_bounds__(256) scan_add_kernel(ScanPair p, const int *__
 static int64_t scan_tmp_ints(int64_t n) { return pce_div_up(n, SCAN_TILE) + 1; }
 
 // exclusive scans of a[0..na) and b[0..nb) in place (b may be null); tmp holds one int per block
-static int scan_exclusive2(int *a, int64_t na, int *b, int64_t nb, int *tmp, hipStream_t s) {
+static int scan_exclusive2(int *a, int64_t na, int *b, int64_t nb, int *tmp, hipStream_t s,
+                           const unsigned *popc_a = nullptr) {
   ScanPair p;
+  p.popc_a = popc_a;
   p.a = a;
   p.na = na;
   p.b = b;
@@ -326,7 +331,20 @@ __device__ __forceinline__ bool strided_axis(int c, int d, int pad, int stride, 
 // ------------------------------------------------------------------------------------------------
 // output coordinates of a strided layer
 // ------------------------------------------------------------------------------------------------
+// Two ways to the sorted unique output coordinates.  When the caller bounds the batch count and the
+// output bounding box is small enough, every candidate sets one bit of an occupancy bitmap laid
+// out in (b,x,y,z) order: a popcount scan then yields count, order and de-duplication at once.
+// Otherwise candidates are de-duplicated through a hash table and their codes radix-sorted.
+struct BitGrid {
+  int lo[3], ext[3];
+  int n_batch;
+};
+
 struct OutCoordLayout {
+  int bitmap;          // 1: occupancy bitmap, 0: hash table + radix sort
+  BitGrid grid;
+  int64_t words;       // 32-bit words of the bitmap (one spare word of zeros at the end)
+  int64_t off_bits, off_cnt;
   int64_t upper;       // bound on the number of candidates that survive
   int64_t slots;       // de-duplication table
   int64_t off_table, off_codes_a, off_codes_b, off_hist, off_scan, off_counters, total;
@@ -334,12 +352,47 @@ struct OutCoordLayout {
 };
 
 #define SORT_KEYS_PER_BLOCK 1024  // one wavefront per block, 16 rounds of 64 keys
+#define BITMAP_MAX_BITS (1ll << 28)
 
-static void outcoord_layout(int64_t n_in, const GeomDev &g, OutCoordLayout *L) {
+static void outcoord_layout(int64_t n_in, const GeomDev &g, int n_batch, OutCoordLayout *L) {
   int64_t per = 1;
   for (int a = 0; a < 3; ++a) per *= pce_div_up(g.ks[a], g.stride[a]);
   L->upper = n_in * per;
   if (L->upper < 1) L->upper = 1;
+  L->bitmap = 0;
+  L->words = 0;
+  if (n_batch > 0) {
+    int64_t bits = n_batch;
+    bool ok = true;
+    for (int a = 0; a < 3; ++a) {
+      int lo = g.cmin[a] > 0 ? g.cmin[a] : 0;
+      int hi = g.cmax[a] < PCE_COORD_BOUND - 1 ? g.cmax[a] : PCE_COORD_BOUND - 1;
+      L->grid.lo[a] = lo;
+      L->grid.ext[a] = hi - lo + 1;
+      if (hi < lo) ok = false;
+      else bits *= (hi - lo + 1);   // <= 32768 * 3259^3 < 2^63
+    }
+    L->grid.n_batch = n_batch;
+    int64_t words = pce_div_up(bits, 32) + 1;
+    int64_t dense_enough = 32 * L->upper > (1ll << 16) ? 32 * L->upper : (1ll << 16);
+    if (ok && bits <= BITMAP_MAX_BITS && words <= dense_enough) {
+      L->bitmap = 1;
+      L->words = words;
+    }
+  }
+  if (L->bitmap) {
+    int64_t o = 0;
+    L->off_bits = o;
+    o += pce_align_up(L->words * 4, 256);
+    L->off_counters = o;  // directly behind the bitmap: one fill clears both
+    o += 256;
+    L->off_cnt = o;
+    o += pce_align_up(L->words * 4, 256);
+    L->off_scan = o;
+    o += pce_align_up(scan_tmp_ints(L->words) * 4, 256);
+    L->total = o;
+    return;
+  }
   L->slots = pce_hash_slots(L->upper);
   L->sort_blocks = pce_div_up(L->upper, SORT_KEYS_PER_BLOCK);
   int64_t o = 0;
@@ -356,6 +409,61 @@ static void outcoord_layout(int64_t n_in, const GeomDev &g, OutCoordLayout *L) {
   L->off_counters = o;
   o += 256;
   L->total = o;
+}
+
+// status[0]: coordinate out of range, status[2]: batch index >= the caller's batch count
+__global__ void __launch_bounds__(256) outcoord_mark_kernel(const int4 *__restrict__ coords, long long n_in, GeomDev g,
+                                                            BitGrid grid, unsigned *__restrict__ bits, int *status) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_in) return;
+  int4 c = coords[i];
+  if (!pce_coord_ok(c.x, c.y, c.z, c.w)) {
+    status[0] = 1;
+    return;
+  }
+  if (c.x >= grid.n_batch) {
+    status[2] = 1;
+    return;
+  }
+  OffsetIter it;
+  it.init();
+  for (int kp = 0; kp < g.kv; ++kp, it.next(g)) {
+    int ox, oy, oz;
+    bool ok = strided_axis(c.y, it.dx(g), g.pad[0], g.stride[0], g.cmin[0], g.cmax[0], &ox);
+    ok &= strided_axis(c.z, it.dy(g), g.pad[1], g.stride[1], g.cmin[1], g.cmax[1], &oy);
+    ok &= strided_axis(c.w, it.dz(g), g.pad[2], g.stride[2], g.cmin[2], g.cmax[2], &oz);
+    if (!ok) continue;
+    if (ox < 0 || oy < 0 || oz < 0 || ox >= PCE_COORD_BOUND || oy >= PCE_COORD_BOUND || oz >= PCE_COORD_BOUND) {
+      status[0] = 1;
+      continue;
+    }
+    long long bit = (((long long)c.x * grid.ext[0] + (ox - grid.lo[0])) * grid.ext[1] + (oy - grid.lo[1])) * grid.ext[2] +
+                    (oz - grid.lo[2]);
+    atomicOr(&bits[bit >> 5], 1u << (bit & 31));
+  }
+}
+
+// cnt[w] = number of set bits before word w (exclusive scan of the popcounts)
+__global__ void __launch_bounds__(256) outcoord_expand_kernel(const unsigned *__restrict__ bits, const int *__restrict__ cnt,
+                                                              long long words, BitGrid grid, int4 *__restrict__ out) {
+  long long w = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (w >= words) return;
+  unsigned m = bits[w];
+  if (!m) return;
+  int o = cnt[w];
+  while (m) {
+    int b = __ffs((int)m) - 1;
+    m &= m - 1;
+    long long idx = w * 32 + b;
+    int4 c;
+    c.w = (int)(idx % grid.ext[2]) + grid.lo[2];
+    idx /= grid.ext[2];
+    c.z = (int)(idx % grid.ext[1]) + grid.lo[1];
+    idx /= grid.ext[1];
+    c.y = (int)(idx % grid.ext[0]) + grid.lo[0];
+    c.x = (int)(idx / grid.ext[0]);
+    out[o++] = c;
+  }
 }
 
 // counters[0] = number of unique candidates, counters[1] = largest code
@@ -476,15 +584,15 @@ __global__ void decode_codes_kernel(const unsigned long long *__restrict__ codes
   out[i] = o;
 }
 
-extern "C" int64_t pce_outcoords_workspace_bytes(int64_t n_in, const pce_geom_t *g) {
+extern "C" int64_t pce_outcoords_workspace_bytes(int64_t n_in, const pce_geom_t *g, int32_t n_batch) {
   GeomDev gd;
   if (make_geom(g, &gd)) return -1;
   OutCoordLayout L;
-  outcoord_layout(n_in, gd, &L);
+  outcoord_layout(n_in, gd, n_batch, &L);
   return L.total;
 }
 
-extern "C" int pce_outcoords_build(const int32_t *in_coords, int64_t n_in, const pce_geom_t *g, void *ws,
+extern "C" int pce_outcoords_build(const int32_t *in_coords, int64_t n_in, const pce_geom_t *g, int32_t n_batch, void *ws,
                                    int64_t ws_bytes, int64_t *n_out_host, pce_stream_t stream) {
   hipStream_t s = (hipStream_t)stream;
   GeomDev gd;
@@ -493,10 +601,29 @@ extern "C" int pce_outcoords_build(const int32_t *in_coords, int64_t n_in, const
   if (!in_coords || !ws || !n_out_host) PCE_FAIL(PCE_EINVAL, "pce_outcoords_build: null pointer");
   if (n_in <= 0 || n_in >= (1ll << 31)) PCE_FAIL(PCE_EINVAL, "pce_outcoords_build: n_in=%lld", (long long)n_in);
   OutCoordLayout L;
-  outcoord_layout(n_in, gd, &L);
+  outcoord_layout(n_in, gd, n_batch, &L);
   if (ws_bytes < L.total) PCE_FAIL(PCE_EWORKSPACE, "pce_outcoords_build: workspace %lld < %lld", (long long)ws_bytes, (long long)L.total);
   if (L.upper >= (1ll << 31)) PCE_FAIL(PCE_ECAPACITY, "pce_outcoords_build: candidate bound %lld exceeds int32", (long long)L.upper);
   char *w = (char *)ws;
+  if (L.bitmap) {
+    unsigned *bits = (unsigned *)(w + L.off_bits);
+    int *cnt = (int *)(w + L.off_cnt);
+    int *status = (int *)(w + L.off_counters);
+    if ((rc = fill_u32(bits, (L.off_counters + 256 - L.off_bits) / 4, 0u, s))) return rc;
+    hipLaunchKernelGGL(outcoord_mark_kernel, dim3((unsigned)pce_div_up(n_in, 256)), dim3(256), 0, s,
+                       (const int4 *)in_coords, (long long)n_in, gd, L.grid, bits, status);
+    PCE_LAUNCH_CHECK("outcoord_mark");
+    // the spare last word is zero, so after the scan cnt[words-1] is the number of set bits
+    if ((rc = scan_exclusive2(cnt, L.words, nullptr, 0, (int *)(w + L.off_scan), s, bits))) return rc;
+    int host[4];
+    PCE_HIP(hipMemcpyAsync(&host[0], cnt + (L.words - 1), sizeof(int), hipMemcpyDeviceToHost, s));
+    PCE_HIP(hipMemcpyAsync(&host[1], status, 3 * sizeof(int), hipMemcpyDeviceToHost, s));
+    PCE_HIP(hipStreamSynchronize(s));
+    if (host[1]) PCE_FAIL(PCE_ECOORD, "pce_outcoords_build: coordinate outside [0,%d) or batch index out of range", PCE_COORD_BOUND);
+    if (host[3]) PCE_FAIL(PCE_EINVAL, "pce_outcoords_build: a batch index is >= n_batch=%d", (int)n_batch);
+    *n_out_host = host[0];
+    return PCE_OK;
+  }
   pce_slot_t *table = (pce_slot_t *)(w + L.off_table);
   unsigned long long *ca = (unsigned long long *)(w + L.off_codes_a);
   unsigned long long *cb = (unsigned long long *)(w + L.off_codes_b);
@@ -541,16 +668,24 @@ extern "C" int pce_outcoords_build(const int32_t *in_coords, int64_t n_in, const
   return PCE_OK;
 }
 
-extern "C" int pce_outcoords_emit(const void *ws, int64_t n_in, const pce_geom_t *g, int64_t n_out,
+extern "C" int pce_outcoords_emit(const void *ws, int64_t n_in, const pce_geom_t *g, int32_t n_batch, int64_t n_out,
                                   int32_t *out_coords, pce_stream_t stream) {
   GeomDev gd;
   int rc = make_geom(g, &gd);
   if (rc) return rc;
   if (!ws || (n_out > 0 && !out_coords)) PCE_FAIL(PCE_EINVAL, "pce_outcoords_emit: null pointer");
   OutCoordLayout L;
-  outcoord_layout(n_in, gd, &L);
+  outcoord_layout(n_in, gd, n_batch, &L);
   if (n_out < 0 || n_out > L.upper) PCE_FAIL(PCE_EINVAL, "pce_outcoords_emit: n_out=%lld out of range", (long long)n_out);
   if (n_out == 0) return PCE_OK;
+  if (L.bitmap) {
+    const char *w = (const char *)ws;
+    hipLaunchKernelGGL(outcoord_expand_kernel, dim3((unsigned)pce_div_up(L.words, 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const unsigned *)(w + L.off_bits), (const int *)(w + L.off_cnt), (long long)L.words, L.grid,
+                       (int4 *)out_coords);
+    PCE_LAUNCH_CHECK("outcoord_expand");
+    return PCE_OK;
+  }
   const unsigned long long *ca = (const unsigned long long *)((const char *)ws + L.off_codes_a);
   hipLaunchKernelGGL(decode_codes_kernel, dim3((unsigned)pce_div_up(n_out, 256)), dim3(256), 0, (hipStream_t)stream, ca,
                      (long long)n_out, (int4 *)out_coords);

@@ -175,7 +175,8 @@ def conv_func(input: spTensor, in_channel, out_channel, kernel, kernel_size_code
             raise NotImplementedError(f"unknown init_tag entry {tag!r}")
         auto = tag in ('end', 'auto')
         km = backend.build_kernel_map(input.coords, ks, stride, pad, coords_min, coords_max, subm,
-                                      want_csr=(tag == 'D1' or auto), want_nbr_out=auto, want_nbr_in=auto and not subm)
+                                      want_csr=(tag == 'D1' or auto), want_nbr_out=auto, want_nbr_in=auto and not subm,
+                                      batchsize=input.batchsize)
         km.tag = tag if tag in ('D1', 'D2') else 'auto'
         input.kmaps[key] = km
         input.cbook[output_stride] = km.out_coords

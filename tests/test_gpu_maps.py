@@ -71,6 +71,10 @@ def test_kernel_map_bit_exact(ks, stride, pad, seed, n, extent, batches):
         return
     km = gpu_map(coords, ks, stride, pad, want_csr=True, want_nbr_out=True, want_nbr_in=True)
     assert_map_equal(km, ref, csr=True)
+    if tuple(stride) != (1, 1, 1):
+        # the same layer through the occupancy-bitmap route to the output coordinates
+        kb = gpu_map(coords, ks, stride, pad, batchsize=batches)
+        assert_map_equal(kb, ref)
 
 
 def test_kernel_map_config1_and_determinism():
@@ -90,12 +94,57 @@ def test_kernel_map_config2_lidar_full_size():
     ref2 = orc.kernel_map(coords, (2, 2, 2), (2, 2, 2))
     km2 = gpu_map(coords, (2, 2, 2), (2, 2, 2), want_csr=True, want_nbr_in=True)
     assert_map_equal(km2, ref2, csr=True)
+    assert torch.equal(gpu_map(coords, (2, 2, 2), (2, 2, 2), batchsize=1).out_coords, km2.out_coords)
     # size-independent properties of a k2s2 map: every input is in exactly one pair
     assert km2.M == len(coords)
     assert torch.equal(torch.sort(km2.imap).values, torch.arange(len(coords), dtype=torch.int32, device=DEV))
     oc = km2.out_coords.cpu().numpy().astype(np.int64)
     code = ((oc[:, 0] * 3259 + oc[:, 1]) * 3259 + oc[:, 2]) * 3259 + oc[:, 3]
     assert (np.diff(code) > 0).all()      # strictly ascending (b,x,y,z)
+
+
+def _out_coords(coords, ks, stride, pad, cmin, cmax_out, n_batch):
+    geom = _lib.Geom.make(ks, stride, pad, cmin, cmax_out, False)
+    return backend.build_out_coords(dev_coords(coords), geom, n_batch).cpu().numpy()
+
+
+@pytest.mark.parametrize("n_batch", [0, 4])
+def test_out_coords_clipped_to_bounds(n_batch):
+    """Bounds that cut candidates away on both sides, hash/sort and bitmap routes alike."""
+    coords = synth.random_cloud(seed=41, n=30000, extent=50, batches=4)
+    for ks, stride, pad, cmin, cmax in [((3, 3, 3), (2, 2, 2), (1, 1, 1), (3, 0, 5), (17, 25, 11)),
+                                        ((2, 2, 2), (2, 2, 2), (0, 0, 0), (0, 2, 0), (24, 9, 24)),
+                                        ((3, 2, 1), (2, 2, 1), (0, 0, 0), (1, 1, 1), (20, 20, 30))]:
+        want = orc.out_coords_strided(coords, ks, stride, pad, cmin, cmax)
+        got = _out_coords(coords, ks, stride, pad, cmin, cmax, n_batch)
+        assert len(want) > 0 and np.array_equal(got, want)
+
+
+def test_out_coords_bitmap_rejects_large_batch_index_and_front_end_recovers():
+    lib = _lib.load()
+    coords = synth.random_cloud(seed=42, n=4000, extent=20, batches=3)
+    geom = _lib.Geom.make((2, 2, 2), (2, 2, 2), (0, 0, 0), [0, 0, 0], [9, 9, 9], False)
+    c = dev_coords(coords)
+    ws_bytes = lib.pce_outcoords_workspace_bytes(len(coords), geom, 2)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=DEV)
+    n_out = _lib.c_int64(0)
+    rc = lib.pce_outcoords_build(c.data_ptr(), len(coords), geom, 2, ws.data_ptr(), ws_bytes, n_out,
+                                 torch.cuda.current_stream().cuda_stream)
+    assert rc == _lib.PCE_EINVAL and b"n_batch" in lib.pce_last_error()
+    # the front end redoes the build without the bound
+    want = orc.out_coords_strided(coords, (2, 2, 2), (2, 2, 2), (0, 0, 0), (0, 0, 0), (9, 9, 9))
+    assert np.array_equal(backend.build_out_coords(c, geom, 2).cpu().numpy(), want)
+
+
+def test_out_coords_sparse_box_falls_back_to_sort():
+    """A handful of points in a huge box: the bitmap would be mostly empty, the library sorts."""
+    lib = _lib.load()
+    rng = np.random.default_rng(43)
+    coords = np.unique(np.concatenate([np.zeros((300, 1), np.int64), rng.integers(0, 3000, (300, 3))], 1), axis=0).astype(np.int32)
+    geom = _lib.Geom.make((2, 2, 2), (2, 2, 2), (0, 0, 0), [0, 0, 0], [1499, 1499, 1499], False)
+    assert lib.pce_outcoords_workspace_bytes(len(coords), geom, 1) == lib.pce_outcoords_workspace_bytes(len(coords), geom, 0)
+    want = orc.out_coords_strided(coords, (2, 2, 2), (2, 2, 2), (0, 0, 0), (0, 0, 0), (1499, 1499, 1499))
+    assert np.array_equal(backend.build_out_coords(dev_coords(coords), geom, 1).cpu().numpy(), want)
 
 
 def test_unsorted_input_rows():

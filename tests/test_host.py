@@ -30,9 +30,9 @@ def test_pure_host_entry_points():
     assert lib.pce_hash_slots(1) == 8 and lib.pce_hash_slots(20000) == 65536 and lib.pce_hash_slots(150000) == 524288
     assert lib.pce_hash_table_bytes(150000) == 524288 * 16
     g = _lib.Geom.make((2, 2, 2), (2, 2, 2), (0, 0, 0), (0, 0, 0), (10, 10, 10), False)
-    assert lib.pce_outcoords_workspace_bytes(1000, g) > 0
+    assert lib.pce_outcoords_workspace_bytes(1000, g, 0) > 0
     bad = _lib.Geom.make((0, 2, 2), (2, 2, 2), (0, 0, 0), (0, 0, 0), (10, 10, 10), False)
-    assert lib.pce_outcoords_workspace_bytes(1000, bad) == -1
+    assert lib.pce_outcoords_workspace_bytes(1000, bad, 0) == -1
     assert lib.pce_kmap_workspace_bytes(1000, 1000, 27, 1) > lib.pce_kmap_workspace_bytes(1000, 1000, 27, 0)
     assert lib.pce_conv_fod_workspace_bytes(1000, 64, _lib.PCE_F16) == 1000 * 64 * 4
     assert lib.pce_conv_fod_workspace_bytes(1000, 64, _lib.PCE_F32) == 0
