@@ -180,13 +180,19 @@ int pce_conv_fwd_gms(const void *in_feats, const void *weight, const void *weigh
  * buffer[ocsr[o] .. ocsr[o+1]) in fp32 and stores output row o once.  `buffer` holds
  * n_pairs*c_out elements of dtype.  kpos_host / qkpos_host are optional host copies of kpos / qkpos
  * (kv+1 entries): with them the kernels take the offsets from their arguments.
+ * omap_dev (optional, may be NULL) is the output row of every pair.  With it, and 16-byte aligned
+ * rows of at most 64 channels, a submanifold layer runs as two launches: pair tiles and centre
+ * GEMM together (neither reads what the other writes), then one pass over the pairs that adds
+ * each output row's partial rows to the centre term already stored there.  Rows with partial
+ * rows are then rounded to dtype twice (centre term, final sum).
  * No counterpart in the reference: it is ConvolutionForwardD2 with the atomic scatter-add replaced
  * by the output-stationary sum of ConvolutionForwardD1 (backend/spconv.cu:149-161), fused with
  * the centre GEMM. */
 int pce_conv_fwd_fds(const void *in_feats, const void *weight, const void *weight_packed,
                      void *out_feats, int32_t dtype, int64_t n_in, int64_t n_out, int32_t c_in,
                      int32_t c_out, int32_t kv, int32_t mid, const int32_t *imap_dev,
-                     const int32_t *oslot_dev, const int32_t *kpos_dev, const int32_t *qkpos_dev,
+                     const int32_t *omap_dev, const int32_t *oslot_dev, const int32_t *kpos_dev,
+                     const int32_t *qkpos_dev,
                      const int32_t *kpos_host, const int32_t *qkpos_host, const int32_t *ocsr_dev,
                      int64_t n_pairs, int64_t qsum, void *buffer_dev, int64_t buffer_elems,
                      pce_stream_t stream);

@@ -294,10 +294,10 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
         need = km.M * c_out
         if buffer is None or buffer.numel() < need or buffer.dtype != feats.dtype or buffer.device != dev:
             buffer = torch.empty(max(need, 1), dtype=feats.dtype, device=dev)
-        imap = km.omap if transposed else km.imap
+        imap, omap = (km.omap, km.imap) if transposed else (km.imap, km.omap)
         ocsr, oslot = (km.icsr, km.islot) if transposed else (km.ocsr, km.oslot)
         _lib.check(lib.pce_conv_fwd_fds(feats.data_ptr(), weight.data_ptr(), _ptr(packed), out.data_ptr(), dt, n_in, n_out,
-                                        c_in, c_out, kv, mid, imap.data_ptr(), oslot.data_ptr(), km.kpos.data_ptr(),
+                                        c_in, c_out, kv, mid, imap.data_ptr(), omap.data_ptr(), oslot.data_ptr(), km.kpos.data_ptr(),
                                         km.qkpos.data_ptr(), km.kpos_host, km.qkpos_host, ocsr.data_ptr(), km.M, km.qsum,
                                         buffer.data_ptr(), buffer.numel(), s))
     elif dataflow == DATAFLOW_GMS:

@@ -517,21 +517,15 @@ __device__ __forceinline__ void store_rows_via_lds(const float (&V)[NB][2][8], v
 // TMODE / TEPI >= 0 fix the mode and the epilogue at compile time (the hot combinations); -1 reads
 // them from the arguments.
 template <typename T, int NB, bool FAST, int TMODE, int TEPI>
-__global__ void __launch_bounds__(256, ((TMODE >= 0 && sizeof(T) == 2 && NB <= 2) ? 5 : 1)) tile_gemm_kernel(TileArgs a) {
+__device__ __forceinline__ void tile_body(const TileArgs &a, long long tile, int slab, T *Wl,
+                                          typename Partials<T, NB>::PV (*Pl)[WaveLds<NB>::PIECES]) {
   const int mode = TMODE >= 0 ? TMODE : a.mode;
   const int epi = TEPI >= 0 ? TEPI : a.epi;
   constexpr int NT = NB * 32;
   constexpr int KC = Cfg<T>::KC;
   typedef Partials<T, NB> P;
-  __shared__ __attribute__((aligned(16))) T Wl[KC * NT];
-  __shared__ __attribute__((aligned(16))) typename P::PV Pl[4][WaveLds<NB>::PIECES];
-
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int l32 = lane & 31, g = lane >> 5;
-  long long tile;
-  int slab;
-  // only the output-stationary mode re-reads rows across tiles; streaming modes keep launch order
-  if (!xcd_item(a.items, a.slabs, mode == MODE_OS, &tile, &slab)) return;
   const int n0 = slab * NT;
   const T *A = (const T *)a.A;
   const T *W = (const T *)a.W;
@@ -665,6 +659,106 @@ __global__ void __launch_bounds__(256, ((TMODE >= 0 && sizeof(T) == 2 && NB <= 2
     else
       store_row_pieces_slow<half_t, NB>(V, (half_t *)a.out, orow, a, n0, g);
   }
+}
+
+template <typename T, int NB, bool FAST, int TMODE, int TEPI>
+__global__ void __launch_bounds__(256, ((TMODE >= 0 && sizeof(T) == 2 && NB <= 2) ? 5 : 1)) tile_gemm_kernel(TileArgs a) {
+  typedef Partials<T, NB> P;
+  __shared__ __attribute__((aligned(16))) T Wl[Cfg<T>::KC * NB * 32];
+  __shared__ __attribute__((aligned(16))) typename P::PV Pl[4][WaveLds<NB>::PIECES];
+  const int mode = TMODE >= 0 ? TMODE : a.mode;
+  long long tile;
+  int slab;
+  // only the output-stationary mode re-reads rows across tiles; streaming modes keep launch order
+  if (!xcd_item(a.items, a.slabs, mode == MODE_OS, &tile, &slab)) return;
+  tile_body<T, NB, FAST, TMODE, TEPI>(a, tile, slab, Wl, Pl);
+}
+
+// ---- wavefront-independent form of the pair tiles and of the centre GEMM -------------------------
+// For fp16 rows of at most 64 channels a layer is bound by memory, and a workgroup that stages its
+// weight tile through LDS behind a barrier makes all resident workgroups read, compute and write in
+// step.  Here every wavefront owns 32 rows (pairs or output rows) and takes its weight fragments
+// straight from the packed copy (8 KB per offset: it stays in cache), so there is no workgroup
+// barrier and wavefronts drift apart, which keeps loads and stores of different wavefronts
+// overlapped.  Chunks [0, pair.items) are pair chunks, the rest rows of the centre GEMM.
+template <int NB, int KS>
+__global__ void __launch_bounds__(256, 5) wave_gemm_kernel(TileArgs pair, TileArgs centre) {
+  __shared__ __attribute__((aligned(16))) half8 Pl[4][WaveLds<NB>::PIECES];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int l32 = lane & 31, g = lane >> 5;
+  long long chunk = (long long)blockIdx.x * 4 + wave;
+  const bool is_pair = chunk < pair.items;
+  if (!is_pair && chunk - pair.items >= centre.items) return;
+  // features, weights and shapes are those of `pair` for both kinds of chunk; only the destination
+  // differs (selecting a whole argument block at run time would copy it to private memory)
+  const TileArgs &a = pair;
+  int arow = -1, orow = -1, widx;
+  if (is_pair) {
+    long long q0 = chunk * 32;
+    widx = 0;
+    for (int i = 0; i < pair.kv; ++i) widx += ((long long)pair.qkpos_h[i + 1] <= q0) ? 1 : 0;
+    if (widx >= pair.kv) return;
+    long long p = q0 - pair.qkpos_h[widx] + pair.kpos_h[widx] + l32;
+    if (p < (long long)pair.kpos_h[widx + 1]) {
+      arow = pair.imap[p];
+      orow = pair.oslot[p];
+    }
+  } else {
+    long long row = (chunk - pair.items) * 32 + l32;
+    widx = centre.w_fixed;
+    if (row < centre.n_rows) arow = orow = (int)row;
+  }
+  const half_t *A = (const half_t *)a.A;
+  const half_t *Wk = (const half_t *)a.Wp + (long long)widx * a.k8_total * a.n_pad * 8;
+  half8 af[KS], wf[KS][NB];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    half8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (arow >= 0) v = *reinterpret_cast<const half8 *>(A + (long long)arow * a.c_in + s * 16 + g * 8);
+    af[s] = v;
+  }
+#pragma unroll
+  for (int s = 0; s < KS; ++s)
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+      wf[s][nb] = *reinterpret_cast<const half8 *>(Wk + ((long long)(2 * s + g) * a.n_pad + nb * 32 + l32) * 8);
+  f32x16 acc[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[nb][j] = 0.f;
+#pragma unroll
+  for (int s = 0; s < KS; ++s)
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[s][nb], af[s], acc[nb], 0, 0, 0);
+  float V[NB][2][8];
+  gather_row_pieces<NB>(acc, V, g);
+  half_t *out = (half_t *)(is_pair ? pair.out : centre.out);
+  store_rows_via_lds<half_t, NB>(V, Pl[wave], out, orow, a, 0, lane, l32, g);
+}
+
+// pair chunks and centre rows of one layer in one launch (either part may be empty)
+static int launch_wave_gemm(const TileArgs &pair, const TileArgs &centre, hipStream_t s) {
+  long long chunks = pair.items + centre.items;
+  if (chunks <= 0) return PCE_OK;
+  if (chunks / 4 >= (1ll << 31) - 8) PCE_FAIL(PCE_ECAPACITY, "chunk count %lld exceeds the grid limit", chunks);
+  unsigned grid = (unsigned)pce_div_up(chunks, 4);
+  int nb = (pair.c_out + 31) / 32, ks = pair.c_in / 16;  // both blocks come from base_args of one layer
+#define PCE_WAVE_CASE(NB_, KS_)                                                                              \
+  if (nb == NB_ && ks == KS_) {                                                                              \
+    hipLaunchKernelGGL((wave_gemm_kernel<NB_, KS_>), dim3(grid), dim3(256), 0, s, pair, centre);             \
+    PCE_LAUNCH_CHECK("wave_gemm");                                                                           \
+    return PCE_OK;                                                                                           \
+  }
+  PCE_WAVE_CASE(1, 1) PCE_WAVE_CASE(1, 2) PCE_WAVE_CASE(1, 3) PCE_WAVE_CASE(1, 4)
+  PCE_WAVE_CASE(2, 1) PCE_WAVE_CASE(2, 2) PCE_WAVE_CASE(2, 3) PCE_WAVE_CASE(2, 4)
+#undef PCE_WAVE_CASE
+  PCE_FAIL(PCE_EINVAL, "wave_gemm: unsupported shape c_in=%d c_out=%d", pair.c_in, pair.c_out);
+}
+
+// shapes the wavefront-independent kernel takes: fp16, packed weights, 16-byte rows everywhere
+static bool wave_gemm_ok(const TileArgs &a, int elem_size) {
+  return elem_size == 2 && a.Wp && a.a_vec && a.o_vec && a.c_in % 16 == 0 && a.c_in <= 64 && a.c_out <= 64;
 }
 
 static unsigned xcd_grid(TileArgs *a, long long tiles, int slabs) {
@@ -814,6 +908,37 @@ __global__ void __launch_bounds__(256) rowsum_kernel(const T *__restrict__ buf, 
 #pragma unroll
     for (int j = 0; j < VEC; ++j) reinterpret_cast<T *>(&y)[j] = (T)acc[j];
     *reinterpret_cast<V *>(&out[row * c_out + (long long)v * VEC]) = y;
+  }
+}
+
+// out[o] += sum of the partial rows of o, for the rows that have any: one group of G lanes per pair;
+// the pair whose partial row is the first of its output row does the whole row.
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256) rowsum_pairs_kernel(const T *__restrict__ buf, long long n_pairs, int c_out, int G,
+                                                           const int *__restrict__ omap, const int *__restrict__ oslot,
+                                                           const int *__restrict__ csr, T *__restrict__ out) {
+  typedef typename VecOf<T, VEC>::type V;
+  long long p = (long long)blockIdx.x * (256 / G) + threadIdx.x / G;
+  int sub = threadIdx.x % G;
+  if (p >= n_pairs) return;
+  int row = omap[p];
+  int e0 = csr[row];
+  if (oslot[p] != e0) return;
+  int e1 = csr[row + 1];
+  int row_vecs = c_out / VEC;
+  for (int v = sub; v < row_vecs; v += G) {
+    V x = *reinterpret_cast<const V *>(&out[(long long)row * c_out + (long long)v * VEC]);
+    float acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[j] = (float)(reinterpret_cast<const T *>(&x)[j]);
+    for (int e = e0; e < e1; ++e) {
+      V y = *reinterpret_cast<const V *>(&buf[(long long)e * c_out + (long long)v * VEC]);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) acc[j] += (float)(reinterpret_cast<const T *>(&y)[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) reinterpret_cast<T *>(&x)[j] = (T)acc[j];
+    *reinterpret_cast<V *>(&out[(long long)row * c_out + (long long)v * VEC]) = x;
   }
 }
 
@@ -1078,11 +1203,36 @@ extern "C" int pce_conv_fwd_gms(const void *in, const void *w, const void *wp, v
 // centre GEMM, which adds each output row's contiguous partial rows in fp32 and stores the row once.
 template <typename T>
 static int fds_impl(const void *in, const void *w, const void *wp, void *out, int64_t n_out, int c_in, int c_out, int kv,
-                    int mid, const int *imap, const int *oslot, const int *kpos, const int *qkpos,
-                    const int32_t *kpos_host, const int32_t *qkpos_host, const int *ocsr, int64_t qsum, T *buffer,
-                    hipStream_t s) {
+                    int mid, const int *imap, const int *omap, const int *oslot, const int *kpos, const int *qkpos,
+                    const int32_t *kpos_host, const int32_t *qkpos_host, const int *ocsr, int64_t n_pairs, int64_t qsum,
+                    T *buffer, hipStream_t s) {
   constexpr int VEC = sizeof(T) == 2 ? 8 : 4;
   int rc;
+  if (mid >= 0 && qsum > 0 && omap && stage_on(4)) {
+    // Pair chunks and centre GEMM share one launch (neither reads what the other writes); a pass
+    // over the pairs then adds every output row's partial rows to the centre term stored there.
+    TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
+    set_out<T>(&a, buffer, false);
+    set_host_pos(&a, kpos_host, qkpos_host);
+    a.imap = imap;
+    a.oslot = oslot;
+    a.items = qsum / 32;
+    TileArgs c = base_args<T>(in, w, wp, kv, c_in, c_out);
+    set_out<T>(&c, out, false);
+    c.w_fixed = mid;
+    c.n_rows = n_out;
+    c.items = pce_div_up(n_out, 32);
+    if (a.host_pos && wave_gemm_ok(a, sizeof(T)) && wave_gemm_ok(c, sizeof(T)) && aligned16(buffer)) {
+      if (stage_on(1) && (rc = launch_wave_gemm(a, c, s))) return rc;
+      if (stage_on(2)) {
+        int G = pow2_at_least(c_out / VEC);
+        hipLaunchKernelGGL((rowsum_pairs_kernel<T, VEC>), dim3((unsigned)pce_div_up(n_pairs, 256 / G)), dim3(256), 0, s,
+                           (const T *)buffer, (long long)n_pairs, c_out, G, omap, oslot, ocsr, (T *)out);
+        PCE_LAUNCH_CHECK("rowsum_pairs");
+      }
+      return PCE_OK;
+    }
+  }
   if (qsum > 0 && stage_on(1)) {
     TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
     set_out<T>(&a, buffer, false);
@@ -1093,7 +1243,14 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
     a.qkpos = qkpos;
     a.mode = MODE_FOD_BUF;
     a.epi = EPI_ROWS;
-    if ((rc = launch_tile<T>(a, qsum / PCE_QUANTUM, s))) return rc;
+    if (a.host_pos && wave_gemm_ok(a, sizeof(T)) && stage_on(4)) {
+      TileArgs none = a;
+      none.items = 0;
+      a.items = qsum / 32;
+      if ((rc = launch_wave_gemm(a, none, s))) return rc;
+    } else if ((rc = launch_tile<T>(a, qsum / PCE_QUANTUM, s))) {
+      return rc;
+    }
   }
   if (!stage_on(2)) return PCE_OK;
   if (mid >= 0) {
@@ -1126,7 +1283,7 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
 
 extern "C" int pce_conv_fwd_fds(const void *in, const void *w, const void *wp, void *out, int32_t dtype, int64_t n_in,
                                 int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv, int32_t mid, const int32_t *imap,
-                                const int32_t *oslot, const int32_t *kpos, const int32_t *qkpos,
+                                const int32_t *omap, const int32_t *oslot, const int32_t *kpos, const int32_t *qkpos,
                                 const int32_t *kpos_host, const int32_t *qkpos_host, const int32_t *ocsr,
                                 int64_t n_pairs, int64_t qsum, void *buffer, int64_t buffer_elems, pce_stream_t stream) {
   int rc = check_common("pce_conv_fwd_fds", in, w, out, dtype, n_in, n_out, c_in, c_out, kv, mid);
@@ -1137,8 +1294,8 @@ extern "C" int pce_conv_fwd_fds(const void *in, const void *w, const void *wp, v
     PCE_FAIL(PCE_EWORKSPACE, "pce_conv_fwd_fds: buffer holds %lld elements, needs %lld", (long long)buffer_elems, (long long)(n_pairs * (int64_t)c_out));
   hipStream_t s = (hipStream_t)stream;
   if (dtype == PCE_F16)
-    return fds_impl<half_t>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, oslot, kpos, qkpos, kpos_host, qkpos_host, ocsr, qsum, (half_t *)buffer, s);
-  return fds_impl<float>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, oslot, kpos, qkpos, kpos_host, qkpos_host, ocsr, qsum, (float *)buffer, s);
+    return fds_impl<half_t>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, omap, oslot, kpos, qkpos, kpos_host, qkpos_host, ocsr, n_pairs, qsum, (half_t *)buffer, s);
+  return fds_impl<float>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, omap, oslot, kpos, qkpos, kpos_host, qkpos_host, ocsr, n_pairs, qsum, (float *)buffer, s);
 }
 
 extern "C" int pce_conv_fwd_os(const void *in, const void *w, const void *wp, void *out, int32_t dtype, int64_t n_in,

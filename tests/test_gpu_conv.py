@@ -84,6 +84,39 @@ def test_wide_channels_dense_map(c_in, c_out):
     assert orc.rel_l2(back.double().cpu().numpy(), want_t) <= 1e-3
 
 
+@pytest.mark.parametrize("c_in,c_out", [(16, 8), (32, 48), (48, 64), (64, 24), (64, 64), (16, 40)])
+def test_narrow_fp16_layers_barrier_free_kernel(c_in, c_out):
+    """fp16 rows of at most 64 channels with packed weights take the wavefront-per-chunk kernel in the
+    deferred-scatter dataflow: submanifold (pairs + centre in one launch), strided and transposed."""
+    from pcengine_amd import _lib
+    lib = _lib.load()
+    coords = synth.random_cloud(seed=44, n=12000, extent=30, batches=2)
+    fd, wd, ref_map, want = _case(coords, (3, 3, 3), (1, 1, 1), (0, 0, 0), c_in, c_out, torch.float16, seed=6)
+    km = gpu_map(coords, (3, 3, 3), want_csr=True)
+    pk = backend.pack_weights(wd)
+    out = backend.conv_forward(fd, wd, km, DATAFLOW_FDS, packed=pk)
+    assert orc.rel_l2(out.double().cpu().numpy(), want) <= 1e-3
+    lib.pce_set_stage_mask(0xFFFFFFFF & ~16)          # the same layer through the workgroup-tile kernels
+    try:
+        old = backend.conv_forward(fd, wd, km, DATAFLOW_FDS, packed=pk)
+    finally:
+        lib.pce_set_stage_mask(0xFFFFFFFF)
+    assert orc.rel_l2(old.double().cpu().numpy(), want) <= 1e-3
+    # rows without neighbours are the centre GEMM alone and agree bit for bit
+    lonely = (km.ocsr[1:] == km.ocsr[:-1])
+    assert lonely.any() and torch.equal(out[lonely], old[lonely])
+    for ks, stride, pad in [((2, 2, 2), (2, 2, 2), (0, 0, 0)), ((3, 3, 3), (2, 2, 2), (1, 1, 1))]:
+        fd2, wd2, ref2, want2 = _case(coords, ks, stride, pad, c_in, c_out, torch.float16, seed=7)
+        km2 = gpu_map(coords, ks, stride, pad, want_csr=True)
+        down = backend.conv_forward(fd2, wd2, km2, DATAFLOW_FDS, packed=backend.pack_weights(wd2))
+        assert orc.rel_l2(down.double().cpu().numpy(), want2) <= 1e-3
+        if c_out % 16 == 0:
+            wt = torch.as_tensor(synth.weights(8, km2.kv, c_out, c_in), device=DEV).half()
+            back = backend.conv_forward(down, wt, km2, DATAFLOW_FDS, transposed=True, packed=backend.pack_weights(wt))
+            want_t = orc.conv_forward(down.double().cpu().numpy(), wt.double().cpu().numpy(), ref2, ks, transposed=True)
+            assert orc.rel_l2(back.double().cpu().numpy(), want_t) <= 1e-3
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 def test_dense_1x1(dtype):
     f = synth.features(3, 5001, 96)
@@ -113,8 +146,13 @@ def test_config2_fp16_c64_full_size():
         assert orc.rel_l2(out.double().cpu().numpy(), want) <= 1e-3, flow
     # linearity in the features holds at any size: conv(2x) == 2 conv(x); scaling by two is exact in
     # fp16 except for results in the subnormal range, whose spacing is 2^-24
-    twice = backend.conv_forward(fd * 2, wd, km, DATAFLOW_FDS, packed=backend.pack_weights(wd))
-    assert torch.allclose(twice.float(), outs[3].float() * 2, rtol=0, atol=2.0 ** -23)
+    # (both runs take the same launch sequence: packed weights select the two-launch form, whose rows
+    # with neighbours are rounded twice)
+    packed = backend.pack_weights(wd)
+    once = backend.conv_forward(fd, wd, km, DATAFLOW_FDS, packed=packed)
+    twice = backend.conv_forward(fd * 2, wd, km, DATAFLOW_FDS, packed=packed)
+    assert orc.rel_l2(once.double().cpu().numpy(), want) <= 1e-3
+    assert torch.allclose(twice.float(), once.float() * 2, rtol=0, atol=2.0 ** -23)
 
 
 def test_reference_named_entry_points_d2_and_d1():
