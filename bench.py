@@ -63,6 +63,7 @@ def main() -> int:
     cmax = coords[:, 1:].max(0).tolist()
 
     def ev_ms(fn, steps, warmup):
+        """Eager launches: HIP events on the current stream around `steps` calls."""
         for _ in range(warmup):
             fn()
         torch.cuda.synchronize()
@@ -74,14 +75,36 @@ def main() -> int:
         torch.cuda.synchronize()
         return a.elapsed_time(b) / steps
 
+    def graph_ms(fn, steps, warmup):
+        """`steps` calls captured into one HIP graph; HIP events around one replay on the current
+        stream.  Two or three launches of 5-15 us each are otherwise paced by the host."""
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(steps):
+                fn()
+        g.replay()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        g.replay()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / steps, g
+
     # ---- kernel map (built once, reused by every step; timed separately) -----------------------
     build = lambda: backend.build_kernel_map(cd, ks, (1, 1, 1), (0, 0, 0), [0, 0, 0], cmax, True, want_csr=True)
     km = build()
-    t0 = time.perf_counter()
-    for _ in range(5):
+    for _ in range(3):
         build()
     torch.cuda.synchronize()
-    map_ms = (time.perf_counter() - t0) / 5 * 1e3
+    t0 = time.perf_counter()
+    for _ in range(20):
+        build()
+    torch.cuda.synchronize()
+    map_ms = (time.perf_counter() - t0) / 20 * 1e3
     M = km.M
 
     names = {DATAFLOW_FOD: "fod", DATAFLOW_GMS: "gms", DATAFLOW_OS: "os", DATAFLOW_FDS: "fds"}
@@ -91,21 +114,33 @@ def main() -> int:
     else:
         flow = {v: k for k, v in names.items()}[args.dataflow]
     buffer = torch.empty(max(km.qsum * (c_in + c_out), 1), dtype=torch.float16, device=dev)
-    step = lambda f=flow: backend.conv_forward(fd, wd, km, f, buffer=buffer, packed=packed)
+    out_buf = torch.empty((n, c_out), dtype=torch.float16, device=dev)
+    step = lambda f=flow: backend.conv_forward(fd, wd, km, f, buffer=buffer, packed=packed, out=out_buf)
 
     # ---- timed region ---------------------------------------------------------------------------
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    # Eager: K calls through the Python front end (what a caller without graphs sees; host paced).
     t_wall = time.perf_counter()
-    start.record()
-    for _ in range(args.steps):
-        step()
-    stop.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t_wall) * 1e3 / args.steps
-    ms = start.elapsed_time(stop) / args.steps
+    eager_ms = ev_ms(step, args.steps, args.warmup)
+    wall_ms = (time.perf_counter() - t_wall) * 1e3 / (args.steps + args.warmup)
+    # Graph: the same K steps as one HIP graph, replayed once between HIP events.  Every replay is
+    # checked against the eager result, with eager work and synchronisations between replays.
+    want = step().clone()
+    launch = "hip_graph"
+    try:
+        ms, graph = graph_ms(step, args.steps, args.warmup)
+        for _ in range(3):
+            out_buf.zero_()
+            step(DATAFLOW_OS)
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            if not torch.equal(out_buf, want):
+                raise RuntimeError("a graph replay disagrees with the eager result")
+        timer = graph_ms
+    except Exception as exc:     # capture not possible: report the eager figure
+        print(f"bench.py: HIP graph capture failed ({exc}); timing eager launches", file=sys.stderr)
+        launch, ms = "eager", eager_ms
+        timer = lambda fn, steps, warmup: (ev_ms(fn, steps, warmup), None)
 
     # calibration for hardware counters: a plain copy of known size (2 x 19.2 MB) runs three times, so
     # that a counter run can scale FETCH_SIZE / WRITE_SIZE by what they read for it
@@ -115,19 +150,21 @@ def main() -> int:
     # ---- per-stage durations of the chosen dataflow (stage mask), and the other dataflows -------
     e = 2
     stages = {}
+    narrow = c_in <= 64 and c_out <= 64     # the barrier-free kernel takes these layers
     stage_names = {DATAFLOW_FOD: {0: "centre_gemm", 1: "fod_pairs", 2: "convert"},
                    DATAFLOW_GMS: {3: "gather", 1: "grouped_gemm", 0: "centre_gemm", 2: "scatter"},
-                   DATAFLOW_FDS: {1: "fod_pairs_to_buffer", 2: "centre_gemm_csr_sum"},
+                   DATAFLOW_FDS: ({1: "pairs_and_centre_gemm", 2: "partial_row_sum"} if narrow else
+                                  {1: "fod_pairs_to_buffer", 2: "centre_gemm_csr_sum"}),
                    DATAFLOW_OS: {1: "os_tile"}}[flow]
     if flow != DATAFLOW_OS:
         for bit, name in stage_names.items():
-            lib.pce_set_stage_mask(1 << bit)
-            stages[name] = ev_ms(step, max(20, args.steps // 4), 5)
+            lib.pce_set_stage_mask((1 << bit) | 16)       # bit 4 keeps the kernel selection of the full run
+            stages[name] = timer(step, max(20, args.steps // 4), 5)[0]
         lib.pce_set_stage_mask(0xFFFFFFFF)
     else:
         stages["os_tile"] = ms
-    others = {names[f]: ev_ms(lambda f=f: backend.conv_forward(fd, wd, km, f, buffer=buffer, packed=packed), max(20, args.steps // 4), 5)
-              for f in names if f != flow}
+    others = {names[f]: timer(lambda f=f: step(f), max(20, args.steps // 4), 5)[0] for f in names if f != flow and f != DATAFLOW_FOD}
+    others[names[DATAFLOW_FOD]] = ev_ms(lambda: step(DATAFLOW_FOD), max(20, args.steps // 4), 5)   # allocates: eager
 
     # algorithmic bytes of the layer: every tensor once + the pair list
     b_conv = n * c_in * e + n * c_out * e + 27 * c_in * c_out * e + 8 * M
@@ -144,6 +181,9 @@ def main() -> int:
         "os_tile": b_conv - 8 * M + 4 * 27 * n,
         "fod_pairs_to_buffer": M * (c_in + c_out) * e + 4 * M + 26 * c_in * c_out * e,
         "centre_gemm_csr_sum": n * c_in * e + n * c_out * e + c_in * c_out * e + M * c_out * e + 4 * M + 4 * (n + 1),
+        # centre rows in and out, pair rows in and partial rows out, the two index lists, every weight once
+        "pairs_and_centre_gemm": n * c_in * e + n * c_out * e + M * (c_in + c_out) * e + 8 * M + 27 * c_in * c_out * e,
+        "partial_row_sum": 3 * M * c_out * e + 8 * M + 4 * (n + 1),
     }[dom]
     achieved = dom_bytes / (stages[dom] * 1e-3) / 1e9
     # HBM bytes per launch of that kernel from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
@@ -167,9 +207,11 @@ def main() -> int:
         "metric": "subm3_conv_layer_ms", "value": round(ms, 5), "unit": "ms", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": False, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
-        "config": {"workload": what.format(n=n, M=M), "dataflow": names[flow], "selector": args.dataflow == "auto"},
+        "config": {"workload": what.format(n=n, M=M), "dataflow": names[flow], "selector": args.dataflow == "auto",
+                   "launch": launch},
         "roofline": roofline,
-        "extra": {"wall_ms_per_step": round(wall_ms, 5), "map_build_ms": round(map_ms, 4),
+        "extra": {"eager_ms_per_step": round(eager_ms, 5), "eager_wall_ms_per_step": round(wall_ms, 5),
+                  "map_build_ms": round(map_ms, 4),
                   "stage_ms": {k: round(v, 5) for k, v in stages.items()},
                   "other_dataflows_ms": {k: round(v, 5) for k, v in others.items()}},
     }

@@ -259,8 +259,13 @@ def dense_forward(feats: torch.Tensor, weight: torch.Tensor, packed: Optional[to
 
 
 def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataflow: int, transposed: bool = False,
-                 buffer: Optional[torch.Tensor] = None, packed: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """One forward convolution over an existing map with the chosen dataflow."""
+                 buffer: Optional[torch.Tensor] = None, packed: Optional[torch.Tensor] = None,
+                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One forward convolution over an existing map with the chosen dataflow.
+
+    ``out`` (optional) is a preallocated [n_out, c_out] tensor of the feature dtype: with it, a
+    large enough ``buffer`` and a dataflow other than plain fetch-on-demand the call allocates
+    nothing, so a loop of layers can be captured into a HIP graph."""
     lib = _lib.load()
     _require_cuda(feats, "feats")
     feats = feats.contiguous()
@@ -281,7 +286,10 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
     dev = feats.device
     s = _stream(dev)
     mid = _mid(km.ks) if km.subm else -1
-    out = torch.empty((n_out, c_out), dtype=feats.dtype, device=dev)
+    if out is None:
+        out = torch.empty((n_out, c_out), dtype=feats.dtype, device=dev)
+    elif out.shape != (n_out, c_out) or out.dtype != feats.dtype or out.device != dev or not out.is_contiguous():
+        raise ValueError(f"out must be a contiguous [{n_out}, {c_out}] {feats.dtype} tensor on {dev}")
     if dataflow == DATAFLOW_FOD:
         imap, omap = (km.omap, km.imap) if transposed else (km.imap, km.omap)
         ws_bytes = lib.pce_conv_fod_workspace_bytes(n_out, c_out, dt)

@@ -517,15 +517,21 @@ __device__ __forceinline__ void store_rows_via_lds(const float (&V)[NB][2][8], v
 // TMODE / TEPI >= 0 fix the mode and the epilogue at compile time (the hot combinations); -1 reads
 // them from the arguments.
 template <typename T, int NB, bool FAST, int TMODE, int TEPI>
-__device__ __forceinline__ void tile_body(const TileArgs &a, long long tile, int slab, T *Wl,
-                                          typename Partials<T, NB>::PV (*Pl)[WaveLds<NB>::PIECES]) {
+__global__ void __launch_bounds__(256, ((TMODE >= 0 && sizeof(T) == 2 && NB <= 2) ? 5 : 1)) tile_gemm_kernel(TileArgs a) {
   const int mode = TMODE >= 0 ? TMODE : a.mode;
   const int epi = TEPI >= 0 ? TEPI : a.epi;
   constexpr int NT = NB * 32;
   constexpr int KC = Cfg<T>::KC;
   typedef Partials<T, NB> P;
+  __shared__ __attribute__((aligned(16))) T Wl[KC * NT];
+  __shared__ __attribute__((aligned(16))) typename P::PV Pl[4][WaveLds<NB>::PIECES];
+
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int l32 = lane & 31, g = lane >> 5;
+  long long tile;
+  int slab;
+  // only the output-stationary mode re-reads rows across tiles; streaming modes keep launch order
+  if (!xcd_item(a.items, a.slabs, mode == MODE_OS, &tile, &slab)) return;
   const int n0 = slab * NT;
   const T *A = (const T *)a.A;
   const T *W = (const T *)a.W;
@@ -659,19 +665,6 @@ __device__ __forceinline__ void tile_body(const TileArgs &a, long long tile, int
     else
       store_row_pieces_slow<half_t, NB>(V, (half_t *)a.out, orow, a, n0, g);
   }
-}
-
-template <typename T, int NB, bool FAST, int TMODE, int TEPI>
-__global__ void __launch_bounds__(256, ((TMODE >= 0 && sizeof(T) == 2 && NB <= 2) ? 5 : 1)) tile_gemm_kernel(TileArgs a) {
-  typedef Partials<T, NB> P;
-  __shared__ __attribute__((aligned(16))) T Wl[Cfg<T>::KC * NB * 32];
-  __shared__ __attribute__((aligned(16))) typename P::PV Pl[4][WaveLds<NB>::PIECES];
-  const int mode = TMODE >= 0 ? TMODE : a.mode;
-  long long tile;
-  int slab;
-  // only the output-stationary mode re-reads rows across tiles; streaming modes keep launch order
-  if (!xcd_item(a.items, a.slabs, mode == MODE_OS, &tile, &slab)) return;
-  tile_body<T, NB, FAST, TMODE, TEPI>(a, tile, slab, Wl, Pl);
 }
 
 // ---- wavefront-independent form of the pair tiles and of the centre GEMM -------------------------

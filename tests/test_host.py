@@ -130,3 +130,30 @@ def test_scheduler_hint_and_buffer_size():
     assert pe.init_layer_scheduler({"stride": [1, 1, 2], "in": [4, 64, 64], "out": [64, 64, 64]}) == "whole"
     buf = pe.build_conv_buffer({"in": [4, 8], "out": [8, 16], "kernel": [3, 2]}, 10, torch.float16, "cpu")
     assert buf.numel() == (8 + 16) * 10 * 16 and buf.dtype == torch.float16
+
+
+def test_no_kernel_uses_scratch_memory(tmp_path):
+    """Register spills turn a memory-bound kernel into a several times slower one without changing a
+    single result: compile the device code with resource remarks and require zero scratch bytes."""
+    import subprocess
+    from pcengine_amd import build as pb
+    procs = []
+    for src in pb.SOURCES:
+        cmd = [pb._hipcc(), *pb.HIPCC_FLAGS, "--cuda-device-only", "-Rpass-analysis=kernel-resource-usage",
+               "-I", os.path.join(ROOT, "include"), "-I", pb.CSRC, "-c", os.path.join(pb.CSRC, src),
+               "-o", str(tmp_path / (src + ".o"))]
+        procs.append(subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True))
+    seen = 0
+    for p in procs:
+        out, _ = p.communicate()
+        assert p.returncode == 0, out[-2000:]
+        name = None
+        for line in out.splitlines():
+            m = re.search(r"Function Name: (\S+)", line)
+            if m:
+                name = m.group(1)
+            m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", line)
+            if m:
+                seen += 1
+                assert int(m.group(1)) == 0, f"{name} spills {m.group(1)} bytes per lane"
+    assert seen > 20
