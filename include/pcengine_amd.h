@@ -146,6 +146,23 @@ int pce_kmap_build(const int32_t *in_coords_dev, int64_t n_in, const int32_t *ou
  * For a transposed layer pass the map with the roles swapped (imap<->omap, icsr<->ocsr), as the
  * reference front end does (script/spconv.py:142-151, 236-244). */
 
+/* Fused epilogue of a forward layer: out = act(conv + bias + residual).  bias[c_out] and
+ * residual[n_out,c_out] have the layer's dtype and live on the device; either may be NULL.
+ * residual must not alias out_feats.  Every forward entry point takes `const pce_epilogue_t *`,
+ * NULL for the plain convolution.  The output-stationary, deferred-scatter and dense entry points
+ * apply it in the kernel that stores the output rows; fetch-on-demand and gather-GEMM-scatter run
+ * one extra in-place pass over the output.  It replaces the separate bias add, activation and
+ * residual add of the reference front end (script/spconv.py:453-454, script/activation.py:6-15,
+ * script/sptensor.py:80-91); a BatchNorm in inference mode folds into weight and bias beforehand
+ * (script/batchnorm.py:7-10). */
+enum { PCE_ACT_NONE = 0, PCE_ACT_RELU = 1, PCE_ACT_LEAKY_RELU = 2 };
+typedef struct pce_epilogue {
+  const void *bias;
+  const void *residual;
+  int32_t act;         /* PCE_ACT_* */
+  float slope;         /* negative slope of PCE_ACT_LEAKY_RELU */
+} pce_epilogue_t;
+
 /* fp16 weights can be handed over a second time in the order the kernels stage them into LDS
  * (pce_pack_weights, once per weight tensor); every forward entry point takes that copy as
  * `weight_packed`, or NULL to stage from the row-major tensor.  fp32 has no packed form. */
@@ -161,7 +178,7 @@ int pce_conv_fwd_fod(const void *in_feats, const void *weight, const void *weigh
                      int64_t n_in, int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv,
                      int32_t mid, const int32_t *imap_dev, const int32_t *omap_dev,
                      const int32_t *kpos_dev, const int32_t *qkpos_dev, int64_t qsum,
-                     void *ws_dev, int64_t ws_bytes, pce_stream_t stream);
+                     void *ws_dev, int64_t ws_bytes, const pce_epilogue_t *epilogue, pce_stream_t stream);
 
 /* Gather - GEMM - scatter: CSR-coded map; `buffer` holds qsum*(c_in+c_out) elements of dtype
  * (first qsum*c_in gathered inputs, then the GEMM outputs; backend/spconv.cu:121). */
@@ -171,7 +188,7 @@ int pce_conv_fwd_gms(const void *in_feats, const void *weight, const void *weigh
                      int32_t mid, const int32_t *icsr_dev, const int32_t *icode_dev,
                      const int32_t *ocsr_dev, const int32_t *ocode_dev, const int32_t *kpos_dev,
                      const int32_t *qkpos_dev, int64_t qsum, void *buffer_dev,
-                     int64_t buffer_elems, pce_stream_t stream);
+                     int64_t buffer_elems, const pce_epilogue_t *epilogue, pce_stream_t stream);
 
 /* Fetch-on-demand with deferred scatter.  Gather side: the pair list (imap, kpos, qkpos).  Scatter
  * side: oslot[p] = position of pair p among the entries of its output row in CSR order, and the
@@ -195,7 +212,7 @@ int pce_conv_fwd_fds(const void *in_feats, const void *weight, const void *weigh
                      const int32_t *qkpos_dev,
                      const int32_t *kpos_host, const int32_t *qkpos_host, const int32_t *ocsr_dev,
                      int64_t n_pairs, int64_t qsum, void *buffer_dev, int64_t buffer_elems,
-                     pce_stream_t stream);
+                     const pce_epilogue_t *epilogue, pce_stream_t stream);
 
 /* Output-stationary: nbr[kv*n_out] from pce_kmap_build (for a transposed layer, a table built
  * with the roles swapped).  One kernel, one store per output row.  No counterpart in the
@@ -204,13 +221,14 @@ int pce_conv_fwd_fds(const void *in_feats, const void *weight, const void *weigh
 int pce_conv_fwd_os(const void *in_feats, const void *weight, const void *weight_packed,
                     void *out_feats, int32_t dtype,
                     int64_t n_in, int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv,
-                    const int32_t *nbr_dev, pce_stream_t stream);
+                    const int32_t *nbr_dev, const pce_epilogue_t *epilogue, pce_stream_t stream);
 
 /* out[n,c_out] = in[n,c_in] * weight[c_in,c_out]: the 1x1 stride-1 shortcut of the front end
  * (script/spconv.py:297-304), on the same MFMA tile kernel. */
 int pce_conv_fwd_dense(const void *in_feats, const void *weight, const void *weight_packed,
                        void *out_feats, int32_t dtype,
-                       int64_t n, int32_t c_in, int32_t c_out, pce_stream_t stream);
+                       int64_t n, int32_t c_in, int32_t c_out, const pce_epilogue_t *epilogue,
+                       pce_stream_t stream);
 
 /* Per-layer dataflow choice from map density (pairs per output row) and channel widths. */
 int pce_select_dataflow(int64_t n_in, int64_t n_out, int64_t n_pairs, int32_t c_in, int32_t c_out,

@@ -34,6 +34,14 @@ class Geom(Structure):
         return g
 
 
+class Epilogue(Structure):
+    """pce_epilogue_t: out = act(conv + bias + residual)."""
+    _fields_ = [("bias", c_void_p), ("residual", c_void_p), ("act", c_int32), ("slope", ctypes.c_float)]
+
+
+ACT_NONE, ACT_RELU, ACT_LEAKY_RELU = 0, 1, 2
+
+
 class PCEError(RuntimeError):
     pass
 
@@ -56,13 +64,14 @@ _SIGNATURES = {
     "pce_pack_weights": (c_int32, [c_void_p, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
     "pce_conv_fwd_fds": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32,
                                    c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, POINTER(c_int32), POINTER(c_int32), c_void_p, c_int64,
-                                   c_int64, c_void_p, c_int64, c_void_p]),
+                                   c_int64, c_void_p, c_int64, POINTER(Epilogue), c_void_p]),
     "pce_conv_fwd_fod": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32,
-                                   c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
+                                   c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, POINTER(Epilogue), c_void_p]),
     "pce_conv_fwd_gms": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32,
-                                   c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
-    "pce_conv_fwd_os": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
-    "pce_conv_fwd_dense": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32, c_void_p]),
+                                   c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64,
+                                   POINTER(Epilogue), c_void_p]),
+    "pce_conv_fwd_os": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_void_p, POINTER(Epilogue), c_void_p]),
+    "pce_conv_fwd_dense": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32, POINTER(Epilogue), c_void_p]),
     "pce_select_dataflow": (c_int32, [c_int64, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32]),
 }
 

@@ -244,8 +244,40 @@ def pack_weights(weight: torch.Tensor) -> Optional[torch.Tensor]:
     return packed
 
 
-def dense_forward(feats: torch.Tensor, weight: torch.Tensor, packed: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """feats @ weight for the 1x1 stride-1 layer (script/spconv.py:297-304)."""
+def _epilogue(feats: torch.Tensor, n_out: int, c_out: int, bias, residual, act):
+    """(ctypes struct or None, tensors to keep alive) for ``out = act(conv + bias + residual)``.
+    ``act``: None, 'relu', or ('leaky_relu', negative_slope)."""
+    if bias is None and residual is None and act is None:
+        return None, ()
+    e = _lib.Epilogue()
+    keep = []
+    if bias is not None:
+        bias = bias.detach().to(device=feats.device, dtype=feats.dtype).contiguous()
+        if bias.numel() != c_out:
+            raise ValueError(f"bias has {bias.numel()} elements, the layer has {c_out} output channels")
+        e.bias = bias.data_ptr()
+        keep.append(bias)
+    if residual is not None:
+        _require_cuda(residual, "residual")
+        if residual.shape != (n_out, c_out) or residual.dtype != feats.dtype:
+            raise ValueError(f"residual must be [{n_out}, {c_out}] {feats.dtype}")
+        residual = residual.contiguous()
+        e.residual = residual.data_ptr()
+        keep.append(residual)
+    if act is None:
+        e.act = _lib.ACT_NONE
+    elif act == "relu":
+        e.act = _lib.ACT_RELU
+    elif isinstance(act, tuple) and len(act) == 2 and act[0] == "leaky_relu":
+        e.act, e.slope = _lib.ACT_LEAKY_RELU, float(act[1])
+    else:
+        raise ValueError(f"unknown activation {act!r}")
+    return e, keep
+
+
+def dense_forward(feats: torch.Tensor, weight: torch.Tensor, packed: Optional[torch.Tensor] = None,
+                  bias: Optional[torch.Tensor] = None, residual: Optional[torch.Tensor] = None, act=None) -> torch.Tensor:
+    """act(feats @ weight + bias + residual) for the 1x1 stride-1 layer (script/spconv.py:297-304)."""
     lib = _lib.load()
     _require_cuda(feats, "feats")
     feats = feats.contiguous()
@@ -253,15 +285,19 @@ def dense_forward(feats: torch.Tensor, weight: torch.Tensor, packed: Optional[to
     if feats.shape[1] != weight.shape[0]:
         raise ValueError("Input feature size and kernel size mismatch")
     out = torch.empty((feats.shape[0], weight.shape[1]), dtype=feats.dtype, device=feats.device)
+    epi, _keep = _epilogue(feats, feats.shape[0], weight.shape[1], bias, residual, act)
     _lib.check(lib.pce_conv_fwd_dense(feats.data_ptr(), weight.data_ptr(), _ptr(packed), out.data_ptr(), _dtype_code(feats),
-                                      feats.shape[0], feats.shape[1], weight.shape[1], _stream(feats.device)))
+                                      feats.shape[0], feats.shape[1], weight.shape[1], epi, _stream(feats.device)))
     return out
 
 
 def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataflow: int, transposed: bool = False,
                  buffer: Optional[torch.Tensor] = None, packed: Optional[torch.Tensor] = None,
-                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """One forward convolution over an existing map with the chosen dataflow.
+                 out: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
+                 residual: Optional[torch.Tensor] = None, act=None) -> torch.Tensor:
+    """One forward convolution over an existing map with the chosen dataflow:
+    ``act(conv(feats) + bias + residual)``, the last three optional and applied inside the kernels
+    (``act``: None, 'relu' or ('leaky_relu', slope)).
 
     ``out`` (optional) is a preallocated [n_out, c_out] tensor of the feature dtype: with it, a
     large enough ``buffer`` and a dataflow other than plain fetch-on-demand the call allocates
@@ -290,13 +326,14 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
         out = torch.empty((n_out, c_out), dtype=feats.dtype, device=dev)
     elif out.shape != (n_out, c_out) or out.dtype != feats.dtype or out.device != dev or not out.is_contiguous():
         raise ValueError(f"out must be a contiguous [{n_out}, {c_out}] {feats.dtype} tensor on {dev}")
+    epi, _keep = _epilogue(feats, n_out, c_out, bias, residual, act)
     if dataflow == DATAFLOW_FOD:
         imap, omap = (km.omap, km.imap) if transposed else (km.imap, km.omap)
         ws_bytes = lib.pce_conv_fod_workspace_bytes(n_out, c_out, dt)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
         _lib.check(lib.pce_conv_fwd_fod(feats.data_ptr(), weight.data_ptr(), _ptr(packed), out.data_ptr(), dt, n_in, n_out,
                                         c_in, c_out, kv, mid, imap.data_ptr(), omap.data_ptr(), km.kpos.data_ptr(),
-                                        km.qkpos.data_ptr(), km.qsum, _ptr(ws), ws_bytes, s))
+                                        km.qkpos.data_ptr(), km.qsum, _ptr(ws), ws_bytes, epi, s))
     elif dataflow == DATAFLOW_FDS:
         ensure_csr(km)
         need = km.M * c_out
@@ -307,7 +344,7 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
         _lib.check(lib.pce_conv_fwd_fds(feats.data_ptr(), weight.data_ptr(), _ptr(packed), out.data_ptr(), dt, n_in, n_out,
                                         c_in, c_out, kv, mid, imap.data_ptr(), omap.data_ptr(), oslot.data_ptr(), km.kpos.data_ptr(),
                                         km.qkpos.data_ptr(), km.kpos_host, km.qkpos_host, ocsr.data_ptr(), km.M, km.qsum,
-                                        buffer.data_ptr(), buffer.numel(), s))
+                                        buffer.data_ptr(), buffer.numel(), epi, s))
     elif dataflow == DATAFLOW_GMS:
         ensure_csr(km)
         need = km.qsum * (c_in + c_out)
@@ -316,12 +353,12 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
         icsr, icode, ocsr, ocode = (km.ocsr, km.ocode, km.icsr, km.icode) if transposed else (km.icsr, km.icode, km.ocsr, km.ocode)
         _lib.check(lib.pce_conv_fwd_gms(feats.data_ptr(), weight.data_ptr(), _ptr(packed), out.data_ptr(), dt, n_in, n_out,
                                         c_in, c_out, kv, mid, icsr.data_ptr(), icode.data_ptr(), ocsr.data_ptr(), ocode.data_ptr(),
-                                        km.kpos.data_ptr(), km.qkpos.data_ptr(), km.qsum, buffer.data_ptr(), buffer.numel(), s))
+                                        km.kpos.data_ptr(), km.qkpos.data_ptr(), km.qsum, buffer.data_ptr(), buffer.numel(), epi, s))
     elif dataflow == DATAFLOW_OS:
         ensure_nbr(km, transposed)
         nbr = km.nbr_in if transposed else km.nbr_out
         _lib.check(lib.pce_conv_fwd_os(feats.data_ptr(), weight.data_ptr(), _ptr(packed), out.data_ptr(), dt, n_in, n_out,
-                                       c_in, c_out, kv, nbr.data_ptr(), s))
+                                       c_in, c_out, kv, nbr.data_ptr(), epi, s))
     else:
         raise NotImplementedError(f"unknown dataflow {dataflow}")
     return out
@@ -389,7 +426,7 @@ def conv_fwd_d2_cuda(in_feats, kernel, ksize_code, sum_nnz, out_feats, kpos, qkp
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=in_feats.device) if ws_bytes else None
     _lib.check(lib.pce_conv_fwd_fod(in_feats.data_ptr(), kernel.data_ptr(), None, out_feats.data_ptr(), dt, n_in, n_out, c_in,
                                     c_out, kv, _ksize_mid(ksize_code, separate_mid), in_map.data_ptr(), out_map.data_ptr(),
-                                    kpos.data_ptr(), qkpos.data_ptr(), int(sum_nnz), _ptr(ws), ws_bytes,
+                                    kpos.data_ptr(), qkpos.data_ptr(), int(sum_nnz), _ptr(ws), ws_bytes, None,
                                     _stream(in_feats.device)))
 
 
@@ -410,7 +447,7 @@ def conv_fwd_d1_cuda(in_feats, kernel, ksize_code, qsum_nnz, out_feats, kpos, qk
     _lib.check(lib.pce_conv_fwd_gms(in_feats.data_ptr(), kernel.data_ptr(), None, out_feats.data_ptr(), dt, in_feats.shape[0],
                                     out_feats.shape[0], c_in, c_out, kv, _ksize_mid(ksize_code, separate_mid),
                                     in_csr.data_ptr(), in_map.data_ptr(), out_csr.data_ptr(), out_map.data_ptr(),
-                                    kpos.data_ptr(), qkpos.data_ptr(), int(qsum_nnz), buffer.data_ptr(), buffer.numel(),
+                                    kpos.data_ptr(), qkpos.data_ptr(), int(qsum_nnz), buffer.data_ptr(), buffer.numel(), None,
                                     _stream(in_feats.device)))
 
 

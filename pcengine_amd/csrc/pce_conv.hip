@@ -61,6 +61,10 @@ struct TileArgs {
   int a_vec, w_vec, o_vec, b_vec;  // 16-byte accesses allowed on A rows / W rows / out rows / buf rows
   int k8_total, n_pad;             // packed weight extents
   int host_pos;                    // kpos_h / qkpos_h are valid
+  const void *bias;                // fused epilogue of the launch that stores output rows: out = act(acc + bias + res)
+  const void *res;
+  int act;
+  float slope;
   int kpos_h[MAX_KV_ARGS + 1];
   int qkpos_h[MAX_KV_ARGS + 1];
 };
@@ -441,6 +445,59 @@ __device__ __forceinline__ void add_partials_slow(float (&V)[NB][2][8], int e0, 
   }
 }
 
+// ---- fused epilogue: out = act(acc + bias + residual) -------------------------------------------
+__device__ __forceinline__ float act_apply(float v, int act, float slope) {
+  if (act == PCE_ACT_RELU) return v > 0.f ? v : 0.f;
+  if (act == PCE_ACT_LEAKY_RELU) return v > 0.f ? v : v * slope;
+  return v;
+}
+
+// eight consecutive elements of a row of T as floats; VEC: the address is 16-byte aligned
+template <typename T, bool VEC>
+__device__ __forceinline__ void add8(float (&v)[8], const T *p, int valid) {
+  if (VEC) {
+    if (sizeof(T) == 2) {
+      half8 x = *reinterpret_cast<const half8 *>(p);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] += (float)x[j];
+    } else {
+      f32x4 x0 = *reinterpret_cast<const f32x4 *>(p), x1 = *reinterpret_cast<const f32x4 *>(p + 4);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v[j] += (float)x0[j];
+        v[4 + j] += (float)x1[j];
+      }
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (j < valid) v[j] += (float)p[j];
+  }
+}
+
+// on the row pieces of the tile epilogue (lane g of row `orow` owns columns n0 + 32*nb + 16*h + 8*g + 0..7)
+template <typename T, int NB, bool VEC>
+__device__ __forceinline__ void epilogue_row_pieces(float (&V)[NB][2][8], const TileArgs &a, int orow, int n0, int g,
+                                                    bool with_act) {
+  const T *bias = (const T *)a.bias;
+  const T *res = (const T *)a.res;
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      int c0 = n0 + nb * 32 + 16 * h + 8 * g;
+      int valid = a.c_out - c0;
+      if (valid > 0 && orow >= 0) {
+        if (bias) add8<T, VEC>(V[nb][h], bias + c0, valid);
+        if (res) add8<T, VEC>(V[nb][h], res + (long long)orow * a.c_out + c0, valid);
+      }
+      if (with_act) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) V[nb][h][j] = act_apply(V[nb][h][j], a.act, a.slope);
+      }
+    }
+}
+
 // element-wise stores straight from the row pieces (rows that are not 16-byte multiples)
 template <typename TO, int NB>
 __device__ __forceinline__ void store_row_pieces_slow(const float (&V)[NB][2][8], TO *out, int orow, const TileArgs &a,
@@ -654,6 +711,12 @@ __global__ void __launch_bounds__(256, ((TMODE >= 0 && sizeof(T) == 2 && NB <= 2
       add_partials_slow<T, NB>(V, e0, e1, a, n0, g);
   }
   const bool f32out = (epi == EPI_ROWS_F32) || sizeof(T) == 4;
+  if (a.bias || a.res || a.act) {  // set only on launches that store finished output rows
+    if (FAST)
+      epilogue_row_pieces<T, NB, true>(V, a, orow, n0, g, a.act != PCE_ACT_NONE);
+    else
+      epilogue_row_pieces<T, NB, false>(V, a, orow, n0, g, a.act != PCE_ACT_NONE);
+  }
   if (FAST || a.o_vec) {
     if (f32out)
       store_rows_via_lds<float, NB>(V, Pl[wave], (float *)a.out, orow, a, n0, lane, l32, g);
@@ -727,6 +790,17 @@ __global__ void __launch_bounds__(256, 5) wave_gemm_kernel(TileArgs pair, TileAr
   float V[NB][2][8];
   gather_row_pieces<NB>(acc, V, g);
   half_t *out = (half_t *)(is_pair ? pair.out : centre.out);
+  if (!is_pair && (centre.bias || centre.res || centre.act)) {
+    // rows that receive partial rows later get their activation from the pass that adds them
+    bool alone = orow >= 0 && centre.ocsr[orow] == centre.ocsr[orow + 1];
+    epilogue_row_pieces<half_t, NB, true>(V, centre, orow, 0, g, false);
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) V[nb][h][j] = alone ? act_apply(V[nb][h][j], centre.act, centre.slope) : V[nb][h][j];
+  }
   store_rows_via_lds<half_t, NB>(V, Pl[wave], out, orow, a, 0, lane, l32, g);
 }
 
@@ -753,6 +827,8 @@ static int launch_wave_gemm(const TileArgs &pair, const TileArgs &centre, hipStr
 static bool wave_gemm_ok(const TileArgs &a, int elem_size) {
   return elem_size == 2 && a.Wp && a.a_vec && a.o_vec && a.c_in % 16 == 0 && a.c_in <= 64 && a.c_out <= 64;
 }
+
+static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 static unsigned xcd_grid(TileArgs *a, long long tiles, int slabs) {
   a->slabs = slabs;
@@ -783,7 +859,7 @@ static int launch_tile(const TileArgs &a, long long tiles, hipStream_t s) {
   if (tiles <= 0) return PCE_OK;
   if (tiles * ((a.c_out + 127) / 128) >= (1ll << 31) - 8) PCE_FAIL(PCE_ECAPACITY, "tile count %lld exceeds the grid limit", tiles);
   bool fast = a.a_vec && a.o_vec && (sizeof(T) == 2 ? a.Wp != nullptr : a.w_vec != 0) &&
-              (a.epi != EPI_ROWS_CSR || a.b_vec);
+              (a.epi != EPI_ROWS_CSR || a.b_vec) && aligned16(a.bias) && aligned16(a.res);
   if (!fast)
     launch_tile_nb<T, false, -1, -1>(a, tiles, s);
   else if (a.mode == MODE_DENSE && a.epi == EPI_ROWS_CSR)
@@ -844,14 +920,16 @@ template <typename T, int VEC>
 __global__ void __launch_bounds__(256) scatter_rows_kernel(const T *__restrict__ buf, long long n_out, int c_out, int G,
                                                            const int *__restrict__ ocsr, const int *__restrict__ ocode,
                                                            const int *__restrict__ qkpos, T *__restrict__ out,
-                                                           int add_existing) {
+                                                           int add_existing, const T *__restrict__ bias,
+                                                           const T *__restrict__ res, int act, float slope) {
   typedef typename VecOf<T, VEC>::type V;
   int rows_per_block = 256 / G;
   long long row = (long long)blockIdx.x * rows_per_block + threadIdx.x / G;
   int sub = threadIdx.x % G;
   if (row >= n_out) return;
   int e0 = ocsr[row], e1 = ocsr[row + 1];
-  if (add_existing && e0 == e1) return;
+  // a row without staging rows keeps its centre term as it is, unless an epilogue has to touch it
+  if (add_existing && e0 == e1 && !bias && !res && act == PCE_ACT_NONE) return;
   int row_vecs = c_out / VEC;
   for (int v = sub; v < row_vecs; v += G) {
     float acc[VEC];
@@ -871,8 +949,18 @@ __global__ void __launch_bounds__(256) scatter_rows_kernel(const T *__restrict__
       for (int j = 0; j < VEC; ++j) acc[j] += (float)(reinterpret_cast<const T *>(&x)[j]);
     }
     V y;
+    if (bias) {
+      V b = *reinterpret_cast<const V *>(&bias[(long long)v * VEC]);
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) reinterpret_cast<T *>(&y)[j] = (T)acc[j];
+      for (int j = 0; j < VEC; ++j) acc[j] += (float)(reinterpret_cast<const T *>(&b)[j]);
+    }
+    if (res) {
+      V r = *reinterpret_cast<const V *>(&res[row * c_out + (long long)v * VEC]);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) acc[j] += (float)(reinterpret_cast<const T *>(&r)[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) reinterpret_cast<T *>(&y)[j] = (T)act_apply(acc[j], act, slope);
     *reinterpret_cast<V *>(&out[row * c_out + (long long)v * VEC]) = y;
   }
 }
@@ -880,7 +968,9 @@ __global__ void __launch_bounds__(256) scatter_rows_kernel(const T *__restrict__
 // out[row] = sum of the contiguous partial rows buf[csr[row] .. csr[row+1]), fp32 accumulate
 template <typename T, int VEC>
 __global__ void __launch_bounds__(256) rowsum_kernel(const T *__restrict__ buf, long long n_out, int c_out, int G,
-                                                     const int *__restrict__ csr, T *__restrict__ out) {
+                                                     const int *__restrict__ csr, T *__restrict__ out,
+                                                     const T *__restrict__ bias, const T *__restrict__ res, int act,
+                                                     float slope) {
   typedef typename VecOf<T, VEC>::type V;
   int rows_per_block = 256 / G;
   long long row = (long long)blockIdx.x * rows_per_block + threadIdx.x / G;
@@ -898,10 +988,50 @@ __global__ void __launch_bounds__(256) rowsum_kernel(const T *__restrict__ buf, 
       for (int j = 0; j < VEC; ++j) acc[j] += (float)(reinterpret_cast<const T *>(&x)[j]);
     }
     V y;
+    if (bias) {
+      V b = *reinterpret_cast<const V *>(&bias[(long long)v * VEC]);
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) reinterpret_cast<T *>(&y)[j] = (T)acc[j];
+      for (int j = 0; j < VEC; ++j) acc[j] += (float)(reinterpret_cast<const T *>(&b)[j]);
+    }
+    if (res) {
+      V r = *reinterpret_cast<const V *>(&res[row * c_out + (long long)v * VEC]);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) acc[j] += (float)(reinterpret_cast<const T *>(&r)[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) reinterpret_cast<T *>(&y)[j] = (T)act_apply(acc[j], act, slope);
     *reinterpret_cast<V *>(&out[row * c_out + (long long)v * VEC]) = y;
   }
+}
+
+// in-place epilogue for the dataflows whose last kernel cannot take it: out = act(out + bias + res)
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256) epilogue_rows_kernel(T *__restrict__ out, long long n_out, int c_out,
+                                                            const T *__restrict__ bias, const T *__restrict__ res,
+                                                            int act, float slope) {
+  typedef typename VecOf<T, VEC>::type V;
+  int row_vecs = c_out / VEC;
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_out * row_vecs) return;
+  long long row = i / row_vecs;
+  int v = (int)(i - row * row_vecs);
+  V x = *reinterpret_cast<const V *>(&out[row * c_out + (long long)v * VEC]);
+  float acc[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) acc[j] = (float)(reinterpret_cast<const T *>(&x)[j]);
+  if (bias) {
+    V b = *reinterpret_cast<const V *>(&bias[(long long)v * VEC]);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[j] += (float)(reinterpret_cast<const T *>(&b)[j]);
+  }
+  if (res) {
+    V r = *reinterpret_cast<const V *>(&res[row * c_out + (long long)v * VEC]);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[j] += (float)(reinterpret_cast<const T *>(&r)[j]);
+  }
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) reinterpret_cast<T *>(&x)[j] = (T)act_apply(acc[j], act, slope);
+  *reinterpret_cast<V *>(&out[row * c_out + (long long)v * VEC]) = x;
 }
 
 // out[o] += sum of the partial rows of o, for the rows that have any: one group of G lanes per pair;
@@ -909,7 +1039,8 @@ __global__ void __launch_bounds__(256) rowsum_kernel(const T *__restrict__ buf, 
 template <typename T, int VEC>
 __global__ void __launch_bounds__(256) rowsum_pairs_kernel(const T *__restrict__ buf, long long n_pairs, int c_out, int G,
                                                            const int *__restrict__ omap, const int *__restrict__ oslot,
-                                                           const int *__restrict__ csr, T *__restrict__ out) {
+                                                           const int *__restrict__ csr, T *__restrict__ out, int act,
+                                                           float slope) {
   typedef typename VecOf<T, VEC>::type V;
   long long p = (long long)blockIdx.x * (256 / G) + threadIdx.x / G;
   int sub = threadIdx.x % G;
@@ -930,7 +1061,7 @@ __global__ void __launch_bounds__(256) rowsum_pairs_kernel(const T *__restrict__
       for (int j = 0; j < VEC; ++j) acc[j] += (float)(reinterpret_cast<const T *>(&y)[j]);
     }
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) reinterpret_cast<T *>(&x)[j] = (T)acc[j];
+    for (int j = 0; j < VEC; ++j) reinterpret_cast<T *>(&x)[j] = (T)act_apply(acc[j], act, slope);
     *reinterpret_cast<V *>(&out[(long long)row * c_out + (long long)v * VEC]) = x;
   }
 }
@@ -973,7 +1104,6 @@ static int pow2_at_least(int v) {
   return p;
 }
 
-static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 static int check_common(const char *fn, const void *in, const void *w, const void *out, int dtype, int64_t n_in,
                         int64_t n_out, int c_in, int c_out, int kv, int mid) {
@@ -1029,6 +1159,55 @@ static void set_host_pos(TileArgs *a, const int32_t *kpos_host, const int32_t *q
   }
 }
 
+struct Epi {
+  const void *bias, *res;
+  int act;
+  float slope;
+  bool any() const { return bias || res || act != PCE_ACT_NONE; }
+};
+
+static int read_epilogue(const char *fn, const pce_epilogue_t *e, const void *out, Epi *o) {
+  o->bias = o->res = nullptr;
+  o->act = PCE_ACT_NONE;
+  o->slope = 0.f;
+  if (!e) return PCE_OK;
+  if (e->act != PCE_ACT_NONE && e->act != PCE_ACT_RELU && e->act != PCE_ACT_LEAKY_RELU)
+    PCE_FAIL(PCE_EINVAL, "%s: unknown activation %d", fn, (int)e->act);
+  if (e->residual && e->residual == out) PCE_FAIL(PCE_EINVAL, "%s: the residual must not alias the output", fn);
+  o->bias = e->bias;
+  o->res = e->residual;
+  o->act = e->act;
+  o->slope = e->slope;
+  return PCE_OK;
+}
+
+static void set_epi(TileArgs *a, const Epi &e) {
+  a->bias = e.bias;
+  a->res = e.res;
+  a->act = e.act;
+  a->slope = e.slope;
+}
+
+static bool epi_aligned(const Epi &e) { return aligned16(e.bias) && aligned16(e.res); }
+
+// one in-place pass: out = act(out + bias + res)
+template <typename T>
+static int launch_epilogue_pass(T *out, int64_t n_out, int c_out, const Epi &e, hipStream_t s) {
+  if (!e.any()) return PCE_OK;
+  constexpr int VEC = sizeof(T) == 2 ? 8 : 4;
+  if (c_out % VEC == 0 && aligned16(out) && epi_aligned(e)) {
+    long long total = (long long)n_out * (c_out / VEC);
+    hipLaunchKernelGGL((epilogue_rows_kernel<T, VEC>), dim3((unsigned)pce_div_up(total, 256)), dim3(256), 0, s, out,
+                       (long long)n_out, c_out, (const T *)e.bias, (const T *)e.res, e.act, e.slope);
+  } else {
+    long long total = (long long)n_out * c_out;
+    hipLaunchKernelGGL((epilogue_rows_kernel<T, 1>), dim3((unsigned)pce_div_up(total, 256)), dim3(256), 0, s, out,
+                       (long long)n_out, c_out, (const T *)e.bias, (const T *)e.res, e.act, e.slope);
+  }
+  PCE_LAUNCH_CHECK("epilogue_rows");
+  return PCE_OK;
+}
+
 extern "C" int64_t pce_packed_weight_bytes(int32_t dtype, int32_t kv, int32_t c_in, int32_t c_out) {
   if (dtype != PCE_F16) return 0;
   return (int64_t)kv * ((c_in + 7) / 8) * ((c_out + 31) / 32 * 32) * 16;
@@ -1055,7 +1234,7 @@ extern "C" int64_t pce_conv_fod_workspace_bytes(int64_t n_out, int32_t c_out, in
 template <typename T>
 static int fod_impl(const void *in, const void *w, const void *wp, void *out, int64_t n_out, int c_in, int c_out, int kv,
                     int mid, const int *imap, const int *omap, const int *kpos, const int *qkpos, int64_t qsum,
-                    float *acc, hipStream_t s) {
+                    float *acc, const Epi &e, hipStream_t s) {
   TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
   set_out<T>(&a, acc, true);
   int rc;
@@ -1084,42 +1263,47 @@ static int fod_impl(const void *in, const void *w, const void *wp, void *out, in
                        (const float *)acc, (half_t *)out, total);
     PCE_LAUNCH_CHECK("convert_f32_f16");
   }
-  return PCE_OK;
+  if (!stage_on(2)) return PCE_OK;
+  return launch_epilogue_pass<T>((T *)out, n_out, c_out, e, s);
 }
 
 extern "C" int pce_conv_fwd_fod(const void *in, const void *w, const void *wp, void *out, int32_t dtype, int64_t n_in,
                                 int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv, int32_t mid, const int32_t *imap,
                                 const int32_t *omap, const int32_t *kpos, const int32_t *qkpos, int64_t qsum, void *ws,
-                                int64_t ws_bytes, pce_stream_t stream) {
+                                int64_t ws_bytes, const pce_epilogue_t *epilogue, pce_stream_t stream) {
   int rc = check_common("pce_conv_fwd_fod", in, w, out, dtype, n_in, n_out, c_in, c_out, kv, mid);
   if (rc || (rc = check_qsum("pce_conv_fwd_fod", qsum))) return rc;
+  Epi e;
+  if ((rc = read_epilogue("pce_conv_fwd_fod", epilogue, out, &e))) return rc;
   if (qsum > 0 && (!imap || !omap || !kpos || !qkpos)) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_fod: null map pointer");
   hipStream_t s = (hipStream_t)stream;
   if (dtype == PCE_F16) {
     int64_t need = pce_conv_fod_workspace_bytes(n_out, c_out, dtype);
     if (!ws || ws_bytes < need) PCE_FAIL(PCE_EWORKSPACE, "pce_conv_fwd_fod: fp16 needs an fp32 accumulator of %lld bytes", (long long)need);
     if (!aligned16(ws) || !aligned16(out)) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_fod: workspace and output must be 16-byte aligned");
-    return fod_impl<half_t>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, omap, kpos, qkpos, qsum, (float *)ws, s);
+    return fod_impl<half_t>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, omap, kpos, qkpos, qsum, (float *)ws, e, s);
   }
   if (!aligned16(out)) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_fod: output must be 16-byte aligned");
-  return fod_impl<float>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, omap, kpos, qkpos, qsum, (float *)out, s);
+  return fod_impl<float>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, omap, kpos, qkpos, qsum, (float *)out, e, s);
 }
 
 template <typename T>
 static int launch_scatter(const T *buf_out, T *out, int64_t n_out, int c_out, const int *ocsr, const int *ocode,
-                          const int *qkpos, int add_existing, hipStream_t s) {
+                          const int *qkpos, int add_existing, const Epi &e, hipStream_t s) {
   constexpr int VEC = sizeof(T) == 2 ? 8 : 4;
-  bool vec_out = (c_out % VEC == 0) && aligned16(out) && aligned16(buf_out);
+  bool vec_out = (c_out % VEC == 0) && aligned16(out) && aligned16(buf_out) && epi_aligned(e);
   if (vec_out) {
     int G = pow2_at_least(c_out / VEC);
     if (G > 64) G = 64;
     hipLaunchKernelGGL((scatter_rows_kernel<T, VEC>), dim3((unsigned)pce_div_up(n_out, 256 / G)), dim3(256), 0, s,
-                       buf_out, (long long)n_out, c_out, G, ocsr, ocode, qkpos, out, add_existing);
+                       buf_out, (long long)n_out, c_out, G, ocsr, ocode, qkpos, out, add_existing, (const T *)e.bias,
+                       (const T *)e.res, e.act, e.slope);
   } else {
     int G = pow2_at_least(c_out);
     if (G > 64) G = 64;
     hipLaunchKernelGGL((scatter_rows_kernel<T, 1>), dim3((unsigned)pce_div_up(n_out, 256 / G)), dim3(256), 0, s,
-                       buf_out, (long long)n_out, c_out, G, ocsr, ocode, qkpos, out, add_existing);
+                       buf_out, (long long)n_out, c_out, G, ocsr, ocode, qkpos, out, add_existing, (const T *)e.bias,
+                       (const T *)e.res, e.act, e.slope);
   }
   PCE_LAUNCH_CHECK("scatter_rows");
   return PCE_OK;
@@ -1128,7 +1312,7 @@ static int launch_scatter(const T *buf_out, T *out, int64_t n_out, int c_out, co
 template <typename T>
 static int gms_impl(const void *in, const void *w, const void *wp, void *out, int64_t n_in, int64_t n_out, int c_in,
                     int c_out, int kv, int mid, const int *icsr, const int *icode, const int *ocsr, const int *ocode,
-                    const int *kpos, const int *qkpos, int64_t qsum, T *buffer, hipStream_t s) {
+                    const int *kpos, const int *qkpos, int64_t qsum, T *buffer, const Epi &e, hipStream_t s) {
   constexpr int VEC = sizeof(T) == 2 ? 8 : 4;
   T *buf_in = buffer;
   T *buf_out = buffer + qsum * c_in;  // backend/spconv.cu:121
@@ -1172,23 +1356,25 @@ static int gms_impl(const void *in, const void *w, const void *wp, void *out, in
   }
   if (!stage_on(2)) return PCE_OK;
   // scatter: output-stationary sum over each row's staging rows, fp32 accumulate
-  return launch_scatter<T>(buf_out, (T *)out, n_out, c_out, ocsr, ocode, qkpos, mid >= 0 ? 1 : 0, s);
+  return launch_scatter<T>(buf_out, (T *)out, n_out, c_out, ocsr, ocode, qkpos, mid >= 0 ? 1 : 0, e, s);
 }
 
 extern "C" int pce_conv_fwd_gms(const void *in, const void *w, const void *wp, void *out, int32_t dtype, int64_t n_in,
                                 int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv, int32_t mid,
                                 const int32_t *icsr, const int32_t *icode, const int32_t *ocsr, const int32_t *ocode,
                                 const int32_t *kpos, const int32_t *qkpos, int64_t qsum, void *buffer,
-                                int64_t buffer_elems, pce_stream_t stream) {
+                                int64_t buffer_elems, const pce_epilogue_t *epilogue, pce_stream_t stream) {
   int rc = check_common("pce_conv_fwd_gms", in, w, out, dtype, n_in, n_out, c_in, c_out, kv, mid);
   if (rc || (rc = check_qsum("pce_conv_fwd_gms", qsum))) return rc;
+  Epi e;
+  if ((rc = read_epilogue("pce_conv_fwd_gms", epilogue, out, &e))) return rc;
   if (!icsr || !ocsr || !kpos || !qkpos || (qsum > 0 && (!icode || !ocode))) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_gms: null map pointer");
   if (qsum > 0 && (!buffer || buffer_elems < qsum * ((int64_t)c_in + c_out)))
     PCE_FAIL(PCE_EWORKSPACE, "pce_conv_fwd_gms: buffer holds %lld elements, needs %lld", (long long)buffer_elems, (long long)(qsum * ((int64_t)c_in + c_out)));
   hipStream_t s = (hipStream_t)stream;
   if (dtype == PCE_F16)
-    return gms_impl<half_t>(in, w, wp, out, n_in, n_out, c_in, c_out, kv, mid, icsr, icode, ocsr, ocode, kpos, qkpos, qsum, (half_t *)buffer, s);
-  return gms_impl<float>(in, w, wp, out, n_in, n_out, c_in, c_out, kv, mid, icsr, icode, ocsr, ocode, kpos, qkpos, qsum, (float *)buffer, s);
+    return gms_impl<half_t>(in, w, wp, out, n_in, n_out, c_in, c_out, kv, mid, icsr, icode, ocsr, ocode, kpos, qkpos, qsum, (half_t *)buffer, e, s);
+  return gms_impl<float>(in, w, wp, out, n_in, n_out, c_in, c_out, kv, mid, icsr, icode, ocsr, ocode, kpos, qkpos, qsum, (float *)buffer, e, s);
 }
 
 // Fetch-on-demand with deferred scatter: pair tiles gather their input rows, multiply and store the
@@ -1198,7 +1384,7 @@ template <typename T>
 static int fds_impl(const void *in, const void *w, const void *wp, void *out, int64_t n_out, int c_in, int c_out, int kv,
                     int mid, const int *imap, const int *omap, const int *oslot, const int *kpos, const int *qkpos,
                     const int32_t *kpos_host, const int32_t *qkpos_host, const int *ocsr, int64_t n_pairs, int64_t qsum,
-                    T *buffer, hipStream_t s) {
+                    T *buffer, const Epi &e, hipStream_t s) {
   constexpr int VEC = sizeof(T) == 2 ? 8 : 4;
   int rc;
   if (mid >= 0 && qsum > 0 && omap && stage_on(4)) {
@@ -1215,12 +1401,14 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
     c.w_fixed = mid;
     c.n_rows = n_out;
     c.items = pce_div_up(n_out, 32);
-    if (a.host_pos && wave_gemm_ok(a, sizeof(T)) && wave_gemm_ok(c, sizeof(T)) && aligned16(buffer)) {
+    c.ocsr = ocsr;
+    set_epi(&c, e);
+    if (a.host_pos && wave_gemm_ok(a, sizeof(T)) && wave_gemm_ok(c, sizeof(T)) && aligned16(buffer) && epi_aligned(e)) {
       if (stage_on(1) && (rc = launch_wave_gemm(a, c, s))) return rc;
       if (stage_on(2)) {
         int G = pow2_at_least(c_out / VEC);
         hipLaunchKernelGGL((rowsum_pairs_kernel<T, VEC>), dim3((unsigned)pce_div_up(n_pairs, 256 / G)), dim3(256), 0, s,
-                           (const T *)buffer, (long long)n_pairs, c_out, G, omap, oslot, ocsr, (T *)out);
+                           (const T *)buffer, (long long)n_pairs, c_out, G, omap, oslot, ocsr, (T *)out, e.act, e.slope);
         PCE_LAUNCH_CHECK("rowsum_pairs");
       }
       return PCE_OK;
@@ -1256,19 +1444,22 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
     a.ocsr = ocsr;
     a.buf = buffer;
     a.b_vec = (c_out % 8 == 0) && aligned16(buffer);
+    set_epi(&a, e);
     return launch_tile<T>(a, pce_div_up(n_out, 128), s);
   }
-  bool vec = (c_out % VEC == 0) && aligned16(out) && aligned16(buffer);
+  bool vec = (c_out % VEC == 0) && aligned16(out) && aligned16(buffer) && epi_aligned(e);
   if (vec) {
     int G = pow2_at_least(c_out / VEC);
     if (G > 64) G = 64;
     hipLaunchKernelGGL((rowsum_kernel<T, VEC>), dim3((unsigned)pce_div_up(n_out, 256 / G)), dim3(256), 0, s,
-                       (const T *)buffer, (long long)n_out, c_out, G, ocsr, (T *)out);
+                       (const T *)buffer, (long long)n_out, c_out, G, ocsr, (T *)out, (const T *)e.bias, (const T *)e.res,
+                       e.act, e.slope);
   } else {
     int G = pow2_at_least(c_out);
     if (G > 64) G = 64;
     hipLaunchKernelGGL((rowsum_kernel<T, 1>), dim3((unsigned)pce_div_up(n_out, 256 / G)), dim3(256), 0, s,
-                       (const T *)buffer, (long long)n_out, c_out, G, ocsr, (T *)out);
+                       (const T *)buffer, (long long)n_out, c_out, G, ocsr, (T *)out, (const T *)e.bias, (const T *)e.res,
+                       e.act, e.slope);
   }
   PCE_LAUNCH_CHECK("rowsum");
   return PCE_OK;
@@ -1278,63 +1469,69 @@ extern "C" int pce_conv_fwd_fds(const void *in, const void *w, const void *wp, v
                                 int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv, int32_t mid, const int32_t *imap,
                                 const int32_t *omap, const int32_t *oslot, const int32_t *kpos, const int32_t *qkpos,
                                 const int32_t *kpos_host, const int32_t *qkpos_host, const int32_t *ocsr,
-                                int64_t n_pairs, int64_t qsum, void *buffer, int64_t buffer_elems, pce_stream_t stream) {
+                                int64_t n_pairs, int64_t qsum, void *buffer, int64_t buffer_elems,
+                                const pce_epilogue_t *epilogue, pce_stream_t stream) {
   int rc = check_common("pce_conv_fwd_fds", in, w, out, dtype, n_in, n_out, c_in, c_out, kv, mid);
   if (rc || (rc = check_qsum("pce_conv_fwd_fds", qsum))) return rc;
+  Epi e;
+  if ((rc = read_epilogue("pce_conv_fwd_fds", epilogue, out, &e))) return rc;
   if (!ocsr || !kpos || !qkpos || (qsum > 0 && (!imap || !oslot))) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_fds: null map pointer");
   if (n_pairs < 0 || n_pairs > qsum) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_fds: n_pairs=%lld outside [0, qsum]", (long long)n_pairs);
   if (n_pairs > 0 && (!buffer || buffer_elems < n_pairs * (int64_t)c_out))
     PCE_FAIL(PCE_EWORKSPACE, "pce_conv_fwd_fds: buffer holds %lld elements, needs %lld", (long long)buffer_elems, (long long)(n_pairs * (int64_t)c_out));
   hipStream_t s = (hipStream_t)stream;
   if (dtype == PCE_F16)
-    return fds_impl<half_t>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, omap, oslot, kpos, qkpos, kpos_host, qkpos_host, ocsr, n_pairs, qsum, (half_t *)buffer, s);
-  return fds_impl<float>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, omap, oslot, kpos, qkpos, kpos_host, qkpos_host, ocsr, n_pairs, qsum, (float *)buffer, s);
+    return fds_impl<half_t>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, omap, oslot, kpos, qkpos, kpos_host, qkpos_host, ocsr, n_pairs, qsum, (half_t *)buffer, e, s);
+  return fds_impl<float>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, omap, oslot, kpos, qkpos, kpos_host, qkpos_host, ocsr, n_pairs, qsum, (float *)buffer, e, s);
 }
 
-extern "C" int pce_conv_fwd_os(const void *in, const void *w, const void *wp, void *out, int32_t dtype, int64_t n_in,
-                               int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv, const int32_t *nbr,
-                               pce_stream_t stream) {
-  int rc = check_common("pce_conv_fwd_os", in, w, out, dtype, n_in, n_out, c_in, c_out, kv, -1);
-  if (rc) return rc;
-  if (!nbr) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_os: null neighbour table");
-  hipStream_t s = (hipStream_t)stream;
-  if (dtype == PCE_F16) {
-    TileArgs a = base_args<half_t>(in, w, wp, kv, c_in, c_out);
-    set_out<half_t>(&a, out, false);
-    a.nbr = nbr;
-    a.n_rows = n_out;
-    a.mode = MODE_OS;
-    a.epi = EPI_ROWS;
-    return launch_tile<half_t>(a, pce_div_up(n_out, 128), s);
-  }
-  TileArgs a = base_args<float>(in, w, wp, kv, c_in, c_out);
-  set_out<float>(&a, out, false);
+template <typename T>
+static int os_impl(const void *in, const void *w, const void *wp, void *out, int64_t n_out, int c_in, int c_out, int kv,
+                   const int *nbr, const Epi &e, hipStream_t s) {
+  TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
+  set_out<T>(&a, out, false);
+  set_epi(&a, e);
   a.nbr = nbr;
   a.n_rows = n_out;
   a.mode = MODE_OS;
   a.epi = EPI_ROWS;
-  return launch_tile<float>(a, pce_div_up(n_out, 128), s);
+  return launch_tile<T>(a, pce_div_up(n_out, 128), s);
 }
 
-extern "C" int pce_conv_fwd_dense(const void *in, const void *w, const void *wp, void *out, int32_t dtype, int64_t n,
-                                  int32_t c_in, int32_t c_out, pce_stream_t stream) {
-  int rc = check_common("pce_conv_fwd_dense", in, w, out, dtype, n, n, c_in, c_out, 1, -1);
+extern "C" int pce_conv_fwd_os(const void *in, const void *w, const void *wp, void *out, int32_t dtype, int64_t n_in,
+                               int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv, const int32_t *nbr,
+                               const pce_epilogue_t *epilogue, pce_stream_t stream) {
+  int rc = check_common("pce_conv_fwd_os", in, w, out, dtype, n_in, n_out, c_in, c_out, kv, -1);
   if (rc) return rc;
+  if (!nbr) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_os: null neighbour table");
+  Epi e;
+  if ((rc = read_epilogue("pce_conv_fwd_os", epilogue, out, &e))) return rc;
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == PCE_F16) {
-    TileArgs a = base_args<half_t>(in, w, wp, 1, c_in, c_out);
-    set_out<half_t>(&a, out, false);
-    a.n_rows = n;
-    a.mode = MODE_DENSE;
-    a.epi = EPI_ROWS;
-    return launch_tile<half_t>(a, pce_div_up(n, 128), s);
-  }
-  TileArgs a = base_args<float>(in, w, wp, 1, c_in, c_out);
-  set_out<float>(&a, out, false);
+  if (dtype == PCE_F16) return os_impl<half_t>(in, w, wp, out, n_out, c_in, c_out, kv, nbr, e, s);
+  return os_impl<float>(in, w, wp, out, n_out, c_in, c_out, kv, nbr, e, s);
+}
+
+template <typename T>
+static int dense_impl(const void *in, const void *w, const void *wp, void *out, int64_t n, int c_in, int c_out,
+                      const Epi &e, hipStream_t s) {
+  TileArgs a = base_args<T>(in, w, wp, 1, c_in, c_out);
+  set_out<T>(&a, out, false);
+  set_epi(&a, e);
   a.n_rows = n;
   a.mode = MODE_DENSE;
   a.epi = EPI_ROWS;
-  return launch_tile<float>(a, pce_div_up(n, 128), s);
+  return launch_tile<T>(a, pce_div_up(n, 128), s);
+}
+
+extern "C" int pce_conv_fwd_dense(const void *in, const void *w, const void *wp, void *out, int32_t dtype, int64_t n,
+                                  int32_t c_in, int32_t c_out, const pce_epilogue_t *epilogue, pce_stream_t stream) {
+  int rc = check_common("pce_conv_fwd_dense", in, w, out, dtype, n, n, c_in, c_out, 1, -1);
+  if (rc) return rc;
+  Epi e;
+  if ((rc = read_epilogue("pce_conv_fwd_dense", epilogue, out, &e))) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == PCE_F16) return dense_impl<half_t>(in, w, wp, out, n, c_in, c_out, e, s);
+  return dense_impl<float>(in, w, wp, out, n, c_in, c_out, e, s);
 }
 
 // Map density rho = pairs per output row.  With few pairs per row the fetch-on-demand family wins:

@@ -43,11 +43,15 @@ class ConvBN(nn.Module):
             self.conv.bias = nn.Parameter(b)
         self.bn = None
 
-    def forward(self, x: spTensor) -> spTensor:
-        x = self.conv(x)
-        if self.bn is not None:
-            x = self.bn(x)
-        return self.relu(x) if self.relu is not None else x
+    def forward(self, x: spTensor, residual: spTensor = None, relu_after_residual: bool = False) -> spTensor:
+        """With the norm folded away, bias, the optional residual and the ReLU run inside the conv kernels."""
+        if self.bn is None:
+            act = "relu" if (self.relu is not None or relu_after_residual) else None
+            return self.conv(x, act=act, residual=residual)
+        x = self.bn(self.conv(x))
+        if residual is not None:
+            x = x + residual
+        return ReLU(True)(x) if (self.relu is not None or relu_after_residual) else x
 
 
 class ResidualBlock(nn.Module):
@@ -59,9 +63,8 @@ class ResidualBlock(nn.Module):
         self.relu = ReLU(True)
 
     def forward(self, x: spTensor) -> spTensor:
-        y = self.b(self.a(x))
         s = x if self.shortcut is None else self.shortcut(x)
-        return self.relu(y + s)
+        return self.b(self.a(x), residual=s, relu_after_residual=True)      # relu(b(a(x)) + s)
 
 
 class SparseResUNet(nn.Module):

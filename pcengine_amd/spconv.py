@@ -9,6 +9,9 @@ Differences a user can see, all supersets of the reference:
   ('end') lets the selector decide per layer.
 * every strided layer uses the generic output-coordinate rule, also when stride == kernel size.
 * forward only.
+* ``forward(input, act=None, residual=None)``: an activation ('relu' or ('leaky_relu', slope)) and
+  a residual tensor (same coordinates) are applied inside the convolution kernels together with
+  the bias, instead of as separate passes over the output.
 """
 from __future__ import annotations
 
@@ -96,12 +99,23 @@ class conv3d(nn.Module):
             self._wcache_key = key
         return self._wcache
 
-    def forward(self, input: spTensor) -> spTensor:
+    def _bias_for(self, dtype):
+        b = self.bias
+        if b is None:
+            return None
+        key = (b.data_ptr(), b._version, dtype, b.device)
+        if getattr(self, "_bcache_key", None) != key:
+            self._bcache = b.detach().to(dtype).contiguous()
+            self._bcache_key = key
+        return self._bcache
+
+    def forward(self, input: spTensor, act=None, residual: Optional[spTensor] = None) -> spTensor:
         w, packed = self._weights_for(input.feats.dtype)
         return conv_func(input=input, in_channel=self.in_channels, out_channel=self.out_channels, kernel=w,
                          kernel_size_code=self.kernel_size_code, stride_code=self.stride_code,
-                         padding_code=self.padding_code, bias=self.bias, transposed=self.transposed,
-                         tensorcore=self.tensorcore, dataflow=self.dataflow, packed=packed)
+                         padding_code=self.padding_code, bias=self._bias_for(input.feats.dtype),
+                         transposed=self.transposed, tensorcore=self.tensorcore, dataflow=self.dataflow, packed=packed,
+                         act=act, residual=None if residual is None else residual.feats)
 
 
 def _pick_dataflow(km: backend.KernelMap, requested: str, c_in: int, c_out: int, dtype, transposed: bool) -> int:
@@ -117,28 +131,28 @@ def _pick_dataflow(km: backend.KernelMap, requested: str, c_in: int, c_out: int,
     return backend.select_dataflow(km, c_in, c_out, dtype, transposed)
 
 
-def _run(input: spTensor, km: backend.KernelMap, kernel, in_channel, out_channel, transposed, dataflow, packed) -> torch.Tensor:
+def _run(input: spTensor, km: backend.KernelMap, kernel, in_channel, out_channel, transposed, dataflow, packed,
+         bias=None, residual=None, act=None) -> torch.Tensor:
     feats = input.feats
     if kernel.dtype != feats.dtype:
         kernel, packed = kernel.to(feats.dtype), None
     df = _pick_dataflow(km, dataflow, in_channel, out_channel, feats.dtype, transposed)
-    out = backend.conv_forward(feats, kernel.detach(), km, df, transposed=transposed, buffer=input.buffer, packed=packed)
+    out = backend.conv_forward(feats, kernel.detach(), km, df, transposed=transposed, buffer=input.buffer, packed=packed,
+                               bias=bias, residual=residual, act=act)
     if layer_log is not None:
         layer_log.append((feats.shape[0], out.shape[0], km.M, in_channel, out_channel, df))
     return out
 
 
 def conv_func(input: spTensor, in_channel, out_channel, kernel, kernel_size_code, stride_code, padding_code, bias,
-              transposed, tensorcore, dataflow: str = "auto", packed=None) -> spTensor:
-    """Map cache lookup / build, dataflow dispatch, bias, metadata propagation
-    (script/spconv.py:291-464)."""
+              transposed, tensorcore, dataflow: str = "auto", packed=None, act=None, residual=None) -> spTensor:
+    """Map cache lookup / build, dataflow dispatch, bias (+ optional residual and activation, all
+    inside the kernels), metadata propagation (script/spconv.py:291-464)."""
     if kernel_size_code == _UNIT and stride_code == _UNIT:
         # 1x1 stride 1: plain matrix product, coordinates unchanged, no map (script/spconv.py:297-304)
         if kernel.dtype != input.feats.dtype:
             kernel, packed = kernel.to(input.feats.dtype), None
-        out_feats = backend.dense_forward(input.feats, kernel.detach(), packed)
-        if bias is not None:
-            out_feats += bias.to(out_feats.dtype)
+        out_feats = backend.dense_forward(input.feats, kernel.detach(), packed, bias=bias, residual=residual, act=act)
         return input._like(out_feats)
 
     if transposed:
@@ -149,9 +163,7 @@ def conv_func(input: spTensor, in_channel, out_channel, kernel, kernel_size_code
             raise KeyError("transposed conv3d found no cached map for this (kernel, stride): "
                            "the matching strided conv3d must run first on the same tensor family")
         out_coords = input.cbook[output_stride]
-        out_feats = _run(input, km, kernel, in_channel, out_channel, True, dataflow, packed)
-        if bias is not None:
-            out_feats += bias.to(out_feats.dtype)
+        out_feats = _run(input, km, kernel, in_channel, out_channel, True, dataflow, packed, bias, residual, act)
         output = spTensor(feats=out_feats, coords=out_coords, buffer=input.buffer, batchsize=input.batchsize,
                           stride=output_stride, init_tag=input.init_tag, coords_max=input.coords_max,
                           coords_min=input.coords_min)
@@ -183,9 +195,7 @@ def conv_func(input: spTensor, in_channel, out_channel, kernel, kernel_size_code
         if tag in ('D1', 'D2'):
             input.init_tag = input.init_tag[1:]
     input.cbook.setdefault(input.stride, input.coords)
-    out_feats = _run(input, km, kernel, in_channel, out_channel, False, dataflow, packed)
-    if bias is not None:
-        out_feats += bias.to(out_feats.dtype)
+    out_feats = _run(input, km, kernel, in_channel, out_channel, False, dataflow, packed, bias, residual, act)
     output = spTensor(feats=out_feats, coords=km.out_coords, buffer=input.buffer, batchsize=input.batchsize,
                       stride=output_stride, init_tag=input.init_tag, coords_max=coords_max, coords_min=coords_min)
     output.kmaps, output.cbook = input.kmaps, input.cbook

@@ -117,6 +117,78 @@ def test_narrow_fp16_layers_barrier_free_kernel(c_in, c_out):
             assert orc.rel_l2(back.double().cpu().numpy(), want_t) <= 1e-3
 
 
+def _act_np(x, act):
+    if act is None:
+        return x
+    if act == "relu":
+        return np.maximum(x, 0.0)
+    return np.where(x > 0, x, x * act[1])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("c_in,c_out", [(64, 64), (32, 20), (16, 48), (96, 160), (5, 7)])
+def test_fused_epilogue_all_dataflows(c_in, c_out, dtype):
+    """out = act(conv + bias + residual) inside the kernels, against the same formula in float64:
+    every dataflow, packed and unpacked weights, submanifold / strided / transposed / 1x1."""
+    coords = synth.random_cloud(seed=45, n=8000, extent=21, batches=2)
+    rng = np.random.default_rng(45)
+    bias = rng.standard_normal(c_out) * 0.5
+    bd = torch.as_tensor(bias, device=DEV).to(dtype)
+    fd, wd, ref_map, want = _case(coords, (3, 3, 3), (1, 1, 1), (0, 0, 0), c_in, c_out, dtype, seed=3)
+    res = rng.standard_normal((len(coords), c_out))
+    rd = torch.as_tensor(res, device=DEV).to(dtype)
+    km = gpu_map(coords, (3, 3, 3), want_csr=True, want_nbr_in=True)
+    packed = backend.pack_weights(wd)
+    combos = [(bd, rd, "relu"), (bd, None, None), (None, rd, ("leaky_relu", 0.1)), (None, None, "relu")]
+    for flow in FLOWS:
+        for pk in ((None, packed) if packed is not None else (None,)):
+            for b, r, act in combos:
+                out = backend.conv_forward(fd, wd, km, flow, packed=pk, bias=b, residual=r, act=act)
+                ref = want + (rounded(bias, dtype) if b is not None else 0) + (rounded(res, dtype) if r is not None else 0)
+                ref = _act_np(ref, act)
+                err = orc.rel_l2(out.double().cpu().numpy(), ref)
+                assert err <= TOL[dtype], (flow, pk is not None, act, err)
+                if act == "relu":
+                    assert (out >= 0).all()
+    # strided down, transposed up, 1x1
+    fd2, wd2, ref2, want2 = _case(coords, (2, 2, 2), (2, 2, 2), (0, 0, 0), c_in, c_out, dtype, seed=4)
+    km2 = gpu_map(coords, (2, 2, 2), (2, 2, 2), want_csr=True, want_nbr_in=True)
+    res2 = rng.standard_normal((km2.n_out, c_out))
+    r2 = torch.as_tensor(res2, device=DEV).to(dtype)
+    wt = synth.weights(10, 8, c_out, c_in)
+    wtd = torch.as_tensor(wt, device=DEV).to(dtype)
+    bt = rng.standard_normal(c_in) * 0.5
+    btd = torch.as_tensor(bt, device=DEV).to(dtype)
+    for flow in FLOWS:
+        down = backend.conv_forward(fd2, wd2, km2, flow, packed=backend.pack_weights(wd2), bias=bd, residual=r2, act="relu")
+        ref = np.maximum(want2 + rounded(bias, dtype) + rounded(res2, dtype), 0.0)
+        assert orc.rel_l2(down.double().cpu().numpy(), ref) <= TOL[dtype], flow
+        up = backend.conv_forward(down, wtd, km2, flow, transposed=True, packed=backend.pack_weights(wtd), bias=btd,
+                                  residual=fd, act=("leaky_relu", 0.2))
+        ref_t = orc.conv_forward(down.double().cpu().numpy(), rounded(wt, dtype), ref2, (2, 2, 2), transposed=True)
+        ref_t = _act_np(ref_t + rounded(bt, dtype) + fd.double().cpu().numpy(), ("leaky_relu", 0.2))
+        assert orc.rel_l2(up.double().cpu().numpy(), ref_t) <= TOL[dtype], flow
+    w1 = wd[0].contiguous()
+    one = backend.dense_forward(fd, w1, backend.pack_weights(w1), bias=bd, residual=rd, act="relu")
+    ref1 = np.maximum(fd.double().cpu().numpy() @ w1.double().cpu().numpy() + rounded(bias, dtype) + rounded(res, dtype), 0.0)
+    assert orc.rel_l2(one.double().cpu().numpy(), ref1) <= TOL[dtype]
+
+
+def test_fused_epilogue_argument_errors():
+    coords = synth.random_cloud(seed=46, n=500, extent=9)
+    fd, wd, _, _ = _case(coords, (3, 3, 3), (1, 1, 1), (0, 0, 0), 16, 16, torch.float16)
+    km = gpu_map(coords, (3, 3, 3))
+    with pytest.raises(ValueError):
+        backend.conv_forward(fd, wd, km, DATAFLOW_OS, bias=torch.zeros(3, device=DEV))
+    with pytest.raises(ValueError):
+        backend.conv_forward(fd, wd, km, DATAFLOW_OS, residual=torch.zeros((2, 16), dtype=torch.float16, device=DEV))
+    with pytest.raises(ValueError):
+        backend.conv_forward(fd, wd, km, DATAFLOW_OS, act="gelu")
+    out = torch.empty((len(coords), 16), dtype=torch.float16, device=DEV)
+    with pytest.raises(ValueError):      # the residual may not be the output tensor
+        backend.conv_forward(fd, wd, km, DATAFLOW_OS, out=out, residual=out)
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 def test_dense_1x1(dtype):
     f = synth.features(3, 5001, 96)

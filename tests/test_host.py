@@ -40,17 +40,23 @@ def test_pure_host_entry_points():
 
 def test_argument_validation_needs_no_gpu():
     lib = _lib.load()
-    assert lib.pce_conv_fwd_fod(None, None, None, None, 0, 1, 1, 1, 1, 1, -1, None, None, None, None, 0, None, 0, None) == _lib.PCE_EINVAL
+    assert lib.pce_conv_fwd_fod(None, None, None, None, 0, 1, 1, 1, 1, 1, -1, None, None, None, None, 0, None, 0, None, None) == _lib.PCE_EINVAL
     with pytest.raises(ValueError):
         _lib.check(_lib.PCE_EINVAL)
     one = 1
-    fod = lambda n_in, n_out, qsum, ws: lib.pce_conv_fwd_fod(one, one, None, one, 0, n_in, n_out, 4, 4, 27, 13, one, one, one, one, qsum, one, ws, None)
+    fod = lambda n_in, n_out, qsum, ws: lib.pce_conv_fwd_fod(one, one, None, one, 0, n_in, n_out, 4, 4, 27, 13, one, one, one, one, qsum, one, ws, None, None)
     assert fod(10, 10, 100, 1 << 20) == _lib.PCE_EINVAL        # qsum % 128
     assert fod(10, 12, 128, 1 << 20) == _lib.PCE_EINVAL        # a centre offset needs n_in == n_out
     assert fod(10, 10, 128, 16) == _lib.PCE_EWORKSPACE
-    assert lib.pce_conv_fwd_gms(one, one, None, one, 0, 10, 10, 4, 4, 27, 13, one, one, one, one, one, one, 128, one, 10, None) == _lib.PCE_EWORKSPACE
-    assert lib.pce_conv_fwd_fds(one, one, None, one, 0, 10, 10, 4, 4, 27, 13, one, one, one, one, one, None, None, one, 100, 128, one, 10, None) == _lib.PCE_EWORKSPACE
-    assert lib.pce_conv_fwd_os(one, one, None, one, 7, 10, 10, 4, 4, 27, one, None) == _lib.PCE_EINVAL      # dtype
+    assert lib.pce_conv_fwd_gms(one, one, None, one, 0, 10, 10, 4, 4, 27, 13, one, one, one, one, one, one, 128, one, 10, None, None) == _lib.PCE_EWORKSPACE
+    assert lib.pce_conv_fwd_fds(one, one, None, one, 0, 10, 10, 4, 4, 27, 13, one, one, one, one, one, None, None, one, 100, 128, one, 10, None, None) == _lib.PCE_EWORKSPACE
+    assert lib.pce_conv_fwd_os(one, one, None, one, 7, 10, 10, 4, 4, 27, one, None, None) == _lib.PCE_EINVAL      # dtype
+    epi = _lib.Epilogue()
+    epi.act = 9
+    assert lib.pce_conv_fwd_os(one, one, None, one, 0, 10, 10, 4, 4, 27, one, epi, None) == _lib.PCE_EINVAL     # activation
+    epi.act, epi.residual = _lib.ACT_RELU, one
+    assert lib.pce_conv_fwd_os(one, one, None, one, 0, 10, 10, 4, 4, 27, one, epi, None) == _lib.PCE_EINVAL     # residual aliases out
+    assert b"alias" in lib.pce_last_error()
     assert lib.pce_packed_weight_bytes(_lib.PCE_F16, 27, 64, 64) == 27 * 8 * 64 * 16
     assert lib.pce_packed_weight_bytes(_lib.PCE_F16, 27, 4, 20) == 27 * 1 * 32 * 16
     assert lib.pce_packed_weight_bytes(_lib.PCE_F32, 27, 64, 64) == 0
