@@ -38,7 +38,7 @@ enum {
   PCE_ECOORD = 5      /* a coordinate is outside the representable range */
 };
 
-enum { PCE_F16 = 0, PCE_F32 = 1 };
+enum { PCE_F16 = 0, PCE_F32 = 1, PCE_F64 = 2 /* points of pce_voxelize only */ };
 
 /* dataflows of the forward convolution */
 enum {
@@ -108,6 +108,27 @@ int pce_outcoords_build(const int32_t *in_coords_dev, int64_t n_in, const pce_ge
 /* Decodes it into out_coords_dev[n_out,4] (same workspace, untouched since _build). */
 int pce_outcoords_emit(const void *ws_dev, int64_t n_in, const pce_geom_t *g, int32_t n_batch, int64_t n_out,
                        int32_t *out_coords_dev, pce_stream_t stream);
+
+/* ---- voxelisation ----------------------------------------------------------------------------- *
+ * Replaces sparse_quantize + ravel_hash (script/utils.py:18-55), which the reference runs in NumPy
+ * on the host: voxel = floor(point / voxel_size) in double precision; the unique voxels in
+ * ascending (x,y,z) order (the order of the ravelled code); for every voxel the first point that
+ * falls into it (numpy.unique return_index); for every point its voxel (return_inverse).
+ * points_dev[n_points,3] are PCE_F32 or PCE_F64.  pce_voxelize synchronises the stream twice
+ * (coordinate bounds, then the voxel count) and returns the count and the bounds of the integer
+ * coordinates on the host; pce_voxelize_emit (same workspace, untouched since; the bounds handed
+ * back) writes coords_out[n_voxels,4] = (batch_index, x, y, z), index_out[n_voxels] and
+ * inverse_out[n_points]; any of the three may be NULL.  Negative coordinates are kept, as in the
+ * reference (the kernel-map entry points need them shifted to >= 0 by the caller,
+ * check_fwd.py:51). */
+int64_t pce_voxelize_workspace_bytes(int64_t n_points);
+int pce_voxelize(const void *points_dev, int32_t dtype, int64_t n_points, const double *voxel_size3_host,
+                 void *ws_dev, int64_t ws_bytes, int64_t *n_voxels_host, int32_t *coords_min3_host,
+                 int32_t *coords_max3_host, pce_stream_t stream);
+int pce_voxelize_emit(const void *ws_dev, int64_t n_points, int64_t n_voxels,
+                      const int32_t *coords_min3_host, const int32_t *coords_max3_host,
+                      int32_t batch_index, int32_t *coords_out_dev, int32_t *index_out_dev,
+                      int32_t *inverse_out_dev, pce_stream_t stream);
 
 /* ---- kernel map ------------------------------------------------------------------------------ *
  * Replaces the four _queryhash_* kernels, exclusive_scan_for_kernel_quantified, mapping_counter and

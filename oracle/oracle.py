@@ -84,6 +84,27 @@ def pack(coords: np.ndarray) -> np.ndarray:
     return ((c[:, 0] << 48) | ((c[:, 1] + off) << 32) | ((c[:, 2] + off) << 16) | (c[:, 3] + off))
 
 
+def ravel_code(q: np.ndarray) -> np.ndarray:
+    """Mixed-radix code of integer voxel coordinates after shifting by the per-axis minimum
+    (ravel_hash, script/utils.py:18-30): ((x-min_x)*E_y + (y-min_y))*E_z + (z-min_z)."""
+    x = (q - q.min(axis=0)).astype(np.uint64)
+    ext = x.max(axis=0).astype(np.uint64) + np.uint64(1)
+    h = np.zeros(len(x), np.uint64)
+    for k in range(x.shape[1] - 1):
+        h += x[:, k]
+        h *= ext[k + 1]
+    return h + x[:, -1]
+
+
+def sparse_quantize(points: np.ndarray, voxel_size):
+    """Voxelisation (sparse_quantize, script/utils.py:33-55): floor(points / voxel) in float64, the
+    unique voxels in ascending ravelled-code order, the first point of each (numpy.unique's
+    return_index) and the voxel of every point (return_inverse)."""
+    q = np.floor(np.asarray(points) / np.asarray(voxel_size, np.float64)).astype(np.int32)
+    _, index, inverse = np.unique(ravel_code(q), return_index=True, return_inverse=True)
+    return q[index], index, inverse
+
+
 def ref_linear_hash(coords: np.ndarray) -> np.ndarray:
     """The reference's hash value (backend/hash.cuh:11-15), wrapping uint64 arithmetic."""
     c = coords.astype(np.int64).astype(np.uint64)  # sign extension like (uint64_t)int

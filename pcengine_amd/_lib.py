@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libpcengine_amd.so")
 
 PCE_OK, PCE_EINVAL, PCE_ECAPACITY, PCE_EHIP, PCE_EWORKSPACE, PCE_ECOORD = range(6)
-PCE_F16, PCE_F32 = 0, 1
+PCE_F16, PCE_F32, PCE_F64 = 0, 1, 2
 DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS, DATAFLOW_FDS = 0, 1, 2, 3
 QUANTUM = 128
 CSR_CODE = 1186111
@@ -57,6 +57,11 @@ _SIGNATURES = {
     "pce_outcoords_workspace_bytes": (c_int64, [c_int64, POINTER(Geom), c_int32]),
     "pce_outcoords_build": (c_int32, [c_void_p, c_int64, POINTER(Geom), c_int32, c_void_p, c_int64, POINTER(c_int64), c_void_p]),
     "pce_outcoords_emit": (c_int32, [c_void_p, c_int64, POINTER(Geom), c_int32, c_int64, c_void_p, c_void_p]),
+    "pce_voxelize_workspace_bytes": (c_int64, [c_int64]),
+    "pce_voxelize": (c_int32, [c_void_p, c_int32, c_int64, POINTER(ctypes.c_double), c_void_p, c_int64, POINTER(c_int64),
+                               POINTER(c_int32), POINTER(c_int32), c_void_p]),
+    "pce_voxelize_emit": (c_int32, [c_void_p, c_int64, c_int64, POINTER(c_int32), POINTER(c_int32), c_int32, c_void_p, c_void_p,
+                                    c_void_p, c_void_p]),
     "pce_kmap_workspace_bytes": (c_int64, [c_int64, c_int64, c_int32, c_int32]),
     "pce_kmap_build": (c_int32, [c_void_p, c_int64, c_void_p, c_int64, POINTER(Geom), c_void_p, c_int64] + [c_void_p] * 14 + [c_void_p]),
     "pce_conv_fod_workspace_bytes": (c_int64, [c_int64, c_int32, c_int32]),

@@ -138,6 +138,46 @@ def build_out_coords(in_coords: torch.Tensor, geom: Geom, batchsize: int = 0) ->
         return out
 
 
+def voxelize(points: torch.Tensor, voxel_size, batch_index: int = 0, return_index: bool = False,
+             return_inverse: bool = False):
+    """Voxelisation on the GPU (sparse_quantize of script/utils.py:33-55): ``points`` [P,3] float32 or
+    float64 on the device -> coords int32 [V,4] = (batch_index, x, y, z) of the unique voxels in
+    ascending (x,y,z) order, optionally the first point of every voxel (int32 [V]) and the voxel of
+    every point (int32 [P]).  Also returns the integer coordinate bounds (min, max) as lists."""
+    lib = _lib.load()
+    _require_cuda(points, "points")
+    if points.dim() != 2 or points.shape[1] != 3 or points.dtype not in (torch.float32, torch.float64):
+        raise ValueError("points must be float32 or float64 [P, 3]")
+    points = points.contiguous()
+    n = points.shape[0]
+    if n == 0:
+        raise ValueError("no points to voxelise")
+    if isinstance(voxel_size, (int, float)):
+        voxel_size = (voxel_size,) * 3
+    vs = (_lib.ctypes.c_double * 3)(*[float(v) for v in voxel_size])
+    dev = points.device
+    s = _stream(dev)
+    ws_bytes = lib.pce_voxelize_workspace_bytes(n)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    n_vox = _lib.c_int64(0)
+    cmin, cmax = (_lib.c_int32 * 3)(), (_lib.c_int32 * 3)()
+    dt = _lib.PCE_F32 if points.dtype == torch.float32 else _lib.PCE_F64
+    _lib.check(lib.pce_voxelize(points.data_ptr(), dt, n, vs, ws.data_ptr(), ws_bytes, n_vox, cmin, cmax, s))
+    v = n_vox.value
+    coords = torch.empty((v, 4), dtype=torch.int32, device=dev)
+    index = torch.empty(v, dtype=torch.int32, device=dev) if return_index else None
+    inverse = torch.empty(n, dtype=torch.int32, device=dev) if return_inverse else None
+    _lib.check(lib.pce_voxelize_emit(ws.data_ptr(), n, v, cmin, cmax, int(batch_index), coords.data_ptr(), _ptr(index),
+                                     _ptr(inverse), s))
+    outs = [coords]
+    if return_index:
+        outs.append(index)
+    if return_inverse:
+        outs.append(inverse)
+    outs.append((list(cmin), list(cmax)))
+    return tuple(outs)
+
+
 def build_kernel_map(in_coords: torch.Tensor, ks, stride, pad, cmin, cmax_out, subm: bool,
                      want_csr: bool = False, want_nbr_out: bool = True, want_nbr_in: bool = False,
                      out_coords: Optional[torch.Tensor] = None, batchsize: int = 0) -> KernelMap:

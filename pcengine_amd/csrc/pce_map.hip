@@ -569,6 +569,30 @@ __global__ void __launch_bounds__(64) sort_scatter_kernel(const unsigned long lo
   }
 }
 
+// ascending sort of n 64-bit keys whose values need `bits` bits; the result is in *sorted (a or b)
+static int radix_sort_u64(unsigned long long *a, unsigned long long *b, int64_t n, int bits, int *hist, int *scan_tmp,
+                          hipStream_t s, unsigned long long **sorted) {
+  int passes = (bits + 7) / 8;
+  if (passes < 1) passes = 1;
+  int nblocks = (int)pce_div_up(n, SORT_KEYS_PER_BLOCK);
+  unsigned long long *src = a, *dst = b;
+  int rc;
+  for (int p = 0; p < passes; ++p) {
+    hipLaunchKernelGGL(sort_hist_kernel, dim3(nblocks), dim3(64), 0, s, (const unsigned long long *)src, (long long)n,
+                       8 * p, hist, nblocks);
+    PCE_LAUNCH_CHECK("sort_hist");
+    if ((rc = scan_exclusive(hist, 256ll * nblocks, scan_tmp, s))) return rc;
+    hipLaunchKernelGGL(sort_scatter_kernel, dim3(nblocks), dim3(64), 0, s, (const unsigned long long *)src, dst,
+                       (long long)n, 8 * p, (const int *)hist, nblocks);
+    PCE_LAUNCH_CHECK("sort_scatter");
+    unsigned long long *t = src;
+    src = dst;
+    dst = t;
+  }
+  *sorted = src;
+  return PCE_OK;
+}
+
 __global__ void decode_codes_kernel(const unsigned long long *__restrict__ codes, long long n, int4 *__restrict__ out) {
   long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
@@ -648,22 +672,8 @@ extern "C" int pce_outcoords_build(const int32_t *in_coords, int64_t n_in, const
   if (n == 0) return PCE_OK;
   int bits = 0;
   while (bits < 64 && (host[1] >> bits)) ++bits;
-  int passes = (bits + 7) / 8;
-  if (passes < 1) passes = 1;
-  int nblocks = (int)pce_div_up(n, SORT_KEYS_PER_BLOCK);
-  unsigned long long *src = ca, *dst = cb;
-  for (int p = 0; p < passes; ++p) {
-    hipLaunchKernelGGL(sort_hist_kernel, dim3(nblocks), dim3(64), 0, s, (const unsigned long long *)src, (long long)n,
-                       8 * p, hist, nblocks);
-    PCE_LAUNCH_CHECK("sort_hist");
-    if ((rc = scan_exclusive(hist, 256ll * nblocks, scan_tmp, s))) return rc;
-    hipLaunchKernelGGL(sort_scatter_kernel, dim3(nblocks), dim3(64), 0, s, (const unsigned long long *)src, dst,
-                       (long long)n, 8 * p, (const int *)hist, nblocks);
-    PCE_LAUNCH_CHECK("sort_scatter");
-    unsigned long long *t = src;
-    src = dst;
-    dst = t;
-  }
+  unsigned long long *src = nullptr;
+  if ((rc = radix_sort_u64(ca, cb, n, bits, hist, scan_tmp, s, &src))) return rc;
   if (src != ca) PCE_HIP(hipMemcpyAsync(ca, src, (size_t)n * 8, hipMemcpyDeviceToDevice, s));
   return PCE_OK;
 }
@@ -690,6 +700,222 @@ extern "C" int pce_outcoords_emit(const void *ws, int64_t n_in, const pce_geom_t
   hipLaunchKernelGGL(decode_codes_kernel, dim3((unsigned)pce_div_up(n_out, 256)), dim3(256), 0, (hipStream_t)stream, ca,
                      (long long)n_out, (int4 *)out_coords);
   PCE_LAUNCH_CHECK("decode_codes");
+  return PCE_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// voxelisation: floor(point / voxel), one representative per voxel, lexicographic (x,y,z) order
+// ------------------------------------------------------------------------------------------------
+// Follows sparse_quantize (script/utils.py:33-55): the unique voxels come out in ascending order of
+// the ravelled code ((x-min_x)*E_y + (y-min_y))*E_z + (z-min_z) (ravel_hash, script/utils.py:18-30),
+// index[v] is the first point (smallest point index) that falls into voxel v and inverse[p] the
+// voxel of point p (numpy.unique's return_index / return_inverse).
+//
+// Sort key = code << idx_bits | point index, so that equal codes are ordered by point index.
+#define VOX_LIMIT (1 << 30)
+
+struct VoxLayout {
+  int64_t off_q, off_keys_a, off_keys_b, off_hist, off_scan, off_flags, off_counters, total;
+};
+
+static void vox_layout(int64_t n, VoxLayout *L) {
+  int64_t nblocks = pce_div_up(n, SORT_KEYS_PER_BLOCK);
+  int64_t o = 0;
+  L->off_q = o;
+  o += pce_align_up(n * 16, 256);
+  L->off_keys_a = o;
+  o += pce_align_up(n * 8, 256);
+  L->off_keys_b = o;
+  o += pce_align_up(n * 8, 256);
+  L->off_hist = o;
+  o += pce_align_up((256 * nblocks + 1) * 4, 256);
+  L->off_scan = o;
+  int64_t scan_n = 256 * nblocks + 1 > n + 1 ? 256 * nblocks + 1 : n + 1;
+  o += pce_align_up(scan_tmp_ints(scan_n) * 4, 256);
+  L->off_flags = o;
+  o += pce_align_up((n + 1) * 4, 256);
+  L->off_counters = o;  // int[16]: min xyz, max xyz, status
+  o += 256;
+  L->total = o;
+}
+
+// counters: [0..2] min, [3..5] max, [6] a point is not finite or its voxel index exceeds +-2^30
+template <typename F>
+__global__ void __launch_bounds__(256) vox_quantize_kernel(const F *__restrict__ pts, long long n, double vx, double vy,
+                                                           double vz, int4 *__restrict__ q, int *counters) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  int lo[3] = {VOX_LIMIT, VOX_LIMIT, VOX_LIMIT}, hi[3] = {-VOX_LIMIT, -VOX_LIMIT, -VOX_LIMIT};
+  if (i < n) {
+    double c[3] = {floor((double)pts[3 * i] / vx), floor((double)pts[3 * i + 1] / vy), floor((double)pts[3 * i + 2] / vz)};
+    bool ok = true;
+#pragma unroll
+    for (int a = 0; a < 3; ++a) ok &= (c[a] > -(double)VOX_LIMIT) && (c[a] < (double)VOX_LIMIT);  // false for NaN
+    if (!ok) {
+      counters[6] = 1;
+      c[0] = c[1] = c[2] = 0.0;
+    }
+    q[i] = make_int4((int)c[0], (int)c[1], (int)c[2], 0);
+#pragma unroll
+    for (int a = 0; a < 3; ++a) lo[a] = hi[a] = (int)c[a];
+  }
+#pragma unroll
+  for (int a = 0; a < 3; ++a) {
+    for (int d = 32; d >= 1; d >>= 1) {
+      int l = __shfl_xor(lo[a], d, PCE_WAVE), h = __shfl_xor(hi[a], d, PCE_WAVE);
+      lo[a] = l < lo[a] ? l : lo[a];
+      hi[a] = h > hi[a] ? h : hi[a];
+    }
+    if (__lane_id() == 0 && lo[a] <= hi[a]) {
+      atomicMin(&counters[a], lo[a]);
+      atomicMax(&counters[3 + a], hi[a]);
+    }
+  }
+}
+
+struct VoxGrid {
+  int lo[3];
+  long long ey, ez;  // extents of y and z
+  int idx_bits;
+};
+
+__global__ void __launch_bounds__(256) vox_keys_kernel(const int4 *__restrict__ q, long long n, VoxGrid g,
+                                                       unsigned long long *__restrict__ keys) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  int4 c = q[i];
+  unsigned long long code = ((unsigned long long)(c.x - g.lo[0]) * g.ey + (c.y - g.lo[1])) * g.ez + (c.z - g.lo[2]);
+  keys[i] = (code << g.idx_bits) | (unsigned long long)i;
+}
+
+// flags[i] = 1 where sorted position i starts a new voxel; flags[n] = 0 (takes the total after the scan)
+__global__ void __launch_bounds__(256) vox_flag_kernel(const unsigned long long *__restrict__ keys, long long n,
+                                                       int idx_bits, int *__restrict__ flags) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i > n) return;
+  int f = 0;
+  if (i < n) f = (i == 0) || ((keys[i] >> idx_bits) != (keys[i - 1] >> idx_bits));
+  flags[i] = f;
+}
+
+// ex = exclusive scan of the flags: sorted position i belongs to voxel ex[i+1]-1 and opens it iff ex[i+1] != ex[i]
+__global__ void __launch_bounds__(256) vox_emit_kernel(const unsigned long long *__restrict__ keys, long long n,
+                                                       const int *__restrict__ ex, VoxGrid g, int batch,
+                                                       int4 *__restrict__ coords, int *__restrict__ index,
+                                                       int *__restrict__ inverse) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  unsigned long long key = keys[i];
+  int v = ex[i + 1] - 1;
+  int idx = (int)(key & ((1ull << g.idx_bits) - 1));
+  if (inverse) inverse[idx] = v;
+  if (ex[i + 1] != ex[i]) {
+    unsigned long long code = key >> g.idx_bits;
+    int z = (int)(code % (unsigned long long)g.ez);
+    code /= (unsigned long long)g.ez;
+    int y = (int)(code % (unsigned long long)g.ey);
+    int x = (int)(code / (unsigned long long)g.ey);
+    if (coords) coords[v] = make_int4(batch, x + g.lo[0], y + g.lo[1], z + g.lo[2]);
+    if (index) index[v] = idx;
+  }
+}
+
+extern "C" int64_t pce_voxelize_workspace_bytes(int64_t n_points) {
+  if (n_points <= 0) return -1;
+  VoxLayout L;
+  vox_layout(n_points, &L);
+  return L.total;
+}
+
+extern "C" int pce_voxelize(const void *points, int32_t dtype, int64_t n_points, const double *voxel_size, void *ws,
+                            int64_t ws_bytes, int64_t *n_voxels_host, int32_t *coords_min_host, int32_t *coords_max_host,
+                            pce_stream_t stream) {
+  hipStream_t s = (hipStream_t)stream;
+  if (!points || !voxel_size || !ws || !n_voxels_host || !coords_min_host || !coords_max_host) PCE_FAIL(PCE_EINVAL, "pce_voxelize: null pointer");
+  if (dtype != PCE_F32 && dtype != PCE_F64) PCE_FAIL(PCE_EINVAL, "pce_voxelize: points must be PCE_F32 or PCE_F64");
+  if (n_points <= 0 || n_points >= (1ll << 29)) PCE_FAIL(PCE_EINVAL, "pce_voxelize: n_points=%lld outside (0, 2^29)", (long long)n_points);
+  for (int a = 0; a < 3; ++a)
+    if (!(voxel_size[a] > 0.0)) PCE_FAIL(PCE_EINVAL, "pce_voxelize: voxel sizes must be positive");
+  VoxLayout L;
+  vox_layout(n_points, &L);
+  if (ws_bytes < L.total) PCE_FAIL(PCE_EWORKSPACE, "pce_voxelize: workspace %lld < %lld", (long long)ws_bytes, (long long)L.total);
+  char *w = (char *)ws;
+  int4 *q = (int4 *)(w + L.off_q);
+  unsigned long long *ka = (unsigned long long *)(w + L.off_keys_a), *kb = (unsigned long long *)(w + L.off_keys_b);
+  int *counters = (int *)(w + L.off_counters);
+  int *flags = (int *)(w + L.off_flags);
+  int rc;
+  int init[16] = {VOX_LIMIT, VOX_LIMIT, VOX_LIMIT, -VOX_LIMIT, -VOX_LIMIT, -VOX_LIMIT, 0};
+  PCE_HIP(hipMemcpyAsync(counters, init, sizeof(init), hipMemcpyHostToDevice, s));
+  unsigned blocks = (unsigned)pce_div_up(n_points, 256);
+  if (dtype == PCE_F32)
+    hipLaunchKernelGGL(vox_quantize_kernel<float>, dim3(blocks), dim3(256), 0, s, (const float *)points,
+                       (long long)n_points, voxel_size[0], voxel_size[1], voxel_size[2], q, counters);
+  else
+    hipLaunchKernelGGL(vox_quantize_kernel<double>, dim3(blocks), dim3(256), 0, s, (const double *)points,
+                       (long long)n_points, voxel_size[0], voxel_size[1], voxel_size[2], q, counters);
+  PCE_LAUNCH_CHECK("vox_quantize");
+  int host[8];
+  PCE_HIP(hipMemcpyAsync(host, counters, sizeof(host), hipMemcpyDeviceToHost, s));
+  PCE_HIP(hipStreamSynchronize(s));
+  if (host[6]) PCE_FAIL(PCE_ECOORD, "pce_voxelize: a point is not finite or its voxel index exceeds +-2^30");
+  VoxGrid g;
+  int idx_bits = 1;
+  while ((1ll << idx_bits) < n_points) ++idx_bits;
+  g.idx_bits = idx_bits;
+  long long ext[3];
+  for (int a = 0; a < 3; ++a) {
+    g.lo[a] = host[a];
+    ext[a] = (long long)host[3 + a] - host[a] + 1;
+    coords_min_host[a] = host[a];
+    coords_max_host[a] = host[3 + a];
+  }
+  g.ey = ext[1];
+  g.ez = ext[2];
+  // ext <= 2^31 each: the product is formed in floating point first to stay clear of overflow
+  double cells = (double)ext[0] * (double)ext[1] * (double)ext[2];
+  int code_bits = 1;
+  while (code_bits < 64 && cells > (double)(1ull << code_bits)) ++code_bits;
+  if (code_bits + idx_bits > 64)
+    PCE_FAIL(PCE_ECAPACITY, "pce_voxelize: %lld x %lld x %lld cells with %lld points do not fit a 64-bit sort key",
+             ext[0], ext[1], ext[2], (long long)n_points);
+  hipLaunchKernelGGL(vox_keys_kernel, dim3(blocks), dim3(256), 0, s, (const int4 *)q, (long long)n_points, g, ka);
+  PCE_LAUNCH_CHECK("vox_keys");
+  unsigned long long *sorted = nullptr;
+  if ((rc = radix_sort_u64(ka, kb, n_points, code_bits + idx_bits, (int *)(w + L.off_hist), (int *)(w + L.off_scan), s,
+                           &sorted)))
+    return rc;
+  hipLaunchKernelGGL(vox_flag_kernel, dim3((unsigned)pce_div_up(n_points + 1, 256)), dim3(256), 0, s,
+                     (const unsigned long long *)sorted, (long long)n_points, idx_bits, flags);
+  PCE_LAUNCH_CHECK("vox_flag");
+  if ((rc = scan_exclusive(flags, n_points + 1, (int *)(w + L.off_scan), s))) return rc;
+  if (sorted != ka) PCE_HIP(hipMemcpyAsync(ka, sorted, (size_t)n_points * 8, hipMemcpyDeviceToDevice, s));
+  int total = 0;
+  PCE_HIP(hipMemcpyAsync(&total, flags + n_points, sizeof(int), hipMemcpyDeviceToHost, s));
+  PCE_HIP(hipStreamSynchronize(s));
+  *n_voxels_host = total;
+  return PCE_OK;
+}
+
+extern "C" int pce_voxelize_emit(const void *ws, int64_t n_points, int64_t n_voxels, const int32_t *coords_min_host,
+                                 const int32_t *coords_max_host, int32_t batch_index,
+                                 int32_t *coords_out, int32_t *index_out, int32_t *inverse_out, pce_stream_t stream) {
+  if (!ws || !coords_min_host || !coords_max_host) PCE_FAIL(PCE_EINVAL, "pce_voxelize_emit: null pointer");
+  if (n_points <= 0 || n_points >= (1ll << 29) || n_voxels <= 0 || n_voxels > n_points)
+    PCE_FAIL(PCE_EINVAL, "pce_voxelize_emit: n_points=%lld n_voxels=%lld", (long long)n_points, (long long)n_voxels);
+  VoxLayout L;
+  vox_layout(n_points, &L);
+  VoxGrid g;
+  g.idx_bits = 1;
+  while ((1ll << g.idx_bits) < n_points) ++g.idx_bits;
+  for (int a = 0; a < 3; ++a) g.lo[a] = coords_min_host[a];
+  g.ey = (long long)coords_max_host[1] - coords_min_host[1] + 1;
+  g.ez = (long long)coords_max_host[2] - coords_min_host[2] + 1;
+  const char *w = (const char *)ws;
+  const unsigned long long *sorted = (const unsigned long long *)(w + L.off_keys_a);
+  hipLaunchKernelGGL(vox_emit_kernel, dim3((unsigned)pce_div_up(n_points, 256)), dim3(256), 0, (hipStream_t)stream, sorted,
+                     (long long)n_points, (const int *)(w + L.off_flags), g, (int)batch_index, (int4 *)coords_out, index_out,
+                     inverse_out);
+  PCE_LAUNCH_CHECK("vox_emit");
   return PCE_OK;
 }
 

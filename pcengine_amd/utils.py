@@ -56,10 +56,18 @@ def ravel_hash(x: np.ndarray) -> np.ndarray:
 
 def sparse_quantize(coords, voxel_size: Union[float, Tuple[float, ...]] = 1, *, return_index: bool = False,
                     return_inverse: bool = False):
-    """floor(coords / voxel) and one representative per voxel (script/utils.py:33-55)."""
+    """floor(coords / voxel) and one representative per voxel (script/utils.py:33-55).
+
+    A NumPy array is handled on the host exactly as in the reference; a device tensor [P,3] goes
+    through the GPU voxelisation and device tensors come back (coords int32 [V,3], indices int64)."""
     if isinstance(voxel_size, (float, int)):
         voxel_size = tuple(repeat(voxel_size, 3))
     assert isinstance(voxel_size, tuple) and len(voxel_size) == 3
+    if isinstance(coords, torch.Tensor) and coords.is_cuda:
+        from . import backend
+        res = backend.voxelize(coords, voxel_size, 0, return_index=return_index, return_inverse=return_inverse)
+        outs = [res[0][:, 1:].contiguous()] + [t.long() for t in res[1:-1]]
+        return outs[0] if len(outs) == 1 else outs
     q = np.floor(coords / np.array(voxel_size)).astype(np.int32)
     _, idx, inv = np.unique(ravel_hash(q), return_index=True, return_inverse=True)
     outs = [q[idx]]

@@ -173,3 +173,43 @@ def test_error_paths():
     lib = _lib.load()
     rc = lib.pce_kmap_build(None, 1, None, 1, None, None, 0, *([None] * 14), None)
     assert rc == _lib.PCE_EINVAL and b"null" in lib.pce_last_error()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_voxelize_matches_oracle(dtype):
+    rng = np.random.default_rng(51)
+    pts = rng.uniform(-20.0, 35.0, size=(200000, 3)).astype(np.float32 if dtype == torch.float32 else np.float64)
+    pts[0:199995:5] = pts[2:199997:5]              # exact duplicates
+    pd = torch.as_tensor(pts, device=DEV)
+    for voxel in [(0.1, 0.1, 0.1), (0.5, 0.25, 2.0)]:
+        coords, index, inverse, (cmin, cmax) = backend.voxelize(pd, voxel, batch_index=3, return_index=True, return_inverse=True)
+        oc, oi, ov = orc.sparse_quantize(pts, voxel)
+        c = coords.cpu().numpy()
+        assert (c[:, 0] == 3).all() and np.array_equal(c[:, 1:], oc)
+        assert np.array_equal(index.cpu().numpy(), oi) and np.array_equal(inverse.cpu().numpy(), ov)
+        assert cmin == oc.min(0).tolist() and cmax == oc.max(0).tolist()
+    # the reference's interface on a device tensor
+    from pcengine_amd import utils
+    c3, idx = utils.sparse_quantize(pd, 0.2, return_index=True)
+    oc, oi, _ = orc.sparse_quantize(pts, (0.2, 0.2, 0.2))
+    assert c3.dtype == torch.int32 and np.array_equal(c3.cpu().numpy(), oc) and np.array_equal(idx.cpu().numpy(), oi)
+
+
+def test_voxelize_edge_cases():
+    one = torch.tensor([[0.3, -0.2, 7.9]], device=DEV)
+    coords, index, inverse, _ = backend.voxelize(one, 1.0, return_index=True, return_inverse=True)
+    assert coords.cpu().tolist() == [[0, 0, -1, 7]] and index.cpu().tolist() == [0] and inverse.cpu().tolist() == [0]
+    same = torch.zeros((1000, 3), device=DEV)
+    coords, index, _ = backend.voxelize(same, 0.5, return_index=True)
+    assert coords.cpu().tolist() == [[0, 0, 0, 0]] and index.cpu().tolist() == [0]
+    with pytest.raises(_lib.PCEError):
+        backend.voxelize(torch.tensor([[0.0, float("nan"), 0.0]], device=DEV), 1.0)
+    with pytest.raises(_lib.PCEError):
+        backend.voxelize(torch.tensor([[1e12, 0.0, 0.0]], device=DEV), 1.0)
+    with pytest.raises(ValueError):
+        backend.voxelize(torch.zeros((4, 3), device=DEV), -1.0)
+    with pytest.raises(OverflowError):       # 1e9 cells along every axis exceed the 64-bit sort key
+        backend.voxelize(torch.tensor([[0.0, 0.0, 0.0], [1.0e9, 1.0e9, 1.0e9]], dtype=torch.float64, device=DEV), 1.0)
+    far = torch.tensor([[0.0, 0.0, 0.0], [1.0e9, 1000.0, 1000.0], [0.0, 0.0, 0.0]], dtype=torch.float64, device=DEV)
+    coords, inverse, _ = backend.voxelize(far, 1.0, return_inverse=True)     # a huge but representable box
+    assert coords.cpu().tolist() == [[0, 0, 0, 0], [0, 1000000000, 1000, 1000]] and inverse.cpu().tolist() == [0, 1, 0]

@@ -260,3 +260,33 @@ def test_dense_neighbour_table_symmetry():
     assert np.array_equal((nbr >= 0).sum(1), (nbr[::-1] >= 0).sum(1))
     kp, o = np.nonzero(nbr >= 0)
     assert np.array_equal(nbr[26 - kp, nbr[kp, o]], o)
+
+
+def test_sparse_quantize_pinned_by_lexicographic_unique_and_brute_force():
+    """The ravelled-code order is the lexicographic (x,y,z) order; first-occurrence and inverse are
+    checked against a dictionary walk over the points."""
+    rng = np.random.default_rng(3)
+    pts = rng.uniform(-3.0, 5.0, size=(4000, 3))
+    pts[0:3997:7] = pts[3:4000:7]                         # exact duplicates of other points
+    for voxel in [(0.5, 0.5, 0.5), (0.3, 1.1, 0.25)]:
+        coords, index, inverse = orc.sparse_quantize(pts, voxel)
+        q = np.floor(pts / np.array(voxel)).astype(np.int64)
+        want = np.unique(q, axis=0)                       # rows in lexicographic order
+        assert np.array_equal(coords, want)
+        first = {}
+        for i, row in enumerate(map(tuple, q)):
+            first.setdefault(row, i)
+        assert [first[tuple(r)] for r in want] == index.tolist()
+        assert np.array_equal(coords[inverse], q)
+    # hand example: voxel 1, points in cells (0,0,0), (-1,0,2), (0,0,0), (-1,0,1)
+    c, idx, inv = orc.sparse_quantize(np.array([[0.5, 0.2, 0.9], [-0.1, 0.0, 2.0], [0.0, 0.99, 0.0], [-1.0, 0.5, 1.5]]), (1, 1, 1))
+    assert c.tolist() == [[-1, 0, 1], [-1, 0, 2], [0, 0, 0]] and idx.tolist() == [3, 1, 0] and inv.tolist() == [2, 1, 2, 0]
+
+
+def test_front_end_sparse_quantize_on_numpy_matches_oracle():
+    from pcengine_amd import utils
+    rng = np.random.default_rng(4)
+    pts = rng.uniform(0, 10, size=(3000, 3))
+    c, idx, inv = utils.sparse_quantize(pts, 0.4, return_index=True, return_inverse=True)
+    oc, oi, ov = orc.sparse_quantize(pts, (0.4, 0.4, 0.4))
+    assert np.array_equal(c, oc) and np.array_equal(idx, oi) and np.array_equal(inv, ov)
