@@ -15,7 +15,7 @@ from torch import nn
 
 from .activation import ReLU
 from .batchnorm import BatchNorm
-from .spconv import conv3d
+from .spconv import conv3d, prebuild_maps
 from .sptensor import spTensor
 from .utils import cat
 
@@ -101,7 +101,15 @@ class SparseResUNet(nn.Module):
                 m.fuse()
         return self
 
+    def map_plan(self):
+        """(kernel_size, stride, padding) of the layers that need a kernel map, in execution order."""
+        plan = [(3, 1, 0)]
+        for _ in self.down:
+            plan += [(2, 2, 0), (3, 1, 0)]
+        return plan
+
     def forward(self, x: spTensor) -> spTensor:
+        prebuild_maps(x, self.map_plan())      # no host wait is left between the layers below
         x = self.stem(x)
         feats = [x]
         for down, enc in zip(self.down, self.enc):

@@ -144,6 +144,59 @@ def _run(input: spTensor, km: backend.KernelMap, kernel, in_channel, out_channel
     return out
 
 
+def ensure_map(input: spTensor, kernel_size_code: int, stride_code: int, padding_code: int):
+    """Kernel map of a (non-transposed) layer on this tensor: looked up in the shared cache or built
+    and stored there (script/spconv.py:331-437).  Returns (map, output tensor stride, output
+    coords_min, output coords_max).  Maps depend on coordinates only, so a network can call this for
+    all its layers before the first convolution: the host then never waits for the device between
+    layers (see ``prebuild_maps``)."""
+    output_stride = output_stride_compute(stride_code, input.stride, 0)
+    key = (kernel_size_code, input.stride, stride_code)
+    km = input.kmaps.get(key)
+    subm = stride_code == _UNIT
+    coords_max = list(input.coords_max[:3])
+    coords_min = list(input.coords_min[:3])
+    ks = conv_info_decoder(kernel_size_code)
+    stride = conv_info_decoder(stride_code)
+    pad = conv_info_decoder(padding_code)
+    if not subm:
+        coords_max = backend.strided_coords_max(input.coords_max, ks, stride, pad)   # script/spconv.py:358-360
+    if km is None:
+        tag = input.init_tag[0] if input.init_tag else 'end'
+        if tag not in ('D1', 'D2', 'end', 'auto'):
+            raise NotImplementedError(f"unknown init_tag entry {tag!r}")
+        auto = tag in ('end', 'auto')
+        km = backend.build_kernel_map(input.coords, ks, stride, pad, coords_min, coords_max, subm,
+                                      want_csr=(tag == 'D1' or auto), want_nbr_out=auto, want_nbr_in=auto and not subm,
+                                      batchsize=input.batchsize)
+        km.tag = tag if tag in ('D1', 'D2') else 'auto'
+        input.kmaps[key] = km
+        input.cbook[output_stride] = km.out_coords
+        if tag in ('D1', 'D2'):
+            input.init_tag = input.init_tag[1:]
+    input.cbook.setdefault(input.stride, input.coords)
+    return km, output_stride, coords_min, coords_max
+
+
+def prebuild_maps(input: spTensor, layers) -> None:
+    """Build, ahead of any convolution, the maps a network will ask for.  ``layers`` lists
+    (kernel_size, stride, padding) in network order (ints or triples; transposed layers and 1x1
+    layers need no entry); a strided entry moves on to its output coordinates, as the network does.
+    Every map build reads two counters back from the device: done here, with no convolution queued,
+    those waits are short, and the layers that follow find every map in the cache."""
+    x = input
+    for ks, stride, pad in layers:
+        ksc, sc, pc = (conv_info_encoder(_triple(v, "layer")) for v in (ks, stride, pad))
+        if ksc == _UNIT and sc == _UNIT:
+            continue
+        km, out_stride, cmin, cmax = ensure_map(x, ksc, sc, pc)
+        if sc != _UNIT:
+            nxt = spTensor(feats=x.feats, coords=km.out_coords, buffer=x.buffer, batchsize=x.batchsize, stride=out_stride,
+                           init_tag=x.init_tag, coords_max=cmax, coords_min=cmin)
+            nxt.kmaps, nxt.cbook = x.kmaps, x.cbook
+            x = nxt
+
+
 def conv_func(input: spTensor, in_channel, out_channel, kernel, kernel_size_code, stride_code, padding_code, bias,
               transposed, tensorcore, dataflow: str = "auto", packed=None, act=None, residual=None) -> spTensor:
     """Map cache lookup / build, dataflow dispatch, bias (+ optional residual and activation, all
@@ -170,31 +223,7 @@ def conv_func(input: spTensor, in_channel, out_channel, kernel, kernel_size_code
         output.kmaps, output.cbook = input.kmaps, input.cbook
         return output
 
-    output_stride = output_stride_compute(stride_code, input.stride, 0)
-    key = (kernel_size_code, input.stride, stride_code)
-    km = input.kmaps.get(key)
-    subm = stride_code == _UNIT
-    coords_max = list(input.coords_max[:3])
-    coords_min = list(input.coords_min[:3])
-    ks = conv_info_decoder(kernel_size_code)
-    stride = conv_info_decoder(stride_code)
-    pad = conv_info_decoder(padding_code)
-    if not subm:
-        coords_max = backend.strided_coords_max(input.coords_max, ks, stride, pad)   # script/spconv.py:358-360
-    if km is None:
-        tag = input.init_tag[0] if input.init_tag else 'end'
-        if tag not in ('D1', 'D2', 'end', 'auto'):
-            raise NotImplementedError(f"unknown init_tag entry {tag!r}")
-        auto = tag in ('end', 'auto')
-        km = backend.build_kernel_map(input.coords, ks, stride, pad, coords_min, coords_max, subm,
-                                      want_csr=(tag == 'D1' or auto), want_nbr_out=auto, want_nbr_in=auto and not subm,
-                                      batchsize=input.batchsize)
-        km.tag = tag if tag in ('D1', 'D2') else 'auto'
-        input.kmaps[key] = km
-        input.cbook[output_stride] = km.out_coords
-        if tag in ('D1', 'D2'):
-            input.init_tag = input.init_tag[1:]
-    input.cbook.setdefault(input.stride, input.coords)
+    km, output_stride, coords_min, coords_max = ensure_map(input, kernel_size_code, stride_code, padding_code)
     out_feats = _run(input, km, kernel, in_channel, out_channel, False, dataflow, packed, bias, residual, act)
     output = spTensor(feats=out_feats, coords=km.out_coords, buffer=input.buffer, batchsize=input.batchsize,
                       stride=output_stride, init_tag=input.init_tag, coords_max=coords_max, coords_min=coords_min)

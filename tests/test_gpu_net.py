@@ -115,3 +115,29 @@ def test_unet_fp16_runs_close_to_fp32():
     assert out.dtype == torch.float16
     # forty fp16 layers deep: storage rounding accumulates, the per-layer bar (1e-3) does not apply end to end
     assert orc.rel_l2(out.double().cpu().numpy(), ref.double().cpu().numpy()) <= 2e-2
+
+
+def test_prebuilt_maps_cover_the_whole_network(monkeypatch):
+    """prebuild_maps builds the nine maps of the U-Net (five submanifold, four strided) before any
+    convolution; the layers then find all of them cached, and the result does not depend on it."""
+    from pcengine_amd import backend, spconv
+    coords = synth.random_cloud(seed=63, n=6000, extent=32)
+    f = synth.features(10, len(coords), 4)
+    model = _model(2).fuse_bn()
+    mk = lambda: pe.spTensor(torch.as_tensor(f, device=DEV).float(), torch.as_tensor(coords, device=DEV), None,
+                             [0, 0, 0], coords[:, 1:].max(0).tolist())
+    x = mk()
+    spconv.prebuild_maps(x, model.map_plan())
+    assert len(x.kmaps) == 9 and len(x.cbook) == 5
+    calls = []
+    real = backend.build_kernel_map
+    monkeypatch.setattr(backend, "build_kernel_map", lambda *a, **k: calls.append(1) or real(*a, **k))
+    with torch.no_grad():
+        y = model(x)
+    assert calls == []
+    # without the prebuild (maps built lazily, layer by layer) the output is bit-identical
+    monkeypatch.setattr(spconv, "prebuild_maps", lambda *a, **k: None)
+    monkeypatch.setattr(nets, "prebuild_maps", lambda *a, **k: None)
+    with torch.no_grad():
+        z = model(mk())
+    assert len(calls) == 9 and torch.equal(y.feats, z.feats)
