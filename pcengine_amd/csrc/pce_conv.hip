@@ -832,7 +832,161 @@ static bool wave_gemm_ok(const TileArgs &a, int elem_size) {
   return elem_size == 2 && a.Wp && a.a_vec && a.o_vec && a.c_in % 16 == 0 && a.c_in <= 64 && a.c_out <= 64;
 }
 
+static unsigned g_stage_mask = 0xFFFFFFFFu;
+static inline bool stage_on(int bit) { return (g_stage_mask >> bit) & 1u; }
+
+// ---- pipelined tile GEMM for wide fp16 layers ---------------------------------------------------
+// The single-offset modes (pair tiles, centre / dense GEMM) at wide channels: 128 rows x 128 columns
+// per workgroup, 32 rows per wavefront.  K advances in chunks of 32; the chunk's weight tile (8 KB) is
+// copied global -> LDS without passing through registers, two chunks ahead, into a ring of three
+// stages; the feature fragments of the next chunk are requested before the MFMAs of the current one.
+// One workgroup barrier per chunk.  (An output-stationary variant of this kernel, with 256-row tiles
+// as well, was measured and lost to the single-stage tile kernel except where tile counts happened to
+// fill the machine better; it is not kept.)
+#define PIPE_KC 32
+#define PIPE_ST 3
+#define PIPE_NB 4
+
+__device__ __forceinline__ void pipe_wait_barrier(bool more_in_flight) {
+  // loads complete in issue order: leaving the two youngest (the next-but-one weight chunk of this
+  // wavefront) in flight still guarantees that the chunk about to be used has landed
+  if (more_in_flight)
+    asm volatile("s_waitcnt vmcnt(2)\n\ts_barrier" ::: "memory");
+  else
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// this wavefront's quarter of the weight chunk (k0 .. k0+31, columns n0 .. n0+127) -> LDS stage
+__device__ __forceinline__ void pipe_issue_weights(const half_t *Wk, int k0, int n0, int n_pad, half8 *stage, int wave,
+                                                   int lane) {
+  // stage layout [k8 = 0..3][n = 0..127] of 16-byte fragments; one instruction moves 64 of them
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    int part = wave * 2 + i;          // 0..7: k8 = part / 2, column half = part % 2
+    int k8 = part >> 1, nh = part & 1;
+    int n = n0 + nh * 64 + lane;
+    n = n < n_pad ? n : n_pad - 1;    // columns past the padded width are never stored: any valid address will do
+    const half_t *src = Wk + ((long long)(k0 / 8 + k8) * n_pad + n) * 8;
+    half8 *dst = stage + k8 * 128 + nh * 64;  // wave-uniform; the hardware adds lane * 16 bytes
+    // issued by every wavefront in every round: pipe_wait_barrier counts on it
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                     (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
+  }
+}
+
+// always issued (row 0 stands in for a missing row; the caller zeroes it when the fragment is taken into
+// use): the wait before the barrier relies on at least two loads younger than the weight chunk it
+// waits for
+__device__ __forceinline__ void pipe_load_rows(half8 (&af)[2], const half_t *A, int arow, int c_in, int k0, int g) {
+  int r = arow >= 0 ? arow : 0;
+#pragma unroll
+  for (int s2 = 0; s2 < 2; ++s2) af[s2] = *reinterpret_cast<const half8 *>(A + (long long)r * c_in + k0 + s2 * 16 + g * 8);
+}
+
+template <int PMODE>
+__global__ void __launch_bounds__(256, 4) pipe_gemm_kernel(TileArgs a) {
+  constexpr int NB = PIPE_NB, NT = 128, KC = PIPE_KC;
+  constexpr int STAGE = (KC / 8) * NT;                       // fragments per stage
+  constexpr int RING = PIPE_ST * STAGE;
+  constexpr int EPI = 4 * WaveLds<NB>::PIECES;               // epilogue staging reuses the ring
+  __shared__ __attribute__((aligned(16))) half8 lds[RING > EPI ? RING : EPI];
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int l32 = lane & 31, g = lane >> 5;
+  const long long item = blockIdx.x;
+  if (item >= a.items) return;
+  const long long tile = item / a.slabs;
+  const int n0 = (int)(item % a.slabs) * NT;
+  const half_t *A = (const half_t *)a.A;
+  const int kch = a.c_in / KC;
+
+  int orow = -1, arow = -1, widx;
+  if (PMODE == MODE_DENSE) {
+    long long row = tile * 128 + wave * 32 + l32;
+    orow = arow = row < a.n_rows ? (int)row : -1;
+    widx = a.w_fixed;
+  } else {  // pair tile: one 128-pair quantum of one offset
+    long long q0 = tile * 128;
+    widx = 0;
+    for (int i = 0; i < a.kv; ++i) widx += ((long long)a.qkpos_h[i + 1] <= q0) ? 1 : 0;
+    if (widx >= a.kv) return;
+    long long p = q0 - a.qkpos_h[widx] + a.kpos_h[widx] + wave * 32 + l32;
+    if (p < (long long)a.kpos_h[widx + 1]) {
+      orow = a.oslot[p];
+      arow = a.imap[p];
+    }
+  }
+  const half_t *Wk = (const half_t *)a.Wp + (long long)widx * a.k8_total * a.n_pad * 8;
+
+  f32x16 acc[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[nb][j] = 0.f;
+
+  // prologue: weight chunks 0 and 1, feature chunk 0
+  pipe_issue_weights(Wk, 0, n0, a.n_pad, lds, wave, lane);
+  if (kch > 1) pipe_issue_weights(Wk, KC, n0, a.n_pad, lds + STAGE, wave, lane);
+  half8 af[2], raw[2];
+  pipe_load_rows(raw, A, arow, a.c_in, 0, g);
+  const bool wave_has = __ballot(arow >= 0) != 0ull;
+  const half8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  int st = 0, st2 = 2 % PIPE_ST;
+  for (int t = 0; t < kch; ++t) {
+    pipe_wait_barrier(t + 1 < kch);
+    // the fragments requested one round ago become the operands of this round
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) af[s2] = arow >= 0 ? raw[s2] : zero;
+    // features of chunk t+1 first, so that the weight loads below are the youngest in flight
+    if (t + 1 < kch) pipe_load_rows(raw, A, arow, a.c_in, (t + 1) * KC, g);
+    // weight chunk t+2 -> the stage that chunk t-1 has just released
+    if (t + 2 < kch) {
+      pipe_issue_weights(Wk, (t + 2) * KC, n0, a.n_pad, lds + st2 * STAGE, wave, lane);
+      st2 = st2 + 1 == PIPE_ST ? 0 : st2 + 1;
+    }
+    if (wave_has) {
+      const half8 *stp = lds + st * STAGE;
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          half8 b = stp[(2 * s2 + g) * NT + nb * 32 + l32];
+          acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b, af[s2], acc[nb], 0, 0, 0);
+        }
+    }
+    st = st + 1 == PIPE_ST ? 0 : st + 1;
+  }
+  __syncthreads();  // the ring becomes the epilogue staging area
+  float V[NB][2][8];
+  gather_row_pieces<NB>(acc, V, g);
+  if (a.bias || a.res || a.act) {
+    bool with_act = a.act != PCE_ACT_NONE;
+    if (with_act && a.act_alone_only) with_act = orow >= 0 && a.ocsr[orow] == a.ocsr[orow + 1];
+    epilogue_row_pieces<half_t, NB, true>(V, a, orow, n0, g, with_act);
+  }
+  store_rows_via_lds<half_t, NB>(V, lds + wave * WaveLds<NB>::PIECES, (half_t *)a.out, orow, a, n0, lane, l32, g);
+}
+
 static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+// shapes the pipelined kernel takes
+static bool pipe_gemm_ok(const TileArgs &a, int elem_size) {
+  return elem_size == 2 && a.Wp && a.a_vec && a.o_vec && a.c_in % PIPE_KC == 0 && a.c_in >= 64 && a.c_out >= 96 &&
+         aligned16(a.bias) && aligned16(a.res) && a.epi == EPI_ROWS &&
+         (a.mode == MODE_DENSE || (a.mode == MODE_FOD_BUF && a.host_pos));
+}
+
+static int launch_pipe_gemm(TileArgs a, long long tiles, hipStream_t s) {
+  a.slabs = (a.c_out + 127) / 128;
+  a.items = tiles * a.slabs;
+  if (a.items >= (1ll << 31) - 8) PCE_FAIL(PCE_ECAPACITY, "tile count %lld exceeds the grid limit", tiles);
+  if (a.mode == MODE_DENSE)
+    hipLaunchKernelGGL((pipe_gemm_kernel<MODE_DENSE>), dim3((unsigned)a.items), dim3(256), 0, s, a);
+  else
+    hipLaunchKernelGGL((pipe_gemm_kernel<MODE_FOD_BUF>), dim3((unsigned)a.items), dim3(256), 0, s, a);
+  PCE_LAUNCH_CHECK("pipe_gemm");
+  return PCE_OK;
+}
 
 static unsigned xcd_grid(TileArgs *a, long long tiles, int slabs) {
   a->slabs = slabs;
@@ -862,6 +1016,8 @@ template <typename T>
 static int launch_tile(const TileArgs &a, long long tiles, hipStream_t s) {
   if (tiles <= 0) return PCE_OK;
   if (tiles * ((a.c_out + 127) / 128) >= (1ll << 31) - 8) PCE_FAIL(PCE_ECAPACITY, "tile count %lld exceeds the grid limit", tiles);
+  if (stage_on(5) && pipe_gemm_ok(a, sizeof(T)))
+    return launch_pipe_gemm(a, tiles, s);
   bool fast = a.a_vec && a.o_vec && (sizeof(T) == 2 ? a.Wp != nullptr : a.w_vec != 0) &&
               (a.epi != EPI_ROWS_CSR || a.b_vec) && aligned16(a.bias) && aligned16(a.res);
   if (!fast)
@@ -1098,9 +1254,7 @@ __global__ void zero_f32_kernel(float *p, long long n) {
   }
 }
 
-static unsigned g_stage_mask = 0xFFFFFFFFu;
 extern "C" void pce_set_stage_mask(uint32_t mask) { g_stage_mask = mask; }
-static inline bool stage_on(int bit) { return (g_stage_mask >> bit) & 1u; }
 
 static int pow2_at_least(int v) {
   int p = 1;
@@ -1570,7 +1724,8 @@ extern "C" int pce_conv_fwd_dense(const void *in, const void *w, const void *wp,
 // output-stationary kernel touches no intermediate memory but multiplies every offset of every
 // 128-row tile, populated or not.  Measured on a MinkUNet-style network (100 k voxels, fp16): deferred
 // scatter wins up to rho = 3 at every width and at rho = 9 for 256 channels; output-stationary wins at
-// rho = 9 up to 128 channels, at rho = 20 everywhere, and (by a little) on 2x2x2 stride-2 layers of
+// rho = 6 to 9 up to 128 channels, at rho = 20 everywhere (at rho = 13 and 256 channels deferred scatter
+// still leads), and (by a little) on 2x2x2 stride-2 layers of
 // at most 64 channels, where 8 offsets cover every input exactly once.  The atomic fetch-on-demand
 // and the staged gather-GEMM-scatter dataflows of the reference were never the fastest.
 extern "C" int pce_select_dataflow(int64_t n_in, int64_t n_out, int64_t n_pairs, int32_t c_in, int32_t c_out, int32_t kv,
@@ -1579,7 +1734,7 @@ extern "C" int pce_select_dataflow(int64_t n_in, int64_t n_out, int64_t n_pairs,
   if (n_out <= 0) return PCE_DATAFLOW_FDS;
   double rho = (double)n_pairs / (double)n_out;
   if (kv == 1) return PCE_DATAFLOW_OS;
-  if (rho >= 14.0) return PCE_DATAFLOW_OS;
+  if (rho >= 16.0) return PCE_DATAFLOW_OS;
   if (rho >= 6.0) return ((int64_t)c_in * c_out <= 128 * 128) ? PCE_DATAFLOW_OS : PCE_DATAFLOW_FDS;
   if (kv <= 8 && rho >= 1.0 && c_in <= 64 && c_out <= 64 && n_out <= n_in) return PCE_DATAFLOW_OS;
   return PCE_DATAFLOW_FDS;
