@@ -29,6 +29,9 @@ def main() -> int:
                     help="cfg2: the headline layer; deep: a decoder-like layer (dense map, C 256->256) for the MFMA roofline")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-net", action="store_true", help="skip the MinkUNet-style forward (configuration 4)")
+    ap.add_argument("--all-configs", action="store_true",
+                    help="also time configurations 1 (fp32 C16 layer), 3 (k2s2 down + transposed up) and 5 (8-scene indoor "
+                         "batch, widened network); results go to extra.cfg1 / cfg3 / cfg5")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this engine has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -251,6 +254,61 @@ def main() -> int:
         os.environ.pop("PCENGINE_DATAFLOW", None)
         result["extra"]["cfg4_minkunet"] = {"voxels": int(len(c4)), "dtype": "f16", "selector": net["auto"],
                                             "all_fetch_on_demand": net["fod"], "all_gather_gemm_scatter": net["gms"]}
+
+    # ---- configurations 1, 3 and 5 (opt-in) ------------------------------------------------------------
+    if args.all_configs:
+        import pcengine_amd as pe
+        from pcengine_amd import nets
+        # cfg1: fp32, C 16 -> 16, ~20 k voxels
+        c1 = synth.sphere_plane_cloud()
+        f1 = torch.as_tensor(synth.features(1, len(c1), 16), device=dev).float()
+        w1 = torch.as_tensor(synth.weights(1, 27, 16, 16), device=dev).float()
+        km1 = backend.build_kernel_map(torch.as_tensor(c1, device=dev), ks, (1, 1, 1), (0, 0, 0), [0, 0, 0],
+                                       c1[:, 1:].max(0).tolist(), True, want_csr=True)
+        o1 = torch.empty((len(c1), 16), dtype=torch.float32, device=dev)
+        fl1 = backend.select_dataflow(km1, 16, 16, torch.float32)
+        b1 = torch.empty(max(km1.qsum * 32, 1), dtype=torch.float32, device=dev)
+        t1 = timer(lambda: backend.conv_forward(f1, w1, km1, fl1, buffer=b1, out=o1), 100, 10)[0]
+        result["extra"]["cfg1"] = {"voxels": int(len(c1)), "pairs": int(km1.M), "dtype": "f32", "dataflow": names[fl1],
+                                   "layer_ms": round(t1, 5)}
+        # cfg3: k2s2 down 64 -> 128 on the cfg2 cloud, transposed k2s2 128 -> 64 back
+        g3 = [(c - 1) // 2 for c in cmax]
+        km3 = backend.build_kernel_map(cd, (2, 2, 2), (2, 2, 2), (0, 0, 0), [0, 0, 0], g3, False, want_csr=True,
+                                       want_nbr_in=True, batchsize=1)
+        wdn = torch.as_tensor(synth.weights(3, 8, 64, 128), device=dev).half()
+        wup = torch.as_tensor(synth.weights(3, 8, 128, 64), device=dev).half()
+        pdn, pup = backend.pack_weights(wdn), backend.pack_weights(wup)
+        mid3 = torch.empty((km3.n_out, 128), dtype=torch.float16, device=dev)
+        back3 = torch.empty((n, 64), dtype=torch.float16, device=dev)
+        b3 = torch.empty(max(km3.qsum * 192, 1), dtype=torch.float16, device=dev)
+        fd3 = backend.select_dataflow(km3, 64, 128, torch.float16)
+        fu3 = backend.select_dataflow(km3, 128, 64, torch.float16, transposed=True)
+
+        def down_up():
+            backend.conv_forward(fd, wdn, km3, fd3, buffer=b3, packed=pdn, out=mid3)
+            backend.conv_forward(mid3, wup, km3, fu3, transposed=True, buffer=b3, packed=pup, out=back3)
+        t3 = timer(down_up, 100, 10)[0]
+        result["extra"]["cfg3"] = {"voxels_in": int(n), "voxels_out": int(km3.n_out), "pairs": int(km3.M),
+                                   "dataflow_down": names[fd3], "dataflow_up": names[fu3], "down_up_ms": round(t3, 5)}
+        # cfg5: 8 indoor scenes, the cfg4 network with channels doubled
+        c5 = synth.indoor_batch()
+        f5 = torch.as_tensor(synth.features(5, len(c5), 4), device=dev).half()
+        c5d = torch.as_tensor(c5, device=dev)
+        torch.manual_seed(5)
+        model5 = nets.SparseResUNet(4, 20, stem=64, enc=(64, 128, 256, 512), dec=(512, 256, 192, 192)).to(dev).eval().fuse_bn().half()
+        cmax5 = c5[:, 1:].max(0).tolist()
+
+        def forward5(keep=None):
+            x = pe.spTensor(f5, c5d, None, [0, 0, 0], cmax5, batchsize=8)
+            if keep is not None:
+                x.kmaps, x.cbook = keep.kmaps, keep.cbook
+            with torch.no_grad():
+                return model5(x)
+        y5 = forward5()
+        result["extra"]["cfg5"] = {"voxels": int(len(c5)), "scenes": 8, "dtype": "f16",
+                                   "forward_ms_with_map_build": round(ev_ms(forward5, 5, 1), 3),
+                                   "forward_ms_cached_maps": round(ev_ms(lambda: forward5(y5), 10, 2), 3)}
+        del model5, y5, f5, c5d
 
     # ---- CPU baseline: the oracle's torch path on this box's host cores, same workload ---------
     if not args.no_cpu:
