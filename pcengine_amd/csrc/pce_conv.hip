@@ -1722,20 +1722,34 @@ extern "C" int pce_conv_fwd_dense(const void *in, const void *w, const void *wp,
 // Map density rho = pairs per output row.  The deferred-scatter dataflow does only the useful
 // multiplications and pays M*(c_in + 2*c_out) elements of gather / partial-row traffic for them; the
 // output-stationary kernel touches no intermediate memory but multiplies every offset of every
-// 128-row tile, populated or not.  Measured on a MinkUNet-style network (100 k voxels, fp16): deferred
-// scatter wins up to rho = 3 at every width and at rho = 9 for 256 channels; output-stationary wins at
-// rho = 6 to 9 up to 128 channels, at rho = 20 everywhere (at rho = 13 and 256 channels deferred scatter
-// still leads), and (by a little) on 2x2x2 stride-2 layers of
-// at most 64 channels, where 8 offsets cover every input exactly once.  The atomic fetch-on-demand
-// and the staged gather-GEMM-scatter dataflows of the reference were never the fastest.
+// 128-row tile, populated or not.  So the density at which output-stationary takes over rises with the
+// channel product: the wider the layer, the dearer its wasted multiplications and the cheaper, per
+// flop, the partial-row traffic.  Thresholds from two MinkUNet-style networks measured layer by layer
+// with every dataflow (100 k LiDAR voxels, channels 32..256; 954 k indoor voxels in 8 scenes, channels
+// 64..512): up to 64x64 channels output-stationary leads from rho = 4 (2x at rho = 5), up to 128x128
+// from rho = 5..6, up to 256x256 the two are within 10 % between rho = 9 and 13 and output-stationary
+// leads by 1.35x at rho = 20; at 512 channels deferred scatter leads at every density seen.  A
+// 2x2x2 stride-2 layer covers every input exactly once and favours output-stationary up to 64x64.
+// The atomic fetch-on-demand and the staged gather-GEMM-scatter dataflows of the reference were never
+// the fastest (gather-GEMM-scatter comes first only on a 4-channel input layer, by 10 %).
 extern "C" int pce_select_dataflow(int64_t n_in, int64_t n_out, int64_t n_pairs, int32_t c_in, int32_t c_out, int32_t kv,
                                    int32_t dtype) {
-  (void)dtype;
   if (n_out <= 0) return PCE_DATAFLOW_FDS;
-  double rho = (double)n_pairs / (double)n_out;
   if (kv == 1) return PCE_DATAFLOW_OS;
-  if (rho >= 16.0) return PCE_DATAFLOW_OS;
-  if (rho >= 6.0) return ((int64_t)c_in * c_out <= 128 * 128) ? PCE_DATAFLOW_OS : PCE_DATAFLOW_FDS;
-  if (kv <= 8 && rho >= 1.0 && c_in <= 64 && c_out <= 64 && n_out <= n_in) return PCE_DATAFLOW_OS;
-  return PCE_DATAFLOW_FDS;
+  const double rho = (double)n_pairs / (double)n_out;
+  const int64_t prod = (int64_t)c_in * c_out;
+  if (kv <= 8 && n_out <= n_in && rho >= 1.0 && prod <= 64 * 64 && dtype == PCE_F16) return PCE_DATAFLOW_OS;
+  double takeover;
+  if (prod <= 64 * 64)
+    takeover = 4.0;
+  else if (prod <= 128 * 128)
+    takeover = 5.0;
+  else if (prod <= 256 * 256)
+    takeover = 12.0;
+  else
+    return PCE_DATAFLOW_FDS;
+  // fp32 multiplies at a fraction of the fp16 MFMA rate: wasted multiplications cost more (configuration 1,
+  // fp32 16x16 channels at rho = 4.7, is 1.35x faster with deferred scatter)
+  if (dtype == PCE_F32) takeover *= 2.0;
+  return rho >= takeover ? PCE_DATAFLOW_OS : PCE_DATAFLOW_FDS;
 }
