@@ -1194,29 +1194,50 @@ __global__ void __launch_bounds__(256) epilogue_rows_kernel(T *__restrict__ out,
   *reinterpret_cast<V *>(&out[row * c_out + (long long)v * VEC]) = x;
 }
 
-// out[o] += sum of the partial rows of o, for the rows that have any: one group of G lanes per pair;
-// the pair whose partial row is the first of its output row does the whole row.
-template <typename T, int VEC>
-__global__ void __launch_bounds__(256) rowsum_pairs_kernel(const T *__restrict__ buf, long long n_pairs, int c_out, int G,
+// out[o] = act(out[o] + sum of the partial rows of o) for the rows that have any.  BY_ROW = false: one
+// group of G lanes per pair, and the pair whose partial row is the first of its output row does the
+// whole row (few pairs per row: most rows are never visited).  BY_ROW = true: one group per output row
+// (more pairs than rows).  Partial rows are requested four at a time.
+template <typename T, int VEC, bool BY_ROW>
+__global__ void __launch_bounds__(256) rowsum_pairs_kernel(const T *__restrict__ buf, long long n_items, int c_out, int G,
                                                            const int *__restrict__ omap, const int *__restrict__ oslot,
                                                            const int *__restrict__ csr, T *__restrict__ out, int act,
                                                            float slope) {
   typedef typename VecOf<T, VEC>::type V;
-  long long p = (long long)blockIdx.x * (256 / G) + threadIdx.x / G;
+  long long item = (long long)blockIdx.x * (256 / G) + threadIdx.x / G;
   int sub = threadIdx.x % G;
-  if (p >= n_pairs) return;
-  int row = omap[p];
-  int e0 = csr[row];
-  if (oslot[p] != e0) return;
-  int e1 = csr[row + 1];
+  if (item >= n_items) return;
+  int row, e0, e1;
+  if (BY_ROW) {
+    row = (int)item;
+    e0 = csr[row];
+    e1 = csr[row + 1];
+    if (e0 >= e1) return;
+  } else {
+    row = omap[item];
+    e0 = csr[row];
+    if (oslot[item] != e0) return;
+    e1 = csr[row + 1];
+  }
   int row_vecs = c_out / VEC;
   for (int v = sub; v < row_vecs; v += G) {
+    const T *bp = buf + (long long)v * VEC;
     V x = *reinterpret_cast<const V *>(&out[(long long)row * c_out + (long long)v * VEC]);
     float acc[VEC];
 #pragma unroll
     for (int j = 0; j < VEC; ++j) acc[j] = (float)(reinterpret_cast<const T *>(&x)[j]);
-    for (int e = e0; e < e1; ++e) {
-      V y = *reinterpret_cast<const V *>(&buf[(long long)e * c_out + (long long)v * VEC]);
+    int e = e0;
+    for (; e + 4 <= e1; e += 4) {
+      V y[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) y[u] = *reinterpret_cast<const V *>(bp + (long long)(e + u) * c_out);
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[j] += (float)(reinterpret_cast<const T *>(&y[u])[j]);
+    }
+    for (; e < e1; ++e) {
+      V y = *reinterpret_cast<const V *>(bp + (long long)e * c_out);
 #pragma unroll
       for (int j = 0; j < VEC; ++j) acc[j] += (float)(reinterpret_cast<const T *>(&y)[j]);
     }
@@ -1225,6 +1246,36 @@ __global__ void __launch_bounds__(256) rowsum_pairs_kernel(const T *__restrict__
     *reinterpret_cast<V *>(&out[(long long)row * c_out + (long long)v * VEC]) = x;
   }
 }
+
+// picks the vector width and the iteration space of the row sum
+template <typename T>
+static int launch_rowsum_pairs(const T *buffer, T *out, int64_t n_out, int64_t n_pairs, int c_out, const int *omap,
+                               const int *oslot, const int *ocsr, int act, float slope, hipStream_t s) {
+  if (n_pairs <= 0) return PCE_OK;
+  constexpr int VEC = sizeof(T) == 2 ? 8 : 4;
+  const bool vec = (c_out % VEC == 0) && (((uintptr_t)out | (uintptr_t)buffer) & 15) == 0;
+  int G = 1;
+  while (G < (vec ? c_out / VEC : c_out)) G <<= 1;
+  if (G > 64) G = 64;
+  const bool by_row = n_pairs > n_out;
+  const long long items = by_row ? n_out : n_pairs;
+  dim3 grid((unsigned)pce_div_up(items, 256 / G)), block(256);
+#define PCE_ROWSUM(V_, B_)                                                                                        \
+  hipLaunchKernelGGL((rowsum_pairs_kernel<T, V_, B_>), grid, block, 0, s, buffer, items, c_out, G, omap, oslot, ocsr, out, \
+                     act, slope)
+  if (vec && by_row)
+    PCE_ROWSUM(VEC, true);
+  else if (vec)
+    PCE_ROWSUM(VEC, false);
+  else if (by_row)
+    PCE_ROWSUM(1, true);
+  else
+    PCE_ROWSUM(1, false);
+#undef PCE_ROWSUM
+  PCE_LAUNCH_CHECK("rowsum_pairs");
+  return PCE_OK;
+}
+
 
 __global__ void __launch_bounds__(256) convert_f32_f16_kernel(const float *__restrict__ in, half_t *__restrict__ out,
                                                               long long n) {
@@ -1563,12 +1614,9 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
     set_epi(&c, e);
     if (a.host_pos && wave_gemm_ok(a, sizeof(T)) && wave_gemm_ok(c, sizeof(T)) && aligned16(buffer) && epi_aligned(e)) {
       if (stage_on(1) && (rc = launch_wave_gemm(a, c, s))) return rc;
-      if (stage_on(2)) {
-        int G = pow2_at_least(c_out / VEC);
-        hipLaunchKernelGGL((rowsum_pairs_kernel<T, VEC>), dim3((unsigned)pce_div_up(n_pairs, 256 / G)), dim3(256), 0, s,
-                           (const T *)buffer, (long long)n_pairs, c_out, G, omap, oslot, ocsr, (T *)out, e.act, e.slope);
-        PCE_LAUNCH_CHECK("rowsum_pairs");
-      }
+      if (stage_on(2) && (rc = launch_rowsum_pairs<T>((const T *)buffer, (T *)out, n_out, n_pairs, c_out, omap, oslot, ocsr,
+                                                      e.act, e.slope, s)))
+        return rc;
       return PCE_OK;
     }
   }
@@ -1605,19 +1653,7 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
     a.act_alone_only = 1;
     set_epi(&a, e);
     if ((rc = launch_tile<T>(a, pce_div_up(n_out, 128), s))) return rc;
-    if (n_pairs > 0) {
-      bool vec = (c_out % VEC == 0) && aligned16(out) && aligned16(buffer);
-      int G = pow2_at_least(vec ? c_out / VEC : c_out);
-      if (G > 64) G = 64;
-      if (vec)
-        hipLaunchKernelGGL((rowsum_pairs_kernel<T, VEC>), dim3((unsigned)pce_div_up(n_pairs, 256 / G)), dim3(256), 0, s,
-                           (const T *)buffer, (long long)n_pairs, c_out, G, omap, oslot, ocsr, (T *)out, e.act, e.slope);
-      else
-        hipLaunchKernelGGL((rowsum_pairs_kernel<T, 1>), dim3((unsigned)pce_div_up(n_pairs, 256 / G)), dim3(256), 0, s,
-                           (const T *)buffer, (long long)n_pairs, c_out, G, omap, oslot, ocsr, (T *)out, e.act, e.slope);
-      PCE_LAUNCH_CHECK("rowsum_pairs");
-    }
-    return PCE_OK;
+    return launch_rowsum_pairs<T>((const T *)buffer, (T *)out, n_out, n_pairs, c_out, omap, oslot, ocsr, e.act, e.slope, s);
   }
   if (mid >= 0) {
     TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
