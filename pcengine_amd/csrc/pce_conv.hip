@@ -1142,8 +1142,19 @@ __global__ void __launch_bounds__(256) rowsum_kernel(const T *__restrict__ buf, 
     float acc[VEC];
 #pragma unroll
     for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
-    for (int e = e0; e < e1; ++e) {
-      V x = *reinterpret_cast<const V *>(&buf[(long long)e * c_out + (long long)v * VEC]);
+    const T *bp = buf + (long long)v * VEC;
+    int e = e0;
+    for (; e + 4 <= e1; e += 4) {  // four partial rows in flight
+      V x[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) x[u] = *reinterpret_cast<const V *>(bp + (long long)(e + u) * c_out);
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[j] += (float)(reinterpret_cast<const T *>(&x[u])[j]);
+    }
+    for (; e < e1; ++e) {
+      V x = *reinterpret_cast<const V *>(bp + (long long)e * c_out);
 #pragma unroll
       for (int j = 0; j < VEC; ++j) acc[j] += (float)(reinterpret_cast<const T *>(&x)[j]);
     }
