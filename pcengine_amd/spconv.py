@@ -94,6 +94,10 @@ class conv3d(nn.Module):
         if getattr(self, "_wcache_key", None) != key:
             w = k.detach()
             w = w if w.dtype == dtype else w.to(dtype)
+            if dtype == torch.float16 and w.is_cuda and w.dim() == 3 and w.shape[1] < 16:
+                # a 3- or 4-channel input layer: zero rows up to 16 input channels make the rows 16-byte
+                # multiples, which the vector kernels need (the features are padded to match in _run)
+                w = torch.nn.functional.pad(w, (0, 0, 0, 16 - w.shape[1]))
             w = w.contiguous()
             self._wcache = (w, backend.pack_weights(w) if w.is_cuda else None)
             self._wcache_key = key
@@ -136,6 +140,8 @@ def _run(input: spTensor, km: backend.KernelMap, kernel, in_channel, out_channel
     feats = input.feats
     if kernel.dtype != feats.dtype:
         kernel, packed = kernel.to(feats.dtype), None
+    if kernel.dim() == 3 and feats.shape[1] < kernel.shape[1]:
+        feats = torch.nn.functional.pad(feats, (0, kernel.shape[1] - feats.shape[1]))    # see conv3d._weights_for
     df = _pick_dataflow(km, dataflow, in_channel, out_channel, feats.dtype, transposed)
     out = backend.conv_forward(feats, kernel.detach(), km, df, transposed=transposed, buffer=input.buffer, packed=packed,
                                bias=bias, residual=residual, act=act)
