@@ -254,6 +254,21 @@ int pce_conv_fwd_dense(const void *in_feats, const void *weight, const void *wei
                        int64_t n, int32_t c_in, int32_t c_out, const pce_epilogue_t *epilogue,
                        pce_stream_t stream);
 
+/* ---- backward ------------------------------------------------------------------------------- *
+ * Replaces ConvolutionBackwardD1 (backend/spconv.h:43-58, backend/spconv.cu:400-629).
+ * The gradient with respect to the features is a forward call: pass grad_out as in_feats, the
+ * kernel with every offset transposed ([kv, c_out, c_in]) as weight and the map with the roles
+ * swapped; any forward entry point and dataflow serves.  The gradient with respect to the kernel is
+ * pce_conv_wgrad: grad_w[kp] = sum over the pairs of offset kp of in_feats[imap[p]]^T (x)
+ * grad_out[omap[p]], plus in_feats^T * grad_out for the centre offset when mid >= 0.  grad_w is
+ * fp32 [kv, c_in, c_out] whatever `dtype` the features have; the call zeroes it first.  Pair lists
+ * as for pce_conv_fwd_fod (swap imap / omap for a transposed layer; n_in rows of in_feats, n_out
+ * rows of grad_out). */
+int pce_conv_wgrad(const void *in_feats, const void *grad_out, int32_t dtype, int64_t n_in,
+                   int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv, int32_t mid,
+                   const int32_t *imap_dev, const int32_t *omap_dev, const int32_t *kpos_dev,
+                   const int32_t *qkpos_dev, int64_t qsum, float *grad_w_f32_dev, pce_stream_t stream);
+
 /* Per-layer dataflow choice from map density (pairs per output row) and channel widths. */
 int pce_select_dataflow(int64_t n_in, int64_t n_out, int64_t n_pairs, int32_t c_in, int32_t c_out,
                         int32_t kv, int32_t dtype);

@@ -319,6 +319,32 @@ def conv_forward(feats: np.ndarray, weight: np.ndarray, km: KernelMap, ks,
     return out
 
 
+def conv_backward(feats: np.ndarray, weight: np.ndarray, km: KernelMap, ks, grad_out: np.ndarray,
+                  transposed: bool = False):
+    """float64 gradients of ``conv_forward`` with respect to features and kernel
+    (ConvolutionBackwardD1, backend/spconv.cu:400-629; script/spconv.py:172-201): for every pair
+    (src row s, dst row d, offset kp): grad_feats[s] += grad_out[d] @ W[kp]^T and
+    grad_W[kp] += feats[s]^T (x) grad_out[d]; the centre offset of a submanifold layer pairs every
+    row with itself."""
+    f = feats.astype(np.float64)
+    w = weight.astype(np.float64)
+    g = grad_out.astype(np.float64)
+    src, dst = (km.omap, km.imap) if transposed else (km.imap, km.omap)
+    gf = np.zeros_like(f)
+    gw = np.zeros_like(w)
+    if km.subm:
+        m = mid_offset(ks)
+        gf += g @ w[m].T
+        gw[m] += f.T @ g
+    for kp in range(km.kv):
+        a, b = int(km.kpos[kp]), int(km.kpos[kp + 1])
+        if a == b:
+            continue
+        np.add.at(gf, src[a:b], g[dst[a:b]] @ w[kp].T)
+        gw[kp] += f[src[a:b]].T @ g[dst[a:b]]
+    return gf, gw
+
+
 def brute_force_pairs(in_coords: np.ndarray, out_coords: np.ndarray, ks, stride, pad, subm: bool):
     """O(N_in * N_out * kv) definition straight from the geometry; tiny inputs only."""
     d = offsets(ks, strided=not subm)

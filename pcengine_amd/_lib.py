@@ -77,6 +77,8 @@ _SIGNATURES = {
                                    POINTER(Epilogue), c_void_p]),
     "pce_conv_fwd_os": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_void_p, POINTER(Epilogue), c_void_p]),
     "pce_conv_fwd_dense": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32, POINTER(Epilogue), c_void_p]),
+    "pce_conv_wgrad": (c_int32, [c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p,
+                                 c_void_p, c_void_p, c_int64, c_void_p, c_void_p]),
     "pce_select_dataflow": (c_int32, [c_int64, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32]),
 }
 

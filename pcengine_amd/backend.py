@@ -355,6 +355,11 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
         raise ValueError("Input feature size and kernel size mismatch")   # backend/spconv.cu:38-40
     if kv != km.kv:
         raise ValueError(f"kernel volume {kv} does not match the map ({km.kv})")
+    if transposed and km.subm:
+        # a submanifold map is its own mirror image: pair (i, o, kp) exists iff (o, i, kv-1-kp) does, so the
+        # transposed layer is the plain layer with the offsets of the kernel reversed
+        weight, packed, transposed = weight.flip(0).contiguous(), None, False
+        packed = pack_weights(weight)
     n_in, n_out = (km.n_out, km.n_in) if transposed else (km.n_in, km.n_out)
     if feats.shape[0] != n_in:
         raise ValueError(f"features have {feats.shape[0]} rows, the map expects {n_in}")
@@ -402,6 +407,42 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
     else:
         raise NotImplementedError(f"unknown dataflow {dataflow}")
     return out
+
+
+def conv_wgrad(feats: torch.Tensor, grad_out: torch.Tensor, km: KernelMap, transposed: bool = False) -> torch.Tensor:
+    """Gradient of ``conv_forward`` with respect to the kernel: fp32 [kv, c_in, c_out]."""
+    lib = _lib.load()
+    _require_cuda(feats, "feats")
+    feats, grad_out = feats.contiguous(), grad_out.contiguous()
+    if feats.dtype != grad_out.dtype:
+        raise TypeError(f"features are {feats.dtype} but the output gradient is {grad_out.dtype}")
+    n_in, n_out = (km.n_out, km.n_in) if transposed else (km.n_in, km.n_out)
+    if feats.shape[0] != n_in or grad_out.shape[0] != n_out:
+        raise ValueError(f"the map expects {n_in} feature rows and {n_out} gradient rows")
+    imap, omap = (km.omap, km.imap) if transposed else (km.imap, km.omap)
+    c_in, c_out = feats.shape[1], grad_out.shape[1]
+    gw = torch.empty((km.kv, c_in, c_out), dtype=torch.float32, device=feats.device)
+    _lib.check(lib.pce_conv_wgrad(feats.data_ptr(), grad_out.data_ptr(), _dtype_code(feats), n_in, n_out, c_in, c_out, km.kv,
+                                  _mid(km.ks) if km.subm else -1, imap.data_ptr(), omap.data_ptr(), km.kpos.data_ptr(),
+                                  km.qkpos.data_ptr(), km.qsum, gw.data_ptr(), _stream(feats.device)))
+    return gw
+
+
+def conv_backward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, grad_out: torch.Tensor, transposed: bool = False,
+                  need_feats: bool = True, need_weight: bool = True, dataflow: Optional[int] = None):
+    """(grad_feats, grad_weight) of ``conv_forward``.  The feature gradient is the convolution of
+    ``grad_out`` with the per-offset transposed kernel over the same pairs with the roles swapped,
+    run by the forward kernels; the kernel gradient comes from ``pce_conv_wgrad`` (fp32 sums,
+    returned in the kernel's dtype)."""
+    gf = gw = None
+    w3 = weight if weight.dim() == 3 else weight.unsqueeze(0)
+    if need_feats:
+        wt = w3.transpose(1, 2).contiguous()
+        df = dataflow if dataflow is not None else select_dataflow(km, wt.shape[1], wt.shape[2], wt.dtype, not transposed)
+        gf = conv_forward(grad_out.contiguous(), wt, km, df, transposed=not transposed, packed=pack_weights(wt))
+    if need_weight:
+        gw = conv_wgrad(feats, grad_out, km, transposed).to(weight.dtype).reshape(weight.shape)
+    return gf, gw
 
 
 # ---------------------------------------------------------------------------------------------
@@ -491,6 +532,51 @@ def conv_fwd_d1_cuda(in_feats, kernel, ksize_code, qsum_nnz, out_feats, kpos, qk
                                     _stream(in_feats.device)))
 
 
-def conv_bwd_d1_cuda(*args, **kwargs):
-    """ConvolutionBackwardD1 (backend/spconv.h:43-58) belongs to training; this engine is forward-only."""
-    raise NotImplementedError("pcengine_amd is an inference engine: the backward pass is not provided")
+def conv_bwd_d1_cuda(out_feats_grad, in_feats, kernel, ksize_code, sum_nnz, in_feats_grad, kernel_grad, kernel_nnz,
+                     kernel_pos, in_map, out_map, in_csr, out_csr, buffer, tensorcore):
+    """ConvolutionBackwardD1 (backend/spconv.h:43-58): fills ``in_feats_grad`` and ``kernel_grad``
+    from the CSR-coded map of ``mapping_d1_cuda``.  The coded lists are decoded into the plain pair
+    lists first (entry = kp * 1186111 + rank, pair index = kpos[kp] + rank)."""
+    lib = _lib.load()
+    _require_cuda(in_feats, "in_feats")
+    if in_feats.shape[1] != kernel.shape[1]:
+        raise ValueError("Input feature size and kernel size mismatch")
+    kv, c_in, c_out = kernel.shape
+    n_in, n_out = in_feats.shape[0], out_feats_grad.shape[0]
+    dev = in_feats.device
+    M = int(in_csr[n_in].item())
+    kpos = kernel_pos[:kv].to(torch.int64)
+    kpos_full = torch.cat([kpos, torch.tensor([M], device=dev, dtype=torch.int64)])
+
+    def pairs(csr, code, n):
+        rows = torch.repeat_interleave(torch.arange(n, device=dev, dtype=torch.int32), (csr[1:n + 1] - csr[:n]).long())
+        c = code[:M].long()
+        idx = kpos[c // CSR_CODE] + c % CSR_CODE
+        out = torch.empty(M, dtype=torch.int32, device=dev)
+        out[idx] = rows
+        return out
+    imap, omap = pairs(in_csr, in_map, n_in), pairs(out_csr, out_map, n_out)
+    knnz = (kpos_full[1:] - kpos_full[:-1])
+    q = (knnz + QUANTUM - 1) // QUANTUM * QUANTUM
+    qkpos = torch.cat([torch.zeros(1, dtype=torch.int64, device=dev), torch.cumsum(q, 0)]).to(torch.int32)
+    kp32 = kpos_full.to(torch.int32)
+    qsum = int(qkpos[-1].item())
+    separate_mid = n_in == n_out
+    mid = _ksize_mid(ksize_code, separate_mid)
+    dt = _dtype_code(in_feats)
+    s = _stream(dev)
+    gw = torch.empty((kv, c_in, c_out), dtype=torch.float32, device=dev)
+    _lib.check(lib.pce_conv_wgrad(in_feats.data_ptr(), out_feats_grad.contiguous().data_ptr(), dt, n_in, n_out, c_in, c_out, kv,
+                                  mid, imap.data_ptr(), omap.data_ptr(), kp32.data_ptr(), qkpos.data_ptr(), qsum,
+                                  gw.data_ptr(), s))
+    kernel_grad.copy_(gw.to(kernel_grad.dtype))
+    wt = kernel.transpose(1, 2).contiguous()
+    ws_bytes = lib.pce_conv_fod_workspace_bytes(n_in, c_in, dt)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+    g = out_feats_grad.contiguous()
+    tmp = in_feats_grad if in_feats_grad.dtype == in_feats.dtype else torch.empty_like(in_feats)
+    _lib.check(lib.pce_conv_fwd_fod(g.data_ptr(), wt.data_ptr(), None, tmp.data_ptr(), dt, n_out, n_in, c_out, c_in, kv, mid,
+                                    omap.data_ptr(), imap.data_ptr(), kp32.data_ptr(), qkpos.data_ptr(), qsum, _ptr(ws),
+                                    ws_bytes, None, s))
+    if tmp is not in_feats_grad:
+        in_feats_grad.copy_(tmp.to(in_feats_grad.dtype))

@@ -1766,6 +1766,114 @@ extern "C" int pce_conv_fwd_dense(const void *in, const void *w, const void *wp,
   return dense_impl<float>(in, w, wp, out, n, c_in, c_out, e, s);
 }
 
+// ---- weight gradient ------------------------------------------------------------------------------
+// grad_W[kp][ci][co] = sum over the pairs p of offset kp of in[imap[p]][ci] * grad_out[omap[p]][co]
+// (ConvolutionBackwardD1's per-offset GEMM, backend/spconv.cu:400-629).  A workgroup takes one
+// 128-pair quantum (or 128 rows of the centre offset) and a 64 x 64 block of (ci, co): rows are staged
+// in LDS 32 at a time as fp32, every thread accumulates a 4 x 4 block in registers and adds it to the
+// fp32 result with atomics (the order of the additions, and so the last bits, vary from run to run).
+template <typename T>
+__global__ void __launch_bounds__(256) wgrad_kernel(const T *__restrict__ in, const T *__restrict__ gout, long long n_rows,
+                                                    int c_in, int c_out, int kv, int mid, const int *__restrict__ imap,
+                                                    const int *__restrict__ omap, const int *__restrict__ kpos,
+                                                    const int *__restrict__ qkpos, long long pair_tiles, int ci_tiles,
+                                                    int co_tiles, float *__restrict__ gw) {
+  __shared__ float As[32][64 + 4];
+  __shared__ float Gs[32][64 + 4];
+  __shared__ int rows_in[128], rows_out[128];
+  long long tile = blockIdx.x / (ci_tiles * co_tiles);
+  int rest = (int)(blockIdx.x % (ci_tiles * co_tiles));
+  const int ci0 = (rest / co_tiles) * 64, co0 = (rest % co_tiles) * 64;
+  int widx;
+  if (tile < pair_tiles) {
+    long long q0 = tile * 128;
+    widx = 0;
+    for (int i = 0; i < kv; ++i) widx += ((long long)qkpos[i + 1] <= q0) ? 1 : 0;
+    if (widx >= kv) return;
+    if (threadIdx.x < 128) {
+      long long p = q0 - qkpos[widx] + kpos[widx] + threadIdx.x;
+      bool ok = p < (long long)kpos[widx + 1];
+      rows_in[threadIdx.x] = ok ? imap[p] : -1;
+      rows_out[threadIdx.x] = ok ? omap[p] : -1;
+    }
+  } else {  // centre offset of a submanifold layer: every row pairs with itself
+    widx = mid;
+    if (threadIdx.x < 128) {
+      long long row = (tile - pair_tiles) * 128 + threadIdx.x;
+      rows_in[threadIdx.x] = rows_out[threadIdx.x] = row < n_rows ? (int)row : -1;
+    }
+  }
+  __syncthreads();
+  const int tci = (threadIdx.x / 16) * 4, tco = (threadIdx.x % 16) * 4;
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+  for (int p0 = 0; p0 < 128; p0 += 32) {
+    // stage 32 rows x 64 channels of both operands: 8 elements per thread and matrix
+    {
+      int r = threadIdx.x / 8, c = (threadIdx.x % 8) * 8;
+      int ri = rows_in[p0 + r], ro = rows_out[p0 + r];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        int ci = ci0 + c + j, co = co0 + c + j;
+        As[r][c + j] = (ri >= 0 && ci < c_in) ? (float)in[(long long)ri * c_in + ci] : 0.f;
+        Gs[r][c + j] = (ro >= 0 && co < c_out) ? (float)gout[(long long)ro * c_out + co] : 0.f;
+      }
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int k = 0; k < 32; ++k) {
+      float av[4], gv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        av[i] = As[k][tci + i];
+        gv[i] = Gs[k][tco + i];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] += av[i] * gv[j];
+    }
+    __syncthreads();
+  }
+  float *dst = gw + (long long)widx * c_in * c_out;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int ci = ci0 + tci + i, co = co0 + tco + j;
+      if (ci < c_in && co < c_out && acc[i][j] != 0.f) unsafeAtomicAdd(dst + (long long)ci * c_out + co, acc[i][j]);
+    }
+}
+
+extern "C" int pce_conv_wgrad(const void *in, const void *gout, int32_t dtype, int64_t n_in, int64_t n_out, int32_t c_in,
+                              int32_t c_out, int32_t kv, int32_t mid, const int32_t *imap, const int32_t *omap,
+                              const int32_t *kpos, const int32_t *qkpos, int64_t qsum, float *gw, pce_stream_t stream) {
+  int rc = check_common("pce_conv_wgrad", in, gout, gw, dtype, n_in, n_out, c_in, c_out, kv, mid);
+  if (rc || (rc = check_qsum("pce_conv_wgrad", qsum))) return rc;
+  if (!kpos || !qkpos || (qsum > 0 && (!imap || !omap))) PCE_FAIL(PCE_EINVAL, "pce_conv_wgrad: null map pointer");
+  hipStream_t s = (hipStream_t)stream;
+  long long total = (long long)kv * c_in * c_out;
+  hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)pce_div_up(total, 1024)), dim3(256), 0, s, gw, total);
+  PCE_LAUNCH_CHECK("zero_f32");
+  long long pair_tiles = qsum / PCE_QUANTUM;
+  long long tiles = pair_tiles + (mid >= 0 ? pce_div_up(n_out, 128) : 0);
+  int ci_tiles = (c_in + 63) / 64, co_tiles = (c_out + 63) / 64;
+  long long blocks = tiles * ci_tiles * co_tiles;
+  if (blocks <= 0) return PCE_OK;
+  if (blocks >= (1ll << 31)) PCE_FAIL(PCE_ECAPACITY, "pce_conv_wgrad: %lld workgroups exceed the grid limit", blocks);
+  if (dtype == PCE_F16)
+    hipLaunchKernelGGL(wgrad_kernel<half_t>, dim3((unsigned)blocks), dim3(256), 0, s, (const half_t *)in, (const half_t *)gout,
+                       (long long)n_out, c_in, c_out, kv, mid, imap, omap, kpos, qkpos, pair_tiles, ci_tiles, co_tiles, gw);
+  else
+    hipLaunchKernelGGL(wgrad_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, s, (const float *)in, (const float *)gout,
+                       (long long)n_out, c_in, c_out, kv, mid, imap, omap, kpos, qkpos, pair_tiles, ci_tiles, co_tiles, gw);
+  PCE_LAUNCH_CHECK("wgrad");
+  return PCE_OK;
+}
+
 // Map density rho = pairs per output row.  The deferred-scatter dataflow does only the useful
 // multiplications and pays M*(c_in + 2*c_out) elements of gather / partial-row traffic for them; the
 // output-stationary kernel touches no intermediate memory but multiplies every offset of every

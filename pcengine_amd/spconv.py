@@ -8,7 +8,11 @@ Differences a user can see, all supersets of the reference:
   fetch-on-demand exactly as in the reference (script/spconv.py:343, 388); the default tag
   ('end') lets the selector decide per layer.
 * every strided layer uses the generic output-coordinate rule, also when stride == kernel size.
-* forward only.
+* training: when gradients are enabled and the features or the parameters require them, the layer
+  runs through an autograd function whose backward uses the same kernels (feature gradient =
+  convolution of the output gradient with the transposed kernel over the swapped map; kernel
+  gradient = ``pce_conv_wgrad``).  The reference has a backward for gather-GEMM-scatter only
+  (script/spconv.py:172-201); here it serves every dataflow.
 * ``forward(input, act=None, residual=None)``: an activation ('relu' or ('leaky_relu', slope)) and
   a residual tensor (same coordinates) are applied inside the convolution kernels together with
   the bias, instead of as separate passes over the output.
@@ -114,6 +118,13 @@ class conv3d(nn.Module):
         return self._bcache
 
     def forward(self, input: spTensor, act=None, residual: Optional[spTensor] = None) -> spTensor:
+        if _wants_grad(input.feats, self.kernel, self.bias):
+            # training: the parameters themselves go to the autograd function (no cached copies)
+            return conv_func(input=input, in_channel=self.in_channels, out_channel=self.out_channels, kernel=self.kernel,
+                             kernel_size_code=self.kernel_size_code, stride_code=self.stride_code,
+                             padding_code=self.padding_code, bias=self.bias, transposed=self.transposed,
+                             tensorcore=self.tensorcore, dataflow=self.dataflow, packed=None, act=act,
+                             residual=None if residual is None else residual.feats)
         w, packed = self._weights_for(input.feats.dtype)
         return conv_func(input=input, in_channel=self.in_channels, out_channel=self.out_channels, kernel=w,
                          kernel_size_code=self.kernel_size_code, stride_code=self.stride_code,
@@ -135,9 +146,80 @@ def _pick_dataflow(km: backend.KernelMap, requested: str, c_in: int, c_out: int,
     return backend.select_dataflow(km, c_in, c_out, dtype, transposed)
 
 
+class _ConvFunction(torch.autograd.Function):
+    """conv (+ bias) with gradients for features, kernel and bias (conv_d1 / conv_d2,
+    script/spconv.py:110-288)."""
+
+    @staticmethod
+    def forward(ctx, feats, kernel, bias, km, df, transposed, buffer):
+        k = kernel.detach()
+        out = backend.conv_forward(feats.detach(), k, km, df, transposed=transposed, buffer=buffer,
+                                   packed=backend.pack_weights(k), bias=None if bias is None else bias.detach())
+        ctx.save_for_backward(feats, kernel)
+        ctx.km, ctx.transposed, ctx.has_bias = km, transposed, bias is not None
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        feats, kernel = ctx.saved_tensors
+        grad_out = grad_out.contiguous()
+        gf, gw = backend.conv_backward(feats.detach(), kernel.detach(), ctx.km, grad_out, transposed=ctx.transposed,
+                                       need_feats=ctx.needs_input_grad[0], need_weight=ctx.needs_input_grad[1])
+        gb = grad_out.sum(0) if (ctx.has_bias and ctx.needs_input_grad[2]) else None
+        return gf, gw, gb, None, None, None, None
+
+
+class _DenseFunction(torch.autograd.Function):
+    """The 1x1 layer (feats @ kernel + bias) with the same backward kernels."""
+
+    @staticmethod
+    def forward(ctx, feats, kernel, bias):
+        k = kernel.detach()
+        out = backend.dense_forward(feats.detach(), k, backend.pack_weights(k), bias=None if bias is None else bias.detach())
+        ctx.save_for_backward(feats, kernel)
+        ctx.has_bias = bias is not None
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        feats, kernel = ctx.saved_tensors
+        grad_out = grad_out.contiguous()
+        gf = gw = None
+        if ctx.needs_input_grad[0]:
+            kt = kernel.detach().t().contiguous()
+            gf = backend.dense_forward(grad_out, kt, backend.pack_weights(kt))
+        if ctx.needs_input_grad[1]:
+            gw = (feats.detach().float().t() @ grad_out.float()).to(kernel.dtype)
+        gb = grad_out.sum(0) if (ctx.has_bias and ctx.needs_input_grad[2]) else None
+        return gf, gw, gb
+
+
+def _wants_grad(*tensors) -> bool:
+    return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
+
+
+def _apply_unfused(out: torch.Tensor, residual, act) -> torch.Tensor:
+    """Residual and activation as differentiable torch ops (the training path does not fuse them)."""
+    if residual is not None:
+        out = out + residual
+    if act == "relu":
+        out = torch.relu(out)
+    elif isinstance(act, tuple) and act[0] == "leaky_relu":
+        out = torch.nn.functional.leaky_relu(out, act[1])
+    elif act is not None:
+        raise ValueError(f"unknown activation {act!r}")
+    return out
+
+
 def _run(input: spTensor, km: backend.KernelMap, kernel, in_channel, out_channel, transposed, dataflow, packed,
          bias=None, residual=None, act=None) -> torch.Tensor:
     feats = input.feats
+    if _wants_grad(feats, kernel, bias):
+        k = kernel if kernel.dtype == feats.dtype else kernel.to(feats.dtype)
+        b = bias if bias is None or bias.dtype == feats.dtype else bias.to(feats.dtype)
+        df = _pick_dataflow(km, dataflow, in_channel, out_channel, feats.dtype, transposed)
+        out = _ConvFunction.apply(feats, k, b, km, df, transposed, input.buffer)
+        return _apply_unfused(out, residual, act)
     if kernel.dtype != feats.dtype:
         kernel, packed = kernel.to(feats.dtype), None
     if kernel.dim() == 3 and feats.shape[1] < kernel.shape[1]:
@@ -209,6 +291,10 @@ def conv_func(input: spTensor, in_channel, out_channel, kernel, kernel_size_code
     inside the kernels), metadata propagation (script/spconv.py:291-464)."""
     if kernel_size_code == _UNIT and stride_code == _UNIT:
         # 1x1 stride 1: plain matrix product, coordinates unchanged, no map (script/spconv.py:297-304)
+        if _wants_grad(input.feats, kernel, bias):
+            k = kernel if kernel.dtype == input.feats.dtype else kernel.to(input.feats.dtype)
+            b = bias if bias is None or bias.dtype == input.feats.dtype else bias.to(input.feats.dtype)
+            return input._like(_apply_unfused(_DenseFunction.apply(input.feats, k, b), residual, act))
         if kernel.dtype != input.feats.dtype:
             kernel, packed = kernel.to(input.feats.dtype), None
         out_feats = backend.dense_forward(input.feats, kernel.detach(), packed, bias=bias, residual=residual, act=act)

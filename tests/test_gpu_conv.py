@@ -274,5 +274,12 @@ def test_reference_named_entry_points_d2_and_d1():
     assert orc.rel_l2(out.double().cpu().numpy(), want) <= 1e-3
     with pytest.raises(ValueError):     # backend/spconv.cu:38-40
         backend.conv_fwd_d2_cuda(fd[:, :16].contiguous(), wd, enc([3, 3, 3]), qsum, out, kpos, qkpos, imap, omap, True, False)
-    with pytest.raises(NotImplementedError):
-        backend.conv_bwd_d1_cuda()
+    # backward with the reference's protocol (script/spconv.py:182-198): fp32, caller-allocated gradients
+    f32, w32 = fd.float(), wd.float()
+    g = np.random.default_rng(4).standard_normal((n, co))
+    gd = torch.as_tensor(g, device=DEV).float()
+    in_grad = torch.zeros((n, ci), dtype=torch.float, device=DEV)
+    w_grad = torch.zeros((kv, ci, co), dtype=torch.float, device=DEV)
+    backend.conv_bwd_d1_cuda(gd, f32, w32, enc([3, 3, 3]), qsum, in_grad, w_grad, knnz, kpos, imap, omap, icsr, ocsr, buffer, 1)
+    gf, gw = orc.conv_backward(f32.double().cpu().numpy(), w32.double().cpu().numpy(), ref_map, (3, 3, 3), rounded(g, torch.float32))
+    assert orc.rel_l2(in_grad.double().cpu().numpy(), gf) <= 1e-5 and orc.rel_l2(w_grad.double().cpu().numpy(), gw) <= 1e-5

@@ -290,3 +290,45 @@ def test_front_end_sparse_quantize_on_numpy_matches_oracle():
     c, idx, inv = utils.sparse_quantize(pts, 0.4, return_index=True, return_inverse=True)
     oc, oi, ov = orc.sparse_quantize(pts, (0.4, 0.4, 0.4))
     assert np.array_equal(c, oc) and np.array_equal(idx, oi) and np.array_equal(inv, ov)
+
+
+@pytest.mark.parametrize("ks,stride,pad", [((3, 3, 3), (1, 1, 1), (0, 0, 0)), ((2, 2, 2), (2, 2, 2), (0, 0, 0)),
+                                           ((3, 3, 3), (2, 2, 2), (1, 1, 1)), ((3, 1, 3), (1, 1, 1), (0, 0, 0))])
+def test_backward_vs_autograd_through_dense_conv3d(ks, stride, pad):
+    """grad_feats and grad_W of the oracle against torch.autograd on the densified convolution
+    (and on conv_transpose3d for the transposed layer), loss = sum(out * G) at the active sites."""
+    ext = 9
+    subm = tuple(stride) == (1, 1, 1)
+    coords = synth.random_cloud(seed=23, n=260, extent=ext, batches=2)
+    coords = np.unique(np.concatenate([coords, np.array([[0, ext - 1, ext - 1, ext - 1]], np.int32)]), axis=0)
+    ci, co = 4, 6
+    kv = ks[0] * ks[1] * ks[2]
+    f = synth.features(3, len(coords), ci, np.float64)
+    w = synth.weights(3, kv, ci, co, np.float64)
+    km = orc.kernel_map(coords, ks, stride, pad)
+    g = np.random.default_rng(3).standard_normal((km.n_out, co))
+    gf, gw = orc.conv_backward(f, w, km, ks, g)
+    ft = torch.as_tensor(f).requires_grad_(True)
+    wt = torch.as_tensor(w).requires_grad_(True)
+    c = torch.as_tensor(coords.astype(np.int64))
+    dense = torch.zeros((2, ext, ext, ext, ci), dtype=torch.float64).index_put((c[:, 0], c[:, 1], c[:, 2], c[:, 3]), ft).permute(0, 4, 1, 2, 3)
+    wd = wt.reshape(ks[0], ks[1], ks[2], ci, co).permute(4, 3, 0, 1, 2)
+    ref = F.conv3d(dense, wd, stride=stride, padding=[(k - 1) // 2 for k in ks] if subm else pad)
+    oc = torch.as_tensor(km.out_coords.astype(np.int64))
+    (ref[oc[:, 0], :, oc[:, 1], oc[:, 2], oc[:, 3]] * torch.as_tensor(g)).sum().backward()
+    assert orc.rel_l2(gf, ft.grad.numpy()) < 1e-12 and orc.rel_l2(gw, wt.grad.numpy()) < 1e-12
+    if not subm:
+        # transposed layer: features live on the output coordinates, gradients flow back to them
+        fo = synth.features(4, km.n_out, co, np.float64)
+        wT = synth.weights(4, kv, co, ci, np.float64)
+        gi = np.random.default_rng(4).standard_normal((len(coords), ci))
+        gfo, gwT = orc.conv_backward(fo, wT, km, ks, gi, transposed=True)
+        fot = torch.as_tensor(fo).requires_grad_(True)
+        wTt = torch.as_tensor(wT).requires_grad_(True)
+        dense_o = torch.zeros((2,) + tuple(ref.shape[2:]) + (co,), dtype=torch.float64).index_put(
+            (oc[:, 0], oc[:, 1], oc[:, 2], oc[:, 3]), fot).permute(0, 4, 1, 2, 3)
+        wdt = wTt.reshape(ks[0], ks[1], ks[2], co, ci).permute(3, 4, 0, 1, 2)
+        opad = [(ext + 2 * pad[a] - ks[a]) % stride[a] for a in range(3)]
+        up = F.conv_transpose3d(dense_o, wdt, stride=stride, padding=pad, output_padding=opad)
+        (up[c[:, 0], :, c[:, 1], c[:, 2], c[:, 3]] * torch.as_tensor(gi)).sum().backward()
+        assert orc.rel_l2(gfo, fot.grad.numpy()) < 1e-12 and orc.rel_l2(gwT, wTt.grad.numpy()) < 1e-12
