@@ -1,4 +1,4 @@
-"""pcengine_amd — sparse 3-D convolution inference engine for AMD MI355X (gfx950).
+"""pcengine_amd — sparse 3-D convolution engine for AMD MI355X (gfx950).
 
 Front end with the names of PCEngine's ``script`` package (conv3d, spTensor, BatchNorm, ReLU,
 LeakyReLU, cat, sparse_collate, sparse_quantize, ...) over a hand-written HIP backend reached

@@ -269,7 +269,7 @@ def select_dataflow(km: KernelMap, c_in: int, c_out: int, dtype: torch.dtype, tr
 
 def pack_weights(weight: torch.Tensor) -> Optional[torch.Tensor]:
     """fp16 weights [kv, c_in, c_out] in the order the kernels stage them into LDS (None for fp32).
-    Weights are constants of an inference engine: callers pack once and pass the copy along."""
+    At inference the weights are constants: callers pack once and pass the copy along."""
     lib = _lib.load()
     if weight.dtype != torch.float16:
         return None
