@@ -741,75 +741,87 @@ __global__ void __launch_bounds__(256, ((TMODE >= 0 && sizeof(T) == 2 && NB <= 2
 // straight from the packed copy (8 KB per offset: it stays in cache), so there is no workgroup
 // barrier and wavefronts drift apart, which keeps loads and stores of different wavefronts
 // overlapped.  Chunks [0, pair.items) are pair chunks, the rest rows of the centre GEMM.
-template <int NB, int KS>
-__global__ void __launch_bounds__(256, 5) wave_gemm_kernel(TileArgs pair, TileArgs centre) {
+template <int NB, int KS, int RB>
+__global__ void __launch_bounds__(256, RB == 1 ? 5 : 3) wave_gemm_kernel(TileArgs pair, TileArgs centre) {
   __shared__ __attribute__((aligned(16))) half8 Pl[4][WaveLds<NB>::PIECES];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int l32 = lane & 31, g = lane >> 5;
-  long long chunk = (long long)blockIdx.x * 4 + wave;
+  long long chunk = (long long)blockIdx.x * 4 + wave;   // 32*RB rows (pairs or output rows) per wavefront
   const bool is_pair = chunk < pair.items;
   if (!is_pair && chunk - pair.items >= centre.items) return;
   // features, weights and shapes are those of `pair` for both kinds of chunk; only the destination
   // differs (selecting a whole argument block at run time would copy it to private memory)
   const TileArgs &a = pair;
-  int arow = -1, orow = -1, widx;
+  int arow[RB], orow[RB], widx;
   if (is_pair) {
-    long long q0 = chunk * 32;
+    long long q0 = chunk * (32 * RB);
     widx = 0;
     for (int i = 0; i < pair.kv; ++i) widx += ((long long)pair.qkpos_h[i + 1] <= q0) ? 1 : 0;
     if (widx >= pair.kv) return;
-    long long p = q0 - pair.qkpos_h[widx] + pair.kpos_h[widx] + l32;
-    if (p < (long long)pair.kpos_h[widx + 1]) {
-      arow = pair.imap[p];
-      orow = pair.oslot[p];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      long long p = q0 - pair.qkpos_h[widx] + pair.kpos_h[widx] + rb * 32 + l32;
+      bool ok = p < (long long)pair.kpos_h[widx + 1];
+      arow[rb] = ok ? pair.imap[p] : -1;
+      orow[rb] = ok ? pair.oslot[p] : -1;
     }
   } else {
-    long long row = (chunk - pair.items) * 32 + l32;
     widx = centre.w_fixed;
-    if (row < centre.n_rows) arow = orow = (int)row;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      long long row = (chunk - pair.items) * (32 * RB) + rb * 32 + l32;
+      arow[rb] = orow[rb] = row < centre.n_rows ? (int)row : -1;
+    }
   }
   const half_t *A = (const half_t *)a.A;
   const half_t *Wk = (const half_t *)a.Wp + (long long)widx * a.k8_total * a.n_pad * 8;
-  half8 af[KS], wf[KS][NB];
+  half8 af[RB][KS], wf[KS][NB];
 #pragma unroll
-  for (int s = 0; s < KS; ++s) {
-    half8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (arow >= 0) v = *reinterpret_cast<const half8 *>(A + (long long)arow * a.c_in + s * 16 + g * 8);
-    af[s] = v;
-  }
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      half8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (arow[rb] >= 0) v = *reinterpret_cast<const half8 *>(A + (long long)arow[rb] * a.c_in + s * 16 + g * 8);
+      af[rb][s] = v;
+    }
 #pragma unroll
   for (int s = 0; s < KS; ++s)
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
       wf[s][nb] = *reinterpret_cast<const half8 *>(Wk + ((long long)(2 * s + g) * a.n_pad + nb * 32 + l32) * 8);
-  f32x16 acc[NB];
-#pragma unroll
-  for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-    for (int j = 0; j < 16; ++j) acc[nb][j] = 0.f;
-#pragma unroll
-  for (int s = 0; s < KS; ++s)
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[s][nb], af[s], acc[nb], 0, 0, 0);
-  float V[NB][2][8];
-  gather_row_pieces<NB>(acc, V, g);
   half_t *out = (half_t *)(is_pair ? pair.out : centre.out);
-  if (!is_pair && (centre.bias || centre.res || centre.act)) {
-    // rows that receive partial rows later get their activation from the pass that adds them
-    bool alone = orow >= 0 && centre.ocsr[orow] == centre.ocsr[orow + 1];
-    epilogue_row_pieces<half_t, NB, true>(V, centre, orow, 0, g, false);
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    f32x16 acc[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-      for (int h = 0; h < 2; ++h)
+      for (int j = 0; j < 16; ++j) acc[nb][j] = 0.f;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) V[nb][h][j] = alone ? act_apply(V[nb][h][j], centre.act, centre.slope) : V[nb][h][j];
+    for (int s = 0; s < KS; ++s)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+        acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[s][nb], af[rb][s], acc[nb], 0, 0, 0);
+    float V[NB][2][8];
+    gather_row_pieces<NB>(acc, V, g);
+    if (!is_pair && (centre.bias || centre.res || centre.act)) {
+      // rows that receive partial rows later get their activation from the pass that adds them
+      bool alone = orow[rb] >= 0 && centre.ocsr[orow[rb]] == centre.ocsr[orow[rb] + 1];
+      epilogue_row_pieces<half_t, NB, true>(V, centre, orow[rb], 0, g, false);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) V[nb][h][j] = alone ? act_apply(V[nb][h][j], centre.act, centre.slope) : V[nb][h][j];
+    }
+    store_rows_via_lds<half_t, NB>(V, Pl[wave], out, orow[rb], a, 0, lane, l32, g);
   }
-  store_rows_via_lds<half_t, NB>(V, Pl[wave], out, orow, a, 0, lane, l32, g);
 }
 
-// pair chunks and centre rows of one layer in one launch (either part may be empty)
-static int launch_wave_gemm(const TileArgs &pair, const TileArgs &centre, hipStream_t s) {
+// pair chunks and centre rows of one layer in one launch (either part may be empty); `rb` = 32-row
+// blocks per wavefront, the caller sizes pair.items / centre.items for it
+static int launch_wave_gemm(const TileArgs &pair, const TileArgs &centre, int rb, hipStream_t s) {
   long long chunks = pair.items + centre.items;
   if (chunks <= 0) return PCE_OK;
   if (chunks / 4 >= (1ll << 31) - 8) PCE_FAIL(PCE_ECAPACITY, "chunk count %lld exceeds the grid limit", chunks);
@@ -817,7 +829,10 @@ static int launch_wave_gemm(const TileArgs &pair, const TileArgs &centre, hipStr
   int nb = (pair.c_out + 31) / 32, ks = pair.c_in / 16;  // both blocks come from base_args of one layer
 #define PCE_WAVE_CASE(NB_, KS_)                                                                              \
   if (nb == NB_ && ks == KS_) {                                                                              \
-    hipLaunchKernelGGL((wave_gemm_kernel<NB_, KS_>), dim3(grid), dim3(256), 0, s, pair, centre);             \
+    if (rb == 2)                                                                                             \
+      hipLaunchKernelGGL((wave_gemm_kernel<NB_, KS_, 2>), dim3(grid), dim3(256), 0, s, pair, centre);        \
+    else                                                                                                     \
+      hipLaunchKernelGGL((wave_gemm_kernel<NB_, KS_, 1>), dim3(grid), dim3(256), 0, s, pair, centre);        \
     PCE_LAUNCH_CHECK("wave_gemm");                                                                           \
     return PCE_OK;                                                                                           \
   }
@@ -1613,18 +1628,21 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
     TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
     set_out<T>(&a, buffer, false);
     set_host_pos(&a, kpos_host, qkpos_host);
+    // 64 rows per wavefront once there are enough of them to keep every CU busy: the weight fragments are
+    // fetched once per two row blocks and the first block's stores overlap the second block's arithmetic
+    const int rb = (qsum / 32 + pce_div_up(n_out, 32)) >= 16 * 256 ? 2 : 1;
     a.imap = imap;
     a.oslot = oslot;
-    a.items = qsum / 32;
+    a.items = qsum / (32 * rb);
     TileArgs c = base_args<T>(in, w, wp, kv, c_in, c_out);
     set_out<T>(&c, out, false);
     c.w_fixed = mid;
     c.n_rows = n_out;
-    c.items = pce_div_up(n_out, 32);
+    c.items = pce_div_up(n_out, 32 * rb);
     c.ocsr = ocsr;
     set_epi(&c, e);
     if (a.host_pos && wave_gemm_ok(a, sizeof(T)) && wave_gemm_ok(c, sizeof(T)) && aligned16(buffer) && epi_aligned(e)) {
-      if (stage_on(1) && (rc = launch_wave_gemm(a, c, s))) return rc;
+      if (stage_on(1) && (rc = launch_wave_gemm(a, c, rb, s))) return rc;
       if (stage_on(2) && (rc = launch_rowsum_pairs<T>((const T *)buffer, (T *)out, n_out, n_pairs, c_out, omap, oslot, ocsr,
                                                       e.act, e.slope, s)))
         return rc;
@@ -1645,7 +1663,7 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
       TileArgs none = a;
       none.items = 0;
       a.items = qsum / 32;
-      if ((rc = launch_wave_gemm(a, none, s))) return rc;
+      if ((rc = launch_wave_gemm(a, none, 1, s))) return rc;
     } else if ((rc = launch_tile<T>(a, qsum / PCE_QUANTUM, s))) {
       return rc;
     }
