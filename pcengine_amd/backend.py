@@ -109,6 +109,13 @@ class KernelMap:
         return self._as_list()[i]
 
 
+@dataclass
+class PendingMap:
+    """A map build whose kernels are queued but whose counts have not been read back yet."""
+    out_coords: torch.Tensor
+    finish: object      # () -> KernelMap, valid after the stream of the build has been synchronised
+
+
 def strided_coords_max(cmax, ks, stride, pad):
     """script/spconv.py:358-360."""
     return [(int(cmax[a]) + 2 * pad[a] - (ks[a] - 1)) // stride[a] for a in range(3)]
@@ -180,10 +187,13 @@ def voxelize(points: torch.Tensor, voxel_size, batch_index: int = 0, return_inde
 
 def build_kernel_map(in_coords: torch.Tensor, ks, stride, pad, cmin, cmax_out, subm: bool,
                      want_csr: bool = False, want_nbr_out: bool = True, want_nbr_in: bool = False,
-                     out_coords: Optional[torch.Tensor] = None, batchsize: int = 0) -> KernelMap:
+                     out_coords: Optional[torch.Tensor] = None, batchsize: int = 0, defer: bool = False):
     """Hash the output coordinates, probe every (input row, offset) and emit the canonical map.
 
-    ``cmax_out`` is the bound on output coordinates (already reduced for strided layers)."""
+    ``cmax_out`` is the bound on output coordinates (already reduced for strided layers).
+    ``defer=True`` returns a ``PendingMap`` instead of waiting for the pair counts: its output
+    coordinates are final, ``finish()`` yields the ``KernelMap`` once the stream has been
+    synchronised.  A network uses it to queue the builds of all its layers behind each other."""
     lib = _lib.load()
     _require_cuda(in_coords, "coords")
     if in_coords.dtype != torch.int32 or in_coords.dim() != 2 or in_coords.shape[1] != 4:
@@ -221,25 +231,34 @@ def build_kernel_map(in_coords: torch.Tensor, ks, stride, pad, cmin, cmax_out, s
                                   pairs[0].data_ptr(), pairs[1].data_ptr(), knnz.data_ptr(), kpos.data_ptr(),
                                   qkpos.data_ptr(), _ptr(icsr), _ptr(icode), _ptr(ocsr), _ptr(ocode), _ptr(islot),
                                   _ptr(oslot), _ptr(nbr_out), _ptr(nbr_in), status.data_ptr(), s))
-    host = meta.cpu().tolist()   # the one synchronisation of a map build
-    st = host[3 * kv + 2:]
-    if st[0]:
-        raise ValueError(f"a coordinate is outside the supported range (|c| < {32000}, batch < 32768)")
-    if st[1]:
-        raise _lib.PCEError("hash table exhausted while building the kernel map")
-    if want_csr and st[2]:
-        raise OverflowError(f"an offset holds >= {CSR_CODE} pairs: the CSR code of the gather-GEMM-scatter map overflows")
-    M, qsum = host[2 * kv], host[3 * kv + 1]
-    km = KernelMap(ks=tuple(ks), stride=tuple(stride), pad=tuple(pad), subm=bool(subm), n_in=n_in, n_out=n_out, kv=kv,
-                   M=M, qsum=qsum, imap=pairs[0, :M], omap=pairs[1, :M], knnz=knnz, kpos=kpos, qkpos=qkpos,
-                   out_coords=out_coords, nbr_out=nbr_out, nbr_in=nbr_in, icsr=icsr, ocsr=ocsr,
-                   icode=None if icode is None else icode[:M], ocode=None if ocode is None else ocode[:M],
-                   islot=None if islot is None else islot[:M], oslot=None if oslot is None else oslot[:M],
-                   in_coords=in_coords, geom=geom, knnz_host=host[:kv])
-    km._cmin, km._cmax = list(cmin), list(cmax_out)
-    km.kpos_host = (_lib.c_int32 * (kv + 1))(*host[kv:2 * kv + 1])
-    km.qkpos_host = (_lib.c_int32 * (kv + 1))(*host[2 * kv + 1:3 * kv + 2])
-    return km
+
+    def finish(host: list) -> KernelMap:
+        st = host[3 * kv + 2:]
+        if st[0]:
+            raise ValueError(f"a coordinate is outside the supported range (|c| < {32000}, batch < 32768)")
+        if st[1]:
+            raise _lib.PCEError("hash table exhausted while building the kernel map")
+        if want_csr and st[2]:
+            raise OverflowError(f"an offset holds >= {CSR_CODE} pairs: the CSR code of the gather-GEMM-scatter map overflows")
+        M, qsum = host[2 * kv], host[3 * kv + 1]
+        km = KernelMap(ks=tuple(ks), stride=tuple(stride), pad=tuple(pad), subm=bool(subm), n_in=n_in, n_out=n_out, kv=kv,
+                       M=M, qsum=qsum, imap=pairs[0, :M], omap=pairs[1, :M], knnz=knnz, kpos=kpos, qkpos=qkpos,
+                       out_coords=out_coords, nbr_out=nbr_out, nbr_in=nbr_in, icsr=icsr, ocsr=ocsr,
+                       icode=None if icode is None else icode[:M], ocode=None if ocode is None else ocode[:M],
+                       islot=None if islot is None else islot[:M], oslot=None if oslot is None else oslot[:M],
+                       in_coords=in_coords, geom=geom, knnz_host=host[:kv])
+        km._cmin, km._cmax = list(cmin), list(cmax_out)
+        km.kpos_host = (_lib.c_int32 * (kv + 1))(*host[kv:2 * kv + 1])
+        km.qkpos_host = (_lib.c_int32 * (kv + 1))(*host[2 * kv + 1:3 * kv + 2])
+        return km
+
+    if defer:
+        # the counts travel to pinned host memory behind the build's kernels; the caller synchronises the
+        # stream once for several builds and then calls finish() on each
+        meta_host = torch.empty(meta.shape, dtype=torch.int32, pin_memory=True)
+        meta_host.copy_(meta, non_blocking=True)
+        return PendingMap(out_coords=out_coords, finish=lambda: finish(meta_host.tolist()))
+    return finish(meta.cpu().tolist())   # the one synchronisation of a map build
 
 
 def ensure_csr(km: KernelMap) -> None:

@@ -232,12 +232,8 @@ def _run(input: spTensor, km: backend.KernelMap, kernel, in_channel, out_channel
     return out
 
 
-def ensure_map(input: spTensor, kernel_size_code: int, stride_code: int, padding_code: int):
-    """Kernel map of a (non-transposed) layer on this tensor: looked up in the shared cache or built
-    and stored there (script/spconv.py:331-437).  Returns (map, output tensor stride, output
-    coords_min, output coords_max).  Maps depend on coordinates only, so a network can call this for
-    all its layers before the first convolution: the host then never waits for the device between
-    layers (see ``prebuild_maps``)."""
+def _map_request(input: spTensor, kernel_size_code: int, stride_code: int, padding_code: int, defer: bool):
+    """Cache lookup, or the build (finished, or queued when ``defer``), of one layer's map."""
     output_stride = output_stride_compute(stride_code, input.stride, 0)
     key = (kernel_size_code, input.stride, stride_code)
     km = input.kmaps.get(key)
@@ -249,6 +245,7 @@ def ensure_map(input: spTensor, kernel_size_code: int, stride_code: int, padding
     pad = conv_info_decoder(padding_code)
     if not subm:
         coords_max = backend.strided_coords_max(input.coords_max, ks, stride, pad)   # script/spconv.py:358-360
+    tag = None
     if km is None:
         tag = input.init_tag[0] if input.init_tag else 'end'
         if tag not in ('D1', 'D2', 'end', 'auto'):
@@ -256,12 +253,26 @@ def ensure_map(input: spTensor, kernel_size_code: int, stride_code: int, padding
         auto = tag in ('end', 'auto')
         km = backend.build_kernel_map(input.coords, ks, stride, pad, coords_min, coords_max, subm,
                                       want_csr=(tag == 'D1' or auto), want_nbr_out=auto, want_nbr_in=auto and not subm,
-                                      batchsize=input.batchsize)
-        km.tag = tag if tag in ('D1', 'D2') else 'auto'
-        input.kmaps[key] = km
-        input.cbook[output_stride] = km.out_coords
+                                      batchsize=input.batchsize, defer=defer)
         if tag in ('D1', 'D2'):
             input.init_tag = input.init_tag[1:]
+    return km, key, tag, output_stride, coords_min, coords_max
+
+
+def _map_store(input: spTensor, km: backend.KernelMap, key, tag, output_stride) -> None:
+    km.tag = tag if tag in ('D1', 'D2') else 'auto'
+    input.kmaps[key] = km
+    input.cbook[output_stride] = km.out_coords
+
+
+def ensure_map(input: spTensor, kernel_size_code: int, stride_code: int, padding_code: int):
+    """Kernel map of a (non-transposed) layer on this tensor: looked up in the shared cache or built
+    and stored there (script/spconv.py:331-437).  Returns (map, output tensor stride, output
+    coords_min, output coords_max).  Maps depend on coordinates only, so a network can ask for all of
+    them before the first convolution (``prebuild_maps``)."""
+    km, key, tag, output_stride, coords_min, coords_max = _map_request(input, kernel_size_code, stride_code, padding_code, False)
+    if tag is not None:
+        _map_store(input, km, key, tag, output_stride)
     input.cbook.setdefault(input.stride, input.coords)
     return km, output_stride, coords_min, coords_max
 
@@ -270,19 +281,29 @@ def prebuild_maps(input: spTensor, layers) -> None:
     """Build, ahead of any convolution, the maps a network will ask for.  ``layers`` lists
     (kernel_size, stride, padding) in network order (ints or triples; transposed layers and 1x1
     layers need no entry); a strided entry moves on to its output coordinates, as the network does.
-    Every map build reads two counters back from the device: done here, with no convolution queued,
-    those waits are short, and the layers that follow find every map in the cache."""
+    The builds are queued behind each other and their pair counts are read back together after one
+    synchronisation (only the output coordinates of a strided layer have to reach the host in
+    between, for their number), so the device does not idle between the ~17 small kernels of each build
+    and the layers that follow find every map in the cache."""
     x = input
+    pending = []
     for ks, stride, pad in layers:
         ksc, sc, pc = (conv_info_encoder(_triple(v, "layer")) for v in (ks, stride, pad))
         if ksc == _UNIT and sc == _UNIT:
             continue
-        km, out_stride, cmin, cmax = ensure_map(x, ksc, sc, pc)
+        km, key, tag, out_stride, cmin, cmax = _map_request(x, ksc, sc, pc, True)
+        if tag is not None:
+            pending.append((x, km, key, tag, out_stride))
+        x.cbook.setdefault(x.stride, x.coords)
         if sc != _UNIT:
             nxt = spTensor(feats=x.feats, coords=km.out_coords, buffer=x.buffer, batchsize=x.batchsize, stride=out_stride,
                            init_tag=x.init_tag, coords_max=cmax, coords_min=cmin)
             nxt.kmaps, nxt.cbook = x.kmaps, x.cbook
             x = nxt
+    if pending:
+        torch.cuda.current_stream(input.coords.device).synchronize()
+        for t, pm, key, tag, out_stride in pending:
+            _map_store(t, pm.finish(), key, tag, out_stride)
 
 
 def conv_func(input: spTensor, in_channel, out_channel, kernel, kernel_size_code, stride_code, padding_code, bias,
