@@ -162,6 +162,31 @@ int pce_kmap_build(const int32_t *in_coords_dev, int64_t n_in, const int32_t *ou
                    int32_t *ocode_dev, int32_t *islot_dev, int32_t *oslot_dev, int32_t *nbr_out_dev,
                    int32_t *nbr_in_dev, int32_t *status_dev, pce_stream_t stream);
 
+/* The maps of several layers in one call (a network needs one per distinct layer geometry of a
+ * point cloud: script/spconv.py:330-372 runs once per such layer).  Every stage of the build is
+ * one launch shared by all problems of the batch, so a batch costs the launches of one build.
+ * Each problem carries the arguments of pce_kmap_build with the same meaning and its own
+ * workspace; the problems must not share outputs or workspaces, and the output coordinates of
+ * every problem must be complete before the call.  At most PCE_KMAP_MAX_BATCH problems.
+ * The call queues one small host-to-device copy (the descriptors of the batch, from pinned memory
+ * the library keeps) ahead of its kernels and does not wait for the stream. */
+#define PCE_KMAP_MAX_BATCH 16
+typedef struct pce_kmap_problem {
+  const int32_t *in_coords;
+  int64_t n_in;
+  const int32_t *out_coords;
+  int64_t n_out;
+  pce_geom_t geom;
+  void *ws;
+  int64_t ws_bytes;
+  int32_t *imap, *omap, *knnz, *kpos, *qkpos;
+  int32_t *icsr, *icode, *ocsr, *ocode; /* all four or none */
+  int32_t *islot, *oslot;               /* optional, with the CSR outputs */
+  int32_t *nbr_out, *nbr_in;            /* optional */
+  int32_t *status;                      /* int32[4] per problem, zeroed by the caller */
+} pce_kmap_problem_t;
+int pce_kmap_build_batch(const pce_kmap_problem_t *problems_host, int32_t n_problems, pce_stream_t stream);
+
 /* ---- forward convolution --------------------------------------------------------------------- *
  * Common arguments: in_feats[n_in,c_in], weight[kv,c_in,c_out], out_feats[n_out,c_out], all of
  * `dtype` (PCE_F16: fp16 storage, fp32 accumulate; PCE_F32), row-major, device.

@@ -34,6 +34,14 @@ class Geom(Structure):
         return g
 
 
+class KmapProblem(Structure):
+    """pce_kmap_problem_t: the arguments of one kernel-map build inside a batch."""
+    _fields_ = ([("in_coords", c_void_p), ("n_in", c_int64), ("out_coords", c_void_p), ("n_out", c_int64),
+                 ("geom", Geom), ("ws", c_void_p), ("ws_bytes", c_int64)] +
+                [(name, c_void_p) for name in ("imap", "omap", "knnz", "kpos", "qkpos", "icsr", "icode", "ocsr", "ocode",
+                                               "islot", "oslot", "nbr_out", "nbr_in", "status")])
+
+
 class Epilogue(Structure):
     """pce_epilogue_t: out = act(conv + bias + residual)."""
     _fields_ = [("bias", c_void_p), ("residual", c_void_p), ("act", c_int32), ("slope", ctypes.c_float)]
@@ -63,6 +71,7 @@ _SIGNATURES = {
     "pce_voxelize_emit": (c_int32, [c_void_p, c_int64, c_int64, POINTER(c_int32), POINTER(c_int32), c_int32, c_void_p, c_void_p,
                                     c_void_p, c_void_p]),
     "pce_kmap_workspace_bytes": (c_int64, [c_int64, c_int64, c_int32, c_int32]),
+    "pce_kmap_build_batch": (c_int32, [POINTER(KmapProblem), c_int32, c_void_p]),
     "pce_kmap_build": (c_int32, [c_void_p, c_int64, c_void_p, c_int64, POINTER(Geom), c_void_p, c_int64] + [c_void_p] * 14 + [c_void_p]),
     "pce_conv_fod_workspace_bytes": (c_int64, [c_int64, c_int32, c_int32]),
     "pce_packed_weight_bytes": (c_int64, [c_int32, c_int32, c_int32, c_int32]),

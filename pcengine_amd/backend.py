@@ -14,7 +14,7 @@ Torch is used for device memory and the current stream only.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Optional, Sequence, Tuple
+from typing import List, Optional, Sequence, Tuple
 
 import torch
 
@@ -185,6 +185,146 @@ def voxelize(points: torch.Tensor, voxel_size, batch_index: int = 0, return_inde
     return tuple(outs)
 
 
+class _MapJob:
+    """One kernel-map build between its preparation (outputs allocated, arguments laid out) and the
+    read-back of its counts."""
+
+    def __init__(self, in_coords, ks, stride, pad, cmin, cmax_out, subm, want_csr, want_nbr_out, want_nbr_in,
+                 out_coords, batchsize):
+        lib = _lib.load()
+        _require_cuda(in_coords, "coords")
+        if in_coords.dtype != torch.int32 or in_coords.dim() != 2 or in_coords.shape[1] != 4:
+            raise ValueError("coords must be int32 [N, 4] = (b, x, y, z)")
+        in_coords = in_coords.contiguous()
+        dev = in_coords.device
+        n_in = in_coords.shape[0]
+        kv = int(ks[0]) * int(ks[1]) * int(ks[2])
+        geom = Geom.make(ks, stride, pad, cmin, cmax_out, subm)
+        if subm:
+            out_coords = in_coords
+        elif out_coords is None:
+            out_coords = build_out_coords(in_coords, geom, batchsize)
+        n_out = out_coords.shape[0]
+        if n_in == 0 or n_out == 0:
+            raise ValueError(f"empty sparse tensor (n_in={n_in}, n_out={n_out})")
+        self.args = (tuple(ks), tuple(stride), tuple(pad), list(cmin), list(cmax_out), bool(subm))
+        self.in_coords, self.out_coords, self.geom = in_coords, out_coords, geom
+        self.n_in, self.n_out, self.kv, self.want_csr, self.dev = n_in, n_out, kv, bool(want_csr), dev
+        self.meta_len = kv + 2 * (kv + 1) + 4      # knnz | kpos | qkpos | status
+        self.ws_bytes = lib.pce_kmap_workspace_bytes(n_in, n_out, kv, int(want_csr))
+        self.ws = torch.empty(self.ws_bytes, dtype=torch.uint8, device=dev)
+        self.pairs = torch.empty((2, kv * n_in), dtype=torch.int32, device=dev)
+        self.nbr_out = torch.empty(kv * n_out, dtype=torch.int32, device=dev) if want_nbr_out else None
+        self.nbr_in = torch.empty(kv * n_in, dtype=torch.int32, device=dev) if want_nbr_in else None
+        if want_csr:
+            # icsr | ocsr | icode | ocode | islot | oslot in one allocation
+            cap = kv * n_in
+            buf = torch.empty(n_in + 1 + n_out + 1 + 4 * cap, dtype=torch.int32, device=dev)
+            self.icsr, self.ocsr = buf[:n_in + 1], buf[n_in + 1:n_in + n_out + 2]
+            codes = buf[n_in + n_out + 2:].view(4, cap)
+            self.icode, self.ocode, self.islot, self.oslot = codes[0], codes[1], codes[2], codes[3]
+        else:
+            self.icsr = self.ocsr = self.icode = self.ocode = self.islot = self.oslot = None
+
+    def problem(self, meta: torch.Tensor) -> "_lib.KmapProblem":
+        """``meta`` is this job's zeroed slice of the batch's count tensor."""
+        kv = self.kv
+        self.knnz, self.kpos, self.qkpos = meta[:kv], meta[kv:2 * kv + 1], meta[2 * kv + 1:3 * kv + 2]
+        status = meta[3 * kv + 2:]
+        p = _lib.KmapProblem()
+        p.in_coords, p.n_in = self.in_coords.data_ptr(), self.n_in
+        p.out_coords, p.n_out = self.out_coords.data_ptr(), self.n_out
+        p.geom = self.geom
+        p.ws, p.ws_bytes = self.ws.data_ptr(), self.ws_bytes
+        p.imap, p.omap = self.pairs[0].data_ptr(), self.pairs[1].data_ptr()
+        p.knnz, p.kpos, p.qkpos = self.knnz.data_ptr(), self.kpos.data_ptr(), self.qkpos.data_ptr()
+        p.icsr, p.icode, p.ocsr, p.ocode = _ptr(self.icsr), _ptr(self.icode), _ptr(self.ocsr), _ptr(self.ocode)
+        p.islot, p.oslot = _ptr(self.islot), _ptr(self.oslot)
+        p.nbr_out, p.nbr_in = _ptr(self.nbr_out), _ptr(self.nbr_in)
+        p.status = status.data_ptr()
+        return p
+
+    def finish(self, host: list) -> KernelMap:
+        kv, M = self.kv, None
+        st = host[3 * kv + 2:]
+        if st[0]:
+            raise ValueError(f"a coordinate is outside the supported range (|c| < {32000}, batch < 32768)")
+        if st[1]:
+            raise _lib.PCEError("hash table exhausted while building the kernel map")
+        if self.want_csr and st[2]:
+            raise OverflowError(f"an offset holds >= {CSR_CODE} pairs: the CSR code of the gather-GEMM-scatter map overflows")
+        M, qsum = host[2 * kv], host[3 * kv + 1]
+        ks, stride, pad, cmin, cmax_out, subm = self.args
+        cut = lambda t: None if t is None else t[:M]
+        km = KernelMap(ks=ks, stride=stride, pad=pad, subm=subm, n_in=self.n_in, n_out=self.n_out, kv=kv,
+                       M=M, qsum=qsum, imap=self.pairs[0, :M], omap=self.pairs[1, :M], knnz=self.knnz, kpos=self.kpos,
+                       qkpos=self.qkpos, out_coords=self.out_coords, nbr_out=self.nbr_out, nbr_in=self.nbr_in,
+                       icsr=self.icsr, ocsr=self.ocsr, icode=cut(self.icode), ocode=cut(self.ocode),
+                       islot=cut(self.islot), oslot=cut(self.oslot), in_coords=self.in_coords, geom=self.geom,
+                       knnz_host=host[:kv])
+        km._cmin, km._cmax = cmin, cmax_out
+        km.kpos_host = (_lib.c_int32 * (kv + 1))(*host[kv:2 * kv + 1])
+        km.qkpos_host = (_lib.c_int32 * (kv + 1))(*host[2 * kv + 1:3 * kv + 2])
+        return km
+
+
+KMAP_MAX_BATCH = 16
+
+
+def prepare_map(in_coords: torch.Tensor, ks, stride, pad, cmin, cmax_out, subm: bool, want_csr: bool = False,
+                want_nbr_out: bool = True, want_nbr_in: bool = False, out_coords: Optional[torch.Tensor] = None,
+                batchsize: int = 0) -> _MapJob:
+    """First half of a map build: the output coordinates of a strided layer (``.out_coords``, final)
+    and the output buffers.  ``build_kernel_maps`` takes the result in place of a request."""
+    return _MapJob(in_coords, ks, stride, pad, cmin, cmax_out, subm, want_csr, want_nbr_out, want_nbr_in, out_coords,
+                   batchsize)
+
+
+def build_kernel_maps(requests: List[dict], defer: bool = False):
+    """Build the kernel maps of several layers with the launches of one build.
+
+    Every request holds the keyword arguments of ``build_kernel_map`` (without ``defer``), or is the
+    result of ``prepare_map`` on them.  The
+    output coordinates of strided layers are computed first, request by request; the builds then
+    run as batches of up to ``KMAP_MAX_BATCH`` problems, each stage one launch over the whole
+    batch, and the counts of all maps come back in one copy.  ``defer=True`` returns
+    ``PendingMap`` objects whose ``finish()`` may be called once the stream has been synchronised."""
+    lib = _lib.load()
+    jobs = [r if isinstance(r, _MapJob) else prepare_map(**r) for r in requests]
+    if not jobs:
+        return []
+    dev = jobs[0].dev
+    if any(j.dev != dev for j in jobs):
+        raise ValueError("the maps of one batch live on one device")
+    s = _stream(dev)
+    starts = [0]
+    for j in jobs:
+        starts.append(starts[-1] + j.meta_len)
+    # the counts and status words of every map in one tensor: a single device->host copy reads them all
+    meta = torch.zeros(starts[-1], dtype=torch.int32, device=dev)
+    for b0 in range(0, len(jobs), KMAP_MAX_BATCH):
+        chunk = jobs[b0:b0 + KMAP_MAX_BATCH]
+        probs = (_lib.KmapProblem * len(chunk))(*[j.problem(meta[starts[b0 + k]:starts[b0 + k + 1]])
+                                                  for k, j in enumerate(chunk)])
+        _lib.check(lib.pce_kmap_build_batch(probs, len(chunk), s))
+    if defer:
+        # the counts travel to pinned host memory behind the kernels; the caller synchronises the stream
+        # once and then calls finish() on each
+        meta_host = torch.empty(meta.shape, dtype=torch.int32, pin_memory=True)
+        meta_host.copy_(meta, non_blocking=True)
+        cache = {}
+
+        def finisher(k):
+            def fin():
+                if "host" not in cache:
+                    cache["host"] = meta_host.tolist()
+                return jobs[k].finish(cache["host"][starts[k]:starts[k + 1]])
+            return fin
+        return [PendingMap(out_coords=j.out_coords, finish=finisher(k)) for k, j in enumerate(jobs)]
+    host = meta.cpu().tolist()   # the one synchronisation of the builds
+    return [j.finish(host[starts[k]:starts[k + 1]]) for k, j in enumerate(jobs)]
+
+
 def build_kernel_map(in_coords: torch.Tensor, ks, stride, pad, cmin, cmax_out, subm: bool,
                      want_csr: bool = False, want_nbr_out: bool = True, want_nbr_in: bool = False,
                      out_coords: Optional[torch.Tensor] = None, batchsize: int = 0, defer: bool = False):
@@ -193,72 +333,10 @@ def build_kernel_map(in_coords: torch.Tensor, ks, stride, pad, cmin, cmax_out, s
     ``cmax_out`` is the bound on output coordinates (already reduced for strided layers).
     ``defer=True`` returns a ``PendingMap`` instead of waiting for the pair counts: its output
     coordinates are final, ``finish()`` yields the ``KernelMap`` once the stream has been
-    synchronised.  A network uses it to queue the builds of all its layers behind each other."""
-    lib = _lib.load()
-    _require_cuda(in_coords, "coords")
-    if in_coords.dtype != torch.int32 or in_coords.dim() != 2 or in_coords.shape[1] != 4:
-        raise ValueError("coords must be int32 [N, 4] = (b, x, y, z)")
-    in_coords = in_coords.contiguous()
-    dev = in_coords.device
-    n_in = in_coords.shape[0]
-    kv = int(ks[0]) * int(ks[1]) * int(ks[2])
-    geom = Geom.make(ks, stride, pad, cmin, cmax_out, subm)
-    if subm:
-        out_coords = in_coords
-    elif out_coords is None:
-        out_coords = build_out_coords(in_coords, geom, batchsize)
-    n_out = out_coords.shape[0]
-    if n_in == 0 or n_out == 0:
-        raise ValueError(f"empty sparse tensor (n_in={n_in}, n_out={n_out})")
-    s = _stream(dev)
-    ws_bytes = lib.pce_kmap_workspace_bytes(n_in, n_out, kv, int(want_csr))
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-    pairs = torch.empty((2, kv * n_in), dtype=torch.int32, device=dev)
-    # knnz | kpos | qkpos | status in one tensor: a single device->host copy reads all of them
-    meta = torch.zeros(kv + 2 * (kv + 1) + 4, dtype=torch.int32, device=dev)
-    knnz, kpos, qkpos = meta[:kv], meta[kv:2 * kv + 1], meta[2 * kv + 1:3 * kv + 2]
-    status = meta[3 * kv + 2:]
-    nbr_out = torch.empty(kv * n_out, dtype=torch.int32, device=dev) if want_nbr_out else None
-    nbr_in = torch.empty(kv * n_in, dtype=torch.int32, device=dev) if want_nbr_in else None
-    if want_csr:
-        icsr = torch.empty(n_in + 1, dtype=torch.int32, device=dev)
-        ocsr = torch.empty(n_out + 1, dtype=torch.int32, device=dev)
-        codes = torch.empty((4, kv * n_in), dtype=torch.int32, device=dev)
-        icode, ocode, islot, oslot = codes[0], codes[1], codes[2], codes[3]
-    else:
-        icsr = ocsr = icode = ocode = islot = oslot = None
-    _lib.check(lib.pce_kmap_build(in_coords.data_ptr(), n_in, out_coords.data_ptr(), n_out, geom, ws.data_ptr(), ws_bytes,
-                                  pairs[0].data_ptr(), pairs[1].data_ptr(), knnz.data_ptr(), kpos.data_ptr(),
-                                  qkpos.data_ptr(), _ptr(icsr), _ptr(icode), _ptr(ocsr), _ptr(ocode), _ptr(islot),
-                                  _ptr(oslot), _ptr(nbr_out), _ptr(nbr_in), status.data_ptr(), s))
-
-    def finish(host: list) -> KernelMap:
-        st = host[3 * kv + 2:]
-        if st[0]:
-            raise ValueError(f"a coordinate is outside the supported range (|c| < {32000}, batch < 32768)")
-        if st[1]:
-            raise _lib.PCEError("hash table exhausted while building the kernel map")
-        if want_csr and st[2]:
-            raise OverflowError(f"an offset holds >= {CSR_CODE} pairs: the CSR code of the gather-GEMM-scatter map overflows")
-        M, qsum = host[2 * kv], host[3 * kv + 1]
-        km = KernelMap(ks=tuple(ks), stride=tuple(stride), pad=tuple(pad), subm=bool(subm), n_in=n_in, n_out=n_out, kv=kv,
-                       M=M, qsum=qsum, imap=pairs[0, :M], omap=pairs[1, :M], knnz=knnz, kpos=kpos, qkpos=qkpos,
-                       out_coords=out_coords, nbr_out=nbr_out, nbr_in=nbr_in, icsr=icsr, ocsr=ocsr,
-                       icode=None if icode is None else icode[:M], ocode=None if ocode is None else ocode[:M],
-                       islot=None if islot is None else islot[:M], oslot=None if oslot is None else oslot[:M],
-                       in_coords=in_coords, geom=geom, knnz_host=host[:kv])
-        km._cmin, km._cmax = list(cmin), list(cmax_out)
-        km.kpos_host = (_lib.c_int32 * (kv + 1))(*host[kv:2 * kv + 1])
-        km.qkpos_host = (_lib.c_int32 * (kv + 1))(*host[2 * kv + 1:3 * kv + 2])
-        return km
-
-    if defer:
-        # the counts travel to pinned host memory behind the build's kernels; the caller synchronises the
-        # stream once for several builds and then calls finish() on each
-        meta_host = torch.empty(meta.shape, dtype=torch.int32, pin_memory=True)
-        meta_host.copy_(meta, non_blocking=True)
-        return PendingMap(out_coords=out_coords, finish=lambda: finish(meta_host.tolist()))
-    return finish(meta.cpu().tolist())   # the one synchronisation of a map build
+    synchronised."""
+    return build_kernel_maps([dict(in_coords=in_coords, ks=ks, stride=stride, pad=pad, cmin=cmin, cmax_out=cmax_out,
+                                   subm=subm, want_csr=want_csr, want_nbr_out=want_nbr_out, want_nbr_in=want_nbr_in,
+                                   out_coords=out_coords, batchsize=batchsize)], defer=defer)[0]
 
 
 def ensure_csr(km: KernelMap) -> None:

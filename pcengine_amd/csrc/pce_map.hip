@@ -7,6 +7,8 @@
 #include <stdarg.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "pce_common.h"
 
 // ------------------------------------------------------------------------------------------------
@@ -922,9 +924,16 @@ extern "C" int pce_voxelize_emit(const void *ws, int64_t n_points, int64_t n_vox
 // ------------------------------------------------------------------------------------------------
 // kernel map
 // ------------------------------------------------------------------------------------------------
+// One build call serves a batch of layers: every stage is ONE launch whose workgroups are dealt to the
+// problems of the batch (a build is ~12 small kernels, most of them at the few-microsecond floor of a
+// launch; a network needs nine maps per point cloud).  The problem descriptors, the work lists of the
+// stages and the lists of arrays to fill and to scan travel to the device in one copy.
+#define PCE_MAX_BATCH PCE_KMAP_MAX_BATCH
+#define KMAP_DESC_BYTES 32768  // descriptor area at the end of every kernel-map workspace
+
 struct KmapLayout {
   int64_t slots, nseg, scan_len;
-  int64_t off_table, off_dense, off_seg, off_scan, off_orank, off_irank, total;
+  int64_t off_table, off_dense, off_seg, off_scan, off_orank, off_irank, off_desc, total;
 };
 
 static void kmap_layout(int64_t n_in, int64_t n_out, int kv, int want_csr, int subm, KmapLayout *L) {
@@ -944,7 +953,82 @@ static void kmap_layout(int64_t n_in, int64_t n_out, int kv, int want_csr, int s
   if (want_csr && !subm) o += pce_align_up((int64_t)kv * n_out * 4, 256);
   L->off_irank = o;
   if (want_csr) o += pce_align_up((int64_t)kv * n_in * 4, 256);
+  L->off_desc = o;
+  o += KMAP_DESC_BYTES;
   L->total = o;
+}
+
+// device-side view of one problem of the batch
+struct ProbDev {
+  const int4 *in_coords, *out_coords;
+  long long n_in, n_out, nseg;
+  GeomDev g;
+  pce_slot_t *table;
+  unsigned long long slots;
+  int *dense, *irank, *orank, *seg;
+  int *imap, *omap, *knnz, *kpos, *qkpos, *icsr, *icode, *ocsr, *ocode, *islot, *oslot, *nbr_out, *status;
+  int want_csr;
+};
+
+// a contiguous range of workgroups of one launch: workgroups [blk0, next job's blk0) work on `prob`
+struct Job {
+  unsigned blk0;
+  int prob;
+  int kind;
+  int pad;
+};
+enum { JOB_CSR_SUBM = 0, JOB_CSR_IN = 1, JOB_CSR_COUNT_OUT = 2, JOB_CSR_OUT = 3 };
+
+struct FillRegion {
+  unsigned *p;
+  long long n_words;
+  unsigned blk0;
+  unsigned pad;
+};
+
+struct ScanArr {
+  int *data;
+  long long n;
+  int *sums;  // one int per tile of this array
+  unsigned blk0;
+  unsigned pad;
+};
+
+struct JobList {
+  const Job *jobs;
+  int n;
+};
+
+__device__ __forceinline__ const Job &find_job(const JobList &l, unsigned b) {
+  int j = 0;
+  while (j + 1 < l.n && b >= l.jobs[j + 1].blk0) ++j;
+  return l.jobs[j];
+}
+
+#define FILL_WORDS_PER_BLOCK (256 * 8)
+__global__ void __launch_bounds__(256) multi_fill_kernel(const FillRegion *__restrict__ regs, int n_regs, unsigned value) {
+  int r = 0;
+  while (r + 1 < n_regs && blockIdx.x >= regs[r + 1].blk0) ++r;
+  const FillRegion reg = regs[r];
+  long long base = (long long)(blockIdx.x - reg.blk0) * FILL_WORDS_PER_BLOCK;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    long long i = base + k * 256 + threadIdx.x;
+    if (i < reg.n_words) reg.p[i] = value;
+  }
+}
+
+__global__ void __launch_bounds__(256) batch_insert_kernel(const ProbDev *__restrict__ P, JobList jl) {
+  const Job &job = find_job(jl, blockIdx.x);
+  const ProbDev &q = P[job.prob];
+  long long i = (long long)(blockIdx.x - job.blk0) * blockDim.x + threadIdx.x;
+  if (i >= q.n_out) return;
+  int4 c = q.out_coords[i];
+  if (!pce_coord_ok(c.x, c.y, c.z, c.w)) {
+    q.status[0] = 1;
+    return;
+  }
+  if (!table_insert(q.table, q.slots, pce_pack_key(c.x, c.y, c.z, c.w), (unsigned)i, nullptr)) q.status[1] = 1;
 }
 
 // Probe batches: the first-probe loads of PROBE_BATCH offsets are issued together, then resolved;
@@ -957,17 +1041,21 @@ static void kmap_layout(int64_t n_in, int64_t n_out, int kv, int want_csr, int s
 //   strided:     out = (in - d(kp) + pad) / stride when it divides
 // dense[kp*n_in + i] = output row or -1.
 // A submanifold map is symmetric: pair (i,o,kp) <=> pair (o,i,kv-1-kp).  Only the offsets below the
-// centre are probed; a hit also writes the mirrored entry dense[(kv-1-kp)*n + o] = i.  The caller
-// pre-fills the rows of dense from the centre upwards with -1.
-__global__ void __launch_bounds__(256) kmap_query_kernel(const int4 *__restrict__ in_coords, long long n_in, GeomDev g,
-                                                         const pce_slot_t *__restrict__ table,
-                                                         unsigned long long slots, int *__restrict__ dense,
-                                                         int *status) {
-  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+// centre are probed; a hit also writes the mirrored entry dense[(kv-1-kp)*n + o] = i.  The rows of
+// dense from the centre upwards are pre-filled with -1.
+__global__ void __launch_bounds__(256) kmap_query_kernel(const ProbDev *__restrict__ P, JobList jl) {
+  const Job &job = find_job(jl, blockIdx.x);
+  const ProbDev &q = P[job.prob];
+  const GeomDev &g = q.g;
+  const long long n_in = q.n_in;
+  const pce_slot_t *__restrict__ table = q.table;
+  const unsigned long long slots = q.slots;
+  int *__restrict__ dense = q.dense;
+  long long i = (long long)(blockIdx.x - job.blk0) * blockDim.x + threadIdx.x;
   bool live = i < n_in;
-  int4 c = live ? in_coords[i] : make_int4(0, 0, 0, 0);
+  int4 c = live ? q.in_coords[i] : make_int4(0, 0, 0, 0);
   if (live && !pce_coord_ok(c.x, c.y, c.z, c.w)) {
-    status[0] = 1;
+    q.status[0] = 1;
     live = false;
   }
   const int kend = g.subm ? g.mid : g.kv;
@@ -1035,10 +1123,15 @@ __global__ void __launch_bounds__(256) kmap_query_kernel(const int4 *__restrict_
 
 // One pass over the probe results: hits per (offset, 64-row segment) from wave ballots, and hits per
 // row (the row lengths of the CSR view, mapping_counter of backend/hash.cuh:422-437).
-__global__ void __launch_bounds__(256) kmap_count_kernel(long long n_in, int kv, const int *__restrict__ dense,
-                                                         int *__restrict__ segcnt, long long nseg,
-                                                         int *__restrict__ rowcnt) {
-  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+__global__ void __launch_bounds__(256) kmap_count_kernel(const ProbDev *__restrict__ P, JobList jl) {
+  const Job &job = find_job(jl, blockIdx.x);
+  const ProbDev &q = P[job.prob];
+  const long long n_in = q.n_in, nseg = q.nseg;
+  const int kv = q.g.kv;
+  const int *__restrict__ dense = q.dense;
+  int *__restrict__ segcnt = q.seg;
+  int *__restrict__ rowcnt = q.want_csr ? q.icsr : nullptr;
+  long long i = (long long)(blockIdx.x - job.blk0) * blockDim.x + threadIdx.x;
   long long seg = i >> 6;
   bool live = i < n_in;
   int c = 0;
@@ -1059,17 +1152,87 @@ __global__ void __launch_bounds__(256) kmap_count_kernel(long long n_in, int kv,
   if (i == 0) segcnt[(long long)kv * nseg] = 0;
 }
 
+// Exclusive scans of several arrays in two launches: every workgroup scans its SCAN_TILE items in place
+// and records its total; then every workgroup adds the totals of the workgroups before it in its array.
+__global__ void __launch_bounds__(256) multi_scan_local_kernel(const ScanArr *__restrict__ arrs, int n_arrs) {
+  int a = 0;
+  while (a + 1 < n_arrs && blockIdx.x >= arrs[a + 1].blk0) ++a;
+  const ScanArr arr = arrs[a];
+  const int blk = blockIdx.x - arr.blk0;
+  long long base = (long long)blk * SCAN_TILE + (long long)threadIdx.x * SCAN_ITEMS;
+  int v[SCAN_ITEMS];
+  int acc = 0;
+#pragma unroll
+  for (int j = 0; j < SCAN_ITEMS; ++j) {
+    v[j] = base + j < arr.n ? arr.data[base + j] : 0;
+    acc += v[j];
+  }
+  int total;
+  int run = block_exclusive_scan(acc, &total);
+#pragma unroll
+  for (int j = 0; j < SCAN_ITEMS; ++j) {
+    if (base + j < arr.n) arr.data[base + j] = run;
+    run += v[j];
+  }
+  if (threadIdx.x == 0) arr.sums[blk] = total;
+}
+
+__global__ void __launch_bounds__(256) multi_scan_add_kernel(const ScanArr *__restrict__ arrs, int n_arrs) {
+  int a = 0;
+  while (a + 1 < n_arrs && blockIdx.x >= arrs[a + 1].blk0) ++a;
+  const ScanArr arr = arrs[a];
+  const int blk = blockIdx.x - arr.blk0;
+  if (blk == 0) return;
+  int acc = 0;
+  for (int j = threadIdx.x; j < blk; j += 256) acc += arr.sums[j];
+  int total;
+  block_exclusive_scan(acc, &total);
+  long long base = (long long)blk * SCAN_TILE + (long long)threadIdx.x * SCAN_ITEMS;
+#pragma unroll
+  for (int j = 0; j < SCAN_ITEMS; ++j)
+    if (base + j < arr.n) arr.data[base + j] += total;
+}
+
+// kpos[kp] = first pair of offset kp; then the scan of counts rounded up to the tile height
+// (backend/hash.cuh:478-497).  One workgroup per problem.
+__global__ void kmap_offsets_kernel(const ProbDev *__restrict__ P) {
+  const ProbDev &q = P[blockIdx.x];
+  const int *__restrict__ segoff = q.seg;
+  const long long nseg = q.nseg;
+  const int kv = q.g.kv;
+  for (int kp = threadIdx.x; kp <= kv; kp += blockDim.x) {
+    int a = segoff[(long long)kp * nseg];
+    q.kpos[kp] = a;
+    if (kp < kv) q.knnz[kp] = segoff[(long long)(kp + 1) * nseg] - a;
+  }
+  if (threadIdx.x == 0) {
+    int qq = 0;
+    q.qkpos[0] = 0;
+    for (int kp = 0; kp < kv; ++kp) {
+      int c = segoff[(long long)(kp + 1) * nseg] - segoff[(long long)kp * nseg];
+      qq += (c + PCE_QUANTUM - 1) / PCE_QUANTUM * PCE_QUANTUM;
+      q.qkpos[kp + 1] = qq;
+    }
+  }
+}
+
 // segoff = exclusive scan of segcnt in (kp, segment) order = position of the segment's first pair.
 // Emits the pair lists in (offset, input row) order from ballot ranks, the rank of every pair inside
 // its offset (irank, and orank scattered by output row for strided layers), and the output-major
 // neighbour table: scattered for strided layers, read off the mirrored row for submanifold ones.
-__global__ void __launch_bounds__(256) kmap_fill_kernel(long long n_in, long long n_out, int kv, int subm, int mid,
-                                                        const int *__restrict__ dense, const int *__restrict__ segoff,
-                                                        long long nseg, int *__restrict__ imap,
-                                                        int *__restrict__ omap, int *__restrict__ irank,
-                                                        int *__restrict__ orank, int *__restrict__ nbr_out,
-                                                        int *status) {
-  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+__global__ void __launch_bounds__(256) kmap_fill_kernel(const ProbDev *__restrict__ P, JobList jl) {
+  const Job &job = find_job(jl, blockIdx.x);
+  const ProbDev &q = P[job.prob];
+  const long long n_in = q.n_in, n_out = q.n_out, nseg = q.nseg;
+  const int kv = q.g.kv, subm = q.g.subm, mid = q.g.mid;
+  const int *__restrict__ dense = q.dense;
+  const int *__restrict__ segoff = q.seg;
+  int *__restrict__ imap = q.imap;
+  int *__restrict__ omap = q.omap;
+  int *__restrict__ irank = q.irank;
+  int *__restrict__ orank = q.orank;
+  int *__restrict__ nbr_out = q.nbr_out;
+  long long i = (long long)(blockIdx.x - job.blk0) * blockDim.x + threadIdx.x;
   long long seg = i >> 6;
   bool live = i < n_in;
   for (int kp0 = 0; kp0 < kv; kp0 += ROW_BATCH) {
@@ -1096,7 +1259,7 @@ __global__ void __launch_bounds__(256) kmap_fill_kernel(long long n_in, long lon
         omap[p] = v;
         if (nbr_out && !subm) nbr_out[(long long)kp * n_out + v] = (int)i;
         rank = p - first[j];
-        if (irank && rank >= PCE_CSR_CODE) status[2] = 1;
+        if (irank && rank >= PCE_CSR_CODE) q.status[2] = 1;
         if (orank) orank[(long long)kp * n_out + v] = rank;
       }
       if (irank && live) irank[(long long)kp * n_in + i] = rank;
@@ -1106,43 +1269,19 @@ __global__ void __launch_bounds__(256) kmap_fill_kernel(long long n_in, long lon
   }
 }
 
-__global__ void kmap_offsets_kernel(const int *__restrict__ segoff, long long nseg, int kv, int *knnz, int *kpos,
-                                    int *qkpos) {
-  // kpos[kp] = first pair of offset kp; then the scan of counts rounded up to the tile height
-  // (backend/hash.cuh:478-497)
-  for (int kp = threadIdx.x; kp <= kv; kp += blockDim.x) {
-    int a = segoff[(long long)kp * nseg];
-    kpos[kp] = a;
-    if (kp < kv) knnz[kp] = segoff[(long long)(kp + 1) * nseg] - a;
-  }
-  if (threadIdx.x == 0) {
-    int q = 0;
-    qkpos[0] = 0;
-    for (int kp = 0; kp < kv; ++kp) {
-      int c = segoff[(long long)(kp + 1) * nseg] - segoff[(long long)kp * nseg];
-      q += (c + PCE_QUANTUM - 1) / PCE_QUANTUM * PCE_QUANTUM;
-      qkpos[kp + 1] = q;
-    }
-  }
-}
-
-// rank[kp*n + r] >= 0 marks an entry of row r; count them (mapping_counter, backend/hash.cuh:422-437)
-__global__ void __launch_bounds__(256) csr_count_kernel(const int *__restrict__ rank, long long n, int kv,
-                                                        int *__restrict__ cnt) {
-  long long r = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (r > n) return;
-  int c = 0;
-  if (r < n)
-    for (int kp = 0; kp < kv; ++kp) c += rank[(long long)kp * n + r] >= 0;
-  cnt[r] = c;  // cnt[n] = 0 receives the total after the scan
-}
-
-// CSR-coded entries of every row in ascending offset order, plus, for every pair (offset kp, rank rk),
-// the slot of its entry in this order: slot_of_pair[kpos[kp] + rk] = position in `code`.
-__global__ void __launch_bounds__(256) csr_fill_kernel(const int *__restrict__ rank, long long n, int kv,
-                                                       const int *__restrict__ csr, int *__restrict__ code,
-                                                       const int *__restrict__ kpos, int *__restrict__ slot_of_pair) {
-  long long r = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+// CSR-coded views.  Entries of every row in ascending offset order, code = kp * PCE_CSR_CODE + rank, plus,
+// for every pair (offset kp, rank rk), the slot of its entry: slot_of_pair[kpos[kp] + rk] = position.
+// Jobs of one launch (the kind is uniform over a workgroup):
+//   JOB_CSR_SUBM      submanifold map, both views in one pass: the input-side entry of row r at offset kp
+//                     is the pair (r, dense[kp][r], kp); the output-side entry is the pair
+//                     (dense[kv-1-kp][r], r, kp), whose rank is read from the rank table at its input row.
+//                     Both views have the same row pointers.
+//   JOB_CSR_IN / JOB_CSR_OUT   one view of a strided map from its rank table (irank / orank)
+//   JOB_CSR_COUNT_OUT          entries per output row of a strided map (mapping_counter,
+//                              backend/hash.cuh:422-437), scanned before JOB_CSR_OUT runs
+__device__ __forceinline__ void csr_fill_rows(const int *__restrict__ rank, long long n, int kv, const int *__restrict__ csr,
+                                              int *__restrict__ code, const int *__restrict__ kpos,
+                                              int *__restrict__ slot_of_pair, long long r) {
   if (r >= n) return;
   int pos = csr[r];
   for (int kp = 0; kp < kv; ++kp) {
@@ -1155,22 +1294,45 @@ __global__ void __launch_bounds__(256) csr_fill_kernel(const int *__restrict__ r
   }
 }
 
-// Submanifold map: both CSR views in one pass.  The input-side entry of row r at offset kp is the
-// pair (r, dense[kp][r], kp); the output-side entry is the pair (dense[kv-1-kp][r], r, kp), whose
-// rank is read from the rank table at its input row.  Both views have the same row pointers.
-__global__ void __launch_bounds__(256) csr_fill_subm_kernel(const int *__restrict__ dense, const int *__restrict__ irank,
-                                                            long long n, int kv, const int *__restrict__ csr,
-                                                            const int *__restrict__ kpos, int *__restrict__ icode,
-                                                            int *__restrict__ ocode, int *__restrict__ islot,
-                                                            int *__restrict__ oslot, int *__restrict__ ocsr) {
-  long long r = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+__global__ void __launch_bounds__(256) csr_stage_kernel(const ProbDev *__restrict__ P, JobList jl) {
+  const Job &job = find_job(jl, blockIdx.x);
+  const ProbDev &q = P[job.prob];
+  const int kv = q.g.kv;
+  long long r = (long long)(blockIdx.x - job.blk0) * blockDim.x + threadIdx.x;
+  if (job.kind == JOB_CSR_IN) {
+    csr_fill_rows(q.irank, q.n_in, kv, q.icsr, q.icode, q.kpos, q.islot, r);
+    return;
+  }
+  if (job.kind == JOB_CSR_OUT) {
+    csr_fill_rows(q.orank, q.n_out, kv, q.ocsr, q.ocode, q.kpos, q.oslot, r);
+    return;
+  }
+  if (job.kind == JOB_CSR_COUNT_OUT) {
+    const long long n = q.n_out;
+    if (r > n) return;
+    int c = 0;
+    if (r < n)
+      for (int kp = 0; kp < kv; ++kp) c += q.orank[(long long)kp * n + r] >= 0;
+    q.ocsr[r] = c;  // ocsr[n] = 0 receives the total after the scan
+    return;
+  }
+  // JOB_CSR_SUBM
+  const long long n = q.n_in;
+  const int *__restrict__ dense = q.dense;
+  const int *__restrict__ irank = q.irank;
+  const int *__restrict__ csr = q.icsr;
+  const int *__restrict__ kpos = q.kpos;
+  int *__restrict__ icode = q.icode;
+  int *__restrict__ ocode = q.ocode;
+  int *__restrict__ islot = q.islot;
+  int *__restrict__ oslot = q.oslot;
   if (r > n) return;
   if (r == n) {
-    ocsr[n] = csr[n];
+    q.ocsr[n] = csr[n];
     return;
   }
   int pi = csr[r], po = pi;
-  ocsr[r] = pi;
+  q.ocsr[r] = pi;
   for (int kp0 = 0; kp0 < kv; kp0 += ROW_BATCH) {
     int rk[ROW_BATCH], src[ROW_BATCH], rk2[ROW_BATCH], kb[ROW_BATCH];
 #pragma unroll
@@ -1206,83 +1368,233 @@ extern "C" int64_t pce_kmap_workspace_bytes(int64_t n_in, int64_t n_out, int32_t
   return L.total;
 }
 
+// host-side image of everything the kernels of one batch read
+struct BatchImage {
+  ProbDev prob[PCE_MAX_BATCH];
+  Job jobs[8][2 * PCE_MAX_BATCH];      // per stage
+  int n_jobs[8];
+  FillRegion fills[3 * PCE_MAX_BATCH];
+  ScanArr scans[2][2 * PCE_MAX_BATCH];  // first scan (segments, input rows), second scan (output rows)
+};
+enum { ST_INSERT = 0, ST_QUERY, ST_COUNT, ST_FILL, ST_CSR_A, ST_CSR_B };
+
+// The descriptor block travels from pinned host memory, so the copy is queued like a kernel and the
+// host does not wait for earlier work on the stream.  A small ring of pinned blocks per device; a
+// block is reused once the copy that read it has completed.
+#define DESC_RING 8
+#define DESC_MAX_DEVICES 16
+struct DescRing {
+  BatchImage *host[DESC_RING];
+  hipEvent_t done[DESC_RING];
+  int next;
+  bool ready;
+};
+static DescRing g_desc_ring[DESC_MAX_DEVICES];
+static std::mutex g_desc_mutex;
+
+static int desc_upload(const BatchImage &img, void *dst, hipStream_t s) {
+  int dev = 0;
+  PCE_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= DESC_MAX_DEVICES) PCE_FAIL(PCE_ECAPACITY, "device index %d not supported", dev);
+  std::lock_guard<std::mutex> lock(g_desc_mutex);
+  DescRing &r = g_desc_ring[dev];
+  if (!r.ready) {
+    for (int k = 0; k < DESC_RING; ++k) {
+      PCE_HIP(hipHostMalloc((void **)&r.host[k], sizeof(BatchImage), hipHostMallocDefault));
+      PCE_HIP(hipEventCreateWithFlags(&r.done[k], hipEventDisableTiming));
+    }
+    r.next = 0;
+    r.ready = true;
+  }
+  const int k = r.next;
+  r.next = (k + 1) % DESC_RING;
+  PCE_HIP(hipEventSynchronize(r.done[k]));  // returns at once for an event never recorded
+  memcpy(r.host[k], &img, sizeof(BatchImage));
+  PCE_HIP(hipMemcpyAsync(dst, r.host[k], sizeof(BatchImage), hipMemcpyHostToDevice, s));
+  PCE_HIP(hipEventRecord(r.done[k], s));
+  return PCE_OK;
+}
+
+extern "C" int pce_kmap_build_batch(const pce_kmap_problem_t *probs, int32_t n_probs, pce_stream_t stream) {
+  hipStream_t s = (hipStream_t)stream;
+  if (!probs || n_probs < 1 || n_probs > PCE_MAX_BATCH)
+    PCE_FAIL(PCE_EINVAL, "pce_kmap_build_batch: 1..%d problems per call", PCE_MAX_BATCH);
+  static_assert(sizeof(BatchImage) <= KMAP_DESC_BYTES, "descriptor area too small");
+  BatchImage img;
+  memset(&img, 0, sizeof(img));
+  unsigned blk[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  unsigned fill_blk = 0, scan_blk[2] = {0, 0};
+  int n_fill = 0, n_scan[2] = {0, 0};
+  auto add_job = [&](int stage, int prob, int kind, long long items) {
+    Job &j = img.jobs[stage][img.n_jobs[stage]++];
+    j.blk0 = blk[stage];
+    j.prob = prob;
+    j.kind = kind;
+    blk[stage] += (unsigned)pce_div_up(items, 256);
+  };
+  auto add_fill = [&](void *p, long long words) {
+    if (words <= 0) return;
+    FillRegion &f = img.fills[n_fill++];
+    f.p = (unsigned *)p;
+    f.n_words = words;
+    f.blk0 = fill_blk;
+    fill_blk += (unsigned)pce_div_up(words, FILL_WORDS_PER_BLOCK);
+  };
+  auto add_scan = [&](int which, int *data, long long n, int *sums) {
+    ScanArr &a = img.scans[which][n_scan[which]++];
+    a.data = data;
+    a.n = n;
+    a.sums = sums;
+    a.blk0 = scan_blk[which];
+    scan_blk[which] += (unsigned)pce_div_up(n, SCAN_TILE);
+  };
+  long long total_blocks = 0;
+  for (int p = 0; p < n_probs; ++p) {
+    const pce_kmap_problem_t &u = probs[p];
+    ProbDev &q = img.prob[p];
+    int rc = make_geom(&u.geom, &q.g);
+    if (rc) return rc;
+    if (!u.in_coords || !u.out_coords || !u.ws || !u.imap || !u.omap || !u.knnz || !u.kpos || !u.qkpos || !u.status)
+      PCE_FAIL(PCE_EINVAL, "pce_kmap_build: null pointer");
+    int ncsr = (u.icsr != nullptr) + (u.icode != nullptr) + (u.ocsr != nullptr) + (u.ocode != nullptr);
+    if (ncsr != 0 && ncsr != 4) PCE_FAIL(PCE_EINVAL, "pce_kmap_build: pass all four CSR outputs or none");
+    const int want_csr = ncsr == 4;
+    if (!want_csr && (u.islot || u.oslot)) PCE_FAIL(PCE_EINVAL, "pce_kmap_build: slot outputs need the CSR outputs");
+    const int64_t n_in = u.n_in, n_out = u.n_out;
+    if (n_in <= 0 || n_out <= 0) PCE_FAIL(PCE_EINVAL, "pce_kmap_build: empty tensor (n_in=%lld, n_out=%lld)", (long long)n_in, (long long)n_out);
+    if (q.g.subm && n_in != n_out) PCE_FAIL(PCE_EINVAL, "pce_kmap_build: submanifold layer needs n_in == n_out");
+    if ((int64_t)q.g.kv * n_in >= (1ll << 31) || (int64_t)q.g.kv * n_out >= (1ll << 31))
+      PCE_FAIL(PCE_ECAPACITY, "pce_kmap_build: kv*n exceeds int32 pair indexing");
+    KmapLayout L;
+    kmap_layout(n_in, n_out, q.g.kv, want_csr, q.g.subm, &L);
+    if (u.ws_bytes < L.total) PCE_FAIL(PCE_EWORKSPACE, "pce_kmap_build: workspace %lld < %lld", (long long)u.ws_bytes, (long long)L.total);
+    char *w = (char *)u.ws;
+    q.in_coords = (const int4 *)u.in_coords;
+    q.out_coords = (const int4 *)u.out_coords;
+    q.n_in = n_in;
+    q.n_out = n_out;
+    q.nseg = L.nseg;
+    q.table = (pce_slot_t *)(w + L.off_table);
+    q.slots = (unsigned long long)L.slots;
+    q.dense = u.nbr_in ? u.nbr_in : (int *)(w + L.off_dense);  // the input-major table is the probe result itself
+    q.irank = want_csr ? (int *)(w + L.off_irank) : nullptr;
+    q.orank = (want_csr && !q.g.subm) ? (int *)(w + L.off_orank) : nullptr;
+    q.seg = (int *)(w + L.off_seg);
+    q.imap = u.imap;
+    q.omap = u.omap;
+    q.knnz = u.knnz;
+    q.kpos = u.kpos;
+    q.qkpos = u.qkpos;
+    q.icsr = u.icsr;
+    q.icode = u.icode;
+    q.ocsr = u.ocsr;
+    q.ocode = u.ocode;
+    q.islot = u.islot;
+    q.oslot = u.oslot;
+    q.nbr_out = u.nbr_out;
+    q.status = u.status;
+    q.want_csr = want_csr;
+    // 1. table over the output coordinates (for a submanifold layer these are the input coordinates)
+    add_fill(q.table, L.slots * 4);
+    if (q.g.subm) {
+      // rows of the probe table that the mirrored writes only touch on a hit (and the centre row)
+      add_fill(q.dense + (int64_t)q.g.mid * n_in, (int64_t)(q.g.kv - q.g.mid) * n_in);
+    } else {
+      if (q.nbr_out) add_fill(q.nbr_out, (int64_t)q.g.kv * n_out);
+      if (q.orank) add_fill(q.orank, (int64_t)q.g.kv * n_out);
+    }
+    add_job(ST_INSERT, p, 0, n_out);
+    // 2. probe, count per (offset, segment) and per row; 3. their scans; 4. pair lists
+    add_job(ST_QUERY, p, 0, n_in);
+    add_job(ST_COUNT, p, 0, n_in + 1);
+    int *scan_tmp = (int *)(w + L.off_scan);
+    add_scan(0, q.seg, L.scan_len, scan_tmp);
+    if (want_csr) add_scan(0, q.icsr, n_in + 1, scan_tmp + scan_tmp_ints(L.scan_len));
+    add_job(ST_FILL, p, 0, n_in);
+    // 5. CSR-coded views
+    if (want_csr && q.g.subm) {
+      add_job(ST_CSR_A, p, JOB_CSR_SUBM, n_in + 1);
+    } else if (want_csr) {
+      add_job(ST_CSR_A, p, JOB_CSR_IN, n_in);
+      add_job(ST_CSR_A, p, JOB_CSR_COUNT_OUT, n_out + 1);
+      add_scan(1, q.ocsr, n_out + 1, scan_tmp + scan_tmp_ints(L.scan_len) + scan_tmp_ints(n_in + 1));
+      add_job(ST_CSR_B, p, JOB_CSR_OUT, n_out);
+    }
+    total_blocks += pce_div_up(n_in + 1, 256) + pce_div_up(n_out + 1, 256) + pce_div_up(L.slots * 4, FILL_WORDS_PER_BLOCK) +
+                    3 * pce_div_up((int64_t)q.g.kv * (n_in > n_out ? n_in : n_out), FILL_WORDS_PER_BLOCK);
+  }
+  if (total_blocks >= (1ll << 31)) PCE_FAIL(PCE_ECAPACITY, "pce_kmap_build_batch: the batch exceeds the grid limit");
+  // one copy carries the descriptors; they live in the first problem's workspace
+  KmapLayout L0;
+  kmap_layout(probs[0].n_in, probs[0].n_out, img.prob[0].g.kv, img.prob[0].want_csr, img.prob[0].g.subm, &L0);
+  char *desc = (char *)probs[0].ws + L0.off_desc;
+  if (int rc = desc_upload(img, desc, s)) return rc;
+  const BatchImage *D = (const BatchImage *)desc;
+  const ProbDev *P = D->prob;
+  auto jl = [&](int stage) {
+    JobList l;
+    l.jobs = D->jobs[stage];
+    l.n = img.n_jobs[stage];
+    return l;
+  };
+  hipLaunchKernelGGL(multi_fill_kernel, dim3(fill_blk), dim3(256), 0, s, (const FillRegion *)D->fills, n_fill, 0xFFFFFFFFu);
+  PCE_LAUNCH_CHECK("multi_fill");
+  hipLaunchKernelGGL(batch_insert_kernel, dim3(blk[ST_INSERT]), dim3(256), 0, s, P, jl(ST_INSERT));
+  PCE_LAUNCH_CHECK("hash_insert");
+  hipLaunchKernelGGL(kmap_query_kernel, dim3(blk[ST_QUERY]), dim3(256), 0, s, P, jl(ST_QUERY));
+  PCE_LAUNCH_CHECK("kmap_query");
+  hipLaunchKernelGGL(kmap_count_kernel, dim3(blk[ST_COUNT]), dim3(256), 0, s, P, jl(ST_COUNT));
+  PCE_LAUNCH_CHECK("kmap_count");
+  hipLaunchKernelGGL(multi_scan_local_kernel, dim3(scan_blk[0]), dim3(256), 0, s, (const ScanArr *)D->scans[0], n_scan[0]);
+  PCE_LAUNCH_CHECK("scan_local");
+  hipLaunchKernelGGL(multi_scan_add_kernel, dim3(scan_blk[0]), dim3(256), 0, s, (const ScanArr *)D->scans[0], n_scan[0]);
+  PCE_LAUNCH_CHECK("scan_add");
+  hipLaunchKernelGGL(kmap_offsets_kernel, dim3(n_probs), dim3(128), 0, s, P);
+  PCE_LAUNCH_CHECK("kmap_offsets");
+  hipLaunchKernelGGL(kmap_fill_kernel, dim3(blk[ST_FILL]), dim3(256), 0, s, P, jl(ST_FILL));
+  PCE_LAUNCH_CHECK("kmap_fill");
+  if (blk[ST_CSR_A]) {
+    hipLaunchKernelGGL(csr_stage_kernel, dim3(blk[ST_CSR_A]), dim3(256), 0, s, P, jl(ST_CSR_A));
+    PCE_LAUNCH_CHECK("csr_stage_a");
+  }
+  if (blk[ST_CSR_B]) {
+    hipLaunchKernelGGL(multi_scan_local_kernel, dim3(scan_blk[1]), dim3(256), 0, s, (const ScanArr *)D->scans[1], n_scan[1]);
+    PCE_LAUNCH_CHECK("scan_local");
+    hipLaunchKernelGGL(multi_scan_add_kernel, dim3(scan_blk[1]), dim3(256), 0, s, (const ScanArr *)D->scans[1], n_scan[1]);
+    PCE_LAUNCH_CHECK("scan_add");
+    hipLaunchKernelGGL(csr_stage_kernel, dim3(blk[ST_CSR_B]), dim3(256), 0, s, P, jl(ST_CSR_B));
+    PCE_LAUNCH_CHECK("csr_stage_b");
+  }
+  return PCE_OK;
+}
+
 extern "C" int pce_kmap_build(const int32_t *in_coords, int64_t n_in, const int32_t *out_coords, int64_t n_out,
                               const pce_geom_t *g, void *ws, int64_t ws_bytes, int32_t *imap, int32_t *omap,
                               int32_t *knnz, int32_t *kpos, int32_t *qkpos, int32_t *icsr, int32_t *icode,
                               int32_t *ocsr, int32_t *ocode, int32_t *islot, int32_t *oslot, int32_t *nbr_out,
                               int32_t *nbr_in, int32_t *status, pce_stream_t stream) {
-  hipStream_t s = (hipStream_t)stream;
-  GeomDev gd;
-  int rc = make_geom(g, &gd);
-  if (rc) return rc;
-  if (!in_coords || !out_coords || !ws || !imap || !omap || !knnz || !kpos || !qkpos || !status)
-    PCE_FAIL(PCE_EINVAL, "pce_kmap_build: null pointer");
-  int ncsr = (icsr != nullptr) + (icode != nullptr) + (ocsr != nullptr) + (ocode != nullptr);
-  if (ncsr != 0 && ncsr != 4) PCE_FAIL(PCE_EINVAL, "pce_kmap_build: pass all four CSR outputs or none");
-  int want_csr = ncsr == 4;
-  if (!want_csr && (islot || oslot)) PCE_FAIL(PCE_EINVAL, "pce_kmap_build: slot outputs need the CSR outputs");
-  if (n_in <= 0 || n_out <= 0) PCE_FAIL(PCE_EINVAL, "pce_kmap_build: empty tensor (n_in=%lld, n_out=%lld)", (long long)n_in, (long long)n_out);
-  if (gd.subm && n_in != n_out) PCE_FAIL(PCE_EINVAL, "pce_kmap_build: submanifold layer needs n_in == n_out");
-  if ((int64_t)gd.kv * n_in >= (1ll << 31) || (int64_t)gd.kv * n_out >= (1ll << 31))
-    PCE_FAIL(PCE_ECAPACITY, "pce_kmap_build: kv*n exceeds int32 pair indexing");
-  KmapLayout L;
-  kmap_layout(n_in, n_out, gd.kv, want_csr, gd.subm, &L);
-  if (ws_bytes < L.total) PCE_FAIL(PCE_EWORKSPACE, "pce_kmap_build: workspace %lld < %lld", (long long)ws_bytes, (long long)L.total);
-  char *w = (char *)ws;
-  pce_slot_t *table = (pce_slot_t *)(w + L.off_table);
-  int *dense = nbr_in ? nbr_in : (int *)(w + L.off_dense);  // the input-major table is the probe result itself
-  int *irank = want_csr ? (int *)(w + L.off_irank) : nullptr;
-  int *seg = (int *)(w + L.off_seg);
-  int *scan_tmp = (int *)(w + L.off_scan);
-  int *orank = (want_csr && !gd.subm) ? (int *)(w + L.off_orank) : nullptr;
-
-  // 1. table over the output coordinates (for a submanifold layer these are the input coordinates)
-  if ((rc = table_clear(table, L.slots, s))) return rc;
-  hipLaunchKernelGGL(hash_insert_kernel, dim3((unsigned)pce_div_up(n_out, 256)), dim3(256), 0, s, table,
-                     (unsigned long long)L.slots, (const int4 *)out_coords, (long long)n_out, status);
-  PCE_LAUNCH_CHECK("hash_insert");
-  if (gd.subm) {
-    // rows of the probe table that the mirrored writes only touch on a hit (and the centre row)
-    if ((rc = fill_u32(dense + (int64_t)gd.mid * n_in, (int64_t)(gd.kv - gd.mid) * n_in, 0xFFFFFFFFu, s))) return rc;
-  } else {
-    if (nbr_out && (rc = fill_u32(nbr_out, (int64_t)gd.kv * n_out, 0xFFFFFFFFu, s))) return rc;
-    if (orank && (rc = fill_u32(orank, (int64_t)gd.kv * n_out, 0xFFFFFFFFu, s))) return rc;
-  }
-  // 2. probe, then count per (offset, segment) and per row
-  unsigned blocks = (unsigned)pce_div_up(n_in, 256);
-  hipLaunchKernelGGL(kmap_query_kernel, dim3(blocks), dim3(256), 0, s, (const int4 *)in_coords, (long long)n_in, gd,
-                     (const pce_slot_t *)table, (unsigned long long)L.slots, dense, status);
-  PCE_LAUNCH_CHECK("kmap_query");
-  hipLaunchKernelGGL(kmap_count_kernel, dim3((unsigned)pce_div_up(n_in + 1, 256)), dim3(256), 0, s, (long long)n_in, gd.kv,
-                     (const int *)dense, seg, (long long)L.nseg, want_csr ? icsr : nullptr);
-  PCE_LAUNCH_CHECK("kmap_count");
-  // 3. positions: scan of the segment counts and, in the same launches, of the input row lengths
-  if ((rc = scan_exclusive2(seg, L.scan_len, want_csr ? icsr : nullptr, n_in + 1, scan_tmp, s))) return rc;
-  hipLaunchKernelGGL(kmap_offsets_kernel, dim3(1), dim3(128), 0, s, (const int *)seg, (long long)L.nseg, gd.kv, knnz,
-                     kpos, qkpos);
-  PCE_LAUNCH_CHECK("kmap_offsets");
-  // 4. pair lists in (offset, input row) order
-  hipLaunchKernelGGL(kmap_fill_kernel, dim3(blocks), dim3(256), 0, s, (long long)n_in, (long long)n_out, gd.kv, gd.subm,
-                     gd.mid, (const int *)dense, (const int *)seg, (long long)L.nseg, imap, omap, irank, orank, nbr_out,
-                     status);
-  PCE_LAUNCH_CHECK("kmap_fill");
-  // 5. CSR-coded view
-  if (want_csr && gd.subm) {
-    hipLaunchKernelGGL(csr_fill_subm_kernel, dim3((unsigned)pce_div_up(n_in + 1, 256)), dim3(256), 0, s,
-                       (const int *)dense, (const int *)irank, (long long)n_in, gd.kv, (const int *)icsr,
-                       (const int *)kpos, icode, ocode, islot, oslot, ocsr);
-    PCE_LAUNCH_CHECK("csr_fill_subm");
-  } else if (want_csr) {
-    hipLaunchKernelGGL(csr_fill_kernel, dim3((unsigned)pce_div_up(n_in, 256)), dim3(256), 0, s, (const int *)irank,
-                       (long long)n_in, gd.kv, (const int *)icsr, icode, (const int *)kpos, islot);
-    PCE_LAUNCH_CHECK("csr_fill(in)");
-    hipLaunchKernelGGL(csr_count_kernel, dim3((unsigned)pce_div_up(n_out + 1, 256)), dim3(256), 0, s, (const int *)orank,
-                       (long long)n_out, gd.kv, ocsr);
-    PCE_LAUNCH_CHECK("csr_count(out)");
-    if ((rc = scan_exclusive(ocsr, n_out + 1, scan_tmp, s))) return rc;
-    hipLaunchKernelGGL(csr_fill_kernel, dim3((unsigned)pce_div_up(n_out, 256)), dim3(256), 0, s, (const int *)orank,
-                       (long long)n_out, gd.kv, (const int *)ocsr, ocode, (const int *)kpos, oslot);
-    PCE_LAUNCH_CHECK("csr_fill(out)");
-  }
-  return PCE_OK;
+  if (!g) PCE_FAIL(PCE_EINVAL, "geometry is null");
+  pce_kmap_problem_t u;
+  u.in_coords = in_coords;
+  u.n_in = n_in;
+  u.out_coords = out_coords;
+  u.n_out = n_out;
+  u.geom = *g;
+  u.ws = ws;
+  u.ws_bytes = ws_bytes;
+  u.imap = imap;
+  u.omap = omap;
+  u.knnz = knnz;
+  u.kpos = kpos;
+  u.qkpos = qkpos;
+  u.icsr = icsr;
+  u.icode = icode;
+  u.ocsr = ocsr;
+  u.ocode = ocode;
+  u.islot = islot;
+  u.oslot = oslot;
+  u.nbr_out = nbr_out;
+  u.nbr_in = nbr_in;
+  u.status = status;
+  return pce_kmap_build_batch(&u, 1, stream);
 }

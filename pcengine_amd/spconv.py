@@ -232,8 +232,9 @@ def _run(input: spTensor, km: backend.KernelMap, kernel, in_channel, out_channel
     return out
 
 
-def _map_request(input: spTensor, kernel_size_code: int, stride_code: int, padding_code: int, defer: bool):
-    """Cache lookup, or the build (finished, or queued when ``defer``), of one layer's map."""
+def _map_request(input: spTensor, kernel_size_code: int, stride_code: int, padding_code: int):
+    """Cache lookup of one layer's map.  Returns (map or None, build request or None, cache key, tag,
+    output tensor stride, output coords_min, output coords_max)."""
     output_stride = output_stride_compute(stride_code, input.stride, 0)
     key = (kernel_size_code, input.stride, stride_code)
     km = input.kmaps.get(key)
@@ -245,18 +246,18 @@ def _map_request(input: spTensor, kernel_size_code: int, stride_code: int, paddi
     pad = conv_info_decoder(padding_code)
     if not subm:
         coords_max = backend.strided_coords_max(input.coords_max, ks, stride, pad)   # script/spconv.py:358-360
-    tag = None
+    tag = request = None
     if km is None:
         tag = input.init_tag[0] if input.init_tag else 'end'
         if tag not in ('D1', 'D2', 'end', 'auto'):
             raise NotImplementedError(f"unknown init_tag entry {tag!r}")
         auto = tag in ('end', 'auto')
-        km = backend.build_kernel_map(input.coords, ks, stride, pad, coords_min, coords_max, subm,
-                                      want_csr=(tag == 'D1' or auto), want_nbr_out=auto, want_nbr_in=auto and not subm,
-                                      batchsize=input.batchsize, defer=defer)
+        request = dict(in_coords=input.coords, ks=ks, stride=stride, pad=pad, cmin=coords_min, cmax_out=coords_max,
+                       subm=subm, want_csr=(tag == 'D1' or auto), want_nbr_out=auto, want_nbr_in=auto and not subm,
+                       batchsize=input.batchsize)
         if tag in ('D1', 'D2'):
             input.init_tag = input.init_tag[1:]
-    return km, key, tag, output_stride, coords_min, coords_max
+    return km, request, key, tag, output_stride, coords_min, coords_max
 
 
 def _map_store(input: spTensor, km: backend.KernelMap, key, tag, output_stride) -> None:
@@ -270,8 +271,9 @@ def ensure_map(input: spTensor, kernel_size_code: int, stride_code: int, padding
     and stored there (script/spconv.py:331-437).  Returns (map, output tensor stride, output
     coords_min, output coords_max).  Maps depend on coordinates only, so a network can ask for all of
     them before the first convolution (``prebuild_maps``)."""
-    km, key, tag, output_stride, coords_min, coords_max = _map_request(input, kernel_size_code, stride_code, padding_code, False)
-    if tag is not None:
+    km, request, key, tag, output_stride, coords_min, coords_max = _map_request(input, kernel_size_code, stride_code, padding_code)
+    if request is not None:
+        km = backend.build_kernel_map(**request)
         _map_store(input, km, key, tag, output_stride)
     input.cbook.setdefault(input.stride, input.coords)
     return km, output_stride, coords_min, coords_max
@@ -281,29 +283,37 @@ def prebuild_maps(input: spTensor, layers) -> None:
     """Build, ahead of any convolution, the maps a network will ask for.  ``layers`` lists
     (kernel_size, stride, padding) in network order (ints or triples; transposed layers and 1x1
     layers need no entry); a strided entry moves on to its output coordinates, as the network does.
-    The builds are queued behind each other and their pair counts are read back together after one
-    synchronisation (only the output coordinates of a strided layer have to reach the host in
-    between, for their number), so the device does not idle between the ~17 small kernels of each build
-    and the layers that follow find every map in the cache."""
+    The output coordinates of the strided layers are computed first, level by level (their number has
+    to reach the host); then all maps are built together, every stage of the build as one launch over
+    all layers, and their pair counts are read back in one copy.  The layers that follow find every
+    map in the cache."""
     x = input
     pending = []
-    for ks, stride, pad in layers:
-        ksc, sc, pc = (conv_info_encoder(_triple(v, "layer")) for v in (ks, stride, pad))
-        if ksc == _UNIT and sc == _UNIT:
-            continue
-        km, key, tag, out_stride, cmin, cmax = _map_request(x, ksc, sc, pc, True)
-        if tag is not None:
-            pending.append((x, km, key, tag, out_stride))
-        x.cbook.setdefault(x.stride, x.coords)
-        if sc != _UNIT:
-            nxt = spTensor(feats=x.feats, coords=km.out_coords, buffer=x.buffer, batchsize=x.batchsize, stride=out_stride,
-                           init_tag=x.init_tag, coords_max=cmax, coords_min=cmin)
-            nxt.kmaps, nxt.cbook = x.kmaps, x.cbook
-            x = nxt
-    if pending:
-        torch.cuda.current_stream(input.coords.device).synchronize()
-        for t, pm, key, tag, out_stride in pending:
-            _map_store(t, pm.finish(), key, tag, out_stride)
+    try:
+        for ks, stride, pad in layers:
+            ksc, sc, pc = (conv_info_encoder(_triple(v, "layer")) for v in (ks, stride, pad))
+            if ksc == _UNIT and sc == _UNIT:
+                continue
+            km, request, key, tag, out_stride, cmin, cmax = _map_request(x, ksc, sc, pc)
+            if request is not None:
+                km = backend.prepare_map(**request)
+                pending.append((x, km, key, tag, out_stride))
+                x.kmaps[key] = km          # placeholder: a later entry with the same key is the same map
+            x.cbook.setdefault(x.stride, x.coords)
+            if sc != _UNIT:
+                nxt = spTensor(feats=x.feats, coords=km.out_coords, buffer=x.buffer, batchsize=x.batchsize,
+                               stride=out_stride, init_tag=x.init_tag, coords_max=cmax, coords_min=cmin)
+                nxt.kmaps, nxt.cbook = x.kmaps, x.cbook
+                x = nxt
+        if pending:
+            built = backend.build_kernel_maps([job for _, job, _, _, _ in pending], defer=True)
+            torch.cuda.current_stream(input.coords.device).synchronize()
+            for (t, _, key, tag, out_stride), pm in zip(pending, built):
+                _map_store(t, pm.finish(), key, tag, out_stride)
+    finally:
+        for t, job, key, _, _ in pending:       # a failed build leaves no placeholder behind
+            if t.kmaps.get(key) is job:
+                del t.kmaps[key]
 
 
 def conv_func(input: spTensor, in_channel, out_channel, kernel, kernel_size_code, stride_code, padding_code, bias,

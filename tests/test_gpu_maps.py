@@ -103,6 +103,47 @@ def test_kernel_map_config2_lidar_full_size():
     assert (np.diff(code) > 0).all()      # strictly ascending (b,x,y,z)
 
 
+def _request(coords, ks, stride, pad, **kw):
+    subm = tuple(stride) == (1, 1, 1)
+    cmax = coords[:, 1:].max(axis=0).tolist()
+    if not subm:
+        cmax = orc.strided_coords_max(cmax, ks, stride, pad)
+    return dict(in_coords=dev_coords(coords), ks=ks, stride=stride, pad=pad, cmin=[0, 0, 0], cmax_out=cmax, subm=subm, **kw)
+
+
+@pytest.mark.parametrize("defer", [False, True])
+def test_kernel_maps_batched_build_bit_exact(defer):
+    """Several layers per call: every stage of the build is one launch over all problems.  Mixed
+    geometries, sizes from one row to 20k, with and without the optional outputs; 19 problems, so the
+    call is split into two batches."""
+    cases = []
+    for k, (ks, stride, pad) in enumerate(GEOMS + GEOMS + GEOMS[:3]):
+        n, extent, batches = [(500, 9, 3), (20000, 40, 2), (63, 5, 1), (1, 3, 1), (3000, 20, 1)][k % 5]
+        coords = synth.random_cloud(seed=100 + k, n=n, extent=extent, batches=batches)
+        ref = orc.kernel_map(coords, ks, stride, pad)
+        if ref.n_out == 0:
+            continue
+        full = k % 3 != 2
+        cases.append((ref, full, _request(coords, ks, stride, pad, want_csr=full, want_nbr_out=True, want_nbr_in=full,
+                                          batchsize=batches if k % 2 else 0)))
+    assert len(cases) > backend.KMAP_MAX_BATCH
+    maps = backend.build_kernel_maps([c[2] for c in cases], defer=defer)
+    if defer:
+        torch.cuda.synchronize()
+        maps = [m.finish() for m in maps]
+    for (ref, full, _), km in zip(cases, maps):
+        assert_map_equal(km, ref, csr=full)
+
+
+def test_kernel_maps_batch_argument_errors():
+    lib = _lib.load()
+    probs = (_lib.KmapProblem * 1)()
+    assert lib.pce_kmap_build_batch(probs, 0, None) == _lib.PCE_EINVAL
+    assert lib.pce_kmap_build_batch(probs, backend.KMAP_MAX_BATCH + 1, None) == _lib.PCE_EINVAL
+    assert lib.pce_kmap_build_batch(probs, 1, None) == _lib.PCE_EINVAL          # zeroed problem: bad geometry
+    assert backend.build_kernel_maps([]) == []
+
+
 def _out_coords(coords, ks, stride, pad, cmin, cmax_out, n_batch):
     geom = _lib.Geom.make(ks, stride, pad, cmin, cmax_out, False)
     return backend.build_out_coords(dev_coords(coords), geom, n_batch).cpu().numpy()
