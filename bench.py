@@ -25,8 +25,9 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--dataflow", default="auto")
-    ap.add_argument("--workload", default="cfg2", choices=["cfg2", "deep"],
-                    help="cfg2: the headline layer; deep: a decoder-like layer (dense map, C 256->256) for the MFMA roofline")
+    ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg2x8", "deep"],
+                    help="cfg2: the headline layer; cfg2x8: the same layer on a batch of 8 such scans (1.2 M voxels, a working "
+                         "set beyond the last-level cache); deep: a decoder-like layer (dense map, C 256->256) for the MFMA roofline")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-net", action="store_true", help="skip the MinkUNet-style forward (configuration 4)")
     ap.add_argument("--all-configs", action="store_true",
@@ -51,6 +52,15 @@ def main() -> int:
         coords = synth.lidar_cloud()
         what = "cfg2: submanifold 3x3x3 conv, fp16 storage / fp32 accumulate, C 64->64, batch 1, N={n} voxels " \
                "(64x2048 LiDAR-like rays + ground plane @0.1 m), M={M} pairs, cached kernel map"
+    elif args.workload == "cfg2x8":
+        c_in = c_out = 64
+        scans = [synth.lidar_cloud(seed=2 + b) for b in range(8)]
+        for b, sc in enumerate(scans):
+            sc[:, 0] = b
+        coords = np.concatenate(scans, axis=0)
+        args.no_net = True
+        what = "cfg2x8: the configuration-2 layer (submanifold 3x3x3, fp16, C 64->64) on a batch of 8 LiDAR-like scans, " \
+               "N={n} voxels, M={M} pairs, cached kernel map"
     else:
         c_in = c_out = 256
         coords = synth.random_cloud(seed=7, n=90000, extent=58)
@@ -193,7 +203,7 @@ def main() -> int:
     # HBM bytes per launch of that kernel from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
     # profiles/pmc_traffic_cfg2.md (scaled by the copy-kernel calibration); counters cannot be read here
     measured_traffic = {("cfg2", "centre_gemm_csr_sum"): 43.46e6, ("cfg2", "pairs_and_centre_gemm"): 47.54e6}
-    if args.workload == "cfg2":
+    if args.workload in ("cfg2", "cfg2x8"):
         roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic.get((args.workload, dom)),
                     "algorithmic_bytes": dom_bytes, "kernel_ms": round(stages[dom], 5),
