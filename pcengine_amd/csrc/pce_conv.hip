@@ -862,14 +862,38 @@ static inline bool stage_on(int bit) { return (g_stage_mask >> bit) & 1u; }
 #define PIPE_ST 3
 #define PIPE_NB 4
 
-__device__ __forceinline__ void pipe_wait_barrier(bool more_in_flight) {
-  // loads complete in issue order: leaving the two youngest (the next-but-one weight chunk of this
-  // wavefront) in flight still guarantees that the chunk about to be used has landed
-  if (more_in_flight)
-    asm volatile("s_waitcnt vmcnt(2)\n\ts_barrier" ::: "memory");
-  else
-    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+// The feature fragments of the pipelined kernel are requested by loads the compiler does not track:
+// it would otherwise wait for every outstanding load (the ones just issued included) before the first
+// use of a fragment inside the loop.  The waits are written by hand instead (pipe_wait_barrier).
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ u32x4 load16_untracked(const void *p) {
+  u32x4 v;
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+  return v;
 }
+
+// Waits until at most `leave_in_flight` loads are outstanding, joins the workgroup barrier and only then
+// reads the two fragments: the copies are made inside the same statement, after the wait, so that no read
+// of a fragment register can be scheduled before its load has landed.
+#define PCE_PIPE_WAIT_COPY(CNT_)                                                                              \
+  asm volatile("s_waitcnt vmcnt(" #CNT_ ")\n\ts_barrier\n\t"                                                  \
+               "v_mov_b32 %0, %8\n\tv_mov_b32 %1, %9\n\tv_mov_b32 %2, %10\n\tv_mov_b32 %3, %11\n\t"           \
+               "v_mov_b32 %4, %12\n\tv_mov_b32 %5, %13\n\tv_mov_b32 %6, %14\n\tv_mov_b32 %7, %15"              \
+               : "=&v"(o0.x), "=&v"(o0.y), "=&v"(o0.z), "=&v"(o0.w), "=&v"(o1.x), "=&v"(o1.y), "=&v"(o1.z),    \
+                 "=&v"(o1.w)                                                                                  \
+               : "v"(f0.x), "v"(f0.y), "v"(f0.z), "v"(f0.w), "v"(f1.x), "v"(f1.y), "v"(f1.z), "v"(f1.w)       \
+               : "memory")
+__device__ __forceinline__ void pipe_wait_barrier(int leave_in_flight, const u32x4 &f0, const u32x4 &f1, u32x4 &o0,
+                                                  u32x4 &o1) {
+  // loads complete in issue order: leaving the youngest ones in flight (the feature fragments and the
+  // weight chunk requested one round ago) still guarantees that the chunk about to be used has landed
+  if (leave_in_flight >= 4)
+    PCE_PIPE_WAIT_COPY(4);
+  else
+    PCE_PIPE_WAIT_COPY(0);
+}
+#undef PCE_PIPE_WAIT_COPY
 
 // this wavefront's quarter of the weight chunk (k0 .. k0+31, columns n0 .. n0+127) -> LDS stage
 __device__ __forceinline__ void pipe_issue_weights(const half_t *Wk, int k0, int n0, int n_pad, half8 *stage, int wave,
@@ -890,12 +914,11 @@ __device__ __forceinline__ void pipe_issue_weights(const half_t *Wk, int k0, int
 }
 
 // always issued (row 0 stands in for a missing row; the caller zeroes it when the fragment is taken into
-// use): the wait before the barrier relies on at least two loads younger than the weight chunk it
-// waits for
-__device__ __forceinline__ void pipe_load_rows(half8 (&af)[2], const half_t *A, int arow, int c_in, int k0, int g) {
+// use): the wait before the barrier counts the loads of a round
+__device__ __forceinline__ void pipe_load_rows(u32x4 (&raw)[2], const half_t *A, int arow, int c_in, int k0, int g) {
   int r = arow >= 0 ? arow : 0;
 #pragma unroll
-  for (int s2 = 0; s2 < 2; ++s2) af[s2] = *reinterpret_cast<const half8 *>(A + (long long)r * c_in + k0 + s2 * 16 + g * 8);
+  for (int s2 = 0; s2 < 2; ++s2) raw[s2] = load16_untracked(A + (long long)r * c_in + k0 + s2 * 16 + g * 8);
 }
 
 template <int PMODE>
@@ -908,10 +931,11 @@ __global__ void __launch_bounds__(256, 4) pipe_gemm_kernel(TileArgs a) {
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int l32 = lane & 31, g = lane >> 5;
-  const long long item = blockIdx.x;
-  if (item >= a.items) return;
-  const long long tile = item / a.slabs;
-  const int n0 = (int)(item % a.slabs) * NT;
+  // contiguous item ranges per XCD: the column slabs of a tile, and the tiles of one offset, share an L2
+  long long tile;
+  int slab;
+  if (!xcd_item(a.items, a.slabs, true, &tile, &slab)) return;
+  const int n0 = slab * NT;
   const half_t *A = (const half_t *)a.A;
   const int kch = a.c_in / KC;
 
@@ -939,38 +963,49 @@ __global__ void __launch_bounds__(256, 4) pipe_gemm_kernel(TileArgs a) {
 #pragma unroll
     for (int j = 0; j < 16; ++j) acc[nb][j] = 0.f;
 
-  // prologue: weight chunks 0 and 1, feature chunk 0
+  // prologue: weight chunks 0 and 1, feature chunks 0 and 1 (issue order: W0, A0, W1, A1)
+  u32x4 raw[2][2];
   pipe_issue_weights(Wk, 0, n0, a.n_pad, lds, wave, lane);
-  if (kch > 1) pipe_issue_weights(Wk, KC, n0, a.n_pad, lds + STAGE, wave, lane);
-  half8 af[2], raw[2];
-  pipe_load_rows(raw, A, arow, a.c_in, 0, g);
+  pipe_load_rows(raw[0], A, arow, a.c_in, 0, g);
+  if (kch > 1) {
+    pipe_issue_weights(Wk, KC, n0, a.n_pad, lds + STAGE, wave, lane);
+    pipe_load_rows(raw[1], A, arow, a.c_in, KC, g);
+  }
   const bool wave_has = __ballot(arow >= 0) != 0ull;
   const half8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
   int st = 0, st2 = 2 % PIPE_ST;
-  for (int t = 0; t < kch; ++t) {
-    pipe_wait_barrier(t + 1 < kch);
-    // the fragments requested one round ago become the operands of this round
-#pragma unroll
-    for (int s2 = 0; s2 < 2; ++s2) af[s2] = arow >= 0 ? raw[s2] : zero;
-    // features of chunk t+1 first, so that the weight loads below are the youngest in flight
-    if (t + 1 < kch) pipe_load_rows(raw, A, arow, a.c_in, (t + 1) * KC, g);
-    // weight chunk t+2 -> the stage that chunk t-1 has just released
-    if (t + 2 < kch) {
-      pipe_issue_weights(Wk, (t + 2) * KC, n0, a.n_pad, lds + st2 * STAGE, wave, lane);
-      st2 = st2 + 1 == PIPE_ST ? 0 : st2 + 1;
-    }
-    if (wave_has) {
-      const half8 *stp = lds + st * STAGE;
-#pragma unroll
-      for (int s2 = 0; s2 < 2; ++s2)
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-          half8 b = stp[(2 * s2 + g) * NT + nb * 32 + l32];
-          acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b, af[s2], acc[nb], 0, 0, 0);
-        }
-    }
-    st = st + 1 == PIPE_ST ? 0 : st + 1;
+  // One round: the features of chunk t were requested two rounds ago, its weights too.  Everything
+  // issued before the weights of chunk t has landed once at most the loads of the previous round (the
+  // features of chunk t+1, the weights of chunk t+1) are still in flight.
+#define PCE_PIPE_ROUND(T_, SLOT_)                                                                          \
+  {                                                                                                        \
+    const int t = (T_);                                                                                    \
+    u32x4 landed[2];                                                                                       \
+    pipe_wait_barrier(4 * (t + 1 < kch), raw[SLOT_][0], raw[SLOT_][1], landed[0], landed[1]);              \
+    half8 af[2];                                                                                           \
+    _Pragma("unroll") for (int s2 = 0; s2 < 2; ++s2)                                                       \
+        af[s2] = arow >= 0 ? __builtin_bit_cast(half8, landed[s2]) : zero;                                 \
+    /* features of chunk t+2 first, so that the weight loads below are the youngest in flight */           \
+    if (t + 2 < kch) {                                                                                     \
+      pipe_load_rows(raw[SLOT_], A, arow, a.c_in, (t + 2) * KC, g);                                        \
+      /* weight chunk t+2 -> the stage that chunk t-1 has just released */                                 \
+      pipe_issue_weights(Wk, (t + 2) * KC, n0, a.n_pad, lds + st2 * STAGE, wave, lane);                    \
+      st2 = st2 + 1 == PIPE_ST ? 0 : st2 + 1;                                                              \
+    }                                                                                                      \
+    if (wave_has) {                                                                                        \
+      const half8 *stp = lds + st * STAGE;                                                                 \
+      _Pragma("unroll") for (int s2 = 0; s2 < 2; ++s2) _Pragma("unroll") for (int nb = 0; nb < NB; ++nb) { \
+        half8 b = stp[(2 * s2 + g) * NT + nb * 32 + l32];                                                  \
+        acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b, af[s2], acc[nb], 0, 0, 0);                     \
+      }                                                                                                    \
+    }                                                                                                      \
+    st = st + 1 == PIPE_ST ? 0 : st + 1;                                                                   \
   }
+  for (int t0 = 0; t0 < kch; t0 += 2) {
+    PCE_PIPE_ROUND(t0, 0)
+    if (t0 + 1 < kch) PCE_PIPE_ROUND(t0 + 1, 1)
+  }
+#undef PCE_PIPE_ROUND
   __syncthreads();  // the ring becomes the epilogue staging area
   float V[NB][2][8];
   gather_row_pieces<NB>(acc, V, g);
@@ -995,10 +1030,11 @@ static int launch_pipe_gemm(TileArgs a, long long tiles, hipStream_t s) {
   a.slabs = (a.c_out + 127) / 128;
   a.items = tiles * a.slabs;
   if (a.items >= (1ll << 31) - 8) PCE_FAIL(PCE_ECAPACITY, "tile count %lld exceeds the grid limit", tiles);
+  const unsigned grid = (unsigned)(pce_div_up(a.items, PCE_XCDS) * PCE_XCDS);
   if (a.mode == MODE_DENSE)
-    hipLaunchKernelGGL((pipe_gemm_kernel<MODE_DENSE>), dim3((unsigned)a.items), dim3(256), 0, s, a);
+    hipLaunchKernelGGL((pipe_gemm_kernel<MODE_DENSE>), dim3(grid), dim3(256), 0, s, a);
   else
-    hipLaunchKernelGGL((pipe_gemm_kernel<MODE_FOD_BUF>), dim3((unsigned)a.items), dim3(256), 0, s, a);
+    hipLaunchKernelGGL((pipe_gemm_kernel<MODE_FOD_BUF>), dim3(grid), dim3(256), 0, s, a);
   PCE_LAUNCH_CHECK("pipe_gemm");
   return PCE_OK;
 }
