@@ -171,7 +171,7 @@ def main() -> int:
                    DATAFLOW_OS: {1: "os_tile"}}[flow]
     if flow != DATAFLOW_OS:
         for bit, name in stage_names.items():
-            lib.pce_set_stage_mask((1 << bit) | 16)       # bit 4 keeps the kernel selection of the full run
+            lib.pce_set_stage_mask((1 << bit) | 0xFFFFFFF0)   # bits 4 and up keep the kernel selection of the full run
             stages[name] = timer(step, max(20, args.steps // 4), 5)[0]
         lib.pce_set_stage_mask(0xFFFFFFFF)
     else:
