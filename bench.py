@@ -202,7 +202,7 @@ def main() -> int:
     achieved = dom_bytes / (stages[dom] * 1e-3) / 1e9
     # HBM bytes per launch of that kernel from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
     # profiles/pmc_traffic_cfg2.md (scaled by the copy-kernel calibration); counters cannot be read here
-    measured_traffic = {("cfg2", "centre_gemm_csr_sum"): 43.46e6, ("cfg2", "pairs_and_centre_gemm"): 47.54e6}
+    measured_traffic = {("cfg2", "centre_gemm_csr_sum"): 43.46e6, ("cfg2", "pairs_and_centre_gemm"): 47.09e6}
     if args.workload in ("cfg2", "cfg2x8"):
         roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic.get((args.workload, dom)),
