@@ -1,0 +1,84 @@
+"""Configurations 3 and 5 at their full sizes: parity with the oracle where it finishes in seconds, and
+properties that hold at any size (every dataflow computes the same sums; map symmetries; sortedness)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+from pcengine_amd import backend, synth
+from pcengine_amd.backend import DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS, DATAFLOW_FDS
+from tests.util import DEV, assert_map_equal, dev_coords, gpu_map, rounded
+
+pytestmark = pytest.mark.gpu
+
+FLOWS = [DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS, DATAFLOW_FDS]
+
+
+def test_config3_down_then_transposed_up_full_size():
+    """k2s2 64->128 on the 150 k-voxel LiDAR cloud, then the transposed layer 128->64 back onto the input
+    coordinates over the same map (script/spconv.py:306-329)."""
+    coords = synth.lidar_cloud()
+    ks, st, pad = (2, 2, 2), (2, 2, 2), (0, 0, 0)
+    ref = orc.kernel_map(coords, ks, st, pad)
+    km = gpu_map(coords, ks, st, pad, want_csr=True, want_nbr_in=True, batchsize=1)
+    assert_map_equal(km, ref, csr=True)
+    f = synth.features(3, len(coords), 64)
+    w_down = synth.weights(3, 8, 64, 128)
+    w_up = synth.weights(4, 8, 128, 64)
+    dt = torch.float16
+    mid_want = orc.conv_forward(rounded(f, dt), rounded(w_down, dt), ref, ks)
+    fd = torch.as_tensor(f, device=DEV).to(dt)
+    wd, wu = (torch.as_tensor(w, device=DEV).to(dt) for w in (w_down, w_up))
+    for flow in FLOWS:
+        mid = backend.conv_forward(fd, wd, km, flow)
+        assert orc.rel_l2(mid.double().cpu().numpy(), mid_want) <= 1e-3, flow
+        # the transposed layer sees the fp16 rows the down layer stored
+        up_want = orc.conv_forward(mid.double().cpu().numpy(), rounded(w_up, dt), ref, ks, transposed=True)
+        up = backend.conv_forward(mid, wu, km, flow, transposed=True)
+        assert up.shape == (len(coords), 64)
+        assert orc.rel_l2(up.double().cpu().numpy(), up_want) <= 1e-3, flow
+
+
+def test_config5_indoor_batch_full_size():
+    """Eight indoor scenes, ~954 k voxels: the submanifold map against the oracle, its symmetry, and the
+    four dataflows against each other and against linearity on a C 64 layer."""
+    coords = synth.indoor_batch()
+    n = len(coords)
+    assert 900_000 < n < 1_000_000 and coords[:, 0].max() == 7
+    km = gpu_map(coords, (3, 3, 3), want_csr=True)
+    ref = orc.kernel_map(coords, (3, 3, 3))
+    assert_map_equal(km, ref, csr=True)
+    # pair (i, o, kp) <=> pair (o, i, kv-1-kp): the mirrored pair list is the same set
+    kp_of = torch.repeat_interleave(torch.arange(27, device=DEV), km.knnz.long())
+    fwd = (kp_of * n + km.imap.long()) * n + km.omap.long()
+    mir = ((26 - kp_of) * n + km.omap.long()) * n + km.imap.long()
+    assert torch.equal(torch.sort(fwd).values, torch.sort(mir).values)
+    # strided level: sorted unique output coordinates; an input is in at most one k2s2 pair (inputs on the
+    # far walls fall outside the reference's output bound, script/spconv.py:358-360, and have none)
+    k2 = gpu_map(coords, (2, 2, 2), (2, 2, 2), batchsize=8)
+    assert_map_equal(k2, orc.kernel_map(coords, (2, 2, 2), (2, 2, 2)))
+    oc = k2.out_coords.cpu().numpy().astype(np.int64)
+    code = ((oc[:, 0] * 3259 + oc[:, 1]) * 3259 + oc[:, 2]) * 3259 + oc[:, 3]
+    assert (np.diff(code) > 0).all()
+    assert torch.unique(k2.imap).numel() == k2.M and k2.M < n
+    f = synth.features(5, n, 64)
+    w = synth.weights(5, 27, 64, 64)
+    fd = torch.as_tensor(f, device=DEV).half()
+    wd = torch.as_tensor(w, device=DEV).half()
+    want = orc.conv_forward(rounded(f, torch.float16), rounded(w, torch.float16), ref, (3, 3, 3))
+    packed = backend.pack_weights(wd)
+    outs = {flow: backend.conv_forward(fd, wd, km, flow, packed=packed) for flow in FLOWS}
+    for flow, out in outs.items():
+        assert orc.rel_l2(out.double().cpu().numpy(), want) <= 1e-3, flow
+    # linearity: conv(2x) == 2 conv(x).  Doubling is exact in fp16 and fp32 except for values stored in the
+    # fp16 subnormal range (spacing 2^-24): the output itself and each of the up to 26 partial rows of a
+    # row.  Such a difference in a partial row (< 1e-7) can also tip the final rounding of the row's sum:
+    # one ulp, on a few elements in a million (none with the output-stationary dataflow, which stores no
+    # partial rows).  A dropped or doubled pair would change an element by ~0.2.
+    for flow in (DATAFLOW_FDS, DATAFLOW_OS):
+        twice = backend.conv_forward(fd * 2, wd, km, flow, packed=packed).float()
+        ref2 = outs[flow].float() * 2
+        diff = (twice - ref2).abs()
+        assert bool((diff <= 2.0 ** -10 * ref2.abs() + 27 * 2.0 ** -23).all()), flow
+        tipped = int((diff > 27 * 2.0 ** -23).sum())
+        assert tipped <= (0 if flow == DATAFLOW_OS else diff.numel() // 100_000), (flow, tipped)
