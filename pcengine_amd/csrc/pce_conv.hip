@@ -921,8 +921,13 @@ __device__ __forceinline__ void pipe_load_rows(u32x4 (&raw)[2], const half_t *A,
   for (int s2 = 0; s2 < 2; ++s2) raw[s2] = load16_untracked(A + (long long)r * c_in + k0 + s2 * 16 + g * 8);
 }
 
+// PMODE = MODE_DENSE or MODE_FOD_BUF: every tile is of that kind and `c` is not read.  PMODE = PIPE_BOTH:
+// the pair tiles of `a` come first, then the centre tiles of `c` (same features, weights and widths; its
+// own output, epilogue and row count) -- the centre GEMM of a deferred-scatter layer is too small to fill
+// the machine by itself and neither kind of tile reads what the other writes.
+#define PIPE_BOTH 100
 template <int PMODE>
-__global__ void __launch_bounds__(256, 4) pipe_gemm_kernel(TileArgs a) {
+__global__ void __launch_bounds__(256, 4) pipe_gemm_kernel(TileArgs a, TileArgs c) {
   constexpr int NB = PIPE_NB, NT = 128, KC = PIPE_KC;
   constexpr int STAGE = (KC / 8) * NT;                       // fragments per stage
   constexpr int RING = PIPE_ST * STAGE;
@@ -934,16 +939,21 @@ __global__ void __launch_bounds__(256, 4) pipe_gemm_kernel(TileArgs a) {
   // contiguous item ranges per XCD: the column slabs of a tile, and the tiles of one offset, share an L2
   long long tile;
   int slab;
-  if (!xcd_item(a.items, a.slabs, true, &tile, &slab)) return;
+  if (!xcd_item(PMODE == PIPE_BOTH ? a.items + c.items : a.items, a.slabs, true, &tile, &slab)) return;
   const int n0 = slab * NT;
   const half_t *A = (const half_t *)a.A;
   const int kch = a.c_in / KC;
+  // the argument block is never selected as a whole at run time (that would copy it to private memory)
+  const long long pair_tiles = PMODE == PIPE_BOTH ? a.items / a.slabs : 0;
+  const bool dense = PMODE == MODE_DENSE || (PMODE == PIPE_BOTH && tile >= pair_tiles);
+  const long long n_rows = PMODE == PIPE_BOTH ? c.n_rows : a.n_rows;
+  const int w_fixed = PMODE == PIPE_BOTH ? c.w_fixed : a.w_fixed;
 
   int orow = -1, arow = -1, widx;
-  if (PMODE == MODE_DENSE) {
-    long long row = tile * 128 + wave * 32 + l32;
-    orow = arow = row < a.n_rows ? (int)row : -1;
-    widx = a.w_fixed;
+  if (dense) {
+    long long row = (tile - pair_tiles) * 128 + wave * 32 + l32;
+    orow = arow = row < n_rows ? (int)row : -1;
+    widx = w_fixed;
   } else {  // pair tile: one 128-pair quantum of one offset
     long long q0 = tile * 128;
     widx = 0;
@@ -1009,12 +1019,19 @@ __global__ void __launch_bounds__(256, 4) pipe_gemm_kernel(TileArgs a) {
   __syncthreads();  // the ring becomes the epilogue staging area
   float V[NB][2][8];
   gather_row_pieces<NB>(acc, V, g);
-  if (a.bias || a.res || a.act) {
+  if (PMODE == PIPE_BOTH) {
+    if (dense && (c.bias || c.res || c.act)) {
+      bool with_act = c.act != PCE_ACT_NONE;
+      if (with_act && c.act_alone_only) with_act = orow >= 0 && c.ocsr[orow] == c.ocsr[orow + 1];
+      epilogue_row_pieces<half_t, NB, true>(V, c, orow, n0, g, with_act);
+    }
+  } else if (a.bias || a.res || a.act) {
     bool with_act = a.act != PCE_ACT_NONE;
     if (with_act && a.act_alone_only) with_act = orow >= 0 && a.ocsr[orow] == a.ocsr[orow + 1];
     epilogue_row_pieces<half_t, NB, true>(V, a, orow, n0, g, with_act);
   }
-  store_rows_via_lds<half_t, NB>(V, lds + wave * WaveLds<NB>::PIECES, (half_t *)a.out, orow, a, n0, lane, l32, g);
+  half_t *out = (half_t *)((PMODE == PIPE_BOTH && dense) ? c.out : a.out);
+  store_rows_via_lds<half_t, NB>(V, lds + wave * WaveLds<NB>::PIECES, out, orow, a, n0, lane, l32, g);
 }
 
 static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
@@ -1032,9 +1049,23 @@ static int launch_pipe_gemm(TileArgs a, long long tiles, hipStream_t s) {
   if (a.items >= (1ll << 31) - 8) PCE_FAIL(PCE_ECAPACITY, "tile count %lld exceeds the grid limit", tiles);
   const unsigned grid = (unsigned)(pce_div_up(a.items, PCE_XCDS) * PCE_XCDS);
   if (a.mode == MODE_DENSE)
-    hipLaunchKernelGGL((pipe_gemm_kernel<MODE_DENSE>), dim3(grid), dim3(256), 0, s, a);
+    hipLaunchKernelGGL((pipe_gemm_kernel<MODE_DENSE>), dim3(grid), dim3(256), 0, s, a, a);
   else
-    hipLaunchKernelGGL((pipe_gemm_kernel<MODE_FOD_BUF>), dim3(grid), dim3(256), 0, s, a);
+    hipLaunchKernelGGL((pipe_gemm_kernel<MODE_FOD_BUF>), dim3(grid), dim3(256), 0, s, a, a);
+  PCE_LAUNCH_CHECK("pipe_gemm");
+  return PCE_OK;
+}
+
+// pair tiles (a: MODE_FOD_BUF) and centre tiles (c: MODE_DENSE) of one layer in one launch
+static int launch_pipe_both(TileArgs a, long long pair_tiles, TileArgs c, long long centre_tiles, hipStream_t s) {
+  a.slabs = c.slabs = (a.c_out + 127) / 128;
+  a.items = pair_tiles * a.slabs;
+  c.items = centre_tiles * c.slabs;
+  const long long items = a.items + c.items;
+  if (items <= 0) return PCE_OK;
+  if (items >= (1ll << 31) - 8) PCE_FAIL(PCE_ECAPACITY, "tile count %lld exceeds the grid limit", items);
+  const unsigned grid = (unsigned)(pce_div_up(items, PCE_XCDS) * PCE_XCDS);
+  hipLaunchKernelGGL((pipe_gemm_kernel<PIPE_BOTH>), dim3(grid), dim3(256), 0, s, a, c);
   PCE_LAUNCH_CHECK("pipe_gemm");
   return PCE_OK;
 }
@@ -1695,6 +1726,28 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
     a.qkpos = qkpos;
     a.mode = MODE_FOD_BUF;
     a.epi = EPI_ROWS;
+    if (mid >= 0 && omap && stage_on(2) && stage_on(4) && stage_on(5) && stage_on(6) && qsum <= 4 * n_out &&
+        pce_div_up(n_out, 128) * ((c_out + 127) / 128) < 2048 && pipe_gemm_ok(a, sizeof(T))) {
+      // wide fp16 layer with few pairs per row: pair tiles and the plain centre GEMM (bias and residual fused,
+      // activation on rows without partial rows) share one launch, then the pass that adds each row's partial
+      // rows.  Measured: 24 instead of 31 us at 0.3 pairs per row (C 96), 55 instead of 61 at 2.4 (C 128), equal
+      // at 9 (C 128), 4-6 % slower at 9-13 pairs per row with 256 channels, where the launches stay separate;
+      // so do those of a centre GEMM that fills the machine twice over by itself (nothing to gain, and a
+      // network on 954 k voxels ran 3 % slower with them combined).
+      TileArgs c = base_args<T>(in, w, wp, kv, c_in, c_out);
+      set_out<T>(&c, out, false);
+      c.mode = MODE_DENSE;
+      c.epi = EPI_ROWS;
+      c.w_fixed = mid;
+      c.n_rows = n_out;
+      c.ocsr = ocsr;
+      c.act_alone_only = 1;
+      set_epi(&c, e);
+      if (pipe_gemm_ok(c, sizeof(T))) {
+        if ((rc = launch_pipe_both(a, qsum / PCE_QUANTUM, c, pce_div_up(n_out, 128), s))) return rc;
+        return launch_rowsum_pairs<T>((const T *)buffer, (T *)out, n_out, n_pairs, c_out, omap, oslot, ocsr, e.act, e.slope, s);
+      }
+    }
     if (a.host_pos && wave_gemm_ok(a, sizeof(T)) && stage_on(4)) {
       TileArgs none = a;
       none.items = 0;
