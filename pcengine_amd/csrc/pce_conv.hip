@@ -1873,86 +1873,145 @@ extern "C" int pce_conv_fwd_dense(const void *in, const void *w, const void *wp,
   return dense_impl<float>(in, w, wp, out, n, c_in, c_out, e, s);
 }
 
-// ---- weight gradient ------------------------------------------------------------------------------
-// grad_W[kp][ci][co] = sum over the pairs p of offset kp of in[imap[p]][ci] * grad_out[omap[p]][co]
-// (ConvolutionBackwardD1's per-offset GEMM, backend/spconv.cu:400-629).  A workgroup takes one
-// 128-pair quantum (or 128 rows of the centre offset) and a 64 x 64 block of (ci, co): rows are staged
-// in LDS 32 at a time as fp32, every thread accumulates a 4 x 4 block in registers and adds it to the
-// fp32 result with atomics (the order of the additions, and so the last bits, vary from run to run).
-template <typename T>
+// Kernel gradient: gw[kp][ci][co] = sum over the pairs p of offset kp of in[imap[p]][ci] * gout[omap[p]][co]
+// (ConvolutionBackwardD1's per-offset GEMM, backend/spconv.cu:400-629): per offset a GEMM whose reduction
+// runs over the pairs.  A workgroup owns a BLK x BLK block of (ci, co) and a run of consecutive 128-pair
+// quanta (then 128-row tiles of the centre offset); its four wavefronts hold (BLK/2) x (BLK/2) each in
+// fp32 MFMA accumulators (v_mfma_f32_32x32x2_f32, also for fp16 tensors: they are widened when staged, and
+// with the pair index as the reduction index the fp16 MFMA would need its operands transposed).  Rows
+// are staged in LDS 32 pairs at a time.  The accumulators are added to the fp32 result with atomics only
+// when the offset changes or the run ends: one atomic per element per run instead of one per quantum (the
+// order of the additions, and so the last bits, still vary from run to run).
+#define WGRAD_KP 32   // pairs per LDS stage
+
+// PER consecutive channels of one row as fp32 (zeros for a missing row or past the last channel)
+template <typename T, int PER>
+__device__ __forceinline__ void wgrad_fetch(float (&v)[PER], const T *__restrict__ base, int row, int c_total, int c0,
+                                            bool vec) {
+  constexpr int EPV = 16 / (int)sizeof(T);
+  typedef typename VecOfC<T, EPV>::type V;
+  if (vec) {
+#pragma unroll
+    for (int q = 0; q < PER / EPV; ++q) {
+      V x;
+#pragma unroll
+      for (int j = 0; j < EPV; ++j) x[j] = (T)0;
+      if (row >= 0) x = *reinterpret_cast<const V *>(base + (long long)row * c_total + c0 + q * EPV);
+#pragma unroll
+      for (int j = 0; j < EPV; ++j) v[q * EPV + j] = (float)x[j];
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < PER; ++j) v[j] = (row >= 0 && c0 + j < c_total) ? (float)base[(long long)row * c_total + c0 + j] : 0.f;
+  }
+}
+template <typename T, int BLK>
 __global__ void __launch_bounds__(256) wgrad_kernel(const T *__restrict__ in, const T *__restrict__ gout, long long n_rows,
                                                     int c_in, int c_out, int kv, int mid, const int *__restrict__ imap,
                                                     const int *__restrict__ omap, const int *__restrict__ kpos,
-                                                    const int *__restrict__ qkpos, long long pair_tiles, int ci_tiles,
-                                                    int co_tiles, float *__restrict__ gw) {
-  __shared__ float As[32][64 + 4];
-  __shared__ float Gs[32][64 + 4];
+                                                    const int *__restrict__ qkpos, long long pair_tiles, long long tiles,
+                                                    int run, int ci_blocks, int co_blocks, float *__restrict__ gw) {
+  constexpr int R = BLK / 64;              // 32x32 MFMA tiles per wavefront and dimension
+  constexpr int LD = BLK + 32;             // row stride in floats: the two k rows an MFMA reads fall into different banks
+  constexpr int PER = BLK / 8;             // channels a thread stages per row
+  __shared__ float As[WGRAD_KP][LD];
+  __shared__ float Gs[WGRAD_KP][LD];
   __shared__ int rows_in[128], rows_out[128];
-  long long tile = blockIdx.x / (ci_tiles * co_tiles);
-  int rest = (int)(blockIdx.x % (ci_tiles * co_tiles));
-  const int ci0 = (rest / co_tiles) * 64, co0 = (rest % co_tiles) * 64;
-  int widx;
-  if (tile < pair_tiles) {
-    long long q0 = tile * 128;
-    widx = 0;
-    for (int i = 0; i < kv; ++i) widx += ((long long)qkpos[i + 1] <= q0) ? 1 : 0;
-    if (widx >= kv) return;
-    if (threadIdx.x < 128) {
-      long long p = q0 - qkpos[widx] + kpos[widx] + threadIdx.x;
-      bool ok = p < (long long)kpos[widx + 1];
-      rows_in[threadIdx.x] = ok ? imap[p] : -1;
-      rows_out[threadIdx.x] = ok ? omap[p] : -1;
-    }
-  } else {  // centre offset of a submanifold layer: every row pairs with itself
-    widx = mid;
-    if (threadIdx.x < 128) {
-      long long row = (tile - pair_tiles) * 128 + threadIdx.x;
-      rows_in[threadIdx.x] = rows_out[threadIdx.x] = row < n_rows ? (int)row : -1;
-    }
-  }
-  __syncthreads();
-  const int tci = (threadIdx.x / 16) * 4, tco = (threadIdx.x % 16) * 4;
-  float acc[4][4];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int l32 = lane & 31, g = lane >> 5;
+  const int wr = wave >> 1, wc = wave & 1;
+  const long long grp = blockIdx.x / (ci_blocks * co_blocks);
+  const int rest = (int)(blockIdx.x % (ci_blocks * co_blocks));
+  const int ci0 = (rest / co_blocks) * BLK, co0 = (rest % co_blocks) * BLK;
+
+  f32x16 acc[R][R];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < R; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
-  for (int p0 = 0; p0 < 128; p0 += 32) {
-    // stage 32 rows x 64 channels of both operands: 8 elements per thread and matrix
-    {
-      int r = threadIdx.x / 8, c = (threadIdx.x % 8) * 8;
-      int ri = rows_in[p0 + r], ro = rows_out[p0 + r];
+    for (int j = 0; j < R; ++j)
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        int ci = ci0 + c + j, co = co0 + c + j;
-        As[r][c + j] = (ri >= 0 && ci < c_in) ? (float)in[(long long)ri * c_in + ci] : 0.f;
-        Gs[r][c + j] = (ro >= 0 && co < c_out) ? (float)gout[(long long)ro * c_out + co] : 0.f;
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  int cur = -1;  // offset the accumulators belong to
+
+  auto flush = [&](int widx) {
+    float *dst = gw + (long long)widx * c_in * c_out;
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+#pragma unroll
+      for (int j = 0; j < R; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          int ci = ci0 + wr * (BLK / 2) + i * 32 + (e / 4) * 8 + g * 4 + (e % 4);
+          int co = co0 + wc * (BLK / 2) + j * 32 + l32;
+          float v = acc[i][j][e];
+          if (ci < c_in && co < c_out && v != 0.f) unsafeAtomicAdd(dst + (long long)ci * c_out + co, v);
+          acc[i][j][e] = 0.f;
+        }
+  };
+
+  // 16-byte loads when a thread's channels lie inside the tensor and its rows are 16-byte multiples
+  constexpr int EPV = 16 / (int)sizeof(T);
+  const bool vec_in = (c_in % EPV == 0) && ci0 + BLK <= c_in && (((uintptr_t)in) & 15) == 0;
+  const bool vec_out = (c_out % EPV == 0) && co0 + BLK <= c_out && (((uintptr_t)gout) & 15) == 0;
+  const long long t_end = (grp + 1) * run < tiles ? (grp + 1) * run : tiles;
+  for (long long tile = grp * run; tile < t_end; ++tile) {
+    int widx;
+    __syncthreads();  // rows_in / rows_out of the previous tile are no longer read
+    if (tile < pair_tiles) {
+      long long q0 = tile * 128;
+      widx = 0;
+      for (int i = 0; i < kv; ++i) widx += ((long long)qkpos[i + 1] <= q0) ? 1 : 0;
+      if (widx >= kv) break;  // uniform
+      if (threadIdx.x < 128) {
+        long long p = q0 - qkpos[widx] + kpos[widx] + threadIdx.x;
+        bool ok = p < (long long)kpos[widx + 1];
+        rows_in[threadIdx.x] = ok ? imap[p] : -1;
+        rows_out[threadIdx.x] = ok ? omap[p] : -1;
+      }
+    } else {  // centre offset of a submanifold layer: every row pairs with itself
+      widx = mid;
+      if (threadIdx.x < 128) {
+        long long row = (tile - pair_tiles) * 128 + threadIdx.x;
+        rows_in[threadIdx.x] = rows_out[threadIdx.x] = row < n_rows ? (int)row : -1;
       }
     }
+    if (cur >= 0 && widx != cur) flush(cur);
+    cur = widx;
     __syncthreads();
-#pragma unroll 8
-    for (int k = 0; k < 32; ++k) {
-      float av[4], gv[4];
+    // stage 32 rows x BLK channels of both operands as fp32: PER consecutive channels per thread and matrix.
+    // The rows of stage s+1 are requested before the MFMAs of stage s.
+    const int r = threadIdx.x / 8, c = (threadIdx.x % 8) * PER;
+    float va[PER], vg[PER];
+    auto fetch = [&](int p0) {
+      const int ri = rows_in[p0 + r], ro = rows_out[p0 + r];
+      wgrad_fetch<T, PER>(va, in, ri, c_in, ci0 + c, vec_in);
+      wgrad_fetch<T, PER>(vg, gout, ro, c_out, co0 + c, vec_out);
+    };
+    fetch(0);
+    for (int p0 = 0; p0 < 128; p0 += WGRAD_KP) {
+      __syncthreads();  // the MFMAs of the previous stage have read their operands
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        av[i] = As[k][tci + i];
-        gv[i] = Gs[k][tco + i];
+      for (int j = 0; j < PER; ++j) {
+        As[r][c + j] = va[j];
+        Gs[r][c + j] = vg[j];
       }
+      __syncthreads();
+      if (p0 + WGRAD_KP < 128) fetch(p0 + WGRAD_KP);
+#pragma unroll 4
+      for (int k = 0; k < WGRAD_KP; k += 2) {
+        float av[R], bv[R];
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < R; ++i) av[i] = As[k + g][wr * (BLK / 2) + i * 32 + l32];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] += av[i] * gv[j];
+        for (int j = 0; j < R; ++j) bv[j] = Gs[k + g][wc * (BLK / 2) + j * 32 + l32];
+#pragma unroll
+        for (int i = 0; i < R; ++i)
+#pragma unroll
+          for (int j = 0; j < R; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[j], acc[i][j], 0, 0, 0);
+      }
     }
-    __syncthreads();
   }
-  float *dst = gw + (long long)widx * c_in * c_out;
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      int ci = ci0 + tci + i, co = co0 + tco + j;
-      if (ci < c_in && co < c_out && acc[i][j] != 0.f) unsafeAtomicAdd(dst + (long long)ci * c_out + co, acc[i][j]);
-    }
+  if (cur >= 0) flush(cur);
 }
 
 extern "C" int pce_conv_wgrad(const void *in, const void *gout, int32_t dtype, int64_t n_in, int64_t n_out, int32_t c_in,
@@ -1967,16 +2026,28 @@ extern "C" int pce_conv_wgrad(const void *in, const void *gout, int32_t dtype, i
   PCE_LAUNCH_CHECK("zero_f32");
   long long pair_tiles = qsum / PCE_QUANTUM;
   long long tiles = pair_tiles + (mid >= 0 ? pce_div_up(n_out, 128) : 0);
-  int ci_tiles = (c_in + 63) / 64, co_tiles = (c_out + 63) / 64;
-  long long blocks = tiles * ci_tiles * co_tiles;
-  if (blocks <= 0) return PCE_OK;
+  if (tiles <= 0) return PCE_OK;
+  // 128 x 128 blocks of (ci, co) for wide layers, 64 x 64 otherwise; runs of tiles long enough to leave about
+  // two thousand workgroups (every run ends with one atomic per element of its block)
+  const int blk = (c_in > 64 || c_out > 64) ? 128 : 64;
+  const int ci_blocks = (c_in + blk - 1) / blk, co_blocks = (c_out + blk - 1) / blk;
+  long long run = tiles * ci_blocks * co_blocks / 2048;
+  run = run < 1 ? 1 : (run > 64 ? 64 : run);
+  long long blocks = pce_div_up(tiles, run) * ci_blocks * co_blocks;
   if (blocks >= (1ll << 31)) PCE_FAIL(PCE_ECAPACITY, "pce_conv_wgrad: %lld workgroups exceed the grid limit", blocks);
-  if (dtype == PCE_F16)
-    hipLaunchKernelGGL(wgrad_kernel<half_t>, dim3((unsigned)blocks), dim3(256), 0, s, (const half_t *)in, (const half_t *)gout,
-                       (long long)n_out, c_in, c_out, kv, mid, imap, omap, kpos, qkpos, pair_tiles, ci_tiles, co_tiles, gw);
+#define PCE_WGRAD(T_, BLK_)                                                                                              \
+  hipLaunchKernelGGL((wgrad_kernel<T_, BLK_>), dim3((unsigned)blocks), dim3(256), 0, s, (const T_ *)in, (const T_ *)gout, \
+                     (long long)n_out, c_in, c_out, kv, mid, imap, omap, kpos, qkpos, pair_tiles, tiles, (int)run,       \
+                     ci_blocks, co_blocks, gw)
+  if (dtype == PCE_F16 && blk == 128)
+    PCE_WGRAD(half_t, 128);
+  else if (dtype == PCE_F16)
+    PCE_WGRAD(half_t, 64);
+  else if (blk == 128)
+    PCE_WGRAD(float, 128);
   else
-    hipLaunchKernelGGL(wgrad_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, s, (const float *)in, (const float *)gout,
-                       (long long)n_out, c_in, c_out, kv, mid, imap, omap, kpos, qkpos, pair_tiles, ci_tiles, co_tiles, gw);
+    PCE_WGRAD(float, 64);
+#undef PCE_WGRAD
   PCE_LAUNCH_CHECK("wgrad");
   return PCE_OK;
 }

@@ -98,3 +98,21 @@ def test_unet_training_step_produces_finite_gradients():
                          coords[:, 1:].max(0).tolist())
         after = float(torch.nn.functional.cross_entropy(model(x2).feats, target))
     assert after < before
+
+
+@pytest.mark.parametrize("dtype,c_in,c_out", [(torch.float32, 16, 24), (torch.float16, 72, 136)])
+def test_kernel_gradient_long_runs(dtype, c_in, c_out):
+    """Enough pairs that a workgroup of the kernel-gradient kernel takes a run of several 128-pair quanta
+    and crosses from one offset to the next inside the run (its accumulators are flushed there), with
+    channel counts that leave partial blocks."""
+    coords = synth.random_cloud(seed=81, n=70000, extent=42)
+    ref = orc.kernel_map(coords, (3, 3, 3))
+    assert (ref.M // 128 + len(coords) // 128) * (1 if c_in <= 64 and c_out <= 64 else 4) >= 2 * 2048
+    f = synth.features(12, len(coords), c_in)
+    go = synth.features(13, len(coords), c_out)
+    w = synth.weights(12, 27, c_in, c_out)
+    _, gw_want = orc.conv_backward(rounded(f, dtype), rounded(w, dtype), ref, (3, 3, 3), rounded(go, dtype))
+    km = gpu_map(coords, (3, 3, 3), want_csr=True)
+    gw = backend.conv_wgrad(torch.as_tensor(f, device=DEV).to(dtype), torch.as_tensor(go, device=DEV).to(dtype), km)
+    assert gw.dtype == torch.float32 and gw.shape == (27, c_in, c_out)
+    assert orc.rel_l2(gw.double().cpu().numpy(), gw_want) <= 1e-5
