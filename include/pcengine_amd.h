@@ -74,7 +74,9 @@ const char *pce_last_error(void);
  * for A/B measurements: 4 = the deferred-scatter forms with a pair-driven row sum (cleared: centre
  * GEMM with the partial-row sum in its epilogue), 5 = the pipelined tile kernel for wide fp16 layers
  * (cleared: the single-stage tile kernel), 6 = pair tiles and centre GEMM of a wide deferred-scatter
- * layer in one launch (cleared: two launches).  Default: all bits set.  Process-wide. */
+ * layer in one launch (cleared: two launches), 9 = the pipelined output-stationary kernel for wide
+ * fp16 layers of few tiles (cleared: the single-stage tile kernel).  Default: all bits set.
+ * Process-wide. */
 void pce_set_stage_mask(uint32_t mask);
 
 /* ---- coordinate hash table: open addressing on the packed (b,x,y,z) 64-bit key ------------- */

@@ -1034,6 +1034,139 @@ __global__ void __launch_bounds__(256, 4) pipe_gemm_kernel(TileArgs a, TileArgs 
   store_rows_via_lds<half_t, NB>(V, lds + wave * WaveLds<NB>::PIECES, out, orow, a, n0, lane, l32, g);
 }
 
+// The eight weight fragments of a step are requested before its first MFMA, and every MFMA waits only for
+// its own fragment (LDS reads return in order).  Left to the compiler the reads are issued two at a time,
+// each pair in front of the MFMAs that use it, which leaves the LDS latency exposed four times per step
+// when few wavefronts share a SIMD.
+__device__ __forceinline__ void step_mfma(f32x16 (&acc)[4], const half8 (&af)[2], const half8 *frag0) {
+  unsigned addr = (unsigned)(uintptr_t)(__attribute__((address_space(3))) void *)frag0;
+  u32x4 b0, b1, b2, b3, b4, b5, b6, b7;
+  asm volatile(
+      "ds_read_b128 %0, %14\n\t"
+      "ds_read_b128 %1, %14 offset:512\n\t"
+      "ds_read_b128 %2, %14 offset:1024\n\t"
+      "ds_read_b128 %3, %14 offset:1536\n\t"
+      "ds_read_b128 %4, %14 offset:4096\n\t"
+      "ds_read_b128 %5, %14 offset:4608\n\t"
+      "ds_read_b128 %6, %14 offset:5120\n\t"
+      "ds_read_b128 %7, %14 offset:5632\n\t"
+      "s_waitcnt lgkmcnt(7)\n\tv_mfma_f32_32x32x16_f16 %8, %0, %12, %8\n\t"
+      "s_waitcnt lgkmcnt(6)\n\tv_mfma_f32_32x32x16_f16 %9, %1, %12, %9\n\t"
+      "s_waitcnt lgkmcnt(5)\n\tv_mfma_f32_32x32x16_f16 %10, %2, %12, %10\n\t"
+      "s_waitcnt lgkmcnt(4)\n\tv_mfma_f32_32x32x16_f16 %11, %3, %12, %11\n\t"
+      "s_waitcnt lgkmcnt(3)\n\tv_mfma_f32_32x32x16_f16 %8, %4, %13, %8\n\t"
+      "s_waitcnt lgkmcnt(2)\n\tv_mfma_f32_32x32x16_f16 %9, %5, %13, %9\n\t"
+      "s_waitcnt lgkmcnt(1)\n\tv_mfma_f32_32x32x16_f16 %10, %6, %13, %10\n\t"
+      "s_waitcnt lgkmcnt(0)\n\tv_mfma_f32_32x32x16_f16 %11, %7, %13, %11"
+      : "=&v"(b0), "=&v"(b1), "=&v"(b2), "=&v"(b3), "=&v"(b4), "=&v"(b5), "=&v"(b6), "=&v"(b7), "+v"(acc[0]),
+        "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3])
+      : "v"(af[0]), "v"(af[1]), "v"(addr)
+      : "memory");
+}
+
+// ---- pipelined output-stationary kernel for wide fp16 layers ----------------------------------------
+// The single-stage tile kernel requests the weight chunk and the gathered rows of a (offset, K chunk) step
+// right before it needs them; a layer of a few hundred tiles is one round of workgroups with nothing
+// else resident to hide that latency (1.6 us per step against 0.2 us of MFMA work on 26 k rows x 256
+// channels).  Here the steps of a tile -- its populated offsets times the K chunks -- form one sequence
+// that runs through the ring of pipe_gemm_kernel: weights global -> LDS and feature fragments by
+// untracked loads, both two steps ahead, one barrier per step.  The neighbour rows of all offsets are
+// read once into LDS; an offset none of the tile's rows has a neighbour at is left out of the sequence,
+// and a wavefront skips the MFMAs of an offset none of its own 32 rows has.
+#define OSP_MAX_KV 32
+__global__ void __launch_bounds__(256, 3) os_pipe_kernel(TileArgs a) {
+  constexpr int NB = PIPE_NB, NT = 128, KC = PIPE_KC;
+  constexpr int STAGE = (KC / 8) * NT;
+  constexpr int RING = PIPE_ST * STAGE;
+  constexpr int EPI = 4 * WaveLds<NB>::PIECES;
+  __shared__ __attribute__((aligned(16))) half8 lds[RING > EPI ? RING : EPI];
+  __shared__ int nbrs[OSP_MAX_KV][128];
+  __shared__ unsigned wave_masks[4];
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int l32 = lane & 31, g = lane >> 5;
+  long long tile;
+  int slab;
+  if (!xcd_item(a.items, a.slabs, true, &tile, &slab)) return;
+  const int n0 = slab * NT;
+  const half_t *A = (const half_t *)a.A;
+  const int kch = a.c_in / KC;
+  const long long row = tile * 128 + wave * 32 + l32;
+  const int orow = row < a.n_rows ? (int)row : -1;
+
+  // neighbour rows of every offset -> LDS; offsets this wavefront / this tile has any neighbour at
+  unsigned wmask = 0;
+  for (int kp = 0; kp < a.kv; ++kp) {
+    int nb_row = orow >= 0 ? a.nbr[(long long)kp * a.n_rows + orow] : -1;
+    if (g == 0) nbrs[kp][wave * 32 + l32] = nb_row;
+    if (__ballot(nb_row >= 0) != 0ull) wmask |= 1u << kp;
+  }
+  if (lane == 0) wave_masks[wave] = wmask;
+  __syncthreads();
+  const unsigned active = wave_masks[0] | wave_masks[1] | wave_masks[2] | wave_masks[3];
+  const int rounds = __popc(active) * kch;
+
+  f32x16 acc[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[nb][j] = 0.f;
+
+  // issue cursor (two steps ahead of the consume cursor): offset, chunk, LDS stage
+  int ikp = active ? __ffs(active) - 1 : -1, it = 0, ist = 0;
+  int ckp = ikp, ct = 0, cst = 0;
+  u32x4 raw[2][2];
+  const half8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  int carow[2] = {-1, -1};   // the row whose fragments sit in raw[slot]
+#define OSP_ISSUE(SLOT_)                                                                                     \
+  {                                                                                                          \
+    const half_t *Wk = (const half_t *)a.Wp + (long long)ikp * a.k8_total * a.n_pad * 8;                     \
+    const int arow_i = nbrs[ikp][wave * 32 + l32];                                                           \
+    carow[SLOT_] = arow_i;                                                                                   \
+    pipe_load_rows(raw[SLOT_], A, arow_i, a.c_in, it * KC, g);                                               \
+    pipe_issue_weights(Wk, it * KC, n0, a.n_pad, lds + ist * STAGE, wave, lane);                             \
+    ist = ist + 1 == PIPE_ST ? 0 : ist + 1;                                                                  \
+    if (++it == kch) {                                                                                       \
+      it = 0;                                                                                                \
+      unsigned rest = ikp >= 31 ? 0u : (active & ~((2u << ikp) - 1u));                                       \
+      ikp = rest ? __ffs(rest) - 1 : -1;                                                                     \
+    }                                                                                                        \
+  }
+  // issue order per step: feature fragments, then weights; the prologue issues steps 0 and 1
+  if (rounds > 0) OSP_ISSUE(0)
+  if (rounds > 1) OSP_ISSUE(1)
+#define OSP_ROUND(R_, SLOT_)                                                                                 \
+  {                                                                                                          \
+    const int r = (R_);                                                                                      \
+    u32x4 landed[2];                                                                                         \
+    /* everything older than the loads of step r+1 (issued one step ago) has landed */                      \
+    pipe_wait_barrier(4 * (r + 1 < rounds), raw[SLOT_][0], raw[SLOT_][1], landed[0], landed[1]);             \
+    half8 af[2];                                                                                             \
+    const int arow_c = carow[SLOT_];                                                                         \
+    _Pragma("unroll") for (int s2 = 0; s2 < 2; ++s2)                                                         \
+        af[s2] = arow_c >= 0 ? __builtin_bit_cast(half8, landed[s2]) : zero;                                 \
+    if (r + 2 < rounds) OSP_ISSUE(SLOT_)                                                                     \
+    if ((wmask >> ckp) & 1u) step_mfma(acc, af, lds + cst * STAGE + g * NT + l32);                           \
+    cst = cst + 1 == PIPE_ST ? 0 : cst + 1;                                                                  \
+    if (++ct == kch) {                                                                                       \
+      ct = 0;                                                                                                \
+      unsigned rest = ckp >= 31 ? 0u : (active & ~((2u << ckp) - 1u));                                       \
+      ckp = rest ? __ffs(rest) - 1 : 0;                                                                      \
+    }                                                                                                        \
+  }
+  for (int r0 = 0; r0 < rounds; r0 += 2) {
+    OSP_ROUND(r0, 0)
+    if (r0 + 1 < rounds) OSP_ROUND(r0 + 1, 1)
+  }
+#undef OSP_ROUND
+#undef OSP_ISSUE
+  __syncthreads();  // the ring becomes the epilogue staging area
+  float V[NB][2][8];
+  gather_row_pieces<NB>(acc, V, g);
+  if (a.bias || a.res || a.act) epilogue_row_pieces<half_t, NB, true>(V, a, orow, n0, g, a.act != PCE_ACT_NONE);
+  store_rows_via_lds<half_t, NB>(V, lds + wave * WaveLds<NB>::PIECES, (half_t *)a.out, orow, a, n0, lane, l32, g);
+}
+
 static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 // shapes the pipelined kernel takes
@@ -1070,6 +1203,22 @@ static int launch_pipe_both(TileArgs a, long long pair_tiles, TileArgs c, long l
   return PCE_OK;
 }
 
+// shapes the pipelined output-stationary kernel takes
+static bool os_pipe_ok(const TileArgs &a, int elem_size) {
+  return elem_size == 2 && a.mode == MODE_OS && a.epi == EPI_ROWS && a.Wp && a.a_vec && a.o_vec && a.c_in % PIPE_KC == 0 &&
+         a.c_in >= 64 && a.c_out >= 96 && a.kv <= OSP_MAX_KV && aligned16(a.bias) && aligned16(a.res);
+}
+
+static int launch_os_pipe(TileArgs a, long long tiles, hipStream_t s) {
+  a.slabs = (a.c_out + 127) / 128;
+  a.items = tiles * a.slabs;
+  if (a.items >= (1ll << 31) - 8) PCE_FAIL(PCE_ECAPACITY, "tile count %lld exceeds the grid limit", tiles);
+  const unsigned grid = (unsigned)(pce_div_up(a.items, PCE_XCDS) * PCE_XCDS);
+  hipLaunchKernelGGL(os_pipe_kernel, dim3(grid), dim3(256), 0, s, a);
+  PCE_LAUNCH_CHECK("os_pipe");
+  return PCE_OK;
+}
+
 static unsigned xcd_grid(TileArgs *a, long long tiles, int slabs) {
   a->slabs = slabs;
   a->items = tiles * slabs;
@@ -1100,6 +1249,9 @@ static int launch_tile(const TileArgs &a, long long tiles, hipStream_t s) {
   if (tiles * ((a.c_out + 127) / 128) >= (1ll << 31) - 8) PCE_FAIL(PCE_ECAPACITY, "tile count %lld exceeds the grid limit", tiles);
   if (stage_on(5) && pipe_gemm_ok(a, sizeof(T)))
     return launch_pipe_gemm(a, tiles, s);
+  // measured: 154 instead of 177 us and 88 instead of 96 us on 406 (tile, slab) items (26 k rows, 256 output
+  // channels), 66 instead of 62 us and 113 instead of 111 us on 515 (66 k rows, 128 output channels)
+  if (stage_on(9) && os_pipe_ok(a, sizeof(T)) && tiles * ((a.c_out + 127) / 128) <= 448) return launch_os_pipe(a, tiles, s);
   bool fast = a.a_vec && a.o_vec && (sizeof(T) == 2 ? a.Wp != nullptr : a.w_vec != 0) &&
               (a.epi != EPI_ROWS_CSR || a.b_vec) && aligned16(a.bias) && aligned16(a.res);
   if (!fast)
