@@ -275,6 +275,41 @@ int pce_conv_fwd_os(const void *in_feats, const void *weight, const void *weight
                     int64_t n_in, int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv,
                     const int32_t *nbr_dev, const pce_epilogue_t *epilogue, pce_stream_t stream);
 
+/* ---- batch normalisation over the rows of a feature matrix ------------------------------------- *
+ * The reference normalises the features of a sparse tensor with torch.nn.BatchNorm1d
+ * (script/batchnorm.py:7-10).  Its forward and backward passes are two column reductions and two
+ * per-column affine maps over feats[n,c] (dtype PCE_F16 or PCE_F32, row-major, device); the c-element
+ * arithmetic between them (mean, variance, running statistics, coefficients) is the caller's.
+ *   pce_col_sums:   out[j] = sum_r a[r][j],  out[c+j] = sum_r a[r][j] * b[r][j]   (b NULL: b = a)
+ *                   fp64 results, same bits every run; ws holds pce_col_sums_workspace_bytes(n, c)
+ *                   forward statistics: (x, NULL); backward: (dy, x)
+ *   pce_col_affine: y[r][j] = act(x[r][j]*kx[j] + d[r][j]*kd[j] + k0[j])   (d, kd NULL: no second term)
+ *                   forward: kx = w*rstd, k0 = b - mean*kx; backward dx: x := dy, d := x,
+ *                   kx = w*rstd, kd = -w*rstd^2*S/n, k0 = -w*rstd*sum(dy)/n + w*rstd^2*mean*S/n,
+ *                   S = sum(dy * xhat).  y may alias x or d. */
+int64_t pce_col_sums_workspace_bytes(int64_t n, int32_t c);
+int pce_col_sums(const void *a_dev, const void *b_dev, int32_t dtype, int64_t n, int32_t c, void *ws_dev,
+                 int64_t ws_bytes, double *out_dev /* [2c] */, pce_stream_t stream);
+int pce_col_affine(const void *x_dev, const void *d_dev, void *y_dev, int32_t dtype, int64_t n, int32_t c,
+                   const float *kx_dev, const float *kd_dev, const float *k0_dev, int32_t act, float slope,
+                   pce_stream_t stream);
+/* The whole pass in one call (three launches: partial sums, one thread per channel for the statistics
+ * and coefficients, the affine map).  weight, bias (fp32 [c], NULL: 1 and 0), running_mean / running_var
+ * (fp32 [c]; updated in place with `momentum` and the unbiased variance when use_batch_stats and
+ * momentum >= 0; read when !use_batch_stats) follow torch.nn.BatchNorm1d.  save_mean / save_rstd (fp32 [c])
+ * receive what pce_bn_backward needs.  grad_weight / grad_bias (fp32 [c]) may be NULL.  ws: device,
+ * pce_bn_workspace_bytes(n, c).  y may alias x; dx may alias dy. */
+int64_t pce_bn_workspace_bytes(int64_t n, int32_t c);
+int pce_bn_forward(const void *x_dev, void *y_dev, int32_t dtype, int64_t n, int32_t c, const float *weight_dev,
+                   const float *bias_dev, float *running_mean_dev, float *running_var_dev,
+                   int32_t use_batch_stats, float momentum, float eps, float *save_mean_dev,
+                   float *save_rstd_dev, void *ws_dev, int64_t ws_bytes, int32_t act, float slope,
+                   pce_stream_t stream);
+int pce_bn_backward(const void *x_dev, const void *dy_dev, void *dx_dev, int32_t dtype, int64_t n, int32_t c,
+                    const float *weight_dev, const float *save_mean_dev, const float *save_rstd_dev,
+                    int32_t use_batch_stats, float *grad_weight_dev, float *grad_bias_dev, void *ws_dev,
+                    int64_t ws_bytes, pce_stream_t stream);
+
 /* out[n,c_out] = in[n,c_in] * weight[c_in,c_out]: the 1x1 stride-1 shortcut of the front end
  * (script/spconv.py:297-304), on the same MFMA tile kernel. */
 int pce_conv_fwd_dense(const void *in_feats, const void *weight, const void *weight_packed,

@@ -70,6 +70,16 @@ _SIGNATURES = {
                                POINTER(c_int32), POINTER(c_int32), c_void_p]),
     "pce_voxelize_emit": (c_int32, [c_void_p, c_int64, c_int64, POINTER(c_int32), POINTER(c_int32), c_int32, c_void_p, c_void_p,
                                     c_void_p, c_void_p]),
+    "pce_col_sums_workspace_bytes": (c_int64, [c_int64, c_int32]),
+    "pce_col_sums": (c_int32, [c_void_p, c_void_p, c_int32, c_int64, c_int32, c_void_p, c_int64, c_void_p, c_void_p]),
+    "pce_col_affine": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_int32,
+                                 ctypes.c_float, c_void_p]),
+    "pce_bn_workspace_bytes": (c_int64, [c_int64, c_int32]),
+    "pce_bn_forward": (c_int32, [c_void_p, c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_int32,
+                                 ctypes.c_float, ctypes.c_float, c_void_p, c_void_p, c_void_p, c_int64, c_int32, ctypes.c_float,
+                                 c_void_p]),
+    "pce_bn_backward": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_int32,
+                                  c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
     "pce_kmap_workspace_bytes": (c_int64, [c_int64, c_int64, c_int32, c_int32]),
     "pce_kmap_build_batch": (c_int32, [POINTER(KmapProblem), c_int32, c_void_p]),
     "pce_kmap_build": (c_int32, [c_void_p, c_int64, c_void_p, c_int64, POINTER(Geom), c_void_p, c_int64] + [c_void_p] * 14 + [c_void_p]),

@@ -381,6 +381,17 @@ def pack_weights(weight: torch.Tensor) -> Optional[torch.Tensor]:
     return packed
 
 
+def _act_code(act) -> Tuple[int, float]:
+    """``act``: None, 'relu', or ('leaky_relu', negative_slope) -> (PCE_ACT_*, slope)."""
+    if act is None:
+        return _lib.ACT_NONE, 0.0
+    if act == "relu":
+        return _lib.ACT_RELU, 0.0
+    if isinstance(act, tuple) and len(act) == 2 and act[0] == "leaky_relu":
+        return _lib.ACT_LEAKY_RELU, float(act[1])
+    raise ValueError(f"unknown activation {act!r}")
+
+
 def _epilogue(feats: torch.Tensor, n_out: int, c_out: int, bias, residual, act):
     """(ctypes struct or None, tensors to keep alive) for ``out = act(conv + bias + residual)``.
     ``act``: None, 'relu', or ('leaky_relu', negative_slope)."""
@@ -401,14 +412,7 @@ def _epilogue(feats: torch.Tensor, n_out: int, c_out: int, bias, residual, act):
         residual = residual.contiguous()
         e.residual = residual.data_ptr()
         keep.append(residual)
-    if act is None:
-        e.act = _lib.ACT_NONE
-    elif act == "relu":
-        e.act = _lib.ACT_RELU
-    elif isinstance(act, tuple) and len(act) == 2 and act[0] == "leaky_relu":
-        e.act, e.slope = _lib.ACT_LEAKY_RELU, float(act[1])
-    else:
-        raise ValueError(f"unknown activation {act!r}")
+    e.act, e.slope = _act_code(act)
     return e, keep
 
 
@@ -504,6 +508,85 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
     else:
         raise NotImplementedError(f"unknown dataflow {dataflow}")
     return out
+
+
+def col_sums(a: torch.Tensor, b: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """float64 [2, c]: column sums of ``a`` [n, c] and of ``a * b`` (``a * a`` without ``b``)."""
+    lib = _lib.load()
+    _require_cuda(a, "a")
+    if a.dim() != 2 or a.dtype not in (torch.float16, torch.float32) or (b is not None and (b.shape != a.shape or b.dtype != a.dtype)):
+        raise ValueError("col_sums takes fp16 or fp32 matrices of one shape and dtype")
+    a = a.contiguous()
+    b = None if b is None else b.contiguous()
+    n, c = a.shape
+    out = torch.empty((2, c), dtype=torch.float64, device=a.device)
+    ws_bytes = lib.pce_col_sums_workspace_bytes(n, c)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=a.device)
+    _lib.check(lib.pce_col_sums(a.data_ptr(), _ptr(b), _dtype_code(a), n, c, ws.data_ptr(), ws_bytes, out.data_ptr(),
+                                _stream(a.device)))
+    return out
+
+
+def col_affine(x: torch.Tensor, kx: torch.Tensor, k0: torch.Tensor, d: Optional[torch.Tensor] = None,
+               kd: Optional[torch.Tensor] = None, act=None) -> torch.Tensor:
+    """``act(x * kx + d * kd + k0)`` with fp32 per-column coefficients; the result has x's dtype."""
+    lib = _lib.load()
+    _require_cuda(x, "x")
+    x = x.contiguous()
+    d = None if d is None else d.contiguous()
+    n, c = x.shape
+    coef = [None if k is None else k.to(device=x.device, dtype=torch.float32).contiguous() for k in (kx, kd, k0)]
+    y = torch.empty_like(x)
+    code, slope = _act_code(act)
+    _lib.check(lib.pce_col_affine(x.data_ptr(), _ptr(d), y.data_ptr(), _dtype_code(x), n, c, _ptr(coef[0]), _ptr(coef[1]),
+                                  _ptr(coef[2]), code, slope, _stream(x.device)))
+    return y
+
+
+def _f32(t: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    return None if t is None else t.detach().to(dtype=torch.float32).contiguous()
+
+
+def bn_forward(x: torch.Tensor, weight, bias, running_mean, running_var, use_batch_stats: bool, momentum: float, eps: float,
+               act=None):
+    """Batch normalisation of the rows of ``x`` [n, c] (fp16 / fp32) in three launches.  ``momentum`` < 0
+    leaves the running statistics alone; they must be fp32 and are updated in place otherwise.
+    Returns (y, save_mean, save_rstd)."""
+    lib = _lib.load()
+    _require_cuda(x, "x")
+    x = x.contiguous()
+    n, c = x.shape
+    for name, t in (("running_mean", running_mean), ("running_var", running_var)):
+        if t is not None and (t.dtype != torch.float32 or not t.is_contiguous() or t.numel() != c):
+            raise ValueError(f"{name} must be a contiguous fp32 tensor of {c} elements")
+    w, b = _f32(weight), _f32(bias)
+    y = torch.empty_like(x)
+    save = torch.empty((2, c), dtype=torch.float32, device=x.device)
+    ws_bytes = lib.pce_bn_workspace_bytes(n, c)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+    code, slope = _act_code(act)
+    _lib.check(lib.pce_bn_forward(x.data_ptr(), y.data_ptr(), _dtype_code(x), n, c, _ptr(w), _ptr(b), _ptr(running_mean),
+                                  _ptr(running_var), int(use_batch_stats), float(momentum), float(eps), save[0].data_ptr(),
+                                  save[1].data_ptr(), ws.data_ptr(), ws_bytes, code, slope, _stream(x.device)))
+    return y, save[0], save[1]
+
+
+def bn_backward(x: torch.Tensor, dy: torch.Tensor, weight, save_mean: torch.Tensor, save_rstd: torch.Tensor,
+                use_batch_stats: bool):
+    """(dx, grad_weight fp32, grad_bias fp32) of ``bn_forward`` (without activation)."""
+    lib = _lib.load()
+    x = x.contiguous()
+    dy = dy.to(x.dtype).contiguous()
+    n, c = x.shape
+    w = _f32(weight)
+    dx = torch.empty_like(x)
+    grads = torch.empty((2, c), dtype=torch.float32, device=x.device)
+    ws_bytes = lib.pce_bn_workspace_bytes(n, c)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+    _lib.check(lib.pce_bn_backward(x.data_ptr(), dy.data_ptr(), dx.data_ptr(), _dtype_code(x), n, c, _ptr(w),
+                                   save_mean.data_ptr(), save_rstd.data_ptr(), int(use_batch_stats), grads[0].data_ptr(),
+                                   grads[1].data_ptr(), ws.data_ptr(), ws_bytes, _stream(x.device)))
+    return dx, grads[0], grads[1]
 
 
 def conv_wgrad(feats: torch.Tensor, grad_out: torch.Tensor, km: KernelMap, transposed: bool = False) -> torch.Tensor:

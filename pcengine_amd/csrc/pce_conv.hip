@@ -2204,6 +2204,311 @@ extern "C" int pce_conv_wgrad(const void *in, const void *gout, int32_t dtype, i
   return PCE_OK;
 }
 
+// ---- batch normalisation over the rows of a feature matrix (script/batchnorm.py:7-10) -----------------
+// Two kernels carry the forward and the backward pass of nn.BatchNorm1d on [n, c]:
+//   column sums:   out[j] = sum_r a[r][j],  out[c + j] = sum_r a[r][j] * b[r][j]   (b = a when b is null)
+//     forward statistics from (x, x): sum and sum of squares; backward from (dy, x): sum dy, sum dy*x
+//   column affine: y[r][j] = act(x[r][j] * kx[j] + d[r][j] * kd[j] + k0[j])         (d may be null)
+//     forward: y = x * (w*rstd) + (b - mean*w*rstd); backward: dx = dy*k1 + x*k2 + k3
+// The per-channel coefficients between them are c-element vector arithmetic left to the caller.
+// Sums are accumulated in fp32 over 16 rows per thread, then in fp64: per workgroup through LDS, across
+// workgroups by a second kernel over the per-workgroup partial sums (no atomics: same bits every run).
+#define BN_ROWS_PER_THREAD 16
+template <typename T>
+__global__ void __launch_bounds__(256) col_sums_partial_kernel(const T *__restrict__ a, const T *__restrict__ b, long long n,
+                                                               int c, int cols_per_block, double *__restrict__ partial) {
+  // thread -> (column group, row lane): a workgroup covers cols_per_block columns (a divisor of 256 or c itself)
+  // with 256 / cols_per_block row lanes; blockIdx.y walks over the column blocks
+  const int col = blockIdx.y * cols_per_block + threadIdx.x % cols_per_block;
+  const int lanes = 256 / cols_per_block, rl = threadIdx.x / cols_per_block;
+  const long long r0 = (long long)blockIdx.x * lanes * BN_ROWS_PER_THREAD;
+  double s1 = 0.0, s2 = 0.0;
+  if (col < c && rl < lanes) {
+    // all loads of a thread are requested before the first is used
+    float xs[BN_ROWS_PER_THREAD], ys[BN_ROWS_PER_THREAD];
+#pragma unroll
+    for (int k = 0; k < BN_ROWS_PER_THREAD; ++k) {
+      long long r = r0 + (long long)k * lanes + rl;
+      xs[k] = r < n ? (float)a[r * c + col] : 0.f;
+      ys[k] = (b && r < n) ? (float)b[r * c + col] : xs[k];
+    }
+    float f1 = 0.f, f2 = 0.f;
+#pragma unroll
+    for (int k = 0; k < BN_ROWS_PER_THREAD; ++k) {
+      f1 += xs[k];
+      f2 += xs[k] * ys[k];
+    }
+    s1 = f1;
+    s2 = f2;
+  }
+  __shared__ double red[2][256];
+  red[0][threadIdx.x] = s1;
+  red[1][threadIdx.x] = s2;
+  __syncthreads();
+  if (threadIdx.x < cols_per_block && col < c) {
+    double t1 = 0.0, t2 = 0.0;
+    for (int l = 0; l < lanes; ++l) {
+      t1 += red[0][l * cols_per_block + threadIdx.x];
+      t2 += red[1][l * cols_per_block + threadIdx.x];
+    }
+    partial[((long long)blockIdx.x * 2 + 0) * c + col] = t1;
+    partial[((long long)blockIdx.x * 2 + 1) * c + col] = t2;
+  }
+}
+
+// both partial sums of channel j over all workgroups, by one wavefront; the result is valid in lane 0
+__device__ __forceinline__ void wave_sum_partials(const double *__restrict__ partial, long long blocks, int c, int j,
+                                                  double *s1, double *s2) {
+  double a = 0.0, b = 0.0;
+  for (long long i = threadIdx.x; i < blocks; i += 64) {
+    a += partial[(i * 2 + 0) * c + j];
+    b += partial[(i * 2 + 1) * c + j];
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    a += __shfl_down(a, off, 64);
+    b += __shfl_down(b, off, 64);
+  }
+  *s1 = a;
+  *s2 = b;
+}
+
+__global__ void __launch_bounds__(64) col_sums_final_kernel(const double *__restrict__ partial, long long blocks, int c,
+                                                             double *__restrict__ out) {
+  const int col = blockIdx.x;   // one wavefront per column
+  double s1 = 0.0, s2 = 0.0;
+  wave_sum_partials(partial, blocks, c, col, &s1, &s2);
+  if (threadIdx.x == 0) {
+    out[col] = s1;
+    out[c + col] = s2;
+  }
+}
+
+static int bn_cols_per_block(int c) {
+  if (c >= 256) return 256;
+  int p = 1;
+  while (p < c) p <<= 1;
+  return p;   // power of two >= c: divides 256
+}
+
+extern "C" int64_t pce_col_sums_workspace_bytes(int64_t n, int32_t c) {
+  if (n <= 0 || c <= 0) return 0;
+  const int cpb = bn_cols_per_block(c);
+  const int64_t rows_per_block = (int64_t)(256 / cpb) * BN_ROWS_PER_THREAD;
+  return pce_div_up(n, rows_per_block) * 2 * c * (int64_t)sizeof(double);
+}
+
+extern "C" int pce_col_sums(const void *a, const void *b, int32_t dtype, int64_t n, int32_t c, void *ws, int64_t ws_bytes,
+                            double *out, pce_stream_t stream) {
+  if (!a || !out) PCE_FAIL(PCE_EINVAL, "pce_col_sums: null pointer");
+  if (dtype != PCE_F16 && dtype != PCE_F32) PCE_FAIL(PCE_EINVAL, "pce_col_sums: dtype %d", (int)dtype);
+  if (n <= 0 || c <= 0) PCE_FAIL(PCE_EINVAL, "pce_col_sums: n=%lld c=%d", (long long)n, (int)c);
+  const int64_t need = pce_col_sums_workspace_bytes(n, c);
+  if (!ws || ws_bytes < need) PCE_FAIL(PCE_EWORKSPACE, "pce_col_sums: workspace %lld < %lld", (long long)ws_bytes, (long long)need);
+  hipStream_t s = (hipStream_t)stream;
+  const int cpb = bn_cols_per_block(c);
+  const int64_t rows_per_block = (int64_t)(256 / cpb) * BN_ROWS_PER_THREAD;
+  const int64_t blocks = pce_div_up(n, rows_per_block);
+  if (blocks >= (1ll << 31)) PCE_FAIL(PCE_ECAPACITY, "pce_col_sums: %lld workgroups exceed the grid limit", (long long)blocks);
+  dim3 grid((unsigned)blocks, (unsigned)pce_div_up(c, cpb));
+  if (dtype == PCE_F16)
+    hipLaunchKernelGGL(col_sums_partial_kernel<half_t>, grid, dim3(256), 0, s, (const half_t *)a, (const half_t *)b,
+                       (long long)n, c, cpb, (double *)ws);
+  else
+    hipLaunchKernelGGL(col_sums_partial_kernel<float>, grid, dim3(256), 0, s, (const float *)a, (const float *)b, (long long)n,
+                       c, cpb, (double *)ws);
+  PCE_LAUNCH_CHECK("col_sums_partial");
+  hipLaunchKernelGGL(col_sums_final_kernel, dim3((unsigned)c), dim3(64), 0, s, (const double *)ws,
+                     (long long)blocks, c, out);
+  PCE_LAUNCH_CHECK("col_sums_final");
+  return PCE_OK;
+}
+
+// One wavefront per channel: adds up the per-workgroup partial sums and turns them into what the affine pass
+// needs.  Forward (sums of x and x*x): mean, biased variance, rstd; coefficients kx = w*rstd,
+// k0 = b - mean*kx; running statistics updated with the unbiased variance (torch.nn.BatchNorm1d).
+__global__ void __launch_bounds__(64) bn_finish_forward_kernel(const double *__restrict__ partial, long long blocks,
+                                                                long long n, int c, const float *__restrict__ weight,
+                                                                const float *__restrict__ bias, float *running_mean,
+                                                                float *running_var, int use_batch_stats, float momentum,
+                                                                float eps, float *__restrict__ save_mean,
+                                                                float *__restrict__ save_rstd, float *__restrict__ kx,
+                                                                float *__restrict__ k0) {
+  const int j = blockIdx.x;   // one wavefront per channel
+  double mean, var;
+  if (use_batch_stats) {
+    double s1 = 0.0, s2 = 0.0;
+    wave_sum_partials(partial, blocks, c, j, &s1, &s2);
+    if (threadIdx.x != 0) return;
+    mean = s1 / (double)n;
+    var = s2 / (double)n - mean * mean;
+    if (var < 0.0) var = 0.0;
+    if (momentum >= 0.f && running_mean && running_var) {
+      double unbiased = n > 1 ? var * ((double)n / (double)(n - 1)) : var;
+      running_mean[j] = (float)((1.0 - momentum) * running_mean[j] + momentum * mean);
+      running_var[j] = (float)((1.0 - momentum) * running_var[j] + momentum * unbiased);
+    }
+  } else {
+    if (threadIdx.x != 0) return;
+    mean = running_mean[j];
+    var = running_var[j];
+  }
+  double rstd = 1.0 / sqrt(var + (double)eps);
+  double w = weight ? (double)weight[j] : 1.0, b = bias ? (double)bias[j] : 0.0;
+  save_mean[j] = (float)mean;
+  save_rstd[j] = (float)rstd;
+  kx[j] = (float)(w * rstd);
+  k0[j] = (float)(b - mean * w * rstd);
+}
+
+// Backward (sums of dy and dy*x): grad_bias = sum dy, grad_weight = S = sum dy*xhat,
+// dx = dy*k1 + x*kd + k0 with k1 = w*rstd, kd = -k1*rstd*S/n, k0 = -k1*sum(dy)/n - kd*mean
+// (statistics of the batch), or dx = dy*k1 (fixed statistics).
+__global__ void __launch_bounds__(64) bn_finish_backward_kernel(const double *__restrict__ partial, long long blocks,
+                                                                 long long n, int c, const float *__restrict__ weight,
+                                                                 const float *__restrict__ save_mean,
+                                                                 const float *__restrict__ save_rstd, int use_batch_stats,
+                                                                 float *__restrict__ grad_weight, float *__restrict__ grad_bias,
+                                                                 float *__restrict__ k1, float *__restrict__ kd,
+                                                                 float *__restrict__ k0) {
+  const int j = blockIdx.x;   // one wavefront per channel
+  double s1 = 0.0, s2 = 0.0;
+  wave_sum_partials(partial, blocks, c, j, &s1, &s2);
+  if (threadIdx.x != 0) return;
+  const double mean = save_mean[j], rstd = save_rstd[j], w = weight ? (double)weight[j] : 1.0;
+  const double S = rstd * (s2 - mean * s1);
+  if (grad_weight) grad_weight[j] = (float)S;
+  if (grad_bias) grad_bias[j] = (float)s1;
+  const double a = w * rstd;
+  k1[j] = (float)a;
+  if (use_batch_stats) {
+    const double d = -a * rstd * S / (double)n;
+    kd[j] = (float)d;
+    k0[j] = (float)(-a * s1 / (double)n - d * mean);
+  } else {
+    kd[j] = 0.f;
+    k0[j] = 0.f;
+  }
+}
+
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256) col_affine_kernel(const T *__restrict__ x, const T *__restrict__ d, T *__restrict__ y,
+                                                         long long n, int c, const float *__restrict__ kx,
+                                                         const float *__restrict__ kd, const float *__restrict__ k0, int act,
+                                                         float slope) {
+  typedef typename VecOf<T, VEC>::type V;
+  const int row_vecs = c / VEC;
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n * row_vecs) return;
+  const int v = (int)(i % row_vecs);
+  V xv = *reinterpret_cast<const V *>(x + i * VEC);
+  V dv = xv;
+  if (d) dv = *reinterpret_cast<const V *>(d + i * VEC);
+  V out;
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    const int col = v * VEC + j;
+    float r = (float)(reinterpret_cast<const T *>(&xv)[j]) * kx[col] + k0[col];
+    if (d) r += (float)(reinterpret_cast<const T *>(&dv)[j]) * kd[col];
+    reinterpret_cast<T *>(&out)[j] = (T)act_apply(r, act, slope);
+  }
+  *reinterpret_cast<V *>(y + i * VEC) = out;
+}
+
+extern "C" int pce_col_affine(const void *x, const void *d, void *y, int32_t dtype, int64_t n, int32_t c, const float *kx,
+                              const float *kd, const float *k0, int32_t act, float slope, pce_stream_t stream) {
+  if (!x || !y || !kx || !k0 || (d && !kd)) PCE_FAIL(PCE_EINVAL, "pce_col_affine: null pointer");
+  if (dtype != PCE_F16 && dtype != PCE_F32) PCE_FAIL(PCE_EINVAL, "pce_col_affine: dtype %d", (int)dtype);
+  if (n <= 0 || c <= 0) PCE_FAIL(PCE_EINVAL, "pce_col_affine: n=%lld c=%d", (long long)n, (int)c);
+  if (act != PCE_ACT_NONE && act != PCE_ACT_RELU && act != PCE_ACT_LEAKY_RELU) PCE_FAIL(PCE_EINVAL, "pce_col_affine: activation %d", (int)act);
+  hipStream_t s = (hipStream_t)stream;
+  const int vec = dtype == PCE_F16 ? 8 : 4;
+  const bool aligned = aligned16(x) && aligned16(y) && aligned16(d) && c % vec == 0;
+  const long long items = aligned ? n * (c / vec) : n * c;
+  if (pce_div_up(items, 256) >= (1ll << 31)) PCE_FAIL(PCE_ECAPACITY, "pce_col_affine: tensor too large for one launch");
+  dim3 grid((unsigned)pce_div_up(items, 256));
+#define PCE_AFFINE(T_, V_)                                                                                               \
+  hipLaunchKernelGGL((col_affine_kernel<T_, V_>), grid, dim3(256), 0, s, (const T_ *)x, (const T_ *)d, (T_ *)y, (long long)n, c, \
+                     kx, kd, k0, act, slope)
+  if (dtype == PCE_F16 && aligned)
+    PCE_AFFINE(half_t, 8);
+  else if (dtype == PCE_F16)
+    PCE_AFFINE(half_t, 1);
+  else if (aligned)
+    PCE_AFFINE(float, 4);
+  else
+    PCE_AFFINE(float, 1);
+#undef PCE_AFFINE
+  PCE_LAUNCH_CHECK("col_affine");
+  return PCE_OK;
+}
+
+// workspace of the fused entry points: the partial sums, then 3*c floats of coefficients
+extern "C" int64_t pce_bn_workspace_bytes(int64_t n, int32_t c) {
+  if (n <= 0 || c <= 0) return 0;
+  return pce_align_up(pce_col_sums_workspace_bytes(n, c), 256) + 3 * (int64_t)c * (int64_t)sizeof(float);
+}
+
+static int bn_partial(const void *a, const void *b, int32_t dtype, int64_t n, int32_t c, double *partial, int64_t *blocks_out,
+                      hipStream_t s) {
+  const int cpb = bn_cols_per_block(c);
+  const int64_t rows_per_block = (int64_t)(256 / cpb) * BN_ROWS_PER_THREAD;
+  const int64_t blocks = pce_div_up(n, rows_per_block);
+  if (blocks >= (1ll << 31)) PCE_FAIL(PCE_ECAPACITY, "batch norm: %lld workgroups exceed the grid limit", (long long)blocks);
+  dim3 grid((unsigned)blocks, (unsigned)pce_div_up(c, cpb));
+  if (dtype == PCE_F16)
+    hipLaunchKernelGGL(col_sums_partial_kernel<half_t>, grid, dim3(256), 0, s, (const half_t *)a, (const half_t *)b,
+                       (long long)n, c, cpb, partial);
+  else
+    hipLaunchKernelGGL(col_sums_partial_kernel<float>, grid, dim3(256), 0, s, (const float *)a, (const float *)b, (long long)n,
+                       c, cpb, partial);
+  PCE_LAUNCH_CHECK("col_sums_partial");
+  *blocks_out = blocks;
+  return PCE_OK;
+}
+
+extern "C" int pce_bn_forward(const void *x, void *y, int32_t dtype, int64_t n, int32_t c, const float *weight,
+                              const float *bias, float *running_mean, float *running_var, int32_t use_batch_stats,
+                              float momentum, float eps, float *save_mean, float *save_rstd, void *ws, int64_t ws_bytes,
+                              int32_t act, float slope, pce_stream_t stream) {
+  if (!x || !y || !save_mean || !save_rstd) PCE_FAIL(PCE_EINVAL, "pce_bn_forward: null pointer");
+  if (dtype != PCE_F16 && dtype != PCE_F32) PCE_FAIL(PCE_EINVAL, "pce_bn_forward: dtype %d", (int)dtype);
+  if (n <= 0 || c <= 0) PCE_FAIL(PCE_EINVAL, "pce_bn_forward: n=%lld c=%d", (long long)n, (int)c);
+  if (!use_batch_stats && (!running_mean || !running_var)) PCE_FAIL(PCE_EINVAL, "pce_bn_forward: fixed statistics need running_mean and running_var");
+  if (!ws || ws_bytes < pce_bn_workspace_bytes(n, c)) PCE_FAIL(PCE_EWORKSPACE, "pce_bn_forward: workspace %lld < %lld", (long long)ws_bytes, (long long)pce_bn_workspace_bytes(n, c));
+  hipStream_t s = (hipStream_t)stream;
+  double *partial = (double *)ws;
+  float *coef = (float *)((char *)ws + pce_align_up(pce_col_sums_workspace_bytes(n, c), 256));
+  int64_t blocks = 0;
+  int rc;
+  if (use_batch_stats && (rc = bn_partial(x, nullptr, dtype, n, c, partial, &blocks, s))) return rc;
+  hipLaunchKernelGGL(bn_finish_forward_kernel, dim3((unsigned)c), dim3(64), 0, s, (const double *)partial,
+                     (long long)blocks, (long long)n, c, weight, bias, running_mean, running_var, use_batch_stats, momentum, eps,
+                     save_mean, save_rstd, coef, coef + c);
+  PCE_LAUNCH_CHECK("bn_finish_forward");
+  return pce_col_affine(x, nullptr, y, dtype, n, c, coef, nullptr, coef + c, act, slope, stream);
+}
+
+extern "C" int pce_bn_backward(const void *x, const void *dy, void *dx, int32_t dtype, int64_t n, int32_t c,
+                               const float *weight, const float *save_mean, const float *save_rstd, int32_t use_batch_stats,
+                               float *grad_weight, float *grad_bias, void *ws, int64_t ws_bytes, pce_stream_t stream) {
+  if (!x || !dy || !dx || !save_mean || !save_rstd) PCE_FAIL(PCE_EINVAL, "pce_bn_backward: null pointer");
+  if (dtype != PCE_F16 && dtype != PCE_F32) PCE_FAIL(PCE_EINVAL, "pce_bn_backward: dtype %d", (int)dtype);
+  if (n <= 0 || c <= 0) PCE_FAIL(PCE_EINVAL, "pce_bn_backward: n=%lld c=%d", (long long)n, (int)c);
+  if (!ws || ws_bytes < pce_bn_workspace_bytes(n, c)) PCE_FAIL(PCE_EWORKSPACE, "pce_bn_backward: workspace %lld < %lld", (long long)ws_bytes, (long long)pce_bn_workspace_bytes(n, c));
+  hipStream_t s = (hipStream_t)stream;
+  double *partial = (double *)ws;
+  float *coef = (float *)((char *)ws + pce_align_up(pce_col_sums_workspace_bytes(n, c), 256));
+  int64_t blocks = 0;
+  int rc = bn_partial(dy, x, dtype, n, c, partial, &blocks, s);
+  if (rc) return rc;
+  hipLaunchKernelGGL(bn_finish_backward_kernel, dim3((unsigned)c), dim3(64), 0, s, (const double *)partial,
+                     (long long)blocks, (long long)n, c, weight, save_mean, save_rstd, use_batch_stats, grad_weight, grad_bias, coef,
+                     coef + c, coef + 2 * c);
+  PCE_LAUNCH_CHECK("bn_finish_backward");
+  return pce_col_affine(dy, x, dx, dtype, n, c, coef, coef + c, coef + 2 * c, PCE_ACT_NONE, 0.f, stream);
+}
+
 // Map density rho = pairs per output row.  The deferred-scatter dataflow does only the useful
 // multiplications and pays M*(c_in + 2*c_out) elements of gather / partial-row traffic for them; the
 // output-stationary kernel touches no intermediate memory but multiplies every offset of every
