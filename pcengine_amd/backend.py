@@ -608,6 +608,31 @@ def conv_wgrad(feats: torch.Tensor, grad_out: torch.Tensor, km: KernelMap, trans
     return gw
 
 
+_ZERO_POS = {}
+
+
+def dense_wgrad(feats: torch.Tensor, grad_out: torch.Tensor) -> torch.Tensor:
+    """Gradient of ``dense_forward`` with respect to its [c_in, c_out] matrix, in fp32: the kernel-gradient
+    kernel run over row tiles only (one offset, every row paired with itself, no pair list)."""
+    lib = _lib.load()
+    _require_cuda(feats, "feats")
+    feats, grad_out = feats.contiguous(), grad_out.contiguous()
+    if feats.dtype != grad_out.dtype:
+        raise TypeError(f"features are {feats.dtype} but the output gradient is {grad_out.dtype}")
+    if feats.dim() != 2 or grad_out.dim() != 2 or feats.shape[0] != grad_out.shape[0]:
+        raise ValueError("features and output gradient must be matrices with the same number of rows")
+    n, c_in, c_out = feats.shape[0], feats.shape[1], grad_out.shape[1]
+    pos = _ZERO_POS.get(feats.device)
+    if pos is None:
+        pos = _ZERO_POS[feats.device] = torch.zeros(2, dtype=torch.int32, device=feats.device)
+    if n == 0:  # empty tensors have no data pointer to hand over
+        return torch.zeros((c_in, c_out), dtype=torch.float32, device=feats.device)
+    gw = torch.empty((c_in, c_out), dtype=torch.float32, device=feats.device)
+    _lib.check(lib.pce_conv_wgrad(feats.data_ptr(), grad_out.data_ptr(), _dtype_code(feats), n, n, c_in, c_out, 1, 0, None, None,
+                                  pos.data_ptr(), pos.data_ptr(), 0, gw.data_ptr(), _stream(feats.device)))
+    return gw
+
+
 def conv_backward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, grad_out: torch.Tensor, transposed: bool = False,
                   need_feats: bool = True, need_weight: bool = True, dataflow: Optional[int] = None):
     """(grad_feats, grad_weight) of ``conv_forward``.  The feature gradient is the convolution of

@@ -866,6 +866,7 @@ static inline bool stage_on(int bit) { return (g_stage_mask >> bit) & 1u; }
 // it would otherwise wait for every outstanding load (the ones just issued included) before the first
 // use of a fragment inside the loop.  The waits are written by hand instead (pipe_wait_barrier).
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ u32x4 load16_untracked(const void *p) {
   u32x4 v;
@@ -2057,6 +2058,144 @@ __device__ __forceinline__ void wgrad_fetch(float (&v)[PER], const T *__restrict
     for (int j = 0; j < PER; ++j) v[j] = (row >= 0 && c0 + j < c_total) ? (float)base[(long long)row * c_total + c0 + j] : 0.f;
   }
 }
+// fp16 tensors: the same block / run structure on the fp16 MFMA (32x32x16: 8 consecutive pairs per lane
+// and operand).  Its operands are [channel][pair], the transpose of how rows lie in memory.  A thread
+// fetches the same 8 channels of 4 consecutive pairs (four 16-byte loads), regroups them in registers into
+// 8 channel rows of 4 pairs and writes each as one 8-byte LDS store; the MFMA fragments are then 16
+// contiguous bytes.  A stage holds KP pairs (64 for 128-wide blocks, the whole tile for 64-wide ones) and
+// channel rows lie KP + 8 halfs apart, which keeps both the 8-byte stores of a half wavefront and the
+// 16-byte fragment reads of 16 consecutive channels in distinct banks.
+template <int BLK>
+__global__ void __launch_bounds__(256, 2) wgrad_f16_kernel(const half_t *__restrict__ in, const half_t *__restrict__ gout,
+                                                        long long n_rows, int c_in, int c_out, int kv, int mid,
+                                                        const int *__restrict__ imap, const int *__restrict__ omap,
+                                                        const int *__restrict__ kpos, const int *__restrict__ qkpos,
+                                                        long long pair_tiles, long long tiles, int run, int ci_blocks,
+                                                        int co_blocks, float *__restrict__ gw) {
+  constexpr int R = BLK / 64;
+  constexpr int KP = BLK == 128 ? 64 : 128;  // pairs per stage
+  constexpr int PG = KP / 4;                 // groups of 4 pairs; PG * (BLK / 8) == 256 threads
+  constexpr int LD = KP + 8;                 // halfs per channel row
+  static_assert(PG * (BLK / 8) == 256, "one thread per (4 pairs, 8 channels) cell of a stage");
+  __shared__ __attribute__((aligned(16))) half_t At[BLK][LD];
+  __shared__ __attribute__((aligned(16))) half_t Gt[BLK][LD];
+  __shared__ int rows_in[128], rows_out[128];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int l32 = lane & 31, g = lane >> 5;
+  const int wr = wave >> 1, wc = wave & 1;
+  const long long grp = blockIdx.x / (ci_blocks * co_blocks);
+  const int rest = (int)(blockIdx.x % (ci_blocks * co_blocks));
+  const int ci0 = (rest / co_blocks) * BLK, co0 = (rest % co_blocks) * BLK;
+
+  f32x16 acc[R][R];
+#pragma unroll
+  for (int i = 0; i < R; ++i)
+#pragma unroll
+    for (int j = 0; j < R; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  int cur = -1;
+  auto flush = [&](int widx) {
+    float *dst = gw + (long long)widx * c_in * c_out;
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+#pragma unroll
+      for (int j = 0; j < R; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          int ci = ci0 + wr * (BLK / 2) + i * 32 + (e / 4) * 8 + g * 4 + (e % 4);
+          int co = co0 + wc * (BLK / 2) + j * 32 + l32;
+          float v = acc[i][j][e];
+          if (ci < c_in && co < c_out && v != 0.f) unsafeAtomicAdd(dst + (long long)ci * c_out + co, v);
+          acc[i][j][e] = 0.f;
+        }
+  };
+  const bool vec_in = (c_in % 8 == 0) && ci0 + BLK <= c_in && (((uintptr_t)in) & 15) == 0;
+  const bool vec_out = (c_out % 8 == 0) && co0 + BLK <= c_out && (((uintptr_t)gout) & 15) == 0;
+  const int pg = threadIdx.x % PG, cg = threadIdx.x / PG;  // the thread's cell: pairs 4 pg .. +3, channels 8 cg .. +7
+  // one operand's 8 channels of one pair as 4 dwords (channels 2d, 2d + 1 in dword d)
+  auto fetch_row = [&](const half_t *base, int row, int c, int c0, bool vec) -> u32x4 {
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (row < 0) return v;
+    const half_t *src = base + (long long)row * c + c0 + cg * 8;
+    if (vec) return *reinterpret_cast<const u32x4 *>(src);
+    half8 h = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (c0 + cg * 8 + j < c) h[j] = src[j];
+    return *reinterpret_cast<u32x4 *>(&h);
+  };
+  // [4 pairs][8 channels] in registers -> 8 channel rows of 4 pairs in LDS
+  auto put = [&](half_t (*dst)[LD], const u32x4 (&v)[4]) {
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      u32x2 even, odd;
+      even[0] = __builtin_amdgcn_perm(v[1][d], v[0][d], 0x05040100u);
+      even[1] = __builtin_amdgcn_perm(v[3][d], v[2][d], 0x05040100u);
+      odd[0] = __builtin_amdgcn_perm(v[1][d], v[0][d], 0x07060302u);
+      odd[1] = __builtin_amdgcn_perm(v[3][d], v[2][d], 0x07060302u);
+      *reinterpret_cast<u32x2 *>(&dst[cg * 8 + 2 * d][pg * 4]) = even;
+      *reinterpret_cast<u32x2 *>(&dst[cg * 8 + 2 * d + 1][pg * 4]) = odd;
+    }
+  };
+  const long long t_end = (grp + 1) * run < tiles ? (grp + 1) * run : tiles;
+  for (long long tile = grp * run; tile < t_end; ++tile) {
+    int widx;
+    __syncthreads();
+    if (tile < pair_tiles) {
+      long long q0 = tile * 128;
+      widx = 0;
+      for (int i = 0; i < kv; ++i) widx += ((long long)qkpos[i + 1] <= q0) ? 1 : 0;
+      if (widx >= kv) break;  // uniform
+      if (threadIdx.x < 128) {
+        long long p = q0 - qkpos[widx] + kpos[widx] + threadIdx.x;
+        bool ok = p < (long long)kpos[widx + 1];
+        rows_in[threadIdx.x] = ok ? imap[p] : -1;
+        rows_out[threadIdx.x] = ok ? omap[p] : -1;
+      }
+    } else {
+      widx = mid;
+      if (threadIdx.x < 128) {
+        long long row = (tile - pair_tiles) * 128 + threadIdx.x;
+        rows_in[threadIdx.x] = rows_out[threadIdx.x] = row < n_rows ? (int)row : -1;
+      }
+    }
+    if (cur >= 0 && widx != cur) flush(cur);
+    cur = widx;
+    __syncthreads();
+    u32x4 va[4], vg[4];
+    auto fetch = [&](int p0) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        va[q] = fetch_row(in, rows_in[p0 + pg * 4 + q], c_in, ci0, vec_in);
+        vg[q] = fetch_row(gout, rows_out[p0 + pg * 4 + q], c_out, co0, vec_out);
+      }
+    };
+    fetch(0);
+#pragma unroll
+    for (int p0 = 0; p0 < 128; p0 += KP) {
+      if (p0) __syncthreads();  // the MFMAs of the previous stage have read their operands
+      put(At, va);
+      put(Gt, vg);
+      __syncthreads();
+      if (p0 + KP < 128) fetch(p0 + KP);
+#pragma unroll
+      for (int k0 = 0; k0 < KP; k0 += 16) {
+        half8 av[R], bv[R];
+#pragma unroll
+        for (int i = 0; i < R; ++i) av[i] = *reinterpret_cast<const half8 *>(&At[wr * (BLK / 2) + i * 32 + l32][k0 + 8 * g]);
+#pragma unroll
+        for (int j = 0; j < R; ++j) bv[j] = *reinterpret_cast<const half8 *>(&Gt[wc * (BLK / 2) + j * 32 + l32][k0 + 8 * g]);
+#pragma unroll
+        for (int i = 0; i < R; ++i)
+#pragma unroll
+          for (int j = 0; j < R; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[i], bv[j], acc[i][j], 0, 0, 0);
+      }
+    }
+  }
+  if (cur >= 0) flush(cur);
+}
+
 template <typename T, int BLK>
 __global__ void __launch_bounds__(256) wgrad_kernel(const T *__restrict__ in, const T *__restrict__ gout, long long n_rows,
                                                     int c_in, int c_out, int kv, int mid, const int *__restrict__ imap,
@@ -2191,15 +2330,20 @@ extern "C" int pce_conv_wgrad(const void *in, const void *gout, int32_t dtype, i
   hipLaunchKernelGGL((wgrad_kernel<T_, BLK_>), dim3((unsigned)blocks), dim3(256), 0, s, (const T_ *)in, (const T_ *)gout, \
                      (long long)n_out, c_in, c_out, kv, mid, imap, omap, kpos, qkpos, pair_tiles, tiles, (int)run,       \
                      ci_blocks, co_blocks, gw)
+#define PCE_WGRAD16(BLK_)                                                                                            \
+  hipLaunchKernelGGL((wgrad_f16_kernel<BLK_>), dim3((unsigned)blocks), dim3(256), 0, s, (const half_t *)in,            \
+                     (const half_t *)gout, (long long)n_out, c_in, c_out, kv, mid, imap, omap, kpos, qkpos, pair_tiles, \
+                     tiles, (int)run, ci_blocks, co_blocks, gw)
   if (dtype == PCE_F16 && blk == 128)
-    PCE_WGRAD(half_t, 128);
+    PCE_WGRAD16(128);
   else if (dtype == PCE_F16)
-    PCE_WGRAD(half_t, 64);
+    PCE_WGRAD16(64);
   else if (blk == 128)
     PCE_WGRAD(float, 128);
   else
     PCE_WGRAD(float, 64);
 #undef PCE_WGRAD
+#undef PCE_WGRAD16
   PCE_LAUNCH_CHECK("wgrad");
   return PCE_OK;
 }
@@ -2400,16 +2544,39 @@ __global__ void __launch_bounds__(256) col_affine_kernel(const T *__restrict__ x
   const int row_vecs = c / VEC;
   long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n * row_vecs) return;
-  const int v = (int)(i % row_vecs);
+  const int v = (int)(i - (i / row_vecs) * row_vecs);
   V xv = *reinterpret_cast<const V *>(x + i * VEC);
   V dv = xv;
   if (d) dv = *reinterpret_cast<const V *>(d + i * VEC);
   V out;
+  // the thread's VEC coefficients are contiguous: 16-byte loads when VEC is a multiple of four
+  float cx[VEC], c0[VEC], cd[VEC];
+  if (VEC % 4 == 0) {
+#pragma unroll
+    for (int q = 0; q < VEC / 4; ++q) {
+      f32x4 a = *reinterpret_cast<const f32x4 *>(kx + v * VEC + q * 4);
+      f32x4 b = *reinterpret_cast<const f32x4 *>(k0 + v * VEC + q * 4);
+      f32x4 e = a;
+      if (d) e = *reinterpret_cast<const f32x4 *>(kd + v * VEC + q * 4);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        cx[q * 4 + j] = a[j];
+        c0[q * 4 + j] = b[j];
+        cd[q * 4 + j] = e[j];
+      }
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      cx[j] = kx[v * VEC + j];
+      c0[j] = k0[v * VEC + j];
+      cd[j] = d ? kd[v * VEC + j] : 0.f;
+    }
+  }
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
-    const int col = v * VEC + j;
-    float r = (float)(reinterpret_cast<const T *>(&xv)[j]) * kx[col] + k0[col];
-    if (d) r += (float)(reinterpret_cast<const T *>(&dv)[j]) * kd[col];
+    float r = (float)(reinterpret_cast<const T *>(&xv)[j]) * cx[j] + c0[j];
+    if (d) r += (float)(reinterpret_cast<const T *>(&dv)[j]) * cd[j];
     reinterpret_cast<T *>(&out)[j] = (T)act_apply(r, act, slope);
   }
   *reinterpret_cast<V *>(y + i * VEC) = out;

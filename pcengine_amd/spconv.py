@@ -189,7 +189,7 @@ class _DenseFunction(torch.autograd.Function):
             kt = kernel.detach().t().contiguous()
             gf = backend.dense_forward(grad_out, kt, backend.pack_weights(kt))
         if ctx.needs_input_grad[1]:
-            gw = (feats.detach().float().t() @ grad_out.float()).to(kernel.dtype)
+            gw = backend.dense_wgrad(feats.detach(), grad_out).to(kernel.dtype)
         gb = grad_out.sum(0) if (ctx.has_bias and ctx.needs_input_grad[2]) else None
         return gf, gw, gb
 

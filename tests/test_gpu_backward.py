@@ -116,3 +116,22 @@ def test_kernel_gradient_long_runs(dtype, c_in, c_out):
     gw = backend.conv_wgrad(torch.as_tensor(f, device=DEV).to(dtype), torch.as_tensor(go, device=DEV).to(dtype), km)
     assert gw.dtype == torch.float32 and gw.shape == (27, c_in, c_out)
     assert orc.rel_l2(gw.double().cpu().numpy(), gw_want) <= 1e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("n,c_in,c_out", [(0, 8, 8), (1, 3, 5), (127, 32, 20), (5000, 96, 20), (40000, 64, 128), (3001, 130, 70)])
+def test_dense_layer_kernel_gradient(n, c_in, c_out, dtype):
+    """The 1x1 layer's kernel gradient is feats^T @ grad_out: checked against that product in float64 on
+    the rounded operands (the kernel sums in fp32; rows are summed in a different order per run)."""
+    g = torch.Generator().manual_seed(n + c_in)
+    a = torch.randn(n, c_in, generator=g).to(dtype).to(DEV)
+    b = torch.randn(n, c_out, generator=g).to(dtype).to(DEV)
+    gw = backend.dense_wgrad(a, b)
+    assert gw.dtype == torch.float32 and tuple(gw.shape) == (c_in, c_out)
+    ref = a.double().t() @ b.double()
+    scale = float(ref.abs().max()) if n else 1.0
+    assert float((gw.double() - ref).abs().max()) <= 1e-5 * max(scale, 1.0) + 1e-6 * max(n, 1) ** 0.5
+    with pytest.raises(TypeError):
+        backend.dense_wgrad(a, b.to(torch.float64))
+    with pytest.raises(ValueError):
+        backend.dense_wgrad(a, torch.zeros(n + 1, c_out, dtype=dtype, device=DEV))
