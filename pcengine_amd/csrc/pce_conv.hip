@@ -2037,7 +2037,8 @@ extern "C" int pce_conv_fwd_dense(const void *in, const void *w, const void *wp,
 // order of the additions, and so the last bits, still vary from run to run).
 #define WGRAD_KP 32   // pairs per LDS stage
 
-// PER consecutive channels of one row as fp32 (zeros for a missing row or past the last channel)
+// PER consecutive channels of one row as fp32 (zeros for a missing row or past the last channel); the vector
+// form needs a channel count that is a multiple of the 16-byte vector, so a vector lies inside the row or past it
 template <typename T, int PER>
 __device__ __forceinline__ void wgrad_fetch(float (&v)[PER], const T *__restrict__ base, int row, int c_total, int c0,
                                             bool vec) {
@@ -2049,7 +2050,7 @@ __device__ __forceinline__ void wgrad_fetch(float (&v)[PER], const T *__restrict
       V x;
 #pragma unroll
       for (int j = 0; j < EPV; ++j) x[j] = (T)0;
-      if (row >= 0) x = *reinterpret_cast<const V *>(base + (long long)row * c_total + c0 + q * EPV);
+      if (row >= 0 && c0 + q * EPV < c_total) x = *reinterpret_cast<const V *>(base + (long long)row * c_total + c0 + q * EPV);
 #pragma unroll
       for (int j = 0; j < EPV; ++j) v[q * EPV + j] = (float)x[j];
     }
@@ -2083,8 +2084,11 @@ __global__ void __launch_bounds__(256, 2) wgrad_f16_kernel(const half_t *__restr
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int l32 = lane & 31, g = lane >> 5;
   const int wr = wave >> 1, wc = wave & 1;
-  const long long grp = blockIdx.x / (ci_blocks * co_blocks);
-  const int rest = (int)(blockIdx.x % (ci_blocks * co_blocks));
+  // workgroups are dealt to the 8 XCDs in turn: all (ci, co) blocks of one run of tiles go to the same XCD,
+  // whose L2 then serves the rows they gather in common; groups past the last run find no tile
+  const long long slot = blockIdx.x >> 3;
+  const int rest = (int)(slot % (ci_blocks * co_blocks));
+  const long long grp = (slot / (ci_blocks * co_blocks)) * 8 + (blockIdx.x & 7);
   const int ci0 = (rest / co_blocks) * BLK, co0 = (rest % co_blocks) * BLK;
 
   f32x16 acc[R][R];
@@ -2110,15 +2114,15 @@ __global__ void __launch_bounds__(256, 2) wgrad_f16_kernel(const half_t *__restr
           acc[i][j][e] = 0.f;
         }
   };
-  const bool vec_in = (c_in % 8 == 0) && ci0 + BLK <= c_in && (((uintptr_t)in) & 15) == 0;
-  const bool vec_out = (c_out % 8 == 0) && co0 + BLK <= c_out && (((uintptr_t)gout) & 15) == 0;
+  const bool vec_in = (c_in % 8 == 0) && (((uintptr_t)in) & 15) == 0;
+  const bool vec_out = (c_out % 8 == 0) && (((uintptr_t)gout) & 15) == 0;
   const int pg = threadIdx.x % PG, cg = threadIdx.x / PG;  // the thread's cell: pairs 4 pg .. +3, channels 8 cg .. +7
   // one operand's 8 channels of one pair as 4 dwords (channels 2d, 2d + 1 in dword d)
   auto fetch_row = [&](const half_t *base, int row, int c, int c0, bool vec) -> u32x4 {
     u32x4 v = {0u, 0u, 0u, 0u};
-    if (row < 0) return v;
+    if (row < 0 || c0 + cg * 8 >= c) return v;
     const half_t *src = base + (long long)row * c + c0 + cg * 8;
-    if (vec) return *reinterpret_cast<const u32x4 *>(src);
+    if (vec) return *reinterpret_cast<const u32x4 *>(src);  // c is a multiple of 8: the 8 channels lie inside the row
     half8 h = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
     for (int j = 0; j < 8; ++j)
@@ -2211,8 +2215,11 @@ __global__ void __launch_bounds__(256) wgrad_kernel(const T *__restrict__ in, co
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int l32 = lane & 31, g = lane >> 5;
   const int wr = wave >> 1, wc = wave & 1;
-  const long long grp = blockIdx.x / (ci_blocks * co_blocks);
-  const int rest = (int)(blockIdx.x % (ci_blocks * co_blocks));
+  // workgroups are dealt to the 8 XCDs in turn: all (ci, co) blocks of one run of tiles go to the same XCD,
+  // whose L2 then serves the rows they gather in common; groups past the last run find no tile
+  const long long slot = blockIdx.x >> 3;
+  const int rest = (int)(slot % (ci_blocks * co_blocks));
+  const long long grp = (slot / (ci_blocks * co_blocks)) * 8 + (blockIdx.x & 7);
   const int ci0 = (rest / co_blocks) * BLK, co0 = (rest % co_blocks) * BLK;
 
   f32x16 acc[R][R];
@@ -2242,8 +2249,8 @@ __global__ void __launch_bounds__(256) wgrad_kernel(const T *__restrict__ in, co
 
   // 16-byte loads when a thread's channels lie inside the tensor and its rows are 16-byte multiples
   constexpr int EPV = 16 / (int)sizeof(T);
-  const bool vec_in = (c_in % EPV == 0) && ci0 + BLK <= c_in && (((uintptr_t)in) & 15) == 0;
-  const bool vec_out = (c_out % EPV == 0) && co0 + BLK <= c_out && (((uintptr_t)gout) & 15) == 0;
+  const bool vec_in = (c_in % EPV == 0) && (((uintptr_t)in) & 15) == 0;
+  const bool vec_out = (c_out % EPV == 0) && (((uintptr_t)gout) & 15) == 0;
   const long long t_end = (grp + 1) * run < tiles ? (grp + 1) * run : tiles;
   for (long long tile = grp * run; tile < t_end; ++tile) {
     int widx;
@@ -2318,13 +2325,17 @@ extern "C" int pce_conv_wgrad(const void *in, const void *gout, int32_t dtype, i
   long long pair_tiles = qsum / PCE_QUANTUM;
   long long tiles = pair_tiles + (mid >= 0 ? pce_div_up(n_out, 128) : 0);
   if (tiles <= 0) return PCE_OK;
-  // 128 x 128 blocks of (ci, co) for wide layers, 64 x 64 otherwise; runs of tiles long enough to leave about
-  // two thousand workgroups (every run ends with one atomic per element of its block)
+  // 128 x 128 blocks of (ci, co) for wide layers, 64 x 64 otherwise.  Every run of tiles ends with one atomic
+  // per element of its block, so runs are made long enough to leave about 512 workgroups (one resident set:
+  // two per CU), or about 1024 where several blocks share many tiles (measured on 100k-voxel layers: a
+  // 128 -> 128 layer of 5111 tiles takes 174 / 131 / 122 us at 2048 / 1024 / 512 workgroups)
   const int blk = (c_in > 64 || c_out > 64) ? 128 : 64;
   const int ci_blocks = (c_in + blk - 1) / blk, co_blocks = (c_out + blk - 1) / blk;
-  long long run = tiles * ci_blocks * co_blocks / 2048;
-  run = run < 1 ? 1 : (run > 64 ? 64 : run);
-  long long blocks = pce_div_up(tiles, run) * ci_blocks * co_blocks;
+  const long long tile_blocks = tiles * ci_blocks * co_blocks;
+  const long long target_wgs = (ci_blocks * co_blocks > 1 && tile_blocks >= 8192) ? 1024 : 512;
+  long long run = tile_blocks / target_wgs;
+  run = run < 1 ? 1 : (run > 256 ? 256 : run);
+  long long blocks = pce_div_up(pce_div_up(tiles, run), 8) * 8 * ci_blocks * co_blocks;
   if (blocks >= (1ll << 31)) PCE_FAIL(PCE_ECAPACITY, "pce_conv_wgrad: %lld workgroups exceed the grid limit", blocks);
 #define PCE_WGRAD(T_, BLK_)                                                                                              \
   hipLaunchKernelGGL((wgrad_kernel<T_, BLK_>), dim3((unsigned)blocks), dim3(256), 0, s, (const T_ *)in, (const T_ *)gout, \
