@@ -2366,48 +2366,92 @@ extern "C" int pce_conv_wgrad(const void *in, const void *gout, int32_t dtype, i
 //   column affine: y[r][j] = act(x[r][j] * kx[j] + d[r][j] * kd[j] + k0[j])         (d may be null)
 //     forward: y = x * (w*rstd) + (b - mean*w*rstd); backward: dx = dy*k1 + x*k2 + k3
 // The per-channel coefficients between them are c-element vector arithmetic left to the caller.
-// Sums are accumulated in fp32 over 16 rows per thread, then in fp64: per workgroup through LDS, across
-// workgroups by a second kernel over the per-workgroup partial sums (no atomics: same bits every run).
-#define BN_ROWS_PER_THREAD 16
-template <typename T>
+// A thread owns VEC adjacent columns (one 16-byte vector when the layout allows) and walks down the rows in
+// steps of the grid, 8 rows requested at a time; sums are accumulated in fp32 over those 8 rows, then in fp64:
+// per workgroup through LDS, across workgroups by a second kernel over the per-workgroup partial sums (no
+// atomics: same bits every run).  At most BN_MAX_ROW_BLOCKS workgroups share the rows.
+#define BN_ROWS_IN_FLIGHT 8
+#define BN_MAX_ROW_BLOCKS 1024
+template <typename T, int VEC>
 __global__ void __launch_bounds__(256) col_sums_partial_kernel(const T *__restrict__ a, const T *__restrict__ b, long long n,
                                                                int c, int cols_per_block, double *__restrict__ partial) {
-  // thread -> (column group, row lane): a workgroup covers cols_per_block columns (a divisor of 256 or c itself)
-  // with 256 / cols_per_block row lanes; blockIdx.y walks over the column blocks
-  const int col = blockIdx.y * cols_per_block + threadIdx.x % cols_per_block;
+  typedef typename VecOf<T, VEC>::type V;
+  // thread -> (vector column, row lane): a workgroup covers cols_per_block vector columns (a power of two up to
+  // 256) with 256 / cols_per_block row lanes; blockIdx.y walks over the column blocks
+  const int tc = threadIdx.x % cols_per_block;
+  const int col0 = (blockIdx.y * cols_per_block + tc) * VEC;
   const int lanes = 256 / cols_per_block, rl = threadIdx.x / cols_per_block;
-  const long long r0 = (long long)blockIdx.x * lanes * BN_ROWS_PER_THREAD;
-  double s1 = 0.0, s2 = 0.0;
-  if (col < c && rl < lanes) {
-    // all loads of a thread are requested before the first is used
-    float xs[BN_ROWS_PER_THREAD], ys[BN_ROWS_PER_THREAD];
+  double s1[VEC], s2[VEC];
 #pragma unroll
-    for (int k = 0; k < BN_ROWS_PER_THREAD; ++k) {
-      long long r = r0 + (long long)k * lanes + rl;
-      xs[k] = r < n ? (float)a[r * c + col] : 0.f;
-      ys[k] = (b && r < n) ? (float)b[r * c + col] : xs[k];
-    }
-    float f1 = 0.f, f2 = 0.f;
+  for (int j = 0; j < VEC; ++j) s1[j] = s2[j] = 0.0;
+  if (col0 < c) {
+    const long long stride = (long long)gridDim.x * lanes;
+    for (long long r0 = (long long)blockIdx.x * lanes + rl; r0 < n; r0 += stride * BN_ROWS_IN_FLIGHT) {
+      // all loads of a step are requested before the first is used
+      V xs[BN_ROWS_IN_FLIGHT], ys[BN_ROWS_IN_FLIGHT];
 #pragma unroll
-    for (int k = 0; k < BN_ROWS_PER_THREAD; ++k) {
-      f1 += xs[k];
-      f2 += xs[k] * ys[k];
+      for (int k = 0; k < BN_ROWS_IN_FLIGHT; ++k) {
+        const long long r = r0 + k * stride;
+        V zero;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) reinterpret_cast<T *>(&zero)[j] = (T)0;
+        xs[k] = r < n ? *reinterpret_cast<const V *>(a + r * c + col0) : zero;
+        ys[k] = b ? (r < n ? *reinterpret_cast<const V *>(b + r * c + col0) : zero) : xs[k];
+      }
+      float f1[VEC], f2[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) f1[j] = f2[j] = 0.f;
+#pragma unroll
+      for (int k = 0; k < BN_ROWS_IN_FLIGHT; ++k)
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float x = (float)reinterpret_cast<const T *>(&xs[k])[j], y = (float)reinterpret_cast<const T *>(&ys[k])[j];
+          f1[j] += x;
+          f2[j] += x * y;
+        }
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        s1[j] += (double)f1[j];
+        s2[j] += (double)f2[j];
+      }
     }
-    s1 = f1;
-    s2 = f2;
   }
-  __shared__ double red[2][256];
-  red[0][threadIdx.x] = s1;
-  red[1][threadIdx.x] = s2;
+  // the row lanes of a column are cols_per_block threads apart: halving tree over them, both sums at once
+  __shared__ double red[2 * VEC * 256];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    red[j * 256 + threadIdx.x] = s1[j];
+    red[(VEC + j) * 256 + threadIdx.x] = s2[j];
+  }
   __syncthreads();
-  if (threadIdx.x < cols_per_block && col < c) {
-    double t1 = 0.0, t2 = 0.0;
-    for (int l = 0; l < lanes; ++l) {
-      t1 += red[0][l * cols_per_block + threadIdx.x];
-      t2 += red[1][l * cols_per_block + threadIdx.x];
+  // a thread keeps its own sums in registers and publishes them only while a later step still reads them
+  for (int off = lanes >> 1; off >= 1; off >>= 1) {
+    if (rl < off) {
+      double other[2 * VEC];
+#pragma unroll
+      for (int q = 0; q < 2 * VEC; ++q) other[q] = red[q * 256 + threadIdx.x + off * cols_per_block];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        s1[j] += other[j];
+        s2[j] += other[VEC + j];
+      }
+      if (rl >= (off >> 1) && off > 1) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          red[j * 256 + threadIdx.x] = s1[j];
+          red[(VEC + j) * 256 + threadIdx.x] = s2[j];
+        }
+      }
     }
-    partial[((long long)blockIdx.x * 2 + 0) * c + col] = t1;
-    partial[((long long)blockIdx.x * 2 + 1) * c + col] = t2;
+    __syncthreads();
+  }
+  if (rl == 0 && col0 < c) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j)
+      if (col0 + j < c) {
+        partial[((long long)blockIdx.x * 2 + 0) * c + col0 + j] = s1[j];
+        partial[((long long)blockIdx.x * 2 + 1) * c + col0 + j] = s2[j];
+      }
   }
 }
 
@@ -2415,9 +2459,20 @@ __global__ void __launch_bounds__(256) col_sums_partial_kernel(const T *__restri
 __device__ __forceinline__ void wave_sum_partials(const double *__restrict__ partial, long long blocks, int c, int j,
                                                   double *s1, double *s2) {
   double a = 0.0, b = 0.0;
-  for (long long i = threadIdx.x; i < blocks; i += 64) {
-    a += partial[(i * 2 + 0) * c + j];
-    b += partial[(i * 2 + 1) * c + j];
+  // four blocks per lane and step, all eight loads requested before the first is added
+  for (long long i0 = threadIdx.x; i0 < blocks; i0 += 256) {
+    double x[4], y[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const long long i = i0 + 64 * k;
+      x[k] = i < blocks ? partial[(i * 2 + 0) * c + j] : 0.0;
+      y[k] = i < blocks ? partial[(i * 2 + 1) * c + j] : 0.0;
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      a += x[k];
+      b += y[k];
+    }
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
@@ -2439,18 +2494,44 @@ __global__ void __launch_bounds__(64) col_sums_final_kernel(const double *__rest
   }
 }
 
-static int bn_cols_per_block(int c) {
-  if (c >= 256) return 256;
-  int p = 1;
-  while (p < c) p <<= 1;
-  return p;   // power of two >= c: divides 256
+// upper bound of the row blocks of any layout of n rows (the workspace is sized for it)
+static int64_t bn_max_row_blocks(int64_t n) {
+  const int64_t by_rows = pce_div_up(n, BN_ROWS_IN_FLIGHT);
+  return by_rows < BN_MAX_ROW_BLOCKS ? by_rows : BN_MAX_ROW_BLOCKS;
 }
 
 extern "C" int64_t pce_col_sums_workspace_bytes(int64_t n, int32_t c) {
   if (n <= 0 || c <= 0) return 0;
-  const int cpb = bn_cols_per_block(c);
-  const int64_t rows_per_block = (int64_t)(256 / cpb) * BN_ROWS_PER_THREAD;
-  return pce_div_up(n, rows_per_block) * 2 * c * (int64_t)sizeof(double);
+  return bn_max_row_blocks(n) * 2 * c * (int64_t)sizeof(double);
+}
+
+// launches the partial-sum kernel; *blocks_out = row blocks written (partial[block][2][c])
+static int bn_partial(const void *a, const void *b, int32_t dtype, int64_t n, int32_t c, double *partial, int64_t *blocks_out,
+                      hipStream_t s) {
+  const int full = dtype == PCE_F16 ? 8 : 4;
+  const int vec = (c % full == 0 && aligned16(a) && aligned16(b)) ? full : 1;
+  const int vcols = c / vec;
+  int cpb = 1;   // vector columns per workgroup: the power of two >= vcols, at most 256
+  while (cpb < vcols && cpb < 256) cpb <<= 1;
+  const int lanes = 256 / cpb;
+  int64_t blocks = pce_div_up(n, (int64_t)lanes * BN_ROWS_IN_FLIGHT);
+  if (blocks > BN_MAX_ROW_BLOCKS) blocks = BN_MAX_ROW_BLOCKS;
+  dim3 grid((unsigned)blocks, (unsigned)pce_div_up(vcols, cpb));
+#define PCE_COLSUMS(T_, V_)                                                                                                   \
+  hipLaunchKernelGGL((col_sums_partial_kernel<T_, V_>), grid, dim3(256), 0, s, (const T_ *)a, (const T_ *)b, (long long)n, c, \
+                     cpb, partial)
+  if (dtype == PCE_F16 && vec == 8)
+    PCE_COLSUMS(half_t, 8);
+  else if (dtype == PCE_F16)
+    PCE_COLSUMS(half_t, 1);
+  else if (vec == 4)
+    PCE_COLSUMS(float, 4);
+  else
+    PCE_COLSUMS(float, 1);
+#undef PCE_COLSUMS
+  PCE_LAUNCH_CHECK("col_sums_partial");
+  *blocks_out = blocks;
+  return PCE_OK;
 }
 
 extern "C" int pce_col_sums(const void *a, const void *b, int32_t dtype, int64_t n, int32_t c, void *ws, int64_t ws_bytes,
@@ -2461,18 +2542,9 @@ extern "C" int pce_col_sums(const void *a, const void *b, int32_t dtype, int64_t
   const int64_t need = pce_col_sums_workspace_bytes(n, c);
   if (!ws || ws_bytes < need) PCE_FAIL(PCE_EWORKSPACE, "pce_col_sums: workspace %lld < %lld", (long long)ws_bytes, (long long)need);
   hipStream_t s = (hipStream_t)stream;
-  const int cpb = bn_cols_per_block(c);
-  const int64_t rows_per_block = (int64_t)(256 / cpb) * BN_ROWS_PER_THREAD;
-  const int64_t blocks = pce_div_up(n, rows_per_block);
-  if (blocks >= (1ll << 31)) PCE_FAIL(PCE_ECAPACITY, "pce_col_sums: %lld workgroups exceed the grid limit", (long long)blocks);
-  dim3 grid((unsigned)blocks, (unsigned)pce_div_up(c, cpb));
-  if (dtype == PCE_F16)
-    hipLaunchKernelGGL(col_sums_partial_kernel<half_t>, grid, dim3(256), 0, s, (const half_t *)a, (const half_t *)b,
-                       (long long)n, c, cpb, (double *)ws);
-  else
-    hipLaunchKernelGGL(col_sums_partial_kernel<float>, grid, dim3(256), 0, s, (const float *)a, (const float *)b, (long long)n,
-                       c, cpb, (double *)ws);
-  PCE_LAUNCH_CHECK("col_sums_partial");
+  int64_t blocks = 0;
+  int rc = bn_partial(a, b, dtype, n, c, (double *)ws, &blocks, s);
+  if (rc) return rc;
   hipLaunchKernelGGL(col_sums_final_kernel, dim3((unsigned)c), dim3(64), 0, s, (const double *)ws,
                      (long long)blocks, c, out);
   PCE_LAUNCH_CHECK("col_sums_final");
@@ -2625,24 +2697,6 @@ extern "C" int pce_col_affine(const void *x, const void *d, void *y, int32_t dty
 extern "C" int64_t pce_bn_workspace_bytes(int64_t n, int32_t c) {
   if (n <= 0 || c <= 0) return 0;
   return pce_align_up(pce_col_sums_workspace_bytes(n, c), 256) + 3 * (int64_t)c * (int64_t)sizeof(float);
-}
-
-static int bn_partial(const void *a, const void *b, int32_t dtype, int64_t n, int32_t c, double *partial, int64_t *blocks_out,
-                      hipStream_t s) {
-  const int cpb = bn_cols_per_block(c);
-  const int64_t rows_per_block = (int64_t)(256 / cpb) * BN_ROWS_PER_THREAD;
-  const int64_t blocks = pce_div_up(n, rows_per_block);
-  if (blocks >= (1ll << 31)) PCE_FAIL(PCE_ECAPACITY, "batch norm: %lld workgroups exceed the grid limit", (long long)blocks);
-  dim3 grid((unsigned)blocks, (unsigned)pce_div_up(c, cpb));
-  if (dtype == PCE_F16)
-    hipLaunchKernelGGL(col_sums_partial_kernel<half_t>, grid, dim3(256), 0, s, (const half_t *)a, (const half_t *)b,
-                       (long long)n, c, cpb, partial);
-  else
-    hipLaunchKernelGGL(col_sums_partial_kernel<float>, grid, dim3(256), 0, s, (const float *)a, (const float *)b, (long long)n,
-                       c, cpb, partial);
-  PCE_LAUNCH_CHECK("col_sums_partial");
-  *blocks_out = blocks;
-  return PCE_OK;
 }
 
 extern "C" int pce_bn_forward(const void *x, void *y, int32_t dtype, int64_t n, int32_t c, const float *weight,
