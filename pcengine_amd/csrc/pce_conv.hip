@@ -2067,20 +2067,23 @@ __device__ __forceinline__ void wgrad_fetch(float (&v)[PER], const T *__restrict
 // channel rows lie KP + 8 halfs apart, which keeps both the 8-byte stores of a half wavefront and the
 // 16-byte fragment reads of 16 consecutive channels in distinct banks.
 template <int BLK>
-__global__ void __launch_bounds__(256, 2) wgrad_f16_kernel(const half_t *__restrict__ in, const half_t *__restrict__ gout,
+__global__ void __launch_bounds__(BLK == 256 ? 512 : 256, BLK == 256 ? 1 : 2) wgrad_f16_kernel(const half_t *__restrict__ in, const half_t *__restrict__ gout,
                                                         long long n_rows, int c_in, int c_out, int kv, int mid,
                                                         const int *__restrict__ imap, const int *__restrict__ omap,
                                                         const int *__restrict__ kpos, const int *__restrict__ qkpos,
                                                         long long pair_tiles, long long tiles, int run, int ci_blocks,
                                                         int co_blocks, float *__restrict__ gw) {
-  constexpr int R = BLK / 64;
-  constexpr int KP = BLK == 128 ? 64 : 128;  // pairs per stage
-  constexpr int PG = KP / 4;                 // groups of 4 pairs; PG * (BLK / 8) == 256 threads
-  constexpr int LD = KP + 8;                 // halfs per channel row
-  static_assert(PG * (BLK / 8) == 256, "one thread per (4 pairs, 8 channels) cell of a stage");
+  constexpr int NT = BLK == 256 ? 512 : 256;  // threads: 4 x 2 wavefronts on a 256-wide block, else 2 x 2
+  constexpr int WR = NT / 128;                // wavefronts along ci (two along co)
+  constexpr int RI = BLK / (32 * WR), RJ = BLK / 64;  // 32 x 32 MFMA tiles per wavefront along ci, co
+  constexpr int KP = BLK == 64 ? 128 : 64;    // pairs per stage
+  constexpr int PG = KP / 4;                  // groups of 4 pairs; PG * (BLK / 8) == NT threads
+  constexpr int LD = KP + 8;                  // halfs per channel row
+  static_assert(PG * (BLK / 8) == NT, "one thread per (4 pairs, 8 channels) cell of a stage");
   __shared__ __attribute__((aligned(16))) half_t At[BLK][LD];
   __shared__ __attribute__((aligned(16))) half_t Gt[BLK][LD];
-  __shared__ int rows_in[128], rows_out[128];
+  __shared__ int rows_in[4][128], rows_out[4][128];  // row indices of a tile, a ring of four tiles
+  __shared__ int tile_w[4];                          // and its offset (-1: none)
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int l32 = lane & 31, g = lane >> 5;
   const int wr = wave >> 1, wc = wave & 1;
@@ -2091,23 +2094,23 @@ __global__ void __launch_bounds__(256, 2) wgrad_f16_kernel(const half_t *__restr
   const long long grp = (slot / (ci_blocks * co_blocks)) * 8 + (blockIdx.x & 7);
   const int ci0 = (rest / co_blocks) * BLK, co0 = (rest % co_blocks) * BLK;
 
-  f32x16 acc[R][R];
+  f32x16 acc[RI][RJ];
 #pragma unroll
-  for (int i = 0; i < R; ++i)
+  for (int i = 0; i < RI; ++i)
 #pragma unroll
-    for (int j = 0; j < R; ++j)
+    for (int j = 0; j < RJ; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
   int cur = -1;
   auto flush = [&](int widx) {
     float *dst = gw + (long long)widx * c_in * c_out;
 #pragma unroll
-    for (int i = 0; i < R; ++i)
+    for (int i = 0; i < RI; ++i)
 #pragma unroll
-      for (int j = 0; j < R; ++j)
+      for (int j = 0; j < RJ; ++j)
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-          int ci = ci0 + wr * (BLK / 2) + i * 32 + (e / 4) * 8 + g * 4 + (e % 4);
+          int ci = ci0 + wr * (BLK / WR) + i * 32 + (e / 4) * 8 + g * 4 + (e % 4);
           int co = co0 + wc * (BLK / 2) + j * 32 + l32;
           float v = acc[i][j][e];
           if (ci < c_in && co < c_out && v != 0.f) unsafeAtomicAdd(dst + (long long)ci * c_out + co, v);
@@ -2142,60 +2145,96 @@ __global__ void __launch_bounds__(256, 2) wgrad_f16_kernel(const half_t *__restr
       *reinterpret_cast<u32x2 *>(&dst[cg * 8 + 2 * d + 1][pg * 4]) = odd;
     }
   };
+  const long long t_begin = grp * run;
   const long long t_end = (grp + 1) * run < tiles ? (grp + 1) * run : tiles;
-  for (long long tile = grp * run; tile < t_end; ++tile) {
-    int widx;
-    __syncthreads();
+  if (t_begin >= t_end) return;  // uniform
+  constexpr int SPT = 128 / KP;  // stages per tile
+  const int n_stage = (int)(t_end - t_begin) * SPT;
+
+  // The loop runs over the stages of all tiles of the run as one sequence.  What stage s multiplies was
+  // gathered during stages s - 2 and s - 1 (two register sets alternate) from row indices published in LDS at
+  // the top of stage s - 2 and loaded from the map during stage s - 3, so neither the map read nor the gather
+  // is waited for at a tile boundary, and two stages of rows are in flight while one is multiplied.
+  int lw = 0;  // offset of the tile whose rows are loaded next (tiles of a run come in offset order)
+  if (t_begin < pair_tiles)
+    for (int i = 0; i < kv; ++i) lw += ((long long)qkpos[i + 1] <= t_begin * 128) ? 1 : 0;
+  int nri = -1, nro = -1, nw = -1;
+  auto load_rows = [&](long long tile) {  // map entries of a tile into registers
+    nri = nro = nw = -1;
+    if (tile >= t_end) return;
     if (tile < pair_tiles) {
-      long long q0 = tile * 128;
-      widx = 0;
-      for (int i = 0; i < kv; ++i) widx += ((long long)qkpos[i + 1] <= q0) ? 1 : 0;
-      if (widx >= kv) break;  // uniform
-      if (threadIdx.x < 128) {
-        long long p = q0 - qkpos[widx] + kpos[widx] + threadIdx.x;
-        bool ok = p < (long long)kpos[widx + 1];
-        rows_in[threadIdx.x] = ok ? imap[p] : -1;
-        rows_out[threadIdx.x] = ok ? omap[p] : -1;
+      const long long q0 = tile * 128;
+      while (lw < kv && (long long)qkpos[lw + 1] <= q0) ++lw;
+      if (lw >= kv) return;
+      nw = lw;
+      const long long p = q0 - qkpos[lw] + kpos[lw] + threadIdx.x;
+      if (threadIdx.x < 128 && p < (long long)kpos[lw + 1]) {
+        nri = imap[p];
+        nro = omap[p];
       }
     } else {
-      widx = mid;
-      if (threadIdx.x < 128) {
-        long long row = (tile - pair_tiles) * 128 + threadIdx.x;
-        rows_in[threadIdx.x] = rows_out[threadIdx.x] = row < n_rows ? (int)row : -1;
-      }
+      nw = mid;
+      const long long row = (tile - pair_tiles) * 128 + threadIdx.x;
+      if (threadIdx.x < 128 && row < n_rows) nri = nro = (int)row;
     }
-    if (cur >= 0 && widx != cur) flush(cur);
-    cur = widx;
+  };
+  auto store_rows = [&](int buf) {
+    if (threadIdx.x < 128) {
+      rows_in[buf][threadIdx.x] = nri;
+      rows_out[buf][threadIdx.x] = nro;
+    }
+    if (threadIdx.x == 0) tile_w[buf] = nw;
+  };
+  u32x4 va0[4], vg0[4], va1[4], vg1[4];
+  auto fetch = [&](u32x4 (&va)[4], u32x4 (&vg)[4], int stage) {
+    const int buf = (stage / SPT) & 3, p0 = (stage % SPT) * KP;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      va[q] = fetch_row(in, rows_in[buf][p0 + pg * 4 + q], c_in, ci0, vec_in);
+      vg[q] = fetch_row(gout, rows_out[buf][p0 + pg * 4 + q], c_out, co0, vec_out);
+    }
+  };
+  auto body = [&](int v, u32x4 (&va)[4], u32x4 (&vg)[4]) {
+    if ((v + 2) % SPT == 0) store_rows(((v + 2) / SPT) & 3);  // rows of the tile of stage v + 2, loaded a stage ago
+    __syncthreads();  // the MFMAs of the previous stage have read their operands
+    put(At, va);
+    put(Gt, vg);
     __syncthreads();
-    u32x4 va[4], vg[4];
-    auto fetch = [&](int p0) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        va[q] = fetch_row(in, rows_in[p0 + pg * 4 + q], c_in, ci0, vec_in);
-        vg[q] = fetch_row(gout, rows_out[p0 + pg * 4 + q], c_out, co0, vec_out);
-      }
-    };
-    fetch(0);
-#pragma unroll
-    for (int p0 = 0; p0 < 128; p0 += KP) {
-      if (p0) __syncthreads();  // the MFMAs of the previous stage have read their operands
-      put(At, va);
-      put(Gt, vg);
-      __syncthreads();
-      if (p0 + KP < 128) fetch(p0 + KP);
-#pragma unroll
-      for (int k0 = 0; k0 < KP; k0 += 16) {
-        half8 av[R], bv[R];
-#pragma unroll
-        for (int i = 0; i < R; ++i) av[i] = *reinterpret_cast<const half8 *>(&At[wr * (BLK / 2) + i * 32 + l32][k0 + 8 * g]);
-#pragma unroll
-        for (int j = 0; j < R; ++j) bv[j] = *reinterpret_cast<const half8 *>(&Gt[wc * (BLK / 2) + j * 32 + l32][k0 + 8 * g]);
-#pragma unroll
-        for (int i = 0; i < R; ++i)
-#pragma unroll
-          for (int j = 0; j < R; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[i], bv[j], acc[i][j], 0, 0, 0);
+    if (v % SPT == 0) {  // first stage of a tile: do its sums go to another offset's block than the last tile's?
+      const int w = __builtin_amdgcn_readfirstlane(tile_w[(v / SPT) & 3]);
+      if (w >= 0 && w != cur) {
+        if (cur >= 0) flush(cur);
+        cur = w;
       }
     }
+    if ((v + 3) % SPT == 0) load_rows(t_begin + (v + 3) / SPT);
+    if (v + 2 < n_stage) fetch(va, vg, v + 2);
+#pragma unroll
+    for (int k0 = 0; k0 < KP; k0 += 16) {
+      half8 av[RI], bv[RJ];
+#pragma unroll
+      for (int i = 0; i < RI; ++i) av[i] = *reinterpret_cast<const half8 *>(&At[wr * (BLK / WR) + i * 32 + l32][k0 + 8 * g]);
+#pragma unroll
+      for (int j = 0; j < RJ; ++j) bv[j] = *reinterpret_cast<const half8 *>(&Gt[wc * (BLK / 2) + j * 32 + l32][k0 + 8 * g]);
+#pragma unroll
+      for (int i = 0; i < RI; ++i)
+#pragma unroll
+        for (int j = 0; j < RJ; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[i], bv[j], acc[i][j], 0, 0, 0);
+    }
+  };
+  // what stages -3, -2 and -1 would have done for stages 0 and 1
+  load_rows(t_begin);
+  store_rows(0);
+  __syncthreads();
+  if (SPT == 1) load_rows(t_begin + 1);
+  fetch(va0, vg0, 0);
+  if (SPT == 1) store_rows(1);
+  __syncthreads();
+  load_rows(t_begin + 2 / SPT);
+  if (1 < n_stage) fetch(va1, vg1, 1);
+  for (int v = 0; v < n_stage; v += 2) {
+    body(v, va0, vg0);
+    if (v + 1 < n_stage) body(v + 1, va1, vg1);
   }
   if (cur >= 0) flush(cur);
 }
@@ -2326,13 +2365,16 @@ extern "C" int pce_conv_wgrad(const void *in, const void *gout, int32_t dtype, i
   long long tiles = pair_tiles + (mid >= 0 ? pce_div_up(n_out, 128) : 0);
   if (tiles <= 0) return PCE_OK;
   // 128 x 128 blocks of (ci, co) for wide layers, 64 x 64 otherwise.  Every run of tiles ends with one atomic
-  // per element of its block, so runs are made long enough to leave about 512 workgroups (one resident set:
-  // two per CU), or about 1024 where several blocks share many tiles (measured on 100k-voxel layers: a
-  // 128 -> 128 layer of 5111 tiles takes 174 / 131 / 122 us at 2048 / 1024 / 512 workgroups)
+  // per element of its block, and on layers of 10^5 rows those atomics cost as much as the tiles: runs are
+  // made long enough to leave one workgroup per CU, more only where the tiles are many (measured on the
+  // layers of a 100k-voxel U-Net: 128 -> 128, 5111 tiles: 135 / 87 / 98 / 113 / 168 us at 128 / 256 / 512 /
+  // 1024 / 2048 workgroups; 256 -> 256, four blocks, 5111 tiles: 498 / 279 / 268 / 246 / 247 us)
   const int blk = (c_in > 64 || c_out > 64) ? 128 : 64;
   const int ci_blocks = (c_in + blk - 1) / blk, co_blocks = (c_out + blk - 1) / blk;
   const long long tile_blocks = tiles * ci_blocks * co_blocks;
-  const long long target_wgs = (ci_blocks * co_blocks > 1 && tile_blocks >= 8192) ? 1024 : 512;
+  long long target_wgs = 256;
+  if (blk == 128 && ci_blocks * co_blocks >= 4) target_wgs = 1024;
+  if (blk == 64 && tile_blocks >= 2048) target_wgs = 512;
   long long run = tile_blocks / target_wgs;
   run = run < 1 ? 1 : (run > 256 ? 256 : run);
   long long blocks = pce_div_up(pce_div_up(tiles, run), 8) * 8 * ci_blocks * co_blocks;
