@@ -293,22 +293,30 @@ int pce_col_sums(const void *a_dev, const void *b_dev, int32_t dtype, int64_t n,
 int pce_col_affine(const void *x_dev, const void *d_dev, void *y_dev, int32_t dtype, int64_t n, int32_t c,
                    const float *kx_dev, const float *kd_dev, const float *k0_dev, int32_t act, float slope,
                    pce_stream_t stream);
-/* The whole pass in one call (three launches: partial sums, one thread per channel for the statistics
+/* The whole pass in one call (three launches: partial sums, one wavefront per channel for the statistics
  * and coefficients, the affine map).  weight, bias (fp32 [c], NULL: 1 and 0), running_mean / running_var
  * (fp32 [c]; updated in place with `momentum` and the unbiased variance when use_batch_stats and
  * momentum >= 0; read when !use_batch_stats) follow torch.nn.BatchNorm1d.  save_mean / save_rstd (fp32 [c])
  * receive what pce_bn_backward needs.  grad_weight / grad_bias (fp32 [c]) may be NULL.  ws: device,
- * pce_bn_workspace_bytes(n, c).  y may alias x; dx may alias dy. */
+ * pce_bn_workspace_bytes(n, c).  y may alias x; dx may alias dy.
+ * The block that follows the norm in the reference's networks -- the residual sum of spTensor.__add__
+ * (script/sptensor.py:80-91) and the ReLU / LeakyReLU of script/activation.py:6-15 -- can ride on the same
+ * passes: forward y = act(bn(x) + residual) (residual_dev [n,c] of the same dtype, or NULL); backward takes
+ * dy with respect to y together with y itself (y_act_dev) and the activation, multiplies dy by the
+ * activation's derivative (y > 0 ? 1 : 0 or slope) while it reads it, and returns the gradient with respect
+ * to x; the gradient with respect to the residual is that masked dy, which the caller forms itself when it
+ * needs it (then it passes the masked dy and PCE_ACT_NONE).  LeakyReLU needs slope > 0. */
 int64_t pce_bn_workspace_bytes(int64_t n, int32_t c);
-int pce_bn_forward(const void *x_dev, void *y_dev, int32_t dtype, int64_t n, int32_t c, const float *weight_dev,
-                   const float *bias_dev, float *running_mean_dev, float *running_var_dev,
+int pce_bn_forward(const void *x_dev, const void *residual_dev, void *y_dev, int32_t dtype, int64_t n, int32_t c,
+                   const float *weight_dev, const float *bias_dev, float *running_mean_dev, float *running_var_dev,
                    int32_t use_batch_stats, float momentum, float eps, float *save_mean_dev,
                    float *save_rstd_dev, void *ws_dev, int64_t ws_bytes, int32_t act, float slope,
                    pce_stream_t stream);
-int pce_bn_backward(const void *x_dev, const void *dy_dev, void *dx_dev, int32_t dtype, int64_t n, int32_t c,
-                    const float *weight_dev, const float *save_mean_dev, const float *save_rstd_dev,
-                    int32_t use_batch_stats, float *grad_weight_dev, float *grad_bias_dev, void *ws_dev,
-                    int64_t ws_bytes, pce_stream_t stream);
+int pce_bn_backward(const void *x_dev, const void *dy_dev, const void *y_act_dev, int32_t act, float slope,
+                    void *dx_dev, int32_t dtype, int64_t n, int32_t c, const float *weight_dev,
+                    const float *save_mean_dev, const float *save_rstd_dev, int32_t use_batch_stats,
+                    float *grad_weight_dev, float *grad_bias_dev, void *ws_dev, int64_t ws_bytes,
+                    pce_stream_t stream);
 
 /* out[n,c_out] = in[n,c_in] * weight[c_in,c_out]: the 1x1 stride-1 shortcut of the front end
  * (script/spconv.py:297-304), on the same MFMA tile kernel. */

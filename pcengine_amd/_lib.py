@@ -75,11 +75,11 @@ _SIGNATURES = {
     "pce_col_affine": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_int32,
                                  ctypes.c_float, c_void_p]),
     "pce_bn_workspace_bytes": (c_int64, [c_int64, c_int32]),
-    "pce_bn_forward": (c_int32, [c_void_p, c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_int32,
-                                 ctypes.c_float, ctypes.c_float, c_void_p, c_void_p, c_void_p, c_int64, c_int32, ctypes.c_float,
-                                 c_void_p]),
-    "pce_bn_backward": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_int32,
-                                  c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
+    "pce_bn_forward": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p,
+                                 c_int32, ctypes.c_float, ctypes.c_float, c_void_p, c_void_p, c_void_p, c_int64, c_int32,
+                                 ctypes.c_float, c_void_p]),
+    "pce_bn_backward": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, ctypes.c_float, c_void_p, c_int32, c_int64, c_int32,
+                                  c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
     "pce_kmap_workspace_bytes": (c_int64, [c_int64, c_int64, c_int32, c_int32]),
     "pce_kmap_build_batch": (c_int32, [POINTER(KmapProblem), c_int32, c_void_p]),
     "pce_kmap_build": (c_int32, [c_void_p, c_int64, c_void_p, c_int64, POINTER(Geom), c_void_p, c_int64] + [c_void_p] * 14 + [c_void_p]),

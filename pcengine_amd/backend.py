@@ -548,10 +548,10 @@ def _f32(t: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
 
 
 def bn_forward(x: torch.Tensor, weight, bias, running_mean, running_var, use_batch_stats: bool, momentum: float, eps: float,
-               act=None):
-    """Batch normalisation of the rows of ``x`` [n, c] (fp16 / fp32) in three launches.  ``momentum`` < 0
-    leaves the running statistics alone; they must be fp32 and are updated in place otherwise.
-    Returns (y, save_mean, save_rstd)."""
+               act=None, residual: Optional[torch.Tensor] = None):
+    """``act(batch_norm(x) + residual)`` over the rows of ``x`` [n, c] (fp16 / fp32) in three launches.
+    ``momentum`` < 0 leaves the running statistics alone; they must be fp32 and are updated in place
+    otherwise.  Returns (y, save_mean, save_rstd)."""
     lib = _lib.load()
     _require_cuda(x, "x")
     x = x.contiguous()
@@ -559,33 +559,47 @@ def bn_forward(x: torch.Tensor, weight, bias, running_mean, running_var, use_bat
     for name, t in (("running_mean", running_mean), ("running_var", running_var)):
         if t is not None and (t.dtype != torch.float32 or not t.is_contiguous() or t.numel() != c):
             raise ValueError(f"{name} must be a contiguous fp32 tensor of {c} elements")
+    if residual is not None:
+        if residual.shape != x.shape or residual.dtype != x.dtype or residual.device != x.device:
+            raise ValueError("the residual must match the normalised tensor in shape, dtype and device")
+        residual = residual.contiguous()
     w, b = _f32(weight), _f32(bias)
     y = torch.empty_like(x)
     save = torch.empty((2, c), dtype=torch.float32, device=x.device)
     ws_bytes = lib.pce_bn_workspace_bytes(n, c)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
     code, slope = _act_code(act)
-    _lib.check(lib.pce_bn_forward(x.data_ptr(), y.data_ptr(), _dtype_code(x), n, c, _ptr(w), _ptr(b), _ptr(running_mean),
-                                  _ptr(running_var), int(use_batch_stats), float(momentum), float(eps), save[0].data_ptr(),
-                                  save[1].data_ptr(), ws.data_ptr(), ws_bytes, code, slope, _stream(x.device)))
+    _lib.check(lib.pce_bn_forward(x.data_ptr(), _ptr(residual), y.data_ptr(), _dtype_code(x), n, c, _ptr(w), _ptr(b),
+                                  _ptr(running_mean), _ptr(running_var), int(use_batch_stats), float(momentum), float(eps),
+                                  save[0].data_ptr(), save[1].data_ptr(), ws.data_ptr(), ws_bytes, code, slope, _stream(x.device)))
     return y, save[0], save[1]
 
 
 def bn_backward(x: torch.Tensor, dy: torch.Tensor, weight, save_mean: torch.Tensor, save_rstd: torch.Tensor,
-                use_batch_stats: bool):
-    """(dx, grad_weight fp32, grad_bias fp32) of ``bn_forward`` (without activation)."""
+                use_batch_stats: bool, y_act: Optional[torch.Tensor] = None, act=None):
+    """(dx, grad_weight fp32, grad_bias fp32) of ``bn_forward``.  With ``act`` and its output ``y_act`` the
+    incoming gradient is taken with respect to the activation's output and masked while it is read."""
     lib = _lib.load()
     x = x.contiguous()
     dy = dy.to(x.dtype).contiguous()
     n, c = x.shape
     w = _f32(weight)
+    code, slope = _act_code(act)
+    if code != _lib.ACT_NONE:
+        if y_act is None or y_act.shape != x.shape or y_act.dtype != x.dtype:
+            raise ValueError("the gradient of an activation needs its output, shaped and typed like x")
+        if code == _lib.ACT_LEAKY_RELU and not slope > 0:
+            raise ValueError("the output of a LeakyReLU tells the sign of its input only for a positive slope")
+        y_act = y_act.contiguous()
+    else:
+        y_act = None
     dx = torch.empty_like(x)
     grads = torch.empty((2, c), dtype=torch.float32, device=x.device)
     ws_bytes = lib.pce_bn_workspace_bytes(n, c)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
-    _lib.check(lib.pce_bn_backward(x.data_ptr(), dy.data_ptr(), dx.data_ptr(), _dtype_code(x), n, c, _ptr(w),
-                                   save_mean.data_ptr(), save_rstd.data_ptr(), int(use_batch_stats), grads[0].data_ptr(),
-                                   grads[1].data_ptr(), ws.data_ptr(), ws_bytes, _stream(x.device)))
+    _lib.check(lib.pce_bn_backward(x.data_ptr(), dy.data_ptr(), _ptr(y_act), code, slope, dx.data_ptr(), _dtype_code(x), n, c,
+                                   _ptr(w), save_mean.data_ptr(), save_rstd.data_ptr(), int(use_batch_stats),
+                                   grads[0].data_ptr(), grads[1].data_ptr(), ws.data_ptr(), ws_bytes, _stream(x.device)))
     return dx, grads[0], grads[1]
 
 

@@ -452,6 +452,12 @@ __device__ __forceinline__ float act_apply(float v, int act, float slope) {
   if (act == PCE_ACT_LEAKY_RELU) return v > 0.f ? v : v * slope;
   return v;
 }
+// derivative of the activation where its output is `out` (ReLU and LeakyReLU with a positive slope keep the sign)
+__device__ __forceinline__ float act_slope_at(float out, int act, float slope) {
+  if (act == PCE_ACT_RELU) return out > 0.f ? 1.f : 0.f;
+  if (act == PCE_ACT_LEAKY_RELU) return out > 0.f ? 1.f : slope;
+  return 1.f;
+}
 
 // eight consecutive elements of a row of T as floats; VEC: the address is 16-byte aligned
 template <typename T, bool VEC>
@@ -2415,8 +2421,10 @@ extern "C" int pce_conv_wgrad(const void *in, const void *gout, int32_t dtype, i
 #define BN_ROWS_IN_FLIGHT 8
 #define BN_MAX_ROW_BLOCKS 1024
 template <typename T, int VEC>
-__global__ void __launch_bounds__(256) col_sums_partial_kernel(const T *__restrict__ a, const T *__restrict__ b, long long n,
-                                                               int c, int cols_per_block, double *__restrict__ partial) {
+__global__ void __launch_bounds__(256) col_sums_partial_kernel(const T *__restrict__ a, const T *__restrict__ b,
+                                                               const T *__restrict__ gate, int gate_act, float gate_slope,
+                                                               long long n, int c, int cols_per_block,
+                                                               double *__restrict__ partial) {
   typedef typename VecOf<T, VEC>::type V;
   // thread -> (vector column, row lane): a workgroup covers cols_per_block vector columns (a power of two up to
   // 256) with 256 / cols_per_block row lanes; blockIdx.y walks over the column blocks
@@ -2430,7 +2438,7 @@ __global__ void __launch_bounds__(256) col_sums_partial_kernel(const T *__restri
     const long long stride = (long long)gridDim.x * lanes;
     for (long long r0 = (long long)blockIdx.x * lanes + rl; r0 < n; r0 += stride * BN_ROWS_IN_FLIGHT) {
       // all loads of a step are requested before the first is used
-      V xs[BN_ROWS_IN_FLIGHT], ys[BN_ROWS_IN_FLIGHT];
+      V xs[BN_ROWS_IN_FLIGHT], ys[BN_ROWS_IN_FLIGHT], gs[BN_ROWS_IN_FLIGHT];
 #pragma unroll
       for (int k = 0; k < BN_ROWS_IN_FLIGHT; ++k) {
         const long long r = r0 + k * stride;
@@ -2439,6 +2447,7 @@ __global__ void __launch_bounds__(256) col_sums_partial_kernel(const T *__restri
         for (int j = 0; j < VEC; ++j) reinterpret_cast<T *>(&zero)[j] = (T)0;
         xs[k] = r < n ? *reinterpret_cast<const V *>(a + r * c + col0) : zero;
         ys[k] = b ? (r < n ? *reinterpret_cast<const V *>(b + r * c + col0) : zero) : xs[k];
+        gs[k] = (gate && r < n) ? *reinterpret_cast<const V *>(gate + r * c + col0) : zero;
       }
       float f1[VEC], f2[VEC];
 #pragma unroll
@@ -2447,7 +2456,9 @@ __global__ void __launch_bounds__(256) col_sums_partial_kernel(const T *__restri
       for (int k = 0; k < BN_ROWS_IN_FLIGHT; ++k)
 #pragma unroll
         for (int j = 0; j < VEC; ++j) {
-          const float x = (float)reinterpret_cast<const T *>(&xs[k])[j], y = (float)reinterpret_cast<const T *>(&ys[k])[j];
+          float x = (float)reinterpret_cast<const T *>(&xs[k])[j];
+          const float y = b ? (float)reinterpret_cast<const T *>(&ys[k])[j] : x;
+          if (gate) x *= act_slope_at((float)reinterpret_cast<const T *>(&gs[k])[j], gate_act, gate_slope);
           f1[j] += x;
           f2[j] += x * y;
         }
@@ -2548,10 +2559,10 @@ extern "C" int64_t pce_col_sums_workspace_bytes(int64_t n, int32_t c) {
 }
 
 // launches the partial-sum kernel; *blocks_out = row blocks written (partial[block][2][c])
-static int bn_partial(const void *a, const void *b, int32_t dtype, int64_t n, int32_t c, double *partial, int64_t *blocks_out,
-                      hipStream_t s) {
+static int bn_partial(const void *a, const void *b, const void *gate, int gate_act, float gate_slope, int32_t dtype, int64_t n,
+                      int32_t c, double *partial, int64_t *blocks_out, hipStream_t s) {
   const int full = dtype == PCE_F16 ? 8 : 4;
-  const int vec = (c % full == 0 && aligned16(a) && aligned16(b)) ? full : 1;
+  const int vec = (c % full == 0 && aligned16(a) && aligned16(b) && aligned16(gate)) ? full : 1;
   const int vcols = c / vec;
   int cpb = 1;   // vector columns per workgroup: the power of two >= vcols, at most 256
   while (cpb < vcols && cpb < 256) cpb <<= 1;
@@ -2560,8 +2571,8 @@ static int bn_partial(const void *a, const void *b, int32_t dtype, int64_t n, in
   if (blocks > BN_MAX_ROW_BLOCKS) blocks = BN_MAX_ROW_BLOCKS;
   dim3 grid((unsigned)blocks, (unsigned)pce_div_up(vcols, cpb));
 #define PCE_COLSUMS(T_, V_)                                                                                                   \
-  hipLaunchKernelGGL((col_sums_partial_kernel<T_, V_>), grid, dim3(256), 0, s, (const T_ *)a, (const T_ *)b, (long long)n, c, \
-                     cpb, partial)
+  hipLaunchKernelGGL((col_sums_partial_kernel<T_, V_>), grid, dim3(256), 0, s, (const T_ *)a, (const T_ *)b,                 \
+                     (const T_ *)gate, gate_act, gate_slope, (long long)n, c, cpb, partial)
   if (dtype == PCE_F16 && vec == 8)
     PCE_COLSUMS(half_t, 8);
   else if (dtype == PCE_F16)
@@ -2585,7 +2596,7 @@ extern "C" int pce_col_sums(const void *a, const void *b, int32_t dtype, int64_t
   if (!ws || ws_bytes < need) PCE_FAIL(PCE_EWORKSPACE, "pce_col_sums: workspace %lld < %lld", (long long)ws_bytes, (long long)need);
   hipStream_t s = (hipStream_t)stream;
   int64_t blocks = 0;
-  int rc = bn_partial(a, b, dtype, n, c, (double *)ws, &blocks, s);
+  int rc = bn_partial(a, b, nullptr, PCE_ACT_NONE, 0.f, dtype, n, c, (double *)ws, &blocks, s);
   if (rc) return rc;
   hipLaunchKernelGGL(col_sums_final_kernel, dim3((unsigned)c), dim3(64), 0, s, (const double *)ws,
                      (long long)blocks, c, out);
@@ -2602,7 +2613,7 @@ __global__ void __launch_bounds__(64) bn_finish_forward_kernel(const double *__r
                                                                 float *running_var, int use_batch_stats, float momentum,
                                                                 float eps, float *__restrict__ save_mean,
                                                                 float *__restrict__ save_rstd, float *__restrict__ kx,
-                                                                float *__restrict__ k0) {
+                                                                float *__restrict__ k0, float *__restrict__ ones) {
   const int j = blockIdx.x;   // one wavefront per channel
   double mean, var;
   if (use_batch_stats) {
@@ -2628,6 +2639,7 @@ __global__ void __launch_bounds__(64) bn_finish_forward_kernel(const double *__r
   save_rstd[j] = (float)rstd;
   kx[j] = (float)(w * rstd);
   k0[j] = (float)(b - mean * w * rstd);
+  if (ones) ones[j] = 1.f;   // coefficient of the residual term of the affine map
 }
 
 // Backward (sums of dy and dy*x): grad_bias = sum dy, grad_weight = S = sum dy*xhat,
@@ -2664,15 +2676,17 @@ template <typename T, int VEC>
 __global__ void __launch_bounds__(256) col_affine_kernel(const T *__restrict__ x, const T *__restrict__ d, T *__restrict__ y,
                                                          long long n, int c, const float *__restrict__ kx,
                                                          const float *__restrict__ kd, const float *__restrict__ k0, int act,
-                                                         float slope) {
+                                                         float slope, const T *__restrict__ gate, int gate_act,
+                                                         float gate_slope) {
   typedef typename VecOf<T, VEC>::type V;
   const int row_vecs = c / VEC;
   long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n * row_vecs) return;
   const int v = (int)(i - (i / row_vecs) * row_vecs);
   V xv = *reinterpret_cast<const V *>(x + i * VEC);
-  V dv = xv;
+  V dv = xv, gv = xv;
   if (d) dv = *reinterpret_cast<const V *>(d + i * VEC);
+  if (gate) gv = *reinterpret_cast<const V *>(gate + i * VEC);
   V out;
   // the thread's VEC coefficients are contiguous: 16-byte loads when VEC is a multiple of four
   float cx[VEC], c0[VEC], cd[VEC];
@@ -2700,28 +2714,27 @@ __global__ void __launch_bounds__(256) col_affine_kernel(const T *__restrict__ x
   }
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
-    float r = (float)(reinterpret_cast<const T *>(&xv)[j]) * cx[j] + c0[j];
+    float xj = (float)(reinterpret_cast<const T *>(&xv)[j]);
+    if (gate) xj *= act_slope_at((float)(reinterpret_cast<const T *>(&gv)[j]), gate_act, gate_slope);
+    float r = xj * cx[j] + c0[j];
     if (d) r += (float)(reinterpret_cast<const T *>(&dv)[j]) * cd[j];
     reinterpret_cast<T *>(&out)[j] = (T)act_apply(r, act, slope);
   }
   *reinterpret_cast<V *>(y + i * VEC) = out;
 }
 
-extern "C" int pce_col_affine(const void *x, const void *d, void *y, int32_t dtype, int64_t n, int32_t c, const float *kx,
-                              const float *kd, const float *k0, int32_t act, float slope, pce_stream_t stream) {
-  if (!x || !y || !kx || !k0 || (d && !kd)) PCE_FAIL(PCE_EINVAL, "pce_col_affine: null pointer");
-  if (dtype != PCE_F16 && dtype != PCE_F32) PCE_FAIL(PCE_EINVAL, "pce_col_affine: dtype %d", (int)dtype);
-  if (n <= 0 || c <= 0) PCE_FAIL(PCE_EINVAL, "pce_col_affine: n=%lld c=%d", (long long)n, (int)c);
-  if (act != PCE_ACT_NONE && act != PCE_ACT_RELU && act != PCE_ACT_LEAKY_RELU) PCE_FAIL(PCE_EINVAL, "pce_col_affine: activation %d", (int)act);
-  hipStream_t s = (hipStream_t)stream;
+// y = act(x' * kx + d * kd + k0), x' = x times the derivative of another activation where its output was `gate`
+static int col_affine_launch(const char *who, const void *x, const void *d, const void *gate, void *y, int32_t dtype, int64_t n,
+                             int32_t c, const float *kx, const float *kd, const float *k0, int32_t act, float slope,
+                             int32_t gate_act, float gate_slope, hipStream_t s) {
   const int vec = dtype == PCE_F16 ? 8 : 4;
-  const bool aligned = aligned16(x) && aligned16(y) && aligned16(d) && c % vec == 0;
+  const bool aligned = aligned16(x) && aligned16(y) && aligned16(d) && aligned16(gate) && c % vec == 0;
   const long long items = aligned ? n * (c / vec) : n * c;
-  if (pce_div_up(items, 256) >= (1ll << 31)) PCE_FAIL(PCE_ECAPACITY, "pce_col_affine: tensor too large for one launch");
+  if (pce_div_up(items, 256) >= (1ll << 31)) PCE_FAIL(PCE_ECAPACITY, "%s: tensor too large for one launch", who);
   dim3 grid((unsigned)pce_div_up(items, 256));
 #define PCE_AFFINE(T_, V_)                                                                                               \
   hipLaunchKernelGGL((col_affine_kernel<T_, V_>), grid, dim3(256), 0, s, (const T_ *)x, (const T_ *)d, (T_ *)y, (long long)n, c, \
-                     kx, kd, k0, act, slope)
+                     kx, kd, k0, act, slope, (const T_ *)gate, gate_act, gate_slope)
   if (dtype == PCE_F16 && aligned)
     PCE_AFFINE(half_t, 8);
   else if (dtype == PCE_F16)
@@ -2735,13 +2748,25 @@ extern "C" int pce_col_affine(const void *x, const void *d, void *y, int32_t dty
   return PCE_OK;
 }
 
+static bool act_known(int32_t act) { return act == PCE_ACT_NONE || act == PCE_ACT_RELU || act == PCE_ACT_LEAKY_RELU; }
+
+extern "C" int pce_col_affine(const void *x, const void *d, void *y, int32_t dtype, int64_t n, int32_t c, const float *kx,
+                              const float *kd, const float *k0, int32_t act, float slope, pce_stream_t stream) {
+  if (!x || !y || !kx || !k0 || (d && !kd)) PCE_FAIL(PCE_EINVAL, "pce_col_affine: null pointer");
+  if (dtype != PCE_F16 && dtype != PCE_F32) PCE_FAIL(PCE_EINVAL, "pce_col_affine: dtype %d", (int)dtype);
+  if (n <= 0 || c <= 0) PCE_FAIL(PCE_EINVAL, "pce_col_affine: n=%lld c=%d", (long long)n, (int)c);
+  if (!act_known(act)) PCE_FAIL(PCE_EINVAL, "pce_col_affine: activation %d", (int)act);
+  return col_affine_launch("pce_col_affine", x, d, nullptr, y, dtype, n, c, kx, kd, k0, act, slope, PCE_ACT_NONE, 0.f,
+                           (hipStream_t)stream);
+}
+
 // workspace of the fused entry points: the partial sums, then 3*c floats of coefficients
 extern "C" int64_t pce_bn_workspace_bytes(int64_t n, int32_t c) {
   if (n <= 0 || c <= 0) return 0;
   return pce_align_up(pce_col_sums_workspace_bytes(n, c), 256) + 3 * (int64_t)c * (int64_t)sizeof(float);
 }
 
-extern "C" int pce_bn_forward(const void *x, void *y, int32_t dtype, int64_t n, int32_t c, const float *weight,
+extern "C" int pce_bn_forward(const void *x, const void *residual, void *y, int32_t dtype, int64_t n, int32_t c, const float *weight,
                               const float *bias, float *running_mean, float *running_var, int32_t use_batch_stats,
                               float momentum, float eps, float *save_mean, float *save_rstd, void *ws, int64_t ws_bytes,
                               int32_t act, float slope, pce_stream_t stream) {
@@ -2749,24 +2774,30 @@ extern "C" int pce_bn_forward(const void *x, void *y, int32_t dtype, int64_t n, 
   if (dtype != PCE_F16 && dtype != PCE_F32) PCE_FAIL(PCE_EINVAL, "pce_bn_forward: dtype %d", (int)dtype);
   if (n <= 0 || c <= 0) PCE_FAIL(PCE_EINVAL, "pce_bn_forward: n=%lld c=%d", (long long)n, (int)c);
   if (!use_batch_stats && (!running_mean || !running_var)) PCE_FAIL(PCE_EINVAL, "pce_bn_forward: fixed statistics need running_mean and running_var");
+  if (!act_known(act)) PCE_FAIL(PCE_EINVAL, "pce_bn_forward: activation %d", (int)act);
   if (!ws || ws_bytes < pce_bn_workspace_bytes(n, c)) PCE_FAIL(PCE_EWORKSPACE, "pce_bn_forward: workspace %lld < %lld", (long long)ws_bytes, (long long)pce_bn_workspace_bytes(n, c));
   hipStream_t s = (hipStream_t)stream;
   double *partial = (double *)ws;
   float *coef = (float *)((char *)ws + pce_align_up(pce_col_sums_workspace_bytes(n, c), 256));
   int64_t blocks = 0;
   int rc;
-  if (use_batch_stats && (rc = bn_partial(x, nullptr, dtype, n, c, partial, &blocks, s))) return rc;
+  if (use_batch_stats && (rc = bn_partial(x, nullptr, nullptr, PCE_ACT_NONE, 0.f, dtype, n, c, partial, &blocks, s))) return rc;
   hipLaunchKernelGGL(bn_finish_forward_kernel, dim3((unsigned)c), dim3(64), 0, s, (const double *)partial,
                      (long long)blocks, (long long)n, c, weight, bias, running_mean, running_var, use_batch_stats, momentum, eps,
-                     save_mean, save_rstd, coef, coef + c);
+                     save_mean, save_rstd, coef, coef + c, residual ? coef + 2 * c : nullptr);
   PCE_LAUNCH_CHECK("bn_finish_forward");
-  return pce_col_affine(x, nullptr, y, dtype, n, c, coef, nullptr, coef + c, act, slope, stream);
+  return col_affine_launch("pce_bn_forward", x, residual, nullptr, y, dtype, n, c, coef, residual ? coef + 2 * c : nullptr, coef + c,
+                           act, slope, PCE_ACT_NONE, 0.f, s);
 }
 
-extern "C" int pce_bn_backward(const void *x, const void *dy, void *dx, int32_t dtype, int64_t n, int32_t c,
-                               const float *weight, const float *save_mean, const float *save_rstd, int32_t use_batch_stats,
-                               float *grad_weight, float *grad_bias, void *ws, int64_t ws_bytes, pce_stream_t stream) {
+extern "C" int pce_bn_backward(const void *x, const void *dy, const void *y_act, int32_t act, float slope, void *dx,
+                               int32_t dtype, int64_t n, int32_t c, const float *weight, const float *save_mean,
+                               const float *save_rstd, int32_t use_batch_stats, float *grad_weight, float *grad_bias, void *ws,
+                               int64_t ws_bytes, pce_stream_t stream) {
   if (!x || !dy || !dx || !save_mean || !save_rstd) PCE_FAIL(PCE_EINVAL, "pce_bn_backward: null pointer");
+  if (!act_known(act)) PCE_FAIL(PCE_EINVAL, "pce_bn_backward: activation %d", (int)act);
+  if (act != PCE_ACT_NONE && !y_act) PCE_FAIL(PCE_EINVAL, "pce_bn_backward: the gradient of an activation needs its output");
+  if (act == PCE_ACT_NONE) y_act = nullptr;
   if (dtype != PCE_F16 && dtype != PCE_F32) PCE_FAIL(PCE_EINVAL, "pce_bn_backward: dtype %d", (int)dtype);
   if (n <= 0 || c <= 0) PCE_FAIL(PCE_EINVAL, "pce_bn_backward: n=%lld c=%d", (long long)n, (int)c);
   if (!ws || ws_bytes < pce_bn_workspace_bytes(n, c)) PCE_FAIL(PCE_EWORKSPACE, "pce_bn_backward: workspace %lld < %lld", (long long)ws_bytes, (long long)pce_bn_workspace_bytes(n, c));
@@ -2774,13 +2805,14 @@ extern "C" int pce_bn_backward(const void *x, const void *dy, void *dx, int32_t 
   double *partial = (double *)ws;
   float *coef = (float *)((char *)ws + pce_align_up(pce_col_sums_workspace_bytes(n, c), 256));
   int64_t blocks = 0;
-  int rc = bn_partial(dy, x, dtype, n, c, partial, &blocks, s);
+  int rc = bn_partial(dy, x, y_act, act, slope, dtype, n, c, partial, &blocks, s);
   if (rc) return rc;
   hipLaunchKernelGGL(bn_finish_backward_kernel, dim3((unsigned)c), dim3(64), 0, s, (const double *)partial,
                      (long long)blocks, (long long)n, c, weight, save_mean, save_rstd, use_batch_stats, grad_weight, grad_bias, coef,
                      coef + c, coef + 2 * c);
   PCE_LAUNCH_CHECK("bn_finish_backward");
-  return pce_col_affine(dy, x, dx, dtype, n, c, coef, coef + c, coef + 2 * c, PCE_ACT_NONE, 0.f, stream);
+  return col_affine_launch("pce_bn_backward", dy, x, y_act, dx, dtype, n, c, coef, coef + c, coef + 2 * c, PCE_ACT_NONE, 0.f, act,
+                           slope, s);
 }
 
 // Map density rho = pairs per output row.  The deferred-scatter dataflow does only the useful

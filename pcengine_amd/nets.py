@@ -48,10 +48,8 @@ class ConvBN(nn.Module):
         if self.bn is None:
             act = "relu" if (self.relu is not None or relu_after_residual) else None
             return self.conv(x, act=act, residual=residual)
-        x = self.bn(self.conv(x))
-        if residual is not None:
-            x = x + residual
-        return ReLU(True)(x) if (self.relu is not None or relu_after_residual) else x
+        # training form: the residual sum and the ReLU ride on the norm's affine pass
+        return self.bn(self.conv(x), residual=residual, act="relu" if (self.relu is not None or relu_after_residual) else None)
 
 
 class ResidualBlock(nn.Module):

@@ -97,3 +97,57 @@ def test_column_kernels_directly_and_their_errors():
     assert lib.pce_col_affine(one, None, one, 1, 10, 4, one, None, None, 0, 0.0, None) == _lib.PCE_EINVAL   # k0 missing
     assert lib.pce_col_affine(one, one, one, 1, 10, 4, one, None, one, 0, 0.0, None) == _lib.PCE_EINVAL    # d without kd
     assert lib.pce_col_affine(one, None, one, 1, 10, 4, one, None, one, 9, 0.0, None) == _lib.PCE_EINVAL   # activation
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 3e-6), (torch.float16, 1.5e-3)])
+@pytest.mark.parametrize("n,c", [(30000, 64), (777, 20), (4097, 7)])
+@pytest.mark.parametrize("with_residual", [False, True])
+@pytest.mark.parametrize("act", ["relu", ("leaky_relu", 0.1), None])
+def test_batchnorm_with_residual_and_activation(n, c, dtype, tol, with_residual, act):
+    """act(norm(x) + residual) in the norm's own passes against the same composition of torch modules in
+    float64: output and the gradients of x, weight, bias and the residual."""
+    rng = np.random.default_rng(n * 3 + c)
+    f = (rng.standard_normal((n, c)) * 1.5 + 0.3).astype(np.float32)
+    r = rng.standard_normal((n, c)).astype(np.float32)
+    go = rng.standard_normal((n, c)).astype(np.float32)
+    w, b = rng.uniform(0.5, 1.5, c), rng.uniform(-1, 1, c)
+    ref = torch.nn.BatchNorm1d(c).double()
+    bn = pe.BatchNorm(c).to(DEV)
+    with torch.no_grad():
+        ref.weight.copy_(torch.as_tensor(w)); ref.bias.copy_(torch.as_tensor(b))
+        bn.weight.copy_(torch.as_tensor(w)); bn.bias.copy_(torch.as_tensor(b))
+    fr = torch.as_tensor(f).to(dtype).double().requires_grad_(True)
+    rr = torch.as_tensor(r).to(dtype).double().requires_grad_(True)
+    yr = ref(fr) + (rr if with_residual else 0.0)
+    if act == "relu":
+        yr = torch.relu(yr)
+    elif act is not None:
+        yr = torch.nn.functional.leaky_relu(yr, act[1])
+    yr.backward(torch.as_tensor(go).to(dtype).double())
+    x, res = _tensor(f, dtype), _tensor(r, dtype)
+    y = bn(x, residual=res if with_residual else None, act=act)
+    y.feats.backward(torch.as_tensor(go, device=DEV).to(dtype))
+    assert y.feats.dtype == dtype
+    assert orc.rel_l2(y.feats.detach().double().cpu().numpy(), yr.detach().numpy()) <= tol
+    # an output that rounds to zero in fp16 masks its gradient where float64 keeps a tiny positive value
+    assert orc.rel_l2(x.feats.grad.double().cpu().numpy(), fr.grad.numpy()) <= 3 * tol
+    assert orc.rel_l2(bn.weight.grad.double().cpu().numpy(), ref.weight.grad.numpy()) <= 3 * max(tol, 1e-5)
+    assert orc.rel_l2(bn.bias.grad.double().cpu().numpy(), ref.bias.grad.numpy()) <= 3 * max(tol, 1e-5)
+    if with_residual:
+        assert orc.rel_l2(res.feats.grad.double().cpu().numpy(), rr.grad.numpy()) <= 3 * tol
+    else:
+        assert res.feats.grad is None
+
+
+def test_batchnorm_activation_arguments():
+    bn = pe.BatchNorm(8).to(DEV)
+    x = _tensor(np.ones((16, 8), np.float32), torch.float32)
+    with pytest.raises(ValueError):
+        bn(x, act="gelu")
+    with pytest.raises(ValueError):
+        bn(x, act=("leaky_relu", -0.1))
+    y, mean, rstd = backend.bn_forward(x.feats.detach(), None, None, None, None, True, -1.0, 1e-5, act="relu")
+    with pytest.raises(ValueError):
+        backend.bn_backward(x.feats.detach(), y, None, mean, rstd, True, y_act=None, act="relu")
+    with pytest.raises(ValueError):
+        backend.bn_forward(x.feats.detach(), None, None, None, None, True, -1.0, 1e-5, residual=torch.zeros(3, 8, device=DEV))
