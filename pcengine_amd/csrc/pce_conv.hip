@@ -2421,11 +2421,31 @@ extern "C" int pce_conv_wgrad(const void *in, const void *gout, int32_t dtype, i
 #define BN_ROWS_IN_FLIGHT 8
 #define BN_MAX_ROW_BLOCKS 1024
 template <typename T, int VEC>
+__device__ __forceinline__ float vec_get(const typename VecOf<T, VEC>::type &v, int j) {
+  if constexpr (VEC == 1)
+    return (float)v;
+  else
+    return (float)v[j];
+}
+template <typename T, int VEC>
+__device__ __forceinline__ typename VecOf<T, VEC>::type vec_zero() {
+  typename VecOf<T, VEC>::type v;
+  if constexpr (VEC == 1) {
+    v = (T)0;
+  } else {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) v[j] = (T)0;
+  }
+  return v;
+}
+// GATED: a third operand (the gate) is read, and half as many rows are requested per step
+template <typename T, int VEC, bool GATED>
 __global__ void __launch_bounds__(256) col_sums_partial_kernel(const T *__restrict__ a, const T *__restrict__ b,
                                                                const T *__restrict__ gate, int gate_act, float gate_slope,
                                                                long long n, int c, int cols_per_block,
                                                                double *__restrict__ partial) {
   typedef typename VecOf<T, VEC>::type V;
+  constexpr int ROWS = GATED ? BN_ROWS_IN_FLIGHT / 2 : BN_ROWS_IN_FLIGHT;
   // thread -> (vector column, row lane): a workgroup covers cols_per_block vector columns (a power of two up to
   // 256) with 256 / cols_per_block row lanes; blockIdx.y walks over the column blocks
   const int tc = threadIdx.x % cols_per_block;
@@ -2436,29 +2456,27 @@ __global__ void __launch_bounds__(256) col_sums_partial_kernel(const T *__restri
   for (int j = 0; j < VEC; ++j) s1[j] = s2[j] = 0.0;
   if (col0 < c) {
     const long long stride = (long long)gridDim.x * lanes;
-    for (long long r0 = (long long)blockIdx.x * lanes + rl; r0 < n; r0 += stride * BN_ROWS_IN_FLIGHT) {
+    for (long long r0 = (long long)blockIdx.x * lanes + rl; r0 < n; r0 += stride * ROWS) {
       // all loads of a step are requested before the first is used
-      V xs[BN_ROWS_IN_FLIGHT], ys[BN_ROWS_IN_FLIGHT], gs[BN_ROWS_IN_FLIGHT];
+      V xs[ROWS], ys[ROWS], gs[GATED ? ROWS : 1];
+      const V zero = vec_zero<T, VEC>();
 #pragma unroll
-      for (int k = 0; k < BN_ROWS_IN_FLIGHT; ++k) {
+      for (int k = 0; k < ROWS; ++k) {
         const long long r = r0 + k * stride;
-        V zero;
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) reinterpret_cast<T *>(&zero)[j] = (T)0;
         xs[k] = r < n ? *reinterpret_cast<const V *>(a + r * c + col0) : zero;
         ys[k] = b ? (r < n ? *reinterpret_cast<const V *>(b + r * c + col0) : zero) : xs[k];
-        gs[k] = (gate && r < n) ? *reinterpret_cast<const V *>(gate + r * c + col0) : zero;
+        if (GATED) gs[k] = r < n ? *reinterpret_cast<const V *>(gate + r * c + col0) : zero;
       }
       float f1[VEC], f2[VEC];
 #pragma unroll
       for (int j = 0; j < VEC; ++j) f1[j] = f2[j] = 0.f;
 #pragma unroll
-      for (int k = 0; k < BN_ROWS_IN_FLIGHT; ++k)
+      for (int k = 0; k < ROWS; ++k)
 #pragma unroll
         for (int j = 0; j < VEC; ++j) {
-          float x = (float)reinterpret_cast<const T *>(&xs[k])[j];
-          const float y = b ? (float)reinterpret_cast<const T *>(&ys[k])[j] : x;
-          if (gate) x *= act_slope_at((float)reinterpret_cast<const T *>(&gs[k])[j], gate_act, gate_slope);
+          float x = vec_get<T, VEC>(xs[k], j);
+          const float y = vec_get<T, VEC>(ys[k], j);
+          if (GATED) x *= act_slope_at(vec_get<T, VEC>(gs[k], j), gate_act, gate_slope);
           f1[j] += x;
           f2[j] += x * y;
         }
@@ -2571,8 +2589,12 @@ static int bn_partial(const void *a, const void *b, const void *gate, int gate_a
   if (blocks > BN_MAX_ROW_BLOCKS) blocks = BN_MAX_ROW_BLOCKS;
   dim3 grid((unsigned)blocks, (unsigned)pce_div_up(vcols, cpb));
 #define PCE_COLSUMS(T_, V_)                                                                                                   \
-  hipLaunchKernelGGL((col_sums_partial_kernel<T_, V_>), grid, dim3(256), 0, s, (const T_ *)a, (const T_ *)b,                 \
-                     (const T_ *)gate, gate_act, gate_slope, (long long)n, c, cpb, partial)
+  if (gate)                                                                                                                  \
+    hipLaunchKernelGGL((col_sums_partial_kernel<T_, V_, true>), grid, dim3(256), 0, s, (const T_ *)a,       \
+                       (const T_ *)b, (const T_ *)gate, gate_act, gate_slope, (long long)n, c, cpb, partial);                \
+  else                                                                                                                       \
+    hipLaunchKernelGGL((col_sums_partial_kernel<T_, V_, false>), grid, dim3(256), 0, s, (const T_ *)a,                       \
+                       (const T_ *)b, (const T_ *)gate, gate_act, gate_slope, (long long)n, c, cpb, partial)
   if (dtype == PCE_F16 && vec == 8)
     PCE_COLSUMS(half_t, 8);
   else if (dtype == PCE_F16)
