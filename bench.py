@@ -264,6 +264,19 @@ def main() -> int:
         os.environ.pop("PCENGINE_DATAFLOW", None)
         result["extra"]["cfg4_minkunet"] = {"voxels": int(len(c4)), "dtype": "f16", "selector": net["auto"],
                                             "all_fetch_on_demand": net["fod"], "all_gather_gemm_scatter": net["gms"]}
+        # the same network in training mode (BatchNorm on batch statistics, cross-entropy on random labels):
+        # forward + backward with kernel maps built every step, fp16 features and fp32 parameters
+        torch.manual_seed(5)
+        train_model = nets.SparseResUNet(4, 20).to(dev).train()
+        target = torch.randint(0, 20, (len(c4),), device=dev)
+
+        def train_step():
+            train_model.zero_grad(set_to_none=True)
+            x = pe.spTensor(f4, c4d, None, [0, 0, 0], cmax4)
+            loss = torch.nn.functional.cross_entropy(train_model(x).feats.float(), target)
+            loss.backward()
+        result["extra"]["cfg4_minkunet"]["training_step_ms"] = round(ev_ms(train_step, 5, 2), 3)
+        del train_model
 
     # ---- configurations 1, 3 and 5 (opt-in) ------------------------------------------------------------
     if args.all_configs:
