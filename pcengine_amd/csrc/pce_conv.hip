@@ -2417,9 +2417,10 @@ extern "C" int pce_conv_wgrad(const void *in, const void *gout, int32_t dtype, i
 // A thread owns VEC adjacent columns (one 16-byte vector when the layout allows) and walks down the rows in
 // steps of the grid, 8 rows requested at a time; sums are accumulated in fp32 over those 8 rows, then in fp64:
 // per workgroup through LDS, across workgroups by a second kernel over the per-workgroup partial sums (no
-// atomics: same bits every run).  At most BN_MAX_ROW_BLOCKS workgroups share the rows.
+// atomics: same bits every run).  At most BN_MAX_ROW_BLOCKS workgroups share the rows: three per CU, what the
+// vector forms keep resident, so that no second, partial round of workgroups follows the first.
 #define BN_ROWS_IN_FLIGHT 8
-#define BN_MAX_ROW_BLOCKS 1024
+#define BN_MAX_ROW_BLOCKS 768
 template <typename T, int VEC>
 __device__ __forceinline__ float vec_get(const typename VecOf<T, VEC>::type &v, int j) {
   if constexpr (VEC == 1)
