@@ -53,6 +53,8 @@ class BatchNorm(nn.BatchNorm1d):
             native = self.running_mean.dtype == torch.float32 and self.running_var.dtype == torch.float32
         if native and residual is not None:
             native = residual.dtype == x.dtype and residual.shape == x.shape
+        if native and self.training and x.shape[0] == 1:
+            native = False                  # torch refuses batch statistics of a single row: keep its error
         if not native:                      # CPU tensors, other dtypes: torch's own kernels
             y = super().forward(x)
             if residual is not None:

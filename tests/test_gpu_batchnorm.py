@@ -141,6 +141,8 @@ def test_batchnorm_with_residual_and_activation(n, c, dtype, tol, with_residual,
 
 def test_batchnorm_activation_arguments():
     bn = pe.BatchNorm(8).to(DEV)
+    with pytest.raises(ValueError):      # torch.nn.BatchNorm1d refuses batch statistics of one row
+        bn(_tensor(np.ones((1, 8), np.float32), torch.float32))
     x = _tensor(np.ones((16, 8), np.float32), torch.float32)
     with pytest.raises(ValueError):
         bn(x, act="gelu")
