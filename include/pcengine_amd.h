@@ -254,6 +254,10 @@ int pce_conv_fwd_gms(const void *in_feats, const void *weight, const void *weigh
  * GEMM together (neither reads what the other writes), then one pass over the pairs that adds
  * each output row's partial rows to the centre term already stored there.  Rows with partial
  * rows are then rounded to dtype twice (centre term, final sum).
+ * buffer_dev may be NULL when the layer has no centre offset (mid < 0), omap_dev is given and
+ * n_pairs == n_out: the caller then states that every output row has exactly one pair (a transposed
+ * layer whose kernel size equals its stride: every fine voxel has one parent), and each pair's product
+ * is stored straight to its output row with the epilogue, without partial rows or a second pass.
  * No counterpart in the reference: it is ConvolutionForwardD2 with the atomic scatter-add replaced
  * by the output-stationary sum of ConvolutionForwardD1 (backend/spconv.cu:149-161), fused with
  * the centre GEMM. */

@@ -482,15 +482,18 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
                                         km.qkpos.data_ptr(), km.qsum, _ptr(ws), ws_bytes, epi, s))
     elif dataflow == DATAFLOW_FDS:
         ensure_csr(km)
-        need = km.M * c_out
-        if buffer is None or buffer.numel() < need or buffer.dtype != feats.dtype or buffer.device != dev:
+        # A transposed layer whose kernel equals its stride gives every fine voxel at most one parent; when no
+        # parent was clipped away (M == n_out) every output row has exactly one pair and needs no partial rows.
+        single = transposed and tuple(km.ks) == tuple(km.stride) and km.M == n_out and km.M > 0
+        need = 0 if single else km.M * c_out
+        if not single and (buffer is None or buffer.numel() < need or buffer.dtype != feats.dtype or buffer.device != dev):
             buffer = torch.empty(max(need, 1), dtype=feats.dtype, device=dev)
         imap, omap = (km.omap, km.imap) if transposed else (km.imap, km.omap)
         ocsr, oslot = (km.icsr, km.islot) if transposed else (km.ocsr, km.oslot)
         _lib.check(lib.pce_conv_fwd_fds(feats.data_ptr(), weight.data_ptr(), _ptr(packed), out.data_ptr(), dt, n_in, n_out,
                                         c_in, c_out, kv, mid, imap.data_ptr(), omap.data_ptr(), oslot.data_ptr(), km.kpos.data_ptr(),
                                         km.qkpos.data_ptr(), km.kpos_host, km.qkpos_host, ocsr.data_ptr(), km.M, km.qsum,
-                                        buffer.data_ptr(), buffer.numel(), epi, s))
+                                        None if single else buffer.data_ptr(), 0 if single else buffer.numel(), epi, s))
     elif dataflow == DATAFLOW_GMS:
         ensure_csr(km)
         need = km.qsum * (c_in + c_out)

@@ -1848,6 +1848,21 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
                     T *buffer, const Epi &e, hipStream_t s) {
   constexpr int VEC = sizeof(T) == 2 ? 8 : 4;
   int rc;
+  if (!buffer && qsum > 0) {
+    // Every output row has exactly one pair (a transposed layer whose kernel equals its stride: each fine
+    // voxel has one parent): a pair's product is its output row, stored once with the epilogue, no partial rows.
+    TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
+    set_out<T>(&a, out, false);
+    set_host_pos(&a, kpos_host, qkpos_host);
+    a.imap = imap;
+    a.oslot = omap;
+    a.kpos = kpos;
+    a.qkpos = qkpos;
+    a.mode = MODE_FOD_BUF;
+    a.epi = EPI_ROWS;
+    set_epi(&a, e);
+    return launch_tile<T>(a, qsum / PCE_QUANTUM, s);
+  }
   if (mid >= 0 && qsum > 0 && omap && stage_on(4)) {
     // Pair chunks and centre GEMM share one launch (neither reads what the other writes); a pass
     // over the pairs then adds every output row's partial rows to the centre term stored there.
@@ -1975,8 +1990,13 @@ extern "C" int pce_conv_fwd_fds(const void *in, const void *w, const void *wp, v
   if ((rc = read_epilogue("pce_conv_fwd_fds", epilogue, out, &e))) return rc;
   if (!ocsr || !kpos || !qkpos || (qsum > 0 && (!imap || !oslot))) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_fds: null map pointer");
   if (n_pairs < 0 || n_pairs > qsum) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_fds: n_pairs=%lld outside [0, qsum]", (long long)n_pairs);
-  if (n_pairs > 0 && (!buffer || buffer_elems < n_pairs * (int64_t)c_out))
+  if (!buffer && n_pairs > 0) {
+    // no partial-row buffer: the caller states that every output row has exactly one pair
+    if (mid >= 0 || !omap || n_pairs != n_out)
+      PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_fds: without a buffer the layer must have no centre offset, omap and n_pairs == n_out");
+  } else if (n_pairs > 0 && buffer_elems < n_pairs * (int64_t)c_out) {
     PCE_FAIL(PCE_EWORKSPACE, "pce_conv_fwd_fds: buffer holds %lld elements, needs %lld", (long long)buffer_elems, (long long)(n_pairs * (int64_t)c_out));
+  }
   hipStream_t s = (hipStream_t)stream;
   if (dtype == PCE_F16)
     return fds_impl<half_t>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, omap, oslot, kpos, qkpos, kpos_host, qkpos_host, ocsr, n_pairs, qsum, (half_t *)buffer, e, s);

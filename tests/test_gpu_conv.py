@@ -283,3 +283,36 @@ def test_reference_named_entry_points_d2_and_d1():
     backend.conv_bwd_d1_cuda(gd, f32, w32, enc([3, 3, 3]), qsum, in_grad, w_grad, knnz, kpos, imap, omap, icsr, ocsr, buffer, 1)
     gf, gw = orc.conv_backward(f32.double().cpu().numpy(), w32.double().cpu().numpy(), ref_map, (3, 3, 3), rounded(g, torch.float32))
     assert orc.rel_l2(in_grad.double().cpu().numpy(), gf) <= 1e-5 and orc.rel_l2(w_grad.double().cpu().numpy(), gw) <= 1e-5
+
+
+def test_deferred_scatter_without_buffer_needs_one_pair_per_row():
+    """pce_conv_fwd_fds takes no partial-row buffer only for a layer without centre offset whose pair count
+    equals its output rows (a transposed layer with kernel == stride); anything else is an argument error."""
+    from pcengine_amd import _lib
+    lib = _lib.load()
+    coords = synth.random_cloud(seed=47, n=3000, extent=12)
+    fd, wd, _, _ = _case(coords, (3, 3, 3), (1, 1, 1), (0, 0, 0), 32, 32, torch.float16)
+    km = gpu_map(coords, (3, 3, 3), want_csr=True)
+    out = torch.empty((km.n_out, 32), dtype=torch.float16, device=DEV)
+
+    def call(mid, n_pairs):
+        return lib.pce_conv_fwd_fds(fd.data_ptr(), wd.data_ptr(), None, out.data_ptr(), _lib.PCE_F16, km.n_in, km.n_out, 32, 32,
+                                    km.kv, mid, km.imap.data_ptr(), km.omap.data_ptr(), km.oslot.data_ptr(), km.kpos.data_ptr(),
+                                    km.qkpos.data_ptr(), None, None, km.ocsr.data_ptr(), n_pairs, km.qsum, None, 0, None, None)
+    assert call(13, km.M) == _lib.PCE_EINVAL          # centre offset present
+    assert call(-1, km.M) == _lib.PCE_EINVAL          # pairs != output rows
+    # the transposed 2x2x2 stride-2 layer qualifies: same result with and without the caller's buffer
+    km2 = gpu_map(coords, (2, 2, 2), (2, 2, 2), want_csr=True)
+    assert km2.M == km2.n_in
+    down = torch.as_tensor(synth.features(5, km2.n_out, 48), device=DEV).half()
+    wt = torch.as_tensor(synth.weights(5, 8, 48, 32), device=DEV).half()
+    direct = backend.conv_forward(down, wt, km2, DATAFLOW_FDS, transposed=True, packed=backend.pack_weights(wt))
+    buf = torch.empty(km2.M * 32, dtype=torch.float16, device=DEV)
+    back = torch.empty((km2.n_in, 32), dtype=torch.float16, device=DEV)
+    rc = lib.pce_conv_fwd_fds(down.data_ptr(), wt.data_ptr(), backend.pack_weights(wt).data_ptr(), back.data_ptr(), _lib.PCE_F16,
+                              km2.n_out, km2.n_in, 48, 32, 8, -1, km2.omap.data_ptr(), km2.imap.data_ptr(), km2.islot.data_ptr(),
+                              km2.kpos.data_ptr(), km2.qkpos.data_ptr(), None, None, km2.icsr.data_ptr(), km2.M, km2.qsum,
+                              buf.data_ptr(), buf.numel(), None, None)
+    assert rc == _lib.PCE_OK
+    torch.cuda.synchronize()
+    assert torch.equal(direct, back)
