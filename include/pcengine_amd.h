@@ -322,6 +322,13 @@ int pce_bn_backward(const void *x_dev, const void *dy_dev, const void *y_act_dev
                     float *grad_weight_dev, float *grad_bias_dev, void *ws_dev, int64_t ws_bytes,
                     pce_stream_t stream);
 
+/* out[n, c_a + c_b] = (a[n, c_a], b[n, c_b]): the skip concatenation of the reference's `cat`
+ * (script/utils.py:152-164) for two tensors on the same rows.  Rows must be whole 16-byte vectors
+ * (c_a, c_b multiples of 8 for PCE_F16, 4 for PCE_F32) and the pointers 16-byte aligned (PCE_EINVAL
+ * otherwise: the caller concatenates some other way); at most 256 vectors per output row. */
+int pce_concat_cols(const void *a_dev, int32_t c_a, const void *b_dev, int32_t c_b, void *out_dev, int32_t dtype,
+                    int64_t n, pce_stream_t stream);
+
 /* out[n,c_out] = in[n,c_in] * weight[c_in,c_out]: the 1x1 stride-1 shortcut of the front end
  * (script/spconv.py:297-304), on the same MFMA tile kernel. */
 int pce_conv_fwd_dense(const void *in_feats, const void *weight, const void *weight_packed,

@@ -80,6 +80,7 @@ _SIGNATURES = {
                                  ctypes.c_float, c_void_p]),
     "pce_bn_backward": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, ctypes.c_float, c_void_p, c_int32, c_int64, c_int32,
                                   c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
+    "pce_concat_cols": (c_int32, [c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_int32, c_int64, c_void_p]),
     "pce_kmap_workspace_bytes": (c_int64, [c_int64, c_int64, c_int32, c_int32]),
     "pce_kmap_build_batch": (c_int32, [POINTER(KmapProblem), c_int32, c_void_p]),
     "pce_kmap_build": (c_int32, [c_void_p, c_int64, c_void_p, c_int64, POINTER(Geom), c_void_p, c_int64] + [c_void_p] * 14 + [c_void_p]),

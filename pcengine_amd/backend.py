@@ -546,6 +546,25 @@ def col_affine(x: torch.Tensor, kx: torch.Tensor, k0: torch.Tensor, d: Optional[
     return y
 
 
+def concat_cols(a: torch.Tensor, b: torch.Tensor) -> Optional[torch.Tensor]:
+    """``torch.cat([a, b], dim=1)`` for two feature matrices on the same rows in one streaming kernel, or None
+    when the layout does not fit it (rows that are not whole 16-byte vectors, other dtypes, CPU tensors)."""
+    if not (a.is_cuda and b.is_cuda and a.device == b.device and a.dim() == 2 and b.dim() == 2 and a.dtype == b.dtype
+            and a.dtype in (torch.float16, torch.float32) and a.shape[0] == b.shape[0] and a.shape[0] > 0):
+        return None
+    per = 8 if a.dtype == torch.float16 else 4
+    c_a, c_b = a.shape[1], b.shape[1]
+    if c_a == 0 or c_b == 0 or c_a % per or c_b % per or (c_a + c_b) // per > 256:
+        return None
+    a, b = a.contiguous(), b.contiguous()
+    out = torch.empty((a.shape[0], c_a + c_b), dtype=a.dtype, device=a.device)
+    if a.data_ptr() % 16 or b.data_ptr() % 16:
+        return None
+    _lib.check(_lib.load().pce_concat_cols(a.data_ptr(), c_a, b.data_ptr(), c_b, out.data_ptr(), _dtype_code(a), a.shape[0],
+                                           _stream(a.device)))
+    return out
+
+
 def _f32(t: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
     return None if t is None else t.detach().to(dtype=torch.float32).contiguous()
 

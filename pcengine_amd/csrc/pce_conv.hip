@@ -2858,6 +2858,38 @@ extern "C" int pce_bn_backward(const void *x, const void *dy, const void *y_act,
                            slope, s);
 }
 
+// ---- channel concatenation of two feature matrices on the same rows (script/utils.py:152-164) ---------
+// out[r] = (a[r], b[r]).  One 16-byte vector per thread; threadIdx.x walks along the output row, so a
+// wavefront reads and writes whole rows.  va / vb = vectors per row of a / b.
+__global__ void __launch_bounds__(256) concat_cols_kernel(const u32x4 *__restrict__ a, const u32x4 *__restrict__ b,
+                                                          u32x4 *__restrict__ out, long long n, int va, int vb) {
+  const long long r = (long long)blockIdx.x * blockDim.y + threadIdx.y;
+  const int v = threadIdx.x;
+  if (r >= n || v >= va + vb) return;
+  out[r * (va + vb) + v] = v < va ? a[r * va + v] : b[r * vb + (v - va)];
+}
+
+extern "C" int pce_concat_cols(const void *a, int32_t c_a, const void *b, int32_t c_b, void *out, int32_t dtype, int64_t n,
+                               pce_stream_t stream) {
+  if (!a || !b || !out) PCE_FAIL(PCE_EINVAL, "pce_concat_cols: null pointer");
+  if (dtype != PCE_F16 && dtype != PCE_F32) PCE_FAIL(PCE_EINVAL, "pce_concat_cols: dtype %d", (int)dtype);
+  if (n <= 0 || c_a <= 0 || c_b <= 0) PCE_FAIL(PCE_EINVAL, "pce_concat_cols: n=%lld c_a=%d c_b=%d", (long long)n, (int)c_a, (int)c_b);
+  const int per = dtype == PCE_F16 ? 8 : 4;   // elements per 16-byte vector
+  if (c_a % per || c_b % per || !aligned16(a) || !aligned16(b) || !aligned16(out))
+    PCE_FAIL(PCE_EINVAL, "pce_concat_cols: rows of %d and %d elements are not whole 16-byte vectors, or a pointer is unaligned", (int)c_a, (int)c_b);
+  const int va = c_a / per, vb = c_b / per;
+  if (va + vb > 256) PCE_FAIL(PCE_ECAPACITY, "pce_concat_cols: %d channels exceed one workgroup per row", (int)(c_a + c_b));
+  int tx = 1;
+  while (tx < va + vb) tx <<= 1;
+  const int ty = 256 / tx;
+  const long long blocks = pce_div_up(n, ty);
+  if (blocks >= (1ll << 31)) PCE_FAIL(PCE_ECAPACITY, "pce_concat_cols: %lld workgroups exceed the grid limit", blocks);
+  hipLaunchKernelGGL(concat_cols_kernel, dim3((unsigned)blocks), dim3(tx, ty), 0, (hipStream_t)stream, (const u32x4 *)a,
+                     (const u32x4 *)b, (u32x4 *)out, (long long)n, va, vb);
+  PCE_LAUNCH_CHECK("concat_cols");
+  return PCE_OK;
+}
+
 // Map density rho = pairs per output row.  The deferred-scatter dataflow does only the useful
 // multiplications and pays M*(c_in + 2*c_out) elements of gather / partial-row traffic for them; the
 // output-stationary kernel touches no intermediate memory but multiplies every offset of every

@@ -89,3 +89,29 @@ def test_batchnorm_and_residual_fp32():
     mean, var = bn.running_mean.double().cpu().numpy(), bn.running_var.double().cpu().numpy()
     want = np.maximum((z - mean) / np.sqrt(var + bn.eps), 0) + f
     assert orc.rel_l2(y.feats.double().cpu().numpy(), want) <= 1e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("n,c_a,c_b", [(1, 8, 8), (5000, 96, 32), (70001, 192, 64), (333, 256, 128), (4097, 12, 20), (100, 5, 7),
+                                       (64, 1024, 1032)])
+def test_cat_of_two_tensors(n, c_a, c_b, dtype):
+    """`cat` of two tensors (the skip concatenation of a U-Net) is bit-identical to torch.cat, whether the
+    streaming kernel takes the layout or not, and hands the gradient back in two slices."""
+    from pcengine_amd import backend
+    g = torch.Generator().manual_seed(n + c_a)
+    a = torch.randn(n, c_a, generator=g).to(dtype).to(DEV).requires_grad_(True)
+    b = torch.randn(n, c_b, generator=g).to(dtype).to(DEV).requires_grad_(True)
+    coords = torch.zeros((n, 4), dtype=torch.int32, device=DEV)
+    xa = pe.spTensor(a, coords, None, [0, 0, 0], [1, 1, 1])
+    xb = pe.spTensor(b, coords, None, [0, 0, 0], [1, 1, 1])
+    y = pe.cat([xa, xb])
+    want = torch.cat([a.detach(), b.detach()], dim=1)
+    assert y.feats.dtype == dtype and torch.equal(y.feats.detach(), want)
+    per = 8 if dtype == torch.float16 else 4
+    fits = c_a % per == 0 and c_b % per == 0 and (c_a + c_b) // per <= 256
+    assert (backend.concat_cols(a.detach(), b.detach()) is not None) == fits
+    go = torch.randn(n, c_a + c_b, generator=g).to(dtype).to(DEV)
+    y.feats.backward(go)
+    assert torch.equal(a.grad, go[:, :c_a]) and torch.equal(b.grad, go[:, c_a:])
+    z = pe.cat([xa, xb, xa])            # more than two inputs: torch's own concatenation
+    assert torch.equal(z.feats.detach(), torch.cat([want, a.detach()], dim=1))
