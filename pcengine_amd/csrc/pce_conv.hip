@@ -895,10 +895,21 @@ __device__ __forceinline__ void pipe_wait_barrier(int leave_in_flight, const u32
                                                   u32x4 &o1) {
   // loads complete in issue order: leaving the youngest ones in flight (the feature fragments and the
   // weight chunk requested one round ago) still guarantees that the chunk about to be used has landed
-  if (leave_in_flight >= 4)
+  if (leave_in_flight >= 8)
+    PCE_PIPE_WAIT_COPY(8);
+  else if (leave_in_flight >= 4)
     PCE_PIPE_WAIT_COPY(4);
   else
     PCE_PIPE_WAIT_COPY(0);
+}
+// two more fragments that the same wait has covered: volatile statements keep their order, so these copies
+// stay behind the wait of the pipe_wait_barrier in front of them
+__device__ __forceinline__ void pipe_copy_landed(const u32x4 &f0, const u32x4 &f1, u32x4 &o0, u32x4 &o1) {
+  asm volatile("v_mov_b32 %0, %8\n\tv_mov_b32 %1, %9\n\tv_mov_b32 %2, %10\n\tv_mov_b32 %3, %11\n\t"
+               "v_mov_b32 %4, %12\n\tv_mov_b32 %5, %13\n\tv_mov_b32 %6, %14\n\tv_mov_b32 %7, %15"
+               : "=&v"(o0.x), "=&v"(o0.y), "=&v"(o0.z), "=&v"(o0.w), "=&v"(o1.x), "=&v"(o1.y), "=&v"(o1.z), "=&v"(o1.w)
+               : "v"(f0.x), "v"(f0.y), "v"(f0.z), "v"(f0.w), "v"(f1.x), "v"(f1.y), "v"(f1.z), "v"(f1.w)
+               : "memory");
 }
 #undef PCE_PIPE_WAIT_COPY
 
@@ -1080,11 +1091,16 @@ __device__ __forceinline__ void step_mfma(f32x16 (&acc)[4], const half8 (&af)[2]
 // untracked loads, both two steps ahead, one barrier per step.  The neighbour rows of all offsets are
 // read once into LDS; an offset none of the tile's rows has a neighbour at is left out of the sequence,
 // and a wavefront skips the MFMAs of an offset none of its own 32 rows has.
+// SUB K chunks share a step (one wait, one barrier, 8 SUB MFMAs per wavefront): with one or two workgroups
+// per CU the barrier, the wait and the LDS latency in front of a step's first MFMA cost more than its
+// MFMAs, so input widths that are multiples of 64 take two chunks per step.
 #define OSP_MAX_KV 32
-__global__ void __launch_bounds__(256, 3) os_pipe_kernel(TileArgs a) {
+template <int SUB>
+__global__ void __launch_bounds__(256, SUB == 1 ? 3 : 2) os_pipe_kernel(TileArgs a) {
   constexpr int NB = PIPE_NB, NT = 128, KC = PIPE_KC;
-  constexpr int STAGE = (KC / 8) * NT;
-  constexpr int RING = PIPE_ST * STAGE;
+  constexpr int STAGE = (KC / 8) * NT;          // fragments of one chunk
+  constexpr int RSTAGE = SUB * STAGE;           // fragments of one ring stage
+  constexpr int RING = PIPE_ST * RSTAGE;
   constexpr int EPI = 4 * WaveLds<NB>::PIECES;
   __shared__ __attribute__((aligned(16))) half8 lds[RING > EPI ? RING : EPI];
   __shared__ int nbrs[OSP_MAX_KV][128];
@@ -1097,7 +1113,7 @@ __global__ void __launch_bounds__(256, 3) os_pipe_kernel(TileArgs a) {
   if (!xcd_item(a.items, a.slabs, true, &tile, &slab)) return;
   const int n0 = slab * NT;
   const half_t *A = (const half_t *)a.A;
-  const int kch = a.c_in / KC;
+  const int kch = a.c_in / (KC * SUB);   // steps per offset
   const long long row = tile * 128 + wave * 32 + l32;
   const int orow = row < a.n_rows ? (int)row : -1;
 
@@ -1122,7 +1138,7 @@ __global__ void __launch_bounds__(256, 3) os_pipe_kernel(TileArgs a) {
   // issue cursor (two steps ahead of the consume cursor): offset, chunk, LDS stage
   int ikp = active ? __ffs(active) - 1 : -1, it = 0, ist = 0;
   int ckp = ikp, ct = 0, cst = 0;
-  u32x4 raw[2][2];
+  u32x4 raw[2][SUB][2];
   const half8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
   int carow[2] = {-1, -1};   // the row whose fragments sit in raw[slot]
 #define OSP_ISSUE(SLOT_)                                                                                     \
@@ -1130,8 +1146,10 @@ __global__ void __launch_bounds__(256, 3) os_pipe_kernel(TileArgs a) {
     const half_t *Wk = (const half_t *)a.Wp + (long long)ikp * a.k8_total * a.n_pad * 8;                     \
     const int arow_i = nbrs[ikp][wave * 32 + l32];                                                           \
     carow[SLOT_] = arow_i;                                                                                   \
-    pipe_load_rows(raw[SLOT_], A, arow_i, a.c_in, it * KC, g);                                               \
-    pipe_issue_weights(Wk, it * KC, n0, a.n_pad, lds + ist * STAGE, wave, lane);                             \
+    _Pragma("unroll") for (int sub = 0; sub < SUB; ++sub) {                                                  \
+      pipe_load_rows(raw[SLOT_][sub], A, arow_i, a.c_in, (it * SUB + sub) * KC, g);                          \
+      pipe_issue_weights(Wk, (it * SUB + sub) * KC, n0, a.n_pad, lds + ist * RSTAGE + sub * STAGE, wave, lane); \
+    }                                                                                                        \
     ist = ist + 1 == PIPE_ST ? 0 : ist + 1;                                                                  \
     if (++it == kch) {                                                                                       \
       it = 0;                                                                                                \
@@ -1145,15 +1163,19 @@ __global__ void __launch_bounds__(256, 3) os_pipe_kernel(TileArgs a) {
 #define OSP_ROUND(R_, SLOT_)                                                                                 \
   {                                                                                                          \
     const int r = (R_);                                                                                      \
-    u32x4 landed[2];                                                                                         \
-    /* everything older than the loads of step r+1 (issued one step ago) has landed */                      \
-    pipe_wait_barrier(4 * (r + 1 < rounds), raw[SLOT_][0], raw[SLOT_][1], landed[0], landed[1]);             \
-    half8 af[2];                                                                                             \
+    u32x4 landed[SUB][2];                                                                                    \
+    /* everything older than the loads of step r+1 (issued one step ago, 4 SUB of them) has landed */       \
+    pipe_wait_barrier(4 * SUB * (r + 1 < rounds), raw[SLOT_][0][0], raw[SLOT_][0][1], landed[0][0], landed[0][1]); \
+    if (SUB == 2) pipe_copy_landed(raw[SLOT_][SUB - 1][0], raw[SLOT_][SUB - 1][1], landed[SUB - 1][0], landed[SUB - 1][1]); \
+    half8 af[SUB][2];                                                                                        \
     const int arow_c = carow[SLOT_];                                                                         \
-    _Pragma("unroll") for (int s2 = 0; s2 < 2; ++s2)                                                         \
-        af[s2] = arow_c >= 0 ? __builtin_bit_cast(half8, landed[s2]) : zero;                                 \
+    _Pragma("unroll") for (int sub = 0; sub < SUB; ++sub) _Pragma("unroll") for (int s2 = 0; s2 < 2; ++s2)   \
+        af[sub][s2] = arow_c >= 0 ? __builtin_bit_cast(half8, landed[sub][s2]) : zero;                       \
     if (r + 2 < rounds) OSP_ISSUE(SLOT_)                                                                     \
-    if ((wmask >> ckp) & 1u) step_mfma(acc, af, lds + cst * STAGE + g * NT + l32);                           \
+    if ((wmask >> ckp) & 1u) {                                                                               \
+      _Pragma("unroll") for (int sub = 0; sub < SUB; ++sub)                                                  \
+          step_mfma(acc, af[sub], lds + cst * RSTAGE + sub * STAGE + g * NT + l32);                          \
+    }                                                                                                        \
     cst = cst + 1 == PIPE_ST ? 0 : cst + 1;                                                                  \
     if (++ct == kch) {                                                                                       \
       ct = 0;                                                                                                \
@@ -1221,7 +1243,10 @@ static int launch_os_pipe(TileArgs a, long long tiles, hipStream_t s) {
   a.items = tiles * a.slabs;
   if (a.items >= (1ll << 31) - 8) PCE_FAIL(PCE_ECAPACITY, "tile count %lld exceeds the grid limit", tiles);
   const unsigned grid = (unsigned)(pce_div_up(a.items, PCE_XCDS) * PCE_XCDS);
-  hipLaunchKernelGGL(os_pipe_kernel, dim3(grid), dim3(256), 0, s, a);
+  if (a.c_in % (2 * PIPE_KC) == 0)
+    hipLaunchKernelGGL(os_pipe_kernel<2>, dim3(grid), dim3(256), 0, s, a);
+  else
+    hipLaunchKernelGGL(os_pipe_kernel<1>, dim3(grid), dim3(256), 0, s, a);
   PCE_LAUNCH_CHECK("os_pipe");
   return PCE_OK;
 }
