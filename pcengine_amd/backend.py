@@ -557,9 +557,9 @@ def concat_cols(a: torch.Tensor, b: torch.Tensor) -> Optional[torch.Tensor]:
     if c_a == 0 or c_b == 0 or c_a % per or c_b % per or (c_a + c_b) // per > 256:
         return None
     a, b = a.contiguous(), b.contiguous()
-    out = torch.empty((a.shape[0], c_a + c_b), dtype=a.dtype, device=a.device)
     if a.data_ptr() % 16 or b.data_ptr() % 16:
         return None
+    out = torch.empty((a.shape[0], c_a + c_b), dtype=a.dtype, device=a.device)
     _lib.check(_lib.load().pce_concat_cols(a.data_ptr(), c_a, b.data_ptr(), c_b, out.data_ptr(), _dtype_code(a), a.shape[0],
                                            _stream(a.device)))
     return out
