@@ -316,3 +316,26 @@ def test_deferred_scatter_without_buffer_needs_one_pair_per_row():
     assert rc == _lib.PCE_OK
     torch.cuda.synchronize()
     assert torch.equal(direct, back)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("ks,c_in,c_out", [((5, 5, 5), 32, 32), ((5, 5, 5), 64, 128), ((5, 3, 1), 16, 24), ((1, 5, 5), 128, 96)])
+def test_large_and_anisotropic_kernels_forward_and_backward(ks, c_in, c_out, dtype):
+    """Kernel volumes beyond what travels in the kernel arguments (5x5x5 = 125 offsets) and anisotropic
+    kernels, every dataflow, forward and both gradients, against the oracle (whose 5-wide offsets follow the
+    reference's rule, backend/hash.cuh:147-149)."""
+    coords = synth.random_cloud(seed=48, n=4000, extent=15, batches=2)
+    fd, wd, ref_map, want = _case(coords, ks, (1, 1, 1), (0, 0, 0), c_in, c_out, dtype, seed=11)
+    km = gpu_map(coords, ks, want_csr=True, want_nbr_in=True)
+    assert km.M == ref_map.M and torch.equal(km.imap.cpu(), torch.as_tensor(ref_map.imap)) and torch.equal(km.omap.cpu(), torch.as_tensor(ref_map.omap))
+    packed = backend.pack_weights(wd)
+    for flow in FLOWS:
+        out = backend.conv_forward(fd, wd, km, flow, packed=packed)
+        assert orc.rel_l2(out.double().cpu().numpy(), want) <= TOL[dtype], (ks, flow)
+    rng = np.random.default_rng(48)
+    g = rounded(rng.standard_normal((len(coords), c_out)), dtype)
+    gd = torch.as_tensor(g, device=DEV).to(dtype)
+    gf, gw = backend.conv_backward(fd, wd, km, gd)
+    want_f, want_w = orc.conv_backward(fd.double().cpu().numpy(), wd.double().cpu().numpy(), ref_map, ks, g)
+    assert orc.rel_l2(gf.double().cpu().numpy(), want_f) <= TOL[dtype]
+    assert orc.rel_l2(gw.double().cpu().numpy(), want_w) <= TOL[dtype]
