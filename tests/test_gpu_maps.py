@@ -254,3 +254,18 @@ def test_voxelize_edge_cases():
     far = torch.tensor([[0.0, 0.0, 0.0], [1.0e9, 1000.0, 1000.0], [0.0, 0.0, 0.0]], dtype=torch.float64, device=DEV)
     coords, inverse, _ = backend.voxelize(far, 1.0, return_inverse=True)     # a huge but representable box
     assert coords.cpu().tolist() == [[0, 0, 0, 0], [0, 1000000000, 1000, 1000]] and inverse.cpu().tolist() == [0, 1, 0]
+
+
+@pytest.mark.parametrize("shift", [31950, -31950])
+def test_submanifold_map_at_the_edge_of_the_coordinate_range(shift):
+    """Keys pack 16 bits per coordinate and 16 bits of batch index: clouds pushed against |c| < 32000 in both
+    directions, with batch indices up to 32767, build the same maps as the oracle."""
+    base = synth.random_cloud(seed=33, n=3000, extent=40, batches=3)
+    coords = base.copy()
+    coords[:, 1:] = coords[:, 1:] + (shift if shift > 0 else shift - 40)
+    coords[:, 0] = np.array([0, 9, 32767], np.int32)[base[:, 0]]
+    order = np.lexsort((coords[:, 3], coords[:, 2], coords[:, 1], coords[:, 0]))
+    coords = np.ascontiguousarray(coords[order])
+    assert np.abs(coords[:, 1:]).max() < 32000
+    for ks in ((3, 3, 3), (5, 5, 5), (1, 3, 3)):
+        assert_map_equal(gpu_map(coords, ks, want_csr=True), orc.kernel_map(coords, ks), csr=True)
