@@ -339,3 +339,25 @@ def test_large_and_anisotropic_kernels_forward_and_backward(ks, c_in, c_out, dty
     want_f, want_w = orc.conv_backward(fd.double().cpu().numpy(), wd.double().cpu().numpy(), ref_map, ks, g)
     assert orc.rel_l2(gf.double().cpu().numpy(), want_f) <= TOL[dtype]
     assert orc.rel_l2(gw.double().cpu().numpy(), want_w) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("c_in,c_out", [(32, 32), (128, 128), (5, 7)])
+def test_layer_without_pairs_and_single_voxel(c_in, c_out, dtype):
+    """Isolated voxels (no neighbour within the kernel) leave only the centre term; a cloud of one voxel is the
+    smallest tensor there is.  Forward through every dataflow and both gradients."""
+    grid = np.stack(np.meshgrid(np.arange(0, 40, 3), np.arange(0, 40, 3), np.arange(0, 12, 3), indexing="ij"), -1).reshape(-1, 3)
+    for coords in (np.concatenate([np.zeros((len(grid), 1), np.int64), grid], 1).astype(np.int32),
+                   np.array([[0, 5, 6, 7]], np.int32)):
+        fd, wd, ref_map, want = _case(coords, (3, 3, 3), (1, 1, 1), (0, 0, 0), c_in, c_out, dtype, seed=12)
+        km = gpu_map(coords, (3, 3, 3), want_csr=True, want_nbr_in=True)
+        assert km.M == 0 and ref_map.M == 0
+        packed = backend.pack_weights(wd)
+        for flow in FLOWS:
+            out = backend.conv_forward(fd, wd, km, flow, packed=packed)
+            assert orc.rel_l2(out.double().cpu().numpy(), want) <= TOL[dtype], flow
+        g = rounded(np.random.default_rng(3).standard_normal((len(coords), c_out)), dtype)
+        gf, gw = backend.conv_backward(fd, wd, km, torch.as_tensor(g, device=DEV).to(dtype))
+        want_f, want_w = orc.conv_backward(fd.double().cpu().numpy(), wd.double().cpu().numpy(), ref_map, (3, 3, 3), g)
+        assert orc.rel_l2(gf.double().cpu().numpy(), want_f) <= TOL[dtype]
+        assert orc.rel_l2(gw.double().cpu().numpy(), want_w) <= TOL[dtype]
