@@ -135,3 +135,52 @@ def test_dense_layer_kernel_gradient(n, c_in, c_out, dtype):
         backend.dense_wgrad(a, b.to(torch.float64))
     with pytest.raises(ValueError):
         backend.dense_wgrad(a, torch.zeros(n + 1, c_out, dtype=dtype, device=DEV))
+
+
+def test_unet_fused_training_path_matches_the_composition_of_torch_modules():
+    """The training path of the network (norm + residual + ReLU in the norm's own passes, the concatenation
+    kernel, transposed layers that store once) against the same network with torch's BatchNorm1d, add, relu and
+    cat around this package's convolutions: output and every parameter gradient, fp32.
+    The two forwards agree to rounding (1e-6), but a single activation within that distance of zero takes the
+    other branch of its ReLU in one of them, and one changed mask element moves a gradient tensor of 4*10^4
+    elements by 1/sqrt(4*10^4) = 0.5 % of its norm: the gradient bar is 1e-2 (a wrong mask, sign or missing
+    term moves it by order one), the output bar 1e-5."""
+    import copy
+    from pcengine_amd import batchnorm, utils
+    coords = synth.random_cloud(seed=74, n=5000, extent=60)
+    f = synth.features(12, len(coords), 4).astype(np.float32)
+    torch.manual_seed(5)
+    model = nets.SparseResUNet(4, 6, stem=8, enc=(8, 16, 16, 32), dec=(32, 16, 16, 8)).to(DEV).train()
+    twin = copy.deepcopy(model)
+    weight = torch.randn(len(coords), 6, device=DEV)
+
+    def run(net):
+        x = pe.spTensor(torch.as_tensor(f, device=DEV), torch.as_tensor(coords, device=DEV), None, [0, 0, 0],
+                        coords[:, 1:].max(0).tolist())
+        out = net(x).feats
+        (out * weight).sum().backward()
+        return out.detach()
+
+    out_a = run(model)
+
+    def torch_features(self, x, residual=None, act=None):
+        y = torch.nn.BatchNorm1d.forward(self, x)
+        if residual is not None:
+            y = y + residual
+        return torch.relu(y) if act == "relu" else y
+    old_features, old_cat = batchnorm.BatchNorm._features, nets.cat
+    batchnorm.BatchNorm._features = torch_features
+    nets.cat = lambda inputs: inputs[0]._like(torch.cat([t.feats for t in inputs], dim=1))
+    try:
+        out_b = run(twin)
+    finally:
+        batchnorm.BatchNorm._features, nets.cat = old_features, old_cat
+    P = lambda t: t.double().cpu().numpy()
+    assert orc.rel_l2(P(out_a), P(out_b)) <= 1e-5
+    worst = 0.0
+    for (name, p), q in zip(model.named_parameters(), twin.parameters()):
+        assert p.grad is not None and q.grad is not None, name
+        worst = max(worst, orc.rel_l2(P(p.grad), P(q.grad)))
+        assert orc.rel_l2(P(p.grad), P(q.grad)) <= 1e-2, (name, worst)
+    for a, b in zip(model.buffers(), twin.buffers()):
+        assert orc.rel_l2(P(a), P(b)) <= 1e-5
