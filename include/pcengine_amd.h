@@ -345,7 +345,10 @@ int pce_conv_fwd_dense(const void *in_feats, const void *weight, const void *wei
  * grad_out[omap[p]], plus in_feats^T * grad_out for the centre offset when mid >= 0.  grad_w is
  * fp32 [kv, c_in, c_out] whatever `dtype` the features have; the call zeroes it first.  Pair lists
  * as for pce_conv_fwd_fod (swap imap / omap for a transposed layer; n_in rows of in_feats, n_out
- * rows of grad_out). */
+ * rows of grad_out).  Products are accumulated in fp32 on the matrix cores (fp16 tensors on the fp16
+ * MFMA, fp32 tensors on the fp32 MFMA) and runs of pair tiles are combined with fp32 atomic adds, so
+ * the last bits of grad_w depend on the order in which workgroups finish (1e-7 relative from run
+ * to run); a 1x1 layer is the call with kv = 1, mid = 0, qsum = 0 and no pair lists. */
 int pce_conv_wgrad(const void *in_feats, const void *grad_out, int32_t dtype, int64_t n_in,
                    int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv, int32_t mid,
                    const int32_t *imap_dev, const int32_t *omap_dev, const int32_t *kpos_dev,
