@@ -45,11 +45,11 @@ class ConvBN(nn.Module):
 
     def forward(self, x: spTensor, residual: spTensor = None, relu_after_residual: bool = False) -> spTensor:
         """With the norm folded away, bias, the optional residual and the ReLU run inside the conv kernels."""
+        act = self.relu.as_epilogue() if self.relu is not None else ("relu" if relu_after_residual else None)
         if self.bn is None:
-            act = "relu" if (self.relu is not None or relu_after_residual) else None
             return self.conv(x, act=act, residual=residual)
         # training form: the residual sum and the ReLU ride on the norm's affine pass
-        return self.bn(self.conv(x), residual=residual, act="relu" if (self.relu is not None or relu_after_residual) else None)
+        return self.bn(self.conv(x), residual=residual, act=act)
 
 
 class ResidualBlock(nn.Module):
