@@ -116,6 +116,30 @@ def test_module_construction_and_errors():
         pe.conv3d(4, 8, dataflow="magic")
 
 
+def test_sparse_tensor_container_and_activations_on_cpu():
+    """Fields, aliases, in-place movement and shared caches of spTensor (script/sptensor.py:4-91); ReLU and
+    LeakyReLU act on the features only (script/activation.py:6-15) and name their fused-epilogue form."""
+    feats = torch.tensor([[-1.0, 2.0], [3.0, -4.0], [0.0, 0.5]])
+    coords = torch.tensor([[0, 1, 2, 3], [0, 4, 5, 6], [1, 7, 8, 9]], dtype=torch.int32)
+    x = pe.spTensor(feats, coords)
+    assert x.coords_min == [0, 0, 0] and x.coords_max == [7, 8, 9] and x.init_tag == ["end"] and x.batchsize == 1
+    assert x.F is x.feats and x.C is x.coords and len(x) == 3 and "N=3" in repr(x)
+    x.F = feats * 2
+    assert torch.equal(x.feats, feats * 2)
+    x.F = feats
+    y = pe.ReLU()(x)
+    assert torch.equal(y.feats, feats.clamp(min=0)) and y.coords is x.coords and y.kmaps is x.kmaps and y.cbook is x.cbook
+    z = pe.LeakyReLU(0.25)(x)
+    assert torch.equal(z.feats, torch.where(feats > 0, feats, feats * 0.25))
+    assert pe.ReLU().as_epilogue() == "relu" and pe.LeakyReLU(0.25).as_epilogue() == ("leaky_relu", 0.25)
+    assert torch.equal((x + y).feats, feats + feats.clamp(min=0)) and (x + y).kmaps is x.kmaps
+    assert x.detach() is x and x.cpu() is x and x.to("cpu") is x
+    x.build_buffer({"kernel": [3, 2], "in": [4, 16], "out": [8, 32]}, "cpu")
+    assert x.buffer.numel() == (16 + 32) * 3 * 16 and x.buffer.dtype == torch.float32
+    inplace = pe.ReLU(True)(x)
+    assert inplace.feats.data_ptr() == x.feats.data_ptr() and float(x.feats.min()) == 0.0
+
+
 def test_no_cpu_compute_path():
     x = pe.spTensor(torch.zeros(3, 4), torch.zeros(3, 4, dtype=torch.int32), None, [0, 0, 0], [0, 0, 0])
     with pytest.raises(RuntimeError, match="no CPU compute path"):
