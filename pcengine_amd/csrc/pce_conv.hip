@@ -66,6 +66,8 @@ struct TileArgs {
   int act;
   float slope;
   int act_alone_only;               // apply the activation only to rows without partial rows (ocsr tells)
+  void *out_alt;                    // routed pair tiles: destination d < n_split is row d of `out` (a finished output
+  int n_split;                      // row, takes the epilogue), d >= n_split is row d - n_split of `out_alt`
   int kpos_h[MAX_KV_ARGS + 1];
   int qkpos_h[MAX_KV_ARGS + 1];
 };
@@ -447,16 +449,19 @@ __device__ __forceinline__ void add_partials_slow(float (&V)[NB][2][8], int e0, 
 }
 
 // ---- fused epilogue: out = act(acc + bias + residual) -------------------------------------------
+// Written without branches: with `act` a kernel argument the compiler turned the three-way form into scalar
+// compares, jumps and a reload of the slope around every element of an unrolled epilogue.  The two
+// coefficients depend on `act` alone and are hoisted out of the loops.
 __device__ __forceinline__ float act_apply(float v, int act, float slope) {
-  if (act == PCE_ACT_RELU) return v > 0.f ? v : 0.f;
-  if (act == PCE_ACT_LEAKY_RELU) return v > 0.f ? v : v * slope;
-  return v;
+  const float mul = act == PCE_ACT_LEAKY_RELU ? slope : 1.f;   // what a non-positive value is multiplied by ...
+  const unsigned keep = act == PCE_ACT_RELU ? 0u : ~0u;        // ... and whether the product survives
+  const float t = __uint_as_float(__float_as_uint(v * mul) & keep);
+  return v > 0.f ? v : t;                                      // no activation: t == v
 }
 // derivative of the activation where its output is `out` (ReLU and LeakyReLU with a positive slope keep the sign)
 __device__ __forceinline__ float act_slope_at(float out, int act, float slope) {
-  if (act == PCE_ACT_RELU) return out > 0.f ? 1.f : 0.f;
-  if (act == PCE_ACT_LEAKY_RELU) return out > 0.f ? 1.f : slope;
-  return 1.f;
+  const float neg = act == PCE_ACT_RELU ? 0.f : (act == PCE_ACT_LEAKY_RELU ? slope : 1.f);
+  return out > 0.f ? 1.f : neg;
 }
 
 // eight consecutive elements of a row of T as floats; VEC: the address is 16-byte aligned
@@ -524,7 +529,7 @@ __device__ __forceinline__ void store_row_pieces_slow(const float (&V)[NB][2][8]
 // Finished rows -> memory through the wavefront's LDS region: the lane that owns (row, 8 columns)
 // writes its pieces; then 16 bytes per lane are read back along the rows, so that NT*sizeof(TO)/16
 // consecutive lanes store one full row segment (whole 128-byte lines at 64 fp16 channels).
-template <typename TO, int NB, int ROWS = (sizeof(TO) == 2 ? 32 : 16)>
+template <typename TO, int NB, int ROWS = (sizeof(TO) == 2 ? 32 : 16), bool SPLIT = false>
 __device__ __forceinline__ void store_rows_via_lds(const float (&V)[NB][2][8], void *region, TO *out, int orow,
                                                    const TileArgs &a, int n0, int lane, int l32, int g) {
   constexpr int NT = NB * 32;
@@ -569,7 +574,12 @@ __device__ __forceinline__ void store_rows_via_lds(const float (&V)[NB][2][8], v
       int dst = __shfl(orow, pass * ROWS + lr, PCE_WAVE);
       int col = n0 + ch * EPP;
       OV y = R[lr * LDP + ch];
-      if (dst >= 0 && col < a.c_out) *reinterpret_cast<OV *>(out + (long long)dst * a.c_out + col) = y;
+      TO *base = out;
+      if (SPLIT && dst >= a.n_split) {
+        base = (TO *)a.out_alt;
+        dst -= a.n_split;
+      }
+      if (dst >= 0 && col < a.c_out) *reinterpret_cast<OV *>(base + (long long)dst * a.c_out + col) = y;
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -1046,10 +1056,18 @@ __global__ void __launch_bounds__(256, 4) pipe_gemm_kernel(TileArgs a, TileArgs 
   } else if (a.bias || a.res || a.act) {
     bool with_act = a.act != PCE_ACT_NONE;
     if (with_act && a.act_alone_only) with_act = orow >= 0 && a.ocsr[orow] == a.ocsr[orow + 1];
-    epilogue_row_pieces<half_t, NB, true>(V, a, orow, n0, g, with_act);
+    int erow = orow;
+    if (PMODE == MODE_FOD_BUF && a.out_alt && orow >= a.n_split) {  // a partial row: its epilogue comes with the row sum
+      erow = -1;
+      with_act = false;
+    }
+    epilogue_row_pieces<half_t, NB, true>(V, a, erow, n0, g, with_act);
   }
   half_t *out = (half_t *)((PMODE == PIPE_BOTH && dense) ? c.out : a.out);
-  store_rows_via_lds<half_t, NB>(V, lds + wave * WaveLds<NB>::PIECES, out, orow, a, n0, lane, l32, g);
+  if (PMODE == MODE_FOD_BUF && a.out_alt)
+    store_rows_via_lds<half_t, NB, 32, true>(V, lds + wave * WaveLds<NB>::PIECES, out, orow, a, n0, lane, l32, g);
+  else
+    store_rows_via_lds<half_t, NB>(V, lds + wave * WaveLds<NB>::PIECES, out, orow, a, n0, lane, l32, g);
 }
 
 // The eight weight fragments of a step are requested before its first MFMA, and every MFMA waits only for
@@ -1396,13 +1414,14 @@ template <typename T, int VEC>
 __global__ void __launch_bounds__(256) rowsum_kernel(const T *__restrict__ buf, long long n_out, int c_out, int G,
                                                      const int *__restrict__ csr, T *__restrict__ out,
                                                      const T *__restrict__ bias, const T *__restrict__ res, int act,
-                                                     float slope) {
+                                                     float slope, int skip_single) {
   typedef typename VecOf<T, VEC>::type V;
   int rows_per_block = 256 / G;
   long long row = (long long)blockIdx.x * rows_per_block + threadIdx.x / G;
   int sub = threadIdx.x % G;
   if (row >= n_out) return;
   int e0 = csr[row], e1 = csr[row + 1];
+  if (skip_single && e1 - e0 == 1) return;  // the row's only pair has stored it already
   int row_vecs = c_out / VEC;
   for (int v = sub; v < row_vecs; v += G) {
     float acc[VEC];
@@ -1869,10 +1888,11 @@ extern "C" int pce_conv_fwd_gms(const void *in, const void *w, const void *wp, v
 template <typename T>
 static int fds_impl(const void *in, const void *w, const void *wp, void *out, int64_t n_out, int c_in, int c_out, int kv,
                     int mid, const int *imap, const int *omap, const int *oslot, const int *kpos, const int *qkpos,
-                    const int32_t *kpos_host, const int32_t *qkpos_host, const int *ocsr, int64_t n_pairs, int64_t qsum,
-                    T *buffer, const Epi &e, hipStream_t s) {
+                    const int32_t *kpos_host, const int32_t *qkpos_host, const int *ocsr, const int *odst, int64_t n_pairs,
+                    int64_t qsum, T *buffer, const Epi &e, hipStream_t s) {
   constexpr int VEC = sizeof(T) == 2 ? 8 : 4;
   int rc;
+  int skip_single = 0;
   if (!buffer && qsum > 0) {
     // Every output row has exactly one pair (a transposed layer whose kernel equals its stride: each fine
     // voxel has one parent): a pair's product is its output row, stored once with the epilogue, no partial rows.
@@ -1915,7 +1935,28 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
       return PCE_OK;
     }
   }
-  if (qsum > 0 && stage_on(1)) {
+  if (mid < 0 && odst && buffer && qsum > 0 && stage_on(1) && stage_on(2) && stage_on(5) && n_out + n_pairs < (1ll << 31)) {
+    // Routed pair tiles (a layer without centre offset): the only pair of an output row stores the finished row
+    // with the epilogue, the pairs of the other rows store partial rows; the row sum then visits only rows with
+    // two pairs or more.  Taken by the pipelined kernel's shapes; the others ignore the routing.
+    TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
+    set_out<T>(&a, out, false);
+    set_host_pos(&a, kpos_host, qkpos_host);
+    a.imap = imap;
+    a.oslot = odst;
+    a.kpos = kpos;
+    a.qkpos = qkpos;
+    a.mode = MODE_FOD_BUF;
+    a.epi = EPI_ROWS;
+    a.out_alt = buffer;
+    a.n_split = (int)n_out;
+    set_epi(&a, e);
+    if (pipe_gemm_ok(a, sizeof(T)) && aligned16(buffer)) {
+      if ((rc = launch_pipe_gemm(a, qsum / PCE_QUANTUM, s))) return rc;
+      skip_single = 1;
+    }
+  }
+  if (qsum > 0 && stage_on(1) && !skip_single) {
     TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
     set_out<T>(&a, buffer, false);
     set_host_pos(&a, kpos_host, qkpos_host);
@@ -1991,15 +2032,38 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
     if (G > 64) G = 64;
     hipLaunchKernelGGL((rowsum_kernel<T, VEC>), dim3((unsigned)pce_div_up(n_out, 256 / G)), dim3(256), 0, s,
                        (const T *)buffer, (long long)n_out, c_out, G, ocsr, (T *)out, (const T *)e.bias, (const T *)e.res,
-                       e.act, e.slope);
+                       e.act, e.slope, skip_single);
   } else {
     int G = pow2_at_least(c_out);
     if (G > 64) G = 64;
     hipLaunchKernelGGL((rowsum_kernel<T, 1>), dim3((unsigned)pce_div_up(n_out, 256 / G)), dim3(256), 0, s,
                        (const T *)buffer, (long long)n_out, c_out, G, ocsr, (T *)out, (const T *)e.bias, (const T *)e.res,
-                       e.act, e.slope);
+                       e.act, e.slope, skip_single);
   }
   PCE_LAUNCH_CHECK("rowsum");
+  return PCE_OK;
+}
+
+// destination of every pair of a layer without centre offset: the output row itself where the pair is the
+// row's only one, else n_out + the pair's partial-row slot
+__global__ void __launch_bounds__(256) pair_route_kernel(const int *__restrict__ omap, const int *__restrict__ oslot,
+                                                         const int *__restrict__ ocsr, long long n_pairs, int n_out,
+                                                         int *__restrict__ odst) {
+  long long p = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= n_pairs) return;
+  int o = omap[p];
+  odst[p] = (ocsr[o + 1] - ocsr[o] == 1) ? o : n_out + oslot[p];
+}
+
+extern "C" int pce_pair_route(const int32_t *omap, const int32_t *oslot, const int32_t *ocsr, int64_t n_pairs, int64_t n_out,
+                              int32_t *odst, pce_stream_t stream) {
+  if (n_pairs < 0 || n_out < 0) PCE_FAIL(PCE_EINVAL, "pce_pair_route: negative count");
+  if (n_pairs == 0) return PCE_OK;
+  if (!omap || !oslot || !ocsr || !odst) PCE_FAIL(PCE_EINVAL, "pce_pair_route: null pointer");
+  if (n_out + n_pairs >= (1ll << 31)) PCE_FAIL(PCE_ECAPACITY, "pce_pair_route: n_out + n_pairs = %lld exceeds int32", (long long)(n_out + n_pairs));
+  hipLaunchKernelGGL(pair_route_kernel, dim3((unsigned)pce_div_up(n_pairs, 256)), dim3(256), 0, (hipStream_t)stream, omap, oslot,
+                     ocsr, (long long)n_pairs, (int)n_out, odst);
+  PCE_LAUNCH_CHECK("pair_route");
   return PCE_OK;
 }
 
@@ -2007,7 +2071,7 @@ extern "C" int pce_conv_fwd_fds(const void *in, const void *w, const void *wp, v
                                 int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv, int32_t mid, const int32_t *imap,
                                 const int32_t *omap, const int32_t *oslot, const int32_t *kpos, const int32_t *qkpos,
                                 const int32_t *kpos_host, const int32_t *qkpos_host, const int32_t *ocsr,
-                                int64_t n_pairs, int64_t qsum, void *buffer, int64_t buffer_elems,
+                                const int32_t *odst, int64_t n_pairs, int64_t qsum, void *buffer, int64_t buffer_elems,
                                 const pce_epilogue_t *epilogue, pce_stream_t stream) {
   int rc = check_common("pce_conv_fwd_fds", in, w, out, dtype, n_in, n_out, c_in, c_out, kv, mid);
   if (rc || (rc = check_qsum("pce_conv_fwd_fds", qsum))) return rc;
@@ -2024,8 +2088,8 @@ extern "C" int pce_conv_fwd_fds(const void *in, const void *w, const void *wp, v
   }
   hipStream_t s = (hipStream_t)stream;
   if (dtype == PCE_F16)
-    return fds_impl<half_t>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, omap, oslot, kpos, qkpos, kpos_host, qkpos_host, ocsr, n_pairs, qsum, (half_t *)buffer, e, s);
-  return fds_impl<float>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, omap, oslot, kpos, qkpos, kpos_host, qkpos_host, ocsr, n_pairs, qsum, (float *)buffer, e, s);
+    return fds_impl<half_t>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, omap, oslot, kpos, qkpos, kpos_host, qkpos_host, ocsr, odst, n_pairs, qsum, (half_t *)buffer, e, s);
+  return fds_impl<float>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, omap, oslot, kpos, qkpos, kpos_host, qkpos_host, ocsr, odst, n_pairs, qsum, (float *)buffer, e, s);
 }
 
 template <typename T>

@@ -298,7 +298,7 @@ def test_deferred_scatter_without_buffer_needs_one_pair_per_row():
     def call(mid, n_pairs):
         return lib.pce_conv_fwd_fds(fd.data_ptr(), wd.data_ptr(), None, out.data_ptr(), _lib.PCE_F16, km.n_in, km.n_out, 32, 32,
                                     km.kv, mid, km.imap.data_ptr(), km.omap.data_ptr(), km.oslot.data_ptr(), km.kpos.data_ptr(),
-                                    km.qkpos.data_ptr(), None, None, km.ocsr.data_ptr(), n_pairs, km.qsum, None, 0, None, None)
+                                    km.qkpos.data_ptr(), None, None, km.ocsr.data_ptr(), None, n_pairs, km.qsum, None, 0, None, None)
     assert call(13, km.M) == _lib.PCE_EINVAL          # centre offset present
     assert call(-1, km.M) == _lib.PCE_EINVAL          # pairs != output rows
     # the transposed 2x2x2 stride-2 layer qualifies: same result with and without the caller's buffer
@@ -311,11 +311,58 @@ def test_deferred_scatter_without_buffer_needs_one_pair_per_row():
     back = torch.empty((km2.n_in, 32), dtype=torch.float16, device=DEV)
     rc = lib.pce_conv_fwd_fds(down.data_ptr(), wt.data_ptr(), backend.pack_weights(wt).data_ptr(), back.data_ptr(), _lib.PCE_F16,
                               km2.n_out, km2.n_in, 48, 32, 8, -1, km2.omap.data_ptr(), km2.imap.data_ptr(), km2.islot.data_ptr(),
-                              km2.kpos.data_ptr(), km2.qkpos.data_ptr(), None, None, km2.icsr.data_ptr(), km2.M, km2.qsum,
+                              km2.kpos.data_ptr(), km2.qkpos.data_ptr(), None, None, km2.icsr.data_ptr(), None, km2.M, km2.qsum,
                               buf.data_ptr(), buf.numel(), None, None)
     assert rc == _lib.PCE_OK
     torch.cuda.synchronize()
     assert torch.equal(direct, back)
+
+
+@pytest.mark.parametrize("cloud", ["surface", "random"])
+@pytest.mark.parametrize("c_in,c_out", [(64, 128), (128, 256), (96, 104), (64, 64)])
+def test_strided_layer_routes_single_pair_rows(cloud, c_in, c_out):
+    """A k2s2 layer in the deferred-scatter dataflow: the only pair of an output row stores the finished row,
+    the other rows go through partial rows and the row sum.  Without an epilogue the result equals the unrouted
+    one bit for bit (a single partial row is rounded to fp16 once either way); with one, both meet the fp16 bar.
+    (64, 64) is a shape the routed kernel does not take: the routing array is ignored."""
+    from pcengine_amd import _lib
+    lib = _lib.load()
+    if cloud == "surface":
+        coords = synth.sphere_plane_cloud(seed=7, n_sphere=9000, n_plane=3000)       # nearly every coarse voxel has one child
+    else:
+        coords = synth.random_cloud(seed=48, n=9000, extent=20, batches=2)
+    ks = (2, 2, 2)
+    fd, wd, ref_map, want = _case(coords, ks, ks, (0, 0, 0), c_in, c_out, torch.float16, seed=6)
+    km = gpu_map(coords, ks, ks, want_csr=True)
+    pk = backend.pack_weights(wd)
+    # the routing array against its definition
+    odst = backend.pair_route(km).cpu().numpy()
+    ocsr, omap, oslot = km.ocsr.cpu().numpy(), km.omap.cpu().numpy()[:km.M], km.oslot.cpu().numpy()[:km.M]
+    cnt = np.diff(ocsr)
+    assert np.array_equal(odst[:km.M], np.where(cnt[omap] == 1, omap, km.n_out + oslot))
+    singles = int((cnt == 1).sum())
+    assert 0 < singles < km.n_out or cloud == "surface"
+    plain = backend.conv_forward(fd, wd, km, DATAFLOW_FDS, packed=pk, route_single_pairs=False)
+    routed = backend.conv_forward(fd, wd, km, DATAFLOW_FDS, packed=pk)
+    assert torch.equal(plain, routed)
+    assert orc.rel_l2(routed.double().cpu().numpy(), want) <= 1e-3
+    # a second call on the cached routing, into a poisoned output and buffer
+    out = torch.full((km.n_out, c_out), float("nan"), dtype=torch.float16, device=DEV)
+    buf = torch.full((km.M * c_out,), float("nan"), dtype=torch.float16, device=DEV)
+    again = backend.conv_forward(fd, wd, km, DATAFLOW_FDS, packed=pk, out=out, buffer=buf)
+    assert torch.equal(again, routed)
+    rng = np.random.default_rng(48)
+    bias, res = rng.standard_normal(c_out) * 0.5, rng.standard_normal((km.n_out, c_out))
+    bd, rd = torch.as_tensor(bias, device=DEV).half(), torch.as_tensor(res, device=DEV).half()
+    for b, r, act in [(bd, rd, "relu"), (bd, None, None), (None, rd, ("leaky_relu", 0.1)), (None, None, "relu")]:
+        got = backend.conv_forward(fd, wd, km, DATAFLOW_FDS, packed=pk, bias=b, residual=r, act=act)
+        ref = want + (rounded(bias, torch.float16) if b is not None else 0) + (rounded(res, torch.float16) if r is not None else 0)
+        ref = _act_np(ref, act)
+        assert orc.rel_l2(got.double().cpu().numpy(), ref) <= 1e-3, act
+    # argument checks of the routing entry point
+    assert lib.pce_pair_route(None, None, None, 5, 5, None, None) == _lib.PCE_EINVAL
+    assert lib.pce_pair_route(km.omap.data_ptr(), km.oslot.data_ptr(), km.ocsr.data_ptr(), 1 << 30, 1 << 30, 1, None) == _lib.PCE_ECAPACITY
+    assert lib.pce_pair_route(None, None, None, 0, 5, None, None) == _lib.PCE_OK
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])

@@ -49,7 +49,7 @@ def test_argument_validation_needs_no_gpu():
     assert fod(10, 12, 128, 1 << 20) == _lib.PCE_EINVAL        # a centre offset needs n_in == n_out
     assert fod(10, 10, 128, 16) == _lib.PCE_EWORKSPACE
     assert lib.pce_conv_fwd_gms(one, one, None, one, 0, 10, 10, 4, 4, 27, 13, one, one, one, one, one, one, 128, one, 10, None, None) == _lib.PCE_EWORKSPACE
-    assert lib.pce_conv_fwd_fds(one, one, None, one, 0, 10, 10, 4, 4, 27, 13, one, one, one, one, one, None, None, one, 100, 128, one, 10, None, None) == _lib.PCE_EWORKSPACE
+    assert lib.pce_conv_fwd_fds(one, one, None, one, 0, 10, 10, 4, 4, 27, 13, one, one, one, one, one, None, None, one, None, 100, 128, one, 10, None, None) == _lib.PCE_EWORKSPACE
     assert lib.pce_conv_fwd_os(one, one, None, one, 7, 10, 10, 4, 4, 27, one, None, None) == _lib.PCE_EINVAL      # dtype
     epi = _lib.Epilogue()
     epi.act = 9
