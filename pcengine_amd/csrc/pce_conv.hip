@@ -452,12 +452,23 @@ __device__ __forceinline__ void add_partials_slow(float (&V)[NB][2][8], int e0, 
 // Written without branches: with `act` a kernel argument the compiler turned the three-way form into scalar
 // compares, jumps and a reload of the slope around every element of an unrolled epilogue.  The two
 // coefficients depend on `act` alone and are hoisted out of the loops.
-__device__ __forceinline__ float act_apply(float v, int act, float slope) {
-  const float mul = act == PCE_ACT_LEAKY_RELU ? slope : 1.f;   // what a non-positive value is multiplied by ...
-  const unsigned keep = act == PCE_ACT_RELU ? 0u : ~0u;        // ... and whether the product survives
-  const float t = __uint_as_float(__float_as_uint(v * mul) & keep);
-  return v > 0.f ? v : t;                                      // no activation: t == v
+struct ActK {
+  float mul;      // what a non-positive value is multiplied by ...
+  unsigned keep;  // ... and whether the product survives
+};
+// `on` may differ from lane to lane (rows that get their activation in a later pass): it goes into the
+// coefficients, not into a test around every element
+__device__ __forceinline__ ActK act_coeffs(int act, float slope, bool on) {
+  ActK k;
+  k.mul = (on && act == PCE_ACT_LEAKY_RELU) ? slope : 1.f;
+  k.keep = (on && act == PCE_ACT_RELU) ? 0u : ~0u;
+  return k;
 }
+__device__ __forceinline__ float act_apply(float v, const ActK &k) {
+  const float t = __uint_as_float(__float_as_uint(v * k.mul) & k.keep);
+  return v > 0.f ? v : t;  // no activation: t == v
+}
+__device__ __forceinline__ float act_apply(float v, int act, float slope) { return act_apply(v, act_coeffs(act, slope, true)); }
 // derivative of the activation where its output is `out` (ReLU and LeakyReLU with a positive slope keep the sign)
 __device__ __forceinline__ float act_slope_at(float out, int act, float slope) {
   const float neg = act == PCE_ACT_RELU ? 0.f : (act == PCE_ACT_LEAKY_RELU ? slope : 1.f);
@@ -487,7 +498,92 @@ __device__ __forceinline__ void add8(float (&v)[8], const T *p, int valid) {
   }
 }
 
-// on the row pieces of the tile epilogue (lane g of row `orow` owns columns n0 + 32*nb + 16*h + 8*g + 0..7)
+// one 16-byte-aligned piece of eight elements of T, loaded whole (two 16-byte loads for fp32)
+template <typename T>
+struct Piece8;
+template <>
+struct Piece8<half_t> {
+  half8 x;
+  __device__ __forceinline__ void load(const half_t *p) { x = *reinterpret_cast<const half8 *>(p); }
+  __device__ __forceinline__ float at(int j) const { return (float)x[j]; }
+};
+template <>
+struct Piece8<float> {
+  f32x4 x0, x1;
+  __device__ __forceinline__ void load(const float *p) {
+    x0 = *reinterpret_cast<const f32x4 *>(p);
+    x1 = *reinterpret_cast<const f32x4 *>(p + 4);
+  }
+  __device__ __forceinline__ float at(int j) const { return j < 4 ? x0[j] : x1[j - 4]; }
+};
+
+// on the row pieces of the tile epilogue (lane g of row `orow` owns columns n0 + 32*nb + 16*h + 8*g + 0..7).
+// VEC: every piece is 16-byte aligned and lies wholly inside or outside the row.  The pieces of the bias, then
+// those of the residual row, are requested together from addresses that are valid for every lane (a lane
+// without a row or column reads the base and drops the value), so that a lane waits once per operand: loads
+// guarded piece by piece were issued and waited for one after the other, sixteen round trips at the end of
+// every workgroup of a 128-column tile.
+// Used where the register budget is fixed by the launch bounds anyway (the pipelined kernel: 128 registers, four
+// workgroups per CU); in the tile kernel and the barrier-free kernel the addresses and pieces in flight cost a
+// resident wavefront (output-stationary tile kernel at 128 columns: 97 -> 145 us), so those keep the guarded form.
+// NBB: column blocks whose pieces are in flight together (8 registers per block for fp16 rows, 16 for fp32).
+template <typename T, int NB, bool VEC, int NBB>
+__device__ __forceinline__ void epilogue_row_pieces_batched(float (&V)[NB][2][8], const TileArgs &a, int orow, int n0, int g,
+                                                            bool with_act) {
+  const T *bias = (const T *)a.bias;
+  const T *res = (const T *)a.res;
+  if (VEC) {
+#pragma unroll
+    for (int op = 0; op < 2; ++op) {
+      const T *base = op == 0 ? bias : res;
+      if (!base) continue;
+      const long long row_off = op == 0 ? 0ll : (long long)(orow >= 0 ? orow : 0) * a.c_out;
+#pragma unroll
+      for (int nb0 = 0; nb0 < NB; nb0 += NBB) {
+        Piece8<T> x[NBB][2];
+#pragma unroll
+        for (int nb = 0; nb < NBB; ++nb)
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            int c0 = n0 + (nb0 + nb) * 32 + 16 * h + 8 * g;
+            bool ok = nb0 + nb < NB && orow >= 0 && c0 < a.c_out;
+            x[nb][h].load(ok ? base + row_off + c0 : base);
+          }
+#pragma unroll
+        for (int nb = 0; nb < NBB; ++nb)
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            if (nb0 + nb >= NB) continue;
+            int c0 = n0 + (nb0 + nb) * 32 + 16 * h + 8 * g;
+            bool ok = orow >= 0 && c0 < a.c_out;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) V[nb0 + nb][h][j] += ok ? x[nb][h].at(j) : 0.f;
+          }
+      }
+    }
+  } else {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        int c0 = n0 + nb * 32 + 16 * h + 8 * g;
+        int valid = a.c_out - c0;
+        if (valid > 0 && orow >= 0) {
+          if (bias) add8<T, false>(V[nb][h], bias + c0, valid);
+          if (res) add8<T, false>(V[nb][h], res + (long long)orow * a.c_out + c0, valid);
+        }
+      }
+  }
+  const ActK k = act_coeffs(a.act, a.slope, with_act);
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) V[nb][h][j] = act_apply(V[nb][h][j], k);
+}
+
+// the same with every piece guarded and added as it arrives: fewest registers
 template <typename T, int NB, bool VEC>
 __device__ __forceinline__ void epilogue_row_pieces(float (&V)[NB][2][8], const TileArgs &a, int orow, int n0, int g,
                                                     bool with_act) {
@@ -1051,7 +1147,7 @@ __global__ void __launch_bounds__(256, 4) pipe_gemm_kernel(TileArgs a, TileArgs 
     if (dense && (c.bias || c.res || c.act)) {
       bool with_act = c.act != PCE_ACT_NONE;
       if (with_act && c.act_alone_only) with_act = orow >= 0 && c.ocsr[orow] == c.ocsr[orow + 1];
-      epilogue_row_pieces<half_t, NB, true>(V, c, orow, n0, g, with_act);
+      epilogue_row_pieces_batched<half_t, NB, true, NB>(V, c, orow, n0, g, with_act);
     }
   } else if (a.bias || a.res || a.act) {
     bool with_act = a.act != PCE_ACT_NONE;
@@ -1061,7 +1157,7 @@ __global__ void __launch_bounds__(256, 4) pipe_gemm_kernel(TileArgs a, TileArgs 
       erow = -1;
       with_act = false;
     }
-    epilogue_row_pieces<half_t, NB, true>(V, a, erow, n0, g, with_act);
+    epilogue_row_pieces_batched<half_t, NB, true, NB>(V, a, erow, n0, g, with_act);
   }
   half_t *out = (half_t *)((PMODE == PIPE_BOTH && dense) ? c.out : a.out);
   if (PMODE == MODE_FOD_BUF && a.out_alt)
@@ -1210,7 +1306,7 @@ __global__ void __launch_bounds__(256, SUB == 1 ? 3 : 2) os_pipe_kernel(TileArgs
   __syncthreads();  // the ring becomes the epilogue staging area
   float V[NB][2][8];
   gather_row_pieces<NB>(acc, V, g);
-  if (a.bias || a.res || a.act) epilogue_row_pieces<half_t, NB, true>(V, a, orow, n0, g, a.act != PCE_ACT_NONE);
+  if (a.bias || a.res || a.act) epilogue_row_pieces_batched<half_t, NB, true, NB>(V, a, orow, n0, g, a.act != PCE_ACT_NONE);
   store_rows_via_lds<half_t, NB>(V, lds + wave * WaveLds<NB>::PIECES, (half_t *)a.out, orow, a, n0, lane, l32, g);
 }
 
