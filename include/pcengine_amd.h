@@ -258,12 +258,13 @@ int pce_conv_fwd_gms(const void *in_feats, const void *weight, const void *weigh
  * n_pairs == n_out: the caller then states that every output row has exactly one pair (a transposed
  * layer whose kernel size equals its stride: every fine voxel has one parent), and each pair's product
  * is stored straight to its output row with the epilogue, without partial rows or a second pass.
- * odst_dev (optional, may be NULL; from pce_pair_route) routes the pairs of a layer without centre
- * offset: a pair that is the only one of its output row stores the finished row with the epilogue,
- * the others store partial rows, and the row sum visits only rows with two pairs or more (a strided
- * layer whose kernel equals its stride on a surface-like cloud has one pair for nearly every row).
- * Used for fp16 layers with c_in >= 64 a multiple of 32 and c_out >= 96 when the host copies of kpos /
- * qkpos are given; ignored otherwise.  Results are those of the unrouted call bit for bit.
+ * route_dev (optional, may be NULL; the array filled by pce_pair_route) routes the pairs of a layer
+ * without centre offset: a pair that is the only one of its output row stores the finished row with
+ * the epilogue, the others store partial rows, and the row sum visits only the rows whose pair count is
+ * not one (a strided layer whose kernel equals its stride on a surface-like cloud has one pair for
+ * nearly every row).  Used for fp16 layers with c_in >= 64 a multiple of 32 and c_out >= 96 when the
+ * host copies of kpos / qkpos are given; ignored otherwise.  Without an epilogue the output equals that
+ * of the unrouted call bit for bit; with one, a single-pair row is rounded to dtype once instead of twice.
  * No counterpart in the reference: it is ConvolutionForwardD2 with the atomic scatter-add replaced
  * by the output-stationary sum of ConvolutionForwardD1 (backend/spconv.cu:149-161), fused with
  * the centre GEMM. */
@@ -273,16 +274,21 @@ int pce_conv_fwd_fds(const void *in_feats, const void *weight, const void *weigh
                      const int32_t *omap_dev, const int32_t *oslot_dev, const int32_t *kpos_dev,
                      const int32_t *qkpos_dev,
                      const int32_t *kpos_host, const int32_t *qkpos_host, const int32_t *ocsr_dev,
-                     const int32_t *odst_dev, int64_t n_pairs, int64_t qsum, void *buffer_dev,
+                     const int32_t *route_dev, int64_t n_pairs, int64_t qsum, void *buffer_dev,
                      int64_t buffer_elems, const pce_epilogue_t *epilogue, pce_stream_t stream);
 
-/* Routing of the pairs of a layer without centre offset for pce_conv_fwd_fds: odst[p] = omap[p] when
- * pair p is the only pair of its output row (ocsr tells), else n_out + oslot[p].  All arrays on the
- * device, n_pairs entries (ocsr: n_out + 1); n_out + n_pairs must stay below 2^31.  No counterpart in
- * the reference, whose fetch-on-demand kernels add every pair's product atomically
- * (backend/spconv.cuh:1567-1730). */
+/* Routing array of a layer without centre offset for pce_conv_fwd_fds, int32 on the device:
+ *   route[0]              number of output rows whose pair count is not one (route[1..3] are zero)
+ *   route[4 .. 4+M)       destination of pair p: omap[p] when p is the only pair of its output row (ocsr
+ *                         tells), else n_out + oslot[p]
+ *   route[4+M .. 4+M+n_out)  the rows whose pair count is not one, route[0] of them, in no particular order
+ * pce_pair_route_elems gives the length (4 + n_pairs + n_out); n_out + n_pairs must stay below 2^31.
+ * Two launches on `stream`, no read-back.  No counterpart in the reference, whose fetch-on-demand
+ * kernels add every pair's product atomically (backend/spconv.cuh:1567-1730). */
+int64_t pce_pair_route_elems(int64_t n_pairs, int64_t n_out);
 int pce_pair_route(const int32_t *omap_dev, const int32_t *oslot_dev, const int32_t *ocsr_dev,
-                   int64_t n_pairs, int64_t n_out, int32_t *odst_dev, pce_stream_t stream);
+                   int64_t n_pairs, int64_t n_out, int32_t *route_dev, int64_t route_elems,
+                   pce_stream_t stream);
 
 /* Output-stationary: nbr[kv*n_out] from pce_kmap_build (for a transposed layer, a table built
  * with the roles swapped).  One kernel, one store per output row.  No counterpart in the

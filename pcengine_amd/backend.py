@@ -86,7 +86,7 @@ class KernelMap:
     ocode: Optional[torch.Tensor] = None
     islot: Optional[torch.Tensor] = None   # pair -> position of its entry in icode / ocode
     oslot: Optional[torch.Tensor] = None
-    odst: Optional[torch.Tensor] = None    # pair -> routed destination (pair_route), built on first use
+    route: Optional[torch.Tensor] = None   # routing array of a layer without centre offset (pair_route), built on first use
     tag: str = "auto"           # 'D1' / 'D2' when the reference's init_tag protocol fixed it
     in_coords: Optional[torch.Tensor] = None
     geom: Optional[Geom] = None
@@ -351,17 +351,18 @@ def ensure_csr(km: KernelMap) -> None:
 
 
 def pair_route(km: KernelMap) -> torch.Tensor:
-    """Destination of every pair of a layer without centre offset, cached on the map: the output row where the
-    pair is the row's only one, else ``n_out`` + its partial-row slot (``pce_pair_route``)."""
-    odst = km.odst
-    if odst is None:
+    """Routing array of a layer without centre offset, cached on the map (``pce_pair_route``): the number of output
+    rows whose pair count is not one, the destination of every pair (the output row where the pair is the row's
+    only one, else ``n_out`` + its partial-row slot) and the list of those rows."""
+    if km.route is None:
         ensure_csr(km)
         lib = _lib.load()
-        odst = torch.empty(max(km.M, 1), dtype=torch.int32, device=km.omap.device)
+        elems = lib.pce_pair_route_elems(km.M, km.n_out)
+        route = torch.empty(elems, dtype=torch.int32, device=km.omap.device)
         _lib.check(lib.pce_pair_route(km.omap.data_ptr(), km.oslot.data_ptr(), km.ocsr.data_ptr(), km.M, km.n_out,
-                                      odst.data_ptr(), _stream(km.omap.device)))
-        km.odst = odst
-    return odst
+                                      route.data_ptr(), elems, _stream(km.omap.device)))
+        km.route = route
+    return km.route
 
 
 def ensure_nbr(km: KernelMap, transposed: bool) -> None:
@@ -507,13 +508,13 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
         ocsr, oslot = (km.icsr, km.islot) if transposed else (km.ocsr, km.oslot)
         # A strided layer whose kernel equals its stride gives every input one pair; on surface-like clouds nearly
         # every output row then has a single pair, which stores the finished row itself (see pair_route).
-        odst = None
+        route = None
         if (route_single_pairs and not single and not transposed and not km.subm and tuple(km.ks) == tuple(km.stride)
                 and km.M > 0 and feats.dtype == torch.float16 and c_in >= 64 and c_in % 32 == 0 and c_out >= 96 and c_out % 8 == 0):
-            odst = pair_route(km)
+            route = pair_route(km)
         _lib.check(lib.pce_conv_fwd_fds(feats.data_ptr(), weight.data_ptr(), _ptr(packed), out.data_ptr(), dt, n_in, n_out,
                                         c_in, c_out, kv, mid, imap.data_ptr(), omap.data_ptr(), oslot.data_ptr(), km.kpos.data_ptr(),
-                                        km.qkpos.data_ptr(), km.kpos_host, km.qkpos_host, ocsr.data_ptr(), _ptr(odst), km.M, km.qsum,
+                                        km.qkpos.data_ptr(), km.kpos_host, km.qkpos_host, ocsr.data_ptr(), _ptr(route), km.M, km.qsum,
                                         None if single else buffer.data_ptr(), 0 if single else buffer.numel(), epi, s))
     elif dataflow == DATAFLOW_GMS:
         ensure_csr(km)

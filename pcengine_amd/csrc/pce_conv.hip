@@ -37,6 +37,7 @@ enum {
   EPI_ROWS_CSR = 3     // EPI_ROWS plus the sum of partial rows buf[ocsr[row] .. ocsr[row+1])
 };
 
+#define PCE_ROUTE_HEAD 4  // ints in front of the pair destinations of a routing array (pce_pair_route)
 #define MAX_KV_ARGS 32  // kpos / qkpos travel in the kernel arguments up to this kernel volume
 
 struct TileArgs {
@@ -1505,19 +1506,23 @@ __global__ void __launch_bounds__(256) scatter_rows_kernel(const T *__restrict__
   }
 }
 
-// out[row] = sum of the contiguous partial rows buf[csr[row] .. csr[row+1]), fp32 accumulate
+// out[row] = sum of the contiguous partial rows buf[csr[row] .. csr[row+1]), fp32 accumulate.  With `rows` the
+// kernel visits rows[0 .. *count) instead of every row (count read on the device, the grid is sized by the host
+// for the list's capacity and strides over it).
 template <typename T, int VEC>
 __global__ void __launch_bounds__(256) rowsum_kernel(const T *__restrict__ buf, long long n_out, int c_out, int G,
                                                      const int *__restrict__ csr, T *__restrict__ out,
                                                      const T *__restrict__ bias, const T *__restrict__ res, int act,
-                                                     float slope, int skip_single) {
+                                                     float slope, const int *__restrict__ rows,
+                                                     const int *__restrict__ count) {
   typedef typename VecOf<T, VEC>::type V;
   int rows_per_block = 256 / G;
-  long long row = (long long)blockIdx.x * rows_per_block + threadIdx.x / G;
   int sub = threadIdx.x % G;
-  if (row >= n_out) return;
+  const long long n_items = rows ? (long long)*count : n_out;
+  for (long long item = (long long)blockIdx.x * rows_per_block + threadIdx.x / G; item < n_items;
+       item += (long long)gridDim.x * rows_per_block) {
+  long long row = rows ? (long long)rows[item] : item;
   int e0 = csr[row], e1 = csr[row + 1];
-  if (skip_single && e1 - e0 == 1) return;  // the row's only pair has stored it already
   int row_vecs = c_out / VEC;
   for (int v = sub; v < row_vecs; v += G) {
     float acc[VEC];
@@ -1553,6 +1558,7 @@ __global__ void __launch_bounds__(256) rowsum_kernel(const T *__restrict__ buf, 
 #pragma unroll
     for (int j = 0; j < VEC; ++j) reinterpret_cast<T *>(&y)[j] = (T)act_apply(acc[j], act, slope);
     *reinterpret_cast<V *>(&out[row * c_out + (long long)v * VEC]) = y;
+  }
   }
 }
 
@@ -1984,11 +1990,11 @@ extern "C" int pce_conv_fwd_gms(const void *in, const void *w, const void *wp, v
 template <typename T>
 static int fds_impl(const void *in, const void *w, const void *wp, void *out, int64_t n_out, int c_in, int c_out, int kv,
                     int mid, const int *imap, const int *omap, const int *oslot, const int *kpos, const int *qkpos,
-                    const int32_t *kpos_host, const int32_t *qkpos_host, const int *ocsr, const int *odst, int64_t n_pairs,
+                    const int32_t *kpos_host, const int32_t *qkpos_host, const int *ocsr, const int *route, int64_t n_pairs,
                     int64_t qsum, T *buffer, const Epi &e, hipStream_t s) {
   constexpr int VEC = sizeof(T) == 2 ? 8 : 4;
   int rc;
-  int skip_single = 0;
+  const int *multi_rows = nullptr, *multi_count = nullptr;  // set by the routed pair tiles
   if (!buffer && qsum > 0) {
     // Every output row has exactly one pair (a transposed layer whose kernel equals its stride: each fine
     // voxel has one parent): a pair's product is its output row, stored once with the epilogue, no partial rows.
@@ -2031,7 +2037,7 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
       return PCE_OK;
     }
   }
-  if (mid < 0 && odst && buffer && qsum > 0 && stage_on(1) && stage_on(2) && stage_on(5) && n_out + n_pairs < (1ll << 31)) {
+  if (mid < 0 && route && buffer && qsum > 0 && stage_on(1) && stage_on(2) && stage_on(5) && n_out + n_pairs < (1ll << 31)) {
     // Routed pair tiles (a layer without centre offset): the only pair of an output row stores the finished row
     // with the epilogue, the pairs of the other rows store partial rows; the row sum then visits only rows with
     // two pairs or more.  Taken by the pipelined kernel's shapes; the others ignore the routing.
@@ -2039,7 +2045,7 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
     set_out<T>(&a, out, false);
     set_host_pos(&a, kpos_host, qkpos_host);
     a.imap = imap;
-    a.oslot = odst;
+    a.oslot = route + PCE_ROUTE_HEAD;
     a.kpos = kpos;
     a.qkpos = qkpos;
     a.mode = MODE_FOD_BUF;
@@ -2049,10 +2055,11 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
     set_epi(&a, e);
     if (pipe_gemm_ok(a, sizeof(T)) && aligned16(buffer)) {
       if ((rc = launch_pipe_gemm(a, qsum / PCE_QUANTUM, s))) return rc;
-      skip_single = 1;
+      multi_count = route;
+      multi_rows = route + PCE_ROUTE_HEAD + n_pairs;
     }
   }
-  if (qsum > 0 && stage_on(1) && !skip_single) {
+  if (qsum > 0 && stage_on(1) && !multi_rows) {
     TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
     set_out<T>(&a, buffer, false);
     set_host_pos(&a, kpos_host, qkpos_host);
@@ -2126,39 +2133,60 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
   if (vec) {
     int G = pow2_at_least(c_out / VEC);
     if (G > 64) G = 64;
-    hipLaunchKernelGGL((rowsum_kernel<T, VEC>), dim3((unsigned)pce_div_up(n_out, 256 / G)), dim3(256), 0, s,
+    // routed layer: the list holds at most n_out rows; a bounded grid strides over what it holds
+    long long blocks = pce_div_up(n_out, 256 / G);
+    if (multi_rows && blocks > 1024) blocks = 1024;
+    hipLaunchKernelGGL((rowsum_kernel<T, VEC>), dim3((unsigned)blocks), dim3(256), 0, s,
                        (const T *)buffer, (long long)n_out, c_out, G, ocsr, (T *)out, (const T *)e.bias, (const T *)e.res,
-                       e.act, e.slope, skip_single);
+                       e.act, e.slope, multi_rows, multi_count);
   } else {
     int G = pow2_at_least(c_out);
     if (G > 64) G = 64;
-    hipLaunchKernelGGL((rowsum_kernel<T, 1>), dim3((unsigned)pce_div_up(n_out, 256 / G)), dim3(256), 0, s,
+    long long blocks = pce_div_up(n_out, 256 / G);
+    if (multi_rows && blocks > 1024) blocks = 1024;
+    hipLaunchKernelGGL((rowsum_kernel<T, 1>), dim3((unsigned)blocks), dim3(256), 0, s,
                        (const T *)buffer, (long long)n_out, c_out, G, ocsr, (T *)out, (const T *)e.bias, (const T *)e.res,
-                       e.act, e.slope, skip_single);
+                       e.act, e.slope, multi_rows, multi_count);
   }
   PCE_LAUNCH_CHECK("rowsum");
   return PCE_OK;
 }
 
-// destination of every pair of a layer without centre offset: the output row itself where the pair is the
-// row's only one, else n_out + the pair's partial-row slot
+// Routing of the pairs of a layer without centre offset.  route[0] = number of output rows whose pair count is
+// not one, route[4 .. 4+M) = destination of every pair (the output row itself where the pair is the row's only
+// one, else n_out + the pair's partial-row slot), route[4+M .. 4+M+n_out) = the rows whose pair count is not
+// one, in the order in which they were counted (any order serves the row sum, which visits exactly these).
+__global__ void route_clear_kernel(int *route) {
+  if (threadIdx.x < PCE_ROUTE_HEAD) route[threadIdx.x] = 0;
+}
 __global__ void __launch_bounds__(256) pair_route_kernel(const int *__restrict__ omap, const int *__restrict__ oslot,
                                                          const int *__restrict__ ocsr, long long n_pairs, int n_out,
-                                                         int *__restrict__ odst) {
-  long long p = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (p >= n_pairs) return;
-  int o = omap[p];
-  odst[p] = (ocsr[o + 1] - ocsr[o] == 1) ? o : n_out + oslot[p];
+                                                         int *__restrict__ route) {
+  long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < n_pairs) {
+    int o = omap[t];
+    route[PCE_ROUTE_HEAD + t] = (ocsr[o + 1] - ocsr[o] == 1) ? o : n_out + oslot[t];
+  }
+  if (t < n_out && ocsr[t + 1] - ocsr[t] != 1) route[PCE_ROUTE_HEAD + n_pairs + atomicAdd(&route[0], 1)] = (int)t;
+}
+
+extern "C" int64_t pce_pair_route_elems(int64_t n_pairs, int64_t n_out) {
+  return (n_pairs < 0 || n_out < 0) ? 0 : PCE_ROUTE_HEAD + n_pairs + n_out;
 }
 
 extern "C" int pce_pair_route(const int32_t *omap, const int32_t *oslot, const int32_t *ocsr, int64_t n_pairs, int64_t n_out,
-                              int32_t *odst, pce_stream_t stream) {
+                              int32_t *route, int64_t route_elems, pce_stream_t stream) {
   if (n_pairs < 0 || n_out < 0) PCE_FAIL(PCE_EINVAL, "pce_pair_route: negative count");
-  if (n_pairs == 0) return PCE_OK;
-  if (!omap || !oslot || !ocsr || !odst) PCE_FAIL(PCE_EINVAL, "pce_pair_route: null pointer");
+  if (!route || !ocsr || (n_pairs > 0 && (!omap || !oslot))) PCE_FAIL(PCE_EINVAL, "pce_pair_route: null pointer");
   if (n_out + n_pairs >= (1ll << 31)) PCE_FAIL(PCE_ECAPACITY, "pce_pair_route: n_out + n_pairs = %lld exceeds int32", (long long)(n_out + n_pairs));
-  hipLaunchKernelGGL(pair_route_kernel, dim3((unsigned)pce_div_up(n_pairs, 256)), dim3(256), 0, (hipStream_t)stream, omap, oslot,
-                     ocsr, (long long)n_pairs, (int)n_out, odst);
+  if (route_elems < pce_pair_route_elems(n_pairs, n_out))
+    PCE_FAIL(PCE_EWORKSPACE, "pce_pair_route: route holds %lld elements, needs %lld", (long long)route_elems, (long long)pce_pair_route_elems(n_pairs, n_out));
+  hipLaunchKernelGGL(route_clear_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, route);
+  PCE_LAUNCH_CHECK("route_clear");
+  long long threads = n_pairs > n_out ? n_pairs : n_out;
+  if (threads == 0) return PCE_OK;
+  hipLaunchKernelGGL(pair_route_kernel, dim3((unsigned)pce_div_up(threads, 256)), dim3(256), 0, (hipStream_t)stream, omap, oslot,
+                     ocsr, (long long)n_pairs, (int)n_out, route);
   PCE_LAUNCH_CHECK("pair_route");
   return PCE_OK;
 }
@@ -2167,7 +2195,7 @@ extern "C" int pce_conv_fwd_fds(const void *in, const void *w, const void *wp, v
                                 int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv, int32_t mid, const int32_t *imap,
                                 const int32_t *omap, const int32_t *oslot, const int32_t *kpos, const int32_t *qkpos,
                                 const int32_t *kpos_host, const int32_t *qkpos_host, const int32_t *ocsr,
-                                const int32_t *odst, int64_t n_pairs, int64_t qsum, void *buffer, int64_t buffer_elems,
+                                const int32_t *route, int64_t n_pairs, int64_t qsum, void *buffer, int64_t buffer_elems,
                                 const pce_epilogue_t *epilogue, pce_stream_t stream) {
   int rc = check_common("pce_conv_fwd_fds", in, w, out, dtype, n_in, n_out, c_in, c_out, kv, mid);
   if (rc || (rc = check_qsum("pce_conv_fwd_fds", qsum))) return rc;
@@ -2184,8 +2212,8 @@ extern "C" int pce_conv_fwd_fds(const void *in, const void *w, const void *wp, v
   }
   hipStream_t s = (hipStream_t)stream;
   if (dtype == PCE_F16)
-    return fds_impl<half_t>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, omap, oslot, kpos, qkpos, kpos_host, qkpos_host, ocsr, odst, n_pairs, qsum, (half_t *)buffer, e, s);
-  return fds_impl<float>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, omap, oslot, kpos, qkpos, kpos_host, qkpos_host, ocsr, odst, n_pairs, qsum, (float *)buffer, e, s);
+    return fds_impl<half_t>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, omap, oslot, kpos, qkpos, kpos_host, qkpos_host, ocsr, route, n_pairs, qsum, (half_t *)buffer, e, s);
+  return fds_impl<float>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, omap, oslot, kpos, qkpos, kpos_host, qkpos_host, ocsr, route, n_pairs, qsum, (float *)buffer, e, s);
 }
 
 template <typename T>

@@ -336,10 +336,14 @@ def test_strided_layer_routes_single_pair_rows(cloud, c_in, c_out):
     km = gpu_map(coords, ks, ks, want_csr=True)
     pk = backend.pack_weights(wd)
     # the routing array against its definition
-    odst = backend.pair_route(km).cpu().numpy()
+    route = backend.pair_route(km).cpu().numpy()
+    assert len(route) == lib.pce_pair_route_elems(km.M, km.n_out) == 4 + km.M + km.n_out
     ocsr, omap, oslot = km.ocsr.cpu().numpy(), km.omap.cpu().numpy()[:km.M], km.oslot.cpu().numpy()[:km.M]
     cnt = np.diff(ocsr)
-    assert np.array_equal(odst[:km.M], np.where(cnt[omap] == 1, omap, km.n_out + oslot))
+    assert np.array_equal(route[4:4 + km.M], np.where(cnt[omap] == 1, omap, km.n_out + oslot))
+    others = np.flatnonzero(cnt != 1)
+    assert route[0] == len(others) and not route[1:4].any()
+    assert np.array_equal(np.sort(route[4 + km.M:4 + km.M + route[0]]), others)
     singles = int((cnt == 1).sum())
     assert 0 < singles < km.n_out or cloud == "surface"
     plain = backend.conv_forward(fd, wd, km, DATAFLOW_FDS, packed=pk, route_single_pairs=False)
@@ -360,9 +364,10 @@ def test_strided_layer_routes_single_pair_rows(cloud, c_in, c_out):
         ref = _act_np(ref, act)
         assert orc.rel_l2(got.double().cpu().numpy(), ref) <= 1e-3, act
     # argument checks of the routing entry point
-    assert lib.pce_pair_route(None, None, None, 5, 5, None, None) == _lib.PCE_EINVAL
-    assert lib.pce_pair_route(km.omap.data_ptr(), km.oslot.data_ptr(), km.ocsr.data_ptr(), 1 << 30, 1 << 30, 1, None) == _lib.PCE_ECAPACITY
-    assert lib.pce_pair_route(None, None, None, 0, 5, None, None) == _lib.PCE_OK
+    one = km.ocsr.data_ptr()
+    assert lib.pce_pair_route(None, None, None, 5, 5, None, 100, None) == _lib.PCE_EINVAL
+    assert lib.pce_pair_route(one, one, one, 1 << 30, 1 << 30, one, 1 << 40, None) == _lib.PCE_ECAPACITY
+    assert lib.pce_pair_route(one, one, one, 5, 5, one, 13, None) == _lib.PCE_EWORKSPACE
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
