@@ -87,6 +87,7 @@ class KernelMap:
     islot: Optional[torch.Tensor] = None   # pair -> position of its entry in icode / ocode
     oslot: Optional[torch.Tensor] = None
     route: Optional[torch.Tensor] = None   # routing array of a layer without centre offset (pair_route), built on first use
+    route_t: Optional[torch.Tensor] = None # the same for the transposed layer over this map
     tag: str = "auto"           # 'D1' / 'D2' when the reference's init_tag protocol fixed it
     in_coords: Optional[torch.Tensor] = None
     geom: Optional[Geom] = None
@@ -350,19 +351,25 @@ def ensure_csr(km: KernelMap) -> None:
     km.islot, km.oslot = full.islot, full.oslot
 
 
-def pair_route(km: KernelMap) -> torch.Tensor:
+def pair_route(km: KernelMap, transposed: bool = False) -> torch.Tensor:
     """Routing array of a layer without centre offset, cached on the map (``pce_pair_route``): the number of output
     rows whose pair count is not one, the destination of every pair (the output row where the pair is the row's
-    only one, else ``n_out`` + its partial-row slot) and the list of those rows."""
-    if km.route is None:
+    only one, else ``n_out`` + its partial-row slot) and the list of those rows.  ``transposed``: the array of
+    the transposed layer, whose output rows are the map's input rows."""
+    route = km.route_t if transposed else km.route
+    if route is None:
         ensure_csr(km)
         lib = _lib.load()
-        elems = lib.pce_pair_route_elems(km.M, km.n_out)
-        route = torch.empty(elems, dtype=torch.int32, device=km.omap.device)
-        _lib.check(lib.pce_pair_route(km.omap.data_ptr(), km.oslot.data_ptr(), km.ocsr.data_ptr(), km.M, km.n_out,
-                                      route.data_ptr(), elems, _stream(km.omap.device)))
-        km.route = route
-    return km.route
+        omap, oslot, ocsr, n_out = (km.imap, km.islot, km.icsr, km.n_in) if transposed else (km.omap, km.oslot, km.ocsr, km.n_out)
+        elems = lib.pce_pair_route_elems(km.M, n_out)
+        route = torch.empty(elems, dtype=torch.int32, device=omap.device)
+        _lib.check(lib.pce_pair_route(omap.data_ptr(), oslot.data_ptr(), ocsr.data_ptr(), km.M, n_out,
+                                      route.data_ptr(), elems, _stream(omap.device)))
+        if transposed:
+            km.route_t = route
+        else:
+            km.route = route
+    return route
 
 
 def ensure_nbr(km: KernelMap, transposed: bool) -> None:
@@ -507,11 +514,13 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
         imap, omap = (km.omap, km.imap) if transposed else (km.imap, km.omap)
         ocsr, oslot = (km.icsr, km.islot) if transposed else (km.ocsr, km.oslot)
         # A strided layer whose kernel equals its stride gives every input one pair; on surface-like clouds nearly
-        # every output row then has a single pair, which stores the finished row itself (see pair_route).
+        # every output row then has a single pair, which stores the finished row itself (see pair_route).  The
+        # transposed layer over such a map has at most one pair per output row: exactly one unless the voxel's
+        # parent was clipped away, and those rows (no pair) are the only ones left to the row sum.
         route = None
-        if (route_single_pairs and not single and not transposed and not km.subm and tuple(km.ks) == tuple(km.stride)
+        if (route_single_pairs and not single and not km.subm and tuple(km.ks) == tuple(km.stride)
                 and km.M > 0 and feats.dtype == torch.float16 and c_in >= 64 and c_in % 32 == 0 and c_out >= 96 and c_out % 8 == 0):
-            route = pair_route(km)
+            route = pair_route(km, transposed)
         _lib.check(lib.pce_conv_fwd_fds(feats.data_ptr(), weight.data_ptr(), _ptr(packed), out.data_ptr(), dt, n_in, n_out,
                                         c_in, c_out, kv, mid, imap.data_ptr(), omap.data_ptr(), oslot.data_ptr(), km.kpos.data_ptr(),
                                         km.qkpos.data_ptr(), km.kpos_host, km.qkpos_host, ocsr.data_ptr(), _ptr(route), km.M, km.qsum,

@@ -370,6 +370,42 @@ def test_strided_layer_routes_single_pair_rows(cloud, c_in, c_out):
     assert lib.pce_pair_route(one, one, one, 5, 5, one, 13, None) == _lib.PCE_EWORKSPACE
 
 
+@pytest.mark.parametrize("c_in,c_out", [(128, 96), (256, 128)])
+def test_transposed_layer_with_clipped_parents_is_routed(c_in, c_out):
+    """A transposed k2s2 layer over a map whose coarse bound clipped some parents away: the fine voxels without a
+    parent have no pair (their rows are act(bias + residual)), every other row has exactly one, stored by the pair
+    tiles; only the rows without a pair are left to the row sum."""
+    coords = synth.random_cloud(seed=49, n=9000, extent=21, batches=2)     # coordinates 0..20: x = 20 has no parent
+    ks = (2, 2, 2)
+    ref_map = orc.kernel_map(coords, ks, ks, (0, 0, 0))
+    km = gpu_map(coords, ks, ks, want_csr=True)
+    assert 0 < km.M < km.n_in
+    route = backend.pair_route(km, transposed=True).cpu().numpy()
+    cnt = np.diff(km.icsr.cpu().numpy())
+    assert set(np.unique(cnt)) == {0, 1}
+    assert route[0] == (cnt == 0).sum()
+    assert np.array_equal(np.sort(route[4 + km.M:4 + km.M + route[0]]), np.flatnonzero(cnt == 0))
+    assert np.array_equal(route[4:4 + km.M], km.imap.cpu().numpy()[:km.M])
+    coarse = synth.features(8, km.n_out, c_in)
+    wt = synth.weights(8, 8, c_in, c_out)
+    cd, wd = torch.as_tensor(coarse, device=DEV).half(), torch.as_tensor(wt, device=DEV).half()
+    pk = backend.pack_weights(wd)
+    want = orc.conv_forward(rounded(coarse, torch.float16), rounded(wt, torch.float16), ref_map, ks, transposed=True)
+    plain = backend.conv_forward(cd, wd, km, DATAFLOW_FDS, transposed=True, packed=pk, route_single_pairs=False)
+    out = torch.full((km.n_in, c_out), float("nan"), dtype=torch.float16, device=DEV)
+    routed = backend.conv_forward(cd, wd, km, DATAFLOW_FDS, transposed=True, packed=pk, out=out)
+    assert torch.equal(plain, routed)
+    assert (routed[torch.as_tensor(cnt == 0, device=DEV)] == 0).all()
+    assert orc.rel_l2(routed.double().cpu().numpy(), want) <= 1e-3
+    rng = np.random.default_rng(49)
+    bias, res = rng.standard_normal(c_out) * 0.5, rng.standard_normal((km.n_in, c_out))
+    bd, rd = torch.as_tensor(bias, device=DEV).half(), torch.as_tensor(res, device=DEV).half()
+    for b, r, act in [(bd, rd, "relu"), (bd, None, ("leaky_relu", 0.1)), (None, rd, None)]:
+        got = backend.conv_forward(cd, wd, km, DATAFLOW_FDS, transposed=True, packed=pk, bias=b, residual=r, act=act)
+        ref = want + (rounded(bias, torch.float16) if b is not None else 0) + (rounded(res, torch.float16) if r is not None else 0)
+        assert orc.rel_l2(got.double().cpu().numpy(), _act_np(ref, act)) <= 1e-3, act
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 @pytest.mark.parametrize("ks,c_in,c_out", [((5, 5, 5), 32, 32), ((5, 5, 5), 64, 128), ((5, 3, 1), 16, 24), ((1, 5, 5), 128, 96)])
 def test_large_and_anisotropic_kernels_forward_and_backward(ks, c_in, c_out, dtype):
