@@ -82,3 +82,34 @@ def test_config5_indoor_batch_full_size():
         assert bool((diff <= 2.0 ** -10 * ref2.abs() + 27 * 2.0 ** -23).all()), flow
         tipped = int((diff > 27 * 2.0 ** -23).sum())
         assert tipped <= (0 if flow == DATAFLOW_OS else diff.numel() // 100_000), (flow, tipped)
+
+
+@pytest.mark.parametrize("name", ["cfg1", "cfg2", "cfg4", "cfg5"])
+def test_full_size_maps_match_the_frozen_manifest(name):
+    """Every benchmark cloud at its full size: the GPU's output coordinates, per-offset counts and pair lists
+    against the digests that tests/golden/manifest.json holds (written by the CPU oracle, reproduced by it in
+    the CPU suite), submanifold and k2s2 layer, bit for bit."""
+    import hashlib
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "manifest.json")) as f:
+        frozen = json.load(f)[name]
+    gen = {"cfg1": synth.sphere_plane_cloud, "cfg2": synth.lidar_cloud, "cfg4": synth.lidar_cloud_100k,
+           "cfg5": synth.indoor_batch}[name]
+    coords = gen()
+
+    def digest(*tensors):
+        h = hashlib.sha256()
+        for t in tensors:
+            h.update(np.ascontiguousarray(t.cpu().numpy(), dtype="<i4").tobytes())
+        return h.hexdigest()
+    assert len(coords) == frozen["voxels"] and digest(torch.as_tensor(coords)) == frozen["coords_sha256"]
+    for key, want in frozen["layers"].items():
+        ks = tuple(int(c) for c in key[1:4])
+        stride = tuple(int(c) for c in key[6:9])
+        kw = {} if stride == (1, 1, 1) else {"batchsize": frozen["batches"]}
+        km = gpu_map(coords, ks, stride, (0, 0, 0), **kw)
+        assert (km.n_out, km.M, km.qsum) == (want["n_out"], want["pairs"], want["qsum"]), key
+        assert km.knnz.cpu().tolist() == want["knnz"], key
+        assert digest(km.out_coords) == want["out_coords_sha256"], key
+        assert digest(km.imap[:km.M], km.omap[:km.M]) == want["pairs_sha256"], key

@@ -332,3 +332,32 @@ def test_backward_vs_autograd_through_dense_conv3d(ks, stride, pad):
         up = F.conv_transpose3d(dense_o, wdt, stride=stride, padding=pad, output_padding=opad)
         (up[c[:, 0], :, c[:, 1], c[:, 2], c[:, 3]] * torch.as_tensor(gi)).sum().backward()
         assert orc.rel_l2(gfo, fot.grad.numpy()) < 1e-12 and orc.rel_l2(gwT, wTt.grad.numpy()) < 1e-12
+
+
+def _load_make_manifest():
+    import importlib.util
+    import os
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "make_manifest.py")
+    spec = importlib.util.spec_from_file_location("make_manifest", path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+@pytest.mark.parametrize("name", ["cfg1", "cfg2", "cfg4", "cfg5"])
+def test_manifest_of_benchmark_inputs_is_reproduced(name):
+    """tests/golden/manifest.json freezes the voxel counts, pair counts and digests of the benchmark clouds and of
+    their kernel maps: the seeded generators and the oracle reproduce it bit for bit."""
+    import json
+    mm = _load_make_manifest()
+    with open(mm.PATH) as f:
+        frozen = json.load(f)
+    assert set(frozen) == set(mm.CONFIGS)
+    assert mm.config_entry(name) == frozen[name]
+    # what the frozen numbers must satisfy whatever the generator: pair symmetry of submanifold maps
+    sub = frozen[name]["layers"]["k333_s111_p000"]
+    assert sub["knnz"] == sub["knnz"][::-1] and sub["knnz"][13] == 0 and sum(sub["knnz"]) == sub["pairs"]
+    assert sub["n_out"] == frozen[name]["voxels"]
+    down = frozen[name]["layers"].get("k222_s222_p000")
+    if down:
+        assert down["pairs"] <= frozen[name]["voxels"] and down["n_out"] <= down["pairs"]
