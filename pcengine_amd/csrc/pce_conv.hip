@@ -3113,7 +3113,11 @@ extern "C" int pce_concat_cols(const void *a, int32_t c_a, const void *b, int32_
 // 64..512): up to 64x64 channels output-stationary leads from rho = 4 (2x at rho = 5), up to 128x128
 // from rho = 5..6, up to 256x256 the two are within 10 % between rho = 9 and 13 and output-stationary
 // leads by 1.35x at rho = 20; at 512 channels deferred scatter leads at every density seen.  A
-// 2x2x2 stride-2 layer covers every input exactly once and favours output-stationary up to 64x64.
+// 2x2x2 stride-2 layer covers every input exactly once and favours output-stationary up to 64x64; up to
+// 128x128 it does from two pairs per row (128 -> 128 at rho = 4.0: 31 vs 46 us, at rho = 2.5: 22 vs 25 us),
+// while on surface-like clouds (rho near 1) deferred scatter stores nearly every row straight from its only
+// pair and leads (64 -> 128 at rho = 1.03: 23 vs 43 us).  Products up to 128x256 sit between the 128x128 and
+// 256x256 classes: output-stationary leads at rho = 10.3 (155 vs 178 us) and 19.5 (85 vs 154 us).
 // The atomic fetch-on-demand and the staged gather-GEMM-scatter dataflows of the reference were never
 // the fastest (gather-GEMM-scatter comes first only on a 4-channel input layer, by 10 %).
 extern "C" int pce_select_dataflow(int64_t n_in, int64_t n_out, int64_t n_pairs, int32_t c_in, int32_t c_out, int32_t kv,
@@ -3123,11 +3127,14 @@ extern "C" int pce_select_dataflow(int64_t n_in, int64_t n_out, int64_t n_pairs,
   const double rho = (double)n_pairs / (double)n_out;
   const int64_t prod = (int64_t)c_in * c_out;
   if (kv <= 8 && n_out <= n_in && rho >= 1.0 && prod <= 64 * 64 && dtype == PCE_F16) return PCE_DATAFLOW_OS;
+  if (kv <= 8 && n_out <= n_in && rho >= 2.0 && prod <= 128 * 128 && dtype == PCE_F16) return PCE_DATAFLOW_OS;
   double takeover;
   if (prod <= 64 * 64)
     takeover = 4.0;
   else if (prod <= 128 * 128)
     takeover = 5.0;
+  else if (prod <= 128 * 256)
+    takeover = 10.0;
   else if (prod <= 256 * 256)
     takeover = 12.0;
   else

@@ -72,6 +72,25 @@ def test_selector_is_monotone_in_density():
     assert ranks == sorted(ranks)
 
 
+def test_selector_on_measured_layers():
+    """Layers whose four dataflows were timed on the GPU: the selector picks the fastest (or one within 2 % of it)."""
+    lib = _lib.load()
+    FDS, OS = _lib.DATAFLOW_FDS, _lib.DATAFLOW_OS
+    cases = [  # n_in, n_out, pairs, c_in, c_out, kv, expected
+        (149866, 149866, 30620, 64, 64, 27, FDS),      # the headline layer
+        (149866, 146018, 149866, 64, 128, 8, FDS),     # k2s2 on a LiDAR cloud: one pair for nearly every row
+        (216268, 53439, 215000, 128, 128, 8, OS),      # k2s2 on an indoor batch, four pairs per row
+        (65807, 25916, 64194, 128, 128, 8, OS),
+        (53439, 53439, 550000, 128, 256, 27, OS),      # rho = 10.3
+        (53439, 53439, 550000, 256, 256, 27, FDS),
+        (25916, 25916, 506646, 256, 256, 27, OS),      # rho = 19.5
+        (12063, 12063, 140000, 512, 512, 27, FDS),
+        (65807, 65807, 586656, 64, 128, 27, OS),
+    ]
+    for n_in, n_out, pairs, ci, co, kv, want in cases:
+        assert lib.pce_select_dataflow(n_in, n_out, pairs, ci, co, kv, _lib.PCE_F16) == want, (n_in, n_out, ci, co, kv)
+
+
 def test_codes_and_strides():
     assert pe.conv_info_encoder([1, 1, 1]) == 94585
     for v in [(1, 1, 1), (2, 2, 2), (3, 1, 5), (8, 8, 8)]:
