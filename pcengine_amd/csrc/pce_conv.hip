@@ -1521,44 +1521,44 @@ __global__ void __launch_bounds__(256) rowsum_kernel(const T *__restrict__ buf, 
   const long long n_items = rows ? (long long)*count : n_out;
   for (long long item = (long long)blockIdx.x * rows_per_block + threadIdx.x / G; item < n_items;
        item += (long long)gridDim.x * rows_per_block) {
-  long long row = rows ? (long long)rows[item] : item;
-  int e0 = csr[row], e1 = csr[row + 1];
-  int row_vecs = c_out / VEC;
-  for (int v = sub; v < row_vecs; v += G) {
-    float acc[VEC];
+    long long row = rows ? (long long)rows[item] : item;
+    int e0 = csr[row], e1 = csr[row + 1];
+    int row_vecs = c_out / VEC;
+    for (int v = sub; v < row_vecs; v += G) {
+      float acc[VEC];
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
-    const T *bp = buf + (long long)v * VEC;
-    int e = e0;
-    for (; e + 4 <= e1; e += 4) {  // four partial rows in flight
-      V x[4];
+      for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
+      const T *bp = buf + (long long)v * VEC;
+      int e = e0;
+      for (; e + 4 <= e1; e += 4) {  // four partial rows in flight
+        V x[4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) x[u] = *reinterpret_cast<const V *>(bp + (long long)(e + u) * c_out);
+        for (int u = 0; u < 4; ++u) x[u] = *reinterpret_cast<const V *>(bp + (long long)(e + u) * c_out);
 #pragma unroll
-      for (int u = 0; u < 4; ++u)
+        for (int u = 0; u < 4; ++u)
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) acc[j] += (float)(reinterpret_cast<const T *>(&x[u])[j]);
+          for (int j = 0; j < VEC; ++j) acc[j] += (float)(reinterpret_cast<const T *>(&x[u])[j]);
+      }
+      for (; e < e1; ++e) {
+        V x = *reinterpret_cast<const V *>(bp + (long long)e * c_out);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[j] += (float)(reinterpret_cast<const T *>(&x)[j]);
+      }
+      V y;
+      if (bias) {
+        V b = *reinterpret_cast<const V *>(&bias[(long long)v * VEC]);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[j] += (float)(reinterpret_cast<const T *>(&b)[j]);
+      }
+      if (res) {
+        V r = *reinterpret_cast<const V *>(&res[row * c_out + (long long)v * VEC]);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[j] += (float)(reinterpret_cast<const T *>(&r)[j]);
+      }
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) reinterpret_cast<T *>(&y)[j] = (T)act_apply(acc[j], act, slope);
+      *reinterpret_cast<V *>(&out[row * c_out + (long long)v * VEC]) = y;
     }
-    for (; e < e1; ++e) {
-      V x = *reinterpret_cast<const V *>(bp + (long long)e * c_out);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) acc[j] += (float)(reinterpret_cast<const T *>(&x)[j]);
-    }
-    V y;
-    if (bias) {
-      V b = *reinterpret_cast<const V *>(&bias[(long long)v * VEC]);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) acc[j] += (float)(reinterpret_cast<const T *>(&b)[j]);
-    }
-    if (res) {
-      V r = *reinterpret_cast<const V *>(&res[row * c_out + (long long)v * VEC]);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) acc[j] += (float)(reinterpret_cast<const T *>(&r)[j]);
-    }
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) reinterpret_cast<T *>(&y)[j] = (T)act_apply(acc[j], act, slope);
-    *reinterpret_cast<V *>(&out[row * c_out + (long long)v * VEC]) = y;
-  }
   }
 }
 
