@@ -265,6 +265,8 @@ int pce_conv_fwd_gms(const void *in_feats, const void *weight, const void *weigh
  * nearly every row).  Used for fp16 layers with c_in >= 64 a multiple of 32 and c_out >= 96 when the
  * host copies of kpos / qkpos are given; ignored otherwise.  Without an epilogue the output equals that
  * of the unrouted call bit for bit; with one, a single-pair row is rounded to dtype once instead of twice.
+ * The array must have been built from this call's omap_dev / oslot_dev / ocsr_dev with the same n_pairs and
+ * n_out (its entries are row indices the kernels store to, trusted like the map arrays themselves).
  * No counterpart in the reference: it is ConvolutionForwardD2 with the atomic scatter-add replaced
  * by the output-stationary sum of ConvolutionForwardD1 (backend/spconv.cu:149-161), fused with
  * the centre GEMM. */
