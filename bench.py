@@ -30,9 +30,9 @@ def main() -> int:
                          "set beyond the last-level cache); deep: a decoder-like layer (dense map, C 256->256) for the MFMA roofline")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-net", action="store_true", help="skip the MinkUNet-style forward (configuration 4)")
-    ap.add_argument("--all-configs", action="store_true",
-                    help="also time configurations 1 (fp32 C16 layer), 3 (k2s2 down + transposed up) and 5 (8-scene indoor "
-                         "batch, widened network); results go to extra.cfg1 / cfg3 / cfg5")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip configurations 1 (fp32 C16 layer), 3 (k2s2 down + transposed up) and 5 (8-scene indoor "
+                         "batch, widened network), whose timings go to extra.cfg1 / cfg3 / cfg5")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this engine has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -88,9 +88,13 @@ def main() -> int:
         torch.cuda.synchronize()
         return a.elapsed_time(b) / steps
 
-    def graph_ms(fn, steps, warmup):
-        """`steps` calls captured into one HIP graph; HIP events around one replay on the current
-        stream.  Two or three launches of 5-15 us each are otherwise paced by the host."""
+    REPLAYS = 11
+
+    def graph_ms(fn, steps, warmup, replays=REPLAYS, spread=None):
+        """`steps` calls captured into one HIP graph; the graph is replayed `replays` times, each replay
+        between its own pair of HIP events on the current stream (the stream the kernels are launched on);
+        the figure is the median replay divided by `steps` (`spread` receives min / median / max).  Two or
+        three launches of 5-15 us each are otherwise paced by the host."""
         for _ in range(warmup):
             fn()
         torch.cuda.synchronize()
@@ -100,12 +104,18 @@ def main() -> int:
                 fn()
         g.replay()
         torch.cuda.synchronize()
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record()
-        g.replay()
-        b.record()
-        torch.cuda.synchronize()
-        return a.elapsed_time(b) / steps, g
+        times = []
+        for _ in range(replays):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            g.replay()
+            b.record()
+            torch.cuda.synchronize()
+            times.append(a.elapsed_time(b) / steps)
+        times.sort()
+        if spread is not None:
+            spread.update({"min": times[0], "median": times[len(times) // 2], "max": times[-1], "replays": replays})
+        return times[len(times) // 2], g
 
     # ---- kernel map (built once, reused by every step; timed separately) -----------------------
     build = lambda: backend.build_kernel_map(cd, ks, (1, 1, 1), (0, 0, 0), [0, 0, 0], cmax, True, want_csr=True)
@@ -139,8 +149,9 @@ def main() -> int:
     # checked against the eager result, with eager work and synchronisations between replays.
     want = step().clone()
     launch = "hip_graph"
+    spread = {}
     try:
-        ms, graph = graph_ms(step, args.steps, args.warmup)
+        ms, graph = graph_ms(step, args.steps, args.warmup, spread=spread)
         for _ in range(3):
             out_buf.zero_()
             step(DATAFLOW_OS)
@@ -170,10 +181,12 @@ def main() -> int:
                                   {1: "fod_pairs_to_buffer", 2: "centre_gemm_then_row_sum"}),
                    DATAFLOW_OS: {1: "os_tile"}}[flow]
     if flow != DATAFLOW_OS:
-        for bit, name in stage_names.items():
-            lib.pce_set_stage_mask((1 << bit) | 0xFFFFFFF0)   # bits 4 and up keep the kernel selection of the full run
-            stages[name] = timer(step, max(20, args.steps // 4), 5)[0]
-        lib.pce_set_stage_mask(0xFFFFFFFF)
+        # one stage at a time, on the measurement build of the library (the same kernels; the product library has
+        # no stage switch)
+        with _lib.measurement_build() as mlib:
+            for bit, name in stage_names.items():
+                mlib.pce_set_stage_mask((1 << bit) | 0xFFFFFFF0)   # bits 4 and up keep the kernel selection of the full run
+                stages[name] = timer(step, max(20, args.steps // 4), 5)[0]
     else:
         stages["os_tile"] = ms
     others = {names[f]: timer(lambda f=f: step(f), max(20, args.steps // 4), 5)[0] for f in names if f != flow and f != DATAFLOW_FOD}
@@ -200,12 +213,24 @@ def main() -> int:
         "centre_gemm_then_row_sum": n * (c_in + c_out) * e + c_in * c_out * e + 3 * M * c_out * e + 8 * M + 4 * (n + 1),
     }[dom]
     achieved = dom_bytes / (stages[dom] * 1e-3) / 1e9
-    # HBM bytes per launch of that kernel from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
-    # profiles/pmc_traffic_cfg2.md (scaled by the copy-kernel calibration); counters cannot be read here
-    measured_traffic = {("cfg2", "centre_gemm_csr_sum"): 43.46e6, ("cfg2", "pairs_and_centre_gemm"): 47.09e6}
+    # HBM bytes per launch of that kernel: hardware counters cannot be read from inside this process, so the
+    # figure comes from the record the last rocprofv3 --pmc runs left in profiles/ (FETCH_SIZE and WRITE_SIZE,
+    # scaled by what they read for a plain copy), and only while the kernel sources are the ones it was
+    # measured on (the record holds their digest); otherwise null
+    traffic = None
+    try:
+        import hashlib
+        with open(os.path.join(ROOT, "profiles", "pmc_traffic.json")) as fh:
+            rec = json.load(fh).get(f"{args.workload}/{dom}")
+        with open(os.path.join(ROOT, "pcengine_amd", "csrc", "pce_conv.hip"), "rb") as fh:
+            src = hashlib.sha256(fh.read()).hexdigest()[:16]
+        if rec and rec.get("source_sha16") == src:
+            traffic = rec["bytes_per_launch"]
+    except (OSError, ValueError, KeyError):
+        traffic = None
     if args.workload in ("cfg2", "cfg2x8"):
         roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic.get((args.workload, dom)),
+                    "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                     "algorithmic_bytes": dom_bytes, "kernel_ms": round(stages[dom], 5),
                     "layer_bytes": b_conv, "layer_GBs": round(b_conv / (ms * 1e-3) / 1e9, 1),
                     "layer_frac": round(b_conv / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
@@ -228,7 +253,8 @@ def main() -> int:
         "config": {"workload": what.format(n=n, M=M), "dataflow": names[flow], "selector": args.dataflow == "auto",
                    "launch": launch},
         "roofline": roofline,
-        "extra": {"eager_ms_per_step": round(eager_ms, 5), "eager_wall_ms_per_step": round(wall_ms, 5),
+        "extra": {"ms_per_step_replays": {k: (round(v, 5) if k != "replays" else v) for k, v in spread.items()},
+                  "eager_ms_per_step": round(eager_ms, 5), "eager_wall_ms_per_step": round(wall_ms, 5),
                   "map_build_ms": round(map_ms, 4),
                   "stage_ms": {k: round(v, 5) for k, v in stages.items()},
                   "other_dataflows_ms": {k: round(v, 5) for k, v in others.items()}},
@@ -278,8 +304,8 @@ def main() -> int:
         result["extra"]["cfg4_minkunet"]["training_step_ms"] = round(ev_ms(train_step, 5, 2), 3)
         del train_model
 
-    # ---- configurations 1, 3 and 5 (opt-in) ------------------------------------------------------------
-    if args.all_configs:
+    # ---- configurations 1, 3 and 5 ----------------------------------------------------------------------
+    if not args.no_other_configs and args.workload == "cfg2":
         import pcengine_amd as pe
         from pcengine_amd import nets
         # cfg1: fp32, C 16 -> 16, ~20 k voxels
@@ -294,6 +320,12 @@ def main() -> int:
         t1 = timer(lambda: backend.conv_forward(f1, w1, km1, fl1, buffer=b1, out=o1), 100, 10)[0]
         result["extra"]["cfg1"] = {"voxels": int(len(c1)), "pairs": int(km1.M), "dtype": "f32", "dataflow": names[fl1],
                                    "layer_ms": round(t1, 5)}
+        if not args.no_cpu:     # configuration 1 is the reference's CPU-runnable case: the torch CPU path beside it
+            from oracle import cpu_path
+            m1, v1, _, _ = cpu_path.time_layer(c1, f1.cpu().numpy(), w1.cpu().numpy(), ks, warmup=3, runs=10)
+            result["extra"]["cfg1"]["cpu_map_build_ms"] = round(m1, 3)
+            result["extra"]["cfg1"]["cpu_conv_ms"] = round(v1, 3)
+            result["extra"]["cfg1"]["cpu_threads"] = torch.get_num_threads()
         # cfg3: k2s2 down 64 -> 128 on the cfg2 cloud, transposed k2s2 128 -> 64 back
         g3 = [(c - 1) // 2 for c in cmax]
         km3 = backend.build_kernel_map(cd, (2, 2, 2), (2, 2, 2), (0, 0, 0), [0, 0, 0], g3, False, want_csr=True,
@@ -336,16 +368,18 @@ def main() -> int:
     # ---- CPU baseline: the oracle's torch path on this box's host cores, same workload ---------
     if not args.no_cpu:
         from oracle import cpu_path, oracle as orc
-        cores = min(os.cpu_count() or 1, 16)
+        # threads: what torch was given on this host (OMP_NUM_THREADS bounds a one-GPU box's share of the cores),
+        # never more than the machine has
+        cores = max(1, min(torch.get_num_threads(), os.cpu_count() or 1))
         torch.set_num_threads(cores)
         f16 = fd.float().cpu().numpy()
         w16 = wd.float().cpu().numpy()
-        cpu_map_ms, cpu_conv_ms, cpu_out, _ = cpu_path.time_layer(coords, f16, w16, ks, warmup=2, runs=5)
+        cpu_map_ms, cpu_conv_ms, cpu_out, _ = cpu_path.time_layer(coords, f16, w16, ks, warmup=3, runs=10)
         gpu_out = step().float().cpu().numpy()
         result["cpu_baseline"] = {"value": round(cpu_conv_ms, 3), "unit": "ms", "cores": cores, "kind": "port",
                                   "sample": f"the full {args.workload} layer (same N, M, C), fp32 on fp16-rounded inputs, "
-                                            "median of 5 runs after 2 warm-ups; map build timed separately",
-                                  "map_build_ms": round(cpu_map_ms, 3)}
+                                            "median of 10 runs after 3 warm-ups; map build timed separately",
+                                  "map_build_ms": round(cpu_map_ms, 3), "host_cpus": os.cpu_count()}
         result["extra"]["rel_l2_vs_cpu"] = float(orc.rel_l2(gpu_out, cpu_out))
     print(json.dumps(result))
     return 0

@@ -1,9 +1,17 @@
 /* pcengine_amd — C ABI of the MI355X (gfx950) sparse-convolution hot path.
  *
  * Plain pointers and sizes only; every pointer named "device" is HIP device memory owned by the
- * caller.  The library keeps no state between calls, allocates no device memory, and launches all
- * work on the stream it is given.  Functions return PCE_OK (0) or an error code; the text of the
- * last error on the calling thread is returned by pce_last_error().
+ * caller.  The library allocates no device memory and launches all work on the stream it is given.
+ * Functions return PCE_OK (0) or an error code; the text of the last error on the calling thread is
+ * returned by pce_last_error().
+ *
+ * State the library keeps between calls: (1) per device, a ring of eight pinned host blocks (32 KB
+ * each, allocated on the first pce_kmap_build / pce_kmap_build_batch on that device, never freed)
+ * from which the descriptors of a batched map build are copied to the device, guarded by one mutex,
+ * so calls from several host threads are safe; (2) the thread-local text of pce_last_error().
+ * Nothing else: no caches, no tables, no switches.  (The stage mask a benchmark uses to time one
+ * kernel of a dataflow alone exists only in the separately built measurement library, see
+ * pcengine_amd_measure.h.)
  *
  * These entry points are what the reference's five pybind functions
  * (backend/pybind_cuda.cpp:8-14) decompose into:
@@ -16,7 +24,9 @@
  *       -> pce_conv_fwd_fod
  *   conv_fwd_d1_cuda = ConvolutionForwardD1 (backend/spconv.h:11-25, backend/spconv.cu:24-222)
  *       -> pce_conv_fwd_gms
- *   conv_bwd_d1_cuda = ConvolutionBackwardD1 (backend/spconv.h:43-58): training, not provided.
+ *   conv_bwd_d1_cuda = ConvolutionBackwardD1 (backend/spconv.h:43-58, backend/spconv.cu:400-629)
+ *       -> pce_conv_wgrad (kernel gradient) + pce_conv_fwd_fod over the swapped map with the
+ *          per-offset transposed kernel (feature gradient)
  */
 #ifndef PCENGINE_AMD_H
 #define PCENGINE_AMD_H
@@ -67,17 +77,6 @@ typedef struct pce_geom {
 
 int pce_version(void);
 const char *pce_last_error(void);
-
-/* Measurement aid: bit i of the mask enables stage i of the forward entry points below
- * (0: centre GEMM or zero-fill, 1: pair / tile kernel, 2: convert or scatter, 3: gather), so a
- * benchmark can time one kernel of a dataflow alone.  Bits 4 and 5 choose between kernel families
- * for A/B measurements: 4 = the deferred-scatter forms with a pair-driven row sum (cleared: centre
- * GEMM with the partial-row sum in its epilogue), 5 = the pipelined tile kernel for wide fp16 layers
- * (cleared: the single-stage tile kernel), 6 = pair tiles and centre GEMM of a wide deferred-scatter
- * layer in one launch (cleared: two launches), 9 = the pipelined output-stationary kernel for wide
- * fp16 layers of few tiles (cleared: the single-stage tile kernel).  Default: all bits set.
- * Process-wide. */
-void pce_set_stage_mask(uint32_t mask);
 
 /* ---- coordinate hash table: open addressing on the packed (b,x,y,z) 64-bit key ------------- */
 

@@ -11,6 +11,7 @@ from ctypes import c_int32, c_int64, c_void_p, c_char_p, POINTER, Structure
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libpcengine_amd.so")
+MEASURE_LIB_PATH = os.path.join(_HERE, "lib", "libpcengine_amd_measure.so")
 
 PCE_OK, PCE_EINVAL, PCE_ECAPACITY, PCE_EHIP, PCE_EWORKSPACE, PCE_ECOORD = range(6)
 PCE_F16, PCE_F32, PCE_F64 = 0, 1, 2
@@ -57,7 +58,6 @@ class PCEError(RuntimeError):
 _SIGNATURES = {
     "pce_version": (c_int32, []),
     "pce_last_error": (c_char_p, []),
-    "pce_set_stage_mask": (None, [ctypes.c_uint32]),
     "pce_hash_slots": (c_int64, [c_int64]),
     "pce_hash_table_bytes": (c_int64, [c_int64]),
     "pce_hash_build": (c_int32, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p]),
@@ -104,11 +104,22 @@ _SIGNATURES = {
     "pce_select_dataflow": (c_int32, [c_int64, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32]),
 }
 
+# only in the measurement build (include/pcengine_amd_measure.h)
+_MEASURE_SIGNATURES = {"pce_set_stage_mask": (None, [ctypes.c_uint32])}
+
 _lib = None
+_measure_lib = None
 
 
 def exported_names():
     return sorted(_SIGNATURES)
+
+
+def _attach(lib: ctypes.CDLL, signatures: dict) -> None:
+    for name, (res, args) in signatures.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
 
 
 def load() -> ctypes.CDLL:
@@ -121,12 +132,33 @@ def load() -> ctypes.CDLL:
             f"{LIB_PATH} is missing: build it with `python -m pcengine_amd.build` "
             "(hipcc, --offload-arch=gfx950).  pcengine_amd has no other compute path.")
     lib = ctypes.CDLL(LIB_PATH)
-    for name, (res, args) in _SIGNATURES.items():
-        fn = getattr(lib, name)
-        fn.restype = res
-        fn.argtypes = args
+    _attach(lib, _SIGNATURES)
     _lib = lib
     return lib
+
+
+class measurement_build:
+    """Context manager for benchmarks and A/B tests: inside it every operator of the package runs on
+    libpcengine_amd_measure.so (the same kernels, plus ``pce_set_stage_mask``); on exit the mask is reset
+    and the product library is back.  Not for concurrent use."""
+
+    def __enter__(self) -> ctypes.CDLL:
+        global _lib, _measure_lib
+        load()
+        if _measure_lib is None:
+            if not os.path.exists(MEASURE_LIB_PATH):
+                raise PCEError(f"{MEASURE_LIB_PATH} is missing: build it with `python -m pcengine_amd.build`")
+            m = ctypes.CDLL(MEASURE_LIB_PATH)
+            _attach(m, _SIGNATURES)
+            _attach(m, _MEASURE_SIGNATURES)
+            _measure_lib = m
+        self._product, _lib = _lib, _measure_lib
+        return _measure_lib
+
+    def __exit__(self, *exc) -> None:
+        global _lib
+        _measure_lib.pce_set_stage_mask(0xFFFFFFFF)
+        _lib = self._product
 
 
 def check(rc: int) -> None:

@@ -479,9 +479,9 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
         raise ValueError("Input feature size and kernel size mismatch")   # backend/spconv.cu:38-40
     if kv != km.kv:
         raise ValueError(f"kernel volume {kv} does not match the map ({km.kv})")
-    if transposed and km.subm:
-        # a submanifold map is its own mirror image: pair (i, o, kp) exists iff (o, i, kv-1-kp) does, so the
-        # transposed layer is the plain layer with the offsets of the kernel reversed
+    if transposed and km.subm and all(k % 2 == 1 for k in km.ks):
+        # a submanifold map with odd kernel sizes is its own mirror image: pair (i, o, kp) exists iff
+        # (o, i, kv-1-kp) does, so the transposed layer is the plain layer with the offsets of the kernel reversed
         weight, packed, transposed = weight.flip(0).contiguous(), None, False
         packed = pack_weights(weight)
     n_in, n_out = (km.n_out, km.n_in) if transposed else (km.n_in, km.n_out)
@@ -537,6 +537,14 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
     elif dataflow == DATAFLOW_OS:
         ensure_nbr(km, transposed)
         nbr = km.nbr_in if transposed else km.nbr_out
+        if transposed and km.subm:
+            # submanifold layer with an even kernel size (no mirror symmetry): the input-major table is the probe
+            # result, whose centre row is empty; the transposed layer needs the identity there
+            if getattr(km, "_nbr_in_t", None) is None:
+                t = km.nbr_in.clone().view(km.kv, km.n_in)
+                t[_mid(km.ks)] = torch.arange(km.n_in, dtype=torch.int32, device=t.device)
+                km._nbr_in_t = t.view(-1)
+            nbr = km._nbr_in_t
         _lib.check(lib.pce_conv_fwd_os(feats.data_ptr(), weight.data_ptr(), _ptr(packed), out.data_ptr(), dt, n_in, n_out,
                                        c_in, c_out, kv, nbr.data_ptr(), epi, s))
     else:

@@ -960,8 +960,15 @@ static bool wave_gemm_ok(const TileArgs &a, int elem_size) {
   return elem_size == 2 && a.Wp && a.a_vec && a.o_vec && a.c_in % 16 == 0 && a.c_in <= 64 && a.c_out <= 64;
 }
 
+// Stage selection exists in the measurement build only (libpcengine_amd_measure.so, compiled with
+// -DPCE_MEASURE): there a benchmark can run one kernel of a dataflow alone or pick a kernel family.  The
+// product library compiles every test below to `true` and keeps no such state.
+#ifdef PCE_MEASURE
 static unsigned g_stage_mask = 0xFFFFFFFFu;
 static inline bool stage_on(int bit) { return (g_stage_mask >> bit) & 1u; }
+#else
+static constexpr bool stage_on(int) { return true; }
+#endif
 
 // ---- pipelined tile GEMM for wide fp16 layers ---------------------------------------------------
 // The single-offset modes (pair tiles, centre / dense GEMM) at wide channels: 128 rows x 128 columns
@@ -987,27 +994,43 @@ __device__ __forceinline__ u32x4 load16_untracked(const void *p) {
   return v;
 }
 
-// Waits until at most `leave_in_flight` loads are outstanding, joins the workgroup barrier and only then
+// Every wavefront of the pipelined kernels issues, per K chunk, exactly PIPE_CHUNK_VMEM vector-memory
+// operations: PIPE_ROW_LOADS untracked 16-byte loads of its own rows' fragments (pipe_load_rows) and
+// PIPE_W_LOADS global -> LDS copies of its share of the weight chunk (pipe_issue_weights), both issued
+// unconditionally.  Vector-memory operations complete in issue order, so "at most c * PIPE_CHUNK_VMEM
+// outstanding" means "everything but the youngest c chunks has landed": the hand-written wait immediates
+// are derived from these constants and nothing else.  A wavefront that issued fewer operations for some
+// chunk would pass the wait early and read fragment registers before their loads have written them (an
+// ablation build that dropped the weight copies did exactly that and took a memory fault).
+constexpr int PIPE_ROW_LOADS = PIPE_KC / 16;   // one 16-byte load per lane covers k = 16 s2 + 8 g .. + 7 of the lane's row
+constexpr int PIPE_W_LOADS = 2;                // 64 fragments of 16 bytes per instruction and wavefront
+constexpr int PIPE_CHUNK_VMEM = PIPE_ROW_LOADS + PIPE_W_LOADS;
+static_assert(PIPE_ROW_LOADS == 2, "pipe_wait_copy moves exactly two landed fragments");
+static_assert(4 * PIPE_W_LOADS * 64 == (PIPE_KC / 8) * 128, "the copies of four wavefronts cover one 32 x 128 weight chunk exactly");
+static_assert(2 * 2 * PIPE_CHUNK_VMEM <= 63, "vmcnt is a 6-bit counter");
+
+// Waits until at most CNT vector-memory operations are outstanding, joins the workgroup barrier and only then
 // reads the two fragments: the copies are made inside the same statement, after the wait, so that no read
 // of a fragment register can be scheduled before its load has landed.
-#define PCE_PIPE_WAIT_COPY(CNT_)                                                                              \
-  asm volatile("s_waitcnt vmcnt(" #CNT_ ")\n\ts_barrier\n\t"                                                  \
-               "v_mov_b32 %0, %8\n\tv_mov_b32 %1, %9\n\tv_mov_b32 %2, %10\n\tv_mov_b32 %3, %11\n\t"           \
-               "v_mov_b32 %4, %12\n\tv_mov_b32 %5, %13\n\tv_mov_b32 %6, %14\n\tv_mov_b32 %7, %15"              \
-               : "=&v"(o0.x), "=&v"(o0.y), "=&v"(o0.z), "=&v"(o0.w), "=&v"(o1.x), "=&v"(o1.y), "=&v"(o1.z),    \
-                 "=&v"(o1.w)                                                                                  \
-               : "v"(f0.x), "v"(f0.y), "v"(f0.z), "v"(f0.w), "v"(f1.x), "v"(f1.y), "v"(f1.z), "v"(f1.w)       \
-               : "memory")
-__device__ __forceinline__ void pipe_wait_barrier(int leave_in_flight, const u32x4 &f0, const u32x4 &f1, u32x4 &o0,
+template <int CNT>
+__device__ __forceinline__ void pipe_wait_copy(const u32x4 &f0, const u32x4 &f1, u32x4 &o0, u32x4 &o1) {
+  static_assert(CNT % PIPE_CHUNK_VMEM == 0, "waits are counted in whole chunks");
+  asm volatile("s_waitcnt vmcnt(%16)\n\ts_barrier\n\t"
+               "v_mov_b32 %0, %8\n\tv_mov_b32 %1, %9\n\tv_mov_b32 %2, %10\n\tv_mov_b32 %3, %11\n\t"
+               "v_mov_b32 %4, %12\n\tv_mov_b32 %5, %13\n\tv_mov_b32 %6, %14\n\tv_mov_b32 %7, %15"
+               : "=&v"(o0.x), "=&v"(o0.y), "=&v"(o0.z), "=&v"(o0.w), "=&v"(o1.x), "=&v"(o1.y), "=&v"(o1.z), "=&v"(o1.w)
+               : "v"(f0.x), "v"(f0.y), "v"(f0.z), "v"(f0.w), "v"(f1.x), "v"(f1.y), "v"(f1.z), "v"(f1.w), "n"(CNT)
+               : "memory");
+}
+// `chunks_in_flight`: how many of the youngest chunks' operations may still be outstanding (0, 1 or 2)
+__device__ __forceinline__ void pipe_wait_barrier(int chunks_in_flight, const u32x4 &f0, const u32x4 &f1, u32x4 &o0,
                                                   u32x4 &o1) {
-  // loads complete in issue order: leaving the youngest ones in flight (the feature fragments and the
-  // weight chunk requested one round ago) still guarantees that the chunk about to be used has landed
-  if (leave_in_flight >= 8)
-    PCE_PIPE_WAIT_COPY(8);
-  else if (leave_in_flight >= 4)
-    PCE_PIPE_WAIT_COPY(4);
+  if (chunks_in_flight >= 2)
+    pipe_wait_copy<2 * PIPE_CHUNK_VMEM>(f0, f1, o0, o1);
+  else if (chunks_in_flight == 1)
+    pipe_wait_copy<PIPE_CHUNK_VMEM>(f0, f1, o0, o1);
   else
-    PCE_PIPE_WAIT_COPY(0);
+    pipe_wait_copy<0>(f0, f1, o0, o1);
 }
 // two more fragments that the same wait has covered: volatile statements keep their order, so these copies
 // stay behind the wait of the pipe_wait_barrier in front of them
@@ -1018,15 +1041,14 @@ __device__ __forceinline__ void pipe_copy_landed(const u32x4 &f0, const u32x4 &f
                : "v"(f0.x), "v"(f0.y), "v"(f0.z), "v"(f0.w), "v"(f1.x), "v"(f1.y), "v"(f1.z), "v"(f1.w)
                : "memory");
 }
-#undef PCE_PIPE_WAIT_COPY
 
 // this wavefront's quarter of the weight chunk (k0 .. k0+31, columns n0 .. n0+127) -> LDS stage
 __device__ __forceinline__ void pipe_issue_weights(const half_t *Wk, int k0, int n0, int n_pad, half8 *stage, int wave,
                                                    int lane) {
   // stage layout [k8 = 0..3][n = 0..127] of 16-byte fragments; one instruction moves 64 of them
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    int part = wave * 2 + i;          // 0..7: k8 = part / 2, column half = part % 2
+  for (int i = 0; i < PIPE_W_LOADS; ++i) {
+    int part = wave * PIPE_W_LOADS + i;          // 0..7: k8 = part / 2, column half = part % 2
     int k8 = part >> 1, nh = part & 1;
     int n = n0 + nh * 64 + lane;
     n = n < n_pad ? n : n_pad - 1;    // columns past the padded width are never stored: any valid address will do
@@ -1040,10 +1062,10 @@ __device__ __forceinline__ void pipe_issue_weights(const half_t *Wk, int k0, int
 
 // always issued (row 0 stands in for a missing row; the caller zeroes it when the fragment is taken into
 // use): the wait before the barrier counts the loads of a round
-__device__ __forceinline__ void pipe_load_rows(u32x4 (&raw)[2], const half_t *A, int arow, int c_in, int k0, int g) {
+__device__ __forceinline__ void pipe_load_rows(u32x4 (&raw)[PIPE_ROW_LOADS], const half_t *A, int arow, int c_in, int k0, int g) {
   int r = arow >= 0 ? arow : 0;
 #pragma unroll
-  for (int s2 = 0; s2 < 2; ++s2) raw[s2] = load16_untracked(A + (long long)r * c_in + k0 + s2 * 16 + g * 8);
+  for (int s2 = 0; s2 < PIPE_ROW_LOADS; ++s2) raw[s2] = load16_untracked(A + (long long)r * c_in + k0 + s2 * 16 + g * 8);
 }
 
 // PMODE = MODE_DENSE or MODE_FOD_BUF: every tile is of that kind and `c` is not read.  PMODE = PIPE_BOTH:
@@ -1099,7 +1121,7 @@ __global__ void __launch_bounds__(256, 4) pipe_gemm_kernel(TileArgs a, TileArgs 
     for (int j = 0; j < 16; ++j) acc[nb][j] = 0.f;
 
   // prologue: weight chunks 0 and 1, feature chunks 0 and 1 (issue order: W0, A0, W1, A1)
-  u32x4 raw[2][2];
+  u32x4 raw[2][PIPE_ROW_LOADS];
   pipe_issue_weights(Wk, 0, n0, a.n_pad, lds, wave, lane);
   pipe_load_rows(raw[0], A, arow, a.c_in, 0, g);
   if (kch > 1) {
@@ -1116,7 +1138,8 @@ __global__ void __launch_bounds__(256, 4) pipe_gemm_kernel(TileArgs a, TileArgs 
   {                                                                                                        \
     const int t = (T_);                                                                                    \
     u32x4 landed[2];                                                                                       \
-    pipe_wait_barrier(4 * (t + 1 < kch), raw[SLOT_][0], raw[SLOT_][1], landed[0], landed[1]);              \
+    /* only the operations of chunk t+1 (issued one round ago) may still be outstanding */                  \
+    pipe_wait_barrier(t + 1 < kch ? 1 : 0, raw[SLOT_][0], raw[SLOT_][1], landed[0], landed[1]);             \
     half8 af[2];                                                                                           \
     _Pragma("unroll") for (int s2 = 0; s2 < 2; ++s2)                                                       \
         af[s2] = arow >= 0 ? __builtin_bit_cast(half8, landed[s2]) : zero;                                 \
@@ -1253,7 +1276,7 @@ __global__ void __launch_bounds__(256, SUB == 1 ? 3 : 2) os_pipe_kernel(TileArgs
   // issue cursor (two steps ahead of the consume cursor): offset, chunk, LDS stage
   int ikp = active ? __ffs(active) - 1 : -1, it = 0, ist = 0;
   int ckp = ikp, ct = 0, cst = 0;
-  u32x4 raw[2][SUB][2];
+  u32x4 raw[2][SUB][PIPE_ROW_LOADS];
   const half8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
   int carow[2] = {-1, -1};   // the row whose fragments sit in raw[slot]
 #define OSP_ISSUE(SLOT_)                                                                                     \
@@ -1279,8 +1302,8 @@ __global__ void __launch_bounds__(256, SUB == 1 ? 3 : 2) os_pipe_kernel(TileArgs
   {                                                                                                          \
     const int r = (R_);                                                                                      \
     u32x4 landed[SUB][2];                                                                                    \
-    /* everything older than the loads of step r+1 (issued one step ago, 4 SUB of them) has landed */       \
-    pipe_wait_barrier(4 * SUB * (r + 1 < rounds), raw[SLOT_][0][0], raw[SLOT_][0][1], landed[0][0], landed[0][1]); \
+    /* everything older than the SUB chunks of step r+1 (issued one step ago) has landed */                 \
+    pipe_wait_barrier(r + 1 < rounds ? SUB : 0, raw[SLOT_][0][0], raw[SLOT_][0][1], landed[0][0], landed[0][1]); \
     if (SUB == 2) pipe_copy_landed(raw[SLOT_][SUB - 1][0], raw[SLOT_][SUB - 1][1], landed[SUB - 1][0], landed[SUB - 1][1]); \
     half8 af[SUB][2];                                                                                        \
     const int arow_c = carow[SLOT_];                                                                         \
@@ -1703,7 +1726,9 @@ __global__ void zero_f32_kernel(float *p, long long n) {
   }
 }
 
+#ifdef PCE_MEASURE
 extern "C" void pce_set_stage_mask(uint32_t mask) { g_stage_mask = mask; }
+#endif
 
 static int pow2_at_least(int v) {
   int p = 1;

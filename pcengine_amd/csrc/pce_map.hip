@@ -277,6 +277,7 @@ struct GeomDev {
   int bump[3];  // +1 on odd kernel sizes > 1 for strided layers (backend/hash.cuh:235-237)
   int half[3];  // (ks-1)/2
   int subm, kv, mid;
+  int sym;  // submanifold layer whose kernel sizes are all odd: pair (i,o,kp) <=> pair (o,i,kv-1-kp)
 };
 
 static int make_geom(const pce_geom_t *g, GeomDev *d) {
@@ -296,6 +297,7 @@ static int make_geom(const pce_geom_t *g, GeomDev *d) {
   }
   if (kv > 1024) PCE_FAIL(PCE_ECAPACITY, "kernel volume %lld exceeds 1024", (long long)kv);
   d->subm = g->subm ? 1 : 0;
+  d->sym = (g->subm && g->ks[0] % 2 == 1 && g->ks[1] % 2 == 1 && g->ks[2] % 2 == 1) ? 1 : 0;
   d->kv = (int)kv;
   d->mid = d->half[0] * g->ks[1] * g->ks[2] + d->half[1] * g->ks[2] + d->half[2];
   if (g->subm && (g->stride[0] != 1 || g->stride[1] != 1 || g->stride[2] != 1))
@@ -936,7 +938,7 @@ struct KmapLayout {
   int64_t off_table, off_dense, off_seg, off_scan, off_orank, off_irank, off_desc, total;
 };
 
-static void kmap_layout(int64_t n_in, int64_t n_out, int kv, int want_csr, int subm, KmapLayout *L) {
+static void kmap_layout(int64_t n_in, int64_t n_out, int kv, int want_csr, int sym, KmapLayout *L) {
   L->slots = pce_hash_slots(n_out);
   L->nseg = pce_div_up(n_in, PCE_WAVE);
   L->scan_len = (int64_t)kv * L->nseg + 1;
@@ -950,7 +952,7 @@ static void kmap_layout(int64_t n_in, int64_t n_out, int kv, int want_csr, int s
   L->off_scan = o;
   o += pce_align_up((scan_tmp_ints(L->scan_len) + scan_tmp_ints(n_in + 1) + scan_tmp_ints(n_out + 1)) * 4, 256);
   L->off_orank = o;
-  if (want_csr && !subm) o += pce_align_up((int64_t)kv * n_out * 4, 256);
+  if (want_csr && !sym) o += pce_align_up((int64_t)kv * n_out * 4, 256);
   L->off_irank = o;
   if (want_csr) o += pce_align_up((int64_t)kv * n_in * 4, 256);
   L->off_desc = o;
@@ -1040,9 +1042,11 @@ __global__ void __launch_bounds__(256) batch_insert_kernel(const ProbDev *__rest
 //   submanifold: out = in - d(kp)          (pair (i,o,kp) <=> coords[i] == coords[o] + d(kp))
 //   strided:     out = (in - d(kp) + pad) / stride when it divides
 // dense[kp*n_in + i] = output row or -1.
-// A submanifold map is symmetric: pair (i,o,kp) <=> pair (o,i,kv-1-kp).  Only the offsets below the
-// centre are probed; a hit also writes the mirrored entry dense[(kv-1-kp)*n + o] = i.  The rows of
-// dense from the centre upwards are pre-filled with -1.
+// A submanifold map with odd kernel sizes is symmetric: pair (i,o,kp) <=> pair (o,i,kv-1-kp), because
+// d(kv-1-kp) == -d(kp).  Only the offsets below the centre are probed; a hit also writes the mirrored
+// entry dense[(kv-1-kp)*n + o] = i.  The rows of dense from the centre upwards are pre-filled with -1.
+// With an even kernel size on some axis the offsets are not mirror images of each other (2x2x2: d in
+// {0,1}^3, backend/hash.cuh:147-149): every offset but the centre is probed, as the reference does.
 __global__ void __launch_bounds__(256) kmap_query_kernel(const ProbDev *__restrict__ P, JobList jl) {
   const Job &job = find_job(jl, blockIdx.x);
   const ProbDev &q = P[job.prob];
@@ -1058,7 +1062,7 @@ __global__ void __launch_bounds__(256) kmap_query_kernel(const ProbDev *__restri
     q.status[0] = 1;
     live = false;
   }
-  const int kend = g.subm ? g.mid : g.kv;
+  const int kend = g.sym ? g.mid : g.kv;
   OffsetIter it;
   it.init();
   for (int kp0 = 0; kp0 < kend; kp0 += PROBE_BATCH) {
@@ -1067,7 +1071,7 @@ __global__ void __launch_bounds__(256) kmap_query_kernel(const ProbDev *__restri
     bool ok[PROBE_BATCH];
 #pragma unroll
     for (int j = 0; j < PROBE_BATCH; ++j) {
-      ok[j] = live && kp0 + j < kend;
+      ok[j] = live && kp0 + j < kend && !(g.subm && kp0 + j == g.mid);   // the centre offset is never probed
       int ox = 0, oy = 0, oz = 0;
       if (ok[j]) {
         if (g.subm) {
@@ -1112,7 +1116,7 @@ __global__ void __launch_bounds__(256) kmap_query_kernel(const ProbDev *__restri
       }
       if (i < n_in) {
         dense[(long long)kp * n_in + i] = res;
-        if (g.subm && res >= 0) dense[(long long)(g.kv - 1 - kp) * n_in + res] = (int)i;
+        if (g.sym && res >= 0) dense[(long long)(g.kv - 1 - kp) * n_in + res] = (int)i;
       }
     }
   }
@@ -1224,7 +1228,7 @@ __global__ void __launch_bounds__(256) kmap_fill_kernel(const ProbDev *__restric
   const Job &job = find_job(jl, blockIdx.x);
   const ProbDev &q = P[job.prob];
   const long long n_in = q.n_in, n_out = q.n_out, nseg = q.nseg;
-  const int kv = q.g.kv, subm = q.g.subm, mid = q.g.mid;
+  const int kv = q.g.kv, subm = q.g.subm, sym = q.g.sym, mid = q.g.mid;
   const int *__restrict__ dense = q.dense;
   const int *__restrict__ segoff = q.seg;
   int *__restrict__ imap = q.imap;
@@ -1242,7 +1246,7 @@ __global__ void __launch_bounds__(256) kmap_fill_kernel(const ProbDev *__restric
       int kp = kp0 + j;
       bool in = kp < kv;
       vv[j] = (live && in) ? dense[(long long)kp * n_in + i] : -1;
-      mm[j] = (live && in && nbr_out && subm && kp != mid) ? dense[(long long)(kv - 1 - kp) * n_in + i] : -1;
+      mm[j] = (live && in && nbr_out && sym && kp != mid) ? dense[(long long)(kv - 1 - kp) * n_in + i] : -1;
       base[j] = (in && seg < nseg) ? segoff[(long long)kp * nseg + seg] : 0;
       first[j] = in ? segoff[(long long)kp * nseg] : 0;
     }
@@ -1257,14 +1261,15 @@ __global__ void __launch_bounds__(256) kmap_fill_kernel(const ProbDev *__restric
         int p = base[j] + __popcll(bal & lanemask_lt());
         imap[p] = (int)i;
         omap[p] = v;
-        if (nbr_out && !subm) nbr_out[(long long)kp * n_out + v] = (int)i;
+        if (nbr_out && !sym) nbr_out[(long long)kp * n_out + v] = (int)i;
         rank = p - first[j];
         if (irank && rank >= PCE_CSR_CODE) q.status[2] = 1;
         if (orank) orank[(long long)kp * n_out + v] = rank;
       }
       if (irank && live) irank[(long long)kp * n_in + i] = rank;
-      if (nbr_out && subm && live)  // nbr_out[kp][o] = input of the pair whose output is o = mirrored probe result
+      if (nbr_out && sym && live)  // nbr_out[kp][o] = input of the pair whose output is o = mirrored probe result
         nbr_out[(long long)kp * n_out + i] = kp == mid ? (int)i : mm[j];
+      if (nbr_out && subm && !sym && live && kp == mid) nbr_out[(long long)kp * n_out + i] = (int)i;
     }
   }
 }
@@ -1272,7 +1277,7 @@ __global__ void __launch_bounds__(256) kmap_fill_kernel(const ProbDev *__restric
 // CSR-coded views.  Entries of every row in ascending offset order, code = kp * PCE_CSR_CODE + rank, plus,
 // for every pair (offset kp, rank rk), the slot of its entry: slot_of_pair[kpos[kp] + rk] = position.
 // Jobs of one launch (the kind is uniform over a workgroup):
-//   JOB_CSR_SUBM      submanifold map, both views in one pass: the input-side entry of row r at offset kp
+//   JOB_CSR_SUBM      symmetric submanifold map (odd kernel sizes), both views in one pass: the input-side entry of row r at offset kp
 //                     is the pair (r, dense[kp][r], kp); the output-side entry is the pair
 //                     (dense[kv-1-kp][r], r, kp), whose rank is read from the rank table at its input row.
 //                     Both views have the same row pointers.
@@ -1466,7 +1471,7 @@ extern "C" int pce_kmap_build_batch(const pce_kmap_problem_t *probs, int32_t n_p
     if ((int64_t)q.g.kv * n_in >= (1ll << 31) || (int64_t)q.g.kv * n_out >= (1ll << 31))
       PCE_FAIL(PCE_ECAPACITY, "pce_kmap_build: kv*n exceeds int32 pair indexing");
     KmapLayout L;
-    kmap_layout(n_in, n_out, q.g.kv, want_csr, q.g.subm, &L);
+    kmap_layout(n_in, n_out, q.g.kv, want_csr, q.g.sym, &L);
     if (u.ws_bytes < L.total) PCE_FAIL(PCE_EWORKSPACE, "pce_kmap_build: workspace %lld < %lld", (long long)u.ws_bytes, (long long)L.total);
     char *w = (char *)u.ws;
     q.in_coords = (const int4 *)u.in_coords;
@@ -1478,7 +1483,7 @@ extern "C" int pce_kmap_build_batch(const pce_kmap_problem_t *probs, int32_t n_p
     q.slots = (unsigned long long)L.slots;
     q.dense = u.nbr_in ? u.nbr_in : (int *)(w + L.off_dense);  // the input-major table is the probe result itself
     q.irank = want_csr ? (int *)(w + L.off_irank) : nullptr;
-    q.orank = (want_csr && !q.g.subm) ? (int *)(w + L.off_orank) : nullptr;
+    q.orank = (want_csr && !q.g.sym) ? (int *)(w + L.off_orank) : nullptr;
     q.seg = (int *)(w + L.off_seg);
     q.imap = u.imap;
     q.omap = u.omap;
@@ -1496,7 +1501,7 @@ extern "C" int pce_kmap_build_batch(const pce_kmap_problem_t *probs, int32_t n_p
     q.want_csr = want_csr;
     // 1. table over the output coordinates (for a submanifold layer these are the input coordinates)
     add_fill(q.table, L.slots * 4);
-    if (q.g.subm) {
+    if (q.g.sym) {
       // rows of the probe table that the mirrored writes only touch on a hit (and the centre row)
       add_fill(q.dense + (int64_t)q.g.mid * n_in, (int64_t)(q.g.kv - q.g.mid) * n_in);
     } else {
@@ -1512,7 +1517,7 @@ extern "C" int pce_kmap_build_batch(const pce_kmap_problem_t *probs, int32_t n_p
     if (want_csr) add_scan(0, q.icsr, n_in + 1, scan_tmp + scan_tmp_ints(L.scan_len));
     add_job(ST_FILL, p, 0, n_in);
     // 5. CSR-coded views
-    if (want_csr && q.g.subm) {
+    if (want_csr && q.g.sym) {
       add_job(ST_CSR_A, p, JOB_CSR_SUBM, n_in + 1);
     } else if (want_csr) {
       add_job(ST_CSR_A, p, JOB_CSR_IN, n_in);
@@ -1526,7 +1531,7 @@ extern "C" int pce_kmap_build_batch(const pce_kmap_problem_t *probs, int32_t n_p
   if (total_blocks >= (1ll << 31)) PCE_FAIL(PCE_ECAPACITY, "pce_kmap_build_batch: the batch exceeds the grid limit");
   // one copy carries the descriptors; they live in the first problem's workspace
   KmapLayout L0;
-  kmap_layout(probs[0].n_in, probs[0].n_out, img.prob[0].g.kv, img.prob[0].want_csr, img.prob[0].g.subm, &L0);
+  kmap_layout(probs[0].n_in, probs[0].n_out, img.prob[0].g.kv, img.prob[0].want_csr, img.prob[0].g.sym, &L0);
   char *desc = (char *)probs[0].ws + L0.off_desc;
   if (int rc = desc_upload(img, desc, s)) return rc;
   const BatchImage *D = (const BatchImage *)desc;

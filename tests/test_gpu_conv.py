@@ -89,18 +89,15 @@ def test_narrow_fp16_layers_barrier_free_kernel(c_in, c_out):
     """fp16 rows of at most 64 channels with packed weights take the wavefront-per-chunk kernel in the
     deferred-scatter dataflow: submanifold (pairs + centre in one launch), strided and transposed."""
     from pcengine_amd import _lib
-    lib = _lib.load()
     coords = synth.random_cloud(seed=44, n=12000, extent=30, batches=2)
     fd, wd, ref_map, want = _case(coords, (3, 3, 3), (1, 1, 1), (0, 0, 0), c_in, c_out, torch.float16, seed=6)
     km = gpu_map(coords, (3, 3, 3), want_csr=True)
     pk = backend.pack_weights(wd)
     out = backend.conv_forward(fd, wd, km, DATAFLOW_FDS, packed=pk)
     assert orc.rel_l2(out.double().cpu().numpy(), want) <= 1e-3
-    lib.pce_set_stage_mask(0xFFFFFFFF & ~16)          # the same layer through the workgroup-tile kernels
-    try:
+    with _lib.measurement_build() as mlib:            # the same layer through the workgroup-tile kernels
+        mlib.pce_set_stage_mask(0xFFFFFFFF & ~16)
         old = backend.conv_forward(fd, wd, km, DATAFLOW_FDS, packed=pk)
-    finally:
-        lib.pce_set_stage_mask(0xFFFFFFFF)
     assert orc.rel_l2(old.double().cpu().numpy(), want) <= 1e-3
     # rows without neighbours are the centre GEMM alone and agree bit for bit
     lonely = (km.ocsr[1:] == km.ocsr[:-1])
@@ -407,11 +404,13 @@ def test_transposed_layer_with_clipped_parents_is_routed(c_in, c_out):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
-@pytest.mark.parametrize("ks,c_in,c_out", [((5, 5, 5), 32, 32), ((5, 5, 5), 64, 128), ((5, 3, 1), 16, 24), ((1, 5, 5), 128, 96)])
+@pytest.mark.parametrize("ks,c_in,c_out", [((5, 5, 5), 32, 32), ((5, 5, 5), 64, 128), ((5, 3, 1), 16, 24), ((1, 5, 5), 128, 96),
+                                           ((2, 2, 2), 32, 32), ((2, 3, 3), 64, 128), ((2, 2, 2), 128, 128)])
 def test_large_and_anisotropic_kernels_forward_and_backward(ks, c_in, c_out, dtype):
-    """Kernel volumes beyond what travels in the kernel arguments (5x5x5 = 125 offsets) and anisotropic
-    kernels, every dataflow, forward and both gradients, against the oracle (whose 5-wide offsets follow the
-    reference's rule, backend/hash.cuh:147-149)."""
+    """Kernel volumes beyond what travels in the kernel arguments (5x5x5 = 125 offsets), anisotropic kernels and
+    stride-1 layers with even kernel sizes (whose maps have no mirror symmetry: the feature gradient runs the
+    transposed layer over the swapped map), every dataflow, forward and both gradients, against the oracle
+    (whose offsets follow the reference's rule, backend/hash.cuh:147-149)."""
     coords = synth.random_cloud(seed=48, n=4000, extent=15, batches=2)
     fd, wd, ref_map, want = _case(coords, ks, (1, 1, 1), (0, 0, 0), c_in, c_out, dtype, seed=11)
     km = gpu_map(coords, ks, want_csr=True, want_nbr_in=True)

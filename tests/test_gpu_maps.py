@@ -19,6 +19,8 @@ GEOMS = [
     ((2, 3, 1), (2, 1, 1), (0, 1, 0)),
     ((5, 5, 5), (1, 1, 1), (0, 0, 0)),
     ((1, 1, 1), (2, 2, 2), (0, 0, 0)),
+    ((2, 2, 2), (1, 1, 1), (0, 0, 0)),   # stride 1 with even kernel sizes: the map has no mirror symmetry
+    ((2, 3, 3), (1, 1, 1), (0, 0, 0)),
 ]
 
 

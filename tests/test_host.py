@@ -23,6 +23,16 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), f"{name} is declared but not exported"
     assert declared == set(_lib.exported_names())
     assert lib.pce_version() >= 100
+    # the stage mask of the measurement build is no part of the product library
+    assert not hasattr(lib, "pce_set_stage_mask")
+    extra = open(os.path.join(ROOT, "include", "pcengine_amd_measure.h")).read()
+    extra = re.sub(r"/\*.*?\*/", "", extra, flags=re.S)
+    assert set(re.findall(r"\b(pce_[a-z0-9_]+)\s*\(", extra)) == {"pce_set_stage_mask"}
+    with _lib.measurement_build() as mlib:
+        assert _lib.load() is mlib
+        for name in sorted(declared) + ["pce_set_stage_mask"]:
+            assert hasattr(mlib, name), f"{name} is missing from the measurement build"
+    assert _lib.load() is lib
 
 
 def test_pure_host_entry_points():
@@ -201,6 +211,9 @@ def test_no_kernel_uses_scratch_memory(tmp_path):
             m = re.search(r"Function Name: (\S+)", line)
             if m:
                 name = m.group(1)
+            m = re.search(r"VGPRs Spill: (\d+)", line)
+            if m:
+                assert int(m.group(1)) == 0, f"{name} spills {m.group(1)} vector registers"
             m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", line)
             if m:
                 seen += 1
