@@ -113,3 +113,45 @@ def test_full_size_maps_match_the_frozen_manifest(name):
         assert km.knnz.cpu().tolist() == want["knnz"], key
         assert digest(km.out_coords) == want["out_coords_sha256"], key
         assert digest(km.imap[:km.M], km.omap[:km.M]) == want["pairs_sha256"], key
+
+
+@pytest.mark.parametrize("name", ["cfg4", "cfg5"])
+def test_every_map_of_the_network_pyramid_matches_the_frozen_manifest(name):
+    """The nine maps a MinkUNet-style forward builds on a benchmark cloud (five submanifold 3x3x3 maps, four
+    k2s2 maps between the levels, script/spconv.py:330-372 once per layer geometry): each level's coordinates,
+    per-offset counts and pair lists against the digests of tests/golden/manifest.json, bit for bit.  Every
+    level is built from the coordinates the GPU produced for the level before, with the coordinate bound the
+    front end carries along (script/spconv.py:358-360)."""
+    import hashlib
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "manifest.json")) as f:
+        frozen = json.load(f)[name]
+    coords = {"cfg4": synth.lidar_cloud_100k, "cfg5": synth.indoor_batch}[name]()
+
+    def digest(*tensors):
+        h = hashlib.sha256()
+        for t in tensors:
+            h.update(np.ascontiguousarray(t.cpu().numpy(), dtype="<i4").tobytes())
+        return h.hexdigest()
+
+    def check(km, want, key):
+        assert (km.n_out, km.M, km.qsum) == (want["n_out"], want["pairs"], want["qsum"]), key
+        assert km.knnz.cpu().tolist() == want["knnz"], key
+        assert digest(km.out_coords) == want["out_coords_sha256"], key
+        assert digest(km.imap[:km.M], km.omap[:km.M]) == want["pairs_sha256"], key
+
+    cd = dev_coords(coords)
+    cmax = coords[:, 1:].max(axis=0).tolist()
+    assert len(frozen["pyramid"]) == 5
+    for lv in frozen["pyramid"]:
+        key = (name, lv["level"])
+        assert cd.shape[0] == lv["voxels"] and cmax == lv["coords_max"] and digest(cd) == lv["coords_sha256"], key
+        sub = backend.build_kernel_map(cd, (3, 3, 3), (1, 1, 1), (0, 0, 0), [0, 0, 0], cmax, True, want_csr=True)
+        check(sub, lv["layers"]["k333_s111_p000"], key)
+        if "k222_s222_p000" in lv["layers"]:
+            cmax = backend.strided_coords_max(cmax, (2, 2, 2), (2, 2, 2), (0, 0, 0))
+            down = backend.build_kernel_map(cd, (2, 2, 2), (2, 2, 2), (0, 0, 0), [0, 0, 0], cmax, False, want_csr=True,
+                                            batchsize=frozen["batches"])
+            check(down, lv["layers"]["k222_s222_p000"], key)
+            cd = down.out_coords

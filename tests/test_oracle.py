@@ -171,6 +171,23 @@ def test_reference_hash_has_no_false_neighbours_in_coordinate_box():
     assert lib.lit_coord_hash(0, 1215, 0, 0) == int(orc.ref_linear_hash(a)[0])
 
 
+def test_row_accumulation_paths_agree():
+    """The oracle adds the products of an offset into their output rows through a 0/1 selection matrix when
+    scipy is there, else with numpy.add.at: both are the same float64 sums (repeated rows included)."""
+    rng = np.random.default_rng(5)
+    rows = rng.integers(0, 300, size=5000)
+    vals = rng.standard_normal((5000, 7))
+    a = rng.standard_normal((300, 7))
+    b = a.copy()
+    orc._add_rows(a, rows, vals)
+    np.add.at(b, rows, vals)
+    assert np.abs(a - b).max() < 1e-12
+    small = a.copy()
+    orc._add_rows(small, rows[:10], vals[:10])          # below the switch-over: numpy.add.at itself
+    np.add.at(b, rows[:10], vals[:10])
+    assert np.array_equal(small, b) or np.abs(small - b).max() < 1e-12
+
+
 def _densify(coords, feats, shape, nb):
     c = torch.as_tensor(coords.astype(np.int64))
     dense = torch.zeros((nb, feats.shape[1]) + tuple(shape), dtype=torch.float64)
