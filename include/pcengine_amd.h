@@ -231,6 +231,25 @@ int pce_conv_fwd_fod(const void *in_feats, const void *weight, const void *weigh
                      const int32_t *kpos_dev, const int32_t *qkpos_dev, int64_t qsum,
                      void *ws_dev, int64_t ws_bytes, const pce_epilogue_t *epilogue, pce_stream_t stream);
 
+/* pce_conv_fwd_fod without the workspace argument, for callers that cannot allocate device memory (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid it).  It has no counterpart in the
+ * reference.  The fp32 accumulator of the fp16 dataflow lives in a static device array inside the library,
+ * pce_conv_fod_static_capacity_bytes() = 32 MiB per GPU the library runs on, held until the process ends;
+ * a layer whose accumulator (n_out * c_out * 4 bytes) is larger returns PCE_ECAPACITY.  PCE_F32 needs no
+ * accumulator and has no size limit.  The call allocates nothing (no hipMalloc / hipFree, no allocating
+ * library routine) and clears nothing with hipMemsetAsync: the centre GEMM, or a fill kernel when the layer
+ * has no centre offset, overwrites the accumulator rows before they are added to.  All calls on one GPU share
+ * that GPU's array: calls that overlap in time on one GPU (different streams or host threads) race and
+ * must be serialised by the caller.  Same results as pce_conv_fwd_fod up to the order of its fp32 atomic
+ * additions. */
+int64_t pce_conv_fod_static_capacity_bytes(void);
+int pce_conv_fwd_fod_static(const void *in_feats, const void *weight, const void *weight_packed,
+                            void *out_feats, int32_t dtype,
+                            int64_t n_in, int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv,
+                            int32_t mid, const int32_t *imap_dev, const int32_t *omap_dev,
+                            const int32_t *kpos_dev, const int32_t *qkpos_dev, int64_t qsum,
+                            const pce_epilogue_t *epilogue, pce_stream_t stream);
+
 /* Gather - GEMM - scatter: CSR-coded map; `buffer` holds qsum*(c_in+c_out) elements of dtype
  * (first qsum*c_in gathered inputs, then the GEMM outputs; backend/spconv.cu:121). */
 int pce_conv_fwd_gms(const void *in_feats, const void *weight, const void *weight_packed,

@@ -94,6 +94,9 @@ _SIGNATURES = {
     "pce_pair_route_elems": (c_int64, [c_int64, c_int64]),
     "pce_conv_fwd_fod": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32,
                                    c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, POINTER(Epilogue), c_void_p]),
+    "pce_conv_fod_static_capacity_bytes": (c_int64, []),
+    "pce_conv_fwd_fod_static": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32,
+                                          c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, POINTER(Epilogue), c_void_p]),
     "pce_conv_fwd_gms": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32,
                                    c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64,
                                    POINTER(Epilogue), c_void_p]),

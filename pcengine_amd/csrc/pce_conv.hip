@@ -7,6 +7,8 @@
 // The A operand (feature rows) goes global -> registers with 16-byte loads, one row per lane; only
 // the per-offset weight tile passes through LDS, laid out so that a lane's B fragment is one
 // conflict-free 16-byte read.
+#include <mutex>
+
 #include "pce_common.h"
 
 typedef _Float16 half_t;
@@ -1917,6 +1919,61 @@ extern "C" int pce_conv_fwd_fod(const void *in, const void *w, const void *wp, v
   }
   if (!aligned16(out)) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_fod: output must be 16-byte aligned");
   return fod_impl<float>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, omap, kpos, qkpos, qsum, (float *)out, e, s);
+}
+
+// ---- fetch-on-demand without a workspace argument ---------------------------------------------------
+// For callers that cannot allocate device memory (code under HIP graph capture, serving loops, harnesses
+// that forbid it): the fp32 accumulator of the fp16 dataflow lives in a file-scope device array.  Every GPU
+// the library runs on holds its own copy of the array, at its own address, until the process ends; the
+// address is looked up once per device and that pointer -- never the array's name, which in host code is
+// only a stand-in for the symbol -- is what the kernels receive.
+#define PCE_STATIC_SCRATCH_BYTES (32ll << 20)
+#define PCE_STATIC_MAX_DEVICES 16
+static __device__ __align__(256) unsigned char scratch[PCE_STATIC_SCRATCH_BYTES];
+static void *g_scratch_ptr[PCE_STATIC_MAX_DEVICES];
+static std::mutex g_scratch_mutex;
+
+// device address of this device's copy of `scratch` (looked up on the first call on the device)
+static int static_scratch(void **ptr) {
+  int dev = 0;
+  PCE_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= PCE_STATIC_MAX_DEVICES) PCE_FAIL(PCE_ECAPACITY, "device index %d not supported", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void *p = nullptr;
+    PCE_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) PCE_FAIL(PCE_EHIP, "hipGetSymbolAddress returned a null address for the static scratch array");
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return PCE_OK;
+}
+
+extern "C" int64_t pce_conv_fod_static_capacity_bytes(void) { return PCE_STATIC_SCRATCH_BYTES; }
+
+extern "C" int pce_conv_fwd_fod_static(const void *in, const void *w, const void *wp, void *out, int32_t dtype, int64_t n_in,
+                                       int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv, int32_t mid,
+                                       const int32_t *imap, const int32_t *omap, const int32_t *kpos, const int32_t *qkpos,
+                                       int64_t qsum, const pce_epilogue_t *epilogue, pce_stream_t stream) {
+  int rc = check_common("pce_conv_fwd_fod_static", in, w, out, dtype, n_in, n_out, c_in, c_out, kv, mid);
+  if (rc || (rc = check_qsum("pce_conv_fwd_fod_static", qsum))) return rc;
+  Epi e;
+  if ((rc = read_epilogue("pce_conv_fwd_fod_static", epilogue, out, &e))) return rc;
+  if (qsum > 0 && (!imap || !omap || !kpos || !qkpos)) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_fod_static: null map pointer");
+  if (!aligned16(out)) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_fod_static: output must be 16-byte aligned");
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == PCE_F32)  // fp32 accumulates in the output itself: no scratch at all
+    return fod_impl<float>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, omap, kpos, qkpos, qsum, (float *)out, e, s);
+  const int64_t need = pce_conv_fod_workspace_bytes(n_out, c_out, dtype);
+  if (need > PCE_STATIC_SCRATCH_BYTES)
+    PCE_FAIL(PCE_ECAPACITY, "pce_conv_fwd_fod_static: the fp32 accumulator of %lld rows x %d channels needs %lld bytes, the static "
+             "scratch array holds %lld (use pce_conv_fwd_fod with a workspace)", (long long)n_out, (int)c_out, (long long)need,
+             (long long)PCE_STATIC_SCRATCH_BYTES);
+  void *acc = nullptr;
+  if ((rc = static_scratch(&acc))) return rc;
+  // the centre GEMM (or the zero fill of a layer without centre offset) overwrites every accumulator row this
+  // call uses before the pair tiles add to it: nothing of an earlier call's contents is read
+  return fod_impl<half_t>(in, w, wp, out, n_out, c_in, c_out, kv, mid, imap, omap, kpos, qkpos, qsum, (float *)acc, e, s);
 }
 
 template <typename T>
