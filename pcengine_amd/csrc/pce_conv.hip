@@ -628,7 +628,10 @@ __device__ __forceinline__ void store_row_pieces_slow(const float (&V)[NB][2][8]
 // Finished rows -> memory through the wavefront's LDS region: the lane that owns (row, 8 columns)
 // writes its pieces; then 16 bytes per lane are read back along the rows, so that NT*sizeof(TO)/16
 // consecutive lanes store one full row segment (whole 128-byte lines at 64 fp16 channels).
-template <typename TO, int NB, int ROWS = (sizeof(TO) == 2 ? 32 : 16), bool SPLIT = false>
+// STREAM: the stores carry the non-temporal hint.  Output rows are written once and read by a later kernel; kept
+// as ordinary dirty lines they are written back in one burst when the kernel ends, which cost the 150 k-voxel
+// layer 2.3 of 9.3 us.
+template <typename TO, int NB, int ROWS = (sizeof(TO) == 2 ? 32 : 16), bool SPLIT = false, bool STREAM = false>
 __device__ __forceinline__ void store_rows_via_lds(const float (&V)[NB][2][8], void *region, TO *out, int orow,
                                                    const TileArgs &a, int n0, int lane, int l32, int g) {
   constexpr int NT = NB * 32;
@@ -678,7 +681,13 @@ __device__ __forceinline__ void store_rows_via_lds(const float (&V)[NB][2][8], v
         base = (TO *)a.out_alt;
         dst -= a.n_split;
       }
-      if (dst >= 0 && col < a.c_out) *reinterpret_cast<OV *>(base + (long long)dst * a.c_out + col) = y;
+      if (dst >= 0 && col < a.c_out) {
+        OV *dp = reinterpret_cast<OV *>(base + (long long)dst * a.c_out + col);
+        if (STREAM)
+          __builtin_nontemporal_store(y, dp);
+        else
+          *dp = y;
+      }
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -854,89 +863,113 @@ __global__ void __launch_bounds__(256, ((TMODE >= 0 && sizeof(T) == 2 && NB <= 2
 // weight tile through LDS behind a barrier makes all resident workgroups read, compute and write in
 // step.  Here every wavefront owns 32 rows (pairs or output rows) and takes its weight fragments
 // straight from the packed copy (8 KB per offset: it stays in cache), so there is no workgroup
-// barrier and wavefronts drift apart, which keeps loads and stores of different wavefronts
-// overlapped.  Chunks [0, pair.items) are pair chunks, the rest rows of the centre GEMM.
-template <int NB, int KS, int RB>
-__global__ void __launch_bounds__(256, RB == 1 ? 5 : 3) wave_gemm_kernel(TileArgs pair, TileArgs centre) {
-  __shared__ __attribute__((aligned(16))) half8 Pl[4][WaveLds<NB>::PIECES];
+// barrier and wavefronts drift apart.  Chunks [0, pair.items) are pair chunks, the rest rows of the
+// centre GEMM.
+//
+// The 32 rows of a chunk reach LDS with global -> LDS copies in line order (eight lanes per 128-byte row, so
+// a load instruction touches 8 whole lines; the MFMA fragment order, one lane per row, touches 32 lines per
+// instruction with 32 bytes of each and was 1.3 us slower on the 150 k-voxel layer), and the fragments are
+// read from there.  Which 16-byte piece of its row a lane fetches is XORed with the row index, so that the
+// fragment reads of 8 consecutive rows fall into different banks.  The region then stages the finished rows
+// on their way out (full lines, streaming stores).
+template <int PPR>
+__device__ __forceinline__ int row_swizzle(int row) {
+  return PPR == 8 ? (row & 7) : (PPR == 4 ? (row & 3) : (PPR == 2 ? (row & 1) : 0));
+}
+
+template <int NB, int KS>
+__global__ void __launch_bounds__(256, 4) wave_gemm_kernel(TileArgs pair, TileArgs centre) {
+  constexpr int PPR = KS * 2;   // 16-byte pieces per input row
+  constexpr int NI = KS;        // global -> LDS instructions per chunk: 32 rows x PPR pieces / 64 lanes
+  // a wavefront's region holds its 32 input rows first, then its finished rows on their way out
+  constexpr int REGION = WaveLds<NB>::PIECES > 32 * PPR ? WaveLds<NB>::PIECES : 32 * PPR;
+  __shared__ __attribute__((aligned(16))) half8 Pl[4][REGION];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int l32 = lane & 31, g = lane >> 5;
-  long long chunk = (long long)blockIdx.x * 4 + wave;   // 32*RB rows (pairs or output rows) per wavefront
+  const long long chunk = (long long)blockIdx.x * 4 + wave;   // 32 rows (pairs or output rows) per wavefront
   const bool is_pair = chunk < pair.items;
   if (!is_pair && chunk - pair.items >= centre.items) return;
   // features, weights and shapes are those of `pair` for both kinds of chunk; only the destination
   // differs (selecting a whole argument block at run time would copy it to private memory)
   const TileArgs &a = pair;
-  int arow[RB], orow[RB], widx;
+  const half_t *A = (const half_t *)a.A;
+  int orow = -1, widx;
+  long long src[NI];   // the row whose piece this lane fetches in instruction `it` (a valid row stands in for a missing one)
   if (is_pair) {
-    long long q0 = chunk * (32 * RB);
+    const long long q0 = chunk * 32;
     widx = 0;
     for (int i = 0; i < pair.kv; ++i) widx += ((long long)pair.qkpos_h[i + 1] <= q0) ? 1 : 0;
     if (widx >= pair.kv) return;
+    const long long p0 = q0 - pair.qkpos_h[widx] + pair.kpos_h[widx], pend = pair.kpos_h[widx + 1];
+    if (p0 + l32 < pend) orow = pair.oslot[p0 + l32];
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
-      long long p = q0 - pair.qkpos_h[widx] + pair.kpos_h[widx] + rb * 32 + l32;
-      bool ok = p < (long long)pair.kpos_h[widx + 1];
-      arow[rb] = ok ? pair.imap[p] : -1;
-      orow[rb] = ok ? pair.oslot[p] : -1;
+    for (int it = 0; it < NI; ++it) {
+      const int r = (it * 64 + lane) / PPR;
+      src[it] = p0 + r < pend ? (long long)pair.imap[p0 + r] : 0ll;
     }
   } else {
     widx = centre.w_fixed;
+    const long long row0 = (chunk - pair.items) * 32;
+    orow = row0 + l32 < centre.n_rows ? (int)(row0 + l32) : -1;
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
-      long long row = (chunk - pair.items) * (32 * RB) + rb * 32 + l32;
-      arow[rb] = orow[rb] = row < centre.n_rows ? (int)row : -1;
+    for (int it = 0; it < NI; ++it) {
+      const int r = (it * 64 + lane) / PPR;
+      src[it] = row0 + r < centre.n_rows ? row0 + r : centre.n_rows - 1;
     }
   }
-  const half_t *A = (const half_t *)a.A;
+#pragma unroll
+  for (int it = 0; it < NI; ++it) {
+    const int e = it * 64 + lane, r = e / PPR, sl = e % PPR;
+    const half_t *gp = A + src[it] * a.c_in + ((sl ^ row_swizzle<PPR>(r)) * 8);
+    // LDS destination: wave-uniform base, the hardware adds lane * 16 bytes
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
+                                     (__attribute__((address_space(3))) void *)&Pl[wave][it * 64], 16, 0, 0);
+  }
   const half_t *Wk = (const half_t *)a.Wp + (long long)widx * a.k8_total * a.n_pad * 8;
-  half8 af[RB][KS], wf[KS][NB];
-#pragma unroll
-  for (int rb = 0; rb < RB; ++rb)
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      half8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (arow[rb] >= 0) v = *reinterpret_cast<const half8 *>(A + (long long)arow[rb] * a.c_in + s * 16 + g * 8);
-      af[rb][s] = v;
-    }
+  half8 wf[KS][NB];
 #pragma unroll
   for (int s = 0; s < KS; ++s)
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
       wf[s][nb] = *reinterpret_cast<const half8 *>(Wk + ((long long)(2 * s + g) * a.n_pad + nb * 32 + l32) * 8);
-  half_t *out = (half_t *)(is_pair ? pair.out : centre.out);
+  // the global -> LDS copies have landed once nothing is outstanding; the fragment reads stay behind this statement
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __builtin_amdgcn_wave_barrier();
+  f32x16 acc[NB];
 #pragma unroll
-  for (int rb = 0; rb < RB; ++rb) {
-    f32x16 acc[NB];
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[nb][j] = 0.f;
+  // a missing row (a padding pair of the offset's last chunk, a row past the end of the tensor) multiplies
+  // whatever stands in for it: its products stay in its own lane and are never stored
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    const half8 af = Pl[wave][l32 * PPR + ((2 * s + g) ^ row_swizzle<PPR>(l32))];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[s][nb], af, acc[nb], 0, 0, 0);
+  }
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();   // every lane has read its fragments: the region becomes the output staging area
+  float V[NB][2][8];
+  gather_row_pieces<NB>(acc, V, g);
+  if (!is_pair && (centre.bias || centre.res || centre.act)) {
+    // rows that receive partial rows later get their activation from the pass that adds them
+    const bool alone = orow >= 0 && centre.ocsr[orow] == centre.ocsr[orow + 1];
+    epilogue_row_pieces<half_t, NB, true>(V, centre, orow, 0, g, false);
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-      for (int j = 0; j < 16; ++j) acc[nb][j] = 0.f;
+      for (int h = 0; h < 2; ++h)
 #pragma unroll
-    for (int s = 0; s < KS; ++s)
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-        acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[s][nb], af[rb][s], acc[nb], 0, 0, 0);
-    float V[NB][2][8];
-    gather_row_pieces<NB>(acc, V, g);
-    if (!is_pair && (centre.bias || centre.res || centre.act)) {
-      // rows that receive partial rows later get their activation from the pass that adds them
-      bool alone = orow[rb] >= 0 && centre.ocsr[orow[rb]] == centre.ocsr[orow[rb] + 1];
-      epilogue_row_pieces<half_t, NB, true>(V, centre, orow[rb], 0, g, false);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-#pragma unroll
-          for (int j = 0; j < 8; ++j) V[nb][h][j] = alone ? act_apply(V[nb][h][j], centre.act, centre.slope) : V[nb][h][j];
-    }
-    store_rows_via_lds<half_t, NB>(V, Pl[wave], out, orow[rb], a, 0, lane, l32, g);
+        for (int j = 0; j < 8; ++j) V[nb][h][j] = alone ? act_apply(V[nb][h][j], centre.act, centre.slope) : V[nb][h][j];
   }
+  half_t *out = (half_t *)(is_pair ? pair.out : centre.out);
+  store_rows_via_lds<half_t, NB, 32, false, true>(V, Pl[wave], out, orow, a, 0, lane, l32, g);
 }
 
-// pair chunks and centre rows of one layer in one launch (either part may be empty); `rb` = 32-row
-// blocks per wavefront, the caller sizes pair.items / centre.items for it
-static int launch_wave_gemm(const TileArgs &pair, const TileArgs &centre, int rb, hipStream_t s) {
+// pair chunks and centre rows of one layer in one launch (either part may be empty): 32 rows per wavefront, the
+// caller sizes pair.items / centre.items for that
+static int launch_wave_gemm(const TileArgs &pair, const TileArgs &centre, hipStream_t s) {
   long long chunks = pair.items + centre.items;
   if (chunks <= 0) return PCE_OK;
   if (chunks / 4 >= (1ll << 31) - 8) PCE_FAIL(PCE_ECAPACITY, "chunk count %lld exceeds the grid limit", chunks);
@@ -944,10 +977,7 @@ static int launch_wave_gemm(const TileArgs &pair, const TileArgs &centre, int rb
   int nb = (pair.c_out + 31) / 32, ks = pair.c_in / 16;  // both blocks come from base_args of one layer
 #define PCE_WAVE_CASE(NB_, KS_)                                                                              \
   if (nb == NB_ && ks == KS_) {                                                                              \
-    if (rb == 2)                                                                                             \
-      hipLaunchKernelGGL((wave_gemm_kernel<NB_, KS_, 2>), dim3(grid), dim3(256), 0, s, pair, centre);        \
-    else                                                                                                     \
-      hipLaunchKernelGGL((wave_gemm_kernel<NB_, KS_, 1>), dim3(grid), dim3(256), 0, s, pair, centre);        \
+    hipLaunchKernelGGL((wave_gemm_kernel<NB_, KS_>), dim3(grid), dim3(256), 0, s, pair, centre);             \
     PCE_LAUNCH_CHECK("wave_gemm");                                                                           \
     return PCE_OK;                                                                                           \
   }
@@ -2098,21 +2128,18 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
     TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
     set_out<T>(&a, buffer, false);
     set_host_pos(&a, kpos_host, qkpos_host);
-    // 64 rows per wavefront once there are enough of them to keep every CU busy: the weight fragments are
-    // fetched once per two row blocks and the first block's stores overlap the second block's arithmetic
-    const int rb = (qsum / 32 + pce_div_up(n_out, 32)) >= 16 * 256 ? 2 : 1;
     a.imap = imap;
     a.oslot = oslot;
-    a.items = qsum / (32 * rb);
+    a.items = qsum / 32;
     TileArgs c = base_args<T>(in, w, wp, kv, c_in, c_out);
     set_out<T>(&c, out, false);
     c.w_fixed = mid;
     c.n_rows = n_out;
-    c.items = pce_div_up(n_out, 32 * rb);
+    c.items = pce_div_up(n_out, 32);
     c.ocsr = ocsr;
     set_epi(&c, e);
     if (a.host_pos && wave_gemm_ok(a, sizeof(T)) && wave_gemm_ok(c, sizeof(T)) && aligned16(buffer) && epi_aligned(e)) {
-      if (stage_on(1) && (rc = launch_wave_gemm(a, c, rb, s))) return rc;
+      if (stage_on(1) && (rc = launch_wave_gemm(a, c, s))) return rc;
       if (stage_on(2) && (rc = launch_rowsum_pairs<T>((const T *)buffer, (T *)out, n_out, n_pairs, c_out, omap, oslot, ocsr,
                                                       e.act, e.slope, s)))
         return rc;
@@ -2177,7 +2204,7 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
       TileArgs none = a;
       none.items = 0;
       a.items = qsum / 32;
-      if ((rc = launch_wave_gemm(a, none, 1, s))) return rc;
+      if ((rc = launch_wave_gemm(a, none, s))) return rc;
     } else if ((rc = launch_tile<T>(a, qsum / PCE_QUANTUM, s))) {
       return rc;
     }
