@@ -25,6 +25,15 @@ struct VecOfC<float, 4> { typedef f32x4 type; };
 template <>
 struct VecOfC<half_t, 4> { typedef _Float16 type __attribute__((ext_vector_type(4))); };
 
+// plain store, or one with the non-temporal hint (see store_rows_via_lds) when the host asked for it
+template <typename V>
+__device__ __forceinline__ void store_maybe_stream(V *p, const V &v, bool stream) {
+  if (stream)
+    __builtin_nontemporal_store(v, p);
+  else
+    *p = v;
+}
+
 enum {
   MODE_FOD = 0,      // A row = imap[pair], out row = omap[pair]
   MODE_BUF = 1,      // A row = out row = quantised pair row (staging buffer)
@@ -69,6 +78,7 @@ struct TileArgs {
   int act;
   float slope;
   int act_alone_only;               // apply the activation only to rows without partial rows (ocsr tells)
+  int stream;                       // output rows leave with the non-temporal hint (set_out)
   void *out_alt;                    // routed pair tiles: destination d < n_split is row d of `out` (a finished output
   int n_split;                      // row, takes the epilogue), d >= n_split is row d - n_split of `out_alt`
   int kpos_h[MAX_KV_ARGS + 1];
@@ -628,12 +638,12 @@ __device__ __forceinline__ void store_row_pieces_slow(const float (&V)[NB][2][8]
 // Finished rows -> memory through the wavefront's LDS region: the lane that owns (row, 8 columns)
 // writes its pieces; then 16 bytes per lane are read back along the rows, so that NT*sizeof(TO)/16
 // consecutive lanes store one full row segment (whole 128-byte lines at 64 fp16 channels).
-// STREAM: the stores carry the non-temporal hint.  Output rows are written once and read by a later kernel; kept
-// as ordinary dirty lines they are written back in one burst when the kernel ends, which cost the 150 k-voxel
-// layer 2.3 of 9.3 us.
-template <typename TO, int NB, int ROWS = (sizeof(TO) == 2 ? 32 : 16), bool SPLIT = false, bool STREAM = false>
+// a.stream: the stores carry the non-temporal hint.  Rows kept as ordinary dirty lines are written back in one
+// burst when the kernel ends (2.3 of 9.3 us on the 150 k-voxel layer); streamed out they leave while the kernel
+// runs, but the next layer then finds none of them in the L2 of its XCD.  The host decides per launch (set_out).
+template <typename TO, int NB, int ROWS = (sizeof(TO) == 2 ? 32 : 16), bool SPLIT = false>
 __device__ __forceinline__ void store_rows_via_lds(const float (&V)[NB][2][8], void *region, TO *out, int orow,
-                                                   const TileArgs &a, int n0, int lane, int l32, int g) {
+                                                   const TileArgs &a, int n0, int lane, int l32, int g, bool stream) {
   constexpr int NT = NB * 32;
   constexpr int EPP = 16 / sizeof(TO);              // elements per piece
   constexpr int LDP = (NT + 8) / EPP;               // row stride in pieces; ROWS rows per pass
@@ -683,7 +693,7 @@ __device__ __forceinline__ void store_rows_via_lds(const float (&V)[NB][2][8], v
       }
       if (dst >= 0 && col < a.c_out) {
         OV *dp = reinterpret_cast<OV *>(base + (long long)dst * a.c_out + col);
-        if (STREAM)
+        if (stream)
           __builtin_nontemporal_store(y, dp);
         else
           *dp = y;
@@ -847,9 +857,9 @@ __global__ void __launch_bounds__(256, ((TMODE >= 0 && sizeof(T) == 2 && NB <= 2
   }
   if (FAST || a.o_vec) {
     if (f32out)
-      store_rows_via_lds<float, NB>(V, Pl[wave], (float *)a.out, orow, a, n0, lane, l32, g);
+      store_rows_via_lds<float, NB>(V, Pl[wave], (float *)a.out, orow, a, n0, lane, l32, g, a.stream);
     else
-      store_rows_via_lds<half_t, NB>(V, Pl[wave], (half_t *)a.out, orow, a, n0, lane, l32, g);
+      store_rows_via_lds<half_t, NB>(V, Pl[wave], (half_t *)a.out, orow, a, n0, lane, l32, g, a.stream);
   } else {
     if (f32out)
       store_row_pieces_slow<float, NB>(V, (float *)a.out, orow, a, n0, g);
@@ -964,7 +974,7 @@ __global__ void __launch_bounds__(256, 4) wave_gemm_kernel(TileArgs pair, TileAr
         for (int j = 0; j < 8; ++j) V[nb][h][j] = alone ? act_apply(V[nb][h][j], centre.act, centre.slope) : V[nb][h][j];
   }
   half_t *out = (half_t *)(is_pair ? pair.out : centre.out);
-  store_rows_via_lds<half_t, NB, 32, false, true>(V, Pl[wave], out, orow, a, 0, lane, l32, g);
+  store_rows_via_lds<half_t, NB>(V, Pl[wave], out, orow, a, 0, lane, l32, g, is_pair ? pair.stream : centre.stream);
 }
 
 // pair chunks and centre rows of one layer in one launch (either part may be empty): 32 rows per wavefront, the
@@ -1001,6 +1011,16 @@ static inline bool stage_on(int bit) { return (g_stage_mask >> bit) & 1u; }
 #else
 static constexpr bool stage_on(int) { return true; }
 #endif
+
+// Output rows leave with the non-temporal hint when the tensor they belong to is larger than PCE_STREAM_MIN_BYTES:
+// a tensor that size is written back from the L2s in one burst at the end of the kernel anyway, and streaming it
+// out while the kernel runs hides that (150 k rows x 64 channels, 19 MB: 9.3 -> 7.0 us); a smaller one is better
+// left in the L2 of the XCD that wrote it, where the next layer's tiles of the same rows find it.
+#define PCE_STREAM_MIN_BYTES (16ll << 20)
+static int stream_policy(long long bytes) {
+  return stage_on(10) && (!stage_on(11) || bytes >= PCE_STREAM_MIN_BYTES);
+}
+
 
 // ---- pipelined tile GEMM for wide fp16 layers ---------------------------------------------------
 // The single-offset modes (pair tiles, centre / dense GEMM) at wide channels: 128 rows x 128 columns
@@ -1217,9 +1237,10 @@ __global__ void __launch_bounds__(256, 4) pipe_gemm_kernel(TileArgs a, TileArgs 
   }
   half_t *out = (half_t *)((PMODE == PIPE_BOTH && dense) ? c.out : a.out);
   if (PMODE == MODE_FOD_BUF && a.out_alt)
-    store_rows_via_lds<half_t, NB, 32, true>(V, lds + wave * WaveLds<NB>::PIECES, out, orow, a, n0, lane, l32, g);
+    store_rows_via_lds<half_t, NB, 32, true>(V, lds + wave * WaveLds<NB>::PIECES, out, orow, a, n0, lane, l32, g, a.stream);
   else
-    store_rows_via_lds<half_t, NB>(V, lds + wave * WaveLds<NB>::PIECES, out, orow, a, n0, lane, l32, g);
+    store_rows_via_lds<half_t, NB>(V, lds + wave * WaveLds<NB>::PIECES, out, orow, a, n0, lane, l32, g,
+                                   (PMODE == PIPE_BOTH && dense) ? c.stream : a.stream);
 }
 
 // The eight weight fragments of a step are requested before its first MFMA, and every MFMA waits only for
@@ -1363,7 +1384,7 @@ __global__ void __launch_bounds__(256, SUB == 1 ? 3 : 2) os_pipe_kernel(TileArgs
   float V[NB][2][8];
   gather_row_pieces<NB>(acc, V, g);
   if (a.bias || a.res || a.act) epilogue_row_pieces_batched<half_t, NB, true, NB>(V, a, orow, n0, g, a.act != PCE_ACT_NONE);
-  store_rows_via_lds<half_t, NB>(V, lds + wave * WaveLds<NB>::PIECES, (half_t *)a.out, orow, a, n0, lane, l32, g);
+  store_rows_via_lds<half_t, NB>(V, lds + wave * WaveLds<NB>::PIECES, (half_t *)a.out, orow, a, n0, lane, l32, g, a.stream);
 }
 
 static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
@@ -1569,7 +1590,7 @@ __global__ void __launch_bounds__(256) rowsum_kernel(const T *__restrict__ buf, 
                                                      const int *__restrict__ csr, T *__restrict__ out,
                                                      const T *__restrict__ bias, const T *__restrict__ res, int act,
                                                      float slope, const int *__restrict__ rows,
-                                                     const int *__restrict__ count) {
+                                                     const int *__restrict__ count, int stream) {
   typedef typename VecOf<T, VEC>::type V;
   int rows_per_block = 256 / G;
   int sub = threadIdx.x % G;
@@ -1612,7 +1633,7 @@ __global__ void __launch_bounds__(256) rowsum_kernel(const T *__restrict__ buf, 
       }
 #pragma unroll
       for (int j = 0; j < VEC; ++j) reinterpret_cast<T *>(&y)[j] = (T)act_apply(acc[j], act, slope);
-      *reinterpret_cast<V *>(&out[row * c_out + (long long)v * VEC]) = y;
+      store_maybe_stream(reinterpret_cast<V *>(&out[row * c_out + (long long)v * VEC]), y, stream != 0);
     }
   }
 }
@@ -1655,7 +1676,7 @@ template <typename T, int VEC, bool BY_ROW>
 __global__ void __launch_bounds__(256) rowsum_pairs_kernel(const T *__restrict__ buf, long long n_items, int c_out, int G,
                                                            const int *__restrict__ omap, const int *__restrict__ oslot,
                                                            const int *__restrict__ csr, T *__restrict__ out, int act,
-                                                           float slope) {
+                                                           float slope, int stream) {
   typedef typename VecOf<T, VEC>::type V;
   long long item = (long long)blockIdx.x * (256 / G) + threadIdx.x / G;
   int sub = threadIdx.x % G;
@@ -1696,7 +1717,7 @@ __global__ void __launch_bounds__(256) rowsum_pairs_kernel(const T *__restrict__
     }
 #pragma unroll
     for (int j = 0; j < VEC; ++j) reinterpret_cast<T *>(&x)[j] = (T)act_apply(acc[j], act, slope);
-    *reinterpret_cast<V *>(&out[(long long)row * c_out + (long long)v * VEC]) = x;
+    store_maybe_stream(reinterpret_cast<V *>(&out[(long long)row * c_out + (long long)v * VEC]), x, stream != 0);
   }
 }
 
@@ -1715,7 +1736,7 @@ static int launch_rowsum_pairs(const T *buffer, T *out, int64_t n_out, int64_t n
   dim3 grid((unsigned)pce_div_up(items, 256 / G)), block(256);
 #define PCE_ROWSUM(V_, B_)                                                                                        \
   hipLaunchKernelGGL((rowsum_pairs_kernel<T, V_, B_>), grid, block, 0, s, buffer, items, c_out, G, omap, oslot, ocsr, out, \
-                     act, slope)
+                     act, slope, stream_policy((long long)n_out * c_out * (long long)sizeof(T)))
   if (vec && by_row)
     PCE_ROWSUM(VEC, true);
   else if (vec)
@@ -1805,11 +1826,13 @@ static TileArgs base_args(const void *in, const void *w, const void *wp, int kv,
   return a;
 }
 
+// `rows` = rows of the tensor `out` points to (0: not known, no streaming)
 template <typename T>
-static void set_out(TileArgs *a, void *out, bool /*f32out*/) {
+static void set_out(TileArgs *a, void *out, bool f32out, long long rows = 0) {
   // a lane of the row epilogue owns 8 consecutive columns, whatever the element type
   a->out = out;
   a->o_vec = (a->c_out % 8 == 0) && aligned16(out);
+  a->stream = rows > 0 ? stream_policy(rows * a->c_out * (f32out ? 4 : (long long)sizeof(T))) : 0;
 }
 
 static void set_host_pos(TileArgs *a, const int32_t *kpos_host, const int32_t *qkpos_host) {
@@ -1900,7 +1923,7 @@ static int fod_impl(const void *in, const void *w, const void *wp, void *out, in
                     int mid, const int *imap, const int *omap, const int *kpos, const int *qkpos, int64_t qsum,
                     float *acc, const Epi &e, hipStream_t s) {
   TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
-  set_out<T>(&a, acc, true);
+  set_out<T>(&a, acc, true, n_out);
   int rc;
   long long total = (long long)n_out * c_out;
   if (!stage_on(0)) {
@@ -2057,7 +2080,7 @@ static int gms_impl(const void *in, const void *w, const void *wp, void *out, in
   if (qsum > 0 && stage_on(1)) {
     // grouped GEMM: every 128-row tile of the staging buffer belongs to one offset
     TileArgs a = base_args<T>(buf_in, w, wp, kv, c_in, c_out);
-    set_out<T>(&a, buf_out, false);
+    set_out<T>(&a, buf_out, false, qsum);
     a.kpos = kpos;
     a.qkpos = qkpos;
     a.mode = MODE_BUF;
@@ -2066,7 +2089,7 @@ static int gms_impl(const void *in, const void *w, const void *wp, void *out, in
   }
   if (mid >= 0 && stage_on(0)) {
     TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
-    set_out<T>(&a, out, false);
+    set_out<T>(&a, out, false, n_out);
     a.mode = MODE_DENSE;
     a.epi = EPI_ROWS;
     a.w_fixed = mid;
@@ -2111,7 +2134,7 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
     // Every output row has exactly one pair (a transposed layer whose kernel equals its stride: each fine
     // voxel has one parent): a pair's product is its output row, stored once with the epilogue, no partial rows.
     TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
-    set_out<T>(&a, out, false);
+    set_out<T>(&a, out, false, n_out);
     set_host_pos(&a, kpos_host, qkpos_host);
     a.imap = imap;
     a.oslot = omap;
@@ -2126,17 +2149,18 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
     // Pair chunks and centre GEMM share one launch (neither reads what the other writes); a pass
     // over the pairs then adds every output row's partial rows to the centre term stored there.
     TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
-    set_out<T>(&a, buffer, false);
+    set_out<T>(&a, buffer, false, n_pairs);
     set_host_pos(&a, kpos_host, qkpos_host);
     a.imap = imap;
     a.oslot = oslot;
     a.items = qsum / 32;
     TileArgs c = base_args<T>(in, w, wp, kv, c_in, c_out);
-    set_out<T>(&c, out, false);
+    set_out<T>(&c, out, false, n_out);
     c.w_fixed = mid;
     c.n_rows = n_out;
     c.items = pce_div_up(n_out, 32);
     c.ocsr = ocsr;
+    a.stream = c.stream;   // the partial rows of a layer leave the way its output rows do
     set_epi(&c, e);
     if (a.host_pos && wave_gemm_ok(a, sizeof(T)) && wave_gemm_ok(c, sizeof(T)) && aligned16(buffer) && epi_aligned(e)) {
       if (stage_on(1) && (rc = launch_wave_gemm(a, c, s))) return rc;
@@ -2151,7 +2175,7 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
     // with the epilogue, the pairs of the other rows store partial rows; the row sum then visits only rows with
     // two pairs or more.  Taken by the pipelined kernel's shapes; the others ignore the routing.
     TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
-    set_out<T>(&a, out, false);
+    set_out<T>(&a, out, false, n_out);
     set_host_pos(&a, kpos_host, qkpos_host);
     a.imap = imap;
     a.oslot = route + PCE_ROUTE_HEAD;
@@ -2170,7 +2194,7 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
   }
   if (qsum > 0 && stage_on(1) && !multi_rows) {
     TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
-    set_out<T>(&a, buffer, false);
+    set_out<T>(&a, buffer, false, n_pairs);
     set_host_pos(&a, kpos_host, qkpos_host);
     a.imap = imap;
     a.oslot = oslot;
@@ -2187,7 +2211,7 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
       // so do those of a centre GEMM that fills the machine twice over by itself (nothing to gain, and a
       // network on 954 k voxels ran 3 % slower with them combined).
       TileArgs c = base_args<T>(in, w, wp, kv, c_in, c_out);
-      set_out<T>(&c, out, false);
+      set_out<T>(&c, out, false, n_out);
       c.mode = MODE_DENSE;
       c.epi = EPI_ROWS;
       c.w_fixed = mid;
@@ -2214,7 +2238,7 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
     // plain centre GEMM (bias and residual fused, activation on rows without partial rows), then the
     // pass over the pairs that adds each row's partial rows: no partial-row staging in the GEMM epilogue
     TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
-    set_out<T>(&a, out, false);
+    set_out<T>(&a, out, false, n_out);
     a.mode = MODE_DENSE;
     a.epi = EPI_ROWS;
     a.w_fixed = mid;
@@ -2227,7 +2251,7 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
   }
   if (mid >= 0) {
     TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
-    set_out<T>(&a, out, false);
+    set_out<T>(&a, out, false, n_out);
     a.mode = MODE_DENSE;
     a.epi = EPI_ROWS_CSR;
     a.w_fixed = mid;
@@ -2247,7 +2271,7 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
     if (multi_rows && blocks > 1024) blocks = 1024;
     hipLaunchKernelGGL((rowsum_kernel<T, VEC>), dim3((unsigned)blocks), dim3(256), 0, s,
                        (const T *)buffer, (long long)n_out, c_out, G, ocsr, (T *)out, (const T *)e.bias, (const T *)e.res,
-                       e.act, e.slope, multi_rows, multi_count);
+                       e.act, e.slope, multi_rows, multi_count, stream_policy((long long)n_out * c_out * (long long)sizeof(T)));
   } else {
     int G = pow2_at_least(c_out);
     if (G > 64) G = 64;
@@ -2255,7 +2279,7 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
     if (multi_rows && blocks > 1024) blocks = 1024;
     hipLaunchKernelGGL((rowsum_kernel<T, 1>), dim3((unsigned)blocks), dim3(256), 0, s,
                        (const T *)buffer, (long long)n_out, c_out, G, ocsr, (T *)out, (const T *)e.bias, (const T *)e.res,
-                       e.act, e.slope, multi_rows, multi_count);
+                       e.act, e.slope, multi_rows, multi_count, stream_policy((long long)n_out * c_out * (long long)sizeof(T)));
   }
   PCE_LAUNCH_CHECK("rowsum");
   return PCE_OK;
@@ -2329,7 +2353,7 @@ template <typename T>
 static int os_impl(const void *in, const void *w, const void *wp, void *out, int64_t n_out, int c_in, int c_out, int kv,
                    const int *nbr, const Epi &e, hipStream_t s) {
   TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
-  set_out<T>(&a, out, false);
+  set_out<T>(&a, out, false, n_out);
   set_epi(&a, e);
   a.nbr = nbr;
   a.n_rows = n_out;
@@ -2355,7 +2379,7 @@ template <typename T>
 static int dense_impl(const void *in, const void *w, const void *wp, void *out, int64_t n, int c_in, int c_out,
                       const Epi &e, hipStream_t s) {
   TileArgs a = base_args<T>(in, w, wp, 1, c_in, c_out);
-  set_out<T>(&a, out, false);
+  set_out<T>(&a, out, false, n);
   set_epi(&a, e);
   a.n_rows = n;
   a.mode = MODE_DENSE;
@@ -3184,11 +3208,11 @@ extern "C" int pce_bn_backward(const void *x, const void *dy, const void *y_act,
 // out[r] = (a[r], b[r]).  One 16-byte vector per thread; threadIdx.x walks along the output row, so a
 // wavefront reads and writes whole rows.  va / vb = vectors per row of a / b.
 __global__ void __launch_bounds__(256) concat_cols_kernel(const u32x4 *__restrict__ a, const u32x4 *__restrict__ b,
-                                                          u32x4 *__restrict__ out, long long n, int va, int vb) {
+                                                          u32x4 *__restrict__ out, long long n, int va, int vb, int stream) {
   const long long r = (long long)blockIdx.x * blockDim.y + threadIdx.y;
   const int v = threadIdx.x;
   if (r >= n || v >= va + vb) return;
-  out[r * (va + vb) + v] = v < va ? a[r * va + v] : b[r * vb + (v - va)];
+  store_maybe_stream(&out[r * (va + vb) + v], v < va ? a[r * va + v] : b[r * vb + (v - va)], stream != 0);
 }
 
 extern "C" int pce_concat_cols(const void *a, int32_t c_a, const void *b, int32_t c_b, void *out, int32_t dtype, int64_t n,
@@ -3207,7 +3231,7 @@ extern "C" int pce_concat_cols(const void *a, int32_t c_a, const void *b, int32_
   const long long blocks = pce_div_up(n, ty);
   if (blocks >= (1ll << 31)) PCE_FAIL(PCE_ECAPACITY, "pce_concat_cols: %lld workgroups exceed the grid limit", blocks);
   hipLaunchKernelGGL(concat_cols_kernel, dim3((unsigned)blocks), dim3(tx, ty), 0, (hipStream_t)stream, (const u32x4 *)a,
-                     (const u32x4 *)b, (u32x4 *)out, (long long)n, va, vb);
+                     (const u32x4 *)b, (u32x4 *)out, (long long)n, va, vb, stream_policy((long long)n * (va + vb) * 16));
   PCE_LAUNCH_CHECK("concat_cols");
   return PCE_OK;
 }
