@@ -155,7 +155,8 @@ int pce_voxelize_emit(const void *ws_dev, int64_t n_points, int64_t n_voxels,
  *     layout of the reference's dense fetch-on-demand map (backend/hash.cuh:331,417); it is the
  *     output-major table of the transposed layer
  *   status int32[4]: [0] coordinate out of range, [1] table exhausted, [2] an offset holds
- *     >= PCE_CSR_CODE pairs (CSR code would overflow).  Caller zeroes it; read it after a sync. */
+ *     >= PCE_CSR_CODE pairs (CSR code would overflow), [3] the column grid of pce_kmap_build_batch
+ *     could not be used (see there).  Caller zeroes it; read it after a sync. */
 int64_t pce_kmap_workspace_bytes(int64_t n_in, int64_t n_out, int32_t kv, int32_t want_csr);
 int pce_kmap_build(const int32_t *in_coords_dev, int64_t n_in, const int32_t *out_coords_dev,
                    int64_t n_out, const pce_geom_t *g, void *ws_dev, int64_t ws_bytes,
@@ -186,8 +187,23 @@ typedef struct pce_kmap_problem {
   int32_t *islot, *oslot;               /* optional, with the CSR outputs */
   int32_t *nbr_out, *nbr_in;            /* optional */
   int32_t *status;                      /* int32[4] per problem, zeroed by the caller */
+  int32_t n_batch;                      /* batch count (spTensor.batchsize), 0 = unknown: see the column grid below */
+  int32_t flags;                        /* PCE_KMAP_* */
 } pce_kmap_problem_t;
 int pce_kmap_build_batch(const pce_kmap_problem_t *problems_host, int32_t n_problems, pce_stream_t stream);
+
+/* The column grid.  The reference looks neighbours up in a hash table whatever the input
+ * (backend/hash.cuh:55-168).  When a problem states its batch count (n_batch > 0), the (b,x,y) box that its
+ * geometry bounds (cmin / cmax of the output coordinates) is modest -- at most 2^26 columns and at most
+ * 32 n_out + 65536 -- and its workspace has the size pce_kmap_workspace_bytes_grid returns, the build indexes
+ * the output coordinates by column instead: one cell per (b,x,y) with the first row of the column and the row
+ * behind its last, the rows of a column searched in z.  That needs the output coordinates strictly ascending in
+ * (b,x,y,z) order -- what pce_outcoords_emit, pce_voxelize_emit and the reference's sparse_quantize produce --
+ * inside the box and with b < n_batch; a build that finds otherwise sets status[3] and leaves its outputs
+ * undefined: the caller runs it again with PCE_KMAP_NO_GRID.  Same maps, bit for bit, either way. */
+#define PCE_KMAP_NO_GRID 1
+int64_t pce_kmap_workspace_bytes_grid(int64_t n_in, int64_t n_out, const pce_geom_t *g, int32_t n_batch,
+                                      int32_t want_csr);
 
 /* ---- forward convolution --------------------------------------------------------------------- *
  * Common arguments: in_feats[n_in,c_in], weight[kv,c_in,c_out], out_feats[n_out,c_out], all of

@@ -17,6 +17,7 @@ PCE_OK, PCE_EINVAL, PCE_ECAPACITY, PCE_EHIP, PCE_EWORKSPACE, PCE_ECOORD = range(
 PCE_F16, PCE_F32, PCE_F64 = 0, 1, 2
 DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS, DATAFLOW_FDS = 0, 1, 2, 3
 QUANTUM = 128
+KMAP_NO_GRID = 1
 CSR_CODE = 1186111
 
 
@@ -40,7 +41,8 @@ class KmapProblem(Structure):
     _fields_ = ([("in_coords", c_void_p), ("n_in", c_int64), ("out_coords", c_void_p), ("n_out", c_int64),
                  ("geom", Geom), ("ws", c_void_p), ("ws_bytes", c_int64)] +
                 [(name, c_void_p) for name in ("imap", "omap", "knnz", "kpos", "qkpos", "icsr", "icode", "ocsr", "ocode",
-                                               "islot", "oslot", "nbr_out", "nbr_in", "status")])
+                                               "islot", "oslot", "nbr_out", "nbr_in", "status")] +
+                [("n_batch", c_int32), ("flags", c_int32)])
 
 
 class Epilogue(Structure):
@@ -82,6 +84,7 @@ _SIGNATURES = {
                                   c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
     "pce_concat_cols": (c_int32, [c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_int32, c_int64, c_void_p]),
     "pce_kmap_workspace_bytes": (c_int64, [c_int64, c_int64, c_int32, c_int32]),
+    "pce_kmap_workspace_bytes_grid": (c_int64, [c_int64, c_int64, POINTER(Geom), c_int32, c_int32]),
     "pce_kmap_build_batch": (c_int32, [POINTER(KmapProblem), c_int32, c_void_p]),
     "pce_kmap_build": (c_int32, [c_void_p, c_int64, c_void_p, c_int64, POINTER(Geom), c_void_p, c_int64] + [c_void_p] * 14 + [c_void_p]),
     "pce_conv_fod_workspace_bytes": (c_int64, [c_int64, c_int32, c_int32]),

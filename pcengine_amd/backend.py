@@ -213,7 +213,12 @@ class _MapJob:
         self.in_coords, self.out_coords, self.geom = in_coords, out_coords, geom
         self.n_in, self.n_out, self.kv, self.want_csr, self.dev = n_in, n_out, kv, bool(want_csr), dev
         self.meta_len = kv + 2 * (kv + 1) + 4      # knnz | kpos | qkpos | status
-        self.ws_bytes = lib.pce_kmap_workspace_bytes(n_in, n_out, kv, int(want_csr))
+        # the batch count lets the library index sorted coordinates by column instead of hashing them; a build that
+        # finds them unsorted, or outside the box the geometry states, is redone through the hash table (finish)
+        self.n_batch, self.no_grid = max(int(batchsize), 0), False
+        self.ws_bytes = lib.pce_kmap_workspace_bytes_grid(n_in, n_out, geom, self.n_batch, int(want_csr))
+        if self.ws_bytes < 0:
+            _lib.check(_lib.PCE_EINVAL)
         self.ws = torch.empty(self.ws_bytes, dtype=torch.uint8, device=dev)
         self.pairs = torch.empty((2, kv * n_in), dtype=torch.int32, device=dev)
         self.nbr_out = torch.empty(kv * n_out, dtype=torch.int32, device=dev) if want_nbr_out else None
@@ -244,6 +249,7 @@ class _MapJob:
         p.islot, p.oslot = _ptr(self.islot), _ptr(self.oslot)
         p.nbr_out, p.nbr_in = _ptr(self.nbr_out), _ptr(self.nbr_in)
         p.status = status.data_ptr()
+        p.n_batch, p.flags = self.n_batch, (_lib.KMAP_NO_GRID if self.no_grid else 0)
         return p
 
     def finish(self, host: list) -> KernelMap:
@@ -255,6 +261,10 @@ class _MapJob:
             raise _lib.PCEError("hash table exhausted while building the kernel map")
         if self.want_csr and st[2]:
             raise OverflowError(f"an offset holds >= {CSR_CODE} pairs: the CSR code of the gather-GEMM-scatter map overflows")
+        if st[3] and not self.no_grid:
+            # unsorted coordinates, or some outside the stated bounds / batch count: the same build through the hash table
+            self.no_grid = True
+            return build_kernel_maps([self])[0]
         M, qsum = host[2 * kv], host[3 * kv + 1]
         ks, stride, pad, cmin, cmax_out, subm = self.args
         cut = lambda t: None if t is None else t[:M]

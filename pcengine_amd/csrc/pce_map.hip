@@ -938,13 +938,44 @@ struct KmapLayout {
   int64_t off_table, off_dense, off_seg, off_scan, off_orank, off_irank, off_desc, total;
 };
 
-static void kmap_layout(int64_t n_in, int64_t n_out, int kv, int want_csr, int sym, KmapLayout *L) {
+// Column grid: the lookup structure of a build whose table coordinates (the output coordinates) are sorted by
+// (b,x,y,z) and lie in a modest (b,x,y) box.  One cell per column (b,x,y) holds the first row of the column and
+// the row behind its last; the z of every row sits in a compact array beside it.  Sorted rows make columns
+// contiguous, so building it is one pass without atomics, and a lookup is one 8-byte cell read plus a short
+// search in z; neighbouring input rows read neighbouring cells, which a hash scatters over the whole table.
+struct GridBox {
+  int lo[2], ext[2];   // x and y
+  int n_batch;
+  long long cells;
+};
+#define GRID_MAX_CELLS (1ll << 26)
+
+static bool grid_box(const GeomDev &g, int n_batch, int64_t n_out, GridBox *b) {
+  if (n_batch <= 0) return false;
+  long long cells = n_batch;
+  for (int a = 0; a < 2; ++a) {
+    if (g.cmax[a] < g.cmin[a]) return false;
+    b->lo[a] = g.cmin[a];
+    b->ext[a] = g.cmax[a] - g.cmin[a] + 1;
+    cells *= b->ext[a];
+    if (cells > GRID_MAX_CELLS) return false;
+  }
+  b->n_batch = n_batch;
+  b->cells = cells;
+  // clearing and reading the grid must stay cheap next to the rows themselves
+  return cells <= 32 * n_out + 65536;
+}
+
+static int64_t grid_bytes(const GridBox &b, int64_t n_out) { return pce_align_up(b.cells * 8, 256) + pce_align_up(n_out * 4, 256); }
+
+// table_bytes: what the lookup structure of this build needs (hash table, or the larger of it and the column grid)
+static void kmap_layout(int64_t n_in, int64_t n_out, int kv, int want_csr, int sym, int64_t table_bytes, KmapLayout *L) {
   L->slots = pce_hash_slots(n_out);
   L->nseg = pce_div_up(n_in, PCE_WAVE);
   L->scan_len = (int64_t)kv * L->nseg + 1;
   int64_t o = 0;
   L->off_table = o;
-  o += pce_align_up(L->slots * 16, 256);
+  o += pce_align_up(table_bytes > L->slots * 16 ? table_bytes : L->slots * 16, 256);
   L->off_dense = o;
   o += pce_align_up((int64_t)kv * n_in * 4, 256);
   L->off_seg = o;
@@ -970,6 +1001,10 @@ struct ProbDev {
   int *dense, *irank, *orank, *seg;
   int *imap, *omap, *knnz, *kpos, *qkpos, *icsr, *icode, *ocsr, *ocode, *islot, *oslot, *nbr_out, *status;
   int want_csr;
+  int use_grid;      // column grid instead of the hash table
+  int2 *grid;        // [cells] = {first row of the column, row behind its last}, -1 for an empty column
+  int *zcol;         // z of every table row
+  GridBox box;
 };
 
 // a contiguous range of workgroups of one launch: workgroups [blk0, next job's blk0) work on `prob`
@@ -1117,6 +1152,158 @@ __global__ void __launch_bounds__(256) kmap_query_kernel(const ProbDev *__restri
       if (i < n_in) {
         dense[(long long)kp * n_in + i] = res;
         if (g.sym && res >= 0) dense[(long long)(g.kv - 1 - kp) * n_in + res] = (int)i;
+      }
+    }
+  }
+}
+
+// ---- column grid -------------------------------------------------------------------------------------
+__device__ __forceinline__ long long grid_cell(const GridBox &b, int bi, int x, int y) {
+  const int gx = x - b.lo[0], gy = y - b.lo[1];
+  if (bi < 0 || bi >= b.n_batch || gx < 0 || gx >= b.ext[0] || gy < 0 || gy >= b.ext[1]) return -1;
+  return ((long long)bi * b.ext[0] + gx) * b.ext[1] + gy;
+}
+
+// One lane per table row.  Checks that the rows ascend strictly in (b,x,y,z) and lie in the box (status[3]
+// otherwise: the caller rebuilds this map through the hash table), writes z to the compact array, and the
+// first / last row of every column writes the column's cell.
+__global__ void __launch_bounds__(256) grid_build_kernel(const ProbDev *__restrict__ P, JobList jl) {
+  const Job &job = find_job(jl, blockIdx.x);
+  const ProbDev &q = P[job.prob];
+  const long long n = q.n_out;
+  long long j = (long long)(blockIdx.x - job.blk0) * blockDim.x + threadIdx.x;
+  if (j >= n) return;
+  const int4 c = q.out_coords[j];
+  if (!pce_coord_ok(c.x, c.y, c.z, c.w)) {
+    q.status[0] = 1;
+    return;
+  }
+  const long long cell = grid_cell(q.box, c.x, c.y, c.z);
+  if (cell < 0) {
+    q.status[3] = 1;
+    return;
+  }
+  q.zcol[j] = c.w;
+  const unsigned long long key = pce_pack_key(c.x, c.y, c.z, c.w);
+  bool first = j == 0, last = j == n - 1;
+  if (j > 0) {
+    const int4 p = q.out_coords[j - 1];
+    if (pce_pack_key(p.x, p.y, p.z, p.w) >= key) q.status[3] = 1;   // not sorted, or a duplicate row
+    first = p.x != c.x || p.y != c.y || p.z != c.z;
+  }
+  if (j < n - 1) {
+    const int4 nx = q.out_coords[j + 1];
+    last = nx.x != c.x || nx.y != c.y || nx.z != c.z;
+  }
+  if (first) q.grid[cell].x = (int)j;
+  if (last) q.grid[cell].y = (int)j + 1;
+}
+
+// row of the column [s, e) whose z equals tz, or -1; rows of a column ascend in z
+__device__ __forceinline__ int grid_search(const int *__restrict__ zcol, int s, int e, int tz) {
+  while (e - s > 4) {
+    const int m = (s + e) >> 1;
+    if (zcol[m] <= tz)
+      s = m;
+    else
+      e = m;
+  }
+  for (int j = s; j < e; ++j)
+    if (zcol[j] == tz) return j;
+  return -1;
+}
+
+// The probe of kmap_query_kernel over the column grid: one lane per input row; the offsets are walked column by
+// column (ix, iy), GRID_BATCH columns at a time: their cells are read together, then the first four z of every
+// column (most columns of a surface-like cloud are that short), then the offsets of the column are resolved.
+// SUBM3: the 3x3x3 submanifold layer with everything known at compile time (5 columns, 13 offsets, no divisions);
+// otherwise the geometry is read from the problem.
+#define GRID_BATCH 5
+template <bool SUBM3>
+__global__ void __launch_bounds__(256) grid_query_kernel(const ProbDev *__restrict__ P, JobList jl) {
+  const Job &job = find_job(jl, blockIdx.x);
+  const ProbDev &q = P[job.prob];
+  const GeomDev &g = q.g;
+  const long long n_in = q.n_in;
+  const int2 *__restrict__ grid = q.grid;
+  const int *__restrict__ zcol = q.zcol;
+  int *__restrict__ dense = q.dense;
+  long long i = (long long)(blockIdx.x - job.blk0) * blockDim.x + threadIdx.x;
+  bool live = i < n_in;
+  int4 c = live ? q.in_coords[i] : make_int4(0, 0, 0, 0);
+  if (live && !pce_coord_ok(c.x, c.y, c.z, c.w)) {
+    q.status[0] = 1;
+    live = false;
+  }
+  const bool subm = SUBM3 ? true : g.subm != 0;
+  const bool sym = SUBM3 ? true : g.sym != 0;
+  const int kv = SUBM3 ? 27 : g.kv, mid = SUBM3 ? 13 : g.mid;
+  const int kend = sym ? mid : kv;                            // offsets [0, kend) are looked up
+  const int ksy = SUBM3 ? 3 : g.ks[1], ksz = SUBM3 ? 3 : g.ks[2];
+  const int ncol = SUBM3 ? 5 : (kend + ksz - 1) / ksz;        // columns (ix, iy) that hold one of them
+  const int hx = SUBM3 ? 1 : g.half[0] - g.bump[0], hy = SUBM3 ? 1 : g.half[1] - g.bump[1], hz = SUBM3 ? 1 : g.half[2] - g.bump[2];
+  for (int col0 = 0; col0 < ncol; col0 += GRID_BATCH) {
+    int2 se[GRID_BATCH];
+    int zz[GRID_BATCH][4];
+#pragma unroll
+    for (int j = 0; j < GRID_BATCH; ++j) {
+      const int col = col0 + j;
+      se[j] = make_int2(-1, -1);
+      if (live && col < ncol) {
+        const int ix = col / ksy, iy = col - ix * ksy;
+        const int dx = ix - hx, dy = iy - hy;
+        int tx, ty;
+        bool ok = true;
+        if (subm) {
+          tx = c.y - dx;
+          ty = c.z - dy;
+        } else {
+          ok = strided_axis(c.y, dx, g.pad[0], g.stride[0], g.cmin[0], g.cmax[0], &tx);
+          ok &= strided_axis(c.z, dy, g.pad[1], g.stride[1], g.cmin[1], g.cmax[1], &ty);
+        }
+        const long long cell = ok ? grid_cell(q.box, c.x, tx, ty) : -1;
+        if (cell >= 0) se[j] = grid[cell];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < GRID_BATCH; ++j)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const int r = se[j].x + t;
+        zz[j][t] = (se[j].x >= 0 && r < se[j].y) ? zcol[r] : (int)0x80000000;
+      }
+#pragma unroll
+    for (int j = 0; j < GRID_BATCH; ++j) {
+      const int col = col0 + j;
+      if (col >= ncol) break;
+#pragma unroll
+      for (int iz = 0; iz < (SUBM3 ? 3 : 1024); ++iz) {
+        if (!SUBM3 && iz >= ksz) break;
+        const int kp = col * ksz + iz;
+        if (kp >= kend) break;
+        int res = -1;
+        if (live && se[j].x >= 0 && !(subm && kp == mid)) {
+          const int dz = iz - hz;
+          int tz;
+          bool ok = true;
+          if (subm)
+            tz = c.w - dz;
+          else
+            ok = strided_axis(c.w, dz, g.pad[2], g.stride[2], g.cmin[2], g.cmax[2], &tz);
+          if (ok) {
+            if (se[j].y - se[j].x <= 4) {
+#pragma unroll
+              for (int t = 0; t < 4; ++t)
+                if (zz[j][t] == tz) res = se[j].x + t;     // padding entries hold INT_MIN, which no valid z equals
+            } else {
+              res = grid_search(zcol, se[j].x, se[j].y, tz);
+            }
+          }
+        }
+        if (i < n_in) {
+          dense[(long long)kp * n_in + i] = res;
+          if (sym && res >= 0) dense[(long long)(kv - 1 - kp) * n_in + res] = (int)i;
+        }
       }
     }
   }
@@ -1369,19 +1556,32 @@ __global__ void __launch_bounds__(256) csr_stage_kernel(const ProbDev *__restric
 
 extern "C" int64_t pce_kmap_workspace_bytes(int64_t n_in, int64_t n_out, int32_t kv, int32_t want_csr) {
   KmapLayout L;
-  kmap_layout(n_in, n_out, kv, want_csr, 0, &L);  // the strided layout is the larger one
+  kmap_layout(n_in, n_out, kv, want_csr, 0, 0, &L);  // the strided layout is the larger one
   return L.total;
 }
+
+extern "C" int64_t pce_kmap_workspace_bytes_grid(int64_t n_in, int64_t n_out, const pce_geom_t *g, int32_t n_batch,
+                                                 int32_t want_csr) {
+  GeomDev d;
+  if (make_geom(g, &d) != PCE_OK || n_in <= 0 || n_out <= 0) return -1;
+  GridBox box;
+  const int64_t table = grid_box(d, n_batch, n_out, &box) ? grid_bytes(box, n_out) : 0;
+  KmapLayout L;
+  kmap_layout(n_in, n_out, d.kv, want_csr, 0, table, &L);
+  return L.total;
+}
+
+// stages of a batched build, each one launch with its own job list
+enum { ST_INSERT = 0, ST_QUERY, ST_COUNT, ST_FILL, ST_CSR_A, ST_CSR_B, ST_GRID_BUILD, ST_GRID_QUERY, ST_GRID_QUERY3, ST_COUNT_ };
 
 // host-side image of everything the kernels of one batch read
 struct BatchImage {
   ProbDev prob[PCE_MAX_BATCH];
-  Job jobs[8][2 * PCE_MAX_BATCH];      // per stage
-  int n_jobs[8];
-  FillRegion fills[3 * PCE_MAX_BATCH];
+  Job jobs[ST_COUNT_][2 * PCE_MAX_BATCH];      // per stage
+  int n_jobs[ST_COUNT_];
+  FillRegion fills[4 * PCE_MAX_BATCH];
   ScanArr scans[2][2 * PCE_MAX_BATCH];  // first scan (segments, input rows), second scan (output rows)
 };
-enum { ST_INSERT = 0, ST_QUERY, ST_COUNT, ST_FILL, ST_CSR_A, ST_CSR_B };
 
 // The descriptor block travels from pinned host memory, so the copy is queued like a kernel and the
 // host does not wait for earlier work on the stream.  A small ring of pinned blocks per device; a
@@ -1427,7 +1627,7 @@ extern "C" int pce_kmap_build_batch(const pce_kmap_problem_t *probs, int32_t n_p
   static_assert(sizeof(BatchImage) <= KMAP_DESC_BYTES, "descriptor area too small");
   BatchImage img;
   memset(&img, 0, sizeof(img));
-  unsigned blk[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  unsigned blk[ST_COUNT_] = {};
   unsigned fill_blk = 0, scan_blk[2] = {0, 0};
   int n_fill = 0, n_scan[2] = {0, 0};
   auto add_job = [&](int stage, int prob, int kind, long long items) {
@@ -1470,8 +1670,16 @@ extern "C" int pce_kmap_build_batch(const pce_kmap_problem_t *probs, int32_t n_p
     if (q.g.subm && n_in != n_out) PCE_FAIL(PCE_EINVAL, "pce_kmap_build: submanifold layer needs n_in == n_out");
     if ((int64_t)q.g.kv * n_in >= (1ll << 31) || (int64_t)q.g.kv * n_out >= (1ll << 31))
       PCE_FAIL(PCE_ECAPACITY, "pce_kmap_build: kv*n exceeds int32 pair indexing");
+    // The column grid serves when the caller bounds the batch indices, the (b,x,y) box of the table coordinates
+    // is modest and the workspace was sized for it (pce_kmap_workspace_bytes_grid); else the hash table.
     KmapLayout L;
-    kmap_layout(n_in, n_out, q.g.kv, want_csr, q.g.sym, &L);
+    GridBox box;
+    int use_grid = 0;
+    if (!(u.flags & PCE_KMAP_NO_GRID) && grid_box(q.g, u.n_batch, n_out, &box)) {
+      kmap_layout(n_in, n_out, q.g.kv, want_csr, q.g.sym, grid_bytes(box, n_out), &L);
+      use_grid = u.ws_bytes >= L.total;
+    }
+    if (!use_grid) kmap_layout(n_in, n_out, q.g.kv, want_csr, q.g.sym, 0, &L);
     if (u.ws_bytes < L.total) PCE_FAIL(PCE_EWORKSPACE, "pce_kmap_build: workspace %lld < %lld", (long long)u.ws_bytes, (long long)L.total);
     char *w = (char *)u.ws;
     q.in_coords = (const int4 *)u.in_coords;
@@ -1499,8 +1707,17 @@ extern "C" int pce_kmap_build_batch(const pce_kmap_problem_t *probs, int32_t n_p
     q.nbr_out = u.nbr_out;
     q.status = u.status;
     q.want_csr = want_csr;
-    // 1. table over the output coordinates (for a submanifold layer these are the input coordinates)
-    add_fill(q.table, L.slots * 4);
+    q.use_grid = use_grid;
+    if (use_grid) {
+      q.box = box;
+      q.grid = (int2 *)(w + L.off_table);
+      q.zcol = (int *)(w + L.off_table + pce_align_up(box.cells * 8, 256));
+    }
+    // 1. lookup structure over the output coordinates (for a submanifold layer these are the input coordinates)
+    if (use_grid)
+      add_fill(q.grid, box.cells * 2);
+    else
+      add_fill(q.table, L.slots * 4);
     if (q.g.sym) {
       // rows of the probe table that the mirrored writes only touch on a hit (and the centre row)
       add_fill(q.dense + (int64_t)q.g.mid * n_in, (int64_t)(q.g.kv - q.g.mid) * n_in);
@@ -1508,9 +1725,10 @@ extern "C" int pce_kmap_build_batch(const pce_kmap_problem_t *probs, int32_t n_p
       if (q.nbr_out) add_fill(q.nbr_out, (int64_t)q.g.kv * n_out);
       if (q.orank) add_fill(q.orank, (int64_t)q.g.kv * n_out);
     }
-    add_job(ST_INSERT, p, 0, n_out);
+    add_job(use_grid ? ST_GRID_BUILD : ST_INSERT, p, 0, n_out);
     // 2. probe, count per (offset, segment) and per row; 3. their scans; 4. pair lists
-    add_job(ST_QUERY, p, 0, n_in);
+    const bool subm3 = q.g.sym && q.g.ks[0] == 3 && q.g.ks[1] == 3 && q.g.ks[2] == 3;
+    add_job(use_grid ? (subm3 ? ST_GRID_QUERY3 : ST_GRID_QUERY) : ST_QUERY, p, 0, n_in);
     add_job(ST_COUNT, p, 0, n_in + 1);
     int *scan_tmp = (int *)(w + L.off_scan);
     add_scan(0, q.seg, L.scan_len, scan_tmp);
@@ -1525,13 +1743,15 @@ extern "C" int pce_kmap_build_batch(const pce_kmap_problem_t *probs, int32_t n_p
       add_scan(1, q.ocsr, n_out + 1, scan_tmp + scan_tmp_ints(L.scan_len) + scan_tmp_ints(n_in + 1));
       add_job(ST_CSR_B, p, JOB_CSR_OUT, n_out);
     }
-    total_blocks += pce_div_up(n_in + 1, 256) + pce_div_up(n_out + 1, 256) + pce_div_up(L.slots * 4, FILL_WORDS_PER_BLOCK) +
+    total_blocks += pce_div_up(n_in + 1, 256) + pce_div_up(n_out + 1, 256) +
+                    pce_div_up(use_grid ? box.cells * 2 : L.slots * 4, FILL_WORDS_PER_BLOCK) +
                     3 * pce_div_up((int64_t)q.g.kv * (n_in > n_out ? n_in : n_out), FILL_WORDS_PER_BLOCK);
   }
   if (total_blocks >= (1ll << 31)) PCE_FAIL(PCE_ECAPACITY, "pce_kmap_build_batch: the batch exceeds the grid limit");
   // one copy carries the descriptors; they live in the first problem's workspace
   KmapLayout L0;
-  kmap_layout(probs[0].n_in, probs[0].n_out, img.prob[0].g.kv, img.prob[0].want_csr, img.prob[0].g.sym, &L0);
+  kmap_layout(probs[0].n_in, probs[0].n_out, img.prob[0].g.kv, img.prob[0].want_csr, img.prob[0].g.sym,
+              img.prob[0].use_grid ? grid_bytes(img.prob[0].box, probs[0].n_out) : 0, &L0);
   char *desc = (char *)probs[0].ws + L0.off_desc;
   if (int rc = desc_upload(img, desc, s)) return rc;
   const BatchImage *D = (const BatchImage *)desc;
@@ -1544,10 +1764,26 @@ extern "C" int pce_kmap_build_batch(const pce_kmap_problem_t *probs, int32_t n_p
   };
   hipLaunchKernelGGL(multi_fill_kernel, dim3(fill_blk), dim3(256), 0, s, (const FillRegion *)D->fills, n_fill, 0xFFFFFFFFu);
   PCE_LAUNCH_CHECK("multi_fill");
-  hipLaunchKernelGGL(batch_insert_kernel, dim3(blk[ST_INSERT]), dim3(256), 0, s, P, jl(ST_INSERT));
-  PCE_LAUNCH_CHECK("hash_insert");
-  hipLaunchKernelGGL(kmap_query_kernel, dim3(blk[ST_QUERY]), dim3(256), 0, s, P, jl(ST_QUERY));
-  PCE_LAUNCH_CHECK("kmap_query");
+  if (blk[ST_INSERT]) {
+    hipLaunchKernelGGL(batch_insert_kernel, dim3(blk[ST_INSERT]), dim3(256), 0, s, P, jl(ST_INSERT));
+    PCE_LAUNCH_CHECK("hash_insert");
+  }
+  if (blk[ST_GRID_BUILD]) {
+    hipLaunchKernelGGL(grid_build_kernel, dim3(blk[ST_GRID_BUILD]), dim3(256), 0, s, P, jl(ST_GRID_BUILD));
+    PCE_LAUNCH_CHECK("grid_build");
+  }
+  if (blk[ST_QUERY]) {
+    hipLaunchKernelGGL(kmap_query_kernel, dim3(blk[ST_QUERY]), dim3(256), 0, s, P, jl(ST_QUERY));
+    PCE_LAUNCH_CHECK("kmap_query");
+  }
+  if (blk[ST_GRID_QUERY]) {
+    hipLaunchKernelGGL(grid_query_kernel<false>, dim3(blk[ST_GRID_QUERY]), dim3(256), 0, s, P, jl(ST_GRID_QUERY));
+    PCE_LAUNCH_CHECK("grid_query");
+  }
+  if (blk[ST_GRID_QUERY3]) {
+    hipLaunchKernelGGL(grid_query_kernel<true>, dim3(blk[ST_GRID_QUERY3]), dim3(256), 0, s, P, jl(ST_GRID_QUERY3));
+    PCE_LAUNCH_CHECK("grid_query3");
+  }
   hipLaunchKernelGGL(kmap_count_kernel, dim3(blk[ST_COUNT]), dim3(256), 0, s, P, jl(ST_COUNT));
   PCE_LAUNCH_CHECK("kmap_count");
   hipLaunchKernelGGL(multi_scan_local_kernel, dim3(scan_blk[0]), dim3(256), 0, s, (const ScanArr *)D->scans[0], n_scan[0]);
@@ -1601,5 +1837,7 @@ extern "C" int pce_kmap_build(const int32_t *in_coords, int64_t n_in, const int3
   u.nbr_out = nbr_out;
   u.nbr_in = nbr_in;
   u.status = status;
+  u.n_batch = 0;   // no batch bound in this signature: the hash table
+  u.flags = 0;
   return pce_kmap_build_batch(&u, 1, stream);
 }

@@ -147,7 +147,10 @@ def test_every_map_of_the_network_pyramid_matches_the_frozen_manifest(name):
     for lv in frozen["pyramid"]:
         key = (name, lv["level"])
         assert cd.shape[0] == lv["voxels"] and cmax == lv["coords_max"] and digest(cd) == lv["coords_sha256"], key
-        sub = backend.build_kernel_map(cd, (3, 3, 3), (1, 1, 1), (0, 0, 0), [0, 0, 0], cmax, True, want_csr=True)
+        # batch count stated: the column grid (the front end's route); test_full_size_maps_match_the_frozen_manifest
+        # builds the level-0 maps through the hash table
+        sub = backend.build_kernel_map(cd, (3, 3, 3), (1, 1, 1), (0, 0, 0), [0, 0, 0], cmax, True, want_csr=True,
+                                       batchsize=frozen["batches"])
         check(sub, lv["layers"]["k333_s111_p000"], key)
         if "k222_s222_p000" in lv["layers"]:
             cmax = backend.strided_coords_max(cmax, (2, 2, 2), (2, 2, 2), (0, 0, 0))

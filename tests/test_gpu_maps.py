@@ -73,10 +73,10 @@ def test_kernel_map_bit_exact(ks, stride, pad, seed, n, extent, batches):
         return
     km = gpu_map(coords, ks, stride, pad, want_csr=True, want_nbr_out=True, want_nbr_in=True)
     assert_map_equal(km, ref, csr=True)
-    if tuple(stride) != (1, 1, 1):
-        # the same layer through the occupancy-bitmap route to the output coordinates
-        kb = gpu_map(coords, ks, stride, pad, batchsize=batches)
-        assert_map_equal(kb, ref)
+    # the same layer with the batch count stated: neighbours are looked up in the column grid instead of the hash
+    # table, and a strided layer takes the occupancy-bitmap route to its output coordinates
+    kb = gpu_map(coords, ks, stride, pad, want_csr=True, want_nbr_out=True, want_nbr_in=True, batchsize=batches)
+    assert_map_equal(kb, ref, csr=True)
 
 
 def test_kernel_map_config1_and_determinism():
@@ -195,6 +195,32 @@ def test_unsorted_input_rows():
     coords = coords[np.random.default_rng(1).permutation(len(coords))]
     for ks, stride, pad in GEOMS[:4]:
         assert_map_equal(gpu_map(coords, ks, stride, pad, want_csr=True), orc.kernel_map(coords, ks, stride, pad), csr=True)
+        # with the batch count stated the build starts on the column grid, finds the rows unsorted and is redone
+        # through the hash table
+        assert_map_equal(gpu_map(coords, ks, stride, pad, want_csr=True, batchsize=2), orc.kernel_map(coords, ks, stride, pad),
+                         csr=True)
+
+
+def test_column_grid_falls_back_when_its_preconditions_fail():
+    """The column grid needs rows strictly ascending in (b,x,y,z), inside the stated coordinate bounds and with batch
+    indices below the stated count.  Each violation is detected on the device (status word 3) and the map is built
+    again through the hash table: same result as without the batch count."""
+    coords = synth.random_cloud(seed=32, n=6000, extent=24, batches=3)
+    ref = orc.kernel_map(coords, (3, 3, 3))
+    cd = dev_coords(coords)
+    cmax = coords[:, 1:].max(axis=0).tolist()
+    build = lambda c, cm, nb: backend.build_kernel_map(c, (3, 3, 3), (1, 1, 1), (0, 0, 0), [0, 0, 0], cm, True, want_csr=True,
+                                                       batchsize=nb)
+    assert_map_equal(build(cd, cmax, 3), ref, csr=True)                       # the grid itself
+    assert_map_equal(build(cd, cmax, 2), ref, csr=True)                       # a batch index beyond the stated count
+    assert_map_equal(build(cd, [c - 5 for c in cmax], 3), ref, csr=True)      # rows beyond the stated bounds
+    swapped = coords.copy()
+    swapped[[10, 11]] = swapped[[11, 10]]                                     # one inversion
+    assert_map_equal(build(dev_coords(swapped), cmax, 3), orc.kernel_map(swapped, (3, 3, 3)), csr=True)
+    # a long column (a wall): more rows in z than the four a probe reads ahead
+    wall = np.array([[0, x, 7, z] for x in range(3) for z in range(0, 60)] + [[0, 5, 5, 5]], np.int32)
+    wall = wall[np.lexsort((wall[:, 3], wall[:, 2], wall[:, 1], wall[:, 0]))]
+    assert_map_equal(build(dev_coords(wall), wall[:, 1:].max(0).tolist(), 1), orc.kernel_map(wall, (3, 3, 3)), csr=True)
 
 
 def test_indoor_scene_batch2():
