@@ -114,6 +114,23 @@ int pce_outcoords_build(const int32_t *in_coords_dev, int64_t n_in, const pce_ge
 int pce_outcoords_emit(const void *ws_dev, int64_t n_in, const pce_geom_t *g, int32_t n_batch, int64_t n_out,
                        int32_t *out_coords_dev, pce_stream_t stream);
 
+/* The output coordinates of several strided layers in a row -- the levels of a network, each reading the
+ * coordinates the one before it wrote -- with ONE wait of the host instead of one per level: the count of a level
+ * stays on the device for the next and the launches are sized for its bound (the reference builds level by level,
+ * script/spconv.py:363 once per strided layer).  Every level has to qualify for the occupancy bitmap
+ * (n_batch > 0, modest boxes).
+ *   pce_outcoords_chain_plan: PCE_OK and, per level, the workspace bytes and the capacity (rows) its output
+ *       buffer needs; PCE_CHAIN_NOT_APPLICABLE when some level does not qualify (build level by level then).
+ *   pce_outcoords_chain: builds all levels; out_coords_dev[l] receives n_out_host[l] rows of (b,x,y,z), identical
+ *       to what pce_outcoords_build/_emit give level by level.  Synchronises the stream once. */
+#define PCE_MAX_CHAIN 8
+#define PCE_CHAIN_NOT_APPLICABLE 100
+int pce_outcoords_chain_plan(int64_t n_in, int32_t levels, const pce_geom_t *geoms, int32_t n_batch,
+                             int64_t *ws_bytes, int64_t *capacity);
+int pce_outcoords_chain(const int32_t *in_coords_dev, int64_t n_in, int32_t levels, const pce_geom_t *geoms,
+                        int32_t n_batch, void *const *ws_dev, const int64_t *ws_bytes, int32_t *const *out_coords_dev,
+                        int64_t *n_out_host, pce_stream_t stream);
+
 /* ---- voxelisation ----------------------------------------------------------------------------- *
  * Replaces sparse_quantize + ravel_hash (script/utils.py:18-55), which the reference runs in NumPy
  * on the host: voxel = floor(point / voxel_size) in double precision; the unique voxels in

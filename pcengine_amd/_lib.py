@@ -67,6 +67,9 @@ _SIGNATURES = {
     "pce_outcoords_workspace_bytes": (c_int64, [c_int64, POINTER(Geom), c_int32]),
     "pce_outcoords_build": (c_int32, [c_void_p, c_int64, POINTER(Geom), c_int32, c_void_p, c_int64, POINTER(c_int64), c_void_p]),
     "pce_outcoords_emit": (c_int32, [c_void_p, c_int64, POINTER(Geom), c_int32, c_int64, c_void_p, c_void_p]),
+    "pce_outcoords_chain_plan": (c_int32, [c_int64, c_int32, POINTER(Geom), c_int32, POINTER(c_int64), POINTER(c_int64)]),
+    "pce_outcoords_chain": (c_int32, [c_void_p, c_int64, c_int32, POINTER(Geom), c_int32, POINTER(c_void_p), POINTER(c_int64),
+                                      POINTER(c_void_p), POINTER(c_int64), c_void_p]),
     "pce_voxelize_workspace_bytes": (c_int64, [c_int64]),
     "pce_voxelize": (c_int32, [c_void_p, c_int32, c_int64, POINTER(ctypes.c_double), c_void_p, c_int64, POINTER(c_int64),
                                POINTER(c_int32), POINTER(c_int32), c_void_p]),

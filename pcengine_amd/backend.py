@@ -55,6 +55,32 @@ def _mid(ks: Sequence[int]) -> int:
     return (ks[0] - 1) // 2 * ks[1] * ks[2] + (ks[1] - 1) // 2 * ks[2] + (ks[2] - 1) // 2
 
 
+class _Cut:
+    """A per-pair array of a map: allocated for the largest possible pair count and cut to the real one on first
+    use (a network reads a few of the six arrays of each of its maps; cutting all of them up front is Python time
+    the host spends before the first convolution is queued)."""
+
+    def __init__(self, optional: bool):
+        self.optional = optional
+
+    def __set_name__(self, owner, name):
+        self.slot = "_cut_" + name
+
+    def __get__(self, obj, owner=None):
+        if obj is None:
+            if self.optional:
+                return None              # the dataclass default
+            raise AttributeError         # a required field: no default
+        v = obj.__dict__.get(self.slot)
+        if isinstance(v, tuple):         # (array at capacity, pair count)
+            v = v[0][:v[1]]
+            obj.__dict__[self.slot] = v
+        return v
+
+    def __set__(self, obj, value):
+        obj.__dict__[self.slot] = value
+
+
 @dataclass
 class KernelMap:
     """Kernel map of one (kernel size, tensor stride, layer stride) key.
@@ -72,8 +98,8 @@ class KernelMap:
     kv: int
     M: int
     qsum: int
-    imap: torch.Tensor
-    omap: torch.Tensor
+    imap: torch.Tensor = _Cut(False)
+    omap: torch.Tensor = _Cut(False)
     knnz: torch.Tensor
     kpos: torch.Tensor
     qkpos: torch.Tensor
@@ -81,11 +107,11 @@ class KernelMap:
     nbr_out: Optional[torch.Tensor] = None
     nbr_in: Optional[torch.Tensor] = None
     icsr: Optional[torch.Tensor] = None
-    icode: Optional[torch.Tensor] = None
+    icode: Optional[torch.Tensor] = _Cut(True)
     ocsr: Optional[torch.Tensor] = None
-    ocode: Optional[torch.Tensor] = None
-    islot: Optional[torch.Tensor] = None   # pair -> position of its entry in icode / ocode
-    oslot: Optional[torch.Tensor] = None
+    ocode: Optional[torch.Tensor] = _Cut(True)
+    islot: Optional[torch.Tensor] = _Cut(True)   # pair -> position of its entry in icode / ocode
+    oslot: Optional[torch.Tensor] = _Cut(True)
     route: Optional[torch.Tensor] = None   # routing array of a layer without centre offset (pair_route), built on first use
     route_t: Optional[torch.Tensor] = None # the same for the transposed layer over this map
     tag: str = "auto"           # 'D1' / 'D2' when the reference's init_tag protocol fixed it
@@ -145,6 +171,43 @@ def build_out_coords(in_coords: torch.Tensor, geom: Geom, batchsize: int = 0) ->
         out = torch.empty((n_out.value, 4), dtype=torch.int32, device=in_coords.device)
         _lib.check(lib.pce_outcoords_emit(ws.data_ptr(), n_in, geom, n_batch, n_out.value, _ptr(out), s))
         return out
+
+
+CHAIN_NOT_APPLICABLE = 100   # PCE_CHAIN_NOT_APPLICABLE
+MAX_CHAIN = 8                # PCE_MAX_CHAIN
+
+
+def build_out_coords_chain(in_coords: torch.Tensor, geoms: Sequence[Geom], batchsize: int) -> Optional[List[torch.Tensor]]:
+    """Output coordinates of several strided layers in a row (each reads what the one before it wrote) with one
+    wait of the host, or None where that does not apply (a level too large or too empty for the occupancy bitmap,
+    no batch count, a batch index beyond it): the caller then builds level by level."""
+    lib = _lib.load()
+    _require_cuda(in_coords, "coords")
+    levels = len(geoms)
+    if levels < 1 or levels > MAX_CHAIN or batchsize <= 0:
+        return None
+    n_in = in_coords.shape[0]
+    garr = (Geom * levels)(*geoms)
+    ws_bytes, cap = (_lib.c_int64 * levels)(), (_lib.c_int64 * levels)()
+    rc = lib.pce_outcoords_chain_plan(n_in, levels, garr, int(batchsize), ws_bytes, cap)
+    if rc == CHAIN_NOT_APPLICABLE:
+        return None
+    _lib.check(rc)
+    # workspaces and coordinate buffers of all levels in one allocation, each on a 256-byte boundary
+    sizes = []
+    for l in range(levels):
+        for n in ((ws_bytes[l] + 3) // 4, 4 * cap[l]):
+            sizes += [n, -n % 64]
+    pieces = torch.empty(sum(sizes), dtype=torch.int32, device=in_coords.device).split_with_sizes(sizes)
+    ws = (_lib.ctypes.c_void_p * levels)(*[pieces[4 * l].data_ptr() for l in range(levels)])
+    outs = (_lib.ctypes.c_void_p * levels)(*[pieces[4 * l + 2].data_ptr() for l in range(levels)])
+    n_out = (_lib.c_int64 * levels)()
+    rc = lib.pce_outcoords_chain(in_coords.data_ptr(), n_in, levels, garr, int(batchsize), ws, ws_bytes, outs, n_out,
+                                 _stream(in_coords.device))
+    if rc == _lib.PCE_EINVAL and b"n_batch" in lib.pce_last_error():
+        return None
+    _lib.check(rc)
+    return [pieces[4 * l + 2][:4 * n_out[l]].view(n_out[l], 4) for l in range(levels)]
 
 
 def voxelize(points: torch.Tensor, voxel_size, batch_index: int = 0, return_index: bool = False,
@@ -219,19 +282,35 @@ class _MapJob:
         self.ws_bytes = lib.pce_kmap_workspace_bytes_grid(n_in, n_out, geom, self.n_batch, int(want_csr))
         if self.ws_bytes < 0:
             _lib.check(_lib.PCE_EINVAL)
-        self.ws = torch.empty(self.ws_bytes, dtype=torch.uint8, device=dev)
-        self.pairs = torch.empty((2, kv * n_in), dtype=torch.int32, device=dev)
-        self.nbr_out = torch.empty(kv * n_out, dtype=torch.int32, device=dev) if want_nbr_out else None
-        self.nbr_in = torch.empty(kv * n_in, dtype=torch.int32, device=dev) if want_nbr_in else None
+        # the arrays of the build, in int32 elements: one allocation holds those of every job of a batch (place)
+        cap = kv * n_in
+        self.want = [("ws", (self.ws_bytes + 3) // 4), ("imap", cap), ("omap", cap)]
+        if want_nbr_out:
+            self.want.append(("nbr_out", kv * n_out))
+        if want_nbr_in:
+            self.want.append(("nbr_in", kv * n_in))
         if want_csr:
-            # icsr | ocsr | icode | ocode | islot | oslot in one allocation
-            cap = kv * n_in
-            buf = torch.empty(n_in + 1 + n_out + 1 + 4 * cap, dtype=torch.int32, device=dev)
-            self.icsr, self.ocsr = buf[:n_in + 1], buf[n_in + 1:n_in + n_out + 2]
-            codes = buf[n_in + n_out + 2:].view(4, cap)
-            self.icode, self.ocode, self.islot, self.oslot = codes[0], codes[1], codes[2], codes[3]
-        else:
-            self.icsr = self.ocsr = self.icode = self.ocode = self.islot = self.oslot = None
+            self.want += [("icsr", n_in + 1), ("ocsr", n_out + 1), ("icode", cap), ("ocode", cap), ("islot", cap), ("oslot", cap)]
+        self.ws = self.imap = self.omap = self.nbr_out = self.nbr_in = None
+        self.icsr = self.ocsr = self.icode = self.ocode = self.islot = self.oslot = None
+
+    @staticmethod
+    def place(jobs) -> None:
+        """One device allocation for the arrays of all `jobs`, each array on a 256-byte boundary."""
+        jobs = [j for j in jobs if j.ws is None]
+        if not jobs:
+            return
+        sizes = []
+        for j in jobs:
+            for _, n in j.want:
+                sizes += [n, -n % 64]
+        arena = torch.empty(sum(sizes), dtype=torch.int32, device=jobs[0].dev)
+        pieces = arena.split_with_sizes(sizes)
+        k = 0
+        for j in jobs:
+            for name, _ in j.want:
+                setattr(j, name, pieces[k])
+                k += 2
 
     def problem(self, meta: torch.Tensor) -> "_lib.KmapProblem":
         """``meta`` is this job's zeroed slice of the batch's count tensor."""
@@ -243,7 +322,7 @@ class _MapJob:
         p.out_coords, p.n_out = self.out_coords.data_ptr(), self.n_out
         p.geom = self.geom
         p.ws, p.ws_bytes = self.ws.data_ptr(), self.ws_bytes
-        p.imap, p.omap = self.pairs[0].data_ptr(), self.pairs[1].data_ptr()
+        p.imap, p.omap = self.imap.data_ptr(), self.omap.data_ptr()
         p.knnz, p.kpos, p.qkpos = self.knnz.data_ptr(), self.kpos.data_ptr(), self.qkpos.data_ptr()
         p.icsr, p.icode, p.ocsr, p.ocode = _ptr(self.icsr), _ptr(self.icode), _ptr(self.ocsr), _ptr(self.ocode)
         p.islot, p.oslot = _ptr(self.islot), _ptr(self.oslot)
@@ -267,9 +346,9 @@ class _MapJob:
             return build_kernel_maps([self])[0]
         M, qsum = host[2 * kv], host[3 * kv + 1]
         ks, stride, pad, cmin, cmax_out, subm = self.args
-        cut = lambda t: None if t is None else t[:M]
+        cut = lambda t: None if t is None else (t, M)     # cut to the pair count when first read
         km = KernelMap(ks=ks, stride=stride, pad=pad, subm=subm, n_in=self.n_in, n_out=self.n_out, kv=kv,
-                       M=M, qsum=qsum, imap=self.pairs[0, :M], omap=self.pairs[1, :M], knnz=self.knnz, kpos=self.kpos,
+                       M=M, qsum=qsum, imap=cut(self.imap), omap=cut(self.omap), knnz=self.knnz, kpos=self.kpos,
                        qkpos=self.qkpos, out_coords=self.out_coords, nbr_out=self.nbr_out, nbr_in=self.nbr_in,
                        icsr=self.icsr, ocsr=self.ocsr, icode=cut(self.icode), ocode=cut(self.ocode),
                        islot=cut(self.islot), oslot=cut(self.oslot), in_coords=self.in_coords, geom=self.geom,
@@ -314,6 +393,7 @@ def build_kernel_maps(requests: List[dict], defer: bool = False):
         starts.append(starts[-1] + j.meta_len)
     # the counts and status words of every map in one tensor: a single device->host copy reads them all
     meta = torch.zeros(starts[-1], dtype=torch.int32, device=dev)
+    _MapJob.place(jobs)
     for b0 in range(0, len(jobs), KMAP_MAX_BATCH):
         chunk = jobs[b0:b0 + KMAP_MAX_BATCH]
         probs = (_lib.KmapProblem * len(chunk))(*[j.problem(meta[starts[b0 + k]:starts[b0 + k + 1]])

@@ -416,9 +416,13 @@ static void outcoord_layout(int64_t n_in, const GeomDev &g, int n_batch, OutCoor
 }
 
 // status[0]: coordinate out of range, status[2]: batch index >= the caller's batch count
+// n_dev (optional): the number of input rows, on the device -- the count a previous level of a chained build left;
+// n_in is then the bound the grid was sized for.
 __global__ void __launch_bounds__(256) outcoord_mark_kernel(const int4 *__restrict__ coords, long long n_in, GeomDev g,
-                                                            BitGrid grid, unsigned *__restrict__ bits, int *status) {
+                                                            BitGrid grid, unsigned *__restrict__ bits, int *status,
+                                                            const int *__restrict__ n_dev) {
   long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (n_dev) n_in = *n_dev;
   if (i >= n_in) return;
   int4 c = coords[i];
   if (!pce_coord_ok(c.x, c.y, c.z, c.w)) {
@@ -639,7 +643,7 @@ extern "C" int pce_outcoords_build(const int32_t *in_coords, int64_t n_in, const
     int *status = (int *)(w + L.off_counters);
     if ((rc = fill_u32(bits, (L.off_counters + 256 - L.off_bits) / 4, 0u, s))) return rc;
     hipLaunchKernelGGL(outcoord_mark_kernel, dim3((unsigned)pce_div_up(n_in, 256)), dim3(256), 0, s,
-                       (const int4 *)in_coords, (long long)n_in, gd, L.grid, bits, status);
+                       (const int4 *)in_coords, (long long)n_in, gd, L.grid, bits, status, (const int *)nullptr);
     PCE_LAUNCH_CHECK("outcoord_mark");
     // the spare last word is zero, so after the scan cnt[words-1] is the number of set bits
     if ((rc = scan_exclusive2(cnt, L.words, nullptr, 0, (int *)(w + L.off_scan), s, bits))) return rc;
@@ -704,6 +708,87 @@ extern "C" int pce_outcoords_emit(const void *ws, int64_t n_in, const pce_geom_t
   hipLaunchKernelGGL(decode_codes_kernel, dim3((unsigned)pce_div_up(n_out, 256)), dim3(256), 0, (hipStream_t)stream, ca,
                      (long long)n_out, (int4 *)out_coords);
   PCE_LAUNCH_CHECK("decode_codes");
+  return PCE_OK;
+}
+
+// ---- the output coordinates of several strided layers in a row, one wait of the host ---------------------------
+// Level l reads the coordinates level l-1 wrote; their number stays on the device (the last word of the scanned
+// popcounts) and the launches are sized for its bound, so nothing has to reach the host between the levels.
+static int chain_plan(int64_t n_in, int levels, const pce_geom_t *geoms, int32_t n_batch, GeomDev *gd, OutCoordLayout *L,
+                      int64_t *bound_in) {
+  if (levels < 1 || levels > PCE_MAX_CHAIN || !geoms) PCE_FAIL(PCE_EINVAL, "pce_outcoords_chain: levels=%d (1..%d)", levels, PCE_MAX_CHAIN);
+  if (n_in <= 0 || n_in >= (1ll << 31)) PCE_FAIL(PCE_EINVAL, "pce_outcoords_chain: n_in=%lld", (long long)n_in);
+  int64_t bound = n_in;
+  for (int l = 0; l < levels; ++l) {
+    int rc = make_geom(&geoms[l], &gd[l]);
+    if (rc) return rc;
+    bound_in[l] = bound;
+    outcoord_layout(bound, gd[l], n_batch, &L[l]);
+    if (!L[l].bitmap) return -1;   // not an error: the caller builds level by level
+    int64_t cells = (int64_t)L[l].grid.n_batch * L[l].grid.ext[0] * L[l].grid.ext[1] * L[l].grid.ext[2];
+    bound = L[l].upper < cells ? L[l].upper : cells;
+    if (bound >= (1ll << 31)) return -1;
+  }
+  return PCE_OK;
+}
+
+extern "C" int pce_outcoords_chain_plan(int64_t n_in, int32_t levels, const pce_geom_t *geoms, int32_t n_batch,
+                                        int64_t *ws_bytes, int64_t *capacity) {
+  GeomDev gd[PCE_MAX_CHAIN];
+  OutCoordLayout L[PCE_MAX_CHAIN];
+  int64_t bound_in[PCE_MAX_CHAIN];
+  if (!ws_bytes || !capacity) PCE_FAIL(PCE_EINVAL, "pce_outcoords_chain_plan: null pointer");
+  int rc = chain_plan(n_in, levels, geoms, n_batch, gd, L, bound_in);
+  if (rc < 0) return PCE_CHAIN_NOT_APPLICABLE;
+  if (rc) return rc;
+  for (int l = 0; l < levels; ++l) {
+    ws_bytes[l] = L[l].total;
+    int64_t cells = (int64_t)L[l].grid.n_batch * L[l].grid.ext[0] * L[l].grid.ext[1] * L[l].grid.ext[2];
+    capacity[l] = L[l].upper < cells ? L[l].upper : cells;
+  }
+  return PCE_OK;
+}
+
+extern "C" int pce_outcoords_chain(const int32_t *in_coords, int64_t n_in, int32_t levels, const pce_geom_t *geoms,
+                                   int32_t n_batch, void *const *ws, const int64_t *ws_bytes, int32_t *const *out_coords,
+                                   int64_t *n_out_host, pce_stream_t stream) {
+  hipStream_t s = (hipStream_t)stream;
+  GeomDev gd[PCE_MAX_CHAIN];
+  OutCoordLayout L[PCE_MAX_CHAIN];
+  int64_t bound_in[PCE_MAX_CHAIN];
+  if (!in_coords || !ws || !ws_bytes || !out_coords || !n_out_host) PCE_FAIL(PCE_EINVAL, "pce_outcoords_chain: null pointer");
+  int rc = chain_plan(n_in, levels, geoms, n_batch, gd, L, bound_in);
+  if (rc < 0) PCE_FAIL(PCE_EINVAL, "pce_outcoords_chain: a level does not take the occupancy bitmap (ask pce_outcoords_chain_plan first)");
+  if (rc) return rc;
+  int host[PCE_MAX_CHAIN][4];
+  const int4 *src = (const int4 *)in_coords;
+  const int *n_dev = nullptr;
+  for (int l = 0; l < levels; ++l) {
+    if (!ws[l] || !out_coords[l]) PCE_FAIL(PCE_EINVAL, "pce_outcoords_chain: null pointer at level %d", l);
+    if (ws_bytes[l] < L[l].total) PCE_FAIL(PCE_EWORKSPACE, "pce_outcoords_chain: workspace %lld < %lld at level %d", (long long)ws_bytes[l], (long long)L[l].total, l);
+    char *w = (char *)ws[l];
+    unsigned *bits = (unsigned *)(w + L[l].off_bits);
+    int *cnt = (int *)(w + L[l].off_cnt);
+    int *status = (int *)(w + L[l].off_counters);
+    if ((rc = fill_u32(bits, (L[l].off_counters + 256 - L[l].off_bits) / 4, 0u, s))) return rc;
+    hipLaunchKernelGGL(outcoord_mark_kernel, dim3((unsigned)pce_div_up(bound_in[l], 256)), dim3(256), 0, s, src,
+                       (long long)bound_in[l], gd[l], L[l].grid, bits, status, n_dev);
+    PCE_LAUNCH_CHECK("outcoord_mark");
+    if ((rc = scan_exclusive2(cnt, L[l].words, nullptr, 0, (int *)(w + L[l].off_scan), s, bits))) return rc;
+    hipLaunchKernelGGL(outcoord_expand_kernel, dim3((unsigned)pce_div_up(L[l].words, 256)), dim3(256), 0, s,
+                       (const unsigned *)bits, (const int *)cnt, (long long)L[l].words, L[l].grid, (int4 *)out_coords[l]);
+    PCE_LAUNCH_CHECK("outcoord_expand");
+    PCE_HIP(hipMemcpyAsync(&host[l][0], cnt + (L[l].words - 1), sizeof(int), hipMemcpyDeviceToHost, s));
+    PCE_HIP(hipMemcpyAsync(&host[l][1], status, 3 * sizeof(int), hipMemcpyDeviceToHost, s));
+    src = (const int4 *)out_coords[l];
+    n_dev = cnt + (L[l].words - 1);
+  }
+  PCE_HIP(hipStreamSynchronize(s));
+  for (int l = 0; l < levels; ++l) {
+    if (host[l][1]) PCE_FAIL(PCE_ECOORD, "pce_outcoords_chain: coordinate outside [0,%d) or batch index out of range (level %d)", PCE_COORD_BOUND, l);
+    if (host[l][3]) PCE_FAIL(PCE_EINVAL, "pce_outcoords_chain: a batch index is >= n_batch=%d", (int)n_batch);
+    n_out_host[l] = host[l][0];
+  }
   return PCE_OK;
 }
 

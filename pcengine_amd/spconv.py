@@ -279,23 +279,47 @@ def ensure_map(input: spTensor, kernel_size_code: int, stride_code: int, padding
     return km, output_stride, coords_min, coords_max
 
 
-def prebuild_maps(input: spTensor, layers) -> None:
-    """Build, ahead of any convolution, the maps a network will ask for.  ``layers`` lists
-    (kernel_size, stride, padding) in network order (ints or triples; transposed layers and 1x1
-    layers need no entry); a strided entry moves on to its output coordinates, as the network does.
-    The output coordinates of the strided layers are computed first, level by level (their number has
-    to reach the host); then all maps are built together, every stage of the build as one launch over
-    all layers, and their pair counts are read back in one copy.  The layers that follow find every
-    map in the cache."""
+def _chain_out_coords(input: spTensor, layers) -> dict:
+    """{index in `layers`: output coordinates} of the strided entries, computed with one wait of the host for all
+    of them; empty where that does not apply (fewer than two strided entries, one of them cached, no batch count,
+    a level the library's chained build does not take)."""
+    if not input.coords.is_cuda or not input.batchsize or input.batchsize <= 0:
+        return {}
+    geoms, idx = [], []
+    stride, cmax, cmin = input.stride, list(input.coords_max[:3]), list(input.coords_min[:3])
+    for i, (ks, st, pad) in enumerate(layers):
+        ksc, sc, pc = (conv_info_encoder(_triple(v, "layer")) for v in (ks, st, pad))
+        if sc == _UNIT:
+            continue
+        if (ksc, stride, sc) in input.kmaps:
+            return {}
+        k3, s3, p3 = conv_info_decoder(ksc), conv_info_decoder(sc), conv_info_decoder(pc)
+        cmax = backend.strided_coords_max(cmax, k3, s3, p3)
+        geoms.append(backend.Geom.make(k3, s3, p3, cmin, cmax, False))
+        idx.append(i)
+        stride = output_stride_compute(sc, stride, 0)
+    if len(geoms) < 2 or len(geoms) > backend.MAX_CHAIN:
+        return {}
+    outs = backend.build_out_coords_chain(input.coords.contiguous(), geoms, input.batchsize)
+    return dict(zip(idx, outs)) if outs is not None else {}
+
+
+def _prebuild(input: spTensor, layers):
+    """Builds the maps `layers` asks for, starting at `input`.  Returns (the tensor at the coordinates the last
+    entry leaves, the maps that were built now)."""
     x = input
-    pending = []
+    pending, done = [], []
+    layers = list(layers)
+    chained = _chain_out_coords(input, layers)
     try:
-        for ks, stride, pad in layers:
+        for i, (ks, stride, pad) in enumerate(layers):
             ksc, sc, pc = (conv_info_encoder(_triple(v, "layer")) for v in (ks, stride, pad))
             if ksc == _UNIT and sc == _UNIT:
                 continue
             km, request, key, tag, out_stride, cmin, cmax = _map_request(x, ksc, sc, pc)
             if request is not None:
+                if i in chained:
+                    request["out_coords"] = chained[i]
                 km = backend.prepare_map(**request)
                 pending.append((x, km, key, tag, out_stride))
                 x.kmaps[key] = km          # placeholder: a later entry with the same key is the same map
@@ -309,11 +333,25 @@ def prebuild_maps(input: spTensor, layers) -> None:
             built = backend.build_kernel_maps([job for _, job, _, _, _ in pending], defer=True)
             torch.cuda.current_stream(input.coords.device).synchronize()
             for (t, _, key, tag, out_stride), pm in zip(pending, built):
-                _map_store(t, pm.finish(), key, tag, out_stride)
+                km = pm.finish()
+                _map_store(t, km, key, tag, out_stride)
+                done.append(km)
     finally:
         for t, job, key, _, _ in pending:       # a failed build leaves no placeholder behind
             if t.kmaps.get(key) is job:
                 del t.kmaps[key]
+    return x, done
+
+
+def prebuild_maps(input: spTensor, layers) -> None:
+    """Build, ahead of any convolution, the maps a network will ask for.  ``layers`` lists
+    (kernel_size, stride, padding) in network order (ints or triples; transposed layers and 1x1
+    layers need no entry); a strided entry moves on to its output coordinates, as the network does.
+    The output coordinates of the strided layers are computed first, level by level (their number has
+    to reach the host); then all maps are built together, every stage of the build as one launch over
+    all layers, and their pair counts are read back in one copy.  The layers that follow find every
+    map in the cache."""
+    _prebuild(input, layers)
 
 
 def conv_func(input: spTensor, in_channel, out_channel, kernel, kernel_size_code, stride_code, padding_code, bias,

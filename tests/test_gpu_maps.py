@@ -190,6 +190,51 @@ def test_out_coords_sparse_box_falls_back_to_sort():
     assert np.array_equal(backend.build_out_coords(dev_coords(coords), geom, 1).cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("chain", [
+    [((2, 2, 2), (2, 2, 2), (0, 0, 0))] * 4,                                          # the levels of a U-Net
+    [((3, 3, 3), (2, 2, 2), (1, 1, 1)), ((2, 2, 2), (2, 2, 2), (0, 0, 0)), ((3, 2, 1), (2, 2, 1), (0, 0, 0))],
+    [((2, 2, 2), (2, 2, 2), (0, 0, 0))],
+])
+def test_out_coords_chain_equals_the_levels_built_one_by_one(chain):
+    """The chained build (the counts of the levels stay on the device, one wait of the host) against the oracle's
+    coordinates level by level, and against the library's own single-level build."""
+    coords = synth.random_cloud(seed=44, n=40000, extent=70, batches=3)
+    cmin, cmax = [0, 0, 0], coords[:, 1:].max(0).tolist()
+    geoms, want, cur = [], [], coords
+    for ks, stride, pad in chain:
+        cmax = orc.strided_coords_max(cmax, ks, stride, pad)
+        geoms.append(_lib.Geom.make(ks, stride, pad, cmin, cmax, False))
+        cur = orc.out_coords_strided(cur, ks, stride, pad, cmin, cmax)
+        want.append(cur)
+    got = backend.build_out_coords_chain(dev_coords(coords), geoms, 3)
+    assert got is not None and len(got) == len(chain)
+    src = dev_coords(coords)
+    for g, w, geom in zip(got, want, geoms):
+        assert len(w) > 0 and np.array_equal(g.cpu().numpy(), w)
+        assert torch.equal(backend.build_out_coords(src, geom, 3), g)
+        src = g
+
+
+def test_out_coords_chain_declines_what_it_cannot_take():
+    """No batch count, a batch index beyond the stated count, a box too sparse for the bitmap: None, and the
+    front end builds level by level (same maps as ever)."""
+    coords = synth.random_cloud(seed=45, n=5000, extent=24, batches=3)
+    k2 = ((2, 2, 2), (2, 2, 2), (0, 0, 0))
+    geoms = [_lib.Geom.make(*k2, [0, 0, 0], [11, 11, 11], False), _lib.Geom.make(*k2, [0, 0, 0], [5, 5, 5], False)]
+    c = dev_coords(coords)
+    assert backend.build_out_coords_chain(c, geoms, 0) is None
+    assert backend.build_out_coords_chain(c, geoms, 2) is None           # batch index 2 present
+    assert backend.build_out_coords_chain(c, geoms, 3) is not None
+    rng = np.random.default_rng(46)
+    far = np.unique(np.concatenate([np.zeros((300, 1), np.int64), rng.integers(0, 3000, (300, 3))], 1), axis=0).astype(np.int32)
+    sparse = [_lib.Geom.make(*k2, [0, 0, 0], [1499] * 3, False), _lib.Geom.make(*k2, [0, 0, 0], [749] * 3, False)]
+    assert backend.build_out_coords_chain(dev_coords(far), sparse, 1) is None
+    lib = _lib.load()
+    ws, cap = (_lib.c_int64 * 2)(), (_lib.c_int64 * 2)()
+    assert lib.pce_outcoords_chain_plan(len(far), 2, (_lib.Geom * 2)(*sparse), 1, ws, cap) == backend.CHAIN_NOT_APPLICABLE
+    assert lib.pce_outcoords_chain_plan(len(far), 9, None, 1, ws, cap) == _lib.PCE_EINVAL
+
+
 def test_unsorted_input_rows():
     coords = synth.random_cloud(seed=31, n=5000, extent=20, batches=2)
     coords = coords[np.random.default_rng(1).permutation(len(coords))]

@@ -119,7 +119,9 @@ def test_unet_fp16_runs_close_to_fp32():
 
 def test_prebuilt_maps_cover_the_whole_network(monkeypatch):
     """prebuild_maps builds the nine maps of the U-Net (five submanifold, four strided) before any
-    convolution; the layers then find all of them cached, and the result does not depend on it."""
+    convolution -- the output coordinates of the four strided levels in one chained build -- ; the layers then find
+    all of them cached, and the result does not depend on it: built lazily, level by level, the maps and the
+    output are the same bit for bit."""
     from pcengine_amd import backend, spconv
     coords = synth.random_cloud(seed=63, n=6000, extent=32)
     f = synth.features(10, len(coords), 4)
@@ -141,3 +143,6 @@ def test_prebuilt_maps_cover_the_whole_network(monkeypatch):
     with torch.no_grad():
         z = model(mk())
     assert len(calls) == 9 and torch.equal(y.feats, z.feats)
+    for key, km in x.kmaps.items():
+        other = z.kmaps[key]
+        assert torch.equal(km.out_coords, other.out_coords) and torch.equal(km.imap, other.imap) and torch.equal(km.omap, other.omap)
