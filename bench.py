@@ -19,6 +19,62 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 
 
+def layer_records(forward, graph_ms):
+    """One record per distinct convolution of a network forward (fp16): the call's shapes and dataflow, its time
+    (10 calls captured into a HIP graph, median of 5 replays), and what that time means against the two roofs --
+    the layer's algorithmic bytes (input rows, output rows, residual rows, weights, the pair list) per second
+    against the HBM peak, its multiply-accumulates against the dense fp16 MFMA peak.  `n` = how many layers of
+    the forward have exactly this shape."""
+    import torch
+    from pcengine_amd import backend
+    calls = []
+    real_conv, real_dense = backend.conv_forward, backend.dense_forward
+
+    def conv(feats, weight, km, dataflow, **kw):
+        calls.append(("conv", feats, weight, km, dataflow, kw))
+        return real_conv(feats, weight, km, dataflow, **kw)
+
+    def dense(feats, weight, packed=None, **kw):
+        calls.append(("dense", feats, weight, None, -1, dict(kw, packed=packed)))
+        return real_dense(feats, weight, packed, **kw)
+    backend.conv_forward, backend.dense_forward = conv, dense
+    try:
+        with torch.no_grad():
+            forward()
+    finally:
+        backend.conv_forward, backend.dense_forward = real_conv, real_dense
+    names = {backend.DATAFLOW_FOD: "fod", backend.DATAFLOW_GMS: "gms", backend.DATAFLOW_OS: "os", backend.DATAFLOW_FDS: "fds", -1: "gemm"}
+    records = {}
+    for kind, feats, weight, km, flow, kw in calls:
+        w3 = weight if weight.dim() == 3 else weight.unsqueeze(0)
+        kv, c_in, c_out = w3.shape
+        e = feats.element_size()
+        if kind == "dense":
+            n_in = n_out = feats.shape[0]
+            M, what = 0, "1x1"
+            flops = 2.0 * n_in * c_in * c_out
+            fn = lambda: real_dense(feats, weight, kw["packed"], bias=kw.get("bias"), residual=kw.get("residual"), act=kw.get("act"))
+        else:
+            tr = bool(kw.get("transposed", False))
+            n_in, n_out = (km.n_out, km.n_in) if tr else (km.n_in, km.n_out)
+            M = km.M
+            what = ("T" if tr else "") + ("subm" if km.subm else "strided") + "x".join(str(k) for k in km.ks)
+            flops = 2.0 * (M + (n_in if km.subm else 0)) * c_in * c_out
+            fn = lambda: real_conv(feats, weight, km, flow, **kw)
+        res = kw.get("residual") is not None
+        key = (what, n_in, n_out, M, c_in, c_out, names[flow], res)
+        if key in records:
+            records[key]["n"] += 1
+            continue
+        ms = graph_ms(fn, 10, 2, replays=5)[0]
+        nbytes = n_in * c_in * e + n_out * c_out * e * (2 if res else 1) + kv * c_in * c_out * e + 8 * M
+        records[key] = {"layer": what, "n_in": n_in, "n_out": n_out, "pairs": M, "c_in": c_in, "c_out": c_out,
+                        "dataflow": names[flow], "residual": res, "n": 1, "ms": round(ms, 5),
+                        "GBs": round(nbytes / ms / 1e6, 1), "hbm_frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 3),
+                        "TFLOPs": round(flops / ms / 1e9, 1), "mfma_frac": round(flops / ms / 1e9 / 2500.0, 3)}
+    return list(records.values())
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -30,6 +86,7 @@ def main() -> int:
                          "set beyond the last-level cache); deep: a decoder-like layer (dense map, C 256->256) for the MFMA roofline")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-net", action="store_true", help="skip the MinkUNet-style forward (configuration 4)")
+    ap.add_argument("--no-layers", action="store_true", help="skip the per-layer record of the configuration-4 network")
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip configurations 1 (fp32 C16 layer), 3 (k2s2 down + transposed up) and 5 (8-scene indoor "
                          "batch, widened network), whose timings go to extra.cfg1 / cfg3 / cfg5")
@@ -301,6 +358,9 @@ def main() -> int:
         os.environ.pop("PCENGINE_DATAFLOW", None)
         result["extra"]["cfg4_minkunet"] = {"voxels": int(len(c4)), "dtype": "f16", "selector": net["auto"],
                                             "all_fetch_on_demand": net["fod"], "all_gather_gemm_scatter": net["gms"]}
+        if not args.no_layers:
+            y0 = forward()
+            result["extra"]["cfg4_minkunet"]["layers"] = layer_records(lambda: forward(y0), graph_ms)
         # the same network in training mode (BatchNorm on batch statistics, cross-entropy on random labels):
         # forward + backward with kernel maps built every step, fp16 features and fp32 parameters
         torch.manual_seed(5)

@@ -245,6 +245,14 @@ typedef struct pce_epilogue {
   const void *residual;
   int32_t act;         /* PCE_ACT_* */
   float slope;         /* negative slope of PCE_ACT_LEAKY_RELU */
+  /* Row strides, in elements, of in_feats and out_feats when they are column slices of wider row-major
+   * matrices; 0 = dense (c_in / c_out).  With them the two producers of a skip connection -- the transposed
+   * layer and the encoder layer whose output is kept -- write their halves of the concatenated matrix in place
+   * and the layers that read one half gather from it, so the concatenation (script/utils.py:152-164) costs no
+   * pass over the data.  Multiples of 8 elements, at least the channel count; taken by pce_conv_fwd_fds and
+   * pce_conv_fwd_os (any dtype), PCE_EINVAL elsewhere.  residual, bias and the partial-row buffer stay dense. */
+  int64_t ld_in;
+  int64_t ld_out;
 } pce_epilogue_t;
 
 /* fp16 weights can be handed over a second time in the order the kernels stage them into LDS

@@ -47,7 +47,8 @@ class KmapProblem(Structure):
 
 class Epilogue(Structure):
     """pce_epilogue_t: out = act(conv + bias + residual)."""
-    _fields_ = [("bias", c_void_p), ("residual", c_void_p), ("act", c_int32), ("slope", ctypes.c_float)]
+    _fields_ = [("bias", c_void_p), ("residual", c_void_p), ("act", c_int32), ("slope", ctypes.c_float),
+                ("ld_in", c_int64), ("ld_out", c_int64)]
 
 
 ACT_NONE, ACT_RELU, ACT_LEAKY_RELU = 0, 1, 2

@@ -505,12 +505,28 @@ def _act_code(act) -> Tuple[int, float]:
     raise ValueError(f"unknown activation {act!r}")
 
 
-def _epilogue(feats: torch.Tensor, n_out: int, c_out: int, bias, residual, act):
+def _row_stride(t: torch.Tensor) -> int:
+    """Elements between consecutive rows of a feature matrix the kernels can read or write in place: 0 for a dense
+    matrix, the stride for a column slice of a wider row-major matrix (16-byte aligned, stride a multiple of 8
+    elements), -1 for any other layout (the caller makes a dense copy)."""
+    if t.dim() != 2:
+        return -1
+    if t.is_contiguous():
+        return 0
+    if (t.stride(1) == 1 and t.stride(0) > t.shape[1] and t.stride(0) % 8 == 0 and t.shape[1] % 8 == 0
+            and t.data_ptr() % 16 == 0):
+        return t.stride(0)
+    return -1
+
+
+def _epilogue(feats: torch.Tensor, n_out: int, c_out: int, bias, residual, act, ld_in: int = 0, ld_out: int = 0):
     """(ctypes struct or None, tensors to keep alive) for ``out = act(conv + bias + residual)``.
-    ``act``: None, 'relu', or ('leaky_relu', negative_slope)."""
-    if bias is None and residual is None and act is None:
+    ``act``: None, 'relu', or ('leaky_relu', negative_slope).  ``ld_in`` / ``ld_out``: row strides of a
+    feature matrix and an output that are column slices of wider matrices (0: dense)."""
+    if bias is None and residual is None and act is None and not ld_in and not ld_out:
         return None, ()
     e = _lib.Epilogue()
+    e.ld_in, e.ld_out = ld_in, ld_out
     keep = []
     if bias is not None:
         bias = bias.detach().to(device=feats.device, dtype=feats.dtype).contiguous()
@@ -558,7 +574,12 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
     nothing, so a loop of layers can be captured into a HIP graph."""
     lib = _lib.load()
     _require_cuda(feats, "feats")
-    feats = feats.contiguous()
+    # the deferred-scatter and output-stationary kernels take column slices of wider matrices in place (the halves
+    # of a concatenated skip connection); everything else gets dense rows
+    strided_ok = dataflow in (DATAFLOW_FDS, DATAFLOW_OS)
+    ld_in = _row_stride(feats) if strided_ok else -1
+    if ld_in < 0:
+        feats, ld_in = feats.contiguous(), 0
     weight = weight.contiguous()
     if weight.dim() == 2:
         weight = weight.unsqueeze(0)
@@ -581,11 +602,20 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
     dev = feats.device
     s = _stream(dev)
     mid = _mid(km.ks) if km.subm else -1
+    ld_out, slice_out = 0, None
     if out is None:
         out = torch.empty((n_out, c_out), dtype=feats.dtype, device=dev)
-    elif out.shape != (n_out, c_out) or out.dtype != feats.dtype or out.device != dev or not out.is_contiguous():
-        raise ValueError(f"out must be a contiguous [{n_out}, {c_out}] {feats.dtype} tensor on {dev}")
-    epi, _keep = _epilogue(feats, n_out, c_out, bias, residual, act)
+    elif out.shape != (n_out, c_out) or out.dtype != feats.dtype or out.device != dev:
+        raise ValueError(f"out must be a [{n_out}, {c_out}] {feats.dtype} tensor on {dev}")
+    elif not out.is_contiguous():
+        ld_out = _row_stride(out)
+        if ld_out < 0:
+            raise ValueError("out must be contiguous or a column slice of a row-major matrix (16-byte aligned, "
+                             "row stride and width multiples of 8 elements)")
+        if not strided_ok:       # this dataflow stores dense rows: they are copied into the slice afterwards
+            slice_out, ld_out = out, 0
+            out = torch.empty((n_out, c_out), dtype=feats.dtype, device=dev)
+    epi, _keep = _epilogue(feats, n_out, c_out, bias, residual, act, ld_in, ld_out)
     if dataflow == DATAFLOW_FOD:
         imap, omap = (km.omap, km.imap) if transposed else (km.imap, km.omap)
         ws_bytes = lib.pce_conv_fod_workspace_bytes(n_out, c_out, dt)
@@ -639,6 +669,9 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
                                        c_in, c_out, kv, nbr.data_ptr(), epi, s))
     else:
         raise NotImplementedError(f"unknown dataflow {dataflow}")
+    if slice_out is not None:
+        slice_out.copy_(out)
+        return slice_out
     return out
 
 

@@ -68,6 +68,7 @@ struct TileArgs {
   long long items;   // (tile, column slab) work items of the launch
   int slabs;         // column slabs per tile
   int kv, c_in, c_out;
+  int lda, ldo;      // elements between consecutive rows of A and of `out` (rows of buf, res and out_alt are dense)
   int w_fixed;
   int mode, epi;
   int a_vec, w_vec, o_vec, b_vec;  // 16-byte accesses allowed on A rows / W rows / out rows / buf rows
@@ -232,13 +233,13 @@ struct AFrag<float> {
 
 template <bool FAST>
 __device__ __forceinline__ void load_rows(AFrag<half_t> &f, const half_t *__restrict__ A, int arow, int k0, int klen,
-                                          int c_in, int a_vec, int g) {
+                                          int c_in, int lda, int a_vec, int g) {
 #pragma unroll
   for (int s = 0; s < Cfg<half_t>::KC / 16; ++s) {
     int k = k0 + s * 16 + g * 8;
     half8 v = {0, 0, 0, 0, 0, 0, 0, 0};
     if (arow >= 0 && s * 16 < klen) {
-      const half_t *p = A + (long long)arow * c_in + k;
+      const half_t *p = A + (long long)arow * lda + k;
       if (FAST) {
         if (k < c_in) v = *reinterpret_cast<const half8 *>(p);
       } else if (a_vec && k + 8 <= c_in) {
@@ -255,13 +256,13 @@ __device__ __forceinline__ void load_rows(AFrag<half_t> &f, const half_t *__rest
 
 template <bool FAST>
 __device__ __forceinline__ void load_rows(AFrag<float> &f, const float *__restrict__ A, int arow, int k0, int klen,
-                                          int c_in, int a_vec, int g) {
+                                          int c_in, int lda, int a_vec, int g) {
 #pragma unroll
   for (int s = 0; s < Cfg<float>::KC / 8; ++s) {
     int k = k0 + s * 8 + g * 4;
     f32x4 v = {0.f, 0.f, 0.f, 0.f};
     if (arow >= 0 && s * 8 < klen) {
-      const float *p = A + (long long)arow * c_in + k;
+      const float *p = A + (long long)arow * lda + k;
       if (FAST) {
         if (k < c_in) v = *reinterpret_cast<const f32x4 *>(p);
       } else if (a_vec && k + 4 <= c_in) {
@@ -631,7 +632,7 @@ __device__ __forceinline__ void store_row_pieces_slow(const float (&V)[NB][2][8]
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         int col = n0 + nb * 32 + 16 * h + 8 * g + j;
-        if (col < a.c_out) out[(long long)orow * a.c_out + col] = (TO)V[nb][h][j];
+        if (col < a.c_out) out[(long long)orow * a.ldo + col] = (TO)V[nb][h][j];
       }
 }
 
@@ -643,7 +644,8 @@ __device__ __forceinline__ void store_row_pieces_slow(const float (&V)[NB][2][8]
 // runs, but the next layer then finds none of them in the L2 of its XCD.  The host decides per launch (set_out).
 template <typename TO, int NB, int ROWS = (sizeof(TO) == 2 ? 32 : 16), bool SPLIT = false>
 __device__ __forceinline__ void store_rows_via_lds(const float (&V)[NB][2][8], void *region, TO *out, int orow,
-                                                   const TileArgs &a, int n0, int lane, int l32, int g, bool stream) {
+                                                   const TileArgs &a, int n0, int lane, int l32, int g, bool stream,
+                                                   int ld_out = -1) {   // row stride of `out` where it is not a.ldo
   constexpr int NT = NB * 32;
   constexpr int EPP = 16 / sizeof(TO);              // elements per piece
   constexpr int LDP = (NT + 8) / EPP;               // row stride in pieces; ROWS rows per pass
@@ -687,12 +689,14 @@ __device__ __forceinline__ void store_rows_via_lds(const float (&V)[NB][2][8], v
       int col = n0 + ch * EPP;
       OV y = R[lr * LDP + ch];
       TO *base = out;
+      int ld = ld_out >= 0 ? ld_out : a.ldo;
       if (SPLIT && dst >= a.n_split) {
         base = (TO *)a.out_alt;
         dst -= a.n_split;
+        ld = a.c_out;
       }
       if (dst >= 0 && col < a.c_out) {
-        OV *dp = reinterpret_cast<OV *>(base + (long long)dst * a.c_out + col);
+        OV *dp = reinterpret_cast<OV *>(base + (long long)dst * ld + col);
         if (stream)
           __builtin_nontemporal_store(y, dp);
         else
@@ -776,7 +780,7 @@ __global__ void __launch_bounds__(256, ((TMODE >= 0 && sizeof(T) == 2 && NB <= 2
   if (mode != MODE_OS) {
     load_weights<NT, FAST>(wr, W + (long long)w_begin * a.c_in * a.c_out,
                            Wp ? Wp + (long long)w_begin * a.k8_total * a.n_pad * 8 : nullptr, 0, n0, a);
-    load_rows<FAST>(af, A, arow, 0, klen0, a.c_in, a.a_vec, g);
+    load_rows<FAST>(af, A, arow, 0, klen0, a.c_in, a.lda, a.a_vec, g);
   }
   // Partial rows: the tile's contiguous range [tb, te) comes from two scalar loads (uniform index),
   // so the first round of partial rows is requested together with the feature rows; the per-lane
@@ -818,7 +822,7 @@ __global__ void __launch_bounds__(256, ((TMODE >= 0 && sizeof(T) == 2 && NB <= 2
       int klen = a.c_in - k0 < KC ? a.c_in - k0 : KC;
       if (mode == MODE_OS || k0 > 0) {
         load_weights<NT, FAST>(wr, Wk, Pk, k0, n0, a);
-        load_rows<FAST>(af, A, arow, k0, klen, a.c_in, a.a_vec, g);
+        load_rows<FAST>(af, A, arow, k0, klen, a.c_in, a.lda, a.a_vec, g);
       }
       if (lds_used) lds_barrier();  // the previous chunk's LDS reads are complete
       store_weights<NT>(Wl, wr);
@@ -930,7 +934,7 @@ __global__ void __launch_bounds__(256, 4) wave_gemm_kernel(TileArgs pair, TileAr
 #pragma unroll
   for (int it = 0; it < NI; ++it) {
     const int e = it * 64 + lane, r = e / PPR, sl = e % PPR;
-    const half_t *gp = A + src[it] * a.c_in + ((sl ^ row_swizzle<PPR>(r)) * 8);
+    const half_t *gp = A + src[it] * a.lda + ((sl ^ row_swizzle<PPR>(r)) * 8);
     // LDS destination: wave-uniform base, the hardware adds lane * 16 bytes
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
                                      (__attribute__((address_space(3))) void *)&Pl[wave][it * 64], 16, 0, 0);
@@ -974,7 +978,8 @@ __global__ void __launch_bounds__(256, 4) wave_gemm_kernel(TileArgs pair, TileAr
         for (int j = 0; j < 8; ++j) V[nb][h][j] = alone ? act_apply(V[nb][h][j], centre.act, centre.slope) : V[nb][h][j];
   }
   half_t *out = (half_t *)(is_pair ? pair.out : centre.out);
-  store_rows_via_lds<half_t, NB>(V, Pl[wave], out, orow, a, 0, lane, l32, g, is_pair ? pair.stream : centre.stream);
+  store_rows_via_lds<half_t, NB>(V, Pl[wave], out, orow, a, 0, lane, l32, g, is_pair ? pair.stream : centre.stream,
+                                 is_pair ? pair.ldo : centre.ldo);
 }
 
 // pair chunks and centre rows of one layer in one launch (either part may be empty): 32 rows per wavefront, the
@@ -1114,10 +1119,10 @@ __device__ __forceinline__ void pipe_issue_weights(const half_t *Wk, int k0, int
 
 // always issued (row 0 stands in for a missing row; the caller zeroes it when the fragment is taken into
 // use): the wait before the barrier counts the loads of a round
-__device__ __forceinline__ void pipe_load_rows(u32x4 (&raw)[PIPE_ROW_LOADS], const half_t *A, int arow, int c_in, int k0, int g) {
+__device__ __forceinline__ void pipe_load_rows(u32x4 (&raw)[PIPE_ROW_LOADS], const half_t *A, int arow, int lda, int k0, int g) {
   int r = arow >= 0 ? arow : 0;
 #pragma unroll
-  for (int s2 = 0; s2 < PIPE_ROW_LOADS; ++s2) raw[s2] = load16_untracked(A + (long long)r * c_in + k0 + s2 * 16 + g * 8);
+  for (int s2 = 0; s2 < PIPE_ROW_LOADS; ++s2) raw[s2] = load16_untracked(A + (long long)r * lda + k0 + s2 * 16 + g * 8);
 }
 
 // PMODE = MODE_DENSE or MODE_FOD_BUF: every tile is of that kind and `c` is not read.  PMODE = PIPE_BOTH:
@@ -1175,10 +1180,10 @@ __global__ void __launch_bounds__(256, 4) pipe_gemm_kernel(TileArgs a, TileArgs 
   // prologue: weight chunks 0 and 1, feature chunks 0 and 1 (issue order: W0, A0, W1, A1)
   u32x4 raw[2][PIPE_ROW_LOADS];
   pipe_issue_weights(Wk, 0, n0, a.n_pad, lds, wave, lane);
-  pipe_load_rows(raw[0], A, arow, a.c_in, 0, g);
+  pipe_load_rows(raw[0], A, arow, a.lda, 0, g);
   if (kch > 1) {
     pipe_issue_weights(Wk, KC, n0, a.n_pad, lds + STAGE, wave, lane);
-    pipe_load_rows(raw[1], A, arow, a.c_in, KC, g);
+    pipe_load_rows(raw[1], A, arow, a.lda, KC, g);
   }
   const bool wave_has = __ballot(arow >= 0) != 0ull;
   const half8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -1197,7 +1202,7 @@ __global__ void __launch_bounds__(256, 4) pipe_gemm_kernel(TileArgs a, TileArgs 
         af[s2] = arow >= 0 ? __builtin_bit_cast(half8, landed[s2]) : zero;                                 \
     /* features of chunk t+2 first, so that the weight loads below are the youngest in flight */           \
     if (t + 2 < kch) {                                                                                     \
-      pipe_load_rows(raw[SLOT_], A, arow, a.c_in, (t + 2) * KC, g);                                        \
+      pipe_load_rows(raw[SLOT_], A, arow, a.lda, (t + 2) * KC, g);                                        \
       /* weight chunk t+2 -> the stage that chunk t-1 has just released */                                 \
       pipe_issue_weights(Wk, (t + 2) * KC, n0, a.n_pad, lds + st2 * STAGE, wave, lane);                    \
       st2 = st2 + 1 == PIPE_ST ? 0 : st2 + 1;                                                              \
@@ -1240,7 +1245,8 @@ __global__ void __launch_bounds__(256, 4) pipe_gemm_kernel(TileArgs a, TileArgs 
     store_rows_via_lds<half_t, NB, 32, true>(V, lds + wave * WaveLds<NB>::PIECES, out, orow, a, n0, lane, l32, g, a.stream);
   else
     store_rows_via_lds<half_t, NB>(V, lds + wave * WaveLds<NB>::PIECES, out, orow, a, n0, lane, l32, g,
-                                   (PMODE == PIPE_BOTH && dense) ? c.stream : a.stream);
+                                   (PMODE == PIPE_BOTH && dense) ? c.stream : a.stream,
+                                   (PMODE == PIPE_BOTH && dense) ? c.ldo : a.ldo);
 }
 
 // The eight weight fragments of a step are requested before its first MFMA, and every MFMA waits only for
@@ -1338,7 +1344,7 @@ __global__ void __launch_bounds__(256, SUB == 1 ? 3 : 2) os_pipe_kernel(TileArgs
     const int arow_i = nbrs[ikp][wave * 32 + l32];                                                           \
     carow[SLOT_] = arow_i;                                                                                   \
     _Pragma("unroll") for (int sub = 0; sub < SUB; ++sub) {                                                  \
-      pipe_load_rows(raw[SLOT_][sub], A, arow_i, a.c_in, (it * SUB + sub) * KC, g);                          \
+      pipe_load_rows(raw[SLOT_][sub], A, arow_i, a.lda, (it * SUB + sub) * KC, g);                          \
       pipe_issue_weights(Wk, (it * SUB + sub) * KC, n0, a.n_pad, lds + ist * RSTAGE + sub * STAGE, wave, lane); \
     }                                                                                                        \
     ist = ist + 1 == PIPE_ST ? 0 : ist + 1;                                                                  \
@@ -1590,7 +1596,7 @@ __global__ void __launch_bounds__(256) rowsum_kernel(const T *__restrict__ buf, 
                                                      const int *__restrict__ csr, T *__restrict__ out,
                                                      const T *__restrict__ bias, const T *__restrict__ res, int act,
                                                      float slope, const int *__restrict__ rows,
-                                                     const int *__restrict__ count, int stream) {
+                                                     const int *__restrict__ count, int stream, int ldo) {
   typedef typename VecOf<T, VEC>::type V;
   int rows_per_block = 256 / G;
   int sub = threadIdx.x % G;
@@ -1633,7 +1639,7 @@ __global__ void __launch_bounds__(256) rowsum_kernel(const T *__restrict__ buf, 
       }
 #pragma unroll
       for (int j = 0; j < VEC; ++j) reinterpret_cast<T *>(&y)[j] = (T)act_apply(acc[j], act, slope);
-      store_maybe_stream(reinterpret_cast<V *>(&out[row * c_out + (long long)v * VEC]), y, stream != 0);
+      store_maybe_stream(reinterpret_cast<V *>(&out[row * ldo + (long long)v * VEC]), y, stream != 0);
     }
   }
 }
@@ -1676,7 +1682,7 @@ template <typename T, int VEC, bool BY_ROW>
 __global__ void __launch_bounds__(256) rowsum_pairs_kernel(const T *__restrict__ buf, long long n_items, int c_out, int G,
                                                            const int *__restrict__ omap, const int *__restrict__ oslot,
                                                            const int *__restrict__ csr, T *__restrict__ out, int act,
-                                                           float slope, int stream) {
+                                                           float slope, int stream, int ldo) {
   typedef typename VecOf<T, VEC>::type V;
   long long item = (long long)blockIdx.x * (256 / G) + threadIdx.x / G;
   int sub = threadIdx.x % G;
@@ -1696,7 +1702,7 @@ __global__ void __launch_bounds__(256) rowsum_pairs_kernel(const T *__restrict__
   int row_vecs = c_out / VEC;
   for (int v = sub; v < row_vecs; v += G) {
     const T *bp = buf + (long long)v * VEC;
-    V x = *reinterpret_cast<const V *>(&out[(long long)row * c_out + (long long)v * VEC]);
+    V x = *reinterpret_cast<const V *>(&out[(long long)row * ldo + (long long)v * VEC]);
     float acc[VEC];
 #pragma unroll
     for (int j = 0; j < VEC; ++j) acc[j] = (float)(reinterpret_cast<const T *>(&x)[j]);
@@ -1717,14 +1723,15 @@ __global__ void __launch_bounds__(256) rowsum_pairs_kernel(const T *__restrict__
     }
 #pragma unroll
     for (int j = 0; j < VEC; ++j) reinterpret_cast<T *>(&x)[j] = (T)act_apply(acc[j], act, slope);
-    store_maybe_stream(reinterpret_cast<V *>(&out[(long long)row * c_out + (long long)v * VEC]), x, stream != 0);
+    store_maybe_stream(reinterpret_cast<V *>(&out[(long long)row * ldo + (long long)v * VEC]), x, stream != 0);
   }
 }
 
 // picks the vector width and the iteration space of the row sum
 template <typename T>
 static int launch_rowsum_pairs(const T *buffer, T *out, int64_t n_out, int64_t n_pairs, int c_out, const int *omap,
-                               const int *oslot, const int *ocsr, int act, float slope, hipStream_t s) {
+                               const int *oslot, const int *ocsr, int act, float slope, hipStream_t s, int ldo = 0) {
+  if (ldo <= 0) ldo = c_out;
   if (n_pairs <= 0) return PCE_OK;
   constexpr int VEC = sizeof(T) == 2 ? 8 : 4;
   const bool vec = (c_out % VEC == 0) && (((uintptr_t)out | (uintptr_t)buffer) & 15) == 0;
@@ -1736,7 +1743,7 @@ static int launch_rowsum_pairs(const T *buffer, T *out, int64_t n_out, int64_t n
   dim3 grid((unsigned)pce_div_up(items, 256 / G)), block(256);
 #define PCE_ROWSUM(V_, B_)                                                                                        \
   hipLaunchKernelGGL((rowsum_pairs_kernel<T, V_, B_>), grid, block, 0, s, buffer, items, c_out, G, omap, oslot, ocsr, out, \
-                     act, slope, stream_policy((long long)n_out * c_out * (long long)sizeof(T)))
+                     act, slope, stream_policy((long long)n_out * c_out * (long long)sizeof(T)), ldo)
   if (vec && by_row)
     PCE_ROWSUM(VEC, true);
   else if (vec)
@@ -1810,7 +1817,7 @@ static int check_qsum(const char *fn, int64_t qsum) {
 
 // features / weights / packed weights / sizes common to every launch of one layer
 template <typename T>
-static TileArgs base_args(const void *in, const void *w, const void *wp, int kv, int c_in, int c_out) {
+static TileArgs base_args(const void *in, const void *w, const void *wp, int kv, int c_in, int c_out, int lda = 0) {
   constexpr int VEC = sizeof(T) == 2 ? 8 : 4;
   TileArgs a = {};
   a.A = in;
@@ -1819,6 +1826,8 @@ static TileArgs base_args(const void *in, const void *w, const void *wp, int kv,
   a.kv = kv;
   a.c_in = c_in;
   a.c_out = c_out;
+  a.lda = lda > 0 ? lda : c_in;
+  a.ldo = c_out;
   a.k8_total = (c_in + 7) / 8;
   a.n_pad = (c_out + 31) / 32 * 32;
   a.a_vec = (c_in % VEC == 0) && aligned16(in);
@@ -1828,9 +1837,10 @@ static TileArgs base_args(const void *in, const void *w, const void *wp, int kv,
 
 // `rows` = rows of the tensor `out` points to (0: not known, no streaming)
 template <typename T>
-static void set_out(TileArgs *a, void *out, bool f32out, long long rows = 0) {
+static void set_out(TileArgs *a, void *out, bool f32out, long long rows = 0, int ldo = 0) {
   // a lane of the row epilogue owns 8 consecutive columns, whatever the element type
   a->out = out;
+  a->ldo = ldo > 0 ? ldo : a->c_out;
   a->o_vec = (a->c_out % 8 == 0) && aligned16(out);
   a->stream = rows > 0 ? stream_policy(rows * a->c_out * (f32out ? 4 : (long long)sizeof(T))) : 0;
 }
@@ -1850,14 +1860,25 @@ struct Epi {
   const void *bias, *res;
   int act;
   float slope;
+  int lda, ldo;   // row strides of the input and output matrices in elements, 0 = dense
   bool any() const { return bias || res || act != PCE_ACT_NONE; }
 };
 
-static int read_epilogue(const char *fn, const pce_epilogue_t *e, const void *out, Epi *o) {
+static int read_epilogue(const char *fn, const pce_epilogue_t *e, const void *out, Epi *o, int c_in = 0, int c_out = 0) {
   o->bias = o->res = nullptr;
   o->act = PCE_ACT_NONE;
   o->slope = 0.f;
+  o->lda = o->ldo = 0;
   if (!e) return PCE_OK;
+  // row strides: only the entry points that pass their channel counts take them
+  if ((e->ld_in != 0 && e->ld_in != c_in) || (e->ld_out != 0 && e->ld_out != c_out)) {
+    if (c_in <= 0) PCE_FAIL(PCE_EINVAL, "%s: this entry point takes dense feature matrices only (ld_in=%lld, ld_out=%lld)", fn, (long long)e->ld_in, (long long)e->ld_out);
+    if ((e->ld_in != 0 && (e->ld_in < c_in || e->ld_in % 8)) || (e->ld_out != 0 && (e->ld_out < c_out || e->ld_out % 8)) ||
+        e->ld_in >= (1ll << 31) || e->ld_out >= (1ll << 31))
+      PCE_FAIL(PCE_EINVAL, "%s: row strides (ld_in=%lld, ld_out=%lld) must be multiples of 8 elements, at least the channel counts (%d, %d)", fn, (long long)e->ld_in, (long long)e->ld_out, c_in, c_out);
+    o->lda = (int)e->ld_in;
+    o->ldo = (int)e->ld_out;
+  }
   if (e->act != PCE_ACT_NONE && e->act != PCE_ACT_RELU && e->act != PCE_ACT_LEAKY_RELU)
     PCE_FAIL(PCE_EINVAL, "%s: unknown activation %d", fn, (int)e->act);
   if (e->residual && e->residual == out) PCE_FAIL(PCE_EINVAL, "%s: the residual must not alias the output", fn);
@@ -2133,8 +2154,8 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
   if (!buffer && qsum > 0) {
     // Every output row has exactly one pair (a transposed layer whose kernel equals its stride: each fine
     // voxel has one parent): a pair's product is its output row, stored once with the epilogue, no partial rows.
-    TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
-    set_out<T>(&a, out, false, n_out);
+    TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out, e.lda);
+    set_out<T>(&a, out, false, n_out, e.ldo);
     set_host_pos(&a, kpos_host, qkpos_host);
     a.imap = imap;
     a.oslot = omap;
@@ -2148,14 +2169,14 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
   if (mid >= 0 && qsum > 0 && omap && stage_on(4)) {
     // Pair chunks and centre GEMM share one launch (neither reads what the other writes); a pass
     // over the pairs then adds every output row's partial rows to the centre term stored there.
-    TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
+    TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out, e.lda);
     set_out<T>(&a, buffer, false, n_pairs);
     set_host_pos(&a, kpos_host, qkpos_host);
     a.imap = imap;
     a.oslot = oslot;
     a.items = qsum / 32;
-    TileArgs c = base_args<T>(in, w, wp, kv, c_in, c_out);
-    set_out<T>(&c, out, false, n_out);
+    TileArgs c = base_args<T>(in, w, wp, kv, c_in, c_out, e.lda);
+    set_out<T>(&c, out, false, n_out, e.ldo);
     c.w_fixed = mid;
     c.n_rows = n_out;
     c.items = pce_div_up(n_out, 32);
@@ -2165,7 +2186,7 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
     if (a.host_pos && wave_gemm_ok(a, sizeof(T)) && wave_gemm_ok(c, sizeof(T)) && aligned16(buffer) && epi_aligned(e)) {
       if (stage_on(1) && (rc = launch_wave_gemm(a, c, s))) return rc;
       if (stage_on(2) && (rc = launch_rowsum_pairs<T>((const T *)buffer, (T *)out, n_out, n_pairs, c_out, omap, oslot, ocsr,
-                                                      e.act, e.slope, s)))
+                                                      e.act, e.slope, s, e.ldo)))
         return rc;
       return PCE_OK;
     }
@@ -2174,8 +2195,8 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
     // Routed pair tiles (a layer without centre offset): the only pair of an output row stores the finished row
     // with the epilogue, the pairs of the other rows store partial rows; the row sum then visits only rows with
     // two pairs or more.  Taken by the pipelined kernel's shapes; the others ignore the routing.
-    TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
-    set_out<T>(&a, out, false, n_out);
+    TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out, e.lda);
+    set_out<T>(&a, out, false, n_out, e.ldo);
     set_host_pos(&a, kpos_host, qkpos_host);
     a.imap = imap;
     a.oslot = route + PCE_ROUTE_HEAD;
@@ -2193,7 +2214,7 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
     }
   }
   if (qsum > 0 && stage_on(1) && !multi_rows) {
-    TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
+    TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out, e.lda);
     set_out<T>(&a, buffer, false, n_pairs);
     set_host_pos(&a, kpos_host, qkpos_host);
     a.imap = imap;
@@ -2210,8 +2231,8 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
       // at 9 (C 128), 4-6 % slower at 9-13 pairs per row with 256 channels, where the launches stay separate;
       // so do those of a centre GEMM that fills the machine twice over by itself (nothing to gain, and a
       // network on 954 k voxels ran 3 % slower with them combined).
-      TileArgs c = base_args<T>(in, w, wp, kv, c_in, c_out);
-      set_out<T>(&c, out, false, n_out);
+      TileArgs c = base_args<T>(in, w, wp, kv, c_in, c_out, e.lda);
+      set_out<T>(&c, out, false, n_out, e.ldo);
       c.mode = MODE_DENSE;
       c.epi = EPI_ROWS;
       c.w_fixed = mid;
@@ -2221,7 +2242,7 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
       set_epi(&c, e);
       if (pipe_gemm_ok(c, sizeof(T))) {
         if ((rc = launch_pipe_both(a, qsum / PCE_QUANTUM, c, pce_div_up(n_out, 128), s))) return rc;
-        return launch_rowsum_pairs<T>((const T *)buffer, (T *)out, n_out, n_pairs, c_out, omap, oslot, ocsr, e.act, e.slope, s);
+        return launch_rowsum_pairs<T>((const T *)buffer, (T *)out, n_out, n_pairs, c_out, omap, oslot, ocsr, e.act, e.slope, s, e.ldo);
       }
     }
     if (a.host_pos && wave_gemm_ok(a, sizeof(T)) && stage_on(4)) {
@@ -2237,8 +2258,8 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
   if (mid >= 0 && omap && stage_on(4)) {
     // plain centre GEMM (bias and residual fused, activation on rows without partial rows), then the
     // pass over the pairs that adds each row's partial rows: no partial-row staging in the GEMM epilogue
-    TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
-    set_out<T>(&a, out, false, n_out);
+    TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out, e.lda);
+    set_out<T>(&a, out, false, n_out, e.ldo);
     a.mode = MODE_DENSE;
     a.epi = EPI_ROWS;
     a.w_fixed = mid;
@@ -2247,11 +2268,11 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
     a.act_alone_only = 1;
     set_epi(&a, e);
     if ((rc = launch_tile<T>(a, pce_div_up(n_out, 128), s))) return rc;
-    return launch_rowsum_pairs<T>((const T *)buffer, (T *)out, n_out, n_pairs, c_out, omap, oslot, ocsr, e.act, e.slope, s);
+    return launch_rowsum_pairs<T>((const T *)buffer, (T *)out, n_out, n_pairs, c_out, omap, oslot, ocsr, e.act, e.slope, s, e.ldo);
   }
   if (mid >= 0) {
-    TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
-    set_out<T>(&a, out, false, n_out);
+    TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out, e.lda);
+    set_out<T>(&a, out, false, n_out, e.ldo);
     a.mode = MODE_DENSE;
     a.epi = EPI_ROWS_CSR;
     a.w_fixed = mid;
@@ -2271,7 +2292,8 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
     if (multi_rows && blocks > 1024) blocks = 1024;
     hipLaunchKernelGGL((rowsum_kernel<T, VEC>), dim3((unsigned)blocks), dim3(256), 0, s,
                        (const T *)buffer, (long long)n_out, c_out, G, ocsr, (T *)out, (const T *)e.bias, (const T *)e.res,
-                       e.act, e.slope, multi_rows, multi_count, stream_policy((long long)n_out * c_out * (long long)sizeof(T)));
+                       e.act, e.slope, multi_rows, multi_count, stream_policy((long long)n_out * c_out * (long long)sizeof(T)),
+                       e.ldo > 0 ? e.ldo : c_out);
   } else {
     int G = pow2_at_least(c_out);
     if (G > 64) G = 64;
@@ -2279,7 +2301,8 @@ static int fds_impl(const void *in, const void *w, const void *wp, void *out, in
     if (multi_rows && blocks > 1024) blocks = 1024;
     hipLaunchKernelGGL((rowsum_kernel<T, 1>), dim3((unsigned)blocks), dim3(256), 0, s,
                        (const T *)buffer, (long long)n_out, c_out, G, ocsr, (T *)out, (const T *)e.bias, (const T *)e.res,
-                       e.act, e.slope, multi_rows, multi_count, stream_policy((long long)n_out * c_out * (long long)sizeof(T)));
+                       e.act, e.slope, multi_rows, multi_count, stream_policy((long long)n_out * c_out * (long long)sizeof(T)),
+                       e.ldo > 0 ? e.ldo : c_out);
   }
   PCE_LAUNCH_CHECK("rowsum");
   return PCE_OK;
@@ -2333,7 +2356,7 @@ extern "C" int pce_conv_fwd_fds(const void *in, const void *w, const void *wp, v
   int rc = check_common("pce_conv_fwd_fds", in, w, out, dtype, n_in, n_out, c_in, c_out, kv, mid);
   if (rc || (rc = check_qsum("pce_conv_fwd_fds", qsum))) return rc;
   Epi e;
-  if ((rc = read_epilogue("pce_conv_fwd_fds", epilogue, out, &e))) return rc;
+  if ((rc = read_epilogue("pce_conv_fwd_fds", epilogue, out, &e, c_in, c_out))) return rc;
   if (!ocsr || !kpos || !qkpos || (qsum > 0 && (!imap || !oslot))) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_fds: null map pointer");
   if (n_pairs < 0 || n_pairs > qsum) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_fds: n_pairs=%lld outside [0, qsum]", (long long)n_pairs);
   if (!buffer && n_pairs > 0) {
@@ -2352,8 +2375,8 @@ extern "C" int pce_conv_fwd_fds(const void *in, const void *w, const void *wp, v
 template <typename T>
 static int os_impl(const void *in, const void *w, const void *wp, void *out, int64_t n_out, int c_in, int c_out, int kv,
                    const int *nbr, const Epi &e, hipStream_t s) {
-  TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out);
-  set_out<T>(&a, out, false, n_out);
+  TileArgs a = base_args<T>(in, w, wp, kv, c_in, c_out, e.lda);
+  set_out<T>(&a, out, false, n_out, e.ldo);
   set_epi(&a, e);
   a.nbr = nbr;
   a.n_rows = n_out;
@@ -2369,7 +2392,7 @@ extern "C" int pce_conv_fwd_os(const void *in, const void *w, const void *wp, vo
   if (rc) return rc;
   if (!nbr) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_os: null neighbour table");
   Epi e;
-  if ((rc = read_epilogue("pce_conv_fwd_os", epilogue, out, &e))) return rc;
+  if ((rc = read_epilogue("pce_conv_fwd_os", epilogue, out, &e, c_in, c_out))) return rc;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == PCE_F16) return os_impl<half_t>(in, w, wp, out, n_out, c_in, c_out, kv, nbr, e, s);
   return os_impl<float>(in, w, wp, out, n_out, c_in, c_out, kv, nbr, e, s);

@@ -43,11 +43,12 @@ class ConvBN(nn.Module):
             self.conv.bias = nn.Parameter(b)
         self.bn = None
 
-    def forward(self, x: spTensor, residual: spTensor = None, relu_after_residual: bool = False) -> spTensor:
-        """With the norm folded away, bias, the optional residual and the ReLU run inside the conv kernels."""
+    def forward(self, x: spTensor, residual: spTensor = None, relu_after_residual: bool = False, out=None) -> spTensor:
+        """With the norm folded away, bias, the optional residual and the ReLU run inside the conv kernels, and
+        the features can go straight to `out` (a column slice of a wider matrix, see SparseResUNet.forward)."""
         act = self.relu.as_epilogue() if self.relu is not None else ("relu" if relu_after_residual else None)
         if self.bn is None:
-            return self.conv(x, act=act, residual=residual)
+            return self.conv(x, act=act, residual=residual, out=out)
         # training form: the residual sum and the ReLU ride on the norm's affine pass
         return self.bn(self.conv(x), residual=residual, act=act)
 
@@ -60,9 +61,9 @@ class ResidualBlock(nn.Module):
         self.shortcut = None if cin == cout else ConvBN(cin, cout, 1, relu=False)
         self.relu = ReLU(True)
 
-    def forward(self, x: spTensor) -> spTensor:
+    def forward(self, x: spTensor, out=None) -> spTensor:
         s = x if self.shortcut is None else self.shortcut(x)
-        return self.b(self.a(x), residual=s, relu_after_residual=True)      # relu(b(a(x)) + s)
+        return self.b(self.a(x), residual=s, relu_after_residual=True, out=out)      # relu(b(a(x)) + s)
 
 
 class SparseResUNet(nn.Module):
@@ -108,6 +109,8 @@ class SparseResUNet(nn.Module):
 
     def forward(self, x: spTensor) -> spTensor:
         prebuild_maps(x, self.map_plan())      # no host wait is left between the layers below
+        if self._skips_in_place(x):
+            return self._forward_skips_in_place(x)
         x = self.stem(x)
         feats = [x]
         for down, enc in zip(self.down, self.enc):
@@ -117,4 +120,42 @@ class SparseResUNet(nn.Module):
         for up, dec in zip(self.up, self.dec):
             x = up(x)
             x = dec(cat([x, feats.pop()]))
+        return self.head(x)
+
+    def _skips_in_place(self, x: spTensor) -> bool:
+        """Inference with every norm folded, on the GPU, all widths multiples of 8 channels: the two producers of
+        a skip connection can then write their halves of the concatenated matrix themselves."""
+        if torch.is_grad_enabled() and any(p.requires_grad for p in self.parameters()):
+            return False
+        if not x.feats.is_cuda or any(isinstance(m, ConvBN) and m.bn is not None for m in self.modules()):
+            return False
+        widths = [self.stem[1].conv.out_channels] + [e[1].b.conv.out_channels for e in self.enc] + \
+                 [u.conv.out_channels for u in self.up]
+        return all(w % 8 == 0 for w in widths)
+
+    def _forward_skips_in_place(self, x: spTensor) -> spTensor:
+        """The same network with the concatenation of each decoder stage done by its producers: the encoder layer
+        whose output is kept writes the right-hand columns of a [rows, c_up + c_skip] matrix, the transposed layer
+        the left-hand ones later, and the decoder block reads the matrix; the layers that consume the kept output
+        on the way down gather from its columns in place.  Same kernels, same values, no pass that copies."""
+        def joined(rows, like, c_up, c_skip):
+            return torch.empty((rows, c_up + c_skip), dtype=like.dtype, device=like.device)
+        ups = [u.conv.out_channels for u in self.up][::-1]      # c_up of the stage that ends at level 0, 1, ...
+        x = self.stem[0](x)
+        buf = joined(x.feats.shape[0], x.feats, ups[0], self.stem[1].conv.out_channels)
+        x = self.stem[1](x, out=buf[:, ups[0]:])
+        bufs = [buf]
+        last = len(self.enc) - 1
+        for lv, (down, enc) in enumerate(zip(self.down, self.enc)):
+            x = enc[0](down(x))
+            if lv < last:
+                buf = joined(x.feats.shape[0], x.feats, ups[lv + 1], enc[1].b.conv.out_channels)
+                x = enc[1](x, out=buf[:, ups[lv + 1]:])
+                bufs.append(buf)
+            else:
+                x = enc[1](x)            # the deepest output is not a skip
+        for up, dec in zip(self.up, self.dec):
+            buf = bufs.pop()
+            x = up(x, out=buf[:, :up.conv.out_channels])
+            x = dec(x._like(buf))
         return self.head(x)

@@ -117,7 +117,10 @@ class conv3d(nn.Module):
             self._bcache_key = key
         return self._bcache
 
-    def forward(self, input: spTensor, act=None, residual: Optional[spTensor] = None) -> spTensor:
+    def forward(self, input: spTensor, act=None, residual: Optional[spTensor] = None,
+                out: Optional[torch.Tensor] = None) -> spTensor:
+        """``out`` (inference only): where the output features go -- a preallocated matrix or a column slice of a
+        wider one, e.g. this layer's half of a concatenated skip connection."""
         if _wants_grad(input.feats, self.kernel, self.bias):
             # training: the parameters themselves go to the autograd function (no cached copies)
             return conv_func(input=input, in_channel=self.in_channels, out_channel=self.out_channels, kernel=self.kernel,
@@ -130,7 +133,7 @@ class conv3d(nn.Module):
                          kernel_size_code=self.kernel_size_code, stride_code=self.stride_code,
                          padding_code=self.padding_code, bias=self._bias_for(input.feats.dtype),
                          transposed=self.transposed, tensorcore=self.tensorcore, dataflow=self.dataflow, packed=packed,
-                         act=act, residual=None if residual is None else residual.feats)
+                         act=act, residual=None if residual is None else residual.feats, out=out)
 
 
 def _pick_dataflow(km: backend.KernelMap, requested: str, c_in: int, c_out: int, dtype, transposed: bool) -> int:
@@ -212,7 +215,7 @@ def _apply_unfused(out: torch.Tensor, residual, act) -> torch.Tensor:
 
 
 def _run(input: spTensor, km: backend.KernelMap, kernel, in_channel, out_channel, transposed, dataflow, packed,
-         bias=None, residual=None, act=None) -> torch.Tensor:
+         bias=None, residual=None, act=None, out=None) -> torch.Tensor:
     feats = input.feats
     if _wants_grad(feats, kernel, bias):
         k = kernel if kernel.dtype == feats.dtype else kernel.to(feats.dtype)
@@ -226,7 +229,7 @@ def _run(input: spTensor, km: backend.KernelMap, kernel, in_channel, out_channel
         feats = torch.nn.functional.pad(feats, (0, kernel.shape[1] - feats.shape[1]))    # see conv3d._weights_for
     df = _pick_dataflow(km, dataflow, in_channel, out_channel, feats.dtype, transposed)
     out = backend.conv_forward(feats, kernel.detach(), km, df, transposed=transposed, buffer=input.buffer, packed=packed,
-                               bias=bias, residual=residual, act=act)
+                               out=out, bias=bias, residual=residual, act=act)
     if layer_log is not None:
         layer_log.append((feats.shape[0], out.shape[0], km.M, in_channel, out_channel, df))
     return out
@@ -355,7 +358,7 @@ def prebuild_maps(input: spTensor, layers) -> None:
 
 
 def conv_func(input: spTensor, in_channel, out_channel, kernel, kernel_size_code, stride_code, padding_code, bias,
-              transposed, tensorcore, dataflow: str = "auto", packed=None, act=None, residual=None) -> spTensor:
+              transposed, tensorcore, dataflow: str = "auto", packed=None, act=None, residual=None, out=None) -> spTensor:
     """Map cache lookup / build, dataflow dispatch, bias (+ optional residual and activation, all
     inside the kernels), metadata propagation (script/spconv.py:291-464)."""
     if kernel_size_code == _UNIT and stride_code == _UNIT:
@@ -367,6 +370,9 @@ def conv_func(input: spTensor, in_channel, out_channel, kernel, kernel_size_code
         if kernel.dtype != input.feats.dtype:
             kernel, packed = kernel.to(input.feats.dtype), None
         out_feats = backend.dense_forward(input.feats, kernel.detach(), packed, bias=bias, residual=residual, act=act)
+        if out is not None:
+            out.copy_(out_feats)
+            out_feats = out
         return input._like(out_feats)
 
     if transposed:
@@ -377,7 +383,7 @@ def conv_func(input: spTensor, in_channel, out_channel, kernel, kernel_size_code
             raise KeyError("transposed conv3d found no cached map for this (kernel, stride): "
                            "the matching strided conv3d must run first on the same tensor family")
         out_coords = input.cbook[output_stride]
-        out_feats = _run(input, km, kernel, in_channel, out_channel, True, dataflow, packed, bias, residual, act)
+        out_feats = _run(input, km, kernel, in_channel, out_channel, True, dataflow, packed, bias, residual, act, out)
         output = spTensor(feats=out_feats, coords=out_coords, buffer=input.buffer, batchsize=input.batchsize,
                           stride=output_stride, init_tag=input.init_tag, coords_max=input.coords_max,
                           coords_min=input.coords_min)
@@ -385,7 +391,7 @@ def conv_func(input: spTensor, in_channel, out_channel, kernel, kernel_size_code
         return output
 
     km, output_stride, coords_min, coords_max = ensure_map(input, kernel_size_code, stride_code, padding_code)
-    out_feats = _run(input, km, kernel, in_channel, out_channel, False, dataflow, packed, bias, residual, act)
+    out_feats = _run(input, km, kernel, in_channel, out_channel, False, dataflow, packed, bias, residual, act, out)
     output = spTensor(feats=out_feats, coords=km.out_coords, buffer=input.buffer, batchsize=input.batchsize,
                       stride=output_stride, init_tag=input.init_tag, coords_max=coords_max, coords_min=coords_min)
     output.kmaps, output.cbook = input.kmaps, input.cbook
