@@ -125,6 +125,14 @@ class KernelMap:
     def has_csr(self) -> bool:
         return self.icsr is not None
 
+    def device_tensors(self):
+        """Tensors that cover the device allocations this map reads (views share them): what another stream has to
+        be told about (``Tensor.record_stream``) before it uses a map whose memory was allocated on this one."""
+        pair_arrays = self.__dict__.get("_cut_imap")
+        first = pair_arrays[0] if isinstance(pair_arrays, tuple) else pair_arrays
+        return [t for t in (first, self.knnz, self.out_coords, self.nbr_out, self.nbr_in, self.icsr, self.route, self.route_t)
+                if t is not None]
+
     def _as_list(self):
         if self.tag == "D1" and self.has_csr:
             return [self.icode, self.ocode, self.icsr, self.ocsr, self.kpos, self.qkpos, self.qsum, (self.n_in, self.n_out)]

@@ -711,6 +711,139 @@ extern "C" int pce_outcoords_emit(const void *ws, int64_t n_in, const pce_geom_t
   return PCE_OK;
 }
 
+// ---- all levels of a chain at once -------------------------------------------------------------------------------
+// When every layer of the chain has kernel = stride and no padding (the down-sampling layers of a U-Net), the voxel
+// a point falls into at level l is its coordinate divided l times, whatever the other points do: one kernel pushes
+// every first-level point through all levels and marks a bit per level, and the scans and the decoding of all
+// levels share their launches -- five launches for the chain instead of five per level.
+struct ChainLevel {
+  unsigned *bits;
+  int *cnt, *sums, *status;
+  int4 *out;
+  long long words, fill_ints;
+  int fill_blk0, scan_blk0, word_blk0;   // first block of this level in the fill / scan / decode grids
+  BitGrid grid;
+  int stride[3], lo[3], hi[3];
+};
+struct ChainDev {
+  int levels;
+  int *summary;                           // [levels][4]: count, status[0..2]
+  ChainLevel lv[PCE_MAX_CHAIN];
+};
+#define CHAIN_FILL_INTS 2048              // per block
+
+__device__ __forceinline__ int chain_level_of(const ChainDev &d, int blk, int which) {
+  int l = 0;
+  for (int i = 1; i < d.levels; ++i) {
+    int b0 = which == 0 ? d.lv[i].fill_blk0 : (which == 1 ? d.lv[i].scan_blk0 : d.lv[i].word_blk0);
+    if (blk >= b0) l = i;
+  }
+  return l;
+}
+
+__global__ void __launch_bounds__(256) chain_fill_kernel(ChainDev d) {
+  const int l = chain_level_of(d, blockIdx.x, 0);
+  const ChainLevel &v = d.lv[l];
+  long long base = (long long)(blockIdx.x - v.fill_blk0) * CHAIN_FILL_INTS;
+  for (int j = threadIdx.x; j < CHAIN_FILL_INTS; j += 256)
+    if (base + j < v.fill_ints) v.bits[base + j] = 0u;
+}
+
+__global__ void __launch_bounds__(256) chain_mark_kernel(const int4 *__restrict__ coords, long long n_in, ChainDev d) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_in) return;
+  int4 c = coords[i];
+  if (!pce_coord_ok(c.x, c.y, c.z, c.w)) {
+    d.lv[0].status[0] = 1;
+    return;
+  }
+  if (c.x >= d.lv[0].grid.n_batch) {
+    d.lv[0].status[2] = 1;
+    return;
+  }
+  int p[3] = {c.y, c.z, c.w};
+  for (int l = 0; l < d.levels; ++l) {
+    const ChainLevel &v = d.lv[l];
+    bool ok = true;
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+      p[a] = p[a] / v.stride[a];            // kernel = stride, no padding: the one offset that divides
+      ok &= p[a] >= v.lo[a] && p[a] <= v.hi[a];
+    }
+    if (!ok) return;                        // clipped here: absent from every deeper level too
+    long long bit = (((long long)c.x * v.grid.ext[0] + (p[0] - v.grid.lo[0])) * v.grid.ext[1] + (p[1] - v.grid.lo[1])) *
+                        v.grid.ext[2] + (p[2] - v.grid.lo[2]);
+    atomicOr(&v.bits[bit >> 5], 1u << (bit & 31));
+  }
+}
+
+__global__ void __launch_bounds__(256) chain_scan_local_kernel(ChainDev d) {
+  const int l = chain_level_of(d, blockIdx.x, 1);
+  const ChainLevel &v = d.lv[l];
+  const int blk = blockIdx.x - v.scan_blk0;
+  long long base = (long long)blk * SCAN_TILE + (long long)threadIdx.x * SCAN_ITEMS;
+  int x[SCAN_ITEMS];
+  int acc = 0;
+#pragma unroll
+  for (int j = 0; j < SCAN_ITEMS; ++j) {
+    x[j] = base + j < v.words ? __popc(v.bits[base + j]) : 0;
+    acc += x[j];
+  }
+  int total;
+  int run = block_exclusive_scan(acc, &total);
+#pragma unroll
+  for (int j = 0; j < SCAN_ITEMS; ++j) {
+    if (base + j < v.words) v.cnt[base + j] = run;
+    run += x[j];
+  }
+  if (threadIdx.x == 0) v.sums[blk] = total;
+}
+
+__global__ void __launch_bounds__(256) chain_scan_add_kernel(ChainDev d) {
+  const int l = chain_level_of(d, blockIdx.x, 1);
+  const ChainLevel &v = d.lv[l];
+  const int blk = blockIdx.x - v.scan_blk0;
+  if (blk == 0) return;
+  int acc = 0;
+  for (int j = threadIdx.x; j < blk; j += 256) acc += v.sums[j];
+  int total;
+  block_exclusive_scan(acc, &total);
+  long long base = (long long)blk * SCAN_TILE + (long long)threadIdx.x * SCAN_ITEMS;
+#pragma unroll
+  for (int j = 0; j < SCAN_ITEMS; ++j)
+    if (base + j < v.words) v.cnt[base + j] += total;
+}
+
+__global__ void __launch_bounds__(256) chain_expand_kernel(ChainDev d) {
+  const int l = chain_level_of(d, blockIdx.x, 2);
+  const ChainLevel &v = d.lv[l];
+  long long w = (long long)(blockIdx.x - v.word_blk0) * 256 + threadIdx.x;
+  if (w >= v.words) return;
+  if (w == v.words - 1) {                   // the spare last word is zero: its prefix is the level's count
+    int *sm = d.summary + 4 * l;
+    sm[0] = v.cnt[w];
+    sm[1] = d.lv[0].status[0];
+    sm[2] = d.lv[0].status[1];
+    sm[3] = d.lv[0].status[2];
+  }
+  unsigned m = v.bits[w];
+  if (!m) return;
+  int o = v.cnt[w];
+  while (m) {
+    int b = __ffs((int)m) - 1;
+    m &= m - 1;
+    long long idx = w * 32 + b;
+    int4 c;
+    c.w = (int)(idx % v.grid.ext[2]) + v.grid.lo[2];
+    idx /= v.grid.ext[2];
+    c.z = (int)(idx % v.grid.ext[1]) + v.grid.lo[1];
+    idx /= v.grid.ext[1];
+    c.y = (int)(idx % v.grid.ext[0]) + v.grid.lo[0];
+    c.x = (int)(idx / v.grid.ext[0]);
+    v.out[o++] = c;
+  }
+}
+
 // ---- the output coordinates of several strided layers in a row, one wait of the host ---------------------------
 // Level l reads the coordinates level l-1 wrote; their number stays on the device (the last word of the scanned
 // popcounts) and the launches are sized for its bound, so nothing has to reach the host between the levels.
@@ -763,9 +896,61 @@ extern "C" int pce_outcoords_chain(const int32_t *in_coords, int64_t n_in, int32
   int host[PCE_MAX_CHAIN][4];
   const int4 *src = (const int4 *)in_coords;
   const int *n_dev = nullptr;
+  bool all_at_once = levels >= 2;
   for (int l = 0; l < levels; ++l) {
     if (!ws[l] || !out_coords[l]) PCE_FAIL(PCE_EINVAL, "pce_outcoords_chain: null pointer at level %d", l);
     if (ws_bytes[l] < L[l].total) PCE_FAIL(PCE_EWORKSPACE, "pce_outcoords_chain: workspace %lld < %lld at level %d", (long long)ws_bytes[l], (long long)L[l].total, l);
+    for (int a = 0; a < 3; ++a) all_at_once &= gd[l].ks[a] == gd[l].stride[a] && gd[l].pad[a] == 0;
+  }
+  if (all_at_once) {
+    ChainDev d;
+    d.levels = levels;
+    int fill_blk = 0, scan_blk = 0, word_blk = 0;
+    for (int l = 0; l < levels; ++l) {
+      char *w = (char *)ws[l];
+      ChainLevel &v = d.lv[l];
+      v.bits = (unsigned *)(w + L[l].off_bits);
+      v.cnt = (int *)(w + L[l].off_cnt);
+      v.sums = (int *)(w + L[l].off_scan);
+      v.status = (int *)(w + L[l].off_counters);
+      v.out = (int4 *)out_coords[l];
+      v.words = L[l].words;
+      v.fill_ints = (L[l].off_counters + 256 - L[l].off_bits) / 4;   // the bitmap and the counters behind it
+      v.fill_blk0 = fill_blk;
+      v.scan_blk0 = scan_blk;
+      v.word_blk0 = word_blk;
+      fill_blk += (int)pce_div_up(v.fill_ints, CHAIN_FILL_INTS);
+      scan_blk += (int)pce_div_up(v.words, SCAN_TILE);
+      word_blk += (int)pce_div_up(v.words, 256);
+      v.grid = L[l].grid;
+      for (int a = 0; a < 3; ++a) {
+        v.stride[a] = gd[l].stride[a];
+        v.lo[a] = gd[l].cmin[a];
+        v.hi[a] = gd[l].cmax[a];
+      }
+    }
+    d.summary = d.lv[0].status + 16;          // inside the 256 bytes of counters behind the first level's bitmap
+    hipLaunchKernelGGL(chain_fill_kernel, dim3((unsigned)fill_blk), dim3(256), 0, s, d);
+    PCE_LAUNCH_CHECK("chain_fill");
+    hipLaunchKernelGGL(chain_mark_kernel, dim3((unsigned)pce_div_up(n_in, 256)), dim3(256), 0, s, (const int4 *)in_coords,
+                       (long long)n_in, d);
+    PCE_LAUNCH_CHECK("chain_mark");
+    hipLaunchKernelGGL(chain_scan_local_kernel, dim3((unsigned)scan_blk), dim3(256), 0, s, d);
+    PCE_LAUNCH_CHECK("chain_scan_local");
+    hipLaunchKernelGGL(chain_scan_add_kernel, dim3((unsigned)scan_blk), dim3(256), 0, s, d);
+    PCE_LAUNCH_CHECK("chain_scan_add");
+    hipLaunchKernelGGL(chain_expand_kernel, dim3((unsigned)word_blk), dim3(256), 0, s, d);
+    PCE_LAUNCH_CHECK("chain_expand");
+    PCE_HIP(hipMemcpyAsync(&host[0][0], d.summary, (size_t)levels * 4 * sizeof(int), hipMemcpyDeviceToHost, s));
+    PCE_HIP(hipStreamSynchronize(s));
+    for (int l = 0; l < levels; ++l) {
+      if (host[l][1]) PCE_FAIL(PCE_ECOORD, "pce_outcoords_chain: coordinate outside [0,%d) or batch index out of range", PCE_COORD_BOUND);
+      if (host[l][3]) PCE_FAIL(PCE_EINVAL, "pce_outcoords_chain: a batch index is >= n_batch=%d", (int)n_batch);
+      n_out_host[l] = host[l][0];
+    }
+    return PCE_OK;
+  }
+  for (int l = 0; l < levels; ++l) {
     char *w = (char *)ws[l];
     unsigned *bits = (unsigned *)(w + L[l].off_bits);
     int *cnt = (int *)(w + L[l].off_cnt);

@@ -357,6 +357,44 @@ def prebuild_maps(input: spTensor, layers) -> None:
     _prebuild(input, layers)
 
 
+class MapPrefetcher:
+    """Kernel maps of the next cloud, built on a second stream while the network still runs the current one.
+
+    A map build ends in waits of the host for counts; on the stream the convolutions run on, such a wait first drains
+    everything queued there.  A serving loop that knows its next cloud calls ``submit(next)`` right after it has
+    queued the forward of the current one: the host then waits on the second stream only, and the GPU builds the
+    maps beside the convolutions.  ``take(x)`` makes the current stream wait for the maps of ``x`` (a no-op on the
+    GPU by then) -- the layers that follow find every map in the cache.
+
+    The coordinates of a submitted tensor must be complete when ``submit`` is called (they were copied or computed
+    earlier and the stream that did it has been waited for): the second stream does not wait for the first.  Map
+    memory is allocated on the second stream and announced to the consuming one with ``Tensor.record_stream``, so
+    dropping a tensor's maps while convolutions still read them is safe."""
+
+    def __init__(self, layers, device=None):
+        self.layers = list(layers)
+        self.stream = torch.cuda.Stream(device)
+        self.pending = {}
+
+    def submit(self, input: spTensor) -> None:
+        with torch.cuda.stream(self.stream):
+            _, built = _prebuild(input, self.layers)
+            done = torch.cuda.Event()
+            done.record(self.stream)
+        self.pending[id(input)] = (input, built, done)
+
+    def take(self, input: spTensor) -> None:
+        entry = self.pending.pop(id(input), None)
+        if entry is None:
+            return
+        _, built, done = entry
+        main = torch.cuda.current_stream(input.coords.device)
+        main.wait_event(done)
+        for km in built:
+            for t in km.device_tensors():
+                t.record_stream(main)
+
+
 def conv_func(input: spTensor, in_channel, out_channel, kernel, kernel_size_code, stride_code, padding_code, bias,
               transposed, tensorcore, dataflow: str = "auto", packed=None, act=None, residual=None, out=None) -> spTensor:
     """Map cache lookup / build, dataflow dispatch, bias (+ optional residual and activation, all

@@ -194,10 +194,13 @@ def test_out_coords_sparse_box_falls_back_to_sort():
     [((2, 2, 2), (2, 2, 2), (0, 0, 0))] * 4,                                          # the levels of a U-Net
     [((3, 3, 3), (2, 2, 2), (1, 1, 1)), ((2, 2, 2), (2, 2, 2), (0, 0, 0)), ((3, 2, 1), (2, 2, 1), (0, 0, 0))],
     [((2, 2, 2), (2, 2, 2), (0, 0, 0))],
+    [((3, 3, 3), (3, 3, 3), (0, 0, 0)), ((2, 3, 1), (2, 3, 1), (0, 0, 0)), ((2, 2, 2), (2, 2, 2), (0, 0, 0))],   # kernel = stride, odd sizes too
+    [((2, 2, 2), (2, 2, 2), (0, 0, 0)), ((3, 3, 3), (2, 2, 2), (1, 1, 1))],
 ])
 def test_out_coords_chain_equals_the_levels_built_one_by_one(chain):
-    """The chained build (the counts of the levels stay on the device, one wait of the host) against the oracle's
-    coordinates level by level, and against the library's own single-level build."""
+    """The chained build (the counts of the levels stay on the device, one wait of the host; chains whose layers all
+    have kernel = stride and no padding mark every level in one pass over the first level's points) against the
+    oracle's coordinates level by level, and against the library's own single-level build."""
     coords = synth.random_cloud(seed=44, n=40000, extent=70, batches=3)
     cmin, cmax = [0, 0, 0], coords[:, 1:].max(0).tolist()
     geoms, want, cur = [], [], coords

@@ -146,3 +146,37 @@ def test_prebuilt_maps_cover_the_whole_network(monkeypatch):
     for key, km in x.kmaps.items():
         other = z.kmaps[key]
         assert torch.equal(km.out_coords, other.out_coords) and torch.equal(km.imap, other.imap) and torch.equal(km.omap, other.omap)
+
+
+def test_maps_prefetched_on_a_second_stream():
+    """Forwards whose maps were built on a second stream while the previous forward ran (MapPrefetcher), the maps
+    dropped as soon as the host returns: every output equals the plain forward's, bit for bit, and no layer
+    builds a map."""
+    from pcengine_amd import spconv
+    clouds = [synth.random_cloud(seed=70 + i, n=15000 + 1000 * i, extent=36) for i in range(3)]
+    model = _model(2).fuse_bn().half()
+    feats = [torch.as_tensor(synth.features(12 + i, len(c), 4), device=DEV).half() for i, c in enumerate(clouds)]
+    cds = [torch.as_tensor(c, device=DEV) for c in clouds]
+    mk = lambda i: pe.spTensor(feats[i], cds[i], None, [0, 0, 0], clouds[i][:, 1:].max(0).tolist())
+    with torch.no_grad():
+        want = [model(mk(i)).feats.clone() for i in range(3)]
+    torch.cuda.synchronize()
+    pf = spconv.MapPrefetcher(model.map_plan(), DEV)
+    order = [0, 1, 2, 0, 1, 2, 2, 1, 0]
+    outs = []
+    nxt = mk(order[0])
+    pf.submit(nxt)
+    with torch.no_grad():
+        for k, i in enumerate(order):
+            cur = nxt
+            pf.take(cur)
+            assert len(cur.kmaps) == 9
+            outs.append(model(cur).feats)
+            if k + 1 < len(order):
+                nxt = mk(order[k + 1])
+                pf.submit(nxt)
+            del cur
+    torch.cuda.synchronize()
+    for i, o in zip(order, outs):
+        assert torch.equal(o, want[i])
+
