@@ -43,7 +43,8 @@ def layer_records(forward, graph_ms):
             forward()
     finally:
         backend.conv_forward, backend.dense_forward = real_conv, real_dense
-    names = {backend.DATAFLOW_FOD: "fod", backend.DATAFLOW_GMS: "gms", backend.DATAFLOW_OS: "os", backend.DATAFLOW_FDS: "fds", -1: "gemm"}
+    names = {backend.DATAFLOW_FOD: "fod", backend.DATAFLOW_GMS: "gms", backend.DATAFLOW_OS: "os", backend.DATAFLOW_FDS: "fds",
+             backend.DATAFLOW_OSO: "oso", -1: "gemm"}
     records = {}
     for kind, feats, weight, km, flow, kw in calls:
         w3 = weight if weight.dim() == 3 else weight.unsqueeze(0)
@@ -98,7 +99,7 @@ def main() -> int:
     import numpy as np
     import torch
     from pcengine_amd import _lib, backend, synth
-    from pcengine_amd.backend import DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS, DATAFLOW_FDS
+    from pcengine_amd.backend import DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS, DATAFLOW_FDS, DATAFLOW_OSO
 
     lib = _lib.load()
     dev = "cuda:0"
@@ -198,7 +199,7 @@ def main() -> int:
     del km_hash
     M = km.M
 
-    names = {DATAFLOW_FOD: "fod", DATAFLOW_GMS: "gms", DATAFLOW_OS: "os", DATAFLOW_FDS: "fds"}
+    names = {DATAFLOW_FOD: "fod", DATAFLOW_GMS: "gms", DATAFLOW_OS: "os", DATAFLOW_FDS: "fds", DATAFLOW_OSO: "oso"}
     packed = backend.pack_weights(wd)     # weights are constants: packed once, outside the timed region
     if args.dataflow == "auto":
         flow = backend.select_dataflow(km, c_in, c_out, torch.float16)
@@ -247,8 +248,8 @@ def main() -> int:
                    DATAFLOW_GMS: {3: "gather", 1: "grouped_gemm", 0: "centre_gemm", 2: "scatter"},
                    DATAFLOW_FDS: ({1: "pairs_and_centre_gemm", 2: "partial_row_sum"} if narrow else
                                   {1: "fod_pairs_to_buffer", 2: "centre_gemm_then_row_sum"}),
-                   DATAFLOW_OS: {1: "os_tile"}}[flow]
-    if flow != DATAFLOW_OS:
+                   DATAFLOW_OS: {1: "os_tile"}, DATAFLOW_OSO: {1: "ordered_rows"}}[flow]
+    if flow not in (DATAFLOW_OS, DATAFLOW_OSO):
         # one stage at a time, on the measurement build of the library (the same kernels; the product library has
         # no stage switch)
         with _lib.measurement_build() as mlib:
@@ -256,8 +257,10 @@ def main() -> int:
                 mlib.pce_set_stage_mask((1 << bit) | 0xFFFFFFF0)   # bits 4 and up keep the kernel selection of the full run
                 stages[name] = timer(step, max(20, args.steps // 4), 5)[0]
     else:
-        stages["os_tile"] = ms
-    others = {names[f]: timer(lambda f=f: step(f), max(20, args.steps // 4), 5)[0] for f in names if f != flow and f != DATAFLOW_FOD}
+        stages[stage_names[1]] = ms       # one kernel is the whole layer
+    takes = lambda f: f != DATAFLOW_OSO or backend.oso_takes(km, c_in, c_out, torch.float16)
+    others = {names[f]: timer(lambda f=f: step(f), max(20, args.steps // 4), 5)[0]
+              for f in names if f != flow and f != DATAFLOW_FOD and takes(f)}
     others[names[DATAFLOW_FOD]] = ev_ms(lambda: step(DATAFLOW_FOD), max(20, args.steps // 4), 5)   # allocates: eager
 
     # algorithmic bytes of the layer: every tensor once + the pair list
@@ -273,6 +276,9 @@ def main() -> int:
         "grouped_gemm": M * (c_in + c_out) * e + 26 * c_in * c_out * e,
         "scatter": M * c_out * e + 2 * n * c_out * e + 4 * M + 4 * (n + 1),
         "os_tile": b_conv - 8 * M + 4 * 27 * n,
+        # every row in and out once, the gathered neighbour rows, the neighbour index of every pair, the order
+        # (row index and offset mask of every row), every weight once
+        "ordered_rows": n * c_in * e + n * c_out * e + M * c_in * e + 4 * M + 8 * n + 27 * c_in * c_out * e,
         "fod_pairs_to_buffer": M * (c_in + c_out) * e + 4 * M + 26 * c_in * c_out * e,
         "centre_gemm_csr_sum": n * c_in * e + n * c_out * e + c_in * c_out * e + M * c_out * e + 4 * M + 4 * (n + 1),
         # centre rows in and out, pair rows in and partial rows out, the two index lists, every weight once

@@ -55,8 +55,10 @@ enum {
   PCE_DATAFLOW_FOD = 0, /* fetch-on-demand fused gather-matmul-scatter (reference "D2") */
   PCE_DATAFLOW_GMS = 1, /* gather - grouped GEMM - scatter over a staging buffer (reference "D1") */
   PCE_DATAFLOW_OS = 2,  /* output-stationary fetch-on-demand: no atomics, no staging buffer */
-  PCE_DATAFLOW_FDS = 3  /* fetch-on-demand with deferred scatter: pair tiles write partial rows to a
+  PCE_DATAFLOW_FDS = 3, /* fetch-on-demand with deferred scatter: pair tiles write partial rows to a
                            staging buffer, the centre GEMM's epilogue sums them per output row */
+  PCE_DATAFLOW_OSO = 4  /* output-stationary over rows ordered by their neighbour pattern (pce_row_order):
+                           narrow fp16 submanifold layers on sparse clouds, one launch, no partial rows */
 };
 
 #define PCE_QUANTUM 128        /* rows per tile of the pair list; qkpos granularity (backend/hash.cu:203-205) */
@@ -203,9 +205,12 @@ typedef struct pce_kmap_problem {
   int32_t *icsr, *icode, *ocsr, *ocode; /* all four or none */
   int32_t *islot, *oslot;               /* optional, with the CSR outputs */
   int32_t *nbr_out, *nbr_in;            /* optional */
-  int32_t *status;                      /* int32[4] per problem, zeroed by the caller */
+  int32_t *status;                      /* int32[4] per problem (int32[8] with `order`), zeroed by the caller */
   int32_t n_batch;                      /* batch count (spTensor.batchsize), 0 = unknown: see the column grid below */
   int32_t flags;                        /* PCE_KMAP_* */
+  int32_t *order;                       /* optional, needs nbr_out and kv <= 31: the row order of pce_row_order
+                                           (pce_row_order_elems(n_out) ints), built with the map at the cost of three
+                                           launches per batch; status[4] receives its n_heavy */
 } pce_kmap_problem_t;
 int pce_kmap_build_batch(const pce_kmap_problem_t *problems_host, int32_t n_problems, pce_stream_t stream);
 
@@ -250,7 +255,7 @@ typedef struct pce_epilogue {
    * layer and the encoder layer whose output is kept -- write their halves of the concatenated matrix in place
    * and the layers that read one half gather from it, so the concatenation (script/utils.py:152-164) costs no
    * pass over the data.  Multiples of 8 elements, at least the channel count; taken by pce_conv_fwd_fds and
-   * pce_conv_fwd_os (any dtype), PCE_EINVAL elsewhere.  residual, bias and the partial-row buffer stay dense. */
+   * pce_conv_fwd_os (any dtype) and pce_conv_fwd_oso, PCE_EINVAL elsewhere.  residual, bias and the partial-row buffer stay dense. */
   int64_t ld_in;
   int64_t ld_out;
 } pce_epilogue_t;
@@ -359,6 +364,29 @@ int pce_conv_fwd_os(const void *in_feats, const void *weight, const void *weight
                     void *out_feats, int32_t dtype,
                     int64_t n_in, int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv,
                     const int32_t *nbr_dev, const pce_epilogue_t *epilogue, pce_stream_t stream);
+
+/* Output-stationary over ordered rows, for narrow fp16 submanifold layers on clouds where most voxels have few
+ * neighbours (surfaces: 0.2 pairs per voxel on a 64 x 2048 LiDAR scan at 0.1 m).  pce_row_order derives from the
+ * output-major neighbour table, once per map, the order in which the rows are visited -- rows without neighbours
+ * first, in their own order, then the rows with one or two neighbours sorted by the offsets they have them at, then
+ * the rows with three or more, sorted likewise -- and every row's offset mask: order_dev = perm[n_rows] |
+ * mask[n_rows] | 8192 ints of scratch, pce_row_order_elems ints in all; kv <= 31; four launches and one wait for
+ * *n_heavy_host, the number of rows of the last part; the positions of rows with equal keys depend on the run,
+ * the results of the layer do not.  pce_conv_fwd_oso then runs the layer as one launch: a wavefront takes 32 rows
+ * of that order, multiplies their centre rows, gathers for each offset any of them has the neighbours of the rows
+ * that have it, and stores each finished row once (epilogue fused); the rows of the last part, whose offsets are
+ * many, go 32 to a workgroup whose four wavefronts share the offsets.  PCE_F16, c_in a multiple of 16 and at most
+ * 64, c_out a multiple of 8 and at most 64, packed weights, mid >= 0; PCE_EINVAL otherwise.  Takes the row strides
+ * of pce_epilogue_t.  No counterpart in the reference: it computes what the fetch-on-demand kernels compute
+ * (backend/spconv.cuh:1567-1730) with the scatter-add replaced by register accumulation, as pce_conv_fwd_os. */
+int64_t pce_row_order_elems(int64_t n_rows);
+int pce_row_order(const int32_t *nbr_dev, int32_t kv, int64_t n_rows, int32_t mid, int32_t *order_dev,
+                  int64_t order_elems, int64_t *n_heavy_host, pce_stream_t stream);
+int pce_conv_fwd_oso(const void *in_feats, const void *weight, const void *weight_packed,
+                     void *out_feats, int32_t dtype,
+                     int64_t n_in, int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv, int32_t mid,
+                     const int32_t *nbr_dev, const int32_t *order_dev, int64_t n_heavy,
+                     const pce_epilogue_t *epilogue, pce_stream_t stream);
 
 /* ---- batch normalisation over the rows of a feature matrix ------------------------------------- *
  * The reference normalises the features of a sparse tensor with torch.nn.BatchNorm1d

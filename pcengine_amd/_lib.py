@@ -15,7 +15,7 @@ MEASURE_LIB_PATH = os.path.join(_HERE, "lib", "libpcengine_amd_measure.so")
 
 PCE_OK, PCE_EINVAL, PCE_ECAPACITY, PCE_EHIP, PCE_EWORKSPACE, PCE_ECOORD = range(6)
 PCE_F16, PCE_F32, PCE_F64 = 0, 1, 2
-DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS, DATAFLOW_FDS = 0, 1, 2, 3
+DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS, DATAFLOW_FDS, DATAFLOW_OSO = 0, 1, 2, 3, 4
 QUANTUM = 128
 KMAP_NO_GRID = 1
 CSR_CODE = 1186111
@@ -42,7 +42,7 @@ class KmapProblem(Structure):
                  ("geom", Geom), ("ws", c_void_p), ("ws_bytes", c_int64)] +
                 [(name, c_void_p) for name in ("imap", "omap", "knnz", "kpos", "qkpos", "icsr", "icode", "ocsr", "ocode",
                                                "islot", "oslot", "nbr_out", "nbr_in", "status")] +
-                [("n_batch", c_int32), ("flags", c_int32)])
+                [("n_batch", c_int32), ("flags", c_int32), ("order", c_void_p)])
 
 
 class Epilogue(Structure):
@@ -108,6 +108,10 @@ _SIGNATURES = {
                                    c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64,
                                    POINTER(Epilogue), c_void_p]),
     "pce_conv_fwd_os": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_void_p, POINTER(Epilogue), c_void_p]),
+    "pce_conv_fwd_oso": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32,
+                                   c_void_p, c_void_p, c_int64, POINTER(Epilogue), c_void_p]),
+    "pce_row_order": (c_int32, [c_void_p, c_int32, c_int64, c_int32, c_void_p, c_int64, POINTER(c_int64), c_void_p]),
+    "pce_row_order_elems": (c_int64, [c_int64]),
     "pce_conv_fwd_dense": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32, POINTER(Epilogue), c_void_p]),
     "pce_conv_wgrad": (c_int32, [c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p,
                                  c_void_p, c_void_p, c_int64, c_void_p, c_void_p]),

@@ -19,7 +19,7 @@ from typing import List, Optional, Sequence, Tuple
 import torch
 
 from . import _lib
-from ._lib import Geom, DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS, DATAFLOW_FDS, PCE_F16, PCE_F32, QUANTUM, CSR_CODE
+from ._lib import Geom, DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS, DATAFLOW_FDS, DATAFLOW_OSO, PCE_F16, PCE_F32, QUANTUM, CSR_CODE
 
 CODE_A, CODE_B = 94273, 311  # packed 3-vectors, script/utils.py:233-242
 
@@ -114,6 +114,8 @@ class KernelMap:
     oslot: Optional[torch.Tensor] = _Cut(True)
     route: Optional[torch.Tensor] = None   # routing array of a layer without centre offset (pair_route), built on first use
     route_t: Optional[torch.Tensor] = None # the same for the transposed layer over this map
+    order: Optional[torch.Tensor] = None   # rows in neighbour-pattern order and their offset masks (row_order), built on first use
+    order_heavy: int = 0                   # how many rows of that order have three neighbours or more (its last part)
     tag: str = "auto"           # 'D1' / 'D2' when the reference's init_tag protocol fixed it
     in_coords: Optional[torch.Tensor] = None
     geom: Optional[Geom] = None
@@ -263,7 +265,7 @@ class _MapJob:
     read-back of its counts."""
 
     def __init__(self, in_coords, ks, stride, pad, cmin, cmax_out, subm, want_csr, want_nbr_out, want_nbr_in,
-                 out_coords, batchsize):
+                 out_coords, batchsize, want_order=None):
         lib = _lib.load()
         _require_cuda(in_coords, "coords")
         if in_coords.dtype != torch.int32 or in_coords.dim() != 2 or in_coords.shape[1] != 4:
@@ -283,7 +285,12 @@ class _MapJob:
         self.args = (tuple(ks), tuple(stride), tuple(pad), list(cmin), list(cmax_out), bool(subm))
         self.in_coords, self.out_coords, self.geom = in_coords, out_coords, geom
         self.n_in, self.n_out, self.kv, self.want_csr, self.dev = n_in, n_out, kv, bool(want_csr), dev
-        self.meta_len = kv + 2 * (kv + 1) + 4      # knnz | kpos | qkpos | status
+        self.meta_len = kv + 2 * (kv + 1) + 8      # knnz | kpos | qkpos | status (4 words, then the heavy rows of the order)
+        # the row order of the ordered output-stationary dataflow comes with every submanifold map that has the
+        # output-major table it is derived from (three launches per batch of maps, 2 n + 8192 ints)
+        if want_order is None:
+            want_order = subm and want_nbr_out
+        self.want_order = bool(want_order) and want_nbr_out and kv <= 31
         # the batch count lets the library index sorted coordinates by column instead of hashing them; a build that
         # finds them unsorted, or outside the box the geometry states, is redone through the hash table (finish)
         self.n_batch, self.no_grid = max(int(batchsize), 0), False
@@ -297,9 +304,11 @@ class _MapJob:
             self.want.append(("nbr_out", kv * n_out))
         if want_nbr_in:
             self.want.append(("nbr_in", kv * n_in))
+        if self.want_order:
+            self.want.append(("order", 2 * n_out + 8192))
         if want_csr:
             self.want += [("icsr", n_in + 1), ("ocsr", n_out + 1), ("icode", cap), ("ocode", cap), ("islot", cap), ("oslot", cap)]
-        self.ws = self.imap = self.omap = self.nbr_out = self.nbr_in = None
+        self.ws = self.imap = self.omap = self.nbr_out = self.nbr_in = self.order = None
         self.icsr = self.ocsr = self.icode = self.ocode = self.islot = self.oslot = None
 
     @staticmethod
@@ -337,6 +346,7 @@ class _MapJob:
         p.nbr_out, p.nbr_in = _ptr(self.nbr_out), _ptr(self.nbr_in)
         p.status = status.data_ptr()
         p.n_batch, p.flags = self.n_batch, (_lib.KMAP_NO_GRID if self.no_grid else 0)
+        p.order = _ptr(self.order)
         return p
 
     def finish(self, host: list) -> KernelMap:
@@ -360,7 +370,7 @@ class _MapJob:
                        qkpos=self.qkpos, out_coords=self.out_coords, nbr_out=self.nbr_out, nbr_in=self.nbr_in,
                        icsr=self.icsr, ocsr=self.ocsr, icode=cut(self.icode), ocode=cut(self.ocode),
                        islot=cut(self.islot), oslot=cut(self.oslot), in_coords=self.in_coords, geom=self.geom,
-                       knnz_host=host[:kv])
+                       knnz_host=host[:kv], order=self.order, order_heavy=st[4] if self.order is not None else 0)
         km._cmin, km._cmax = cmin, cmax_out
         km.kpos_host = (_lib.c_int32 * (kv + 1))(*host[kv:2 * kv + 1])
         km.qkpos_host = (_lib.c_int32 * (kv + 1))(*host[2 * kv + 1:3 * kv + 2])
@@ -372,11 +382,11 @@ KMAP_MAX_BATCH = 16
 
 def prepare_map(in_coords: torch.Tensor, ks, stride, pad, cmin, cmax_out, subm: bool, want_csr: bool = False,
                 want_nbr_out: bool = True, want_nbr_in: bool = False, out_coords: Optional[torch.Tensor] = None,
-                batchsize: int = 0) -> _MapJob:
+                batchsize: int = 0, want_order: Optional[bool] = None) -> _MapJob:
     """First half of a map build: the output coordinates of a strided layer (``.out_coords``, final)
     and the output buffers.  ``build_kernel_maps`` takes the result in place of a request."""
     return _MapJob(in_coords, ks, stride, pad, cmin, cmax_out, subm, want_csr, want_nbr_out, want_nbr_in, out_coords,
-                   batchsize)
+                   batchsize, want_order)
 
 
 def build_kernel_maps(requests: List[dict], defer: bool = False):
@@ -427,7 +437,8 @@ def build_kernel_maps(requests: List[dict], defer: bool = False):
 
 def build_kernel_map(in_coords: torch.Tensor, ks, stride, pad, cmin, cmax_out, subm: bool,
                      want_csr: bool = False, want_nbr_out: bool = True, want_nbr_in: bool = False,
-                     out_coords: Optional[torch.Tensor] = None, batchsize: int = 0, defer: bool = False):
+                     out_coords: Optional[torch.Tensor] = None, batchsize: int = 0, defer: bool = False,
+                     want_order: Optional[bool] = None):
     """Hash the output coordinates, probe every (input row, offset) and emit the canonical map.
 
     ``cmax_out`` is the bound on output coordinates (already reduced for strided layers).
@@ -436,7 +447,7 @@ def build_kernel_map(in_coords: torch.Tensor, ks, stride, pad, cmin, cmax_out, s
     synchronised."""
     return build_kernel_maps([dict(in_coords=in_coords, ks=ks, stride=stride, pad=pad, cmin=cmin, cmax_out=cmax_out,
                                    subm=subm, want_csr=want_csr, want_nbr_out=want_nbr_out, want_nbr_in=want_nbr_in,
-                                   out_coords=out_coords, batchsize=batchsize)], defer=defer)[0]
+                                   out_coords=out_coords, batchsize=batchsize, want_order=want_order)], defer=defer)[0]
 
 
 def ensure_csr(km: KernelMap) -> None:
@@ -470,19 +481,45 @@ def pair_route(km: KernelMap, transposed: bool = False) -> torch.Tensor:
     return route
 
 
+def row_order(km: KernelMap) -> torch.Tensor:
+    """Row order of the ordered output-stationary dataflow (``pce_row_order``), cached on the map: the output rows
+    of a submanifold layer with rows without neighbours first and the others sorted by the offsets they have."""
+    if km.order is None:
+        ensure_nbr(km, False)
+        lib = _lib.load()
+        elems = lib.pce_row_order_elems(km.n_out)
+        order = torch.empty(elems, dtype=torch.int32, device=km.nbr_out.device)
+        heavy = _lib.c_int64(0)
+        _lib.check(lib.pce_row_order(km.nbr_out.data_ptr(), km.kv, km.n_out, _mid(km.ks) if km.subm else -1, order.data_ptr(),
+                                     elems, heavy, _stream(order.device)))
+        km.order, km.order_heavy = order, heavy.value
+    return km.order
+
+
+def oso_takes(km: KernelMap, c_in: int, c_out: int, dtype: torch.dtype, transposed: bool = False) -> bool:
+    """Shapes the ordered output-stationary dataflow exists for."""
+    return (km.subm and not transposed and dtype == torch.float16 and km.kv <= 31 and c_in % 16 == 0 and c_in <= 64
+            and c_out % 8 == 0 and c_out <= 64)
+
+
 def ensure_nbr(km: KernelMap, transposed: bool) -> None:
     if (km.nbr_in if transposed else km.nbr_out) is not None:
         return
     full = build_kernel_map(km.in_coords, km.ks, km.stride, km.pad, km._cmin, km._cmax, km.subm, want_csr=False,
                             want_nbr_out=True, want_nbr_in=True, out_coords=km.out_coords)
     km.nbr_out, km.nbr_in = full.nbr_out, full.nbr_in
+    if full.order is not None:
+        km.order, km.order_heavy = full.order, full.order_heavy
 
 
 def select_dataflow(km: KernelMap, c_in: int, c_out: int, dtype: torch.dtype, transposed: bool = False) -> int:
     lib = _lib.load()
     n_out = km.n_in if transposed else km.n_out
     n_in = km.n_out if transposed else km.n_in
-    return lib.pce_select_dataflow(n_in, n_out, km.M, c_in, c_out, km.kv, PCE_F16 if dtype == torch.float16 else PCE_F32)
+    df = lib.pce_select_dataflow(n_in, n_out, km.M, c_in, c_out, km.kv, PCE_F16 if dtype == torch.float16 else PCE_F32)
+    if df == DATAFLOW_OSO and not oso_takes(km, c_in, c_out, dtype, transposed):
+        df = DATAFLOW_FDS       # equal row counts and an odd kernel volume, but not a plain submanifold layer
+    return df
 
 
 def pack_weights(weight: torch.Tensor) -> Optional[torch.Tensor]:
@@ -584,7 +621,7 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
     _require_cuda(feats, "feats")
     # the deferred-scatter and output-stationary kernels take column slices of wider matrices in place (the halves
     # of a concatenated skip connection); everything else gets dense rows
-    strided_ok = dataflow in (DATAFLOW_FDS, DATAFLOW_OS)
+    strided_ok = dataflow in (DATAFLOW_FDS, DATAFLOW_OS, DATAFLOW_OSO)
     ld_in = _row_stride(feats) if strided_ok else -1
     if ld_in < 0:
         feats, ld_in = feats.contiguous(), 0
@@ -662,6 +699,15 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
         _lib.check(lib.pce_conv_fwd_gms(feats.data_ptr(), weight.data_ptr(), _ptr(packed), out.data_ptr(), dt, n_in, n_out,
                                         c_in, c_out, kv, mid, icsr.data_ptr(), icode.data_ptr(), ocsr.data_ptr(), ocode.data_ptr(),
                                         km.kpos.data_ptr(), km.qkpos.data_ptr(), km.qsum, buffer.data_ptr(), buffer.numel(), epi, s))
+    elif dataflow == DATAFLOW_OSO:
+        if not oso_takes(km, c_in, c_out, feats.dtype, transposed):
+            raise ValueError("the ordered output-stationary dataflow takes fp16 submanifold layers of at most 64 channels "
+                             "(c_in a multiple of 16, c_out of 8)")
+        if packed is None:
+            packed = pack_weights(weight)
+        order = row_order(km)
+        _lib.check(lib.pce_conv_fwd_oso(feats.data_ptr(), weight.data_ptr(), _ptr(packed), out.data_ptr(), dt, n_in, n_out,
+                                        c_in, c_out, kv, mid, km.nbr_out.data_ptr(), order.data_ptr(), km.order_heavy, epi, s))
     elif dataflow == DATAFLOW_OS:
         ensure_nbr(km, transposed)
         nbr = km.nbr_in if transposed else km.nbr_out

@@ -74,3 +74,21 @@ __host__ __device__ static inline unsigned long long pce_home_slot(unsigned long
   unsigned long long bucket = pce_mix64(key >> 2) & ((slots >> 2) - 1);
   return (bucket << 2) | (key & 3ull);
 }
+
+// ---------------------------------------------------------------------------------------------
+// Row order of the ordered output-stationary dataflow (pce_row_order, pce_conv_fwd_oso):
+// order = perm[n_rows] | mask[n_rows] | tail[PCE_ORDER_TAIL].  The tail holds the histogram, the cursors and
+// the bases of the counting sort over ORDER_KEYS keys -- (lowest, second-lowest) offset of the rows with one or
+// two neighbours, then of the rows with more -- and the counts.
+// ---------------------------------------------------------------------------------------------
+#define PCE_ORDER_TAIL 8192
+#define ORDER_MAX_KV 32
+#define ORDER_KEYS 2048
+#define ORDER_HIST 0
+#define ORDER_CURSOR 2048
+#define ORDER_BASE 4096
+#define ORDER_N_NONZERO 8188  // rows with any neighbour
+#define ORDER_N_HEAVY 8189    // rows with ORDER_HEAVY_POPC neighbours or more
+#define ORDER_PLAIN_CURSOR 8191
+#define ORDER_HEAVY_POPC 3
+

@@ -764,13 +764,20 @@ __global__ void __launch_bounds__(256) chain_mark_kernel(const int4 *__restrict_
   int p[3] = {c.y, c.z, c.w};
   for (int l = 0; l < d.levels; ++l) {
     const ChainLevel &v = d.lv[l];
-    bool ok = true;
+    bool ok = true, bad = false;
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
-      p[a] = p[a] / v.stride[a];            // kernel = stride, no padding: the one offset that divides
-      ok &= p[a] >= v.lo[a] && p[a] <= v.hi[a];
+      int q = p[a] / v.stride[a];           // kernel = stride, no padding: the one offset that divides ...
+      if (p[a] % v.stride[a] < 0) --q;      // ... which is the floor, for a negative coordinate too
+      p[a] = q;
+      ok &= q >= v.lo[a] && q <= v.hi[a];
+      bad |= q < 0 || q >= PCE_COORD_BOUND;
     }
     if (!ok) return;                        // clipped here: absent from every deeper level too
+    if (bad) {                              // inside the stated bounds but outside what a strided layer can address
+      d.lv[0].status[0] = 1;
+      return;
+    }
     long long bit = (((long long)c.x * v.grid.ext[0] + (p[0] - v.grid.lo[0])) * v.grid.ext[1] + (p[1] - v.grid.lo[1])) *
                         v.grid.ext[2] + (p[2] - v.grid.lo[2]);
     atomicOr(&v.bits[bit >> 5], 1u << (bit & 31));
@@ -1270,6 +1277,7 @@ struct ProbDev {
   unsigned long long slots;
   int *dense, *irank, *orank, *seg;
   int *imap, *omap, *knnz, *kpos, *qkpos, *icsr, *icode, *ocsr, *ocode, *islot, *oslot, *nbr_out, *status;
+  int *order;        // row order of the ordered output-stationary dataflow, or null
   int want_csr;
   int use_grid;      // column grid instead of the hash table
   int2 *grid;        // [cells] = {first row of the column, row behind its last}, -1 for an empty column
@@ -1290,7 +1298,7 @@ struct FillRegion {
   unsigned *p;
   long long n_words;
   unsigned blk0;
-  unsigned pad;
+  unsigned zero;   // fill with zeros instead of the launch's value
 };
 
 struct ScanArr {
@@ -1321,7 +1329,7 @@ __global__ void __launch_bounds__(256) multi_fill_kernel(const FillRegion *__res
 #pragma unroll
   for (int k = 0; k < 8; ++k) {
     long long i = base + k * 256 + threadIdx.x;
-    if (i < reg.n_words) reg.p[i] = value;
+    if (i < reg.n_words) reg.p[i] = reg.zero ? 0u : value;
   }
 }
 
@@ -1842,14 +1850,171 @@ extern "C" int64_t pce_kmap_workspace_bytes_grid(int64_t n_in, int64_t n_out, co
 }
 
 // stages of a batched build, each one launch with its own job list
-enum { ST_INSERT = 0, ST_QUERY, ST_COUNT, ST_FILL, ST_CSR_A, ST_CSR_B, ST_GRID_BUILD, ST_GRID_QUERY, ST_GRID_QUERY3, ST_COUNT_ };
+// ---- row order of the ordered output-stationary dataflow -----------------------------------------------------
+// Output rows of a map in an order that puts equal neighbour patterns side by side: rows without neighbours
+// first (block by block, each block's rows in their own order), then the rows with one or two neighbours sorted
+// by the (lowest, second-lowest) offset they have one at, then the rows with ORDER_HEAVY_POPC or more, sorted
+// likewise.  A counting sort: masks and a histogram of the keys, one block that turns the histogram into
+// bases, a scatter pass with one cursor per key.  The kernels exist twice: over the job lists of a batched map
+// build, and with plain arguments for an order requested on its own (pce_row_order).
+__device__ __forceinline__ int order_key(unsigned m) {   // m != 0
+  const int first = __ffs((int)m) - 1;
+  const unsigned rest = m & (m - 1u);
+  const int second = rest ? __ffs((int)rest) - 1 : 31;
+  return (__popc(m) >= ORDER_HEAVY_POPC ? 1024 : 0) + first * 32 + second;
+}
+
+// mask[row] = offsets (other than the centre) at which the row has a neighbour; hist[key] += the block's count.
+// The keys of a block of 256 rows are counted in LDS first: on a dense cloud nearly every row has a key and a few
+// keys hold most rows, and one global atomic per row on those few addresses costs milliseconds.
+__device__ __forceinline__ void order_mask_block(const int *__restrict__ nbr, int kv, long long n_rows, int mid,
+                                                 int *__restrict__ order, unsigned blk) {
+  __shared__ int cnt[ORDER_KEYS];
+  for (int i = threadIdx.x; i < ORDER_KEYS; i += 256) cnt[i] = 0;
+  __syncthreads();
+  const long long row = (long long)blk * 256 + threadIdx.x;
+  if (row < n_rows) {
+    unsigned m = 0;
+    for (int k = 0; k < kv; ++k)
+      if (k != mid && nbr[(long long)k * n_rows + row] >= 0) m |= 1u << k;
+    order[n_rows + row] = (int)m;
+    if (m) atomicAdd(&cnt[order_key(m)], 1);   // rows without neighbours are placed by the scatter pass
+  }
+  __syncthreads();
+  int *hist = order + 2 * n_rows + ORDER_HIST;
+  for (int i = threadIdx.x; i < ORDER_KEYS; i += 256)
+    if (cnt[i]) atomicAdd(&hist[i], cnt[i]);
+}
+
+// base[key] = first position of the key's rows behind the rows without neighbours (one block of 1024); the counts
+__device__ __forceinline__ void order_scan_block(int *tail, int *n_heavy_out) {
+  __shared__ int part[1024];
+  const int *hist = tail + ORDER_HIST;
+  int *base = tail + ORDER_BASE;
+  constexpr int per = ORDER_KEYS / 1024;
+  int sum = 0;
+#pragma unroll
+  for (int j = 0; j < per; ++j) sum += hist[threadIdx.x * per + j];
+  part[threadIdx.x] = sum;
+  __syncthreads();
+  for (int d = 1; d < 1024; d <<= 1) {
+    int v = (int)threadIdx.x >= d ? part[threadIdx.x - d] : 0;
+    __syncthreads();
+    part[threadIdx.x] += v;
+    __syncthreads();
+  }
+  if (threadIdx.x == 1023) {
+    tail[ORDER_N_NONZERO] = part[1023];
+    tail[ORDER_N_HEAVY] = part[1023] - part[511];      // keys 1024 .. 2047 belong to threads 512 .. 1023
+    if (n_heavy_out) *n_heavy_out = part[1023] - part[511];
+  }
+  int run = part[threadIdx.x] - sum;
+#pragma unroll
+  for (int j = 0; j < per; ++j) {
+    base[threadIdx.x * per + j] = run;
+    run += hist[threadIdx.x * per + j];
+  }
+}
+
+// perm: the rows of one block of 256 (block `blk` of the map), placed as described above.  A block takes one range
+// per key it holds (one global atomic per key and block); its rows of a key keep the ranks LDS atomics gave them.
+__device__ __forceinline__ void order_scatter_block(long long n_rows, int *__restrict__ order, unsigned blk) {
+  __shared__ int cnt[ORDER_KEYS], gbase[ORDER_KEYS];
+  __shared__ int wcount[4], wbase;
+  int *perm = order, *tail = order + 2 * n_rows;
+  for (int i = threadIdx.x; i < ORDER_KEYS; i += 256) cnt[i] = 0;
+  const long long n_plain = n_rows - tail[ORDER_N_NONZERO];
+  long long row = (long long)blk * 256 + threadIdx.x;
+  const bool live = row < n_rows;
+  const unsigned m = live ? (unsigned)order[n_rows + row] : 1u;
+  const bool plain = live && m == 0;
+  const unsigned long long b = __ballot(plain);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) wcount[wave] = __popcll(b);
+  __syncthreads();
+  if (threadIdx.x == 0) wbase = atomicAdd(&tail[ORDER_PLAIN_CURSOR], wcount[0] + wcount[1] + wcount[2] + wcount[3]);
+  const int key = (live && !plain) ? order_key(m) : -1;
+  int rank = 0;
+  if (key >= 0) rank = atomicAdd(&cnt[key], 1);
+  __syncthreads();
+  for (int i = threadIdx.x; i < ORDER_KEYS; i += 256)
+    if (cnt[i]) gbase[i] = tail[ORDER_BASE + i] + atomicAdd(&tail[ORDER_CURSOR + i], cnt[i]);
+  __syncthreads();
+  if (plain) {
+    int before = __popcll(b & ((1ull << lane) - 1ull));
+    for (int w2 = 0; w2 < wave; ++w2) before += wcount[w2];
+    perm[wbase + before] = (int)row;
+  } else if (key >= 0) {
+    perm[n_plain + gbase[key] + rank] = (int)row;
+  }
+}
+
+__global__ void order_clear_kernel(int *tail) {
+  for (int i = threadIdx.x; i < PCE_ORDER_TAIL; i += blockDim.x) tail[i] = 0;
+}
+__global__ void __launch_bounds__(256) order_mask_kernel(const int *__restrict__ nbr, int kv, long long n_rows, int mid,
+                                                         int *__restrict__ order) {
+  order_mask_block(nbr, kv, n_rows, mid, order, blockIdx.x);
+}
+__global__ void __launch_bounds__(1024) order_scan_kernel(int *tail) { order_scan_block(tail, nullptr); }
+__global__ void __launch_bounds__(256) order_scatter_kernel(long long n_rows, int *__restrict__ order) {
+  order_scatter_block(n_rows, order, blockIdx.x);
+}
+
+// the same over the problems of a batched build; status[4] of a problem receives its number of heavy rows
+__global__ void __launch_bounds__(256) order_mask_batch_kernel(const ProbDev *__restrict__ P, JobList jl) {
+  const Job &job = find_job(jl, blockIdx.x);
+  const ProbDev &q = P[job.prob];
+  order_mask_block(q.nbr_out, q.g.kv, q.n_out, q.g.subm ? q.g.mid : -1, q.order, blockIdx.x - job.blk0);
+}
+__global__ void __launch_bounds__(1024) order_scan_batch_kernel(const ProbDev *__restrict__ P) {
+  const ProbDev &q = P[blockIdx.x];
+  if (!q.order) return;
+  order_scan_block(q.order + 2 * q.n_out, q.status + 4);
+}
+__global__ void __launch_bounds__(256) order_scatter_batch_kernel(const ProbDev *__restrict__ P, JobList jl) {
+  const Job &job = find_job(jl, blockIdx.x);
+  const ProbDev &q = P[job.prob];
+  order_scatter_block(q.n_out, q.order, blockIdx.x - job.blk0);
+}
+
+extern "C" int64_t pce_row_order_elems(int64_t n_rows) { return n_rows < 0 ? 0 : 2 * n_rows + PCE_ORDER_TAIL; }
+
+extern "C" int pce_row_order(const int32_t *nbr, int32_t kv, int64_t n_rows, int32_t mid, int32_t *order, int64_t order_elems,
+                             int64_t *n_heavy_host, pce_stream_t stream) {
+  if (!nbr || !order || !n_heavy_host) PCE_FAIL(PCE_EINVAL, "pce_row_order: null pointer");
+  if (kv < 1 || kv > ORDER_MAX_KV - 1) PCE_FAIL(PCE_EINVAL, "pce_row_order: kernel volume %d outside [1, %d]", (int)kv, ORDER_MAX_KV - 1);
+  if (n_rows <= 0 || n_rows >= (1ll << 30)) PCE_FAIL(PCE_EINVAL, "pce_row_order: n_rows=%lld", (long long)n_rows);
+  if (mid >= kv) PCE_FAIL(PCE_EINVAL, "pce_row_order: centre offset %d outside the kernel volume %d", (int)mid, (int)kv);
+  if (order_elems < pce_row_order_elems(n_rows))
+    PCE_FAIL(PCE_EWORKSPACE, "pce_row_order: order holds %lld elements, needs %lld", (long long)order_elems, (long long)pce_row_order_elems(n_rows));
+  hipStream_t s = (hipStream_t)stream;
+  int *tail = order + 2 * n_rows;
+  const unsigned blocks = (unsigned)pce_div_up(n_rows, 256);
+  hipLaunchKernelGGL(order_clear_kernel, dim3(1), dim3(1024), 0, s, tail);
+  PCE_LAUNCH_CHECK("order_clear");
+  hipLaunchKernelGGL(order_mask_kernel, dim3(blocks), dim3(256), 0, s, nbr, (int)kv, (long long)n_rows, (int)mid, order);
+  PCE_LAUNCH_CHECK("order_mask");
+  hipLaunchKernelGGL(order_scan_kernel, dim3(1), dim3(1024), 0, s, tail);
+  PCE_LAUNCH_CHECK("order_scan");
+  hipLaunchKernelGGL(order_scatter_kernel, dim3(blocks), dim3(256), 0, s, (long long)n_rows, order);
+  PCE_LAUNCH_CHECK("order_scatter");
+  int heavy = 0;
+  PCE_HIP(hipMemcpyAsync(&heavy, tail + ORDER_N_HEAVY, sizeof(int), hipMemcpyDeviceToHost, s));
+  PCE_HIP(hipStreamSynchronize(s));
+  *n_heavy_host = heavy;
+  return PCE_OK;
+}
+
+enum { ST_INSERT = 0, ST_QUERY, ST_COUNT, ST_FILL, ST_CSR_A, ST_CSR_B, ST_GRID_BUILD, ST_GRID_QUERY, ST_GRID_QUERY3, ST_ORDER_MASK,
+       ST_ORDER_SCATTER, ST_COUNT_ };
 
 // host-side image of everything the kernels of one batch read
 struct BatchImage {
   ProbDev prob[PCE_MAX_BATCH];
   Job jobs[ST_COUNT_][2 * PCE_MAX_BATCH];      // per stage
   int n_jobs[ST_COUNT_];
-  FillRegion fills[4 * PCE_MAX_BATCH];
+  FillRegion fills[5 * PCE_MAX_BATCH];
   ScanArr scans[2][2 * PCE_MAX_BATCH];  // first scan (segments, input rows), second scan (output rows)
 };
 
@@ -1907,11 +2072,12 @@ extern "C" int pce_kmap_build_batch(const pce_kmap_problem_t *probs, int32_t n_p
     j.kind = kind;
     blk[stage] += (unsigned)pce_div_up(items, 256);
   };
-  auto add_fill = [&](void *p, long long words) {
+  auto add_fill = [&](void *p, long long words, unsigned zero = 0) {
     if (words <= 0) return;
     FillRegion &f = img.fills[n_fill++];
     f.p = (unsigned *)p;
     f.n_words = words;
+    f.zero = zero;
     f.blk0 = fill_blk;
     fill_blk += (unsigned)pce_div_up(words, FILL_WORDS_PER_BLOCK);
   };
@@ -1976,6 +2142,17 @@ extern "C" int pce_kmap_build_batch(const pce_kmap_problem_t *probs, int32_t n_p
     q.oslot = u.oslot;
     q.nbr_out = u.nbr_out;
     q.status = u.status;
+    q.order = nullptr;
+    if (u.order) {
+      // the row order of the ordered output-stationary dataflow, derived from the output-major table once it is filled
+      if (!u.nbr_out) PCE_FAIL(PCE_EINVAL, "pce_kmap_build: the row order needs the output-major neighbour table (nbr_out)");
+      if (q.g.kv > ORDER_MAX_KV - 1) PCE_FAIL(PCE_EINVAL, "pce_kmap_build: the row order takes kernel volumes up to %d", ORDER_MAX_KV - 1);
+      if (n_out >= (1ll << 30)) PCE_FAIL(PCE_ECAPACITY, "pce_kmap_build: too many rows for a row order");
+      q.order = u.order;
+      add_fill(u.order + 2 * n_out, PCE_ORDER_TAIL, 1);
+      add_job(ST_ORDER_MASK, p, 0, n_out);
+      add_job(ST_ORDER_SCATTER, p, 0, n_out);
+    }
     q.want_csr = want_csr;
     q.use_grid = use_grid;
     if (use_grid) {
@@ -2076,6 +2253,14 @@ extern "C" int pce_kmap_build_batch(const pce_kmap_problem_t *probs, int32_t n_p
     hipLaunchKernelGGL(csr_stage_kernel, dim3(blk[ST_CSR_B]), dim3(256), 0, s, P, jl(ST_CSR_B));
     PCE_LAUNCH_CHECK("csr_stage_b");
   }
+  if (blk[ST_ORDER_MASK]) {
+    hipLaunchKernelGGL(order_mask_batch_kernel, dim3(blk[ST_ORDER_MASK]), dim3(256), 0, s, P, jl(ST_ORDER_MASK));
+    PCE_LAUNCH_CHECK("order_mask");
+    hipLaunchKernelGGL(order_scan_batch_kernel, dim3(n_probs), dim3(1024), 0, s, P);
+    PCE_LAUNCH_CHECK("order_scan");
+    hipLaunchKernelGGL(order_scatter_batch_kernel, dim3(blk[ST_ORDER_SCATTER]), dim3(256), 0, s, P, jl(ST_ORDER_SCATTER));
+    PCE_LAUNCH_CHECK("order_scatter");
+  }
   return PCE_OK;
 }
 
@@ -2109,5 +2294,6 @@ extern "C" int pce_kmap_build(const int32_t *in_coords, int64_t n_in, const int3
   u.status = status;
   u.n_batch = 0;   // no batch bound in this signature: the hash table
   u.flags = 0;
+  u.order = nullptr;
   return pce_kmap_build_batch(&u, 1, stream);
 }

@@ -28,13 +28,13 @@ import torch
 import torch.nn as nn
 
 from . import backend
-from .backend import DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS, DATAFLOW_FDS
+from .backend import DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS, DATAFLOW_FDS, DATAFLOW_OSO
 from .sptensor import spTensor
 from .utils import conv_info_decoder, conv_info_encoder, output_stride_compute
 
 _UNIT = conv_info_encoder([1, 1, 1])
 _DATAFLOWS = {"fod": DATAFLOW_FOD, "d2": DATAFLOW_FOD, "gms": DATAFLOW_GMS, "d1": DATAFLOW_GMS, "os": DATAFLOW_OS,
-              "fds": DATAFLOW_FDS}
+              "fds": DATAFLOW_FDS, "oso": DATAFLOW_OSO}
 
 # one record per executed layer when enabled: (N_in, N_out, M, C_in, C_out, dataflow)
 layer_log: Optional[list] = None
@@ -138,10 +138,11 @@ class conv3d(nn.Module):
 
 def _pick_dataflow(km: backend.KernelMap, requested: str, c_in: int, c_out: int, dtype, transposed: bool) -> int:
     env = os.environ.get("PCENGINE_DATAFLOW", "").lower()
-    if env in _DATAFLOWS:
-        return _DATAFLOWS[env]
-    if requested in _DATAFLOWS:
-        return _DATAFLOWS[requested]
+    forced = _DATAFLOWS.get(env, _DATAFLOWS.get(requested))
+    if forced is not None:
+        if forced == DATAFLOW_OSO and not backend.oso_takes(km, c_in, c_out, dtype, transposed):
+            return DATAFLOW_FDS     # the ordered dataflow exists for narrow fp16 submanifold layers only
+        return forced
     if km.tag == "D1":
         return DATAFLOW_GMS
     if km.tag == "D2":

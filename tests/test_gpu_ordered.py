@@ -1,0 +1,156 @@
+"""The ordered output-stationary dataflow: the row order (masks, sections, permutation) against the oracle's map,
+and the layer against the float64 oracle through the C ABI.  Bar: rel-L2 <= 1e-3 (fp16 storage, fp32 accumulate)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+from pcengine_amd import _lib, backend, synth
+from pcengine_amd.backend import DATAFLOW_FDS, DATAFLOW_OS, DATAFLOW_OSO
+from tests.util import DEV, dev_coords, rounded
+
+pytestmark = pytest.mark.gpu
+K3, S1, P0 = (3, 3, 3), (1, 1, 1), (0, 0, 0)
+
+CLOUDS = {
+    "lidar": lambda: synth.lidar_cloud_100k()[::3].copy(),                  # rows mostly without neighbours
+    "surface": lambda: synth.sphere_plane_cloud(),                          # 4.7 pairs per row: mostly heavy rows
+    "dense": lambda: synth.random_cloud(seed=91, n=9000, extent=22, batches=2),
+    "tiny": lambda: synth.random_cloud(seed=92, n=45, extent=5),
+}
+
+
+def _subm(coords, **kw):
+    batches = int(coords[:, 0].max()) + 1
+    return backend.build_kernel_map(dev_coords(coords), K3, S1, P0, [0, 0, 0], coords[:, 1:].max(0).tolist(), True, want_csr=True,
+                                    batchsize=batches, **kw)
+
+
+def _oracle_masks(coords):
+    ref = orc.kernel_map(coords, K3)
+    masks = np.zeros(len(coords), np.int64)
+    for kp in range(27):
+        if kp != 13:
+            masks[ref.omap[ref.kpos[kp]:ref.kpos[kp + 1]]] |= 1 << kp
+    return ref, masks
+
+
+def _popcount(m):
+    return np.array([bin(int(v)).count("1") for v in m])
+
+
+def _key(m):
+    bits = [k for k in range(27) if (int(m) >> k) & 1]
+    return (1024 if len(bits) >= 3 else 0) + bits[0] * 32 + (bits[1] if len(bits) > 1 else 31)
+
+
+@pytest.mark.parametrize("cloud", sorted(CLOUDS))
+def test_row_order_built_with_the_map_and_on_its_own(cloud):
+    """perm is a permutation; rows without neighbours come first, in ascending order within each block of 256; then the
+    rows with one or two neighbours in ascending key order, then the rows with three or more likewise; the masks are
+    the oracle's neighbour patterns and the count of heavy rows is theirs.  The order requested on its own
+    (pce_row_order) has the same masks, sections and keys."""
+    coords = CLOUDS[cloud]()
+    ref, masks = _oracle_masks(coords)
+    km = _subm(coords)
+    n = len(coords)
+    assert km.order is not None and km.order.numel() == 2 * n + 8192
+    lazy = _subm(coords, want_order=False)
+    assert lazy.order is None
+    backend.row_order(lazy)
+    pc = _popcount(masks)
+    for m in (km, lazy):
+        order = m.order.cpu().numpy()
+        perm, got_masks = order[:n].astype(np.int64), order[n:2 * n].view(np.uint32).astype(np.int64)
+        assert np.array_equal(got_masks, masks)
+        assert np.array_equal(np.sort(perm), np.arange(n))
+        assert m.order_heavy == int((pc >= 3).sum())
+        n_plain, n_heavy = int((pc == 0).sum()), int((pc >= 3).sum())
+        sect = masks[perm]
+        assert (sect[:n_plain] == 0).all() and (sect[n_plain:] != 0).all()
+        assert (_popcount(sect[n_plain:n - n_heavy]) <= 2).all() and (_popcount(sect[n - n_heavy:]) >= 3).all()
+        keys = np.array([_key(v) for v in sect[n_plain:]])
+        assert (np.diff(keys) >= 0).all()
+        plain = perm[:n_plain]
+        same_block = plain[1:] // 256 == plain[:-1] // 256
+        assert (np.diff(plain)[same_block] > 0).all()        # a block's plain rows keep their order
+
+
+@pytest.mark.parametrize("cloud", sorted(CLOUDS))
+@pytest.mark.parametrize("c_in,c_out", [(64, 64), (32, 32), (16, 32), (48, 24), (64, 8), (16, 64)])
+def test_ordered_dataflow_against_the_oracle(cloud, c_in, c_out):
+    coords = CLOUDS[cloud]()
+    ref, _ = _oracle_masks(coords)
+    km = _subm(coords)
+    n = len(coords)
+    dt = torch.float16
+    f, w = synth.features(c_in, n, c_in), synth.weights(c_out, 27, c_in, c_out)
+    bias = np.random.default_rng(c_in).standard_normal(c_out) * 0.1
+    res = synth.features(c_out + 1, n, c_out)
+    fd, wd = torch.as_tensor(f, device=DEV).to(dt), torch.as_tensor(w, device=DEV).to(dt)
+    bd, rd = torch.as_tensor(bias, device=DEV).to(dt), torch.as_tensor(res, device=DEV).to(dt)
+    packed = backend.pack_weights(wd)
+    plain = orc.conv_forward(rounded(f, dt), rounded(w, dt), ref, K3)
+    out = backend.conv_forward(fd, wd, km, DATAFLOW_OSO, packed=packed)
+    assert orc.rel_l2(out.double().cpu().numpy(), plain) <= 1e-3
+    assert orc.rel_l2(backend.conv_forward(fd, wd, km, DATAFLOW_OSO).double().cpu().numpy(), plain) <= 1e-3    # packs on the fly
+    want = np.maximum(plain + rounded(bias, dt) + rounded(res, dt), 0)
+    out = backend.conv_forward(fd, wd, km, DATAFLOW_OSO, packed=packed, bias=bd, residual=rd, act="relu")
+    assert orc.rel_l2(out.double().cpu().numpy(), want) <= 1e-3
+    leaky = plain + rounded(bias, dt)
+    leaky = np.where(leaky > 0, leaky, 0.1 * leaky)
+    out = backend.conv_forward(fd, wd, km, DATAFLOW_OSO, packed=packed, bias=bd, act=("leaky_relu", 0.1))
+    assert orc.rel_l2(out.double().cpu().numpy(), leaky) <= 1e-3
+    # every row is computed by one wavefront (or one workgroup) alone: two runs agree bit for bit, whatever the
+    # positions the rows of equal keys took in the order
+    again = backend.conv_forward(fd, wd, _subm(coords), DATAFLOW_OSO, packed=packed, bias=bd, act=("leaky_relu", 0.1))
+    assert torch.equal(out, again)
+
+
+def test_ordered_dataflow_on_column_slices_and_the_selector():
+    coords = CLOUDS["lidar"]()
+    km = _subm(coords)
+    n, c = len(coords), 32
+    wide_in = torch.full((n, c + 24), 5.0, dtype=torch.float16, device=DEV)
+    f = torch.as_tensor(synth.features(1, n, c), device=DEV).half()
+    wide_in[:, 8:8 + c] = f
+    wide_out = torch.full((n, 2 * c + 16), -2.0, dtype=torch.float16, device=DEV)
+    w = torch.as_tensor(synth.weights(1, 27, c, c), device=DEV).half()
+    packed = backend.pack_weights(w)
+    want = backend.conv_forward(f, w, km, DATAFLOW_OSO, packed=packed)
+    got = backend.conv_forward(wide_in[:, 8:8 + c], w, km, DATAFLOW_OSO, packed=packed, out=wide_out[:, c:2 * c])
+    assert torch.equal(got, want) and bool((wide_out[:, :c] == -2.0).all()) and bool((wide_out[:, 2 * c:] == -2.0).all())
+    assert backend.select_dataflow(km, c, c, torch.float16) == DATAFLOW_OSO
+    assert backend.select_dataflow(km, c, c, torch.float32) != DATAFLOW_OSO
+    assert backend.select_dataflow(km, 96, 96, torch.float16) != DATAFLOW_OSO
+    # the two pair-proportional dataflows agree to fp16 rounding (they round partial sums at different places)
+    fds = backend.conv_forward(f, w, km, DATAFLOW_FDS, packed=packed)
+    assert float((fds.float() - want.float()).norm() / want.float().norm()) <= 1e-3
+
+
+def test_ordered_dataflow_argument_errors():
+    lib = _lib.load()
+    coords = CLOUDS["tiny"]()
+    km = _subm(coords)
+    n = len(coords)
+    s = torch.cuda.current_stream().cuda_stream
+    f = torch.zeros((n, 32), dtype=torch.float16, device=DEV)
+    w = torch.zeros((27, 32, 32), dtype=torch.float16, device=DEV)
+    pk = backend.pack_weights(w)
+    out = torch.zeros((n, 32), dtype=torch.float16, device=DEV)
+    call = lambda dtype, c_in, c_out, mid, heavy, packed=pk: lib.pce_conv_fwd_oso(
+        f.data_ptr(), w.data_ptr(), packed.data_ptr() if packed is not None else None, out.data_ptr(), dtype, n, n, c_in, c_out, 27, mid,
+        km.nbr_out.data_ptr(), km.order.data_ptr(), heavy, None, s)
+    assert call(_lib.PCE_F16, 32, 32, 13, km.order_heavy) == _lib.PCE_OK
+    assert call(_lib.PCE_F32, 32, 32, 13, km.order_heavy) == _lib.PCE_EINVAL
+    assert call(_lib.PCE_F16, 32, 32, -1, km.order_heavy) == _lib.PCE_EINVAL        # no centre offset
+    assert call(_lib.PCE_F16, 32, 32, 13, n + 1) == _lib.PCE_EINVAL
+    assert call(_lib.PCE_F16, 32, 32, 13, km.order_heavy, None) == _lib.PCE_EINVAL    # weights not packed
+    assert call(_lib.PCE_F16, 128, 32, 13, km.order_heavy) == _lib.PCE_EINVAL
+    heavy = _lib.c_int64(0)
+    order = torch.zeros(lib.pce_row_order_elems(n), dtype=torch.int32, device=DEV)
+    assert lib.pce_row_order(km.nbr_out.data_ptr(), 27, n, 13, order.data_ptr(), order.numel() - 1, heavy, s) == _lib.PCE_EWORKSPACE
+    assert lib.pce_row_order(km.nbr_out.data_ptr(), 125, n, 62, order.data_ptr(), order.numel(), heavy, s) == _lib.PCE_EINVAL
+    with pytest.raises(ValueError):
+        backend.conv_forward(torch.zeros((n, 96), dtype=torch.float16, device=DEV), torch.zeros((27, 96, 32), dtype=torch.float16, device=DEV),
+                             km, DATAFLOW_OSO)

@@ -76,8 +76,8 @@ def test_selector_is_monotone_in_density():
     lib = _lib.load()
     n = 100000
     picks = [lib.pce_select_dataflow(n, n, int(rho * n), 64, 64, 27, 0) for rho in (0.1, 0.5, 1.0, 3.0, 8.0, 20.0)]
-    assert picks[0] == _lib.DATAFLOW_FDS and picks[-1] == _lib.DATAFLOW_OS
-    order = {_lib.DATAFLOW_FDS: 0, _lib.DATAFLOW_FOD: 0, _lib.DATAFLOW_GMS: 1, _lib.DATAFLOW_OS: 2}
+    assert picks[0] == _lib.DATAFLOW_OSO and picks[-1] == _lib.DATAFLOW_OS
+    order = {_lib.DATAFLOW_OSO: 0, _lib.DATAFLOW_FDS: 0, _lib.DATAFLOW_FOD: 0, _lib.DATAFLOW_GMS: 1, _lib.DATAFLOW_OS: 2}
     ranks = [order[p] for p in picks]
     assert ranks == sorted(ranks)
 
@@ -85,9 +85,14 @@ def test_selector_is_monotone_in_density():
 def test_selector_on_measured_layers():
     """Layers whose four dataflows were timed on the GPU: the selector picks the fastest (or one within 2 % of it)."""
     lib = _lib.load()
-    FDS, OS = _lib.DATAFLOW_FDS, _lib.DATAFLOW_OS
+    FDS, OS, OSO = _lib.DATAFLOW_FDS, _lib.DATAFLOW_OS, _lib.DATAFLOW_OSO
     cases = [  # n_in, n_out, pairs, c_in, c_out, kv, expected
-        (149866, 149866, 30620, 64, 64, 27, FDS),      # the headline layer
+        (149866, 149866, 30620, 64, 64, 27, OSO),      # the headline layer
+        (97941, 97941, 80234, 32, 32, 27, OSO),        # narrow layers of a LiDAR network: rho 0.8 and 3.0
+        (89469, 89469, 271786, 64, 64, 27, OSO),
+        (541185, 541185, 2852000, 64, 64, 27, OSO),    # indoor batch, rho 5.3: equal to output-stationary, 0.6 of deferred scatter
+        (99692, 99692, 13406, 96, 96, 27, FDS),        # wider than the ordered kernel takes
+        (65807, 65807, 586656, 64, 64, 27, OS),        # rho 8.9: the dense tiles
         (149866, 146018, 149866, 64, 128, 8, FDS),     # k2s2 on a LiDAR cloud: one pair for nearly every row
         (216268, 53439, 215000, 128, 128, 8, OS),      # k2s2 on an indoor batch, four pairs per row
         (65807, 25916, 64194, 128, 128, 8, OS),
@@ -99,6 +104,9 @@ def test_selector_on_measured_layers():
     ]
     for n_in, n_out, pairs, ci, co, kv, want in cases:
         assert lib.pce_select_dataflow(n_in, n_out, pairs, ci, co, kv, _lib.PCE_F16) == want, (n_in, n_out, ci, co, kv)
+    # fp32 and strided layers never take the ordered dataflow
+    assert lib.pce_select_dataflow(20804, 20804, 98238, 16, 16, 27, _lib.PCE_F32) == FDS
+    assert lib.pce_select_dataflow(149866, 146018, 149866, 32, 32, 8, _lib.PCE_F16) != OSO
 
 
 def test_codes_and_strides():
