@@ -750,17 +750,19 @@ __global__ void __launch_bounds__(256) chain_fill_kernel(ChainDev d) {
 }
 
 __global__ void __launch_bounds__(256) chain_mark_kernel(const int4 *__restrict__ coords, long long n_in, ChainDev d) {
-  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n_in) return;
-  int4 c = coords[i];
-  if (!pce_coord_ok(c.x, c.y, c.z, c.w)) {
+  // no lane leaves early: the lanes of a wavefront combine their bits below
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  bool live = i < n_in;
+  int4 c = live ? coords[i] : make_int4(0, 0, 0, 0);
+  if (live && !pce_coord_ok(c.x, c.y, c.z, c.w)) {
     d.lv[0].status[0] = 1;
-    return;
+    live = false;
   }
-  if (c.x >= d.lv[0].grid.n_batch) {
+  if (live && c.x >= d.lv[0].grid.n_batch) {
     d.lv[0].status[2] = 1;
-    return;
+    live = false;
   }
+  const int lane = threadIdx.x & 63;
   int p[3] = {c.y, c.z, c.w};
   for (int l = 0; l < d.levels; ++l) {
     const ChainLevel &v = d.lv[l];
@@ -773,14 +775,35 @@ __global__ void __launch_bounds__(256) chain_mark_kernel(const int4 *__restrict_
       ok &= q >= v.lo[a] && q <= v.hi[a];
       bad |= q < 0 || q >= PCE_COORD_BOUND;
     }
-    if (!ok) return;                        // clipped here: absent from every deeper level too
-    if (bad) {                              // inside the stated bounds but outside what a strided layer can address
+    if (!ok) live = false;                  // clipped here: absent from every deeper level too
+    if (live && bad) {                      // inside the stated bounds but outside what a strided layer can address
       d.lv[0].status[0] = 1;
-      return;
+      live = false;
     }
-    long long bit = (((long long)c.x * v.grid.ext[0] + (p[0] - v.grid.lo[0])) * v.grid.ext[1] + (p[1] - v.grid.lo[1])) *
-                        v.grid.ext[2] + (p[2] - v.grid.lo[2]);
-    atomicOr(&v.bits[bit >> 5], 1u << (bit & 31));
+    const long long bit = !live ? 0ll
+                                : (((long long)c.x * v.grid.ext[0] + (p[0] - v.grid.lo[0])) * v.grid.ext[1] + (p[1] - v.grid.lo[1])) *
+                                          v.grid.ext[2] + (p[2] - v.grid.lo[2]);
+    const long long word = bit >> 5;
+    const unsigned m = 1u << (bit & 31);
+    bool pending = live;
+    if (l > 0) {
+      // Below the first level many lanes of a wavefront (consecutive points of a sorted cloud) fall into one word:
+      // the lanes of up to four words combine their bits and one lane issues the atomic; what is left goes alone.
+      unsigned long long todo = __ballot(pending);
+      for (int it = 0; it < 4 && todo; ++it) {
+        const int leader = __ffsll((long long)todo) - 1;
+        const long long lw = ((long long)__shfl((int)(word >> 32), leader, PCE_WAVE) << 32) |
+                             (unsigned)__shfl((int)(word & 0xFFFFFFFFll), leader, PCE_WAVE);
+        const bool same = pending && word == lw;
+        unsigned mm = same ? m : 0u;
+#pragma unroll
+        for (int dd = 1; dd < PCE_WAVE; dd <<= 1) mm |= (unsigned)__shfl_xor((int)mm, dd, PCE_WAVE);
+        if (lane == leader) atomicOr(&v.bits[lw], mm);
+        if (same) pending = false;
+        todo &= ~__ballot(same);
+      }
+    }
+    if (pending) atomicOr(&v.bits[word], m);
   }
 }
 
