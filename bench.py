@@ -263,6 +263,18 @@ def main() -> int:
               for f in names if f != flow and f != DATAFLOW_FOD and takes(f)}
     others[names[DATAFLOW_FOD]] = ev_ms(lambda: step(DATAFLOW_FOD), max(20, args.steps // 4), 5)   # allocates: eager
 
+    # What the platform itself reaches on tensors of this size, in the same graph replays: a device copy of the
+    # feature tensor into the output tensor (reads and writes what the layer must at least read and write, with no
+    # indices and no arithmetic) and the centre offset's dense GEMM alone (one launch, rows in storage order).
+    floors = {}
+    if c_in == c_out:
+        dst = torch.empty_like(fd)
+        floors["device_copy_ms"] = timer(lambda: dst.copy_(fd), max(20, args.steps // 4), 5)[0]
+        del dst
+    w_mid = wd[13].contiguous()
+    pk_mid = backend.pack_weights(w_mid)
+    floors["centre_gemm_only_ms"] = timer(lambda: backend.dense_forward(fd, w_mid, packed=pk_mid), max(20, args.steps // 4), 5)[0]
+
     # algorithmic bytes of the layer: every tensor once + the pair list
     b_conv = n * c_in * e + n * c_out * e + 27 * c_in * c_out * e + 8 * M
     flops = 2.0 * (M + n) * c_in * c_out
@@ -331,7 +343,10 @@ def main() -> int:
                   "eager_ms_per_step": round(eager_ms, 5), "eager_wall_ms_per_step": round(wall_ms, 5),
                   "map_build_ms": round(map_ms, 4), "map_build_hash_table_ms": round(map_hash_ms, 4),
                   "stage_ms": {k: round(v, 5) for k, v in stages.items()},
-                  "other_dataflows_ms": {k: round(v, 5) for k, v in others.items()}},
+                  "other_dataflows_ms": {k: round(v, 5) for k, v in others.items()},
+                  "floors": {**{k: round(v, 5) for k, v in floors.items()},
+                             **({"device_copy_frac_of_hbm_peak": round(2 * n * c_in * e / (floors["device_copy_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+                                if "device_copy_ms" in floors else {})}},
     }
 
     # ---- configuration 4: MinkUNet-style forward, ~100k voxels, fp16, BN folded --------------------
