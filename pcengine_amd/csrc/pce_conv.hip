@@ -2423,19 +2423,40 @@ __global__ void __launch_bounds__(256, 4) wave_os_kernel(TileArgs a, const int *
   constexpr int REGION = REGION0 > 256 ? REGION0 : 256;   // also one accumulator block of 64 lanes (see below)
   static_assert(REGION * 16 >= 64 * 64, "a wavefront's region holds one accumulator block of all its lanes");
   __shared__ __attribute__((aligned(16))) half8 Pl[4][REGION];
+  __shared__ __attribute__((aligned(16))) half8 Wc[KS * 2 * NB * 32];   // the centre offset's weights, shared by the workgroup
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int l32 = lane & 31, g = lane >> 5;
+  const half_t *Wp = (const half_t *)a.Wp;
+  const long long wstep = (long long)a.k8_total * a.n_pad * 8;
+  // every wavefront copies its share of the centre weights (one copy of them per workgroup instead of one per wavefront)
+  {
+    constexpr int FR = KS * 2 * NB * 32;   // fragments: [k8][column]
+#pragma unroll
+    for (int i = 0; i < (FR + 255) / 256; ++i) {
+      const int f = i * 256 + wave * 64 + lane;
+      const half_t *gp = Wp + mid * wstep + (long long)(f < FR ? f : FR - 1) * 8;
+      if (i * 256 + wave * 64 < FR)   // wavefront-uniform
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
+                                         (__attribute__((address_space(3))) void *)&Wc[i * 256 + wave * 64], 16, 0, 0);
+    }
+  }
   const bool heavy = (int)blockIdx.x < heavy_wgs;   // the same for the whole workgroup
   long long j0, j_end;
+  bool idle = false;
   if (heavy) {
     j0 = n_main + (long long)blockIdx.x * 32;
     j_end = a.n_rows;
   } else {
     const long long chunks = (n_main + 31) / 32;
     const long long chunk = chunks - 1 - (((long long)blockIdx.x - heavy_wgs) * 4 + wave);
-    if (chunk < 0) return;
-    j0 = chunk * 32;
+    idle = chunk < 0;
+    j0 = idle ? 0 : chunk * 32;
     j_end = n_main;
+  }
+  if (idle) {   // still joins the barrier behind the weight copies
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    return;
   }
   const half_t *A = (const half_t *)a.A;
   const int orow = j0 + l32 < j_end ? perm[j0 + l32] : -1;
@@ -2449,8 +2470,6 @@ __global__ void __launch_bounds__(256, 4) wave_os_kernel(TileArgs a, const int *
   // of a layer does not depend on where the counting sort happened to put a row among those of its key.)
   if (heavy) todo &= 0x11111111u << wave;
   const bool centre = !heavy || wave == 0;
-  const half_t *Wp = (const half_t *)a.Wp;
-  const long long wstep = (long long)a.k8_total * a.n_pad * 8;
   half8 wf[KS][NB];
   if (centre) {
     // centre rows -> LDS, in line order (a valid row stands in for one past the end)
@@ -2462,11 +2481,6 @@ __global__ void __launch_bounds__(256, 4) wave_os_kernel(TileArgs a, const int *
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
                                        (__attribute__((address_space(3))) void *)&Pl[wave][it * 64], 16, 0, 0);
     }
-#pragma unroll
-    for (int s = 0; s < KS; ++s)
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-        wf[s][nb] = *reinterpret_cast<const half8 *>(Wp + mid * wstep + ((long long)(2 * s + g) * a.n_pad + nb * 32 + l32) * 8);
   }
   // the neighbour of this lane's row at the first offset of the union, requested while the centre rows travel
   int k_next = todo ? __ffs((int)todo) - 1 : -1;
@@ -2476,9 +2490,13 @@ __global__ void __launch_bounds__(256, 4) wave_os_kernel(TileArgs a, const int *
   for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
     for (int j = 0; j < 16; ++j) acc[nb][j] = 0.f;
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();   // the centre weights of all four wavefronts' copies (and this wavefront's rows) are in LDS
   if (centre) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) wf[s][nb] = Wc[(2 * s + g) * (NB * 32) + nb * 32 + l32];
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
       const half8 af = Pl[wave][l32 * PPR + ((2 * s + g) ^ row_swizzle<PPR>(l32))];
@@ -2564,6 +2582,8 @@ extern "C" int pce_conv_fwd_oso(const void *in, const void *w, const void *wp, v
   const int *perm = order;
   const unsigned *rmask = (const unsigned *)(order + n_out);
   const int nb = (c_out + 31) / 32, ks = c_in / 16;
+  if (a.n_pad != nb * 32 || a.k8_total != 2 * ks)
+    PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: packed weights are %d x %d fragments per offset, expected %d x %d", a.k8_total, a.n_pad, 2 * ks, nb * 32);
   hipStream_t s = (hipStream_t)stream;
 #define PCE_WOS_CASE(NB_, KS_)                                                                              \
   if (nb == NB_ && ks == KS_) {                                                                              \
