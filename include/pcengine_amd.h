@@ -375,8 +375,9 @@ int pce_conv_fwd_os(const void *in_feats, const void *weight, const void *weight
  * the results of the layer do not.  pce_conv_fwd_oso then runs the layer as one launch: a wavefront takes 32 rows
  * of that order, multiplies their centre rows, gathers for each offset any of them has the neighbours of the rows
  * that have it, and stores each finished row once (epilogue fused); the rows of the last part, whose offsets are
- * many, go 32 to a workgroup whose four wavefronts share the offsets.  PCE_F16, c_in a multiple of 16 and at most
- * 64, c_out a multiple of 8 and at most 64, packed weights, mid >= 0; PCE_EINVAL otherwise.  Takes the row strides
+ * many, go 32 to a workgroup whose four wavefronts share the offsets.  PCE_F16: c_in a multiple of 16 and at most
+ * 64, c_out a multiple of 8 and at most 64, packed weights; PCE_F32: c_in and c_out multiples of 8 and at most 32
+ * (weight_packed is not read); mid >= 0; PCE_EINVAL otherwise.  Takes the row strides
  * of pce_epilogue_t.  No counterpart in the reference: it computes what the fetch-on-demand kernels compute
  * (backend/spconv.cuh:1567-1730) with the scatter-add replaced by register accumulation, as pce_conv_fwd_os. */
 int64_t pce_row_order_elems(int64_t n_rows);

@@ -498,8 +498,11 @@ def row_order(km: KernelMap) -> torch.Tensor:
 
 def oso_takes(km: KernelMap, c_in: int, c_out: int, dtype: torch.dtype, transposed: bool = False) -> bool:
     """Shapes the ordered output-stationary dataflow exists for."""
-    return (km.subm and not transposed and dtype == torch.float16 and km.kv <= 31 and c_in % 16 == 0 and c_in <= 64
-            and c_out % 8 == 0 and c_out <= 64)
+    if not km.subm or transposed or km.kv > 31:
+        return False
+    if dtype == torch.float32:
+        return c_in % 8 == 0 and c_in <= 32 and c_out % 8 == 0 and c_out <= 32
+    return dtype == torch.float16 and c_in % 16 == 0 and c_in <= 64 and c_out % 8 == 0 and c_out <= 64
 
 
 def ensure_nbr(km: KernelMap, transposed: bool) -> None:
@@ -701,10 +704,10 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
                                         km.kpos.data_ptr(), km.qkpos.data_ptr(), km.qsum, buffer.data_ptr(), buffer.numel(), epi, s))
     elif dataflow == DATAFLOW_OSO:
         if not oso_takes(km, c_in, c_out, feats.dtype, transposed):
-            raise ValueError("the ordered output-stationary dataflow takes fp16 submanifold layers of at most 64 channels "
-                             "(c_in a multiple of 16, c_out of 8)")
+            raise ValueError("the ordered output-stationary dataflow takes submanifold layers in fp16 of at most 64 channels "
+                             "(c_in a multiple of 16, c_out of 8) or in fp32 of at most 32 (multiples of 8)")
         if packed is None:
-            packed = pack_weights(weight)
+            packed = pack_weights(weight)      # None for fp32: that form reads the weights as they are
         order = row_order(km)
         _lib.check(lib.pce_conv_fwd_oso(feats.data_ptr(), weight.data_ptr(), _ptr(packed), out.data_ptr(), dt, n_in, n_out,
                                         c_in, c_out, kv, mid, km.nbr_out.data_ptr(), order.data_ptr(), km.order_heavy, epi, s))

@@ -2554,6 +2554,114 @@ __global__ void __launch_bounds__(256, 4) wave_os_kernel(TileArgs a, const int *
   store_rows_via_lds<half_t, NB>(V, Pl[wave], (half_t *)a.out, orow, a, 0, lane, l32, g, a.stream);
 }
 
+// The same dataflow for very narrow fp32 layers (c_in = 8 KQ up to 32, c_out up to 32: the 16-channel fp32 layer
+// of the reference's own test case).  Rows are 32 to 128 bytes, so nothing is staged on the way in: of a row's c_in
+// values the lane with g = 0 holds the first half, the lane with g = 1 the second (KQ 16-byte loads each), and MFMA
+// step (q, e) of v_mfma_f32_32x32x2_f32 contracts k = 4 q + e (lanes 0-31) with k = c_in / 2 + 4 q + e (lanes 32-63);
+// the weights of an offset are read in that order, one value per lane and step, 128 contiguous bytes per half.
+template <int KQ>
+__global__ void __launch_bounds__(256, 4) wave_os_f32_kernel(TileArgs a, const int *__restrict__ perm,
+                                                             const unsigned *__restrict__ rmask, int mid, long long n_main,
+                                                             int heavy_wgs) {
+  constexpr int KH = 4 * KQ;   // values of a row per lane
+  constexpr int REGION = WaveLds<1>::PIECES > 256 ? WaveLds<1>::PIECES : 256;   // output staging; one accumulator block of 64 lanes
+  __shared__ __attribute__((aligned(16))) f32x4 Pl[4][REGION];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int l32 = lane & 31, g = lane >> 5;
+  const bool heavy = (int)blockIdx.x < heavy_wgs;   // the same for the whole workgroup
+  long long j0, j_end;
+  if (heavy) {
+    j0 = n_main + (long long)blockIdx.x * 32;
+    j_end = a.n_rows;
+  } else {
+    const long long chunks = (n_main + 31) / 32;
+    const long long chunk = chunks - 1 - (((long long)blockIdx.x - heavy_wgs) * 4 + wave);
+    if (chunk < 0) return;
+    j0 = chunk * 32;
+    j_end = n_main;
+  }
+  const float *A = (const float *)a.A;
+  const float *W = (const float *)a.W;
+  const int orow = j0 + l32 < j_end ? perm[j0 + l32] : -1;
+  const unsigned m = orow >= 0 ? rmask[orow] : 0u;
+  unsigned u = m;
+#pragma unroll
+  for (int d = 1; d < 32; d <<= 1) u |= (unsigned)__shfl_xor((int)u, d, PCE_WAVE);
+  unsigned todo = __builtin_amdgcn_readfirstlane(u);   // offsets any of the 32 rows has: the same in every lane
+  if (heavy) todo &= 0x11111111u << wave;               // see wave_os_kernel: a split that depends on the offset alone
+  const bool centre = !heavy || wave == 0;
+  const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+  // this lane's half of a row; the weights of offset k in the order the MFMA steps contract them
+  // (every load is issued by every lane, from a valid address, and zeroed afterwards where it does not count: a load
+  // under a lane condition becomes a branch with its own wait, and the loads of an offset would go out in pairs)
+  auto load_row = [&](int row, f32x4 (&af)[KQ]) {
+    const float *p = A + (long long)(row >= 0 ? row : 0) * a.lda + g * KH;
+#pragma unroll
+    for (int q = 0; q < KQ; ++q) af[q] = *reinterpret_cast<const f32x4 *>(p + 4 * q);
+    if (row < 0) {
+#pragma unroll
+      for (int q = 0; q < KQ; ++q) af[q] = zero4;
+    }
+  };
+  auto load_weights = [&](int k, float (&wf)[KH]) {
+    const float *Wk = W + ((long long)k * a.c_in + g * KH) * a.c_out + (l32 < a.c_out ? l32 : 0);
+#pragma unroll
+    for (int s = 0; s < KH; ++s) wf[s] = Wk[(long long)s * a.c_out];
+    if (l32 >= a.c_out) {
+#pragma unroll
+      for (int s = 0; s < KH; ++s) wf[s] = 0.f;
+    }
+  };
+  f32x16 acc[1];
+#pragma unroll
+  for (int j = 0; j < 16; ++j) acc[0][j] = 0.f;
+  int k_next = todo ? __ffs((int)todo) - 1 : -1;
+  int nb_next = (k_next >= 0 && ((m >> k_next) & 1u)) ? a.nbr[(long long)k_next * a.n_rows + orow] : -1;
+  if (centre) {
+    f32x4 af[KQ];
+    float wf[KH];
+    load_row(orow, af);
+    load_weights(mid, wf);
+#pragma unroll
+    for (int s = 0; s < KH; ++s) acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(wf[s], af[s / 4][s % 4], acc[0], 0, 0, 0);
+  }
+  while (k_next >= 0) {
+    const int k = k_next, nrow = nb_next;
+    todo &= todo - 1u;
+    f32x4 af[KQ];
+    float wf[KH];
+    load_row(nrow, af);
+    load_weights(k, wf);
+    k_next = todo ? __ffs((int)todo) - 1 : -1;
+    nb_next = (k_next >= 0 && ((m >> k_next) & 1u)) ? a.nbr[(long long)k_next * a.n_rows + orow] : -1;
+#pragma unroll
+    for (int s = 0; s < KH; ++s) acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(wf[s], af[s / 4][s % 4], acc[0], 0, 0, 0);
+  }
+  if (heavy) {
+    // wavefronts 1..3 hand their accumulators to wavefront 0 through their own regions
+    f32x16 *mine = reinterpret_cast<f32x16 *>(&Pl[wave][0]);
+    if (wave > 0) mine[lane] = acc[0];
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w2 = 1; w2 < 4; ++w2) {
+      const f32x16 other = reinterpret_cast<const f32x16 *>(&Pl[w2][0])[lane];
+#pragma unroll
+      for (int j = 0; j < 16; ++j) acc[0][j] += other[j];
+    }
+  }
+  float V[1][2][8];
+  gather_row_pieces<1>(acc, V, g);
+  if (a.bias || a.res || a.act) epilogue_row_pieces<float, 1, true>(V, a, orow, 0, g, a.act != PCE_ACT_NONE);
+  store_rows_via_lds<float, 1>(V, Pl[wave], (float *)a.out, orow, a, 0, lane, l32, g, a.stream);
+}
+
+// shapes the fp32 form takes
+static bool wave_os_f32_ok(const TileArgs &a, int kv, int mid) {
+  return a.a_vec && a.o_vec && a.c_in % 8 == 0 && a.c_in <= 32 && a.c_out % 8 == 0 && a.c_out <= 32 && kv < ORDER_MAX_KV &&
+         mid >= 0 && mid < kv && aligned16(a.bias) && aligned16(a.res);
+}
+
 // shapes the ordered-row kernel takes: fp16, at most 64 channels either side, a centre offset
 static bool wave_os_ok(const TileArgs &a, int kv, int mid) {
   return wave_gemm_ok(a, 2) && kv < ORDER_MAX_KV && mid >= 0 && mid < kv && aligned16(a.bias) && aligned16(a.res);
@@ -2567,12 +2675,17 @@ extern "C" int pce_conv_fwd_oso(const void *in, const void *w, const void *wp, v
   if (!nbr || !order) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: null neighbour table or row order");
   Epi e;
   if ((rc = read_epilogue("pce_conv_fwd_oso", epilogue, out, &e, c_in, c_out))) return rc;
-  TileArgs a = base_args<half_t>(in, w, wp, kv, c_in, c_out, e.lda);
-  set_out<half_t>(&a, out, false, n_out, e.ldo);
+  const bool f32 = dtype == PCE_F32;
+  TileArgs a = f32 ? base_args<float>(in, w, wp, kv, c_in, c_out, e.lda) : base_args<half_t>(in, w, wp, kv, c_in, c_out, e.lda);
+  if (f32)
+    set_out<float>(&a, out, false, n_out, e.ldo);
+  else
+    set_out<half_t>(&a, out, false, n_out, e.ldo);
   set_epi(&a, e);
-  if (dtype != PCE_F16 || !wave_os_ok(a, kv, mid))
-    PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: takes fp16 submanifold layers of at most 64 channels (multiples of 16 in, 8 out) with packed "
-                         "weights and 16-byte aligned rows; got dtype %d, %d -> %d channels, kv %d, mid %d", (int)dtype, (int)c_in, (int)c_out, (int)kv, (int)mid);
+  if (f32 ? !wave_os_f32_ok(a, kv, mid) : !wave_os_ok(a, kv, mid))
+    PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: takes submanifold layers in fp16 of at most 64 channels (multiples of 16 in, 8 out, packed "
+                         "weights) or in fp32 of at most 32 (multiples of 8), 16-byte aligned rows; got dtype %d, %d -> %d "
+                         "channels, kv %d, mid %d", (int)dtype, (int)c_in, (int)c_out, (int)kv, (int)mid);
   if (n_heavy < 0 || n_heavy > n_out) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: n_heavy=%lld outside [0, n_out]", (long long)n_heavy);
   a.nbr = nbr;
   a.n_rows = n_out;
@@ -2582,6 +2695,19 @@ extern "C" int pce_conv_fwd_oso(const void *in, const void *w, const void *wp, v
   const unsigned grid = (unsigned)(heavy_wgs + main_wgs);
   const int *perm = order;
   const unsigned *rmask = (const unsigned *)(order + n_out);
+  if (f32) {
+    hipStream_t s32 = (hipStream_t)stream;
+#define PCE_WOS32_CASE(KQ_)                                                                                       \
+  if (c_in == 8 * KQ_) {                                                                                           \
+    hipLaunchKernelGGL((wave_os_f32_kernel<KQ_>), dim3(grid), dim3(256), 0, s32, a, perm, rmask, (int)mid, n_main,  \
+                       (int)heavy_wgs);                                                                            \
+    PCE_LAUNCH_CHECK("wave_os_f32");                                                                               \
+    return PCE_OK;                                                                                                 \
+  }
+    PCE_WOS32_CASE(1) PCE_WOS32_CASE(2) PCE_WOS32_CASE(3) PCE_WOS32_CASE(4)
+#undef PCE_WOS32_CASE
+    PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: unsupported fp32 width c_in=%d", (int)c_in);
+  }
   const int nb = (c_out + 31) / 32, ks = c_in / 16;
   if (a.n_pad != nb * 32 || a.k8_total != 2 * ks)
     PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: packed weights are %d x %d fragments per offset, expected %d x %d", a.k8_total, a.n_pad, 2 * ks, nb * 32);
@@ -3487,6 +3613,9 @@ extern "C" int pce_select_dataflow(int64_t n_in, int64_t n_out, int64_t n_pairs,
   // scatter with bias, residual and ReLU fused: 0.78-0.93 of its time at 0.1-0.2 pairs per row (100-150 k voxels,
   // 16-64 channels), 0.62-0.83 at 0.8, 0.64-0.83 at 3, 0.60-0.62 at 5.3 (541 k voxels, where it equals plain
   // output-stationary); beyond that the dense output-stationary tiles below take over.
+  if (dtype == PCE_F32 && n_in == n_out && kv >= 3 && kv <= 31 && (kv & 1) && c_in % 8 == 0 && c_in <= 32 && c_out % 8 == 0 &&
+      c_out <= 32 && rho <= 6.0)
+    return PCE_DATAFLOW_OSO;   // the fp32 form: 20 804 rows, 16 -> 16 channels, 4.7 pairs per row against deferred scatter
   if (dtype == PCE_F16 && n_in == n_out && kv >= 3 && kv <= 31 && (kv & 1) && c_in % 16 == 0 && c_in <= 64 && c_out % 8 == 0 &&
       c_out <= 64 && rho <= 6.0)
     return PCE_DATAFLOW_OSO;

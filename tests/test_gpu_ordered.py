@@ -107,6 +107,39 @@ def test_ordered_dataflow_against_the_oracle(cloud, c_in, c_out):
     assert torch.equal(out, again)
 
 
+@pytest.mark.parametrize("cloud", sorted(CLOUDS))
+@pytest.mark.parametrize("c_in,c_out", [(16, 16), (8, 32), (32, 8), (24, 24), (32, 32)])
+def test_ordered_dataflow_fp32_against_the_oracle(cloud, c_in, c_out):
+    """The fp32 form (at most 32 channels either side): 1e-5 against the float64 oracle, with and without the epilogue."""
+    coords = CLOUDS[cloud]()
+    ref, _ = _oracle_masks(coords)
+    km = _subm(coords)
+    n = len(coords)
+    f, w = synth.features(c_in, n, c_in), synth.weights(c_out, 27, c_in, c_out)
+    bias = (np.random.default_rng(c_in).standard_normal(c_out) * 0.1).astype(np.float32)
+    res = synth.features(c_out + 1, n, c_out)
+    fd, wd = torch.as_tensor(f, device=DEV).float(), torch.as_tensor(w, device=DEV).float()
+    bd, rd = torch.as_tensor(bias, device=DEV).float(), torch.as_tensor(res, device=DEV).float()
+    plain = orc.conv_forward(f.astype(np.float32), w.astype(np.float32), ref, K3)
+    out = backend.conv_forward(fd, wd, km, DATAFLOW_OSO)
+    assert orc.rel_l2(out.double().cpu().numpy(), plain) <= 1e-5
+    want = np.maximum(plain + bias + res.astype(np.float32), 0)
+    out = backend.conv_forward(fd, wd, km, DATAFLOW_OSO, bias=bd, residual=rd, act="relu")
+    assert orc.rel_l2(out.double().cpu().numpy(), want) <= 1e-5
+    leaky = plain + bias
+    leaky = np.where(leaky > 0, leaky, 0.1 * leaky)
+    out = backend.conv_forward(fd, wd, km, DATAFLOW_OSO, bias=bd, act=("leaky_relu", 0.1))
+    assert orc.rel_l2(out.double().cpu().numpy(), leaky) <= 1e-5
+    again = backend.conv_forward(fd, wd, _subm(coords), DATAFLOW_OSO, bias=bd, act=("leaky_relu", 0.1))
+    assert torch.equal(out, again)
+    # column slices in and out, as the skip connections use them
+    wide_in = torch.full((n, c_in + 12), 7.0, dtype=torch.float32, device=DEV)
+    wide_in[:, 4:4 + c_in] = fd
+    wide_out = torch.full((n, c_out + 16), -3.0, dtype=torch.float32, device=DEV)
+    got = backend.conv_forward(wide_in[:, 4:4 + c_in], wd, km, DATAFLOW_OSO, out=wide_out[:, 8:8 + c_out], bias=bd, act=("leaky_relu", 0.1))
+    assert torch.equal(got, out) and bool((wide_out[:, :8] == -3.0).all()) and bool((wide_out[:, 8 + c_out:] == -3.0).all())
+
+
 def test_ordered_dataflow_on_column_slices_and_the_selector():
     coords = CLOUDS["lidar"]()
     km = _subm(coords)
@@ -121,7 +154,8 @@ def test_ordered_dataflow_on_column_slices_and_the_selector():
     got = backend.conv_forward(wide_in[:, 8:8 + c], w, km, DATAFLOW_OSO, packed=packed, out=wide_out[:, c:2 * c])
     assert torch.equal(got, want) and bool((wide_out[:, :c] == -2.0).all()) and bool((wide_out[:, 2 * c:] == -2.0).all())
     assert backend.select_dataflow(km, c, c, torch.float16) == DATAFLOW_OSO
-    assert backend.select_dataflow(km, c, c, torch.float32) != DATAFLOW_OSO
+    assert backend.select_dataflow(km, c, c, torch.float32) == DATAFLOW_OSO        # the fp32 form takes up to 32 channels
+    assert backend.select_dataflow(km, 64, 64, torch.float32) != DATAFLOW_OSO
     assert backend.select_dataflow(km, 96, 96, torch.float16) != DATAFLOW_OSO
     # the two pair-proportional dataflows agree to fp16 rounding (they round partial sums at different places)
     fds = backend.conv_forward(f, w, km, DATAFLOW_FDS, packed=packed)
@@ -142,7 +176,8 @@ def test_ordered_dataflow_argument_errors():
         f.data_ptr(), w.data_ptr(), packed.data_ptr() if packed is not None else None, out.data_ptr(), dtype, n, n, c_in, c_out, 27, mid,
         km.nbr_out.data_ptr(), km.order.data_ptr(), heavy, None, s)
     assert call(_lib.PCE_F16, 32, 32, 13, km.order_heavy) == _lib.PCE_OK
-    assert call(_lib.PCE_F32, 32, 32, 13, km.order_heavy) == _lib.PCE_EINVAL
+    assert call(_lib.PCE_F32, 64, 32, 13, km.order_heavy) == _lib.PCE_EINVAL        # fp32 stops at 32 channels
+    assert call(_lib.PCE_F32, 12, 32, 13, km.order_heavy) == _lib.PCE_EINVAL        # ... in multiples of 8
     assert call(_lib.PCE_F16, 32, 32, -1, km.order_heavy) == _lib.PCE_EINVAL        # no centre offset
     assert call(_lib.PCE_F16, 32, 32, 13, n + 1) == _lib.PCE_EINVAL
     assert call(_lib.PCE_F16, 32, 32, 13, km.order_heavy, None) == _lib.PCE_EINVAL    # weights not packed

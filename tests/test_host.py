@@ -104,8 +104,9 @@ def test_selector_on_measured_layers():
     ]
     for n_in, n_out, pairs, ci, co, kv, want in cases:
         assert lib.pce_select_dataflow(n_in, n_out, pairs, ci, co, kv, _lib.PCE_F16) == want, (n_in, n_out, ci, co, kv)
-    # fp32 and strided layers never take the ordered dataflow
-    assert lib.pce_select_dataflow(20804, 20804, 98238, 16, 16, 27, _lib.PCE_F32) == FDS
+    # fp32: the ordered dataflow up to 32 channels (configuration 1), deferred scatter beyond; strided layers never take it
+    assert lib.pce_select_dataflow(20804, 20804, 98238, 16, 16, 27, _lib.PCE_F32) == OSO
+    assert lib.pce_select_dataflow(20804, 20804, 98238, 64, 64, 27, _lib.PCE_F32) == FDS
     assert lib.pce_select_dataflow(149866, 146018, 149866, 32, 32, 8, _lib.PCE_F16) != OSO
 
 
