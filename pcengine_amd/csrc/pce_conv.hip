@@ -3613,9 +3613,11 @@ extern "C" int pce_select_dataflow(int64_t n_in, int64_t n_out, int64_t n_pairs,
   // scatter with bias, residual and ReLU fused: 0.78-0.93 of its time at 0.1-0.2 pairs per row (100-150 k voxels,
   // 16-64 channels), 0.62-0.83 at 0.8, 0.64-0.83 at 3, 0.60-0.62 at 5.3 (541 k voxels, where it equals plain
   // output-stationary); beyond that the dense output-stationary tiles below take over.
+  // the fp32 form is bound by its MFMAs (v_mfma_f32_32x32x2_f32, c_in / 2 of them per offset and wavefront): measured
+  // against deferred scatter at 4.7 pairs per row 0.76 (8 channels), 0.87 (16), 1.15 (32); at 0.2 pairs per row 0.49, 0.62, 0.82
   if (dtype == PCE_F32 && n_in == n_out && kv >= 3 && kv <= 31 && (kv & 1) && c_in % 8 == 0 && c_in <= 32 && c_out % 8 == 0 &&
-      c_out <= 32 && rho <= 6.0)
-    return PCE_DATAFLOW_OSO;   // the fp32 form: 20 804 rows, 16 -> 16 channels, 4.7 pairs per row against deferred scatter
+      c_out <= 32 && rho <= (c_in <= 16 ? 6.0 : 2.0))
+    return PCE_DATAFLOW_OSO;
   if (dtype == PCE_F16 && n_in == n_out && kv >= 3 && kv <= 31 && (kv & 1) && c_in % 16 == 0 && c_in <= 64 && c_out % 8 == 0 &&
       c_out <= 64 && rho <= 6.0)
     return PCE_DATAFLOW_OSO;

@@ -154,7 +154,7 @@ def test_ordered_dataflow_on_column_slices_and_the_selector():
     got = backend.conv_forward(wide_in[:, 8:8 + c], w, km, DATAFLOW_OSO, packed=packed, out=wide_out[:, c:2 * c])
     assert torch.equal(got, want) and bool((wide_out[:, :c] == -2.0).all()) and bool((wide_out[:, 2 * c:] == -2.0).all())
     assert backend.select_dataflow(km, c, c, torch.float16) == DATAFLOW_OSO
-    assert backend.select_dataflow(km, c, c, torch.float32) == DATAFLOW_OSO        # the fp32 form takes up to 32 channels
+    assert backend.select_dataflow(km, 16, 16, torch.float32) == DATAFLOW_OSO      # the fp32 form: up to 32 channels, by density
     assert backend.select_dataflow(km, 64, 64, torch.float32) != DATAFLOW_OSO
     assert backend.select_dataflow(km, 96, 96, torch.float16) != DATAFLOW_OSO
     # the two pair-proportional dataflows agree to fp16 rounding (they round partial sums at different places)

@@ -107,6 +107,8 @@ def test_selector_on_measured_layers():
     # fp32: the ordered dataflow up to 32 channels (configuration 1), deferred scatter beyond; strided layers never take it
     assert lib.pce_select_dataflow(20804, 20804, 98238, 16, 16, 27, _lib.PCE_F32) == OSO
     assert lib.pce_select_dataflow(20804, 20804, 98238, 64, 64, 27, _lib.PCE_F32) == FDS
+    assert lib.pce_select_dataflow(20804, 20804, 98238, 32, 32, 27, _lib.PCE_F32) == FDS      # 32 channels: only on sparse clouds
+    assert lib.pce_select_dataflow(149866, 149866, 30620, 32, 32, 27, _lib.PCE_F32) == OSO
     assert lib.pce_select_dataflow(149866, 146018, 149866, 32, 32, 8, _lib.PCE_F16) != OSO
 
 
