@@ -354,11 +354,20 @@ __device__ __forceinline__ void gather_row_pieces(const f32x16 (&acc)[NB], float
       const int qa = 2 * h, qb = 2 * h + 1;  // lane g=0 keeps piece qa, lane g=1 keeps piece qb
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        // one instruction swaps the upper half of `lo` with the lower half of `hi`: lanes 0-31 then hold (own lo,
-        // partner's lo), lanes 32-63 (partner's hi, own hi)
-        auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc[nb][4 * qa + i]), __float_as_uint(acc[nb][4 * qb + i]), false, false);
-        V[nb][h][i] = __uint_as_float(r[0]);
-        V[nb][h][4 + i] = __uint_as_float(r[1]);
+        if (NB > 2) {
+          // wide tiles: a shuffle and two selects (the swap below costs the kernels that hold 64 accumulators per lane
+          // a tenth of a network forward)
+          float lo = acc[nb][4 * qa + i], hi = acc[nb][4 * qb + i];
+          float recv = __shfl_xor(g == 0 ? hi : lo, 32, PCE_WAVE);
+          V[nb][h][i] = g == 0 ? lo : recv;
+          V[nb][h][4 + i] = g == 0 ? recv : hi;
+        } else {
+          // one instruction swaps the upper half of `lo` with the lower half of `hi`: lanes 0-31 then hold (own lo,
+          // partner's lo), lanes 32-63 (partner's hi, own hi)
+          auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc[nb][4 * qa + i]), __float_as_uint(acc[nb][4 * qb + i]), false, false);
+          V[nb][h][i] = __uint_as_float(r[0]);
+          V[nb][h][4 + i] = __uint_as_float(r[1]);
+        }
       }
     }
   }
