@@ -58,7 +58,7 @@ enum {
   PCE_DATAFLOW_FDS = 3, /* fetch-on-demand with deferred scatter: pair tiles write partial rows to a
                            staging buffer, the centre GEMM's epilogue sums them per output row */
   PCE_DATAFLOW_OSO = 4  /* output-stationary over rows ordered by their neighbour pattern (pce_row_order):
-                           narrow fp16 submanifold layers on sparse clouds, one launch, no partial rows */
+                           narrow submanifold layers (fp16 up to 64 channels, fp32 up to 32), one launch, no partial rows */
 };
 
 #define PCE_QUANTUM 128        /* rows per tile of the pair list; qkpos granularity (backend/hash.cu:203-205) */
@@ -365,7 +365,7 @@ int pce_conv_fwd_os(const void *in_feats, const void *weight, const void *weight
                     int64_t n_in, int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv,
                     const int32_t *nbr_dev, const pce_epilogue_t *epilogue, pce_stream_t stream);
 
-/* Output-stationary over ordered rows, for narrow fp16 submanifold layers on clouds where most voxels have few
+/* Output-stationary over ordered rows, for narrow submanifold layers on clouds where most voxels have few
  * neighbours (surfaces: 0.2 pairs per voxel on a 64 x 2048 LiDAR scan at 0.1 m).  pce_row_order derives from the
  * output-major neighbour table, once per map, the order in which the rows are visited -- rows without neighbours
  * first, in their own order, then the rows with one or two neighbours sorted by the offsets they have them at, then
