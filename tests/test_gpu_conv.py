@@ -204,6 +204,10 @@ def test_config1_fp32_c16():
     for flow in FLOWS:
         out = backend.conv_forward(fd, wd, km, flow)
         assert orc.rel_l2(out.double().cpu().numpy(), want) <= 1e-5, flow
+    # the selector's choice for this layer: the ordered dataflow in its fp32 form
+    assert backend.select_dataflow(km, 16, 16, torch.float32) == backend.DATAFLOW_OSO
+    out = backend.conv_forward(fd, wd, km, backend.DATAFLOW_OSO)
+    assert orc.rel_l2(out.double().cpu().numpy(), want) <= 1e-5
 
 
 def test_config2_fp16_c64_full_size():
