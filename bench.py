@@ -178,10 +178,11 @@ def main() -> int:
     # ---- kernel map (built once, reused by every step; timed separately) -----------------------
     n_batch = int(coords[:, 0].max()) + 1
 
-    def build_ms(batchsize):
+    def build_ms(batchsize, want_csr=True):
         """Wall time of one map build (CSR views and neighbour table included).  With the batch count stated the
-        sorted coordinates are indexed by column (what the front end does); without it they go through the hash table."""
-        build = lambda: backend.build_kernel_map(cd, ks, (1, 1, 1), (0, 0, 0), [0, 0, 0], cmax, True, want_csr=True,
+        sorted coordinates are indexed by column (what the front end does); without it they go through the hash table.
+        want_csr=False: the neighbour table, the counts and the row order only (what the output-stationary dataflows read)."""
+        build = lambda: backend.build_kernel_map(cd, ks, (1, 1, 1), (0, 0, 0), [0, 0, 0], cmax, True, want_csr=want_csr,
                                                  batchsize=batchsize)
         km = build()
         for _ in range(3):
@@ -194,6 +195,7 @@ def main() -> int:
         return km, (time.perf_counter() - t0) / 20 * 1e3
     km_hash, map_hash_ms = build_ms(0)
     km, map_ms = build_ms(n_batch)
+    _, map_table_only_ms = build_ms(n_batch, want_csr=False)
     if not (torch.equal(km.imap, km_hash.imap) and torch.equal(km.omap, km_hash.omap) and torch.equal(km.ocsr, km_hash.ocsr)):
         raise RuntimeError("the column-grid map and the hash-table map differ")
     del km_hash
@@ -342,6 +344,7 @@ def main() -> int:
         "extra": {"ms_per_step_replays": {k: (round(v, 5) if k != "replays" else v) for k, v in spread.items()},
                   "eager_ms_per_step": round(eager_ms, 5), "eager_wall_ms_per_step": round(wall_ms, 5),
                   "map_build_ms": round(map_ms, 4), "map_build_hash_table_ms": round(map_hash_ms, 4),
+                  "map_build_neighbour_table_and_order_only_ms": round(map_table_only_ms, 4),
                   "stage_ms": {k: round(v, 5) for k, v in stages.items()},
                   "other_dataflows_ms": {k: round(v, 5) for k, v in others.items()},
                   "floors": {**{k: round(v, 5) for k, v in floors.items()},
