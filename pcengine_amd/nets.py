@@ -98,6 +98,7 @@ class SparseResUNet(nn.Module):
         for m in self.modules():
             if isinstance(m, ConvBN):
                 m.fuse()
+        self._in_place_ok = None
         return self
 
     def map_plan(self):
@@ -127,11 +128,16 @@ class SparseResUNet(nn.Module):
         a skip connection can then write their halves of the concatenated matrix themselves."""
         if torch.is_grad_enabled() and any(p.requires_grad for p in self.parameters()):
             return False
-        if not x.feats.is_cuda or any(isinstance(m, ConvBN) and m.bn is not None for m in self.modules()):
+        if not x.feats.is_cuda:
             return False
-        widths = [self.stem[1].conv.out_channels] + [e[1].b.conv.out_channels for e in self.enc] + \
-                 [u.conv.out_channels for u in self.up]
-        return all(w % 8 == 0 for w in widths)
+        ok = getattr(self, "_in_place_ok", None)
+        if ok is None:      # what depends on the modules alone: looked up once, again after fuse_bn()
+            widths = [self.stem[1].conv.out_channels] + [e[1].b.conv.out_channels for e in self.enc] + \
+                     [u.conv.out_channels for u in self.up]
+            ok = all(w % 8 == 0 for w in widths) and \
+                not any(isinstance(m, ConvBN) and m.bn is not None for m in self.modules())
+            self._in_place_ok = ok
+        return ok
 
     def _forward_skips_in_place(self, x: spTensor) -> spTensor:
         """The same network with the concatenation of each decoder stage done by its producers: the encoder layer
