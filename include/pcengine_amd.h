@@ -58,7 +58,8 @@ enum {
   PCE_DATAFLOW_FDS = 3, /* fetch-on-demand with deferred scatter: pair tiles write partial rows to a
                            staging buffer, the centre GEMM's epilogue sums them per output row */
   PCE_DATAFLOW_OSO = 4  /* output-stationary over rows ordered by their neighbour pattern (pce_row_order):
-                           narrow submanifold layers (fp16 up to 64 channels, fp32 up to 32), one launch, no partial rows */
+                           narrow layers (fp16 up to 64 channels, submanifold or stride 2; fp32 submanifold up to 32),
+                           one launch, no partial rows */
 };
 
 #define PCE_QUANTUM 128        /* rows per tile of the pair list; qkpos granularity (backend/hash.cu:203-205) */
@@ -365,7 +366,7 @@ int pce_conv_fwd_os(const void *in_feats, const void *weight, const void *weight
                     int64_t n_in, int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv,
                     const int32_t *nbr_dev, const pce_epilogue_t *epilogue, pce_stream_t stream);
 
-/* Output-stationary over ordered rows, for narrow submanifold layers on clouds where most voxels have few
+/* Output-stationary over ordered rows, for narrow layers on clouds where most voxels have few
  * neighbours (surfaces: 0.2 pairs per voxel on a 64 x 2048 LiDAR scan at 0.1 m).  pce_row_order derives from the
  * output-major neighbour table, once per map, the order in which the rows are visited -- rows without neighbours
  * first, in their own order, then the rows with one or two neighbours sorted by the offsets they have them at, then
@@ -377,7 +378,10 @@ int pce_conv_fwd_os(const void *in_feats, const void *weight, const void *weight
  * that have it, and stores each finished row once (epilogue fused); the rows of the last part, whose offsets are
  * many, go 32 to a workgroup whose four wavefronts share the offsets.  PCE_F16: c_in a multiple of 16 and at most
  * 64, c_out a multiple of 8 and at most 64, packed weights; PCE_F32: c_in and c_out multiples of 8 and at most 32
- * (weight_packed is not read); mid >= 0; PCE_EINVAL otherwise.  Takes the row strides
+ * (weight_packed is not read) and mid >= 0; PCE_EINVAL otherwise.  In PCE_F16 a layer without a centre offset
+ * (mid = -1: a strided layer, n_in != n_out, nbr_dev = its output-major table [kv][n_out], order from pce_row_order
+ * with mid = -1) runs the same way from zero sums: every output row of a 2x2x2 stride-2 layer has one to eight pairs,
+ * the order groups the rows by where they have them.  Takes the row strides
  * of pce_epilogue_t.  No counterpart in the reference: it computes what the fetch-on-demand kernels compute
  * (backend/spconv.cuh:1567-1730) with the scatter-add replaced by register accumulation, as pce_conv_fwd_os. */
 int64_t pce_row_order_elems(int64_t n_rows);

@@ -286,10 +286,11 @@ class _MapJob:
         self.in_coords, self.out_coords, self.geom = in_coords, out_coords, geom
         self.n_in, self.n_out, self.kv, self.want_csr, self.dev = n_in, n_out, kv, bool(want_csr), dev
         self.meta_len = kv + 2 * (kv + 1) + 8      # knnz | kpos | qkpos | status (4 words, then the heavy rows of the order)
-        # the row order of the ordered output-stationary dataflow comes with every submanifold map that has the
-        # output-major table it is derived from (three launches per batch of maps, 2 n + 8192 ints)
+        # the row order of the ordered output-stationary dataflow comes with every submanifold map, and every strided
+        # map of at most 8 offsets (the layers the selector gives to that dataflow), that has the output-major table
+        # it is derived from (three launches per batch of maps, 2 n + 8192 ints)
         if want_order is None:
-            want_order = subm and want_nbr_out
+            want_order = (subm or kv <= 8) and want_nbr_out
         self.want_order = bool(want_order) and want_nbr_out and kv <= 31
         # the batch count lets the library index sorted coordinates by column instead of hashing them; a build that
         # finds them unsorted, or outside the box the geometry states, is redone through the hash table (finish)
@@ -483,7 +484,8 @@ def pair_route(km: KernelMap, transposed: bool = False) -> torch.Tensor:
 
 def row_order(km: KernelMap) -> torch.Tensor:
     """Row order of the ordered output-stationary dataflow (``pce_row_order``), cached on the map: the output rows
-    of a submanifold layer with rows without neighbours first and the others sorted by the offsets they have."""
+    with rows without neighbours first (a submanifold layer has those; the centre offset does not count) and the
+    others sorted by the offsets they have."""
     if km.order is None:
         ensure_nbr(km, False)
         lib = _lib.load()
@@ -498,10 +500,10 @@ def row_order(km: KernelMap) -> torch.Tensor:
 
 def oso_takes(km: KernelMap, c_in: int, c_out: int, dtype: torch.dtype, transposed: bool = False) -> bool:
     """Shapes the ordered output-stationary dataflow exists for."""
-    if not km.subm or transposed or km.kv > 31:
+    if transposed or km.kv > 31:
         return False
     if dtype == torch.float32:
-        return c_in % 8 == 0 and c_in <= 32 and c_out % 8 == 0 and c_out <= 32
+        return km.subm and c_in % 8 == 0 and c_in <= 32 and c_out % 8 == 0 and c_out <= 32
     return dtype == torch.float16 and c_in % 16 == 0 and c_in <= 64 and c_out % 8 == 0 and c_out <= 64
 
 
@@ -521,7 +523,7 @@ def select_dataflow(km: KernelMap, c_in: int, c_out: int, dtype: torch.dtype, tr
     n_in = km.n_out if transposed else km.n_in
     df = lib.pce_select_dataflow(n_in, n_out, km.M, c_in, c_out, km.kv, PCE_F16 if dtype == torch.float16 else PCE_F32)
     if df == DATAFLOW_OSO and not oso_takes(km, c_in, c_out, dtype, transposed):
-        df = DATAFLOW_FDS       # equal row counts and an odd kernel volume, but not a plain submanifold layer
+        df = DATAFLOW_FDS       # the row counts of such a layer, but transposed, or with an even kernel size at stride 1
     return df
 
 
@@ -704,8 +706,9 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
                                         km.kpos.data_ptr(), km.qkpos.data_ptr(), km.qsum, buffer.data_ptr(), buffer.numel(), epi, s))
     elif dataflow == DATAFLOW_OSO:
         if not oso_takes(km, c_in, c_out, feats.dtype, transposed):
-            raise ValueError("the ordered output-stationary dataflow takes submanifold layers in fp16 of at most 64 channels "
-                             "(c_in a multiple of 16, c_out of 8) or in fp32 of at most 32 (multiples of 8)")
+            raise ValueError("the ordered output-stationary dataflow takes layers (not transposed, at most 31 offsets) in fp16 "
+                             "of at most 64 channels (c_in a multiple of 16, c_out of 8) or submanifold layers in fp32 of at "
+                             "most 32 (multiples of 8)")
         if packed is None:
             packed = pack_weights(weight)      # None for fp32: that form reads the weights as they are
         order = row_order(km)

@@ -2423,6 +2423,8 @@ extern "C" int pce_conv_fwd_os(const void *in, const void *w, const void *wp, vo
 // wavefronts share the offsets of the chunk's union among them (wavefront 0 also does the centre product) and add
 // their accumulators through LDS at the end.  The other workgroups take four chunks of the remaining rows, one per
 // wavefront, last chunks first (the rows with one or two neighbours are the last of that part).
+// A strided layer (mid < 0) has no centre term: every output row has one to kv pairs, the same order groups the rows
+// by the offsets of their pairs, and the kernel starts from zero sums.
 template <int NB, int KS>
 __global__ void __launch_bounds__(256, 4) wave_os_kernel(TileArgs a, const int *__restrict__ perm,
                                                          const unsigned *__restrict__ rmask, int mid, long long n_main,
@@ -2438,8 +2440,9 @@ __global__ void __launch_bounds__(256, 4) wave_os_kernel(TileArgs a, const int *
   const int l32 = lane & 31, g = lane >> 5;
   const half_t *Wp = (const half_t *)a.Wp;
   const long long wstep = (long long)a.k8_total * a.n_pad * 8;
-  // every wavefront copies its share of the centre weights (one copy of them per workgroup instead of one per wavefront)
-  {
+  // every wavefront copies its share of the centre weights (one copy of them per workgroup instead of one per wavefront);
+  // a layer without a centre offset (mid < 0: strided) has no such term and starts from zero sums
+  if (mid >= 0) {
     constexpr int FR = KS * 2 * NB * 32;   // fragments: [k8][column]
 #pragma unroll
     for (int i = 0; i < (FR + 255) / 256; ++i) {
@@ -2479,7 +2482,7 @@ __global__ void __launch_bounds__(256, 4) wave_os_kernel(TileArgs a, const int *
   // offset alone: the sums of a row are then grouped the same way whichever rows share its chunk, and the result
   // of a layer does not depend on where the counting sort happened to put a row among those of its key.)
   if (heavy) todo &= 0x11111111u << wave;
-  const bool centre = !heavy || wave == 0;
+  const bool centre = mid >= 0 && (!heavy || wave == 0);
   half8 wf[KS][NB];
   if (centre) {
     // centre rows -> LDS, in line order (a valid row stands in for one past the end)
@@ -2673,7 +2676,7 @@ static bool wave_os_f32_ok(const TileArgs &a, int kv, int mid) {
 
 // shapes the ordered-row kernel takes: fp16, at most 64 channels either side, a centre offset
 static bool wave_os_ok(const TileArgs &a, int kv, int mid) {
-  return wave_gemm_ok(a, 2) && kv < ORDER_MAX_KV && mid >= 0 && mid < kv && aligned16(a.bias) && aligned16(a.res);
+  return wave_gemm_ok(a, 2) && kv < ORDER_MAX_KV && mid < kv && aligned16(a.bias) && aligned16(a.res);
 }
 
 extern "C" int pce_conv_fwd_oso(const void *in, const void *w, const void *wp, void *out, int32_t dtype, int64_t n_in,
@@ -2692,9 +2695,9 @@ extern "C" int pce_conv_fwd_oso(const void *in, const void *w, const void *wp, v
     set_out<half_t>(&a, out, false, n_out, e.ldo);
   set_epi(&a, e);
   if (f32 ? !wave_os_f32_ok(a, kv, mid) : !wave_os_ok(a, kv, mid))
-    PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: takes submanifold layers in fp16 of at most 64 channels (multiples of 16 in, 8 out, packed "
-                         "weights) or in fp32 of at most 32 (multiples of 8), 16-byte aligned rows; got dtype %d, %d -> %d "
-                         "channels, kv %d, mid %d", (int)dtype, (int)c_in, (int)c_out, (int)kv, (int)mid);
+    PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: takes layers in fp16 of at most 64 channels (multiples of 16 in, 8 out, packed "
+                         "weights) or submanifold layers in fp32 of at most 32 (multiples of 8), 16-byte aligned rows, kernel "
+                         "volumes up to 31; got dtype %d, %d -> %d channels, kv %d, mid %d", (int)dtype, (int)c_in, (int)c_out, (int)kv, (int)mid);
   if (n_heavy < 0 || n_heavy > n_out) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: n_heavy=%lld outside [0, n_out]", (long long)n_heavy);
   a.nbr = nbr;
   a.n_rows = n_out;
@@ -3629,6 +3632,12 @@ extern "C" int pce_select_dataflow(int64_t n_in, int64_t n_out, int64_t n_pairs,
     return PCE_DATAFLOW_OSO;
   if (dtype == PCE_F16 && n_in == n_out && kv >= 3 && kv <= 31 && (kv & 1) && c_in % 16 == 0 && c_in <= 64 && c_out % 8 == 0 &&
       c_out <= 64 && rho <= 6.0)
+    return PCE_DATAFLOW_OSO;
+  // narrow fp16 stride-2 layers (every input row in exactly one pair, 1-8 per output row), through the same ordered
+  // rows without a centre term: 0.58-0.66 of the output-stationary tiles' time at 1.0-1.4 pairs per row (66-146 k
+  // output rows, 32 and 64 channels; 680 k rows: 0.71), 0.57 at 2.4 on 27 k rows and 1.05 at 2.5 on 276 k rows of
+  // indoor scenes, where half the rows have three pairs or more
+  if (dtype == PCE_F16 && kv <= 8 && n_out < n_in && c_in % 16 == 0 && c_in <= 64 && c_out % 8 == 0 && c_out <= 64 && rho <= 2.0)
     return PCE_DATAFLOW_OSO;
   if (kv <= 8 && n_out <= n_in && rho >= 1.0 && prod <= 64 * 64 && dtype == PCE_F16) return PCE_DATAFLOW_OS;
   if (kv <= 8 && n_out <= n_in && rho >= 2.0 && prod <= 128 * 128 && dtype == PCE_F16) return PCE_DATAFLOW_OS;

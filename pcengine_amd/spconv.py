@@ -141,7 +141,7 @@ def _pick_dataflow(km: backend.KernelMap, requested: str, c_in: int, c_out: int,
     forced = _DATAFLOWS.get(env, _DATAFLOWS.get(requested))
     if forced is not None:
         if forced == DATAFLOW_OSO and not backend.oso_takes(km, c_in, c_out, dtype, transposed):
-            return DATAFLOW_FDS     # the ordered dataflow exists for narrow submanifold layers only (backend.oso_takes)
+            return DATAFLOW_FDS     # the ordered dataflow exists for narrow layers only (backend.oso_takes)
         return forced
     if km.tag == "D1":
         return DATAFLOW_GMS

@@ -140,6 +140,107 @@ def test_ordered_dataflow_fp32_against_the_oracle(cloud, c_in, c_out):
     assert torch.equal(got, out) and bool((wide_out[:, :8] == -3.0).all()) and bool((wide_out[:, 8 + c_out:] == -3.0).all())
 
 
+STRIDED = [((2, 2, 2), (2, 2, 2), (0, 0, 0)), ((3, 3, 3), (2, 2, 2), (1, 1, 1)), ((2, 3, 1), (2, 1, 1), (0, 1, 0))]
+_strided_refs = {}
+
+
+def _strided_ref(cloud, geom):
+    """(coordinates, oracle map, offset mask of every output row) of a strided layer on a cloud, computed once."""
+    if (cloud, geom) not in _strided_refs:
+        coords = CLOUDS[cloud]()
+        ks, stride, pad = STRIDED[geom]
+        ref = orc.kernel_map(coords, ks, stride, pad)
+        masks = np.zeros(len(ref.out_coords), np.int64)
+        for kp in range(orc.kernel_volume(ks)):
+            masks[ref.omap[ref.kpos[kp]:ref.kpos[kp + 1]]] |= 1 << kp
+        _strided_refs[(cloud, geom)] = (coords, ref, masks)
+    return _strided_refs[(cloud, geom)]
+
+
+def _strided_map(coords, geom, **kw):
+    ks, stride, pad = STRIDED[geom]
+    cmax_out = orc.strided_coords_max(coords[:, 1:].max(0).tolist(), ks, stride, pad)
+    return backend.build_kernel_map(dev_coords(coords), ks, stride, pad, [0, 0, 0], cmax_out, False, want_csr=True,
+                                    batchsize=int(coords[:, 0].max()) + 1, **kw)
+
+
+@pytest.mark.parametrize("cloud", sorted(CLOUDS))
+@pytest.mark.parametrize("geom", range(len(STRIDED)))
+def test_row_order_of_strided_maps(cloud, geom):
+    """A strided layer has no centre offset: every output row has a pair, the masks cover all offsets, the sections
+    are (one or two pairs, sorted by key) and (three or more, likewise).  Maps of at most 8 offsets come with their
+    order; others get it on first use."""
+    coords, ref, masks = _strided_ref(cloud, geom)
+    km = _strided_map(coords, geom)
+    n = km.n_out
+    assert n == len(ref.out_coords) and (masks != 0).all()
+    assert (km.order is not None) == (km.kv <= 8)
+    backend.row_order(km)
+    order = km.order.cpu().numpy()
+    perm, got_masks = order[:n].astype(np.int64), order[n:2 * n].view(np.uint32).astype(np.int64)
+    assert np.array_equal(got_masks, masks)
+    assert np.array_equal(np.sort(perm), np.arange(n))
+    pc = _popcount(masks)
+    n_heavy = int((pc >= 3).sum())
+    assert km.order_heavy == n_heavy
+    sect = masks[perm]
+    assert (_popcount(sect[:n - n_heavy]) <= 2).all() and (_popcount(sect[n - n_heavy:]) >= 3).all()
+    assert (np.diff(np.array([_key(v) for v in sect])) >= 0).all()
+
+
+@pytest.mark.parametrize("cloud", sorted(CLOUDS))
+@pytest.mark.parametrize("geom", range(len(STRIDED)))
+@pytest.mark.parametrize("c_in,c_out", [(32, 32), (64, 64), (16, 64), (48, 24)])
+def test_ordered_dataflow_strided_against_the_oracle(cloud, geom, c_in, c_out):
+    """The ordered rows without a centre term (strided layers, fp16): the float64 oracle within 1e-3, epilogue fused,
+    bit-equal from run to run, column slices on both sides."""
+    coords, ref, _ = _strided_ref(cloud, geom)
+    ks = STRIDED[geom][0]
+    kv = orc.kernel_volume(ks)
+    km = _strided_map(coords, geom)
+    n_in, n_out = len(coords), km.n_out
+    dt = torch.float16
+    f, w = synth.features(c_in + geom, n_in, c_in), synth.weights(c_out, kv, c_in, c_out)
+    bias = np.random.default_rng(c_in).standard_normal(c_out) * 0.1
+    res = synth.features(c_out + 1, n_out, c_out)
+    fd, wd = torch.as_tensor(f, device=DEV).to(dt), torch.as_tensor(w, device=DEV).to(dt)
+    bd, rd = torch.as_tensor(bias, device=DEV).to(dt), torch.as_tensor(res, device=DEV).to(dt)
+    packed = backend.pack_weights(wd)
+    assert backend.oso_takes(km, c_in, c_out, dt) and not backend.oso_takes(km, c_in, c_out, dt, transposed=True)
+    plain = orc.conv_forward(rounded(f, dt), rounded(w, dt), ref, ks)
+    out = backend.conv_forward(fd, wd, km, DATAFLOW_OSO, packed=packed)
+    assert out.shape == (n_out, c_out)
+    assert orc.rel_l2(out.double().cpu().numpy(), plain) <= 1e-3
+    want = np.maximum(plain + rounded(bias, dt) + rounded(res, dt), 0)
+    out = backend.conv_forward(fd, wd, km, DATAFLOW_OSO, packed=packed, bias=bd, residual=rd, act="relu")
+    assert orc.rel_l2(out.double().cpu().numpy(), want) <= 1e-3
+    again = backend.conv_forward(fd, wd, _strided_map(coords, geom), DATAFLOW_OSO, packed=packed, bias=bd, residual=rd, act="relu")
+    assert torch.equal(out, again)
+    wide_in = torch.full((n_in, c_in + 24), 5.0, dtype=dt, device=DEV)
+    wide_in[:, 8:8 + c_in] = fd
+    wide_out = torch.full((n_out, c_out + 16), -2.0, dtype=dt, device=DEV)
+    got = backend.conv_forward(wide_in[:, 8:8 + c_in], wd, km, DATAFLOW_OSO, packed=packed, out=wide_out[:, 8:8 + c_out], bias=bd,
+                               residual=rd, act="relu")
+    assert torch.equal(got, out) and bool((wide_out[:, :8] == -2.0).all()) and bool((wide_out[:, 8 + c_out:] == -2.0).all())
+    # the transposed layer has no ordered form: a request for it falls back to deferred scatter in the front end,
+    # and the backend refuses it
+    with pytest.raises(ValueError):
+        backend.conv_forward(out, torch.zeros((kv, c_out, c_in), dtype=dt, device=DEV), km, DATAFLOW_OSO, transposed=True)
+
+
+def test_selector_gives_narrow_stride_2_layers_to_the_ordered_rows():
+    coords = CLOUDS["lidar"]()
+    km = _strided_map(coords, 0)
+    assert km.M / km.n_out <= 2.0
+    assert backend.select_dataflow(km, 32, 32, torch.float16) == DATAFLOW_OSO
+    assert backend.select_dataflow(km, 64, 64, torch.float16) == DATAFLOW_OSO
+    assert backend.select_dataflow(km, 64, 128, torch.float16) != DATAFLOW_OSO
+    assert backend.select_dataflow(km, 32, 32, torch.float32) != DATAFLOW_OSO
+    assert backend.select_dataflow(km, 32, 32, torch.float16, transposed=True) != DATAFLOW_OSO
+    dense = _strided_map(CLOUDS["dense"](), 0)          # a filled box: close to eight pairs per output row
+    assert dense.M / dense.n_out > 2.0 and backend.select_dataflow(dense, 32, 32, torch.float16) == DATAFLOW_OS
+
+
 def test_ordered_dataflow_on_column_slices_and_the_selector():
     coords = CLOUDS["lidar"]()
     km = _subm(coords)
@@ -178,7 +279,7 @@ def test_ordered_dataflow_argument_errors():
     assert call(_lib.PCE_F16, 32, 32, 13, km.order_heavy) == _lib.PCE_OK
     assert call(_lib.PCE_F32, 64, 32, 13, km.order_heavy) == _lib.PCE_EINVAL        # fp32 stops at 32 channels
     assert call(_lib.PCE_F32, 12, 32, 13, km.order_heavy) == _lib.PCE_EINVAL        # ... in multiples of 8
-    assert call(_lib.PCE_F16, 32, 32, -1, km.order_heavy) == _lib.PCE_EINVAL        # no centre offset
+    assert call(_lib.PCE_F32, 32, 32, -1, km.order_heavy) == _lib.PCE_EINVAL        # fp32 needs a centre offset
     assert call(_lib.PCE_F16, 32, 32, 13, n + 1) == _lib.PCE_EINVAL
     assert call(_lib.PCE_F16, 32, 32, 13, km.order_heavy, None) == _lib.PCE_EINVAL    # weights not packed
     assert call(_lib.PCE_F16, 128, 32, 13, km.order_heavy) == _lib.PCE_EINVAL

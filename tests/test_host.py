@@ -104,12 +104,19 @@ def test_selector_on_measured_layers():
     ]
     for n_in, n_out, pairs, ci, co, kv, want in cases:
         assert lib.pce_select_dataflow(n_in, n_out, pairs, ci, co, kv, _lib.PCE_F16) == want, (n_in, n_out, ci, co, kv)
-    # fp32: the ordered dataflow up to 32 channels (configuration 1), deferred scatter beyond; strided layers never take it
+    # fp32: the ordered dataflow up to 32 channels (configuration 1), deferred scatter beyond
     assert lib.pce_select_dataflow(20804, 20804, 98238, 16, 16, 27, _lib.PCE_F32) == OSO
     assert lib.pce_select_dataflow(20804, 20804, 98238, 64, 64, 27, _lib.PCE_F32) == FDS
     assert lib.pce_select_dataflow(20804, 20804, 98238, 32, 32, 27, _lib.PCE_F32) == FDS      # 32 channels: only on sparse clouds
     assert lib.pce_select_dataflow(149866, 149866, 30620, 32, 32, 27, _lib.PCE_F32) == OSO
-    assert lib.pce_select_dataflow(149866, 146018, 149866, 32, 32, 8, _lib.PCE_F16) != OSO
+    # narrow 2x2x2 stride-2 layers in fp16: the ordered rows up to two pairs per output row, the dense tiles beyond;
+    # never in fp32, never for the transposed layer (more output rows than input rows)
+    assert lib.pce_select_dataflow(149866, 146018, 149866, 32, 32, 8, _lib.PCE_F16) == OSO
+    assert lib.pce_select_dataflow(99692, 97941, 99692, 32, 32, 8, _lib.PCE_F16) == OSO
+    assert lib.pce_select_dataflow(89469, 65807, 89469, 64, 64, 8, _lib.PCE_F16) == OSO       # 1.36 pairs per row
+    assert lib.pce_select_dataflow(679728, 276205, 679728, 64, 64, 8, _lib.PCE_F16) == OS     # 2.46 on an indoor batch
+    assert lib.pce_select_dataflow(149866, 146018, 149866, 32, 32, 8, _lib.PCE_F32) != OSO
+    assert lib.pce_select_dataflow(146018, 149866, 149866, 32, 32, 8, _lib.PCE_F16) != OSO
 
 
 def test_codes_and_strides():
