@@ -461,6 +461,19 @@ def main() -> int:
         t3 = timer(down_up, 100, 10)[0]
         result["extra"]["cfg3"] = {"voxels_in": int(n), "voxels_out": int(km3.n_out), "pairs": int(km3.M),
                                    "dataflow_down": names[fd3], "dataflow_up": names[fu3], "down_up_ms": round(t3, 5)}
+        # the narrow stride-2 layers of a network's first levels on the same map (32 -> 32, 64 -> 64): the dataflow the
+        # selector gives them beside the two others that take them
+        narrow = {}
+        for c3 in (32, 64):
+            f3n = fd[:, :c3].contiguous()
+            w3n = torch.as_tensor(synth.weights(3, 8, c3, c3), device=dev).half()
+            p3n = backend.pack_weights(w3n)
+            o3n = torch.empty((km3.n_out, c3), dtype=torch.float16, device=dev)
+            pick = backend.select_dataflow(km3, c3, c3, torch.float16)
+            flows = {f: timer(lambda f=f: backend.conv_forward(f3n, w3n, km3, f, buffer=b3, packed=p3n, out=o3n), 50, 5)[0]
+                     for f in (DATAFLOW_OS, DATAFLOW_FDS, DATAFLOW_OSO)}
+            narrow[f"{c3}x{c3}"] = {"selector": names[pick], **{names[f] + "_ms": round(t, 5) for f, t in flows.items()}}
+        result["extra"]["cfg3"]["narrow_k2s2_layers"] = narrow
         # cfg5: 8 indoor scenes, the cfg4 network with channels doubled
         c5 = synth.indoor_batch()
         f5 = torch.as_tensor(synth.features(5, len(c5), 4), device=dev).half()

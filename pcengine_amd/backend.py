@@ -504,7 +504,11 @@ def oso_takes(km: KernelMap, c_in: int, c_out: int, dtype: torch.dtype, transpos
         return False
     if dtype == torch.float32:
         return km.subm and c_in % 8 == 0 and c_in <= 32 and c_out % 8 == 0 and c_out <= 32
-    return dtype == torch.float16 and c_in % 16 == 0 and c_in <= 64 and c_out % 8 == 0 and c_out <= 64
+    if dtype != torch.float16 or c_out % 8:
+        return False
+    if c_out <= 64:
+        return c_in % 16 == 0 and c_in <= 64
+    return (c_in in (64, 96) and c_out <= 128) or (c_in == 128 and c_out <= 96)      # the K-stepped form (wave_osw_kernel)
 
 
 def ensure_nbr(km: KernelMap, transposed: bool) -> None:
@@ -707,8 +711,8 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
     elif dataflow == DATAFLOW_OSO:
         if not oso_takes(km, c_in, c_out, feats.dtype, transposed):
             raise ValueError("the ordered output-stationary dataflow takes layers (not transposed, at most 31 offsets) in fp16 "
-                             "of at most 64 channels (c_in a multiple of 16, c_out of 8) or submanifold layers in fp32 of at "
-                             "most 32 (multiples of 8)")
+                             "of at most 64 channels (c_in a multiple of 16, c_out of 8), of 64 or 96 -> 65..128 and 128 -> "
+                             "65..96 channels, or submanifold layers in fp32 of at most 32 (multiples of 8)")
         if packed is None:
             packed = pack_weights(weight)      # None for fp32: that form reads the weights as they are
         order = row_order(km)

@@ -898,7 +898,7 @@ __global__ void __launch_bounds__(256, ((TMODE >= 0 && sizeof(T) == 2 && NB <= 2
 // on their way out (full lines, streaming stores).
 template <int PPR>
 __device__ __forceinline__ int row_swizzle(int row) {
-  return PPR == 8 ? (row & 7) : (PPR == 4 ? (row & 3) : (PPR == 2 ? (row & 1) : 0));
+  return (PPR >= 8 && PPR % 8 == 0) ? (row & 7) : ((PPR == 4 || (PPR > 8 && PPR % 4 == 0)) ? (row & 3) : (PPR == 2 ? (row & 1) : 0));
 }
 
 template <int NB, int KS>
@@ -2566,6 +2566,156 @@ __global__ void __launch_bounds__(256, 4) wave_os_kernel(TileArgs a, const int *
   store_rows_via_lds<half_t, NB>(V, Pl[wave], (half_t *)a.out, orow, a, 0, lane, l32, g, a.stream);
 }
 
+// The same dataflow for layers of 64 to 128 input and 65 to 128 output channels (fp16).  The weights of an offset
+// (12 to 24 KB) come straight from the packed copy in L2, all KS x NB fragments of the offset requested before the
+// first MFMA waits for one (in two batches where they would not leave three wavefronts per SIMD their registers);
+// no workgroup copy of the centre weights, no barrier.  A bare loop lets the scheduler pair every fragment's load
+// with its MFMA, two loads in flight: the layer took 39 us instead of 24, hence the scheduling barriers below.
+template <int NB, int KS>
+__global__ void __launch_bounds__(256, 2) wave_osw_kernel(TileArgs a, const int *__restrict__ perm,
+                                                          const unsigned *__restrict__ rmask, int mid, long long n_main,
+                                                          int heavy_wgs) {
+  constexpr int PPR = KS * 2;   // 16-byte pieces per input row
+  constexpr int NI = KS;        // global -> LDS instructions for the 32 centre rows
+  constexpr int REGION0 = WaveLds<NB>::PIECES > 32 * PPR ? WaveLds<NB>::PIECES : 32 * PPR;
+  constexpr int REGION = REGION0 > 256 ? REGION0 : 256;
+  __shared__ __attribute__((aligned(16))) half8 Pl[4][REGION];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int l32 = lane & 31, g = lane >> 5;
+  const half_t *Wp = (const half_t *)a.Wp;
+  const long long wstep = (long long)a.k8_total * a.n_pad * 8;
+  const bool heavy = (int)blockIdx.x < heavy_wgs;   // the same for the whole workgroup
+  long long j0, j_end;
+  if (heavy) {
+    j0 = n_main + (long long)blockIdx.x * 32;
+    j_end = a.n_rows;
+  } else {
+    const long long chunks = (n_main + 31) / 32;
+    const long long chunk = chunks - 1 - (((long long)blockIdx.x - heavy_wgs) * 4 + wave);
+    if (chunk < 0) return;
+    j0 = chunk * 32;
+    j_end = n_main;
+  }
+  const half_t *A = (const half_t *)a.A;
+  const int orow = j0 + l32 < j_end ? perm[j0 + l32] : -1;
+  const unsigned m = orow >= 0 ? rmask[orow] : 0u;
+  unsigned u = m;
+#pragma unroll
+  for (int d = 1; d < 32; d <<= 1) u |= (unsigned)__shfl_xor((int)u, d, PCE_WAVE);
+  unsigned todo = __builtin_amdgcn_readfirstlane(u);
+  if (heavy) todo &= 0x11111111u << wave;   // see wave_os_kernel: a split that depends on the offset alone
+  const bool centre = mid >= 0 && (!heavy || wave == 0);
+  if (centre) {
+#pragma unroll
+    for (int it = 0; it < NI; ++it) {
+      const int e = it * 64 + lane, r = e / PPR, sl = e % PPR;
+      const long long j = j0 + r < j_end ? j0 + r : j_end - 1;
+      const half_t *gp = A + (long long)perm[j] * a.lda + ((sl ^ row_swizzle<PPR>(r)) * 8);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
+                                       (__attribute__((address_space(3))) void *)&Pl[wave][it * 64], 16, 0, 0);
+    }
+  }
+  int k_next = todo ? __ffs((int)todo) - 1 : -1;
+  int nb_next = (k_next >= 0 && ((m >> k_next) & 1u)) ? a.nbr[(long long)k_next * a.n_rows + orow] : -1;
+  f32x16 acc[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[nb][j] = 0.f;
+  // the weight fragments of an offset, GB K steps at a time: all of them up to 18 (72 registers), else two batches
+  constexpr int GB = KS * NB <= 18 ? KS : KS / 2;
+  if (centre) {
+    const half_t *Wk = Wp + mid * wstep + ((long long)g * a.n_pad + l32) * 8;
+#pragma unroll
+    for (int b0 = 0; b0 < KS; b0 += GB) {
+      half8 wf[GB][NB];
+#pragma unroll
+      for (int s = 0; s < GB; ++s)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+          wf[s][nb] = *reinterpret_cast<const half8 *>(Wk + ((long long)(2 * (b0 + s)) * a.n_pad + nb * 32) * 8);
+      // the global -> LDS copies have landed once nothing is outstanding; the fragment reads stay behind this statement
+      // (the first batch of weights travels with the rows)
+      if (b0 == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int s = 0; s < GB; ++s) {
+        const half8 af = Pl[wave][l32 * PPR + ((2 * (b0 + s) + g) ^ row_swizzle<PPR>(l32))];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[s][nb], af, acc[nb], 0, 0, 0);
+      }
+    }
+  }
+  const half8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  while (k_next >= 0) {
+    const int k = k_next, nrow = nb_next;
+    todo &= todo - 1u;
+    // every load of the offset goes out before anything waits for one (the scheduler, left alone, pairs each weight
+    // fragment's load with its MFMA and keeps two in flight): the row fragments from a valid address, zeroed afterwards
+    // where the row has no neighbour here, the first batch of weight fragments, the next offset's neighbour index
+    half8 af[KS];
+    const half_t *rp = A + (long long)(nrow >= 0 ? nrow : 0) * a.lda + g * 8;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) af[s] = *reinterpret_cast<const half8 *>(rp + s * 16);
+    const half_t *Wk = Wp + k * wstep + ((long long)g * a.n_pad + l32) * 8;
+    k_next = todo ? __ffs((int)todo) - 1 : -1;
+    const long long nidx = (k_next >= 0 && ((m >> k_next) & 1u)) ? (long long)k_next * a.n_rows + orow : 0;
+#pragma unroll
+    for (int b0 = 0; b0 < KS; b0 += GB) {
+      half8 wf[GB][NB];
+#pragma unroll
+      for (int s = 0; s < GB; ++s)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+          wf[s][nb] = *reinterpret_cast<const half8 *>(Wk + ((long long)(2 * (b0 + s)) * a.n_pad + nb * 32) * 8);
+      if (b0 == 0) {
+        nb_next = a.nbr[nidx];
+        __builtin_amdgcn_sched_barrier(0);
+        if (!(k_next >= 0 && ((m >> k_next) & 1u))) nb_next = -1;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) af[s] = nrow >= 0 ? af[s] : zero;
+      } else {
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int s = 0; s < GB; ++s)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[s][nb], af[b0 + s], acc[nb], 0, 0, 0);
+    }
+  }
+  if (heavy) {
+    f32x16 *mine = reinterpret_cast<f32x16 *>(&Pl[wave][0]);
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      __syncthreads();
+      if (wave > 0) mine[lane] = acc[nb];
+      __syncthreads();
+      if (wave == 0) {
+#pragma unroll
+        for (int w2 = 1; w2 < 4; ++w2) {
+          const f32x16 other = reinterpret_cast<const f32x16 *>(&Pl[w2][0])[lane];
+#pragma unroll
+          for (int j = 0; j < 16; ++j) acc[nb][j] += other[j];
+        }
+      }
+    }
+    if (wave > 0) return;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();   // every lane has read its centre fragments: the region becomes the output staging area
+  float V[NB][2][8];
+  gather_row_pieces<NB>(acc, V, g);
+  if (a.bias || a.res || a.act) epilogue_row_pieces<half_t, NB, true>(V, a, orow, 0, g, a.act != PCE_ACT_NONE);
+  store_rows_via_lds<half_t, NB>(V, Pl[wave], (half_t *)a.out, orow, a, 0, lane, l32, g, a.stream);
+}
+
+// shapes the K-stepped form takes: fp16, 64 or 96 channels in and 65 to 128 out, or 128 in and 65 to 96 out (the shapes
+// it was measured to lead on; 128 -> 128 and 192 -> 128 ran 3 to 30 % behind deferred scatter)
+static bool wave_osw_ok(const TileArgs &a, int kv, int mid) {
+  const bool shape = (a.c_in == 64 || a.c_in == 96) ? a.c_out <= 128 : (a.c_in == 128 && a.c_out <= 96);
+  return a.Wp && a.a_vec && a.o_vec && shape && a.c_out % 8 == 0 && a.c_out > 64 && kv < ORDER_MAX_KV && mid < kv &&
+         aligned16(a.bias) && aligned16(a.res);
+}
+
 // The same dataflow for very narrow fp32 layers (c_in = 8 KQ up to 32, c_out up to 32: the 16-channel fp32 layer
 // of the reference's own test case).  Rows are 32 to 128 bytes, so nothing is staged on the way in: of a row's c_in
 // values the lane with g = 0 holds the first half, the lane with g = 1 the second (KQ 16-byte loads each), and MFMA
@@ -2694,10 +2844,12 @@ extern "C" int pce_conv_fwd_oso(const void *in, const void *w, const void *wp, v
   else
     set_out<half_t>(&a, out, false, n_out, e.ldo);
   set_epi(&a, e);
-  if (f32 ? !wave_os_f32_ok(a, kv, mid) : !wave_os_ok(a, kv, mid))
+  const bool wide = !f32 && wave_osw_ok(a, kv, mid);
+  if (!wide && (f32 ? !wave_os_f32_ok(a, kv, mid) : !wave_os_ok(a, kv, mid)))
     PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: takes layers in fp16 of at most 64 channels (multiples of 16 in, 8 out, packed "
-                         "weights) or submanifold layers in fp32 of at most 32 (multiples of 8), 16-byte aligned rows, kernel "
-                         "volumes up to 31; got dtype %d, %d -> %d channels, kv %d, mid %d", (int)dtype, (int)c_in, (int)c_out, (int)kv, (int)mid);
+                         "weights), of 64 or 96 -> 65..128 and 128 -> 65..96 channels, or submanifold layers in fp32 of at most "
+                         "32 (multiples of 8), 16-byte aligned rows, kernel volumes up to 31; got dtype %d, %d -> %d channels, "
+                         "kv %d, mid %d", (int)dtype, (int)c_in, (int)c_out, (int)kv, (int)mid);
   if (n_heavy < 0 || n_heavy > n_out) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: n_heavy=%lld outside [0, n_out]", (long long)n_heavy);
   a.nbr = nbr;
   a.n_rows = n_out;
@@ -2724,6 +2876,18 @@ extern "C" int pce_conv_fwd_oso(const void *in, const void *w, const void *wp, v
   if (a.n_pad != nb * 32 || a.k8_total != 2 * ks)
     PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: packed weights are %d x %d fragments per offset, expected %d x %d", a.k8_total, a.n_pad, 2 * ks, nb * 32);
   hipStream_t s = (hipStream_t)stream;
+  if (wide) {
+#define PCE_WOSW_CASE(NB_, KS_)                                                                              \
+  if (nb == NB_ && ks == KS_) {                                                                              \
+    hipLaunchKernelGGL((wave_osw_kernel<NB_, KS_>), dim3(grid), dim3(256), 0, s, a, perm, rmask, (int)mid, n_main,  \
+                       (int)heavy_wgs);                                                                      \
+    PCE_LAUNCH_CHECK("wave_osw");                                                                            \
+    return PCE_OK;                                                                                           \
+  }
+    PCE_WOSW_CASE(3, 4) PCE_WOSW_CASE(3, 6) PCE_WOSW_CASE(3, 8) PCE_WOSW_CASE(4, 4) PCE_WOSW_CASE(4, 6)
+#undef PCE_WOSW_CASE
+    PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: unsupported shape c_in=%d c_out=%d", (int)c_in, (int)c_out);
+  }
 #define PCE_WOS_CASE(NB_, KS_)                                                                              \
   if (nb == NB_ && ks == KS_) {                                                                              \
     hipLaunchKernelGGL((wave_os_kernel<NB_, KS_>), dim3(grid), dim3(256), 0, s, a, perm, rmask, (int)mid, n_main,   \
@@ -3633,6 +3797,14 @@ extern "C" int pce_select_dataflow(int64_t n_in, int64_t n_out, int64_t n_pairs,
   if (dtype == PCE_F16 && n_in == n_out && kv >= 3 && kv <= 31 && (kv & 1) && c_in % 16 == 0 && c_in <= 64 && c_out % 8 == 0 &&
       c_out <= 64 && rho <= 6.0)
     return PCE_DATAFLOW_OSO;
+  // the K-stepped form of the same kernel (wave_osw_kernel), measured on the levels of a 100 k-voxel LiDAR pyramid
+  // against the faster of deferred scatter and the dense tiles: 64 -> 96, 96 -> 96, 64 -> 128 at 0.8 / 3.0 / 8.9 pairs
+  // per row 0.80-0.88 / 0.71-0.79 / 0.81-0.91 of its time (equal at 0.13 and at 19.5); 128 -> 96 0.91 at 0.8 and 3.0,
+  // 1.03-1.12 elsewhere
+  if (dtype == PCE_F16 && n_in == n_out && kv >= 3 && kv <= 31 && (kv & 1) && c_out % 8 == 0 && c_out > 64) {
+    if ((c_in == 64 || c_in == 96) && c_out <= 128 && rho >= 0.5 && rho <= 12.0) return PCE_DATAFLOW_OSO;
+    if (c_in == 128 && c_out <= 96 && rho >= 0.5 && rho <= 4.0) return PCE_DATAFLOW_OSO;
+  }
   // narrow fp16 stride-2 layers (every input row in exactly one pair, 1-8 per output row), through the same ordered
   // rows without a centre term: 0.58-0.66 of the output-stationary tiles' time at 1.0-1.4 pairs per row (66-146 k
   // output rows, 32 and 64 channels; 680 k rows: 0.71), 0.57 at 2.4 on 27 k rows and 1.05 at 2.5 on 276 k rows of

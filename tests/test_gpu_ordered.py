@@ -77,7 +77,8 @@ def test_row_order_built_with_the_map_and_on_its_own(cloud):
 
 
 @pytest.mark.parametrize("cloud", sorted(CLOUDS))
-@pytest.mark.parametrize("c_in,c_out", [(64, 64), (32, 32), (16, 32), (48, 24), (64, 8), (16, 64)])
+@pytest.mark.parametrize("c_in,c_out", [(64, 64), (32, 32), (16, 32), (48, 24), (64, 8), (16, 64),
+                                        (64, 96), (96, 96), (64, 128), (96, 128), (128, 96), (96, 72)])   # the last six: the K-stepped kernel
 def test_ordered_dataflow_against_the_oracle(cloud, c_in, c_out):
     coords = CLOUDS[cloud]()
     ref, _ = _oracle_masks(coords)
@@ -190,7 +191,7 @@ def test_row_order_of_strided_maps(cloud, geom):
 
 @pytest.mark.parametrize("cloud", sorted(CLOUDS))
 @pytest.mark.parametrize("geom", range(len(STRIDED)))
-@pytest.mark.parametrize("c_in,c_out", [(32, 32), (64, 64), (16, 64), (48, 24)])
+@pytest.mark.parametrize("c_in,c_out", [(32, 32), (64, 64), (16, 64), (48, 24), (64, 96), (128, 80)])
 def test_ordered_dataflow_strided_against_the_oracle(cloud, geom, c_in, c_out):
     """The ordered rows without a centre term (strided layers, fp16): the float64 oracle within 1e-3, epilogue fused,
     bit-equal from run to run, column slices on both sides."""
@@ -257,7 +258,9 @@ def test_ordered_dataflow_on_column_slices_and_the_selector():
     assert backend.select_dataflow(km, c, c, torch.float16) == DATAFLOW_OSO
     assert backend.select_dataflow(km, 16, 16, torch.float32) == DATAFLOW_OSO      # the fp32 form: up to 32 channels, by density
     assert backend.select_dataflow(km, 64, 64, torch.float32) != DATAFLOW_OSO
-    assert backend.select_dataflow(km, 96, 96, torch.float16) != DATAFLOW_OSO
+    assert backend.select_dataflow(km, 128, 128, torch.float16) != DATAFLOW_OSO
+    assert backend.oso_takes(km, 96, 96, torch.float16) and backend.oso_takes(km, 128, 96, torch.float16)
+    assert not backend.oso_takes(km, 128, 128, torch.float16) and not backend.oso_takes(km, 192, 128, torch.float16)
     # the two pair-proportional dataflows agree to fp16 rounding (they round partial sums at different places)
     fds = backend.conv_forward(f, w, km, DATAFLOW_FDS, packed=packed)
     assert float((fds.float() - want.float()).norm() / want.float().norm()) <= 1e-3
@@ -283,10 +286,11 @@ def test_ordered_dataflow_argument_errors():
     assert call(_lib.PCE_F16, 32, 32, 13, n + 1) == _lib.PCE_EINVAL
     assert call(_lib.PCE_F16, 32, 32, 13, km.order_heavy, None) == _lib.PCE_EINVAL    # weights not packed
     assert call(_lib.PCE_F16, 128, 32, 13, km.order_heavy) == _lib.PCE_EINVAL
+    assert call(_lib.PCE_F16, 128, 128, 13, km.order_heavy) == _lib.PCE_EINVAL       # beyond the K-stepped kernel's shapes
     heavy = _lib.c_int64(0)
     order = torch.zeros(lib.pce_row_order_elems(n), dtype=torch.int32, device=DEV)
     assert lib.pce_row_order(km.nbr_out.data_ptr(), 27, n, 13, order.data_ptr(), order.numel() - 1, heavy, s) == _lib.PCE_EWORKSPACE
     assert lib.pce_row_order(km.nbr_out.data_ptr(), 125, n, 62, order.data_ptr(), order.numel(), heavy, s) == _lib.PCE_EINVAL
     with pytest.raises(ValueError):
-        backend.conv_forward(torch.zeros((n, 96), dtype=torch.float16, device=DEV), torch.zeros((27, 96, 32), dtype=torch.float16, device=DEV),
+        backend.conv_forward(torch.zeros((n, 192), dtype=torch.float16, device=DEV), torch.zeros((27, 192, 128), dtype=torch.float16, device=DEV),
                              km, DATAFLOW_OSO)

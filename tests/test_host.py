@@ -91,7 +91,11 @@ def test_selector_on_measured_layers():
         (97941, 97941, 80234, 32, 32, 27, OSO),        # narrow layers of a LiDAR network: rho 0.8 and 3.0
         (89469, 89469, 271786, 64, 64, 27, OSO),
         (541185, 541185, 2852000, 64, 64, 27, OSO),    # indoor batch, rho 5.3: equal to output-stationary, 0.6 of deferred scatter
-        (99692, 99692, 13406, 96, 96, 27, FDS),        # wider than the ordered kernel takes
+        (99692, 99692, 13406, 96, 96, 27, FDS),        # hardly any pairs: the centre GEMM decides, deferred scatter as fast
+        (97941, 97941, 80234, 96, 96, 27, OSO),        # the K-stepped ordered kernel: 28 vs 32 us
+        (97941, 97941, 80234, 128, 96, 27, OSO),       # 31 vs 34 us
+        (89469, 89469, 271786, 128, 128, 27, FDS),     # wider than the ordered kernels take: 64 vs 67 us
+        (89469, 89469, 271786, 192, 128, 27, FDS),
         (65807, 65807, 586656, 64, 64, 27, OS),        # rho 8.9: the dense tiles
         (149866, 146018, 149866, 64, 128, 8, FDS),     # k2s2 on a LiDAR cloud: one pair for nearly every row
         (216268, 53439, 215000, 128, 128, 8, OS),      # k2s2 on an indoor batch, four pairs per row
@@ -100,7 +104,8 @@ def test_selector_on_measured_layers():
         (53439, 53439, 550000, 256, 256, 27, FDS),
         (25916, 25916, 506646, 256, 256, 27, OS),      # rho = 19.5
         (12063, 12063, 140000, 512, 512, 27, FDS),
-        (65807, 65807, 586656, 64, 128, 27, OS),
+        (65807, 65807, 586656, 64, 128, 27, OSO),      # 56 vs 63 us for the dense tiles
+        (25916, 25916, 506646, 64, 128, 27, OS),       # rho = 19.5: 33 vs 37 us
     ]
     for n_in, n_out, pairs, ci, co, kv, want in cases:
         assert lib.pce_select_dataflow(n_in, n_out, pairs, ci, co, kv, _lib.PCE_F16) == want, (n_in, n_out, ci, co, kv)
