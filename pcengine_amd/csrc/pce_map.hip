@@ -1315,7 +1315,7 @@ struct Job {
   int kind;
   int pad;
 };
-enum { JOB_CSR_SUBM = 0, JOB_CSR_IN = 1, JOB_CSR_COUNT_OUT = 2, JOB_CSR_OUT = 3 };
+enum { JOB_CSR_SUBM = 0, JOB_CSR_IN = 1, JOB_CSR_COUNT_OUT = 2, JOB_CSR_OUT = 3, JOB_ORDER_SCATTER = 4 };
 
 struct FillRegion {
   unsigned *p;
@@ -1610,6 +1610,105 @@ __global__ void __launch_bounds__(256) grid_query_kernel(const ProbDev *__restri
   }
 }
 
+// ---- row order of the ordered output-stationary dataflow -----------------------------------------------------
+// Output rows of a map in an order that puts equal neighbour patterns side by side: rows without neighbours
+// first (block by block, each block's rows in their own order), then the rows with one or two neighbours sorted
+// by the (lowest, second-lowest) offset they have one at, then the rows with ORDER_HEAVY_POPC or more, sorted
+// likewise.  A counting sort: masks and a histogram of the keys, one block that turns the histogram into
+// bases, a scatter pass with one cursor per key.  The kernels exist twice: over the job lists of a batched map
+// build, and with plain arguments for an order requested on its own (pce_row_order).
+__device__ __forceinline__ int order_key(unsigned m) {   // m != 0
+  const int first = __ffs((int)m) - 1;
+  const unsigned rest = m & (m - 1u);
+  const int second = rest ? __ffs((int)rest) - 1 : 31;
+  return (__popc(m) >= ORDER_HEAVY_POPC ? 1024 : 0) + first * 32 + second;
+}
+
+// mask[row] = offsets (other than the centre) at which the row has a neighbour; hist[key] += the block's count.
+// The keys of a block of 256 rows are counted in LDS first: on a dense cloud nearly every row has a key and a few
+// keys hold most rows, and one global atomic per row on those few addresses costs milliseconds.
+__device__ __forceinline__ void order_mask_block(const int *__restrict__ nbr, int kv, long long n_rows, int mid,
+                                                 int *__restrict__ order, unsigned blk) {
+  __shared__ int cnt[ORDER_KEYS];
+  for (int i = threadIdx.x; i < ORDER_KEYS; i += 256) cnt[i] = 0;
+  __syncthreads();
+  const long long row = (long long)blk * 256 + threadIdx.x;
+  if (row < n_rows) {
+    unsigned m = 0;
+    for (int k = 0; k < kv; ++k)
+      if (k != mid && nbr[(long long)k * n_rows + row] >= 0) m |= 1u << k;
+    order[n_rows + row] = (int)m;
+    if (m) atomicAdd(&cnt[order_key(m)], 1);   // rows without neighbours are placed by the scatter pass
+  }
+  __syncthreads();
+  int *hist = order + 2 * n_rows + ORDER_HIST;
+  for (int i = threadIdx.x; i < ORDER_KEYS; i += 256)
+    if (cnt[i]) atomicAdd(&hist[i], cnt[i]);
+}
+
+// base[key] = first position of the key's rows behind the rows without neighbours (one block of 1024); the counts
+__device__ __forceinline__ void order_scan_block(int *tail, int *n_heavy_out) {
+  __shared__ int part[1024];
+  const int *hist = tail + ORDER_HIST;
+  int *base = tail + ORDER_BASE;
+  constexpr int per = ORDER_KEYS / 1024;
+  int sum = 0;
+#pragma unroll
+  for (int j = 0; j < per; ++j) sum += hist[threadIdx.x * per + j];
+  part[threadIdx.x] = sum;
+  __syncthreads();
+  for (int d = 1; d < 1024; d <<= 1) {
+    int v = (int)threadIdx.x >= d ? part[threadIdx.x - d] : 0;
+    __syncthreads();
+    part[threadIdx.x] += v;
+    __syncthreads();
+  }
+  if (threadIdx.x == 1023) {
+    tail[ORDER_N_NONZERO] = part[1023];
+    tail[ORDER_N_HEAVY] = part[1023] - part[511];      // keys 1024 .. 2047 belong to threads 512 .. 1023
+    if (n_heavy_out) *n_heavy_out = part[1023] - part[511];
+  }
+  int run = part[threadIdx.x] - sum;
+#pragma unroll
+  for (int j = 0; j < per; ++j) {
+    base[threadIdx.x * per + j] = run;
+    run += hist[threadIdx.x * per + j];
+  }
+}
+
+// perm: the rows of one block of 256 (block `blk` of the map), placed as described above.  A block takes one range
+// per key it holds (one global atomic per key and block); its rows of a key keep the ranks LDS atomics gave them.
+__device__ __forceinline__ void order_scatter_block(long long n_rows, int *__restrict__ order, unsigned blk) {
+  __shared__ int cnt[ORDER_KEYS], gbase[ORDER_KEYS];
+  __shared__ int wcount[4], wbase;
+  int *perm = order, *tail = order + 2 * n_rows;
+  for (int i = threadIdx.x; i < ORDER_KEYS; i += 256) cnt[i] = 0;
+  const long long n_plain = n_rows - tail[ORDER_N_NONZERO];
+  long long row = (long long)blk * 256 + threadIdx.x;
+  const bool live = row < n_rows;
+  const unsigned m = live ? (unsigned)order[n_rows + row] : 1u;
+  const bool plain = live && m == 0;
+  const unsigned long long b = __ballot(plain);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) wcount[wave] = __popcll(b);
+  __syncthreads();
+  if (threadIdx.x == 0) wbase = atomicAdd(&tail[ORDER_PLAIN_CURSOR], wcount[0] + wcount[1] + wcount[2] + wcount[3]);
+  const int key = (live && !plain) ? order_key(m) : -1;
+  int rank = 0;
+  if (key >= 0) rank = atomicAdd(&cnt[key], 1);
+  __syncthreads();
+  for (int i = threadIdx.x; i < ORDER_KEYS; i += 256)
+    if (cnt[i]) gbase[i] = tail[ORDER_BASE + i] + atomicAdd(&tail[ORDER_CURSOR + i], cnt[i]);
+  __syncthreads();
+  if (plain) {
+    int before = __popcll(b & ((1ull << lane) - 1ull));
+    for (int w2 = 0; w2 < wave; ++w2) before += wcount[w2];
+    perm[wbase + before] = (int)row;
+  } else if (key >= 0) {
+    perm[n_plain + gbase[key] + rank] = (int)row;
+  }
+}
+
 // The per-row loops over the offsets below load ROW_BATCH table entries before using any of them.
 #define ROW_BATCH 9
 
@@ -1626,6 +1725,15 @@ __global__ void __launch_bounds__(256) kmap_count_kernel(const ProbDev *__restri
   long long i = (long long)(blockIdx.x - job.blk0) * blockDim.x + threadIdx.x;
   long long seg = i >> 6;
   bool live = i < n_in;
+  // A symmetric map's output-major table is its probe table mirrored (nbr_out[kp] = dense[kv-1-kp]), so the offset
+  // masks and the key histogram of its row order come out of this pass (order_mask_block does the same from nbr_out).
+  const bool masks = q.order && q.g.sym;      // the same for the whole workgroup
+  __shared__ int keycnt[ORDER_KEYS];
+  if (masks) {
+    for (int t = threadIdx.x; t < ORDER_KEYS; t += 256) keycnt[t] = 0;
+    __syncthreads();
+  }
+  unsigned m = 0;
   int c = 0;
   for (int kp0 = 0; kp0 < kv; kp0 += ROW_BATCH) {
     int v[ROW_BATCH];
@@ -1636,12 +1744,23 @@ __global__ void __launch_bounds__(256) kmap_count_kernel(const ProbDev *__restri
       if (kp0 + j >= kv) break;
       bool hit = v[j] >= 0;
       c += hit;
+      if (masks && hit && kp0 + j != q.g.mid) m |= 1u << (kv - 1 - (kp0 + j));
       unsigned long long bal = __ballot(hit);
       if (__lane_id() == 0 && seg < nseg) segcnt[(long long)(kp0 + j) * nseg + seg] = __popcll(bal);
     }
   }
   if (rowcnt && i <= n_in) rowcnt[i] = live ? c : 0;  // rowcnt[n_in] = 0 receives the total after the scan
   if (i == 0) segcnt[(long long)kv * nseg] = 0;
+  if (masks) {
+    if (live) {
+      q.order[n_in + i] = (int)m;
+      if (m) atomicAdd(&keycnt[order_key(m)], 1);
+    }
+    __syncthreads();
+    int *hist = q.order + 2 * n_in + ORDER_HIST;
+    for (int t = threadIdx.x; t < ORDER_KEYS; t += 256)
+      if (keycnt[t]) atomicAdd(&hist[t], keycnt[t]);
+  }
 }
 
 // Exclusive scans of several arrays in two launches: every workgroup scans its SCAN_TILE items in place
@@ -1687,7 +1806,14 @@ __global__ void __launch_bounds__(256) multi_scan_add_kernel(const ScanArr *__re
 
 // kpos[kp] = first pair of offset kp; then the scan of counts rounded up to the tile height
 // (backend/hash.cuh:478-497).  One workgroup per problem.
-__global__ void kmap_offsets_kernel(const ProbDev *__restrict__ P) {
+// Workgroups [n_probs, 2 n_probs): the bases of the row order's counting sort for the maps whose key histogram the
+// counting pass has filled (symmetric maps).
+__global__ void __launch_bounds__(1024) kmap_offsets_kernel(const ProbDev *__restrict__ P, int n_probs) {
+  if ((int)blockIdx.x >= n_probs) {
+    const ProbDev &o = P[blockIdx.x - n_probs];
+    if (o.order && o.g.sym) order_scan_block(o.order + 2 * o.n_out, o.status + 4);   // the same for the whole workgroup
+    return;
+  }
   const ProbDev &q = P[blockIdx.x];
   const int *__restrict__ segoff = q.seg;
   const long long nseg = q.nseg;
@@ -1715,6 +1841,10 @@ __global__ void kmap_offsets_kernel(const ProbDev *__restrict__ P) {
 __global__ void __launch_bounds__(256) kmap_fill_kernel(const ProbDev *__restrict__ P, JobList jl) {
   const Job &job = find_job(jl, blockIdx.x);
   const ProbDev &q = P[job.prob];
+  if (job.kind == JOB_ORDER_SCATTER) {   // the row order of a symmetric map: masks and bases are complete by now
+    order_scatter_block(q.n_out, q.order, blockIdx.x - job.blk0);
+    return;
+  }
   const long long n_in = q.n_in, n_out = q.n_out, nseg = q.nseg;
   const int kv = q.g.kv, subm = q.g.subm, sym = q.g.sym, mid = q.g.mid;
   const int *__restrict__ dense = q.dense;
@@ -1873,105 +2003,6 @@ extern "C" int64_t pce_kmap_workspace_bytes_grid(int64_t n_in, int64_t n_out, co
 }
 
 // stages of a batched build, each one launch with its own job list
-// ---- row order of the ordered output-stationary dataflow -----------------------------------------------------
-// Output rows of a map in an order that puts equal neighbour patterns side by side: rows without neighbours
-// first (block by block, each block's rows in their own order), then the rows with one or two neighbours sorted
-// by the (lowest, second-lowest) offset they have one at, then the rows with ORDER_HEAVY_POPC or more, sorted
-// likewise.  A counting sort: masks and a histogram of the keys, one block that turns the histogram into
-// bases, a scatter pass with one cursor per key.  The kernels exist twice: over the job lists of a batched map
-// build, and with plain arguments for an order requested on its own (pce_row_order).
-__device__ __forceinline__ int order_key(unsigned m) {   // m != 0
-  const int first = __ffs((int)m) - 1;
-  const unsigned rest = m & (m - 1u);
-  const int second = rest ? __ffs((int)rest) - 1 : 31;
-  return (__popc(m) >= ORDER_HEAVY_POPC ? 1024 : 0) + first * 32 + second;
-}
-
-// mask[row] = offsets (other than the centre) at which the row has a neighbour; hist[key] += the block's count.
-// The keys of a block of 256 rows are counted in LDS first: on a dense cloud nearly every row has a key and a few
-// keys hold most rows, and one global atomic per row on those few addresses costs milliseconds.
-__device__ __forceinline__ void order_mask_block(const int *__restrict__ nbr, int kv, long long n_rows, int mid,
-                                                 int *__restrict__ order, unsigned blk) {
-  __shared__ int cnt[ORDER_KEYS];
-  for (int i = threadIdx.x; i < ORDER_KEYS; i += 256) cnt[i] = 0;
-  __syncthreads();
-  const long long row = (long long)blk * 256 + threadIdx.x;
-  if (row < n_rows) {
-    unsigned m = 0;
-    for (int k = 0; k < kv; ++k)
-      if (k != mid && nbr[(long long)k * n_rows + row] >= 0) m |= 1u << k;
-    order[n_rows + row] = (int)m;
-    if (m) atomicAdd(&cnt[order_key(m)], 1);   // rows without neighbours are placed by the scatter pass
-  }
-  __syncthreads();
-  int *hist = order + 2 * n_rows + ORDER_HIST;
-  for (int i = threadIdx.x; i < ORDER_KEYS; i += 256)
-    if (cnt[i]) atomicAdd(&hist[i], cnt[i]);
-}
-
-// base[key] = first position of the key's rows behind the rows without neighbours (one block of 1024); the counts
-__device__ __forceinline__ void order_scan_block(int *tail, int *n_heavy_out) {
-  __shared__ int part[1024];
-  const int *hist = tail + ORDER_HIST;
-  int *base = tail + ORDER_BASE;
-  constexpr int per = ORDER_KEYS / 1024;
-  int sum = 0;
-#pragma unroll
-  for (int j = 0; j < per; ++j) sum += hist[threadIdx.x * per + j];
-  part[threadIdx.x] = sum;
-  __syncthreads();
-  for (int d = 1; d < 1024; d <<= 1) {
-    int v = (int)threadIdx.x >= d ? part[threadIdx.x - d] : 0;
-    __syncthreads();
-    part[threadIdx.x] += v;
-    __syncthreads();
-  }
-  if (threadIdx.x == 1023) {
-    tail[ORDER_N_NONZERO] = part[1023];
-    tail[ORDER_N_HEAVY] = part[1023] - part[511];      // keys 1024 .. 2047 belong to threads 512 .. 1023
-    if (n_heavy_out) *n_heavy_out = part[1023] - part[511];
-  }
-  int run = part[threadIdx.x] - sum;
-#pragma unroll
-  for (int j = 0; j < per; ++j) {
-    base[threadIdx.x * per + j] = run;
-    run += hist[threadIdx.x * per + j];
-  }
-}
-
-// perm: the rows of one block of 256 (block `blk` of the map), placed as described above.  A block takes one range
-// per key it holds (one global atomic per key and block); its rows of a key keep the ranks LDS atomics gave them.
-__device__ __forceinline__ void order_scatter_block(long long n_rows, int *__restrict__ order, unsigned blk) {
-  __shared__ int cnt[ORDER_KEYS], gbase[ORDER_KEYS];
-  __shared__ int wcount[4], wbase;
-  int *perm = order, *tail = order + 2 * n_rows;
-  for (int i = threadIdx.x; i < ORDER_KEYS; i += 256) cnt[i] = 0;
-  const long long n_plain = n_rows - tail[ORDER_N_NONZERO];
-  long long row = (long long)blk * 256 + threadIdx.x;
-  const bool live = row < n_rows;
-  const unsigned m = live ? (unsigned)order[n_rows + row] : 1u;
-  const bool plain = live && m == 0;
-  const unsigned long long b = __ballot(plain);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  if (lane == 0) wcount[wave] = __popcll(b);
-  __syncthreads();
-  if (threadIdx.x == 0) wbase = atomicAdd(&tail[ORDER_PLAIN_CURSOR], wcount[0] + wcount[1] + wcount[2] + wcount[3]);
-  const int key = (live && !plain) ? order_key(m) : -1;
-  int rank = 0;
-  if (key >= 0) rank = atomicAdd(&cnt[key], 1);
-  __syncthreads();
-  for (int i = threadIdx.x; i < ORDER_KEYS; i += 256)
-    if (cnt[i]) gbase[i] = tail[ORDER_BASE + i] + atomicAdd(&tail[ORDER_CURSOR + i], cnt[i]);
-  __syncthreads();
-  if (plain) {
-    int before = __popcll(b & ((1ull << lane) - 1ull));
-    for (int w2 = 0; w2 < wave; ++w2) before += wcount[w2];
-    perm[wbase + before] = (int)row;
-  } else if (key >= 0) {
-    perm[n_plain + gbase[key] + rank] = (int)row;
-  }
-}
-
 __global__ void order_clear_kernel(int *tail) {
   for (int i = threadIdx.x; i < PCE_ORDER_TAIL; i += blockDim.x) tail[i] = 0;
 }
@@ -1992,7 +2023,7 @@ __global__ void __launch_bounds__(256) order_mask_batch_kernel(const ProbDev *__
 }
 __global__ void __launch_bounds__(1024) order_scan_batch_kernel(const ProbDev *__restrict__ P) {
   const ProbDev &q = P[blockIdx.x];
-  if (!q.order) return;
+  if (!q.order || q.g.sym) return;   // a symmetric map's histogram was scanned with the pair offsets
   order_scan_block(q.order + 2 * q.n_out, q.status + 4);
 }
 __global__ void __launch_bounds__(256) order_scatter_batch_kernel(const ProbDev *__restrict__ P, JobList jl) {
@@ -2173,8 +2204,10 @@ extern "C" int pce_kmap_build_batch(const pce_kmap_problem_t *probs, int32_t n_p
       if (n_out >= (1ll << 30)) PCE_FAIL(PCE_ECAPACITY, "pce_kmap_build: too many rows for a row order");
       q.order = u.order;
       add_fill(u.order + 2 * n_out, PCE_ORDER_TAIL, 1);
-      add_job(ST_ORDER_MASK, p, 0, n_out);
-      add_job(ST_ORDER_SCATTER, p, 0, n_out);
+      if (!q.g.sym) {   // a symmetric map's order rides on the counting, offset and fill launches (see there)
+        add_job(ST_ORDER_MASK, p, 0, n_out);
+        add_job(ST_ORDER_SCATTER, p, 0, n_out);
+      }
     }
     q.want_csr = want_csr;
     q.use_grid = use_grid;
@@ -2204,6 +2237,7 @@ extern "C" int pce_kmap_build_batch(const pce_kmap_problem_t *probs, int32_t n_p
     add_scan(0, q.seg, L.scan_len, scan_tmp);
     if (want_csr) add_scan(0, q.icsr, n_in + 1, scan_tmp + scan_tmp_ints(L.scan_len));
     add_job(ST_FILL, p, 0, n_in);
+    if (q.order && q.g.sym) add_job(ST_FILL, p, JOB_ORDER_SCATTER, n_out);
     // 5. CSR-coded views
     if (want_csr && q.g.sym) {
       add_job(ST_CSR_A, p, JOB_CSR_SUBM, n_in + 1);
@@ -2260,7 +2294,7 @@ extern "C" int pce_kmap_build_batch(const pce_kmap_problem_t *probs, int32_t n_p
   PCE_LAUNCH_CHECK("scan_local");
   hipLaunchKernelGGL(multi_scan_add_kernel, dim3(scan_blk[0]), dim3(256), 0, s, (const ScanArr *)D->scans[0], n_scan[0]);
   PCE_LAUNCH_CHECK("scan_add");
-  hipLaunchKernelGGL(kmap_offsets_kernel, dim3(n_probs), dim3(128), 0, s, P);
+  hipLaunchKernelGGL(kmap_offsets_kernel, dim3(2 * n_probs), dim3(1024), 0, s, P, (int)n_probs);
   PCE_LAUNCH_CHECK("kmap_offsets");
   hipLaunchKernelGGL(kmap_fill_kernel, dim3(blk[ST_FILL]), dim3(256), 0, s, P, jl(ST_FILL));
   PCE_LAUNCH_CHECK("kmap_fill");
