@@ -3811,6 +3811,13 @@ extern "C" int pce_select_dataflow(int64_t n_in, int64_t n_out, int64_t n_pairs,
   // indoor scenes, where half the rows have three pairs or more
   if (dtype == PCE_F16 && kv <= 8 && n_out < n_in && c_in % 16 == 0 && c_in <= 64 && c_out % 8 == 0 && c_out <= 64 && rho <= 2.0)
     return PCE_DATAFLOW_OSO;
+  // ... and of the K-stepped kernel's shapes: 64 -> 128, 64 / 96 -> 96, 96 -> 128, 128 -> 96 at 1.0-2.5 pairs per row on
+  // five levels of LiDAR and indoor pyramids (26 k to 541 k output rows) 0.64-0.94 of the faster of deferred scatter
+  // and the dense tiles (64 -> 128 on the 146 k-row level of the headline cloud: 21.3 vs 24.5 us); 128 -> 128, tried
+  // with a sixth instantiation, ran from 0.72 to 1.06 of it with nothing in (rows, density) to tell the cases apart
+  if (dtype == PCE_F16 && kv <= 8 && n_out < n_in && c_out % 8 == 0 && c_out > 64 && rho <= 2.6 &&
+      (((c_in == 64 || c_in == 96) && c_out <= 128) || (c_in == 128 && c_out <= 96)))
+    return PCE_DATAFLOW_OSO;
   if (kv <= 8 && n_out <= n_in && rho >= 1.0 && prod <= 64 * 64 && dtype == PCE_F16) return PCE_DATAFLOW_OS;
   if (kv <= 8 && n_out <= n_in && rho >= 2.0 && prod <= 128 * 128 && dtype == PCE_F16) return PCE_DATAFLOW_OS;
   double takeover;

@@ -235,7 +235,8 @@ def test_selector_gives_narrow_stride_2_layers_to_the_ordered_rows():
     assert km.M / km.n_out <= 2.0
     assert backend.select_dataflow(km, 32, 32, torch.float16) == DATAFLOW_OSO
     assert backend.select_dataflow(km, 64, 64, torch.float16) == DATAFLOW_OSO
-    assert backend.select_dataflow(km, 64, 128, torch.float16) != DATAFLOW_OSO
+    assert backend.select_dataflow(km, 64, 128, torch.float16) == DATAFLOW_OSO       # the K-stepped kernel's shapes too
+    assert backend.select_dataflow(km, 128, 128, torch.float16) != DATAFLOW_OSO
     assert backend.select_dataflow(km, 32, 32, torch.float32) != DATAFLOW_OSO
     assert backend.select_dataflow(km, 32, 32, torch.float16, transposed=True) != DATAFLOW_OSO
     dense = _strided_map(CLOUDS["dense"](), 0)          # a filled box: close to eight pairs per output row

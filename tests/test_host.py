@@ -97,7 +97,9 @@ def test_selector_on_measured_layers():
         (89469, 89469, 271786, 128, 128, 27, FDS),     # wider than the ordered kernels take: 64 vs 67 us
         (89469, 89469, 271786, 192, 128, 27, FDS),
         (65807, 65807, 586656, 64, 64, 27, OS),        # rho 8.9: the dense tiles
-        (149866, 146018, 149866, 64, 128, 8, FDS),     # k2s2 on a LiDAR cloud: one pair for nearly every row
+        (149866, 146018, 149866, 64, 128, 8, OSO),     # k2s2 on a LiDAR cloud, one pair for nearly every row: 21.3 vs 24.5 us (FDS)
+        (149866, 146018, 149866, 128, 128, 8, FDS),    # ... wider than the ordered kernels take: routed deferred scatter
+        (541185, 216268, 539306, 128, 96, 8, OSO),     # indoor batch, 2.5 pairs per row: 60 vs 65 us (OS)
         (216268, 53439, 215000, 128, 128, 8, OS),      # k2s2 on an indoor batch, four pairs per row
         (65807, 25916, 64194, 128, 128, 8, OS),
         (53439, 53439, 550000, 128, 256, 27, OS),      # rho = 10.3
