@@ -461,6 +461,9 @@ def main() -> int:
         t3 = timer(down_up, 100, 10)[0]
         result["extra"]["cfg3"] = {"voxels_in": int(n), "voxels_out": int(km3.n_out), "pairs": int(km3.M),
                                    "dataflow_down": names[fd3], "dataflow_up": names[fu3], "down_up_ms": round(t3, 5)}
+        down = {f: timer(lambda f=f: backend.conv_forward(fd, wdn, km3, f, buffer=b3, packed=pdn, out=mid3), 50, 5)[0]
+                for f in (DATAFLOW_OS, DATAFLOW_FDS, DATAFLOW_OSO)}
+        result["extra"]["cfg3"]["down_ms_by_dataflow"] = {names[f]: round(t, 5) for f, t in down.items()}
         # the narrow stride-2 layers of a network's first levels on the same map (32 -> 32, 64 -> 64): the dataflow the
         # selector gives them beside the two others that take them
         narrow = {}
