@@ -220,7 +220,8 @@ def test_scheduler_hint_and_buffer_size():
 # mangled-name prefixes: wave_os_kernel<2,4>, wave_gemm_kernel<2,4>, tile_gemm_kernel<half,4|3,FAST,MODE_OS,EPI_ROWS>, pipe_gemm_kernel<*>
 _VGPR_CEILINGS = [("_Z14wave_os_kernelILi2ELi4E", 128), ("_Z16wave_gemm_kernelILi2ELi4E", 72),
                   ("_Z16tile_gemm_kernelIDF16_Li4ELb1ELi3ELi1E", 96), ("_Z16tile_gemm_kernelIDF16_Li3ELb1ELi3ELi1E", 80),
-                  ("_Z16pipe_gemm_kernelILi", 128)]
+                  ("_Z16pipe_gemm_kernelILi", 128),
+                  ("_Z15wave_osw_kernelILi", 168)]      # three wavefronts per SIMD for every shape of the K-stepped ordered kernel
 
 def test_no_kernel_uses_scratch_memory(tmp_path):
     """Register spills turn a memory-bound kernel into a several times slower one without changing a
