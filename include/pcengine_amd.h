@@ -58,8 +58,8 @@ enum {
   PCE_DATAFLOW_FDS = 3, /* fetch-on-demand with deferred scatter: pair tiles write partial rows to a
                            staging buffer, the centre GEMM's epilogue sums them per output row */
   PCE_DATAFLOW_OSO = 4  /* output-stationary over rows ordered by their neighbour pattern (pce_row_order):
-                           narrow layers (fp16 up to 64 channels, submanifold or stride 2; fp32 submanifold up to 32),
-                           one launch, no partial rows */
+                           fp16 layers up to 64 channels and of 64 / 96 -> 65..128 and 128 -> 65..96 channels, submanifold
+                           or strided; fp32 submanifold layers up to 32 channels; one launch, no partial rows */
 };
 
 #define PCE_QUANTUM 128        /* rows per tile of the pair list; qkpos granularity (backend/hash.cu:203-205) */
@@ -376,8 +376,10 @@ int pce_conv_fwd_os(const void *in_feats, const void *weight, const void *weight
  * the results of the layer do not.  pce_conv_fwd_oso then runs the layer as one launch: a wavefront takes 32 rows
  * of that order, multiplies their centre rows, gathers for each offset any of them has the neighbours of the rows
  * that have it, and stores each finished row once (epilogue fused); the rows of the last part, whose offsets are
- * many, go 32 to a workgroup whose four wavefronts share the offsets.  PCE_F16: c_in a multiple of 16 and at most
- * 64, c_out a multiple of 8 and at most 64, packed weights; PCE_F32: c_in and c_out multiples of 8 and at most 32
+ * many, go 32 to a workgroup whose four wavefronts share the offsets.  PCE_F16, packed weights: c_in a multiple of
+ * 16 and at most 64 with c_out a multiple of 8 and at most 64; or c_in 64 or 96 with c_out a multiple of 8 in 65..128;
+ * or c_in 128 with c_out a multiple of 8 in 65..96 (these wider shapes stream an offset's weights from the packed copy
+ * K step by K step); PCE_F32: c_in and c_out multiples of 8 and at most 32
  * (weight_packed is not read) and mid >= 0; PCE_EINVAL otherwise.  In PCE_F16 a layer without a centre offset
  * (mid = -1: a strided layer, n_in != n_out, nbr_dev = its output-major table [kv][n_out], order from pce_row_order
  * with mid = -1) runs the same way from zero sums: every output row of a 2x2x2 stride-2 layer has one to eight pairs,
