@@ -228,7 +228,8 @@ def _run(input: spTensor, km: backend.KernelMap, kernel, in_channel, out_channel
         kernel, packed = kernel.to(feats.dtype), None
     if kernel.dim() == 3 and feats.shape[1] < kernel.shape[1]:
         feats = torch.nn.functional.pad(feats, (0, kernel.shape[1] - feats.shape[1]))    # see conv3d._weights_for
-    df = _pick_dataflow(km, dataflow, in_channel, out_channel, feats.dtype, transposed)
+    # the selector sees the width the kernels run at (a 3- or 4-channel input layer runs padded to 16)
+    df = _pick_dataflow(km, dataflow, feats.shape[1], out_channel, feats.dtype, transposed)
     out = backend.conv_forward(feats, kernel.detach(), km, df, transposed=transposed, buffer=input.buffer, packed=packed,
                                out=out, bias=bias, residual=residual, act=act)
     if layer_log is not None:
