@@ -19,12 +19,15 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 
 
-def layer_records(forward, graph_ms):
+def layer_records(forward, graph_ms, regret=True):
     """One record per distinct convolution of a network forward (fp16): the call's shapes and dataflow, its time
     (10 calls captured into a HIP graph, median of 5 replays), and what that time means against the two roofs --
     the layer's algorithmic bytes (input rows, output rows, residual rows, weights, the pair list) per second
     against the HBM peak, its multiply-accumulates against the dense fp16 MFMA peak.  `n` = how many layers of
-    the forward have exactly this shape."""
+    the forward have exactly this shape.  With `regret`, every convolution is also timed in each other dataflow
+    that takes it and can be captured (output-stationary, ordered output-stationary, deferred scatter,
+    gather-GEMM-scatter; atomic fetch-on-demand allocates its accumulator and is left out): `by_dataflow_ms`,
+    `best` and `regret` = picked time / best time."""
     import torch
     from pcengine_amd import backend
     calls = []
@@ -73,7 +76,45 @@ def layer_records(forward, graph_ms):
                         "dataflow": names[flow], "residual": res, "n": 1, "ms": round(ms, 5),
                         "GBs": round(nbytes / ms / 1e6, 1), "hbm_frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 3),
                         "TFLOPs": round(flops / ms / 1e9, 1), "mfma_frac": round(flops / ms / 1e9 / 2500.0, 3)}
+        if regret and kind == "conv":
+            tr = bool(kw.get("transposed", False))
+            by = {names[flow]: ms}
+            for other in (backend.DATAFLOW_OS, backend.DATAFLOW_FDS, backend.DATAFLOW_OSO, backend.DATAFLOW_GMS):
+                if other == flow or (other == backend.DATAFLOW_OSO and not backend.oso_takes(km, c_in, c_out, feats.dtype, tr)):
+                    continue
+                kw2 = dict(kw)
+                if other == backend.DATAFLOW_GMS:       # stores dense rows: give it its own output and staging buffer
+                    kw2["out"] = None
+                    kw2["buffer"] = torch.empty(max(km.qsum * (c_in + c_out), 1), dtype=feats.dtype, device=feats.device)
+                    o2 = torch.empty((n_out, c_out), dtype=feats.dtype, device=feats.device)
+                    kw2["out"] = o2
+                elif kw2.get("buffer") is None and other == backend.DATAFLOW_FDS:
+                    kw2["buffer"] = torch.empty(max(km.M * c_out, 1), dtype=feats.dtype, device=feats.device)
+                if kw2.get("out") is None:
+                    kw2["out"] = torch.empty((n_out, c_out), dtype=feats.dtype, device=feats.device)
+                try:
+                    by[names[other]] = graph_ms(lambda: real_conv(feats, weight, km, other, **kw2), 10, 2, replays=3)[0]
+                except Exception as exc:      # a dataflow that does not take the layer (or cannot be captured) is no candidate
+                    print(f"bench.py: {what} {c_in}->{c_out} in {names[other]}: {exc}", file=sys.stderr)
+            best = min(by, key=by.get)
+            records[key].update({"by_dataflow_ms": {k: round(v, 5) for k, v in by.items()}, "best": best,
+                                 "regret": round(ms / by[best], 3)})
     return list(records.values())
+
+
+def regret_summary(records):
+    """Selector regret over the distinct convolutions of a network: the worst layer, and the whole forward's
+    convolution time as picked against the same with every layer in its best dataflow."""
+    rs = [r for r in records if "regret" in r]
+    if not rs:
+        return None
+    picked = sum(r["ms"] * r["n"] for r in rs)
+    best = sum(min(r["by_dataflow_ms"].values()) * r["n"] for r in rs)
+    worst = max(rs, key=lambda r: r["regret"])
+    return {"layers": len(rs), "max": worst["regret"],
+            "max_at": f'{worst["layer"]} {worst["c_in"]}->{worst["c_out"]} rows {worst["n_out"]} pairs {worst["pairs"]}: '
+                      f'{worst["dataflow"]} picked, {worst["best"]} best',
+            "time_weighted": round(picked / best, 4), "picked_ms": round(picked, 4), "best_ms": round(best, 4)}
 
 
 def main() -> int:
@@ -147,15 +188,20 @@ def main() -> int:
         return a.elapsed_time(b) / steps
 
     REPLAYS = 11
+    MIN_GRAPH_CALLS = 200
 
-    def graph_ms(fn, steps, warmup, replays=REPLAYS, spread=None):
+    def graph_ms(fn, steps, warmup, replays=REPLAYS, spread=None, min_calls=0):
         """`steps` calls captured into one HIP graph; the graph is replayed `replays` times, each replay
         between its own pair of HIP events on the current stream (the stream the kernels are launched on);
-        the figure is the median replay divided by `steps` (`spread` receives min / median / max).  Two or
-        three launches of 5-15 us each are otherwise paced by the host."""
+        the figure is the median replay divided by the calls in the graph (`spread` receives min / median /
+        max).  Two or three launches of 5-15 us each are otherwise paced by the host.  With `min_calls` the
+        `steps` calls are repeated inside the graph until it holds at least that many: the cost of launching
+        a graph (about 20 us) is then spread over as many kernels whatever `steps` is."""
         for _ in range(warmup):
             fn()
         torch.cuda.synchronize()
+        if min_calls > steps:
+            steps *= -(-min_calls // steps)
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
             for _ in range(steps):
@@ -172,7 +218,8 @@ def main() -> int:
             times.append(a.elapsed_time(b) / steps)
         times.sort()
         if spread is not None:
-            spread.update({"min": times[0], "median": times[len(times) // 2], "max": times[-1], "replays": replays})
+            spread.update({"min": times[0], "median": times[len(times) // 2], "max": times[-1], "replays": replays,
+                           "steps_per_graph": steps})
         return times[len(times) // 2], g
 
     # ---- kernel map (built once, reused by every step; timed separately) -----------------------
@@ -222,7 +269,7 @@ def main() -> int:
     launch = "hip_graph"
     spread = {}
     try:
-        ms, graph = graph_ms(step, args.steps, args.warmup, spread=spread)
+        ms, graph = graph_ms(step, args.steps, args.warmup, spread=spread, min_calls=MIN_GRAPH_CALLS)
         for _ in range(3):
             out_buf.zero_()
             step(DATAFLOW_OS)
@@ -235,7 +282,33 @@ def main() -> int:
     except Exception as exc:     # capture not possible: report the eager figure
         print(f"bench.py: HIP graph capture failed ({exc}); timing eager launches", file=sys.stderr)
         launch, ms = "eager", eager_ms
-        timer = lambda fn, steps, warmup: (ev_ms(fn, steps, warmup), None)
+        timer = lambda fn, steps, warmup, **kw: (ev_ms(fn, steps, warmup), None)
+
+    # The same step with nothing left in the 256 MB last-level cache from the step before: twelve pairs of
+    # (feature tensor, output tensor), 460 MB together, taken in turn inside one graph.  Between graph replays of
+    # the single pair above, the 38 MB of the layer never leave that cache; a layer inside a network sees
+    # something in between.  The map, the row order and the weights are shared by all pairs, as the layers of
+    # one level of a network share them.
+    cold = None
+    if args.workload == "cfg2" and launch == "hip_graph":
+        pairs = 12
+        ins = [fd.clone() for _ in range(pairs)]
+        outs = [torch.empty_like(out_buf) for _ in range(pairs)]
+        turn = [0]
+
+        def cold_step():
+            i = turn[0] % pairs
+            turn[0] += 1
+            backend.conv_forward(ins[i], wd, km, flow, buffer=buffer, packed=packed, out=outs[i])
+        turn[0] = 0
+        cold_spread = {}
+        cold_ms = graph_ms(cold_step, 20 * pairs, 0, spread=cold_spread)[0]
+        if not all(torch.equal(o, want) for o in outs):
+            raise RuntimeError("a step over rotated buffers disagrees with the eager result")
+        cold = {"ms_per_step": round(cold_ms, 5), "buffer_pairs": pairs,
+                "working_set_MB": round(pairs * (fd.numel() + out_buf.numel()) * 2 / 1e6, 1),
+                "min": round(cold_spread["min"], 5), "max": round(cold_spread["max"], 5)}
+        del ins, outs
 
     # calibration for hardware counters: a plain copy of known size (2 x 19.2 MB) runs three times, so
     # that a counter run can scale FETCH_SIZE / WRITE_SIZE by what they read for it
@@ -257,7 +330,7 @@ def main() -> int:
         with _lib.measurement_build() as mlib:
             for bit, name in stage_names.items():
                 mlib.pce_set_stage_mask((1 << bit) | 0xFFFFFFF0)   # bits 4 and up keep the kernel selection of the full run
-                stages[name] = timer(step, max(20, args.steps // 4), 5)[0]
+                stages[name] = timer(step, max(20, args.steps // 4), 5, min_calls=MIN_GRAPH_CALLS)[0]
     else:
         stages[stage_names[1]] = ms       # one kernel is the whole layer
     takes = lambda f: f != DATAFLOW_OSO or backend.oso_takes(km, c_in, c_out, torch.float16)
@@ -271,11 +344,12 @@ def main() -> int:
     floors = {}
     if c_in == c_out:
         dst = torch.empty_like(fd)
-        floors["device_copy_ms"] = timer(lambda: dst.copy_(fd), max(20, args.steps // 4), 5)[0]
+        floors["device_copy_ms"] = timer(lambda: dst.copy_(fd), max(20, args.steps // 4), 5, min_calls=MIN_GRAPH_CALLS)[0]
         del dst
     w_mid = wd[13].contiguous()
     pk_mid = backend.pack_weights(w_mid)
-    floors["centre_gemm_only_ms"] = timer(lambda: backend.dense_forward(fd, w_mid, packed=pk_mid), max(20, args.steps // 4), 5)[0]
+    floors["centre_gemm_only_ms"] = timer(lambda: backend.dense_forward(fd, w_mid, packed=pk_mid), max(20, args.steps // 4), 5,
+                                          min_calls=MIN_GRAPH_CALLS)[0]
 
     # algorithmic bytes of the layer: every tensor once + the pair list
     b_conv = n * c_in * e + n * c_out * e + 27 * c_in * c_out * e + 8 * M
@@ -323,6 +397,12 @@ def main() -> int:
                     "layer_bytes": b_conv, "layer_GBs": round(b_conv / (ms * 1e-3) / 1e9, 1),
                     "layer_frac": round(b_conv / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                     "layer_TFLOPs": round(flops / (ms * 1e-3) / 1e12, 2)}
+        if cold is not None:
+            # the same two fractions on the step over rotated buffers (one kernel is the layer, so the step is the
+            # kernel when the ordered dataflow runs)
+            cold["layer_frac"] = round(b_conv / (cold["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+            if len(stages) == 1:
+                cold["frac"] = round(dom_bytes / (cold["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
     else:
         # flops of the dominant kernel alone: the pair products for the pair-tile kernel, everything for the
         # single-kernel output-stationary dataflow
@@ -341,7 +421,8 @@ def main() -> int:
         "config": {"workload": what.format(n=n, M=M), "dataflow": names[flow], "selector": args.dataflow == "auto",
                    "launch": launch},
         "roofline": roofline,
-        "extra": {"ms_per_step_replays": {k: (round(v, 5) if k != "replays" else v) for k, v in spread.items()},
+        "extra": {"ms_per_step_replays": {k: (round(v, 5) if k not in ("replays", "steps_per_graph") else v) for k, v in spread.items()},
+                  **({"cold_ms_per_step": cold["ms_per_step"], "cold": cold} if cold is not None else {}),
                   "eager_ms_per_step": round(eager_ms, 5), "eager_wall_ms_per_step": round(wall_ms, 5),
                   "map_build_ms": round(map_ms, 4), "map_build_hash_table_ms": round(map_hash_ms, 4),
                   "map_build_neighbour_table_and_order_only_ms": round(map_table_only_ms, 4),
@@ -405,7 +486,9 @@ def main() -> int:
                                             "all_fetch_on_demand": net["fod"], "all_gather_gemm_scatter": net["gms"]}
         if not args.no_layers:
             y0 = forward()
-            result["extra"]["cfg4_minkunet"]["layers"] = layer_records(lambda: forward(y0), graph_ms)
+            recs4 = layer_records(lambda: forward(y0), graph_ms)
+            result["extra"]["cfg4_minkunet"]["layers"] = recs4
+            result["extra"].setdefault("selector_regret", {})["cfg4"] = regret_summary(recs4)
         # the same network in training mode (BatchNorm on batch statistics, cross-entropy on random labels):
         # forward + backward with kernel maps built every step, fp16 features and fp32 parameters
         torch.manual_seed(5)
@@ -495,6 +578,10 @@ def main() -> int:
         result["extra"]["cfg5"] = {"voxels": int(len(c5)), "scenes": 8, "dtype": "f16",
                                    "forward_ms_with_map_build": round(ev_ms(forward5, 5, 1), 3),
                                    "forward_ms_cached_maps": round(ev_ms(lambda: forward5(y5), 10, 2), 3)}
+        if not args.no_layers:
+            recs5 = layer_records(lambda: forward5(y5), graph_ms)
+            result["extra"]["cfg5"]["layers"] = recs5
+            result["extra"].setdefault("selector_regret", {})["cfg5"] = regret_summary(recs5)
         del model5, y5, f5, c5d
 
     # ---- CPU baseline: the oracle's torch path on this box's host cores, same workload ---------
@@ -513,6 +600,8 @@ def main() -> int:
                                             "median of 10 runs after 3 warm-ups; map build timed separately",
                                   "map_build_ms": round(cpu_map_ms, 3), "host_cpus": os.cpu_count()}
         result["extra"]["rel_l2_vs_cpu"] = float(orc.rel_l2(gpu_out, cpu_out))
+        if not result["extra"]["rel_l2_vs_cpu"] <= 1e-3:
+            raise RuntimeError(f"the timed layer is {result['extra']['rel_l2_vs_cpu']:.3e} (rel-L2) away from the CPU path: bar 1e-3")
     print(json.dumps(result))
     return 0
 

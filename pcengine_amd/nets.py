@@ -126,8 +126,8 @@ class SparseResUNet(nn.Module):
     def _skips_in_place(self, x: spTensor) -> bool:
         """Inference with every norm folded, on the GPU, all widths multiples of 8 channels: the two producers of
         a skip connection can then write their halves of the concatenated matrix themselves."""
-        if torch.is_grad_enabled() and any(p.requires_grad for p in self.parameters()):
-            return False
+        if torch.is_grad_enabled() and (x.feats.requires_grad or any(p.requires_grad for p in self.parameters())):
+            return False        # autograd results are fresh tensors: nothing can be written in place
         if not x.feats.is_cuda:
             return False
         ok = getattr(self, "_in_place_ok", None)

@@ -127,7 +127,7 @@ class conv3d(nn.Module):
                              kernel_size_code=self.kernel_size_code, stride_code=self.stride_code,
                              padding_code=self.padding_code, bias=self.bias, transposed=self.transposed,
                              tensorcore=self.tensorcore, dataflow=self.dataflow, packed=None, act=act,
-                             residual=None if residual is None else residual.feats)
+                             residual=None if residual is None else residual.feats, out=out)
         w, packed = self._weights_for(input.feats.dtype)
         return conv_func(input=input, in_channel=self.in_channels, out_channel=self.out_channels, kernel=w,
                          kernel_size_code=self.kernel_size_code, stride_code=self.stride_code,
@@ -202,6 +202,14 @@ def _wants_grad(*tensors) -> bool:
     return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
 
 
+def _no_out_with_grad(out) -> None:
+    """``out=`` names memory the kernels write in place; a result autograd has to track is a fresh tensor, so
+    the combination is refused instead of leaving ``out`` unwritten."""
+    if out is not None:
+        raise ValueError("conv3d: out= is for inference; features or parameters that require grad (with grad enabled) "
+                         "produce a new tensor -- call under torch.no_grad() or drop out=")
+
+
 def _apply_unfused(out: torch.Tensor, residual, act) -> torch.Tensor:
     """Residual and activation as differentiable torch ops (the training path does not fuse them)."""
     if residual is not None:
@@ -219,6 +227,7 @@ def _run(input: spTensor, km: backend.KernelMap, kernel, in_channel, out_channel
          bias=None, residual=None, act=None, out=None) -> torch.Tensor:
     feats = input.feats
     if _wants_grad(feats, kernel, bias):
+        _no_out_with_grad(out)
         k = kernel if kernel.dtype == feats.dtype else kernel.to(feats.dtype)
         b = bias if bias is None or bias.dtype == feats.dtype else bias.to(feats.dtype)
         df = _pick_dataflow(km, dataflow, in_channel, out_channel, feats.dtype, transposed)
@@ -404,6 +413,7 @@ def conv_func(input: spTensor, in_channel, out_channel, kernel, kernel_size_code
     if kernel_size_code == _UNIT and stride_code == _UNIT:
         # 1x1 stride 1: plain matrix product, coordinates unchanged, no map (script/spconv.py:297-304)
         if _wants_grad(input.feats, kernel, bias):
+            _no_out_with_grad(out)
             k = kernel if kernel.dtype == input.feats.dtype else kernel.to(input.feats.dtype)
             b = bias if bias is None or bias.dtype == input.feats.dtype else bias.to(input.feats.dtype)
             return input._like(_apply_unfused(_DenseFunction.apply(input.feats, k, b), residual, act))

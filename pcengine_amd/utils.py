@@ -127,55 +127,64 @@ class _Concat2(torch.autograd.Function):
         return grad[:, :ctx.split], grad[:, ctx.split:]
 
 
+def _as_tensor(v):
+    return torch.from_numpy(v) if isinstance(v, np.ndarray) else v
+
+
 def sparse_collate(inputs: List[spTensor]) -> spTensor:
-    """Stack samples, batch index in coordinate column 0 (script/utils.py:167-196)."""
-    coords, feats = [], []
+    """Samples stacked into one batch: sample ``k`` contributes its rows with ``k`` prepended as coordinate column 0,
+    in the order given; numpy members are converted (and left converted on the sample, as the reference leaves
+    them); all samples must share one tensor stride.  The batch's box is [0, max of the spatial columns]
+    (behaviour of script/utils.py:167-196)."""
+    if len(inputs) == 0:
+        raise ValueError("sparse_collate needs at least one sample")
     stride = inputs[0].stride
-    for k, x in enumerate(inputs):
-        if isinstance(x.coords, np.ndarray):
-            x.coords = torch.tensor(x.coords)
-        if isinstance(x.feats, np.ndarray):
-            x.feats = torch.tensor(x.feats)
-        assert isinstance(x.coords, torch.Tensor), type(x.coords)
-        assert isinstance(x.feats, torch.Tensor), type(x.feats)
-        assert x.stride == stride, (x.stride, stride)
-        b = torch.full((x.coords.shape[0], 1), k, device=x.coords.device, dtype=torch.int)
-        coords.append(torch.cat((b, x.coords.int()), dim=1))
-        feats.append(x.feats)
-    coords = torch.cat(coords, dim=0)
-    feats = torch.cat(feats, dim=0)
-    cmax = coords[:, 1:].max(dim=0).values.cpu().numpy().tolist()
+    sizes = []
+    for sample in inputs:
+        sample.coords, sample.feats = _as_tensor(sample.coords), _as_tensor(sample.feats)
+        for member in (sample.coords, sample.feats):
+            if not isinstance(member, torch.Tensor):
+                raise AssertionError(type(member))
+        if sample.stride != stride:
+            raise AssertionError((sample.stride, stride))
+        sizes.append(sample.coords.shape[0])
+    spatial = torch.cat([sample.coords.int() for sample in inputs], dim=0)
+    index = torch.repeat_interleave(torch.arange(len(inputs), dtype=torch.int32, device=spatial.device),
+                                    torch.tensor(sizes, device=spatial.device))
+    coords = torch.cat((index.unsqueeze(1), spatial), dim=1)
+    feats = torch.cat([sample.feats for sample in inputs], dim=0)
+    upper = [int(v) for v in spatial.amax(dim=0).tolist()]
     return spTensor(coords=coords, feats=feats, stride=stride, batchsize=len(inputs), buffer=None,
-                    coords_min=[0, 0, 0], coords_max=cmax)
+                    coords_min=[0, 0, 0], coords_max=upper)
 
 
 def sparse_collate_fn(inputs: List[Any]) -> Any:
-    """script/utils.py:199-217."""
-    if not isinstance(inputs[0], dict):
+    """Collate function for a data loader whose samples are dictionaries: per key, nested dictionaries recurse,
+    arrays and tensors are concatenated along rows, sparse tensors go through ``sparse_collate``, anything else
+    stays a list; samples that are not dictionaries are returned as they came (behaviour of script/utils.py:199-217)."""
+    head = inputs[0]
+    if not isinstance(head, dict):
         return inputs
-    out = {}
-    for name, first in inputs[0].items():
-        vals = [x[name] for x in inputs]
-        if isinstance(first, dict):
-            out[name] = sparse_collate_fn(vals)
-        elif isinstance(first, np.ndarray):
-            out[name] = torch.cat([torch.tensor(v) for v in vals], dim=0)
-        elif isinstance(first, torch.Tensor):
-            out[name] = torch.cat(vals, dim=0)
-        elif isinstance(first, spTensor):
-            out[name] = sparse_collate(vals)
-        else:
-            out[name] = vals
-    return out
+    joiners = ((dict, sparse_collate_fn),
+               (np.ndarray, lambda vals: torch.cat([torch.from_numpy(v) for v in vals], dim=0)),
+               (torch.Tensor, lambda vals: torch.cat(vals, dim=0)),
+               (spTensor, sparse_collate))
+    batch = {}
+    for key, first in head.items():
+        column = [sample[key] for sample in inputs]
+        join = next((fn for kind, fn in joiners if isinstance(first, kind)), None)
+        batch[key] = column if join is None else join(column)
+    return batch
 
 
 def make_ntuple(x, ndim: int) -> Tuple[int, ...]:
-    """script/utils.py:220-230."""
+    """``x`` as a tuple of ``ndim`` entries: an int is repeated, a list or a tensor is spread out; anything that
+    does not end up with ``ndim`` entries fails the assertion (behaviour of script/utils.py:220-230)."""
+    if isinstance(x, torch.Tensor):
+        x = x.reshape(-1).tolist()
     if isinstance(x, int):
-        x = tuple(repeat(x, ndim))
+        x = (x,) * ndim
     elif isinstance(x, list):
         x = tuple(x)
-    elif isinstance(x, torch.Tensor):
-        x = tuple(x.view(-1).cpu().numpy().tolist())
     assert isinstance(x, tuple) and len(x) == ndim, x
     return x

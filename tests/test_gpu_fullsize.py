@@ -29,9 +29,15 @@ def test_config3_down_then_transposed_up_full_size():
     mid_want = orc.conv_forward(rounded(f, dt), rounded(w_down, dt), ref, ks)
     fd = torch.as_tensor(f, device=DEV).to(dt)
     wd, wu = (torch.as_tensor(w, device=DEV).to(dt) for w in (w_down, w_up))
-    for flow in FLOWS:
+    # the selector's picks (the K-stepped ordered form for the down layer) run beside the forced dataflows
+    picked_down = backend.select_dataflow(km, 64, 128, dt)
+    picked_up = backend.select_dataflow(km, 128, 64, dt, transposed=True)
+    assert picked_down == backend.DATAFLOW_OSO
+    for flow in FLOWS + [backend.DATAFLOW_OSO]:
         mid = backend.conv_forward(fd, wd, km, flow)
         assert orc.rel_l2(mid.double().cpu().numpy(), mid_want) <= 1e-3, flow
+        if flow == backend.DATAFLOW_OSO:
+            flow = picked_up        # the ordered form has no transposed layer: the selector's pick runs instead
         # the transposed layer sees the fp16 rows the down layer stored
         up_want = orc.conv_forward(mid.double().cpu().numpy(), rounded(w_up, dt), ref, ks, transposed=True)
         up = backend.conv_forward(mid, wu, km, flow, transposed=True)

@@ -6,6 +6,7 @@ import pytest
 import torch
 
 import pcengine_amd as pe
+from oracle import oracle as orc
 from pcengine_amd import _lib, backend, nets, synth
 from pcengine_amd.backend import DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS, DATAFLOW_FDS
 from tests.util import DEV, dev_coords
@@ -109,6 +110,37 @@ def test_network_concatenates_in_place(monkeypatch):
     x = pe.spTensor(torch.as_tensor(synth.features(4, len(small), 4), device=DEV).float(), dev_coords(small), None, [0, 0, 0],
                     small[:, 1:].max(0).tolist())
     assert not plain._skips_in_place(x)
+
+
+def test_frozen_network_with_input_gradients_keeps_the_copying_forward():
+    """Frozen parameters, grad enabled, input features that require grad (an input-saliency pass over a fused model):
+    autograd results are fresh tensors, so nothing may be written in place -- the network takes the concatenating
+    forward, returns what the plain forward returns and carries the gradient to the input; a layer asked to write
+    ``out=`` on that path refuses."""
+    coords = synth.random_cloud(seed=85, n=4000, extent=26)
+    cd = dev_coords(coords)
+    cmax = coords[:, 1:].max(0).tolist()
+    torch.manual_seed(6)
+    model = nets.SparseResUNet(4, 20, stem=16, enc=(16, 32, 48, 64), dec=(64, 48, 24, 24)).to(DEV).eval().fuse_bn()
+    for p in model.parameters():
+        p.requires_grad_(False)
+    f = torch.as_tensor(synth.features(4, len(coords), 4), device=DEV).float()
+    with torch.no_grad():
+        x0 = pe.spTensor(f, cd, None, [0, 0, 0], cmax)
+        assert model._skips_in_place(x0)
+        want = model(x0).feats
+    fg = f.clone().requires_grad_(True)
+    x = pe.spTensor(fg, cd, None, [0, 0, 0], cmax)
+    assert not model._skips_in_place(x)
+    y = model(x).feats
+    assert orc.rel_l2(y.detach().double().cpu().numpy(), want.double().cpu().numpy()) <= 1e-5
+    y.square().sum().backward()
+    assert fg.grad is not None and bool(torch.isfinite(fg.grad).all()) and float(fg.grad.abs().max()) > 0
+    layer = pe.conv3d(4, 16, 3).to(DEV)
+    for p in layer.parameters():
+        p.requires_grad_(False)
+    with pytest.raises(ValueError, match="out="):
+        layer(pe.spTensor(fg, cd, None, [0, 0, 0], cmax), out=torch.empty((len(coords), 16), device=DEV))
 
 
 def test_row_strides_are_refused_where_rows_must_be_dense():

@@ -153,6 +153,33 @@ def test_quantize_and_collate():
     z = x + x
     assert torch.equal(z.feats, x.feats * 2) and z.kmaps is x.kmaps
     assert x.F is x.feats and x.C is x.coords and x.stride == 94585
+    # rows keep their order, sample k carries k in column 0, numpy members are converted
+    assert torch.equal(x.coords[:len(q), 1:], torch.as_tensor(q)) and int(x.coords[:len(q), 0].max()) == 0
+    assert torch.equal(x.coords[len(q):, 1:], torch.as_tensor(q[:5])) and int(x.coords[len(q):, 0].min()) == 1
+    n1 = pe.spTensor(np.ones((4, 2), np.float32), q[:4].copy(), None, [0, 0, 0], [9, 9, 9])
+    n2 = pe.spTensor(np.ones((3, 2), np.float32), q[:3].copy(), None, [0, 0, 0], [9, 9, 9])
+    xn = pe.sparse_collate([n1, n2])
+    assert isinstance(n1.coords, torch.Tensor) and xn.feats.shape == (7, 2) and xn.coords[:, 0].tolist() == [0] * 4 + [1] * 3
+    odd = pe.spTensor(torch.ones(2, 3), torch.as_tensor(q[:2]), None, [0, 0, 0], [9, 9, 9], stride=94273 * 2 + 311 * 2 + 2)
+    with pytest.raises(AssertionError):
+        pe.sparse_collate([a, odd])
+
+
+def test_collate_fn_and_ntuple():
+    from pcengine_amd.utils import make_ntuple, sparse_collate_fn
+    q = np.arange(12, dtype=np.int32).reshape(4, 3)
+    mk = lambda k: pe.spTensor(torch.full((k, 2), float(k)), torch.as_tensor(q[:k]), None, [0, 0, 0], [11, 11, 11])
+    samples = [{"pc": mk(2), "label": np.array([1, 2]), "t": torch.zeros(2), "name": "a", "nest": {"v": np.array([5])}},
+               {"pc": mk(3), "label": np.array([3, 4, 5]), "t": torch.ones(3), "name": "b", "nest": {"v": np.array([6])}}]
+    out = sparse_collate_fn(samples)
+    assert isinstance(out["pc"], pe.spTensor) and out["pc"].coords.shape == (5, 4) and out["pc"].batchsize == 2
+    assert out["label"].tolist() == [1, 2, 3, 4, 5] and out["t"].tolist() == [0, 0, 1, 1, 1]
+    assert out["name"] == ["a", "b"] and out["nest"]["v"].tolist() == [5, 6]
+    assert sparse_collate_fn([1, 2]) == [1, 2]
+    assert make_ntuple(3, 3) == (3, 3, 3) and make_ntuple([1, 2, 3], 3) == (1, 2, 3)
+    assert make_ntuple(torch.tensor([[2, 2, 2]]), 3) == (2, 2, 2) and make_ntuple((4, 5), 2) == (4, 5)
+    with pytest.raises(AssertionError):
+        make_ntuple([1, 2], 3)
 
 
 def test_module_construction_and_errors():
@@ -259,3 +286,82 @@ def test_no_kernel_uses_scratch_memory(tmp_path):
                         assert int(m.group(1)) <= limit, f"{name} holds {m.group(1)} vector registers, limit {limit}"
                         ceilings_seen.add(prefix)
     assert seen > 20 and ceilings_seen == {p for p, _ in _VGPR_CEILINGS}
+
+
+def _function_bodies(src):
+    """(name, is_kernel, body) of every __global__ / __device__ function of a HIP source, by brace matching."""
+    def closing(text, i, open_ch, close_ch):
+        depth = 0
+        while True:
+            depth += {open_ch: 1, close_ch: -1}.get(text[i], 0)
+            if depth == 0:
+                return i
+            i += 1
+    out = []
+    for m in re.finditer(r"__global__\s+void\s+|__device__\s+(?:__forceinline__\s+)?[\w:<>,\s\*&]*?(?=\b\w+\s*\()", src):
+        i = m.end()
+        if src.startswith("__launch_bounds__", i):
+            i = closing(src, src.index("(", i), "(", ")") + 1
+        nm = re.match(r"\s*(\w+)\s*\(", src[i:])
+        if not nm:
+            continue
+        args_end = closing(src, i + nm.end() - 1, "(", ")")
+        rest = src[args_end + 1:]
+        if not rest.lstrip().startswith("{"):
+            continue
+        start = args_end + 1 + rest.index("{")
+        out.append((nm.group(1), src[m.start():m.start() + 10] == "__global__", src[start:closing(src, start, "{", "}") + 1]))
+    return out
+
+
+def test_every_global_to_lds_copy_is_followed_by_a_hand_written_wait():
+    """The compiler neither tracks nor reliably waits for global -> LDS copies (`global_load_lds`): a read of the
+    copied region must stand behind a hand-written `s_waitcnt vmcnt`.  Checked on the text: in a kernel that
+    issues such a copy itself, the next mention of the destination array after the copy comes after a wait; a
+    helper that issues copies is only called from kernels that also call one of the waiting helpers."""
+    src = open(os.path.join(ROOT, "pcengine_amd", "csrc", "pce_conv.hip")).read()
+    src = re.sub(r"//[^\n]*", "", src)
+    bodies = _function_bodies(src)
+    copy = "__builtin_amdgcn_global_load_lds"
+    wait = re.compile(r"s_waitcnt vmcnt\(")
+    waiting_helpers = [n for n, k, b in bodies if not k and wait.search(b)]
+    assert "pipe_wait_copy" in waiting_helpers
+    grew = True
+    while grew:       # helpers that wait through another helper
+        more = [n for n, k, b in bodies if not k and n not in waiting_helpers
+                and any(re.search(r"\b" + h + r"\b", b) for h in waiting_helpers)]
+        waiting_helpers += more
+        grew = bool(more)
+    copying_helpers = [n for n, k, b in bodies if not k and copy in b]
+    sites = 0
+    for name, is_kernel, body in bodies:
+        if not is_kernel:
+            continue
+        if copy in body:
+            for m in re.finditer(re.escape(copy) + r"\(", body):
+                depth, j = 1, m.end()
+                while depth:
+                    depth += {"(": 1, ")": -1}.get(body[j], 0)
+                    j += 1
+                dest = re.search(r"&\s*(\w+)\s*\[", body[m.end():j])
+                assert dest, f"{name}: no LDS destination found in a global -> LDS copy"
+                sites += 1
+                rest = body[j:]
+                # skip further copies into the same array (their destination operand is a mention too)
+                use = None
+                for u in re.finditer(r"\b" + dest.group(1) + r"\s*\[", rest):
+                    before = rest[:u.start()]
+                    open_copy = before.rfind(copy)
+                    if open_copy >= 0 and before.count("(", open_copy) > before.count(")", open_copy):
+                        continue
+                    use = u
+                    break
+                if use is not None:
+                    assert wait.search(rest[:use.start()]), \
+                        f"{name}: {dest.group(1)} is read after a global -> LDS copy with no s_waitcnt vmcnt in between"
+        called = [h for h in copying_helpers if re.search(r"\b" + h + r"\s*(<[^;]*?>)?\s*\(", body)]
+        if called:
+            sites += 1
+            assert wait.search(body) or any(re.search(r"\b" + h + r"\b", body) for h in waiting_helpers), \
+                f"{name} copies global -> LDS through {called} and never waits by hand"
+    assert sites >= 6

@@ -383,3 +383,22 @@ def test_manifest_of_benchmark_inputs_is_reproduced(name):
     down = frozen[name]["layers"].get("k222_s222_p000")
     if down:
         assert down["pairs"] <= frozen[name]["voxels"] and down["n_out"] <= down["pairs"]
+
+
+@pytest.mark.parametrize("ks,stride,pad", [((3, 3, 3), (1, 1, 1), (0, 0, 0)), ((2, 2, 2), (2, 2, 2), (0, 0, 0)),
+                                           ((3, 3, 3), (2, 2, 2), (1, 1, 1))])
+def test_timed_cpu_path_computes_what_the_oracle_computes(ks, stride, pad):
+    """oracle/cpu_path.py is the torch form bench.py times as the CPU baseline; its values must be the
+    float64 oracle's (which the dense conv3d tests above pin) to fp32 rounding."""
+    from oracle import cpu_path
+    coords = synth.random_cloud(seed=77, n=3000, extent=16, batches=2)
+    kv = ks[0] * ks[1] * ks[2]
+    f = synth.features(7, len(coords), 24).astype(np.float32)
+    w = synth.weights(7, kv, 24, 40).astype(np.float32)
+    km = orc.kernel_map(coords, ks, stride, pad)
+    want = orc.conv_forward(f.astype(np.float64), w.astype(np.float64), km, ks)
+    got = cpu_path.conv_forward_torch(torch.as_tensor(f), torch.as_tensor(w), km, ks).numpy()
+    assert got.shape == want.shape and orc.rel_l2(got.astype(np.float64), want) <= 1e-6
+    if stride == (1, 1, 1):
+        m_ms, c_ms, out, km2 = cpu_path.time_layer(coords, f, w, ks, warmup=0, runs=1)
+        assert m_ms > 0 and c_ms > 0 and np.array_equal(km2.imap, km.imap) and np.array_equal(out, got)
