@@ -226,23 +226,29 @@ def main() -> int:
     n_batch = int(coords[:, 0].max()) + 1
 
     def build_ms(batchsize, want_csr=True):
-        """Wall time of one map build (CSR views and neighbour table included).  With the batch count stated the
-        sorted coordinates are indexed by column (what the front end does); without it they go through the hash table.
-        want_csr=False: the neighbour table, the counts and the row order only (what the output-stationary dataflows read)."""
+        """Wall time of one map build (median of 21, each from the call to the end of its work on the GPU).  With the
+        batch count stated the sorted coordinates are indexed by column (what the front end does); without it they go
+        through the hash table.  want_csr=True: pair lists, CSR views, neighbour table and row order; False: the
+        neighbour table, the counts and the row order only (what the output-stationary dataflows read)."""
         build = lambda: backend.build_kernel_map(cd, ks, (1, 1, 1), (0, 0, 0), [0, 0, 0], cmax, True, want_csr=want_csr,
-                                                 batchsize=batchsize)
+                                                 batchsize=batchsize, want_pairs=want_csr)
         km = build()
         for _ in range(3):
             build()
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(20):
+        times = []
+        for _ in range(21):
+            t0 = time.perf_counter()
             build()
-        torch.cuda.synchronize()
-        return km, (time.perf_counter() - t0) / 20 * 1e3
+            torch.cuda.synchronize()
+            times.append((time.perf_counter() - t0) * 1e3)
+        return km, sorted(times)[len(times) // 2]
     km_hash, map_hash_ms = build_ms(0)
     km, map_ms = build_ms(n_batch)
-    _, map_table_only_ms = build_ms(n_batch, want_csr=False)
+    km_table, map_table_only_ms = build_ms(n_batch, want_csr=False)
+    if not (torch.equal(km_table.nbr_out, km.nbr_out) and torch.equal(km_table.kpos, km.kpos) and km_table.M == km.M):
+        raise RuntimeError("the map built without pair lists and the full map differ")
+    del km_table
     if not (torch.equal(km.imap, km_hash.imap) and torch.equal(km.omap, km_hash.omap) and torch.equal(km.ocsr, km_hash.ocsr)):
         raise RuntimeError("the column-grid map and the hash-table map differ")
     del km_hash

@@ -202,16 +202,18 @@ typedef struct pce_kmap_problem {
   pce_geom_t geom;
   void *ws;
   int64_t ws_bytes;
-  int32_t *imap, *omap, *knnz, *kpos, *qkpos;
+  int32_t *imap, *omap, *knnz, *kpos, *qkpos; /* imap / omap may be NULL with PCE_KMAP_TABLE_ONLY over the column grid */
   int32_t *icsr, *icode, *ocsr, *ocode; /* all four or none */
   int32_t *islot, *oslot;               /* optional, with the CSR outputs */
   int32_t *nbr_out, *nbr_in;            /* optional */
-  int32_t *status;                      /* int32[4] per problem (int32[8] with `order`), zeroed by the caller */
+  int32_t *status;                      /* int32[8] per problem, zeroed by the caller: [0] coordinate out of range, [1] hash
+                                           table exhausted, [2] CSR code overflow, [3] column grid not applicable (see
+                                           below), [4] n_heavy of `order`, [5] 1 = no pair lists were written */
   int32_t n_batch;                      /* batch count (spTensor.batchsize), 0 = unknown: see the column grid below */
   int32_t flags;                        /* PCE_KMAP_* */
   int32_t *order;                       /* optional, needs nbr_out and kv <= 31: the row order of pce_row_order
-                                           (pce_row_order_elems(n_out) ints), built with the map at the cost of three
-                                           launches per batch; status[4] receives its n_heavy */
+                                           (pce_row_order_elems(n_out) ints, 16-byte aligned), built with the map at the
+                                           cost of three launches per batch; status[4] receives its n_heavy */
 } pce_kmap_problem_t;
 int pce_kmap_build_batch(const pce_kmap_problem_t *problems_host, int32_t n_problems, pce_stream_t stream);
 
@@ -225,6 +227,12 @@ int pce_kmap_build_batch(const pce_kmap_problem_t *problems_host, int32_t n_prob
  * inside the box and with b < n_batch; a build that finds otherwise sets status[3] and leaves its outputs
  * undefined: the caller runs it again with PCE_KMAP_NO_GRID.  Same maps, bit for bit, either way. */
 #define PCE_KMAP_NO_GRID 1
+/* The caller reads the neighbour table (nbr_out), the row order and the counts (knnz, kpos, qkpos) only -- what the
+ * output-stationary dataflows read -- and waives the pair lists: a 3x3x3 submanifold problem over the column grid
+ * without CSR outputs and without nbr_in then skips them (status[5] = 1: imap / omap are not written) and is four
+ * launches shorter; any other problem ignores the flag.  The reference always compacts its dense map into pair
+ * lists (script/spconv.py:370-372). */
+#define PCE_KMAP_TABLE_ONLY 2
 int64_t pce_kmap_workspace_bytes_grid(int64_t n_in, int64_t n_out, const pce_geom_t *g, int32_t n_batch,
                                       int32_t want_csr);
 

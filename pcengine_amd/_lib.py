@@ -18,6 +18,7 @@ PCE_F16, PCE_F32, PCE_F64 = 0, 1, 2
 DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS, DATAFLOW_FDS, DATAFLOW_OSO = 0, 1, 2, 3, 4
 QUANTUM = 128
 KMAP_NO_GRID = 1
+KMAP_TABLE_ONLY = 2
 CSR_CODE = 1186111
 
 

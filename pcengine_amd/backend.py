@@ -60,8 +60,9 @@ class _Cut:
     use (a network reads a few of the six arrays of each of its maps; cutting all of them up front is Python time
     the host spends before the first convolution is queued)."""
 
-    def __init__(self, optional: bool):
+    def __init__(self, optional: bool, pairs: bool = False):
         self.optional = optional
+        self.pairs = pairs       # a pair list: a map built without them (has_pairs False) builds them on first read
 
     def __set_name__(self, owner, name):
         self.slot = "_cut_" + name
@@ -71,6 +72,8 @@ class _Cut:
             if self.optional:
                 return None              # the dataclass default
             raise AttributeError         # a required field: no default
+        if self.pairs and not obj.__dict__.get("has_pairs", True):
+            ensure_pairs(obj)
         v = obj.__dict__.get(self.slot)
         if isinstance(v, tuple):         # (array at capacity, pair count)
             v = v[0][:v[1]]
@@ -98,8 +101,8 @@ class KernelMap:
     kv: int
     M: int
     qsum: int
-    imap: torch.Tensor = _Cut(False)
-    omap: torch.Tensor = _Cut(False)
+    imap: torch.Tensor = _Cut(False, pairs=True)
+    omap: torch.Tensor = _Cut(False, pairs=True)
     knnz: torch.Tensor
     kpos: torch.Tensor
     qkpos: torch.Tensor
@@ -122,6 +125,8 @@ class KernelMap:
     knnz_host: list = field(default_factory=list)
     kpos_host: object = None     # ctypes int32 arrays (kv+1) mirrored on the host by the map build's one read-back
     qkpos_host: object = None
+    has_pairs: bool = True       # False: built as neighbour table, row order and counts only (want_pairs=False)
+    batchsize: int = 0           # the batch count the build was given (0: none)
 
     @property
     def has_csr(self) -> bool:
@@ -265,7 +270,7 @@ class _MapJob:
     read-back of its counts."""
 
     def __init__(self, in_coords, ks, stride, pad, cmin, cmax_out, subm, want_csr, want_nbr_out, want_nbr_in,
-                 out_coords, batchsize, want_order=None):
+                 out_coords, batchsize, want_order=None, want_pairs=True):
         lib = _lib.load()
         _require_cuda(in_coords, "coords")
         if in_coords.dtype != torch.int32 or in_coords.dim() != 2 or in_coords.shape[1] != 4:
@@ -295,6 +300,10 @@ class _MapJob:
         # the batch count lets the library index sorted coordinates by column instead of hashing them; a build that
         # finds them unsorted, or outside the box the geometry states, is redone through the hash table (finish)
         self.n_batch, self.no_grid = max(int(batchsize), 0), False
+        # a caller that reads only the neighbour table, the row order and the counts (the output-stationary
+        # dataflows) waives the pair lists; the library then skips them where it can (3x3x3 submanifold map over the
+        # column grid) and says so in its status word 5
+        self.table_only = not want_pairs and not want_csr and want_nbr_out and not want_nbr_in
         self.ws_bytes = lib.pce_kmap_workspace_bytes_grid(n_in, n_out, geom, self.n_batch, int(want_csr))
         if self.ws_bytes < 0:
             _lib.check(_lib.PCE_EINVAL)
@@ -306,7 +315,7 @@ class _MapJob:
         if want_nbr_in:
             self.want.append(("nbr_in", kv * n_in))
         if self.want_order:
-            self.want.append(("order", 2 * n_out + 8192))
+            self.want.append(("order", lib.pce_row_order_elems(n_out)))
         if want_csr:
             self.want += [("icsr", n_in + 1), ("ocsr", n_out + 1), ("icode", cap), ("ocode", cap), ("islot", cap), ("oslot", cap)]
         self.ws = self.imap = self.omap = self.nbr_out = self.nbr_in = self.order = None
@@ -346,7 +355,8 @@ class _MapJob:
         p.islot, p.oslot = _ptr(self.islot), _ptr(self.oslot)
         p.nbr_out, p.nbr_in = _ptr(self.nbr_out), _ptr(self.nbr_in)
         p.status = status.data_ptr()
-        p.n_batch, p.flags = self.n_batch, (_lib.KMAP_NO_GRID if self.no_grid else 0)
+        p.n_batch = self.n_batch
+        p.flags = (_lib.KMAP_NO_GRID if self.no_grid else 0) | (_lib.KMAP_TABLE_ONLY if self.table_only else 0)
         p.order = _ptr(self.order)
         return p
 
@@ -371,7 +381,8 @@ class _MapJob:
                        qkpos=self.qkpos, out_coords=self.out_coords, nbr_out=self.nbr_out, nbr_in=self.nbr_in,
                        icsr=self.icsr, ocsr=self.ocsr, icode=cut(self.icode), ocode=cut(self.ocode),
                        islot=cut(self.islot), oslot=cut(self.oslot), in_coords=self.in_coords, geom=self.geom,
-                       knnz_host=host[:kv], order=self.order, order_heavy=st[4] if self.order is not None else 0)
+                       knnz_host=host[:kv], order=self.order, order_heavy=st[4] if self.order is not None else 0,
+                       has_pairs=not st[5], batchsize=self.n_batch)
         km._cmin, km._cmax = cmin, cmax_out
         km.kpos_host = (_lib.c_int32 * (kv + 1))(*host[kv:2 * kv + 1])
         km.qkpos_host = (_lib.c_int32 * (kv + 1))(*host[2 * kv + 1:3 * kv + 2])
@@ -383,11 +394,11 @@ KMAP_MAX_BATCH = 16
 
 def prepare_map(in_coords: torch.Tensor, ks, stride, pad, cmin, cmax_out, subm: bool, want_csr: bool = False,
                 want_nbr_out: bool = True, want_nbr_in: bool = False, out_coords: Optional[torch.Tensor] = None,
-                batchsize: int = 0, want_order: Optional[bool] = None) -> _MapJob:
+                batchsize: int = 0, want_order: Optional[bool] = None, want_pairs: bool = True) -> _MapJob:
     """First half of a map build: the output coordinates of a strided layer (``.out_coords``, final)
     and the output buffers.  ``build_kernel_maps`` takes the result in place of a request."""
     return _MapJob(in_coords, ks, stride, pad, cmin, cmax_out, subm, want_csr, want_nbr_out, want_nbr_in, out_coords,
-                   batchsize, want_order)
+                   batchsize, want_order, want_pairs)
 
 
 def build_kernel_maps(requests: List[dict], defer: bool = False):
@@ -439,16 +450,29 @@ def build_kernel_maps(requests: List[dict], defer: bool = False):
 def build_kernel_map(in_coords: torch.Tensor, ks, stride, pad, cmin, cmax_out, subm: bool,
                      want_csr: bool = False, want_nbr_out: bool = True, want_nbr_in: bool = False,
                      out_coords: Optional[torch.Tensor] = None, batchsize: int = 0, defer: bool = False,
-                     want_order: Optional[bool] = None):
+                     want_order: Optional[bool] = None, want_pairs: bool = True):
     """Hash the output coordinates, probe every (input row, offset) and emit the canonical map.
 
     ``cmax_out`` is the bound on output coordinates (already reduced for strided layers).
     ``defer=True`` returns a ``PendingMap`` instead of waiting for the pair counts: its output
     coordinates are final, ``finish()`` yields the ``KernelMap`` once the stream has been
-    synchronised."""
+    synchronised.  ``want_pairs=False``: the caller reads the neighbour table, the row order and the counts only
+    (``KernelMap.has_pairs`` tells whether the build skipped the pair lists; reading ``imap`` / ``omap`` of such a
+    map builds them then)."""
     return build_kernel_maps([dict(in_coords=in_coords, ks=ks, stride=stride, pad=pad, cmin=cmin, cmax_out=cmax_out,
                                    subm=subm, want_csr=want_csr, want_nbr_out=want_nbr_out, want_nbr_in=want_nbr_in,
-                                   out_coords=out_coords, batchsize=batchsize, want_order=want_order)], defer=defer)[0]
+                                   out_coords=out_coords, batchsize=batchsize, want_order=want_order,
+                                   want_pairs=want_pairs)], defer=defer)[0]
+
+
+def ensure_pairs(km: KernelMap) -> None:
+    """Pair lists of a map that was built without them (first use of a dataflow that reads them)."""
+    if km.has_pairs:
+        return
+    km.has_pairs = True          # before the build below reads anything of `km`
+    full = build_kernel_map(km.in_coords, km.ks, km.stride, km.pad, km._cmin, km._cmax, km.subm, want_csr=False,
+                            want_nbr_out=False, out_coords=km.out_coords, batchsize=km.batchsize)
+    km.imap, km.omap = full.imap, full.omap
 
 
 def ensure_csr(km: KernelMap) -> None:
@@ -459,6 +483,9 @@ def ensure_csr(km: KernelMap) -> None:
                             want_nbr_out=False, out_coords=km.out_coords)
     km.icsr, km.icode, km.ocsr, km.ocode = full.icsr, full.icode, full.ocsr, full.ocode
     km.islot, km.oslot = full.islot, full.oslot
+    if not km.has_pairs:
+        km.has_pairs = True
+        km.imap, km.omap = full.imap, full.omap
 
 
 def pair_route(km: KernelMap, transposed: bool = False) -> torch.Tensor:

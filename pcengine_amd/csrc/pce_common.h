@@ -77,11 +77,15 @@ __host__ __device__ static inline unsigned long long pce_home_slot(unsigned long
 
 // ---------------------------------------------------------------------------------------------
 // Row order of the ordered output-stationary dataflow (pce_row_order, pce_conv_fwd_oso):
-// order = perm[n_rows] | mask[n_rows] | tail[PCE_ORDER_TAIL].  The tail holds the histogram, the cursors and
-// the bases of the counting sort over ORDER_KEYS keys -- (lowest, second-lowest) offset of the rows with one or
-// two neighbours, then of the rows with more -- and the counts.
+// order = perm[n_rows] | mask[n_rows] | tail[PCE_ORDER_TAIL] | rec[n_rows] (int4, 16-byte aligned).  The tail holds
+// the histogram, the cursors and the bases of the counting sort over ORDER_KEYS keys -- (lowest, second-lowest)
+// offset of the rows with one or two neighbours, then of the rows with more -- and the counts.  rec[p], for the
+// positions p of rows that have a neighbour, repeats what a wavefront needs of the row at perm[p] in one 16-byte
+// load: {row, mask, neighbour at the lowest offset of the mask, neighbour at the second-lowest or -1}.
 // ---------------------------------------------------------------------------------------------
 #define PCE_ORDER_TAIL 8192
+#define PCE_ORDER_REC_OFFSET(n_rows) ((2 * (long long)(n_rows) + PCE_ORDER_TAIL + 3) & ~3ll)
+#define PCE_ORDER_ELEMS(n_rows) (PCE_ORDER_REC_OFFSET(n_rows) + 4 * (long long)(n_rows))
 #define ORDER_MAX_KV 32
 #define ORDER_KEYS 2048
 #define ORDER_HIST 0

@@ -1291,6 +1291,10 @@ static void kmap_layout(int64_t n_in, int64_t n_out, int kv, int want_csr, int s
   L->total = o;
 }
 
+#define PCE_GLOBAL __attribute__((address_space(1)))
+typedef int pce_v2i __attribute__((ext_vector_type(2)));
+typedef int pce_v4i __attribute__((ext_vector_type(4)));
+
 // device-side view of one problem of the batch
 struct ProbDev {
   const int4 *in_coords, *out_coords;
@@ -1302,6 +1306,8 @@ struct ProbDev {
   int *imap, *omap, *knnz, *kpos, *qkpos, *icsr, *icode, *ocsr, *ocode, *islot, *oslot, *nbr_out, *status;
   int *order;        // row order of the ordered output-stationary dataflow, or null
   int want_csr;
+  int fused;         // the probe wrote the output-major table (nbr_out), masks and counts itself: no probe table
+  int lazy;          // no pair lists: counts per offset only (knnz by atomics, kpos / qkpos from them)
   int use_grid;      // column grid instead of the hash table
   int2 *grid;        // [cells] = {first row of the column, row behind its last}, -1 for an empty column
   int *zcol;         // z of every table row
@@ -1546,10 +1552,12 @@ __global__ void __launch_bounds__(256) grid_query_kernel(const ProbDev *__restri
   for (int col0 = 0; col0 < ncol; col0 += GRID_BATCH) {
     int2 se[GRID_BATCH];
     int zz[GRID_BATCH][4];
+    long long cellj[GRID_BATCH];
 #pragma unroll
     for (int j = 0; j < GRID_BATCH; ++j) {
       const int col = col0 + j;
       se[j] = make_int2(-1, -1);
+      cellj[j] = -1;
       if (live && col < ncol) {
         const int ix = col / ksy, iy = col - ix * ksy;
         const int dx = ix - hx, dy = iy - hy;
@@ -1562,16 +1570,24 @@ __global__ void __launch_bounds__(256) grid_query_kernel(const ProbDev *__restri
           ok = strided_axis(c.y, dx, g.pad[0], g.stride[0], g.cmin[0], g.cmax[0], &tx);
           ok &= strided_axis(c.z, dy, g.pad[1], g.stride[1], g.cmin[1], g.cmax[1], &ty);
         }
-        const long long cell = ok ? grid_cell(q.box, c.x, tx, ty) : -1;
-        if (cell >= 0) se[j] = grid[cell];
+        cellj[j] = ok ? grid_cell(q.box, c.x, tx, ty) : -1;
       }
+    }
+    // every load goes out from a valid address and is masked afterwards: loads under a lane condition are compiled
+    // to branches with a wait each, one trip to memory after the other
+#pragma unroll
+    for (int j = 0; j < GRID_BATCH; ++j) {
+      const int2 v = grid[cellj[j] >= 0 ? cellj[j] : 0];
+      if (cellj[j] >= 0) se[j] = v;
     }
 #pragma unroll
     for (int j = 0; j < GRID_BATCH; ++j)
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
         const int r = se[j].x + t;
-        zz[j][t] = (se[j].x >= 0 && r < se[j].y) ? zcol[r] : (int)0x80000000;
+        const bool in = se[j].x >= 0 && r < se[j].y;
+        const int z = zcol[in ? r : 0];
+        zz[j][t] = in ? z : (int)0x80000000;
       }
 #pragma unroll
     for (int j = 0; j < GRID_BATCH; ++j) {
@@ -1678,7 +1694,10 @@ __device__ __forceinline__ void order_scan_block(int *tail, int *n_heavy_out) {
 
 // perm: the rows of one block of 256 (block `blk` of the map), placed as described above.  A block takes one range
 // per key it holds (one global atomic per key and block); its rows of a key keep the ranks LDS atomics gave them.
-__device__ __forceinline__ void order_scatter_block(long long n_rows, int *__restrict__ order, unsigned blk) {
+// `nbr` is the output-major neighbour table, or (mirror >= 0) the probe table of a symmetric map, whose row
+// mirror - k is the output-major row k: the table the same launch may still be writing is never read.
+__device__ __forceinline__ void order_scatter_block(long long n_rows, int *__restrict__ order, unsigned blk,
+                                                    const int *__restrict__ nbr, int mirror) {
   __shared__ int cnt[ORDER_KEYS], gbase[ORDER_KEYS];
   __shared__ int wcount[4], wbase;
   int *perm = order, *tail = order + 2 * n_rows;
@@ -1705,8 +1724,155 @@ __device__ __forceinline__ void order_scatter_block(long long n_rows, int *__res
     for (int w2 = 0; w2 < wave; ++w2) before += wcount[w2];
     perm[wbase + before] = (int)row;
   } else if (key >= 0) {
-    perm[n_plain + gbase[key] + rank] = (int)row;
+    const long long p = n_plain + gbase[key] + rank;
+    perm[p] = (int)row;
+    // the record of the row: what a wavefront of the ordered dataflow reads of it in one load
+    const int k1 = __ffs((int)m) - 1;
+    const unsigned rest = m & (m - 1u);
+    const int k2 = rest ? __ffs((int)rest) - 1 : -1;
+    int4 r;
+    r.x = (int)row;
+    r.y = (int)m;
+    r.z = nbr[(long long)(mirror >= 0 ? mirror - k1 : k1) * n_rows + row];
+    r.w = k2 >= 0 ? nbr[(long long)(mirror >= 0 ? mirror - k2 : k2) * n_rows + row] : -1;
+    reinterpret_cast<int4 *>(order + PCE_ORDER_REC_OFFSET(n_rows))[p] = r;
   }
+}
+
+// The 3x3x3 submanifold map over the column grid in one pass, output-major: lane o looks up all 26 neighbours of
+// its own row (nine cells; a probe of half the offsets with mirrored writes, as above, leaves a row's results
+// scattered over the lanes of other rows) and so holds everything about the row at once -- it writes the
+// output-major table nbr_out[k][o] = row at coords[o] + d(k) (coalesced, the centre row the identity), the row's
+// offset mask and the key histogram of the row order, and what the pair lists need: by the symmetry of such a map
+// row o is the INPUT of a pair at offset k exactly when it has a neighbour at 26 - k, so the wave ballots are the
+// (offset, 64-row segment) counts of the pair lists and the popcount of the mask is the row's CSR length.  No
+// probe table, no counting pass, no -1 prefill.  lazy: no pair lists are wanted; the counts per offset go to knnz
+// through one atomic per offset and workgroup.
+// (Written without branches around loads: every load goes out from a valid address and is masked afterwards, the
+// nine cells together, then the first four z of the nine columns together; pointers read from the problem
+// descriptor are cast to the global address space, or the loads are compiled as flat ones.)
+__global__ void __launch_bounds__(256) grid_query_full3_kernel(const ProbDev *__restrict__ P, JobList jl) {
+  const Job &job = find_job(jl, blockIdx.x);
+  const ProbDev &q = P[job.prob];
+  const long long n = q.n_in, nseg = q.nseg;
+  const PCE_GLOBAL pce_v2i *grid = (const PCE_GLOBAL pce_v2i *)q.grid;
+  const PCE_GLOBAL int *zcol = (const PCE_GLOBAL int *)q.zcol;
+  PCE_GLOBAL int *nbr = (PCE_GLOBAL int *)q.nbr_out;
+  const bool order = q.order != nullptr, lazy = q.lazy != 0, want_csr = q.want_csr != 0;      // the same for the whole workgroup
+  const GridBox box = q.box;
+  const long long i = (long long)(blockIdx.x - job.blk0) * blockDim.x + threadIdx.x;
+  const long long seg = i >> 6;
+  const int lane = __lane_id();
+  bool live = i < n;
+  const pce_v4i cv = ((const PCE_GLOBAL pce_v4i *)q.in_coords)[live ? i : 0];
+  const int4 c = make_int4(cv.x, cv.y, cv.z, cv.w);
+  if (live && !pce_coord_ok(c.x, c.y, c.z, c.w)) {
+    q.status[0] = 1;
+    live = false;
+  }
+  __shared__ int keycnt[ORDER_KEYS];
+  __shared__ int offcnt[32];
+  if (order)
+    for (int t = threadIdx.x; t < ORDER_KEYS; t += 256) keycnt[t] = 0;
+  if (threadIdx.x < 32) offcnt[threadIdx.x] = 0;
+  __syncthreads();
+  int2 se[9];
+#pragma unroll
+  for (int col = 0; col < 9; ++col) {
+    const int ix = col / 3, iy = col - ix * 3;
+    // (no early-out as in grid_cell: a branch per column put a wait behind every one of the nine loads)
+    const int gx = c.y + ix - 1 - box.lo[0], gy = c.z + iy - 1 - box.lo[1];
+    const bool in = live & ((unsigned)c.x < (unsigned)box.n_batch) & ((unsigned)gx < (unsigned)box.ext[0]) &
+                    ((unsigned)gy < (unsigned)box.ext[1]);
+    const long long cell = ((long long)c.x * box.ext[0] + gx) * box.ext[1] + gy;
+    const pce_v2i v = grid[in ? cell : 0];
+    se[col].x = in ? v.x : -1;
+    se[col].y = in ? v.y : -1;
+  }
+  int zz[9][4], lb[9];
+  bool tall = false;
+#pragma unroll
+  for (int col = 0; col < 9; ++col) {
+    lb[col] = se[col].x;
+    tall |= se[col].x >= 0 && se[col].y - se[col].x > 4;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int r = se[col].x + t;
+      const bool in = se[col].x >= 0 && r < se[col].y;
+      const int z = zcol[in ? r : 0];
+      zz[col][t] = in ? z : (int)0x80000000;
+    }
+  }
+  if (__any(tall)) {
+    // a column of more than four rows (a wall, a pole): one search for the first row at or above z - 1; the three
+    // rows from there are the only candidates for z - 1, z and z + 1 (the rows of a column ascend strictly in z)
+#pragma unroll
+    for (int col = 0; col < 9; ++col) {
+      if (se[col].x >= 0 && se[col].y - se[col].x > 4) {
+        int lo = se[col].x, hi = se[col].y;          // first row of [lo, hi) whose z >= c.w - 1, or hi
+        while (lo < hi) {
+          const int md = (lo + hi) >> 1;
+          if (zcol[md] < c.w - 1)
+            lo = md + 1;
+          else
+            hi = md;
+        }
+        lb[col] = lo;
+#pragma unroll
+        for (int t = 0; t < 3; ++t) zz[col][t] = lo + t < se[col].y ? zcol[lo + t] : (int)0x80000000;
+        zz[col][3] = (int)0x80000000;
+      }
+    }
+  }
+  // the 27 results of the row; their ballots are the pair lists' (offset, segment) counts, mirrored
+  int res[27];
+  unsigned m = 0;
+  int mine = 0;       // lane l < 27 ends up with the wavefront's count for offset l
+#pragma unroll
+  for (int kp = 0; kp < 27; ++kp) {
+    const int col = kp / 3, iz = kp - col * 3;
+    int r = -1;
+    if (kp == 13) {
+      r = live ? (int)i : -1;
+    } else {
+      const int tz = c.w + iz - 1;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) r = (zz[col][t] == tz) ? lb[col] + t : r;   // padding entries hold INT_MIN, which no valid z equals
+      r = (live && se[col].x >= 0) ? r : -1;
+    }
+    res[kp] = r;
+    const bool hit = r >= 0 && kp != 13;
+    m |= hit ? 1u << kp : 0u;
+    const int cnt = __popcll(__ballot(hit));
+    mine = lane == kp ? cnt : mine;
+  }
+  if (live) {
+#pragma unroll
+    for (int kp = 0; kp < 27; ++kp) nbr[(long long)kp * n + i] = res[kp];
+  }
+  // row o is the input of a pair at offset k exactly when it has a neighbour at 26 - k
+  if (lane < 27) {
+    if (lazy) {
+      if (mine) atomicAdd(&offcnt[26 - lane], mine);
+    } else if (seg < nseg) {
+      q.seg[(long long)(26 - lane) * nseg + seg] = mine;
+    }
+  }
+  if (!lazy) {
+    if (want_csr && i <= n) q.icsr[i] = live ? __popc(m) : 0;   // icsr[n] = 0 receives the total after the scan
+    if (i == 0) q.seg[27 * nseg] = 0;
+  }
+  if (order && live) {
+    q.order[n + i] = (int)m;
+    if (m) atomicAdd(&keycnt[order_key(m)], 1);   // rows without neighbours are placed by the scatter pass
+  }
+  __syncthreads();
+  if (order) {
+    int *hist = q.order + 2 * n + ORDER_HIST;
+    for (int t = threadIdx.x; t < ORDER_KEYS; t += 256)
+      if (keycnt[t]) atomicAdd(&hist[t], keycnt[t]);
+  }
+  if (lazy && threadIdx.x < 27 && offcnt[threadIdx.x]) atomicAdd(&q.knnz[threadIdx.x], offcnt[threadIdx.x]);
 }
 
 // The per-row loops over the offsets below load ROW_BATCH table entries before using any of them.
@@ -1818,6 +1984,22 @@ __global__ void __launch_bounds__(1024) kmap_offsets_kernel(const ProbDev *__res
   const int *__restrict__ segoff = q.seg;
   const long long nseg = q.nseg;
   const int kv = q.g.kv;
+  if (q.lazy) {   // the counts per offset are complete (the probe added them up): their two scans
+    if (threadIdx.x == 0) {
+      int a = 0, qq = 0;
+      q.kpos[0] = 0;
+      q.qkpos[0] = 0;
+      for (int kp = 0; kp < kv; ++kp) {
+        const int c = q.knnz[kp];
+        a += c;
+        qq += (c + PCE_QUANTUM - 1) / PCE_QUANTUM * PCE_QUANTUM;
+        q.kpos[kp + 1] = a;
+        q.qkpos[kp + 1] = qq;
+      }
+      q.status[5] = 1;   // this map holds no pair lists
+    }
+    return;
+  }
   for (int kp = threadIdx.x; kp <= kv; kp += blockDim.x) {
     int a = segoff[(long long)kp * nseg];
     q.kpos[kp] = a;
@@ -1842,13 +2024,21 @@ __global__ void __launch_bounds__(256) kmap_fill_kernel(const ProbDev *__restric
   const Job &job = find_job(jl, blockIdx.x);
   const ProbDev &q = P[job.prob];
   if (job.kind == JOB_ORDER_SCATTER) {   // the row order of a symmetric map: masks and bases are complete by now
-    order_scatter_block(q.n_out, q.order, blockIdx.x - job.blk0);
+    // (a symmetric map: the fill jobs of this launch may be writing nbr_out, so the probe table is read, mirrored,
+    // unless the probe wrote the output-major table itself)
+    if (q.fused)
+      order_scatter_block(q.n_out, q.order, blockIdx.x - job.blk0, q.nbr_out, -1);
+    else
+      order_scatter_block(q.n_out, q.order, blockIdx.x - job.blk0, q.dense, q.g.kv - 1);
     return;
   }
   const long long n_in = q.n_in, n_out = q.n_out, nseg = q.nseg;
-  const int kv = q.g.kv, subm = q.g.subm, sym = q.g.sym, mid = q.g.mid;
-  const int *__restrict__ dense = q.dense;
-  const int *__restrict__ segoff = q.seg;
+  const int kv = q.g.kv, subm = q.g.subm, sym = q.g.sym, mid = q.g.mid, fused = q.fused;
+  // (pointers read from the descriptor are cast to the global address space, or the loads are compiled as flat
+  // ones; every load of a batch goes out from a valid address and is masked afterwards, or each is compiled to a
+  // branch with a wait behind it)
+  const PCE_GLOBAL int *table = (const PCE_GLOBAL int *)(fused ? q.nbr_out : q.dense);
+  const PCE_GLOBAL int *segoff = (const PCE_GLOBAL int *)q.seg;
   int *__restrict__ imap = q.imap;
   int *__restrict__ omap = q.omap;
   int *__restrict__ irank = q.irank;
@@ -1857,16 +2047,25 @@ __global__ void __launch_bounds__(256) kmap_fill_kernel(const ProbDev *__restric
   long long i = (long long)(blockIdx.x - job.blk0) * blockDim.x + threadIdx.x;
   long long seg = i >> 6;
   bool live = i < n_in;
+  const bool mirror = !fused && nbr_out && sym;
   for (int kp0 = 0; kp0 < kv; kp0 += ROW_BATCH) {
     int vv[ROW_BATCH], mm[ROW_BATCH], base[ROW_BATCH], first[ROW_BATCH];
 #pragma unroll
     for (int j = 0; j < ROW_BATCH; ++j) {
-      int kp = kp0 + j;
-      bool in = kp < kv;
-      vv[j] = (live && in) ? dense[(long long)kp * n_in + i] : -1;
-      mm[j] = (live && in && nbr_out && sym && kp != mid) ? dense[(long long)(kv - 1 - kp) * n_in + i] : -1;
-      base[j] = (in && seg < nseg) ? segoff[(long long)kp * nseg + seg] : 0;
-      first[j] = in ? segoff[(long long)kp * nseg] : 0;
+      const int kp = kp0 + j;
+      const bool in = kp < kv;
+      // (fused: the probe wrote the output-major table, whose row kv-1-kp is the probe table's row kp)
+      const bool want_v = live && in && !(fused && kp == mid);
+      const int v = table[want_v ? (long long)(fused ? kv - 1 - kp : kp) * n_in + i : 0];
+      vv[j] = want_v ? v : -1;
+      const bool want_m = mirror && live && in && kp != mid;
+      const int mv = mirror ? table[want_m ? (long long)(kv - 1 - kp) * n_in + i : 0] : -1;
+      mm[j] = want_m ? mv : -1;
+      const bool want_b = in && seg < nseg;
+      const int b = segoff[want_b ? (long long)kp * nseg + seg : 0];
+      base[j] = want_b ? b : 0;
+      const int f = segoff[in ? (long long)kp * nseg : 0];
+      first[j] = in ? f : 0;
     }
 #pragma unroll
     for (int j = 0; j < ROW_BATCH; ++j) {
@@ -1879,13 +2078,13 @@ __global__ void __launch_bounds__(256) kmap_fill_kernel(const ProbDev *__restric
         int p = base[j] + __popcll(bal & lanemask_lt());
         imap[p] = (int)i;
         omap[p] = v;
-        if (nbr_out && !sym) nbr_out[(long long)kp * n_out + v] = (int)i;
+        if (nbr_out && !sym) nbr_out[(long long)kp * n_out + v] = (int)i;   // (a fused map is symmetric)
         rank = p - first[j];
         if (irank && rank >= PCE_CSR_CODE) q.status[2] = 1;
         if (orank) orank[(long long)kp * n_out + v] = rank;
       }
       if (irank && live) irank[(long long)kp * n_in + i] = rank;
-      if (nbr_out && sym && live)  // nbr_out[kp][o] = input of the pair whose output is o = mirrored probe result
+      if (nbr_out && sym && !fused && live)  // nbr_out[kp][o] = input of the pair whose output is o = mirrored probe result
         nbr_out[(long long)kp * n_out + i] = kp == mid ? (int)i : mm[j];
       if (nbr_out && subm && !sym && live && kp == mid) nbr_out[(long long)kp * n_out + i] = (int)i;
     }
@@ -1941,10 +2140,12 @@ __global__ void __launch_bounds__(256) csr_stage_kernel(const ProbDev *__restric
   }
   // JOB_CSR_SUBM
   const long long n = q.n_in;
-  const int *__restrict__ dense = q.dense;
-  const int *__restrict__ irank = q.irank;
-  const int *__restrict__ csr = q.icsr;
-  const int *__restrict__ kpos = q.kpos;
+  const int fused = q.fused, mid = q.g.mid;
+  // (global address space and unconditional loads from valid addresses, as in kmap_fill_kernel)
+  const PCE_GLOBAL int *table = (const PCE_GLOBAL int *)(fused ? q.nbr_out : q.dense);
+  const PCE_GLOBAL int *irank = (const PCE_GLOBAL int *)q.irank;
+  const PCE_GLOBAL int *csr = (const PCE_GLOBAL int *)q.icsr;
+  const PCE_GLOBAL int *kpos = (const PCE_GLOBAL int *)q.kpos;
   int *__restrict__ icode = q.icode;
   int *__restrict__ ocode = q.ocode;
   int *__restrict__ islot = q.islot;
@@ -1960,14 +2161,23 @@ __global__ void __launch_bounds__(256) csr_stage_kernel(const ProbDev *__restric
     int rk[ROW_BATCH], src[ROW_BATCH], rk2[ROW_BATCH], kb[ROW_BATCH];
 #pragma unroll
     for (int j = 0; j < ROW_BATCH; ++j) {
-      int kp = kp0 + j;
-      bool in = kp < kv;
-      rk[j] = in ? irank[(long long)kp * n + r] : -1;
-      src[j] = in ? dense[(long long)(kv - 1 - kp) * n + r] : -1;
-      kb[j] = in ? kpos[kp] : 0;
+      const int kp = kp0 + j;
+      const bool in = kp < kv;
+      const int a = irank[in ? (long long)kp * n + r : 0];
+      rk[j] = in ? a : -1;
+      // the input of the pair whose output is r at offset kp: the output-major table's entry (fused; its centre
+      // row holds the identity and is no pair), else the probe table's mirrored entry
+      const bool want = in && !(fused && kp == mid);
+      const int b = table[want ? (long long)(fused ? kp : kv - 1 - kp) * n + r : 0];
+      src[j] = want ? b : -1;
+      const int c = kpos[in ? kp : 0];
+      kb[j] = in ? c : 0;
     }
 #pragma unroll
-    for (int j = 0; j < ROW_BATCH; ++j) rk2[j] = src[j] >= 0 ? irank[(long long)(kp0 + j) * n + src[j]] : -1;
+    for (int j = 0; j < ROW_BATCH; ++j) {
+      const int a = irank[src[j] >= 0 ? (long long)(kp0 + j < kv ? kp0 + j : 0) * n + src[j] : 0];
+      rk2[j] = src[j] >= 0 ? a : -1;
+    }
 #pragma unroll
     for (int j = 0; j < ROW_BATCH; ++j) {
       int kp = kp0 + j;
@@ -2011,8 +2221,9 @@ __global__ void __launch_bounds__(256) order_mask_kernel(const int *__restrict__
   order_mask_block(nbr, kv, n_rows, mid, order, blockIdx.x);
 }
 __global__ void __launch_bounds__(1024) order_scan_kernel(int *tail) { order_scan_block(tail, nullptr); }
-__global__ void __launch_bounds__(256) order_scatter_kernel(long long n_rows, int *__restrict__ order) {
-  order_scatter_block(n_rows, order, blockIdx.x);
+__global__ void __launch_bounds__(256) order_scatter_kernel(long long n_rows, int *__restrict__ order,
+                                                            const int *__restrict__ nbr) {
+  order_scatter_block(n_rows, order, blockIdx.x, nbr, -1);
 }
 
 // the same over the problems of a batched build; status[4] of a problem receives its number of heavy rows
@@ -2029,10 +2240,10 @@ __global__ void __launch_bounds__(1024) order_scan_batch_kernel(const ProbDev *_
 __global__ void __launch_bounds__(256) order_scatter_batch_kernel(const ProbDev *__restrict__ P, JobList jl) {
   const Job &job = find_job(jl, blockIdx.x);
   const ProbDev &q = P[job.prob];
-  order_scatter_block(q.n_out, q.order, blockIdx.x - job.blk0);
+  order_scatter_block(q.n_out, q.order, blockIdx.x - job.blk0, q.nbr_out, -1);
 }
 
-extern "C" int64_t pce_row_order_elems(int64_t n_rows) { return n_rows < 0 ? 0 : 2 * n_rows + PCE_ORDER_TAIL; }
+extern "C" int64_t pce_row_order_elems(int64_t n_rows) { return n_rows < 0 ? 0 : PCE_ORDER_ELEMS(n_rows); }
 
 extern "C" int pce_row_order(const int32_t *nbr, int32_t kv, int64_t n_rows, int32_t mid, int32_t *order, int64_t order_elems,
                              int64_t *n_heavy_host, pce_stream_t stream) {
@@ -2040,6 +2251,7 @@ extern "C" int pce_row_order(const int32_t *nbr, int32_t kv, int64_t n_rows, int
   if (kv < 1 || kv > ORDER_MAX_KV - 1) PCE_FAIL(PCE_EINVAL, "pce_row_order: kernel volume %d outside [1, %d]", (int)kv, ORDER_MAX_KV - 1);
   if (n_rows <= 0 || n_rows >= (1ll << 30)) PCE_FAIL(PCE_EINVAL, "pce_row_order: n_rows=%lld", (long long)n_rows);
   if (mid >= kv) PCE_FAIL(PCE_EINVAL, "pce_row_order: centre offset %d outside the kernel volume %d", (int)mid, (int)kv);
+  if ((uintptr_t)order & 15) PCE_FAIL(PCE_EINVAL, "pce_row_order: the order array must be 16-byte aligned");
   if (order_elems < pce_row_order_elems(n_rows))
     PCE_FAIL(PCE_EWORKSPACE, "pce_row_order: order holds %lld elements, needs %lld", (long long)order_elems, (long long)pce_row_order_elems(n_rows));
   hipStream_t s = (hipStream_t)stream;
@@ -2051,7 +2263,7 @@ extern "C" int pce_row_order(const int32_t *nbr, int32_t kv, int64_t n_rows, int
   PCE_LAUNCH_CHECK("order_mask");
   hipLaunchKernelGGL(order_scan_kernel, dim3(1), dim3(1024), 0, s, tail);
   PCE_LAUNCH_CHECK("order_scan");
-  hipLaunchKernelGGL(order_scatter_kernel, dim3(blocks), dim3(256), 0, s, (long long)n_rows, order);
+  hipLaunchKernelGGL(order_scatter_kernel, dim3(blocks), dim3(256), 0, s, (long long)n_rows, order, (const int *)nbr);
   PCE_LAUNCH_CHECK("order_scatter");
   int heavy = 0;
   PCE_HIP(hipMemcpyAsync(&heavy, tail + ORDER_N_HEAVY, sizeof(int), hipMemcpyDeviceToHost, s));
@@ -2060,8 +2272,8 @@ extern "C" int pce_row_order(const int32_t *nbr, int32_t kv, int64_t n_rows, int
   return PCE_OK;
 }
 
-enum { ST_INSERT = 0, ST_QUERY, ST_COUNT, ST_FILL, ST_CSR_A, ST_CSR_B, ST_GRID_BUILD, ST_GRID_QUERY, ST_GRID_QUERY3, ST_ORDER_MASK,
-       ST_ORDER_SCATTER, ST_COUNT_ };
+enum { ST_INSERT = 0, ST_QUERY, ST_COUNT, ST_FILL, ST_CSR_A, ST_CSR_B, ST_GRID_BUILD, ST_GRID_QUERY, ST_GRID_QUERY3, ST_GRID_FULL3,
+       ST_ORDER_MASK, ST_ORDER_SCATTER, ST_COUNT_ };
 
 // host-side image of everything the kernels of one batch read
 struct BatchImage {
@@ -2149,7 +2361,7 @@ extern "C" int pce_kmap_build_batch(const pce_kmap_problem_t *probs, int32_t n_p
     ProbDev &q = img.prob[p];
     int rc = make_geom(&u.geom, &q.g);
     if (rc) return rc;
-    if (!u.in_coords || !u.out_coords || !u.ws || !u.imap || !u.omap || !u.knnz || !u.kpos || !u.qkpos || !u.status)
+    if (!u.in_coords || !u.out_coords || !u.ws || !u.knnz || !u.kpos || !u.qkpos || !u.status)
       PCE_FAIL(PCE_EINVAL, "pce_kmap_build: null pointer");
     int ncsr = (u.icsr != nullptr) + (u.icode != nullptr) + (u.ocsr != nullptr) + (u.ocode != nullptr);
     if (ncsr != 0 && ncsr != 4) PCE_FAIL(PCE_EINVAL, "pce_kmap_build: pass all four CSR outputs or none");
@@ -2171,6 +2383,13 @@ extern "C" int pce_kmap_build_batch(const pce_kmap_problem_t *probs, int32_t n_p
     }
     if (!use_grid) kmap_layout(n_in, n_out, q.g.kv, want_csr, q.g.sym, 0, &L);
     if (u.ws_bytes < L.total) PCE_FAIL(PCE_EWORKSPACE, "pce_kmap_build: workspace %lld < %lld", (long long)u.ws_bytes, (long long)L.total);
+    // the 3x3x3 submanifold map over the column grid is probed output-major in one pass (grid_query_full3_kernel)
+    // when the output-major table is wanted and the probe table is not; without pair lists if the caller waives them
+    const bool subm3 = q.g.sym && q.g.ks[0] == 3 && q.g.ks[1] == 3 && q.g.ks[2] == 3;
+    const int fused = use_grid && subm3 && u.nbr_out && !u.nbr_in;
+    const int lazy = fused && (u.flags & PCE_KMAP_TABLE_ONLY) && !want_csr;
+    if (!lazy && (!u.imap || !u.omap))
+      PCE_FAIL(PCE_EINVAL, "pce_kmap_build: null pair lists (only a map built with PCE_KMAP_TABLE_ONLY over the column grid goes without)");
     char *w = (char *)u.ws;
     q.in_coords = (const int4 *)u.in_coords;
     q.out_coords = (const int4 *)u.out_coords;
@@ -2210,6 +2429,8 @@ extern "C" int pce_kmap_build_batch(const pce_kmap_problem_t *probs, int32_t n_p
       }
     }
     q.want_csr = want_csr;
+    q.fused = fused;
+    q.lazy = lazy;
     q.use_grid = use_grid;
     if (use_grid) {
       q.box = box;
@@ -2221,7 +2442,9 @@ extern "C" int pce_kmap_build_batch(const pce_kmap_problem_t *probs, int32_t n_p
       add_fill(q.grid, box.cells * 2);
     else
       add_fill(q.table, L.slots * 4);
-    if (q.g.sym) {
+    if (fused) {
+      if (lazy) add_fill(q.knnz, q.g.kv, 1);   // the probe adds the counts per offset up with atomics
+    } else if (q.g.sym) {
       // rows of the probe table that the mirrored writes only touch on a hit (and the centre row)
       add_fill(q.dense + (int64_t)q.g.mid * n_in, (int64_t)(q.g.kv - q.g.mid) * n_in);
     } else {
@@ -2230,13 +2453,18 @@ extern "C" int pce_kmap_build_batch(const pce_kmap_problem_t *probs, int32_t n_p
     }
     add_job(use_grid ? ST_GRID_BUILD : ST_INSERT, p, 0, n_out);
     // 2. probe, count per (offset, segment) and per row; 3. their scans; 4. pair lists
-    const bool subm3 = q.g.sym && q.g.ks[0] == 3 && q.g.ks[1] == 3 && q.g.ks[2] == 3;
-    add_job(use_grid ? (subm3 ? ST_GRID_QUERY3 : ST_GRID_QUERY) : ST_QUERY, p, 0, n_in);
-    add_job(ST_COUNT, p, 0, n_in + 1);
+    if (fused) {
+      add_job(ST_GRID_FULL3, p, 0, n_in + 1);
+    } else {
+      add_job(use_grid ? (subm3 ? ST_GRID_QUERY3 : ST_GRID_QUERY) : ST_QUERY, p, 0, n_in);
+      add_job(ST_COUNT, p, 0, n_in + 1);
+    }
     int *scan_tmp = (int *)(w + L.off_scan);
-    add_scan(0, q.seg, L.scan_len, scan_tmp);
-    if (want_csr) add_scan(0, q.icsr, n_in + 1, scan_tmp + scan_tmp_ints(L.scan_len));
-    add_job(ST_FILL, p, 0, n_in);
+    if (!lazy) {
+      add_scan(0, q.seg, L.scan_len, scan_tmp);
+      if (want_csr) add_scan(0, q.icsr, n_in + 1, scan_tmp + scan_tmp_ints(L.scan_len));
+      add_job(ST_FILL, p, 0, n_in);
+    }
     if (q.order && q.g.sym) add_job(ST_FILL, p, JOB_ORDER_SCATTER, n_out);
     // 5. CSR-coded views
     if (want_csr && q.g.sym) {
@@ -2288,16 +2516,26 @@ extern "C" int pce_kmap_build_batch(const pce_kmap_problem_t *probs, int32_t n_p
     hipLaunchKernelGGL(grid_query_kernel<true>, dim3(blk[ST_GRID_QUERY3]), dim3(256), 0, s, P, jl(ST_GRID_QUERY3));
     PCE_LAUNCH_CHECK("grid_query3");
   }
-  hipLaunchKernelGGL(kmap_count_kernel, dim3(blk[ST_COUNT]), dim3(256), 0, s, P, jl(ST_COUNT));
-  PCE_LAUNCH_CHECK("kmap_count");
-  hipLaunchKernelGGL(multi_scan_local_kernel, dim3(scan_blk[0]), dim3(256), 0, s, (const ScanArr *)D->scans[0], n_scan[0]);
-  PCE_LAUNCH_CHECK("scan_local");
-  hipLaunchKernelGGL(multi_scan_add_kernel, dim3(scan_blk[0]), dim3(256), 0, s, (const ScanArr *)D->scans[0], n_scan[0]);
-  PCE_LAUNCH_CHECK("scan_add");
+  if (blk[ST_GRID_FULL3]) {
+    hipLaunchKernelGGL(grid_query_full3_kernel, dim3(blk[ST_GRID_FULL3]), dim3(256), 0, s, P, jl(ST_GRID_FULL3));
+    PCE_LAUNCH_CHECK("grid_query_full3");
+  }
+  if (blk[ST_COUNT]) {
+    hipLaunchKernelGGL(kmap_count_kernel, dim3(blk[ST_COUNT]), dim3(256), 0, s, P, jl(ST_COUNT));
+    PCE_LAUNCH_CHECK("kmap_count");
+  }
+  if (scan_blk[0]) {
+    hipLaunchKernelGGL(multi_scan_local_kernel, dim3(scan_blk[0]), dim3(256), 0, s, (const ScanArr *)D->scans[0], n_scan[0]);
+    PCE_LAUNCH_CHECK("scan_local");
+    hipLaunchKernelGGL(multi_scan_add_kernel, dim3(scan_blk[0]), dim3(256), 0, s, (const ScanArr *)D->scans[0], n_scan[0]);
+    PCE_LAUNCH_CHECK("scan_add");
+  }
   hipLaunchKernelGGL(kmap_offsets_kernel, dim3(2 * n_probs), dim3(1024), 0, s, P, (int)n_probs);
   PCE_LAUNCH_CHECK("kmap_offsets");
-  hipLaunchKernelGGL(kmap_fill_kernel, dim3(blk[ST_FILL]), dim3(256), 0, s, P, jl(ST_FILL));
-  PCE_LAUNCH_CHECK("kmap_fill");
+  if (blk[ST_FILL]) {
+    hipLaunchKernelGGL(kmap_fill_kernel, dim3(blk[ST_FILL]), dim3(256), 0, s, P, jl(ST_FILL));
+    PCE_LAUNCH_CHECK("kmap_fill");
+  }
   if (blk[ST_CSR_A]) {
     hipLaunchKernelGGL(csr_stage_kernel, dim3(blk[ST_CSR_A]), dim3(256), 0, s, P, jl(ST_CSR_A));
     PCE_LAUNCH_CHECK("csr_stage_a");

@@ -54,7 +54,8 @@ def test_row_order_built_with_the_map_and_on_its_own(cloud):
     ref, masks = _oracle_masks(coords)
     km = _subm(coords)
     n = len(coords)
-    assert km.order is not None and km.order.numel() == 2 * n + 8192
+    rec_at = (2 * n + 8192 + 3) // 4 * 4
+    assert km.order is not None and km.order.numel() == rec_at + 4 * n == _lib.load().pce_row_order_elems(n)
     lazy = _subm(coords, want_order=False)
     assert lazy.order is None
     backend.row_order(lazy)
@@ -74,6 +75,48 @@ def test_row_order_built_with_the_map_and_on_its_own(cloud):
         plain = perm[:n_plain]
         same_block = plain[1:] // 256 == plain[:-1] // 256
         assert (np.diff(plain)[same_block] > 0).all()        # a block's plain rows keep their order
+        # the record of every row with a neighbour, at its position in the order: the row, its mask and its
+        # neighbours at the two lowest offsets of the mask (the oracle's pairs)
+        rec = order[rec_at:rec_at + 4 * n].reshape(n, 4).astype(np.int64)[n_plain:]
+        rows = perm[n_plain:]
+        assert np.array_equal(rec[:, 0], rows) and np.array_equal(rec[:, 1], masks[rows])
+        nbr_of = {}
+        for kp in range(27):
+            if kp != 13:
+                a, b = ref.kpos[kp], ref.kpos[kp + 1]
+                nbr_of.update({(int(o), kp): int(i) for i, o in zip(ref.imap[a:b], ref.omap[a:b])})
+        for (row, mask, nb0, nb1) in rec[:: max(1, len(rec) // 500)]:
+            bits = [k for k in range(27) if (mask >> k) & 1]
+            assert nb0 == nbr_of[(row, bits[0])]
+            assert nb1 == (nbr_of[(row, bits[1])] if len(bits) > 1 else -1)
+
+
+@pytest.mark.parametrize("cloud", sorted(CLOUDS))
+def test_map_built_without_pair_lists(cloud):
+    """want_pairs=False: the 3x3x3 submanifold map over the column grid comes as neighbour table, row order and
+    counts only (has_pairs False), all equal to the full build's; the ordered dataflow runs on it as it is; reading
+    a pair list builds both, bit-equal to the oracle's; a build that cannot skip them (no batch count: the hash
+    table) ignores the request."""
+    coords = CLOUDS[cloud]()
+    ref, masks = _oracle_masks(coords)
+    full = _subm(coords)
+    batches = int(coords[:, 0].max()) + 1
+    build = lambda b: backend.build_kernel_map(dev_coords(coords), K3, S1, P0, [0, 0, 0], coords[:, 1:].max(0).tolist(), True,
+                                               want_csr=False, batchsize=b, want_pairs=False)
+    km = build(batches)
+    assert not km.has_pairs and km.M == ref.M and km.qsum == full.qsum
+    for name in ("nbr_out", "knnz", "kpos", "qkpos"):
+        assert torch.equal(getattr(km, name), getattr(full, name)), name
+    n = len(coords)
+    assert km.order_heavy == full.order_heavy and torch.equal(km.order[n:2 * n], full.order[n:2 * n])
+    assert backend.select_dataflow(km, 32, 32, torch.float16) == backend.select_dataflow(full, 32, 32, torch.float16)
+    f = torch.as_tensor(synth.features(3, n, 32), device=DEV).half()
+    w = torch.as_tensor(synth.weights(3, 27, 32, 32), device=DEV).half()
+    assert torch.equal(backend.conv_forward(f, w, km, DATAFLOW_OSO), backend.conv_forward(f, w, full, DATAFLOW_OSO))
+    assert not km.has_pairs
+    assert np.array_equal(km.imap.cpu().numpy(), ref.imap) and np.array_equal(km.omap.cpu().numpy(), ref.omap)
+    assert km.has_pairs
+    assert build(0).has_pairs
 
 
 @pytest.mark.parametrize("cloud", sorted(CLOUDS))
