@@ -208,7 +208,8 @@ typedef struct pce_kmap_problem {
   int32_t *nbr_out, *nbr_in;            /* optional */
   int32_t *status;                      /* int32[8] per problem, zeroed by the caller: [0] coordinate out of range, [1] hash
                                            table exhausted, [2] CSR code overflow, [3] column grid not applicable (see
-                                           below), [4] n_heavy of `order`, [5] 1 = no pair lists were written */
+                                           below), [4] n_heavy of `order`, [5] 1 = no pair lists were written,
+                                           [6] n_nonzero and [7] n_single of `order` */
   int32_t n_batch;                      /* batch count (spTensor.batchsize), 0 = unknown: see the column grid below */
   int32_t flags;                        /* PCE_KMAP_* */
   int32_t *order;                       /* optional, needs nbr_out and kv <= 31: the row order of pce_row_order
@@ -379,9 +380,17 @@ int pce_conv_fwd_os(const void *in_feats, const void *weight, const void *weight
  * output-major neighbour table, once per map, the order in which the rows are visited -- rows without neighbours
  * first, in their own order, then the rows with one or two neighbours sorted by the offsets they have them at, then
  * the rows with three or more, sorted likewise -- and every row's offset mask: order_dev = perm[n_rows] |
- * mask[n_rows] | 8192 ints of scratch, pce_row_order_elems ints in all; kv <= 31; four launches and one wait for
- * *n_heavy_host, the number of rows of the last part; the positions of rows with equal keys depend on the run,
- * the results of the layer do not.  pce_conv_fwd_oso then runs the layer as one launch: a wavefront takes 32 rows
+ * mask[n_rows] | 8192 ints of scratch | rec[n_rows] (16 bytes each, for the positions of rows with a neighbour:
+ * {row, mask, neighbour at the lowest offset of the mask, neighbour at the second-lowest or -1}),
+ * pce_row_order_elems ints in all, 16-byte aligned; kv <= 31; four launches and one wait for counts_host[0] =
+ * n_heavy, the number of rows of the last part, counts_host[1] = n_nonzero, the number of rows with any
+ * neighbour, and counts_host[2] = n_single, the number with exactly one (they come first among the rows with
+ * neighbours, sorted by the offset); the positions of rows with equal keys depend on the run, the results of the
+ * layer do not.  pce_conv_fwd_oso takes the three counts as order_counts_host.  With n_nonzero and n_single stated
+ * (-1: not known), submanifold fp16 layers of at most 64 channels on clouds where at most half the rows have a
+ * neighbour run as three kinds of workgroup: the bulk of the rows streamed in storage order, 64 per wavefront,
+ * stored where their mask is empty; rows with one neighbour by their records; rows with two or more 32 to a
+ * workgroup (two workgroups above 32 output channels) whose wavefronts share the offsets.  pce_conv_fwd_oso then runs the layer as one launch: a wavefront takes 32 rows
  * of that order, multiplies their centre rows, gathers for each offset any of them has the neighbours of the rows
  * that have it, and stores each finished row once (epilogue fused); the rows of the last part, whose offsets are
  * many, go 32 to a workgroup whose four wavefronts share the offsets.  PCE_F16, packed weights: c_in a multiple of
@@ -396,11 +405,11 @@ int pce_conv_fwd_os(const void *in_feats, const void *weight, const void *weight
  * (backend/spconv.cuh:1567-1730) with the scatter-add replaced by register accumulation, as pce_conv_fwd_os. */
 int64_t pce_row_order_elems(int64_t n_rows);
 int pce_row_order(const int32_t *nbr_dev, int32_t kv, int64_t n_rows, int32_t mid, int32_t *order_dev,
-                  int64_t order_elems, int64_t *n_heavy_host, pce_stream_t stream);
+                  int64_t order_elems, int64_t *counts_host /* [3] */, pce_stream_t stream);
 int pce_conv_fwd_oso(const void *in_feats, const void *weight, const void *weight_packed,
                      void *out_feats, int32_t dtype,
                      int64_t n_in, int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv, int32_t mid,
-                     const int32_t *nbr_dev, const int32_t *order_dev, int64_t n_heavy,
+                     const int32_t *nbr_dev, const int32_t *order_dev, const int64_t *order_counts_host /* [3] */,
                      const pce_epilogue_t *epilogue, pce_stream_t stream);
 
 /* ---- batch normalisation over the rows of a feature matrix ------------------------------------- *

@@ -110,7 +110,7 @@ _SIGNATURES = {
                                    POINTER(Epilogue), c_void_p]),
     "pce_conv_fwd_os": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_void_p, POINTER(Epilogue), c_void_p]),
     "pce_conv_fwd_oso": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32,
-                                   c_void_p, c_void_p, c_int64, POINTER(Epilogue), c_void_p]),
+                                   c_void_p, c_void_p, POINTER(c_int64), POINTER(Epilogue), c_void_p]),
     "pce_row_order": (c_int32, [c_void_p, c_int32, c_int64, c_int32, c_void_p, c_int64, POINTER(c_int64), c_void_p]),
     "pce_row_order_elems": (c_int64, [c_int64]),
     "pce_conv_fwd_dense": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32, POINTER(Epilogue), c_void_p]),

@@ -119,6 +119,8 @@ class KernelMap:
     route_t: Optional[torch.Tensor] = None # the same for the transposed layer over this map
     order: Optional[torch.Tensor] = None   # rows in neighbour-pattern order and their offset masks (row_order), built on first use
     order_heavy: int = 0                   # how many rows of that order have three neighbours or more (its last part)
+    order_nonzero: int = -1                # how many have any neighbour (-1: not known)
+    order_single: int = -1                 # how many have exactly one (-1: not known)
     tag: str = "auto"           # 'D1' / 'D2' when the reference's init_tag protocol fixed it
     in_coords: Optional[torch.Tensor] = None
     geom: Optional[Geom] = None
@@ -382,7 +384,8 @@ class _MapJob:
                        icsr=self.icsr, ocsr=self.ocsr, icode=cut(self.icode), ocode=cut(self.ocode),
                        islot=cut(self.islot), oslot=cut(self.oslot), in_coords=self.in_coords, geom=self.geom,
                        knnz_host=host[:kv], order=self.order, order_heavy=st[4] if self.order is not None else 0,
-                       has_pairs=not st[5], batchsize=self.n_batch)
+                       has_pairs=not st[5], batchsize=self.n_batch, order_nonzero=st[6] if self.order is not None else -1,
+                       order_single=st[7] if self.order is not None else -1)
         km._cmin, km._cmax = cmin, cmax_out
         km.kpos_host = (_lib.c_int32 * (kv + 1))(*host[kv:2 * kv + 1])
         km.qkpos_host = (_lib.c_int32 * (kv + 1))(*host[2 * kv + 1:3 * kv + 2])
@@ -518,10 +521,10 @@ def row_order(km: KernelMap) -> torch.Tensor:
         lib = _lib.load()
         elems = lib.pce_row_order_elems(km.n_out)
         order = torch.empty(elems, dtype=torch.int32, device=km.nbr_out.device)
-        heavy = _lib.c_int64(0)
+        counts = (_lib.c_int64 * 3)()
         _lib.check(lib.pce_row_order(km.nbr_out.data_ptr(), km.kv, km.n_out, _mid(km.ks) if km.subm else -1, order.data_ptr(),
-                                     elems, heavy, _stream(order.device)))
-        km.order, km.order_heavy = order, heavy.value
+                                     elems, counts, _stream(order.device)))
+        km.order, km.order_heavy, km.order_nonzero, km.order_single = order, counts[0], counts[1], counts[2]
     return km.order
 
 
@@ -546,6 +549,7 @@ def ensure_nbr(km: KernelMap, transposed: bool) -> None:
     km.nbr_out, km.nbr_in = full.nbr_out, full.nbr_in
     if full.order is not None:
         km.order, km.order_heavy = full.order, full.order_heavy
+        km.order_nonzero, km.order_single = full.order_nonzero, full.order_single
 
 
 def select_dataflow(km: KernelMap, c_in: int, c_out: int, dtype: torch.dtype, transposed: bool = False) -> int:
@@ -744,7 +748,8 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
             packed = pack_weights(weight)      # None for fp32: that form reads the weights as they are
         order = row_order(km)
         _lib.check(lib.pce_conv_fwd_oso(feats.data_ptr(), weight.data_ptr(), _ptr(packed), out.data_ptr(), dt, n_in, n_out,
-                                        c_in, c_out, kv, mid, km.nbr_out.data_ptr(), order.data_ptr(), km.order_heavy, epi, s))
+                                        c_in, c_out, kv, mid, km.nbr_out.data_ptr(), order.data_ptr(),
+                                        (_lib.c_int64 * 3)(km.order_heavy, km.order_nonzero, km.order_single), epi, s))
     elif dataflow == DATAFLOW_OS:
         ensure_nbr(km, transposed)
         nbr = km.nbr_in if transposed else km.nbr_out

@@ -78,8 +78,8 @@ __host__ __device__ static inline unsigned long long pce_home_slot(unsigned long
 // ---------------------------------------------------------------------------------------------
 // Row order of the ordered output-stationary dataflow (pce_row_order, pce_conv_fwd_oso):
 // order = perm[n_rows] | mask[n_rows] | tail[PCE_ORDER_TAIL] | rec[n_rows] (int4, 16-byte aligned).  The tail holds
-// the histogram, the cursors and the bases of the counting sort over ORDER_KEYS keys -- (lowest, second-lowest)
-// offset of the rows with one or two neighbours, then of the rows with more -- and the counts.  rec[p], for the
+// the histogram, the cursors and the bases of the counting sort over ORDER_KEYS keys -- the offset of the rows with
+// one neighbour, then (lowest, second-lowest) offset of the rows with two, then of the rows with more -- and the counts.  rec[p], for the
 // positions p of rows that have a neighbour, repeats what a wavefront needs of the row at perm[p] in one 16-byte
 // load: {row, mask, neighbour at the lowest offset of the mask, neighbour at the second-lowest or -1}.
 // ---------------------------------------------------------------------------------------------
@@ -91,6 +91,7 @@ __host__ __device__ static inline unsigned long long pce_home_slot(unsigned long
 #define ORDER_HIST 0
 #define ORDER_CURSOR 2048
 #define ORDER_BASE 4096
+#define ORDER_N_SINGLE 8187   // rows with exactly one neighbour
 #define ORDER_N_NONZERO 8188  // rows with any neighbour
 #define ORDER_N_HEAVY 8189    // rows with ORDER_HEAVY_POPC neighbours or more
 #define ORDER_PLAIN_CURSOR 8191

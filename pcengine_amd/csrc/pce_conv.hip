@@ -2570,6 +2570,342 @@ __global__ void __launch_bounds__(256, 4) wave_os_kernel(TileArgs a, const int *
   store_rows_via_lds<half_t, NB>(V, Pl[wave], (half_t *)a.out, orow, a, 0, lane, l32, g, a.stream);
 }
 
+// The same layer for clouds where most rows have no neighbour at all (at least half of them), in three kinds of
+// workgroup, so that every wavefront of the launch is resident from the start and none waits for more trips to
+// memory than its rows need (per-wavefront timestamps of wave_os_kernel on the 150 k-voxel scan: two rounds of
+// wavefronts of 7 us each, of which 3 us go to the two dependent loads in front of the rows; beside them chains of
+// one trip per offset, up to twelve in a row, in the chunks whose rows have two neighbours or more):
+//   stream  (the bulk): a wavefront takes 64 consecutive rows in STORAGE order -- no row index to fetch first: the
+//           rows travel to LDS with the first instructions of the wavefront, their offset masks beside them --
+//           multiplies them by the centre weights and stores those whose mask is empty; rows with neighbours are
+//           left to the two other kinds (their centre product is computed twice: a seventh of the rows on a LiDAR scan);
+//   single  32 rows with exactly one neighbour, from the row order's records {row, mask, neighbour, -}: one trip for
+//           the records, one for the centre rows, the neighbour's fragments and the weights of the chunk's first
+//           offset (the order sorts these rows by their offset: a chunk has one offset, two at a boundary);
+//   shared  32 rows with two neighbours or more per workgroup (two workgroups per chunk for 33-64 output channels,
+//           32 columns each), the offsets split over the four wavefronts by k mod 4 as in wave_os_kernel; a
+//           wavefront requests the neighbour indices of all its offsets (at most seven) in one trip and keeps row
+//           fragments and weights of two offsets in flight (16 + 16 registers per offset at 32 columns).
+// Rows with three neighbours or more form their sums as in wave_os_kernel (per wavefront over its offsets in
+// ascending order, then wavefront 0 adds the others' in turn) and come out bit-identical to it; rows with two are
+// summed the same way here and in one wavefront there, so their last bits may differ between the two kernels.
+template <int NB, int KS>
+__global__ void __launch_bounds__(256, 4) wave_os2_kernel(TileArgs a, const int *__restrict__ order, int mid, long long n_plain,
+                                                          long long n_single, int shared_wgs, int single_wgs) {
+  constexpr int PPR = KS * 2;   // 16-byte pieces per input row
+  constexpr int REGION0 = WaveLds<NB>::PIECES > 64 * PPR ? WaveLds<NB>::PIECES : 64 * PPR;
+  constexpr int REGION = REGION0 > 256 ? REGION0 : 256;   // also one accumulator block of 64 lanes
+  static_assert(REGION * 16 >= 64 * 64, "a wavefront's region holds one accumulator block of all its lanes");
+  __shared__ __attribute__((aligned(16))) half8 Pl[4][REGION];
+  __shared__ __attribute__((aligned(16))) half8 Wc[KS * 2 * NB * 32];   // the centre offset's weights, shared by the workgroup
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int l32 = lane & 31, g = lane >> 5;
+  const half_t *Wp = (const half_t *)a.Wp;
+  const half_t *A = (const half_t *)a.A;
+  const long long wstep = (long long)a.k8_total * a.n_pad * 8;
+  const long long n = a.n_rows;
+  {
+    constexpr int FR = KS * 2 * NB * 32;   // fragments: [k8][column]
+#pragma unroll
+    for (int i = 0; i < (FR + 255) / 256; ++i) {
+      const int f = i * 256 + wave * 64 + lane;
+      const half_t *gp = Wp + mid * wstep + (long long)(f < FR ? f : FR - 1) * 8;
+      if (i * 256 + wave * 64 < FR)   // wavefront-uniform
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
+                                         (__attribute__((address_space(3))) void *)&Wc[i * 256 + wave * 64], 16, 0, 0);
+    }
+  }
+  const int first_stream = shared_wgs + single_wgs;
+  if ((int)blockIdx.x >= first_stream) {
+    // ---- stream: 64 consecutive rows --------------------------------------------------------------------------
+    const long long r0 = (((long long)blockIdx.x - first_stream) * 4 + wave) * 64;
+    if (r0 >= n) {   // still joins the barrier behind the weight copies
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      return;
+    }
+#pragma unroll
+    for (int it = 0; it < PPR; ++it) {
+      const int e = it * 64 + lane, r = e / PPR, sl = e % PPR;
+      const long long row = r0 + r < n ? r0 + r : n - 1;
+      const half_t *gp = A + row * a.lda + ((sl ^ row_swizzle<PPR>(r)) * 8);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
+                                       (__attribute__((address_space(3))) void *)&Pl[wave][it * 64], 16, 0, 0);
+    }
+    // the mask of row r0 + lane (no order: a plain GEMM, every row is stored)
+    const unsigned mrow = order ? ((const unsigned *)(order + n))[r0 + lane < n ? r0 + lane : n - 1] : 0u;
+    f32x16 acc[2][NB];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acc[h][nb][j] = 0.f;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();   // the centre weights of all four wavefronts' copies (and this wavefront's rows) are in LDS
+    // (K step by K step: the weight fragments of one step serve both halves of the rows; holding those of all steps
+    // beside 64 accumulator registers spilled)
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      half8 wf[NB];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) wf[nb] = Wc[(2 * s + g) * (NB * 32) + nb * 32 + l32];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int r = h * 32 + l32;
+        const half8 af = Pl[wave][r * PPR + ((2 * s + g) ^ row_swizzle<PPR>(r))];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) acc[h][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[nb], af, acc[h][nb], 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();   // every lane has read its fragments: the region becomes the output staging area
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const long long row = r0 + h * 32 + l32;
+      const unsigned mh = (unsigned)__shfl((int)mrow, h * 32 + l32, PCE_WAVE);
+      const int orow = (row < n && mh == 0u) ? (int)row : -1;   // rows with neighbours belong to the other workgroups
+      float V[NB][2][8];
+      gather_row_pieces<NB>(acc[h], V, g);
+      if (a.bias || a.res || a.act) epilogue_row_pieces<half_t, NB, true>(V, a, orow, 0, g, a.act != PCE_ACT_NONE);
+      store_rows_via_lds<half_t, NB>(V, Pl[wave], (half_t *)a.out, orow, a, 0, lane, l32, g, a.stream);
+    }
+    return;
+  }
+  const int4 *rec = reinterpret_cast<const int4 *>(order + PCE_ORDER_REC_OFFSET(n));
+  const half8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  // a lane's K half of a row, from an address that is valid for every lane; zeroed where there is no row
+#define PCE_OS2_FRAGS(F_, NROW_)                                                                                   \
+  {                                                                                                                \
+    const int nr_ = (NROW_);                                                                                       \
+    const half_t *rp_ = A + (long long)(nr_ >= 0 ? nr_ : 0) * a.lda + g * 8;                                       \
+    _Pragma("unroll") for (int s = 0; s < KS; ++s) F_[s] = *reinterpret_cast<const half8 *>(rp_ + s * 16);         \
+    _Pragma("unroll") for (int s = 0; s < KS; ++s) F_[s] = nr_ >= 0 ? F_[s] : zero;                                \
+  }
+  if ((int)blockIdx.x >= shared_wgs) {
+    // ---- single: 32 rows with one neighbour each ---------------------------------------------------------------
+    const long long p0 = n_plain + (((long long)blockIdx.x - shared_wgs) * 4 + wave) * 32, p_end = n_plain + n_single;
+    if (p0 >= p_end) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      return;
+    }
+    const bool valid = p0 + l32 < p_end;
+    const int4 rc = rec[valid ? p0 + l32 : p0];   // {row, mask (one bit), neighbour, -1}
+    const int orow = valid ? rc.x : -1;
+    const unsigned m = valid ? (unsigned)rc.y : 0u;
+    unsigned u = m;
+#pragma unroll
+    for (int d = 1; d < 32; d <<= 1) u |= (unsigned)__shfl_xor((int)u, d, PCE_WAVE);
+    unsigned todo = __builtin_amdgcn_readfirstlane(u);   // offsets any of the 32 rows has: the same in every lane
+#pragma unroll
+    for (int it = 0; it < KS; ++it) {   // centre rows -> LDS, in line order (the row of a lane past the end is the chunk's first)
+      const int e = it * 64 + lane, r = e / PPR, sl = e % PPR;
+      const int row = __shfl(rc.x, r, PCE_WAVE);
+      const half_t *gp = A + (long long)row * a.lda + ((sl ^ row_swizzle<PPR>(r)) * 8);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
+                                       (__attribute__((address_space(3))) void *)&Pl[wave][it * 64], 16, 0, 0);
+    }
+    half8 fa[KS], wk[KS][NB];
+    PCE_OS2_FRAGS(fa, valid ? rc.z : -1)
+    int k = __ffs((int)todo) - 1;   // a valid chunk has a row, the row an offset
+    todo &= todo - 1u;
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+        wk[s][nb] = *reinterpret_cast<const half8 *>(Wp + k * wstep + ((long long)(2 * s + g) * a.n_pad + nb * 32 + l32) * 8);
+    f32x16 acc[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) acc[nb][j] = 0.f;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const half8 af = Pl[wave][l32 * PPR + ((2 * s + g) ^ row_swizzle<PPR>(l32))];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+        acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(Wc[(2 * s + g) * (NB * 32) + nb * 32 + l32], af, acc[nb], 0, 0, 0);
+    }
+    while (true) {
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        const half8 fs = ((m >> k) & 1u) ? fa[s] : zero;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wk[s][nb], fs, acc[nb], 0, 0, 0);
+      }
+      if (!todo) break;
+      k = __ffs((int)todo) - 1;
+      todo &= todo - 1u;
+#pragma unroll
+      for (int s = 0; s < KS; ++s)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+          wk[s][nb] = *reinterpret_cast<const half8 *>(Wp + k * wstep + ((long long)(2 * s + g) * a.n_pad + nb * 32 + l32) * 8);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();   // every lane has read its centre fragments: the region becomes the output staging area
+    float V[NB][2][8];
+    gather_row_pieces<NB>(acc, V, g);
+    if (a.bias || a.res || a.act) epilogue_row_pieces<half_t, NB, true>(V, a, orow, 0, g, a.act != PCE_ACT_NONE);
+    store_rows_via_lds<half_t, NB>(V, Pl[wave], (half_t *)a.out, orow, a, 0, lane, l32, g, a.stream);
+    return;
+  }
+#undef PCE_OS2_FRAGS
+  // ---- shared: 32 rows with two neighbours or more per workgroup ------------------------------------------------
+  // The four wavefronts split the INPUT CHANNELS, 16 each (one K step of the MFMA), and all walk the offsets of
+  // the chunk's union: a step then holds 16 bytes of a neighbour row and 16 bytes of weights per column block in a
+  // lane -- 12 registers at 64 columns -- so four offsets are in flight per wavefront, where a wavefront that owns
+  // whole offsets (wave_os_kernel: k mod 4) has registers for one and spends one trip to memory per offset, seven in
+  // a row on a dense cluster.  The neighbour indices of the chunk, [offset][row], are fetched once per workgroup
+  // (wavefront w those of the offsets k = w mod 4) into LDS.  Each wavefront adds its share of the centre product;
+  // the four partial sums of a row meet through LDS in wavefront 0, which stores the row.
+  const long long p0 = n_plain + n_single + (long long)blockIdx.x * 32;
+  const bool valid = p0 + l32 < n;
+  const int4 rc = rec[valid ? p0 + l32 : p0];
+  const int orow = valid ? rc.x : -1;
+  const unsigned m = valid ? (unsigned)rc.y : 0u;
+  unsigned uu = m;
+#pragma unroll
+  for (int d = 1; d < 32; d <<= 1) uu |= (unsigned)__shfl_xor((int)uu, d, PCE_WAVE);
+  const unsigned u = (unsigned)__builtin_amdgcn_readfirstlane((int)uu);   // offsets any of the 32 rows has
+  // the table of neighbour indices lives behind the centre rows in wavefront 0's region and runs into wavefront 1's
+  // (wavefront 0 stages the finished rows over it once every wavefront is done with it)
+  int *idxL = reinterpret_cast<int *>(&Pl[0][32 * PPR]);
+  static_assert((32 * PPR) * 16 + 27 * 32 * 4 <= 2 * REGION * 16, "centre rows and index table fit two regions");
+  if (wave == 0) {
+#pragma unroll
+    for (int it = 0; it < KS; ++it) {
+      const int e = it * 64 + lane, r = e / PPR, sl = e % PPR;
+      const int row = __shfl(rc.x, r, PCE_WAVE);
+      const half_t *gp = A + (long long)row * a.lda + ((sl ^ row_swizzle<PPR>(r)) * 8);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
+                                       (__attribute__((address_space(3))) void *)&Pl[0][it * 64], 16, 0, 0);
+    }
+  }
+  {
+    // this wavefront's share of the index table: up to seven offsets, all requested before any is written
+    unsigned rem = u & (0x11111111u << wave);
+    rem = (unsigned)__builtin_amdgcn_readfirstlane((int)rem);
+    int kk[7], vv[7];
+#pragma unroll
+    for (int t = 0; t < 7; ++t) {
+      kk[t] = rem ? __ffs((int)rem) - 1 : -1;
+      rem &= rem - 1u;
+    }
+#pragma unroll
+    for (int t = 0; t < 7; ++t) {
+      const bool has = kk[t] >= 0 && ((m >> (kk[t] >= 0 ? kk[t] : 0)) & 1u);
+      const int v = a.nbr[has ? (long long)kk[t] * n + orow : 0];
+      vv[t] = has ? v : -1;
+    }
+#pragma unroll
+    for (int t = 0; t < 7; ++t)
+      if (kk[t] >= 0 && g == 0) idxL[kk[t] * 32 + l32] = vv[t];
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();   // centre weights, centre rows and the index table are in LDS
+  f32x16 acc[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[nb][j] = 0.f;
+  if (wave < KS) {
+    const int s = wave;   // this wavefront's K step: input channels [16 s, 16 s + 16)
+    {
+      const half8 af = Pl[0][l32 * PPR + ((2 * s + g) ^ row_swizzle<PPR>(l32))];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+        acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(Wc[(2 * s + g) * (NB * 32) + nb * 32 + l32], af, acc[nb], 0, 0, 0);
+    }
+    // six offsets in flight (eight at 32 columns): slot j holds the row fragment, the row's index and the weight fragments of one offset
+    constexpr int SLOTS = NB == 2 ? 6 : 8;
+    half8 rf[SLOTS], wf[SLOTS][NB];
+    int ri[SLOTS];
+    unsigned rem_issue = u;
+    const half_t *Ab = A + s * 16 + g * 8;
+    const half_t *Wb = Wp + ((long long)(2 * s + g) * a.n_pad + l32) * 8;
+    // (every step issues its loads and its MFMAs unconditionally -- a slot beyond the last offset loads from a
+    // valid address and multiplies zeros -- so that the waits in front of the MFMAs are counted exactly and leave the
+    // loads of the three other slots in flight; with the loads under a condition every wait became a full one)
+#define PCE_OS2_ISSUE(J_)                                                                                          \
+  {                                                                                                                \
+    const int k_ = rem_issue ? __ffs((int)rem_issue) - 1 : 0;                                                      \
+    const int v_ = idxL[k_ * 32 + l32];                                                                            \
+    ri[J_] = rem_issue ? v_ : -1;                                                                                  \
+    rem_issue &= rem_issue - 1u;                                                                                   \
+    rf[J_] = *reinterpret_cast<const half8 *>(Ab + (long long)(ri[J_] >= 0 ? ri[J_] : 0) * a.lda);                 \
+    _Pragma("unroll") for (int nb = 0; nb < NB; ++nb)                                                              \
+      wf[J_][nb] = *reinterpret_cast<const half8 *>(Wb + k_ * wstep + nb * 32 * 8);                                \
+  }
+#define PCE_OS2_USE(J_)                                                                                            \
+  {                                                                                                                \
+    const half8 f_ = ri[J_] >= 0 ? rf[J_] : zero;                                                                  \
+    _Pragma("unroll") for (int nb = 0; nb < NB; ++nb)                                                              \
+      acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[J_][nb], f_, acc[nb], 0, 0, 0);                          \
+  }
+#pragma unroll
+    for (int j = 0; j < SLOTS; ++j) PCE_OS2_ISSUE(j)
+    for (int round = (__popc(u) + SLOTS - 1) / SLOTS; round > 0; --round) {   // wavefront-uniform
+#pragma unroll
+      for (int j = 0; j < SLOTS; ++j) {
+        __builtin_amdgcn_sched_barrier(0);
+        PCE_OS2_USE(j)
+        PCE_OS2_ISSUE(j)
+      }
+    }
+#undef PCE_OS2_ISSUE
+#undef PCE_OS2_USE
+  }
+  // wavefronts 1..3 hand their accumulators to wavefront 0, one 32-column block at a time through their own regions
+  // (wavefront 1's region holds the end of the index table: the first barrier below stands behind its last reader)
+  f32x16 *mine = reinterpret_cast<f32x16 *>(&Pl[wave][0]);
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    __syncthreads();
+    if (wave > 0 && wave < KS) mine[lane] = acc[nb];
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+      for (int w2 = 1; w2 < 4; ++w2) {
+        if (w2 < KS) {
+          const f32x16 other = reinterpret_cast<const f32x16 *>(&Pl[w2][0])[lane];
+#pragma unroll
+          for (int j = 0; j < 16; ++j) acc[nb][j] += other[j];
+        }
+      }
+    }
+  }
+  if (wave > 0) return;
+  float V[NB][2][8];
+  gather_row_pieces<NB>(acc, V, g);
+  if (a.bias || a.res || a.act) epilogue_row_pieces<half_t, NB, true>(V, a, orow, 0, g, a.act != PCE_ACT_NONE);
+  store_rows_via_lds<half_t, NB>(V, Pl[0], (half_t *)a.out, orow, a, 0, lane, l32, g, a.stream);
+}
+
+// the three-kind kernel over a row order, or (order == nullptr) its stream workgroups alone: a plain GEMM
+static int launch_wave_os2(const TileArgs &a, const int *order, int mid, long long n_out, long long n_nonzero, long long n_single,
+                           int nb, int ks, hipStream_t s) {
+  const long long n_plain = n_out - n_nonzero, n_shared = n_nonzero - n_single;
+  const long long shared_wgs = pce_div_up(n_shared, 32), single_wgs = pce_div_up(pce_div_up(n_single, 32), 4),
+                  stream_wgs = pce_div_up(pce_div_up(n_out, 64), 4);
+  if (shared_wgs + single_wgs + stream_wgs >= (1ll << 31) - 8) PCE_FAIL(PCE_ECAPACITY, "%lld rows exceed the grid limit", (long long)n_out);
+  const unsigned grid2 = (unsigned)(shared_wgs + single_wgs + stream_wgs);
+#define PCE_WOS2_CASE(NB_, KS_)                                                                                    \
+  if (nb == NB_ && ks == KS_) {                                                                                    \
+    hipLaunchKernelGGL((wave_os2_kernel<NB_, KS_>), dim3(grid2), dim3(256), 0, s, a, order, mid, n_plain, n_single, \
+                       (int)shared_wgs, (int)single_wgs);                                                          \
+    PCE_LAUNCH_CHECK("wave_os2");                                                                                  \
+    return PCE_OK;                                                                                                 \
+  }
+  PCE_WOS2_CASE(1, 1) PCE_WOS2_CASE(1, 2) PCE_WOS2_CASE(1, 3) PCE_WOS2_CASE(1, 4)
+  PCE_WOS2_CASE(2, 1) PCE_WOS2_CASE(2, 2) PCE_WOS2_CASE(2, 3) PCE_WOS2_CASE(2, 4)
+#undef PCE_WOS2_CASE
+  PCE_FAIL(PCE_EINVAL, "wave_os2: unsupported shape c_in=%d c_out=%d", a.c_in, a.c_out);
+}
+
 // The same dataflow for layers of 64 to 128 input and 65 to 128 output channels (fp16).  The weights of an offset
 // (12 to 24 KB) come straight from the packed copy in L2, all KS x NB fragments of the offset requested before the
 // first MFMA waits for one (in two batches where they would not leave three wavefronts per SIMD their registers);
@@ -2835,7 +3171,10 @@ static bool wave_os_ok(const TileArgs &a, int kv, int mid) {
 
 extern "C" int pce_conv_fwd_oso(const void *in, const void *w, const void *wp, void *out, int32_t dtype, int64_t n_in,
                                 int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv, int32_t mid, const int32_t *nbr,
-                                const int32_t *order, int64_t n_heavy, const pce_epilogue_t *epilogue, pce_stream_t stream) {
+                                const int32_t *order, const int64_t *order_counts, const pce_epilogue_t *epilogue,
+                                pce_stream_t stream) {
+  if (!order_counts) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: null order counts");
+  const int64_t n_heavy = order_counts[0], n_nonzero = order_counts[1], n_single = order_counts[2];
   int rc = check_common("pce_conv_fwd_oso", in, w, out, dtype, n_in, n_out, c_in, c_out, kv, mid);
   if (rc) return rc;
   if (!nbr || !order) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: null neighbour table or row order");
@@ -2855,6 +3194,11 @@ extern "C" int pce_conv_fwd_oso(const void *in, const void *w, const void *wp, v
                          "32 (multiples of 8), 16-byte aligned rows, kernel volumes up to 31; got dtype %d, %d -> %d channels, "
                          "kv %d, mid %d", (int)dtype, (int)c_in, (int)c_out, (int)kv, (int)mid);
   if (n_heavy < 0 || n_heavy > n_out) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: n_heavy=%lld outside [0, n_out]", (long long)n_heavy);
+  if (n_nonzero >= 0 && (n_nonzero < n_heavy || n_nonzero > n_out))
+    PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: n_nonzero=%lld outside [n_heavy, n_out]", (long long)n_nonzero);
+  if (n_nonzero >= 0 && n_single >= 0 && n_single > n_nonzero - n_heavy)
+    PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: n_single=%lld exceeds the %lld rows with one or two neighbours", (long long)n_single, (long long)(n_nonzero - n_heavy));
+  if ((uintptr_t)order & 15) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: the order array must be 16-byte aligned");
   a.nbr = nbr;
   a.n_rows = n_out;
   const long long n_main = n_out - n_heavy;
@@ -2892,6 +3236,14 @@ extern "C" int pce_conv_fwd_oso(const void *in, const void *w, const void *wp, v
 #undef PCE_WOSW_CASE
     PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: unsupported shape c_in=%d c_out=%d", (int)c_in, (int)c_out);
   }
+  // Clouds whose rows mostly have no neighbour, and few of them two or more: the three-kind kernel, the bulk streamed
+  // in storage order.  Needs the counts of rows with any neighbour and with exactly one; a caller that does not state
+  // them (-1), a layer without a centre offset and other clouds take the kernel that visits every row through the
+  // order.  Measured on prefixes of the 150 k-voxel scan, this kernel / that one: 7.9 / 10.0 us on 60 k rows (0.7 % of
+  // them with two neighbours or more), 10.0 / 10.2 on 90 k (3.5 %), 12.4 / 11.9 on all (4.1 %): the workgroups of
+  // shared rows are its longest chains, so it takes clouds with at most 1/32 of such rows.
+  if (mid >= 0 && n_nonzero >= 0 && n_single >= 0 && 2 * n_nonzero <= n_out && 32 * (n_nonzero - n_single) <= n_out && stage_on(12))
+    return launch_wave_os2(a, order, (int)mid, n_out, n_nonzero, n_single, nb, ks, s);
 #define PCE_WOS_CASE(NB_, KS_)                                                                              \
   if (nb == NB_ && ks == KS_) {                                                                              \
     hipLaunchKernelGGL((wave_os_kernel<NB_, KS_>), dim3(grid), dim3(256), 0, s, a, perm, rmask, (int)mid, n_main,   \
@@ -2914,6 +3266,10 @@ static int dense_impl(const void *in, const void *w, const void *wp, void *out, 
   a.n_rows = n;
   a.mode = MODE_DENSE;
   a.epi = EPI_ROWS;
+  // narrow fp16 layers: the stream workgroups of the three-kind ordered kernel alone (64 consecutive rows per
+  // wavefront, weights once per workgroup through LDS): 7.1 us on 150 k rows of 64 -> 64 channels, the tile kernel 8.3
+  if (sizeof(T) == 2 && wave_os_ok(a, 1, 0) && stage_on(12))
+    return launch_wave_os2(a, nullptr, 0, n, 0, 0, (c_out + 31) / 32, c_in / 16, s);
   return launch_tile<T>(a, pce_div_up(n, 128), s);
 }
 

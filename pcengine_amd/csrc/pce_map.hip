@@ -1636,8 +1636,12 @@ __global__ void __launch_bounds__(256) grid_query_kernel(const ProbDev *__restri
 __device__ __forceinline__ int order_key(unsigned m) {   // m != 0
   const int first = __ffs((int)m) - 1;
   const unsigned rest = m & (m - 1u);
-  const int second = rest ? __ffs((int)rest) - 1 : 31;
-  return (__popc(m) >= ORDER_HEAVY_POPC ? 1024 : 0) + first * 32 + second;
+  // rows with a single neighbour come first, by its offset (keys 0 .. 31); then the rows with two, by (lowest,
+  // second-lowest) offset (keys 32 .. 1023: first <= 29 whatever the kernel volume up to 31); then, from key 1024,
+  // the rows with ORDER_HEAVY_POPC or more, likewise
+  if (!rest) return first;
+  const int second = __ffs((int)rest) - 1;
+  return (__popc(m) >= ORDER_HEAVY_POPC ? 1024 : 0) + 32 + first * 32 + second;
 }
 
 // mask[row] = offsets (other than the centre) at which the row has a neighbour; hist[key] += the block's count.
@@ -1682,7 +1686,12 @@ __device__ __forceinline__ void order_scan_block(int *tail, int *n_heavy_out) {
   if (threadIdx.x == 1023) {
     tail[ORDER_N_NONZERO] = part[1023];
     tail[ORDER_N_HEAVY] = part[1023] - part[511];      // keys 1024 .. 2047 belong to threads 512 .. 1023
-    if (n_heavy_out) *n_heavy_out = part[1023] - part[511];
+    tail[ORDER_N_SINGLE] = part[32 / per - 1];          // keys 0 .. 31: rows with exactly one neighbour
+    if (n_heavy_out) {   // status words 4, 6 and 7 of a batched build
+      n_heavy_out[0] = part[1023] - part[511];
+      n_heavy_out[2] = part[1023];
+      n_heavy_out[3] = part[32 / per - 1];
+    }
   }
   int run = part[threadIdx.x] - sum;
 #pragma unroll
@@ -2246,8 +2255,8 @@ __global__ void __launch_bounds__(256) order_scatter_batch_kernel(const ProbDev 
 extern "C" int64_t pce_row_order_elems(int64_t n_rows) { return n_rows < 0 ? 0 : PCE_ORDER_ELEMS(n_rows); }
 
 extern "C" int pce_row_order(const int32_t *nbr, int32_t kv, int64_t n_rows, int32_t mid, int32_t *order, int64_t order_elems,
-                             int64_t *n_heavy_host, pce_stream_t stream) {
-  if (!nbr || !order || !n_heavy_host) PCE_FAIL(PCE_EINVAL, "pce_row_order: null pointer");
+                             int64_t *counts_host, pce_stream_t stream) {
+  if (!nbr || !order || !counts_host) PCE_FAIL(PCE_EINVAL, "pce_row_order: null pointer");
   if (kv < 1 || kv > ORDER_MAX_KV - 1) PCE_FAIL(PCE_EINVAL, "pce_row_order: kernel volume %d outside [1, %d]", (int)kv, ORDER_MAX_KV - 1);
   if (n_rows <= 0 || n_rows >= (1ll << 30)) PCE_FAIL(PCE_EINVAL, "pce_row_order: n_rows=%lld", (long long)n_rows);
   if (mid >= kv) PCE_FAIL(PCE_EINVAL, "pce_row_order: centre offset %d outside the kernel volume %d", (int)mid, (int)kv);
@@ -2265,10 +2274,13 @@ extern "C" int pce_row_order(const int32_t *nbr, int32_t kv, int64_t n_rows, int
   PCE_LAUNCH_CHECK("order_scan");
   hipLaunchKernelGGL(order_scatter_kernel, dim3(blocks), dim3(256), 0, s, (long long)n_rows, order, (const int *)nbr);
   PCE_LAUNCH_CHECK("order_scatter");
-  int heavy = 0;
-  PCE_HIP(hipMemcpyAsync(&heavy, tail + ORDER_N_HEAVY, sizeof(int), hipMemcpyDeviceToHost, s));
+  static_assert(ORDER_N_HEAVY == ORDER_N_NONZERO + 1 && ORDER_N_NONZERO == ORDER_N_SINGLE + 1, "the counts are read back in one copy");
+  int counts[3] = {0, 0, 0};
+  PCE_HIP(hipMemcpyAsync(counts, tail + ORDER_N_SINGLE, 3 * sizeof(int), hipMemcpyDeviceToHost, s));
   PCE_HIP(hipStreamSynchronize(s));
-  *n_heavy_host = heavy;
+  counts_host[0] = counts[2];   // rows with three neighbours or more
+  counts_host[1] = counts[1];   // rows with any neighbour
+  counts_host[2] = counts[0];   // rows with exactly one
   return PCE_OK;
 }
 

@@ -40,8 +40,12 @@ def _popcount(m):
 
 
 def _key(m):
+    """Sort key of a row with neighbours: rows with one neighbour by its offset, then rows with two by (lowest,
+    second-lowest) offset, then rows with three or more likewise."""
     bits = [k for k in range(27) if (int(m) >> k) & 1]
-    return (1024 if len(bits) >= 3 else 0) + bits[0] * 32 + (bits[1] if len(bits) > 1 else 31)
+    if len(bits) == 1:
+        return bits[0]
+    return (1024 if len(bits) >= 3 else 0) + 32 + bits[0] * 32 + bits[1]
 
 
 @pytest.mark.parametrize("cloud", sorted(CLOUDS))
@@ -66,6 +70,7 @@ def test_row_order_built_with_the_map_and_on_its_own(cloud):
         assert np.array_equal(got_masks, masks)
         assert np.array_equal(np.sort(perm), np.arange(n))
         assert m.order_heavy == int((pc >= 3).sum())
+        assert m.order_nonzero == int((pc >= 1).sum()) and m.order_single == int((pc == 1).sum())
         n_plain, n_heavy = int((pc == 0).sum()), int((pc >= 3).sum())
         sect = masks[perm]
         assert (sect[:n_plain] == 0).all() and (sect[n_plain:] != 0).all()
@@ -310,6 +315,53 @@ def test_ordered_dataflow_on_column_slices_and_the_selector():
     assert float((fds.float() - want.float()).norm() / want.float().norm()) <= 1e-3
 
 
+SPARSE_CLOUDS = {
+    "lidar": CLOUDS["lidar"],
+    "scan": lambda: synth.lidar_cloud()[:40000].copy(),       # the benchmark's cloud: a few heavy rows, mostly none
+    "thin": lambda: synth.random_cloud(seed=93, n=5000, extent=60, batches=2),   # 5 000 voxels in 2 x 60^3: nearly all alone
+}
+
+
+@pytest.mark.parametrize("cloud", sorted(SPARSE_CLOUDS))
+@pytest.mark.parametrize("c_in,c_out", [(64, 64), (32, 32), (16, 64), (48, 24), (64, 8)])
+def test_streamed_form_against_the_ordered_form(cloud, c_in, c_out):
+    """Clouds where at most half the rows have a neighbour run as three kinds of workgroup (rows without neighbours
+    streamed in storage order, rows with one by their records, the rest shared by four wavefronts): against the
+    oracle, and against the kernel that visits every row through the order (what the same call runs when the count
+    of rows with neighbours is not stated) -- bit-identical on rows with at most one neighbour, to rounding on the
+    others --, with and without the epilogue."""
+    coords = SPARSE_CLOUDS[cloud]()
+    ref, masks = _oracle_masks(coords)
+    km = _subm(coords)
+    n = len(coords)
+    assert km.order_nonzero == int((masks != 0).sum()) and 2 * km.order_nonzero <= n
+    many = torch.as_tensor(_popcount(masks) >= 2, device=DEV)
+    dt = torch.float16
+    f, w = synth.features(c_in + 1, n, c_in), synth.weights(c_out + 2, 27, c_in, c_out)
+    fd, wd = torch.as_tensor(f, device=DEV).to(dt), torch.as_tensor(w, device=DEV).to(dt)
+    bd = torch.as_tensor(np.random.default_rng(5).standard_normal(c_out) * 0.1, device=DEV).to(dt)
+    rd = torch.as_tensor(synth.features(c_out + 3, n, c_out), device=DEV).to(dt)
+    packed = backend.pack_weights(wd)
+    want = orc.conv_forward(rounded(f, dt), rounded(w, dt), ref, K3)
+    for kw in ({}, dict(bias=bd, residual=rd, act="relu")):
+        new = backend.conv_forward(fd, wd, km, DATAFLOW_OSO, packed=packed, **kw)
+        nonzero, km.order_nonzero = km.order_nonzero, -1
+        old = backend.conv_forward(fd, wd, km, DATAFLOW_OSO, packed=packed, **kw)
+        km.order_nonzero = nonzero
+        # rows with two neighbours or more are summed channel quarter by channel quarter here, offset by offset there
+        assert torch.equal(new[~many], old[~many])
+        assert torch.allclose(new[many].float(), old[many].float(), rtol=4e-3, atol=2e-3)
+        if not kw:
+            assert orc.rel_l2(new.double().cpu().numpy(), want) <= 1e-3
+    # rows in a wider matrix, in and out
+    wide_in = torch.full((n, c_in + 16), 7.0, dtype=dt, device=DEV)
+    wide_in[:, 8:8 + c_in] = fd
+    wide_out = torch.full((n, c_out + 24), -3.0, dtype=dt, device=DEV)
+    got = backend.conv_forward(wide_in[:, 8:8 + c_in], wd, km, DATAFLOW_OSO, packed=packed, out=wide_out[:, 16:16 + c_out])
+    assert torch.equal(got, backend.conv_forward(fd, wd, km, DATAFLOW_OSO, packed=packed))
+    assert bool((wide_out[:, :16] == -3.0).all()) and bool((wide_out[:, 16 + c_out:] == -3.0).all())
+
+
 def test_ordered_dataflow_argument_errors():
     lib = _lib.load()
     coords = CLOUDS["tiny"]()
@@ -320,10 +372,14 @@ def test_ordered_dataflow_argument_errors():
     w = torch.zeros((27, 32, 32), dtype=torch.float16, device=DEV)
     pk = backend.pack_weights(w)
     out = torch.zeros((n, 32), dtype=torch.float16, device=DEV)
-    call = lambda dtype, c_in, c_out, mid, heavy, packed=pk: lib.pce_conv_fwd_oso(
+    call = lambda dtype, c_in, c_out, mid, heavy, packed=pk, nonzero=-1, single=-1: lib.pce_conv_fwd_oso(
         f.data_ptr(), w.data_ptr(), packed.data_ptr() if packed is not None else None, out.data_ptr(), dtype, n, n, c_in, c_out, 27, mid,
-        km.nbr_out.data_ptr(), km.order.data_ptr(), heavy, None, s)
+        km.nbr_out.data_ptr(), km.order.data_ptr(), (_lib.c_int64 * 3)(heavy, nonzero, single), None, s)
     assert call(_lib.PCE_F16, 32, 32, 13, km.order_heavy) == _lib.PCE_OK
+    assert call(_lib.PCE_F16, 32, 32, 13, km.order_heavy, nonzero=km.order_nonzero, single=km.order_single) == _lib.PCE_OK
+    assert call(_lib.PCE_F16, 32, 32, 13, km.order_heavy, nonzero=km.order_heavy - 1) == _lib.PCE_EINVAL   # fewer than the heavy rows
+    assert call(_lib.PCE_F16, 32, 32, 13, km.order_heavy, nonzero=n + 1) == _lib.PCE_EINVAL
+    assert call(_lib.PCE_F16, 32, 32, 13, km.order_heavy, nonzero=km.order_nonzero, single=km.order_nonzero + 1) == _lib.PCE_EINVAL
     assert call(_lib.PCE_F32, 64, 32, 13, km.order_heavy) == _lib.PCE_EINVAL        # fp32 stops at 32 channels
     assert call(_lib.PCE_F32, 12, 32, 13, km.order_heavy) == _lib.PCE_EINVAL        # ... in multiples of 8
     assert call(_lib.PCE_F32, 32, 32, -1, km.order_heavy) == _lib.PCE_EINVAL        # fp32 needs a centre offset
@@ -331,7 +387,7 @@ def test_ordered_dataflow_argument_errors():
     assert call(_lib.PCE_F16, 32, 32, 13, km.order_heavy, None) == _lib.PCE_EINVAL    # weights not packed
     assert call(_lib.PCE_F16, 128, 32, 13, km.order_heavy) == _lib.PCE_EINVAL
     assert call(_lib.PCE_F16, 128, 128, 13, km.order_heavy) == _lib.PCE_EINVAL       # beyond the K-stepped kernel's shapes
-    heavy = _lib.c_int64(0)
+    heavy = (_lib.c_int64 * 3)()
     order = torch.zeros(lib.pce_row_order_elems(n), dtype=torch.int32, device=DEV)
     assert lib.pce_row_order(km.nbr_out.data_ptr(), 27, n, 13, order.data_ptr(), order.numel() - 1, heavy, s) == _lib.PCE_EWORKSPACE
     assert lib.pce_row_order(km.nbr_out.data_ptr(), 125, n, 62, order.data_ptr(), order.numel(), heavy, s) == _lib.PCE_EINVAL
