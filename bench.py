@@ -463,10 +463,26 @@ def main() -> int:
             else:
                 os.environ["PCENGINE_DATAFLOW"] = name
             y0 = forward()
+            if name == "auto":
+                y_auto = y0.feats.clone()
             full = ev_ms(forward, 10, 2)
             cached = ev_ms(lambda: forward(y0), 20, 3)
             net[name] = {"forward_ms_with_map_build": round(full, 4), "forward_ms_cached_maps": round(cached, 4)}
         os.environ.pop("PCENGINE_DATAFLOW", None)
+        # the same forward with the maps of every cloud built through the native planner (one allocation for all maps,
+        # two library calls) and the layer outputs cut from one arena: no device allocation in a forward
+        model.use_planner()
+        for _ in range(3):
+            forward()
+        if not torch.equal(forward().feats, y_auto):
+            raise RuntimeError("the planned forward and the plain forward differ")
+        net["auto"]["forward_ms_with_map_build_planned"] = round(ev_ms(forward, 20, 3), 4)
+        torch.cuda.synchronize()
+        n_alloc = torch.cuda.memory_stats()["allocation.all.allocated"]
+        forward()
+        torch.cuda.synchronize()
+        net["auto"]["device_allocations_in_a_planned_forward"] = int(torch.cuda.memory_stats()["allocation.all.allocated"] - n_alloc)
+        model.use_planner(False)
         # a serving loop that knows its next cloud: the maps of cloud i+1 are built on a second stream while the
         # network runs cloud i (every forward still builds all nine maps of its own cloud)
         from pcengine_amd.spconv import MapPrefetcher

@@ -133,6 +133,11 @@ int pce_outcoords_chain_plan(int64_t n_in, int32_t levels, const pce_geom_t *geo
 int pce_outcoords_chain(const int32_t *in_coords_dev, int64_t n_in, int32_t levels, const pce_geom_t *geoms,
                         int32_t n_batch, void *const *ws_dev, const int64_t *ws_bytes, int32_t *const *out_coords_dev,
                         int64_t *n_out_host, pce_stream_t stream);
+/* The same through workspaces laid out for n_plan >= n_in rows (pce_outcoords_chain_plan(n_plan, ...)): whether a level
+ * takes the bitmap depends on the row count, and a plan kept for several clouds must not change its mind. */
+int pce_outcoords_chain_planned(const int32_t *in_coords_dev, int64_t n_in, int64_t n_plan, int32_t levels,
+                                const pce_geom_t *geoms, int32_t n_batch, void *const *ws_dev, const int64_t *ws_bytes,
+                                int32_t *const *out_coords_dev, int64_t *n_out_host, pce_stream_t stream);
 
 /* ---- voxelisation ----------------------------------------------------------------------------- *
  * Replaces sparse_quantize + ravel_hash (script/utils.py:18-55), which the reference runs in NumPy
@@ -236,6 +241,53 @@ int pce_kmap_build_batch(const pce_kmap_problem_t *problems_host, int32_t n_prob
 #define PCE_KMAP_TABLE_ONLY 2
 int64_t pce_kmap_workspace_bytes_grid(int64_t n_in, int64_t n_out, const pce_geom_t *g, int32_t n_batch,
                                       int32_t want_csr);
+
+/* ---- the maps of a whole network in one allocation and two calls ------------------------------- *
+ * The reference builds a network's maps layer by layer as its forward pass meets them, each with its own
+ * allocations (script/spconv.py:331-437; scratch sizing script/sptensor.py:63-78).  pce_pyramid_plan lays the
+ * output coordinates of the strided levels (the chain of pce_outcoords_chain: kernel = stride, no padding, batch
+ * count stated) and every requested map out in ONE allocation from upper bounds: level 0 holds at most n_cap rows,
+ * level l + 1 at most what pce_outcoords_chain_plan reports for it.  A request names the levels its map reads and
+ * writes (equal for a submanifold map; level_out = level_in + 1 for the map of a strided level, whose geometry
+ * repeats strided[level_in]) and what it wants beside pair lists, output-major table and row order.  The plan is
+ * plain data the caller keeps; arena_bytes is the size of the device allocation it needs (256-byte aligned).
+ * pce_pyramid_build then builds everything for one cloud of at most n_cap rows into that allocation -- the chained
+ * coordinates, one wait for their counts, all maps in the launches of one batched build, one wait for their counts
+ * -- and fills level_n and, per map, n_in / n_out / n_pairs / qsum and the host copy `meta` = knnz[kv] | kpos[kv+1] |
+ * qkpos[kv+1] | status[8]; the arrays of map i start at arena + map[i].off[...] (-1: not requested), the
+ * coordinates of level l >= 1 at arena + off_coords[l].  PCE_CHAIN_NOT_APPLICABLE (plan) and PCE_PYR_UNSORTED (build:
+ * a map found rows unsorted or outside the stated box) tell the caller to build that cloud level by level. */
+#define PCE_PYR_MAX_LEVELS 8
+#define PCE_PYR_MAX_MAPS 16
+#define PCE_PYR_UNSORTED 101
+enum { PCE_PYR_IMAP = 0, PCE_PYR_OMAP, PCE_PYR_NBR_OUT, PCE_PYR_NBR_IN, PCE_PYR_ORDER, PCE_PYR_ICSR, PCE_PYR_OCSR, PCE_PYR_ICODE,
+       PCE_PYR_OCODE, PCE_PYR_ISLOT, PCE_PYR_OSLOT, PCE_PYR_META, PCE_PYR_WS, PCE_PYR_ARRAYS };
+typedef struct pce_pyr_request {
+  int32_t level_in, level_out;
+  pce_geom_t geom;
+  int32_t want_csr, want_nbr_in, table_only, pad;
+} pce_pyr_request_t;
+typedef struct pce_pyr_map {
+  int64_t off[PCE_PYR_ARRAYS];
+  int64_t cap_in, cap_out, ws_bytes;
+  int64_t n_in, n_out, n_pairs, qsum;   /* filled by pce_pyramid_build */
+  int32_t meta[3 * 31 + 2 + 8];
+  int32_t kv;
+} pce_pyr_map_t;
+typedef struct pce_pyr_plan {
+  int32_t n_levels, n_maps, n_batch, pad;
+  pce_geom_t strided[PCE_PYR_MAX_LEVELS];
+  int64_t level_cap[PCE_PYR_MAX_LEVELS + 1], level_n[PCE_PYR_MAX_LEVELS + 1];
+  int64_t off_coords[PCE_PYR_MAX_LEVELS + 1], off_chain_ws[PCE_PYR_MAX_LEVELS], chain_ws_bytes[PCE_PYR_MAX_LEVELS];
+  int64_t off_meta, meta_bytes, arena_bytes;
+  pce_pyr_request_t req[PCE_PYR_MAX_MAPS];
+  pce_pyr_map_t map[PCE_PYR_MAX_MAPS];
+} pce_pyr_plan_t;
+int64_t pce_pyramid_plan_sizeof(void);   /* sizeof(pce_pyr_plan_t) as this library was compiled: a binding checks its own */
+int pce_pyramid_plan(int64_t n_cap, int32_t n_levels, const pce_geom_t *strided, int32_t n_batch,
+                     const pce_pyr_request_t *requests, int32_t n_requests, pce_pyr_plan_t *plan_out);
+int pce_pyramid_build(pce_pyr_plan_t *plan, const int32_t *in_coords_dev, int64_t n_in, void *arena_dev, int64_t arena_bytes,
+                      pce_stream_t stream);
 
 /* ---- forward convolution --------------------------------------------------------------------- *
  * Common arguments: in_feats[n_in,c_in], weight[kv,c_in,c_out], out_feats[n_out,c_out], all of

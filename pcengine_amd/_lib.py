@@ -46,6 +46,35 @@ class KmapProblem(Structure):
                 [("n_batch", c_int32), ("flags", c_int32), ("order", c_void_p)])
 
 
+PYR_MAX_LEVELS, PYR_MAX_MAPS, PYR_UNSORTED = 8, 16, 101
+(PYR_IMAP, PYR_OMAP, PYR_NBR_OUT, PYR_NBR_IN, PYR_ORDER, PYR_ICSR, PYR_OCSR, PYR_ICODE, PYR_OCODE, PYR_ISLOT, PYR_OSLOT, PYR_META,
+ PYR_WS, PYR_ARRAYS) = range(14)
+
+
+class PyrRequest(Structure):
+    """pce_pyr_request_t: one map of a network's pyramid."""
+    _fields_ = [("level_in", c_int32), ("level_out", c_int32), ("geom", Geom), ("want_csr", c_int32), ("want_nbr_in", c_int32),
+                ("table_only", c_int32), ("pad", c_int32)]
+
+
+class PyrMap(Structure):
+    """pce_pyr_map_t: where the arrays of one map live in the arena, and what its build counted."""
+    _fields_ = [("off", c_int64 * PYR_ARRAYS), ("cap_in", c_int64), ("cap_out", c_int64), ("ws_bytes", c_int64),
+                ("n_in", c_int64), ("n_out", c_int64), ("n_pairs", c_int64), ("qsum", c_int64),
+                ("meta", c_int32 * (3 * 31 + 2 + 8)), ("kv", c_int32)]
+
+
+class PyrPlan(Structure):
+    """pce_pyr_plan_t."""
+    _fields_ = [("n_levels", c_int32), ("n_maps", c_int32), ("n_batch", c_int32), ("pad", c_int32),
+                ("strided", Geom * PYR_MAX_LEVELS),
+                ("level_cap", c_int64 * (PYR_MAX_LEVELS + 1)), ("level_n", c_int64 * (PYR_MAX_LEVELS + 1)),
+                ("off_coords", c_int64 * (PYR_MAX_LEVELS + 1)), ("off_chain_ws", c_int64 * PYR_MAX_LEVELS),
+                ("chain_ws_bytes", c_int64 * PYR_MAX_LEVELS),
+                ("off_meta", c_int64), ("meta_bytes", c_int64), ("arena_bytes", c_int64),
+                ("req", PyrRequest * PYR_MAX_MAPS), ("map", PyrMap * PYR_MAX_MAPS)]
+
+
 class Epilogue(Structure):
     """pce_epilogue_t: out = act(conv + bias + residual)."""
     _fields_ = [("bias", c_void_p), ("residual", c_void_p), ("act", c_int32), ("slope", ctypes.c_float),
@@ -72,6 +101,8 @@ _SIGNATURES = {
     "pce_outcoords_chain_plan": (c_int32, [c_int64, c_int32, POINTER(Geom), c_int32, POINTER(c_int64), POINTER(c_int64)]),
     "pce_outcoords_chain": (c_int32, [c_void_p, c_int64, c_int32, POINTER(Geom), c_int32, POINTER(c_void_p), POINTER(c_int64),
                                       POINTER(c_void_p), POINTER(c_int64), c_void_p]),
+    "pce_outcoords_chain_planned": (c_int32, [c_void_p, c_int64, c_int64, c_int32, POINTER(Geom), c_int32, POINTER(c_void_p),
+                                              POINTER(c_int64), POINTER(c_void_p), POINTER(c_int64), c_void_p]),
     "pce_voxelize_workspace_bytes": (c_int64, [c_int64]),
     "pce_voxelize": (c_int32, [c_void_p, c_int32, c_int64, POINTER(ctypes.c_double), c_void_p, c_int64, POINTER(c_int64),
                                POINTER(c_int32), POINTER(c_int32), c_void_p]),
@@ -116,6 +147,9 @@ _SIGNATURES = {
     "pce_conv_fwd_dense": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32, POINTER(Epilogue), c_void_p]),
     "pce_conv_wgrad": (c_int32, [c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p,
                                  c_void_p, c_void_p, c_int64, c_void_p, c_void_p]),
+    "pce_pyramid_plan_sizeof": (c_int64, []),
+    "pce_pyramid_plan": (c_int32, [c_int64, c_int32, POINTER(Geom), c_int32, POINTER(PyrRequest), c_int32, POINTER(PyrPlan)]),
+    "pce_pyramid_build": (c_int32, [POINTER(PyrPlan), c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
     "pce_select_dataflow": (c_int32, [c_int64, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32]),
 }
 

@@ -35,6 +35,8 @@ def _ptr(t: Optional[torch.Tensor]):
 
 
 def _stream(device) -> int:
+    if _arena is not None and _arena.stream_device == device:      # inside allocate_from: looked up once per forward
+        return _arena.stream
     return torch.cuda.current_stream(device).cuda_stream
 
 
@@ -75,8 +77,12 @@ class _Cut:
         if self.pairs and not obj.__dict__.get("has_pairs", True):
             ensure_pairs(obj)
         v = obj.__dict__.get(self.slot)
-        if isinstance(v, tuple):         # (array at capacity, pair count)
-            v = v[0][:v[1]]
+        if isinstance(v, tuple):
+            if len(v) == 2:              # (array at capacity, count)
+                v = v[0][:v[1]]
+            else:                        # (int32 view of an arena, first element, count[, shape]): a map of a PyramidPlan
+                t = v[0][v[1]:v[1] + v[2]]
+                v = t.view(v[3]) if len(v) > 3 else t
             obj.__dict__[self.slot] = v
         return v
 
@@ -103,21 +109,21 @@ class KernelMap:
     qsum: int
     imap: torch.Tensor = _Cut(False, pairs=True)
     omap: torch.Tensor = _Cut(False, pairs=True)
-    knnz: torch.Tensor
-    kpos: torch.Tensor
-    qkpos: torch.Tensor
-    out_coords: torch.Tensor
-    nbr_out: Optional[torch.Tensor] = None
-    nbr_in: Optional[torch.Tensor] = None
-    icsr: Optional[torch.Tensor] = None
+    knnz: torch.Tensor = _Cut(False)
+    kpos: torch.Tensor = _Cut(False)
+    qkpos: torch.Tensor = _Cut(False)
+    out_coords: torch.Tensor = _Cut(False)
+    nbr_out: Optional[torch.Tensor] = _Cut(True)
+    nbr_in: Optional[torch.Tensor] = _Cut(True)
+    icsr: Optional[torch.Tensor] = _Cut(True)
     icode: Optional[torch.Tensor] = _Cut(True)
-    ocsr: Optional[torch.Tensor] = None
+    ocsr: Optional[torch.Tensor] = _Cut(True)
     ocode: Optional[torch.Tensor] = _Cut(True)
     islot: Optional[torch.Tensor] = _Cut(True)   # pair -> position of its entry in icode / ocode
     oslot: Optional[torch.Tensor] = _Cut(True)
     route: Optional[torch.Tensor] = None   # routing array of a layer without centre offset (pair_route), built on first use
     route_t: Optional[torch.Tensor] = None # the same for the transposed layer over this map
-    order: Optional[torch.Tensor] = None   # rows in neighbour-pattern order and their offset masks (row_order), built on first use
+    order: Optional[torch.Tensor] = _Cut(True)   # rows in neighbour-pattern order and their offset masks (row_order), built on first use
     order_heavy: int = 0                   # how many rows of that order have three neighbours or more (its last part)
     order_nonzero: int = -1                # how many have any neighbour (-1: not known)
     order_single: int = -1                 # how many have exactly one (-1: not known)
@@ -138,7 +144,10 @@ class KernelMap:
         """Tensors that cover the device allocations this map reads (views share them): what another stream has to
         be told about (``Tensor.record_stream``) before it uses a map whose memory was allocated on this one."""
         pair_arrays = self.__dict__.get("_cut_imap")
-        first = pair_arrays[0] if isinstance(pair_arrays, tuple) else pair_arrays
+        first = pair_arrays[0] if isinstance(pair_arrays, tuple) else pair_arrays     # (for a planned map: the arena)
+        arena = self.__dict__.get("_arena")
+        if arena is not None:
+            return [t for t in (arena, self.route, self.route_t) if t is not None]
         return [t for t in (first, self.knnz, self.out_coords, self.nbr_out, self.nbr_in, self.icsr, self.route, self.route_t)
                 if t is not None]
 
@@ -468,6 +477,178 @@ def build_kernel_map(in_coords: torch.Tensor, ks, stride, pad, cmin, cmax_out, s
                                    want_pairs=want_pairs)], defer=defer)[0]
 
 
+class ForwardArena:
+    """One device allocation the layer outputs of a forward pass are cut from, in the order the layers ask
+    (``allocate_from``), plus one staging buffer all layers share (the reference's ``spTensor.buffer``,
+    script/sptensor.py:63-78).  The first forward over a cloud measures what the network asks for; the arena is then
+    sized with headroom, and forwards that fit it allocate nothing.  A request that does not fit (a larger cloud) is
+    served by ``torch.empty`` and the arena grows before the next forward.  Tensors cut from it, the network's output
+    included, are valid until the next ``begin()``.  ``limit`` bounds the arena; a forward that needs more keeps
+    ``torch.empty`` for what does not fit."""
+
+    def __init__(self, device, limit: int = 8 << 30, headroom: float = 1.125):
+        self.device, self.limit, self.headroom = torch.device(device), int(limit), headroom
+        self.buf = None
+        self.off = self.need = 0
+        self.scratch = None
+        self.stream, self.stream_device = 0, None
+
+    def begin(self) -> None:
+        want = min(int(self.need * self.headroom), self.limit)
+        if self.need and (self.buf is None or self.buf.numel() < min(self.need, self.limit)):
+            self.buf = None        # release before the larger one is taken
+            self.buf = torch.empty(want, dtype=torch.uint8, device=self.device)
+        self.off = self.need = 0
+
+    def empty(self, shape, dtype, device) -> torch.Tensor:
+        shape = (shape,) if isinstance(shape, int) else tuple(shape)
+        numel = 1
+        for d in shape:
+            numel *= int(d)
+        nbytes = numel * _ITEMSIZE[dtype]
+        start = self.need
+        self.need = start + (nbytes + 255) // 256 * 256
+        if self.buf is None or self.need > self.buf.numel() or torch.device(device) != self.device:
+            return torch.empty(shape, dtype=dtype, device=device)
+        return self.buf[start:start + nbytes].view(dtype).view(shape)
+
+    def staging(self, numel: int, dtype, device) -> torch.Tensor:
+        """The shared staging buffer, at least ``numel`` elements of ``dtype`` (grown when a layer needs more)."""
+        nbytes = int(numel) * _ITEMSIZE[dtype]
+        if self.scratch is None or self.scratch.numel() < nbytes or self.scratch.device != torch.device(device):
+            self.scratch = None
+            self.scratch = torch.empty(int(nbytes * self.headroom) + 256, dtype=torch.uint8, device=device)
+        return self.scratch[:nbytes].view(dtype)
+
+
+_ITEMSIZE = {torch.float16: 2, torch.bfloat16: 2, torch.float32: 4, torch.float64: 8, torch.int32: 4, torch.int64: 8, torch.uint8: 1}
+_arena: Optional[ForwardArena] = None
+
+
+class allocate_from:
+    """Context manager: inside it the outputs, routing arrays and staging buffers of the forward operators of this
+    module come from ``arena`` (a ``ForwardArena``) and not from ``torch.empty``.  Not for concurrent use."""
+
+    def __init__(self, arena: Optional[ForwardArena]):
+        self.arena = arena
+
+    def __enter__(self):
+        global _arena
+        self.prev, _arena = _arena, None
+        if self.arena is not None:
+            self.arena.begin()
+            # the stream the forward runs on: the current one as the forward starts (a forward that switches streams
+            # inside the context is not served)
+            self.arena.stream_device = self.arena.device
+            self.arena.stream = torch.cuda.current_stream(self.arena.device).cuda_stream
+        _arena = self.arena
+        return self.arena
+
+    def __exit__(self, *exc):
+        global _arena
+        _arena = self.prev
+
+
+def _new(shape, dtype, device) -> torch.Tensor:
+    """Uninitialised device memory for an operator's output: from the active arena, else from torch."""
+    if _arena is not None:
+        return _arena.empty(shape, dtype, device)
+    return torch.empty(shape, dtype=dtype, device=device)
+
+
+def _staging(numel: int, dtype, device) -> torch.Tensor:
+    if _arena is not None:
+        return _arena.staging(numel, dtype, device)
+    return torch.empty(max(int(numel), 1), dtype=dtype, device=device)
+
+
+class PlanNotApplicable(Exception):
+    """The native planner does not take this pyramid (a level that is not a bitmap chain, an unsorted cloud): the
+    caller builds map by map."""
+
+
+class PyramidPlan:
+    """All kernel maps of a network on one cloud in ONE device allocation and two library calls
+    (``pce_pyramid_plan`` / ``pce_pyramid_build``): the chained output coordinates of the strided levels and every
+    requested map, laid out from upper bounds so that nothing is allocated, sized or described by the host between
+    the two waits for counts.  ``requests``: (level_in, level_out, ks, stride, pad, cmin, cmax_out, subm, want_csr,
+    want_nbr_in, table_only) per map; ``strided``: the geometry of every strided level, in order.  The plan serves
+    any cloud of at most ``n_cap`` rows inside the same box; the maps of a build live in the plan's arena and are
+    valid until its next build."""
+
+    def __init__(self, n_cap: int, strided: Sequence[Geom], requests: Sequence[tuple], n_batch: int, device):
+        lib = _lib.load()
+        if lib.pce_pyramid_plan_sizeof() != _lib.ctypes.sizeof(_lib.PyrPlan):
+            raise _lib.PCEError("pce_pyr_plan_t of the library and of this binding differ")
+        if len(strided) > _lib.PYR_MAX_LEVELS or not 0 < len(requests) <= _lib.PYR_MAX_MAPS or n_batch <= 0:
+            raise PlanNotApplicable()
+        self.plan = _lib.PyrPlan()
+        self.args = []
+        reqs = (_lib.PyrRequest * len(requests))()
+        for r, (lin, lout, ks, stride, pad, cmin, cmax_out, subm, want_csr, want_nbr_in, table_only) in zip(reqs, requests):
+            kv = int(ks[0]) * int(ks[1]) * int(ks[2])
+            if kv > 31:
+                raise PlanNotApplicable()
+            r.level_in, r.level_out = lin, lout
+            r.geom = Geom.make(ks, stride, pad, cmin, cmax_out, subm)
+            r.want_csr, r.want_nbr_in, r.table_only = int(want_csr), int(want_nbr_in), int(table_only)
+            self.args.append((tuple(ks), tuple(stride), tuple(pad), list(cmin), list(cmax_out), bool(subm)))
+        garr = (Geom * max(len(strided), 1))(*strided)
+        rc = lib.pce_pyramid_plan(int(n_cap), len(strided), garr, int(n_batch), reqs, len(requests), self.plan)
+        if rc == CHAIN_NOT_APPLICABLE:
+            raise PlanNotApplicable()
+        _lib.check(rc)
+        self.n_cap, self.n_batch, self.device = int(n_cap), int(n_batch), device
+        self.arena = torch.empty(self.plan.arena_bytes, dtype=torch.uint8, device=device)
+        self.arena32 = self.arena.view(torch.int32)
+
+    def build(self, in_coords: torch.Tensor):
+        """(coordinates of every level, the maps in request order) for one cloud.  Raises ``PlanNotApplicable`` when
+        the cloud has more rows than the plan or its rows are not sorted inside the stated box."""
+        lib = _lib.load()
+        _require_cuda(in_coords, "coords")
+        n = in_coords.shape[0]
+        if n > self.n_cap or n == 0 or in_coords.dtype != torch.int32 or not in_coords.is_contiguous():
+            raise PlanNotApplicable()
+        plan = self.plan
+        rc = lib.pce_pyramid_build(plan, in_coords.data_ptr(), n, self.arena.data_ptr(), self.arena.numel(), _stream(in_coords.device))
+        if rc in (_lib.PYR_UNSORTED, CHAIN_NOT_APPLICABLE) or (rc == _lib.PCE_EINVAL and b"n_batch" in lib.pce_last_error()):
+            raise PlanNotApplicable()
+        _lib.check(rc)
+        a32 = self.arena32
+        coords = [in_coords]
+        for l in range(1, plan.n_levels + 1):
+            nl = plan.level_n[l]
+            coords.append(a32[plan.off_coords[l] // 4:plan.off_coords[l] // 4 + 4 * nl].view(nl, 4))
+        maps = []
+        for i in range(plan.n_maps):
+            m, r = plan.map[i], plan.req[i]
+            kv, n_in, n_out, M = m.kv, m.n_in, m.n_out, m.n_pairs
+            meta = m.meta[:3 * kv + 2 + 8]
+            st = meta[3 * kv + 2:]
+            off = m.off
+            at = lambda a, count: None if off[a] < 0 else (a32, off[a] // 4, count)
+            mo = off[_lib.PYR_META] // 4
+            has_pairs = not st[5]
+            ks, stride, pad, cmin, cmax_out, subm = self.args[i]
+            order = at(_lib.PYR_ORDER, lib.pce_row_order_elems(n_out)) if off[_lib.PYR_ORDER] >= 0 else None
+            km = KernelMap(ks=ks, stride=stride, pad=pad, subm=subm, n_in=n_in, n_out=n_out, kv=kv, M=M, qsum=m.qsum,
+                           imap=at(_lib.PYR_IMAP, M), omap=at(_lib.PYR_OMAP, M), knnz=(a32, mo, kv), kpos=(a32, mo + kv, kv + 1),
+                           qkpos=(a32, mo + 2 * kv + 1, kv + 1), out_coords=coords[r.level_out],
+                           nbr_out=at(_lib.PYR_NBR_OUT, kv * n_out), nbr_in=at(_lib.PYR_NBR_IN, kv * n_in),
+                           icsr=at(_lib.PYR_ICSR, n_in + 1), ocsr=at(_lib.PYR_OCSR, n_out + 1), icode=at(_lib.PYR_ICODE, M),
+                           ocode=at(_lib.PYR_OCODE, M), islot=at(_lib.PYR_ISLOT, M), oslot=at(_lib.PYR_OSLOT, M),
+                           in_coords=coords[r.level_in], geom=r.geom, knnz_host=meta[:kv], order=order,
+                           order_heavy=st[4] if order is not None else 0, has_pairs=has_pairs, batchsize=self.n_batch,
+                           order_nonzero=st[6] if order is not None else -1, order_single=st[7] if order is not None else -1)
+            km._cmin, km._cmax = cmin, cmax_out
+            km.kpos_host = (_lib.c_int32 * (kv + 1))(*meta[kv:2 * kv + 1])
+            km.qkpos_host = (_lib.c_int32 * (kv + 1))(*meta[2 * kv + 1:3 * kv + 2])
+            km._arena = self.arena
+            maps.append(km)
+        return coords, maps
+
+
 def ensure_pairs(km: KernelMap) -> None:
     """Pair lists of a map that was built without them (first use of a dataflow that reads them)."""
     if km.has_pairs:
@@ -502,7 +683,7 @@ def pair_route(km: KernelMap, transposed: bool = False) -> torch.Tensor:
         lib = _lib.load()
         omap, oslot, ocsr, n_out = (km.imap, km.islot, km.icsr, km.n_in) if transposed else (km.omap, km.oslot, km.ocsr, km.n_out)
         elems = lib.pce_pair_route_elems(km.M, n_out)
-        route = torch.empty(elems, dtype=torch.int32, device=omap.device)
+        route = _new(elems, torch.int32, omap.device)
         _lib.check(lib.pce_pair_route(omap.data_ptr(), oslot.data_ptr(), ocsr.data_ptr(), km.M, n_out,
                                       route.data_ptr(), elems, _stream(omap.device)))
         if transposed:
@@ -639,7 +820,7 @@ def dense_forward(feats: torch.Tensor, weight: torch.Tensor, packed: Optional[to
     weight = weight.contiguous()
     if feats.shape[1] != weight.shape[0]:
         raise ValueError("Input feature size and kernel size mismatch")
-    out = torch.empty((feats.shape[0], weight.shape[1]), dtype=feats.dtype, device=feats.device)
+    out = _new((feats.shape[0], weight.shape[1]), feats.dtype, feats.device)
     epi, _keep = _epilogue(feats, feats.shape[0], weight.shape[1], bias, residual, act)
     _lib.check(lib.pce_conv_fwd_dense(feats.data_ptr(), weight.data_ptr(), _ptr(packed), out.data_ptr(), _dtype_code(feats),
                                       feats.shape[0], feats.shape[1], weight.shape[1], epi, _stream(feats.device)))
@@ -689,7 +870,7 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
     mid = _mid(km.ks) if km.subm else -1
     ld_out, slice_out = 0, None
     if out is None:
-        out = torch.empty((n_out, c_out), dtype=feats.dtype, device=dev)
+        out = _new((n_out, c_out), feats.dtype, dev)
     elif out.shape != (n_out, c_out) or out.dtype != feats.dtype or out.device != dev:
         raise ValueError(f"out must be a [{n_out}, {c_out}] {feats.dtype} tensor on {dev}")
     elif not out.is_contiguous():
@@ -699,7 +880,7 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
                              "row stride and width multiples of 8 elements)")
         if not strided_ok:       # this dataflow stores dense rows: they are copied into the slice afterwards
             slice_out, ld_out = out, 0
-            out = torch.empty((n_out, c_out), dtype=feats.dtype, device=dev)
+            out = _new((n_out, c_out), feats.dtype, dev)
     epi, _keep = _epilogue(feats, n_out, c_out, bias, residual, act, ld_in, ld_out)
     if dataflow == DATAFLOW_FOD:
         imap, omap = (km.omap, km.imap) if transposed else (km.imap, km.omap)
@@ -715,7 +896,7 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
         single = transposed and tuple(km.ks) == tuple(km.stride) and km.M == n_out and km.M > 0
         need = 0 if single else km.M * c_out
         if not single and (buffer is None or buffer.numel() < need or buffer.dtype != feats.dtype or buffer.device != dev):
-            buffer = torch.empty(max(need, 1), dtype=feats.dtype, device=dev)
+            buffer = _staging(max(need, 1), feats.dtype, dev)
         imap, omap = (km.omap, km.imap) if transposed else (km.imap, km.omap)
         ocsr, oslot = (km.icsr, km.islot) if transposed else (km.ocsr, km.oslot)
         # A strided layer whose kernel equals its stride gives every input one pair; on surface-like clouds nearly
@@ -734,7 +915,7 @@ def conv_forward(feats: torch.Tensor, weight: torch.Tensor, km: KernelMap, dataf
         ensure_csr(km)
         need = km.qsum * (c_in + c_out)
         if buffer is None or buffer.numel() < need or buffer.dtype != feats.dtype or buffer.device != dev:
-            buffer = torch.empty(max(need, 1), dtype=feats.dtype, device=dev)
+            buffer = _staging(max(need, 1), feats.dtype, dev)
         icsr, icode, ocsr, ocode = (km.ocsr, km.ocode, km.icsr, km.icode) if transposed else (km.icsr, km.icode, km.ocsr, km.ocode)
         _lib.check(lib.pce_conv_fwd_gms(feats.data_ptr(), weight.data_ptr(), _ptr(packed), out.data_ptr(), dt, n_in, n_out,
                                         c_in, c_out, kv, mid, icsr.data_ptr(), icode.data_ptr(), ocsr.data_ptr(), ocode.data_ptr(),

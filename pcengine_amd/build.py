@@ -18,7 +18,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libpcengine_amd.so")
 MEASURE_LIB_PATH = os.path.join(LIB_DIR, "libpcengine_amd_measure.so")
-SOURCES = ["pce_map.hip", "pce_conv.hip"]
+SOURCES = ["pce_map.hip", "pce_conv.hip", "pce_plan.hip"]
 MEASURE_SOURCES = ["pce_conv.hip"]      # the sources that read PCE_MEASURE; the others are shared as objects
 HEADERS = [os.path.join(CSRC, "pce_common.h"), os.path.join(ROOT, "include", "pcengine_amd.h"),
            os.path.join(ROOT, "include", "pcengine_amd_measure.h")]

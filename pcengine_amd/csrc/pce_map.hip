@@ -915,12 +915,21 @@ extern "C" int pce_outcoords_chain_plan(int64_t n_in, int32_t levels, const pce_
 extern "C" int pce_outcoords_chain(const int32_t *in_coords, int64_t n_in, int32_t levels, const pce_geom_t *geoms,
                                    int32_t n_batch, void *const *ws, const int64_t *ws_bytes, int32_t *const *out_coords,
                                    int64_t *n_out_host, pce_stream_t stream) {
+  return pce_outcoords_chain_planned(in_coords, n_in, n_in, levels, geoms, n_batch, ws, ws_bytes, out_coords, n_out_host, stream);
+}
+
+// n_plan: the row count the workspaces were laid out for (pce_outcoords_chain_plan); a smaller cloud runs through
+// the same layout (whether a level takes the bitmap depends on the row count: a plan must not change its mind)
+extern "C" int pce_outcoords_chain_planned(const int32_t *in_coords, int64_t n_in, int64_t n_plan, int32_t levels,
+                                           const pce_geom_t *geoms, int32_t n_batch, void *const *ws, const int64_t *ws_bytes,
+                                           int32_t *const *out_coords, int64_t *n_out_host, pce_stream_t stream) {
   hipStream_t s = (hipStream_t)stream;
   GeomDev gd[PCE_MAX_CHAIN];
   OutCoordLayout L[PCE_MAX_CHAIN];
   int64_t bound_in[PCE_MAX_CHAIN];
   if (!in_coords || !ws || !ws_bytes || !out_coords || !n_out_host) PCE_FAIL(PCE_EINVAL, "pce_outcoords_chain: null pointer");
-  int rc = chain_plan(n_in, levels, geoms, n_batch, gd, L, bound_in);
+  if (n_in <= 0 || n_in > n_plan) PCE_FAIL(PCE_EINVAL, "pce_outcoords_chain: %lld rows, planned for %lld", (long long)n_in, (long long)n_plan);
+  int rc = chain_plan(n_plan, levels, geoms, n_batch, gd, L, bound_in);
   if (rc < 0) PCE_FAIL(PCE_EINVAL, "pce_outcoords_chain: a level does not take the occupancy bitmap (ask pce_outcoords_chain_plan first)");
   if (rc) return rc;
   int host[PCE_MAX_CHAIN][4];
@@ -986,8 +995,9 @@ extern "C" int pce_outcoords_chain(const int32_t *in_coords, int64_t n_in, int32
     int *cnt = (int *)(w + L[l].off_cnt);
     int *status = (int *)(w + L[l].off_counters);
     if ((rc = fill_u32(bits, (L[l].off_counters + 256 - L[l].off_bits) / 4, 0u, s))) return rc;
-    hipLaunchKernelGGL(outcoord_mark_kernel, dim3((unsigned)pce_div_up(bound_in[l], 256)), dim3(256), 0, s, src,
-                       (long long)bound_in[l], gd[l], L[l].grid, bits, status, n_dev);
+    const long long rows_l = l == 0 ? (long long)n_in : (long long)bound_in[l];   // (level 0: the cloud itself, not its plan)
+    hipLaunchKernelGGL(outcoord_mark_kernel, dim3((unsigned)pce_div_up(rows_l, 256)), dim3(256), 0, s, src, rows_l, gd[l], L[l].grid,
+                       bits, status, n_dev);
     PCE_LAUNCH_CHECK("outcoord_mark");
     if ((rc = scan_exclusive2(cnt, L[l].words, nullptr, 0, (int *)(w + L[l].off_scan), s, bits))) return rc;
     hipLaunchKernelGGL(outcoord_expand_kernel, dim3((unsigned)pce_div_up(L[l].words, 256)), dim3(256), 0, s,

@@ -13,6 +13,7 @@ from typing import List, Sequence
 import torch
 from torch import nn
 
+from . import backend
 from .activation import ReLU
 from .batchnorm import BatchNorm
 from .spconv import conv3d, prebuild_maps
@@ -101,6 +102,19 @@ class SparseResUNet(nn.Module):
         self._in_place_ok = None
         return self
 
+    def use_planner(self, on: bool = True) -> "SparseResUNet":
+        """Build the kernel maps of every forward through the native planner (``spconv.MapPlanner``): one allocation,
+        kept and reused from cloud to cloud, and two library calls for the whole pyramid.  The maps of a cloud then
+        live until the next forward of this module; leave it off where maps must outlive that (a tensor whose
+        ``kmaps`` are reused after another cloud went through the network).  In inference the layer outputs, routing
+        arrays and the staging buffer then come from one allocation as well (``backend.ForwardArena``): from the
+        second forward over clouds of one size on, a forward allocates no device memory, and the tensor it returns is
+        valid until the next forward."""
+        from .spconv import MapPlanner
+        self._planner = MapPlanner() if on else None
+        self._arena = None         # made on the first planned forward, on the device of its input
+        return self
+
     def map_plan(self):
         """(kernel_size, stride, padding) of the layers that need a kernel map, in execution order."""
         plan = [(3, 1, 0)]
@@ -109,7 +123,19 @@ class SparseResUNet(nn.Module):
         return plan
 
     def forward(self, x: spTensor) -> spTensor:
-        prebuild_maps(x, self.map_plan())      # no host wait is left between the layers below
+        planner = getattr(self, "_planner", None)
+        if planner is not None and x.feats.is_cuda and not (torch.is_grad_enabled() and (
+                x.feats.requires_grad or any(p.requires_grad for p in self.parameters()))):
+            if getattr(self, "_arena", None) is None or self._arena.device != x.feats.device:
+                self._arena = backend.ForwardArena(x.feats.device)
+            with backend.allocate_from(self._arena):
+                return self._forward(x, planner)
+        return self._forward(x, planner)
+
+    def _forward(self, x: spTensor, planner) -> spTensor:
+        # no host wait is left between the layers below; with a planner (see use_planner) all maps of the cloud are
+        # laid out and built by the library in one allocation
+        prebuild_maps(x, self.map_plan(), planner)
         if self._skips_in_place(x):
             return self._forward_skips_in_place(x)
         x = self.stem(x)
@@ -145,7 +171,7 @@ class SparseResUNet(nn.Module):
         the left-hand ones later, and the decoder block reads the matrix; the layers that consume the kept output
         on the way down gather from its columns in place.  Same kernels, same values, no pass that copies."""
         def joined(rows, like, c_up, c_skip):
-            return torch.empty((rows, c_up + c_skip), dtype=like.dtype, device=like.device)
+            return backend._new((rows, c_up + c_skip), like.dtype, like.device)
         ups = [u.conv.out_channels for u in self.up][::-1]      # c_up of the stage that ends at level 0, 1, ...
         x = self.stem[0](x)
         buf = joined(x.feats.shape[0], x.feats, ups[0], self.stem[1].conv.out_channels)

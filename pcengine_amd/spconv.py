@@ -147,7 +147,12 @@ def _pick_dataflow(km: backend.KernelMap, requested: str, c_in: int, c_out: int,
         return DATAFLOW_GMS
     if km.tag == "D2":
         return DATAFLOW_FOD
-    return backend.select_dataflow(km, c_in, c_out, dtype, transposed)
+    picks = km.__dict__.setdefault("_picks", {})      # the selector's answer per layer shape on this map
+    key = (c_in, c_out, dtype, transposed)
+    df = picks.get(key)
+    if df is None:
+        df = picks[key] = backend.select_dataflow(km, c_in, c_out, dtype, transposed)
+    return df
 
 
 class _ConvFunction(torch.autograd.Function):
@@ -236,7 +241,11 @@ def _run(input: spTensor, km: backend.KernelMap, kernel, in_channel, out_channel
     if kernel.dtype != feats.dtype:
         kernel, packed = kernel.to(feats.dtype), None
     if kernel.dim() == 3 and feats.shape[1] < kernel.shape[1]:
-        feats = torch.nn.functional.pad(feats, (0, kernel.shape[1] - feats.shape[1]))    # see conv3d._weights_for
+        # see conv3d._weights_for (the padded copy comes from the forward's arena where one is active)
+        padded = backend._new((feats.shape[0], kernel.shape[1]), feats.dtype, feats.device)
+        padded[:, feats.shape[1]:].zero_()
+        padded[:, :feats.shape[1]].copy_(feats)
+        feats = padded
     # the selector sees the width the kernels run at (a 3- or 4-channel input layer runs padded to 16)
     df = _pick_dataflow(km, dataflow, feats.shape[1], out_channel, feats.dtype, transposed)
     out = backend.conv_forward(feats, kernel.detach(), km, df, transposed=transposed, buffer=input.buffer, packed=packed,
@@ -285,6 +294,13 @@ def ensure_map(input: spTensor, kernel_size_code: int, stride_code: int, padding
     and stored there (script/spconv.py:331-437).  Returns (map, output tensor stride, output
     coords_min, output coords_max).  Maps depend on coordinates only, so a network can ask for all of
     them before the first convolution (``prebuild_maps``)."""
+    km = input.kmaps.get((kernel_size_code, input.stride, stride_code))
+    if km is not None and not isinstance(km, backend._MapJob):
+        # the usual case inside a network (its maps were built ahead): nothing to decode but the output bound
+        input.cbook.setdefault(input.stride, input.coords)
+        if stride_code == _UNIT:
+            return km, input.stride, input.coords_min, input.coords_max
+        return km, output_stride_compute(stride_code, input.stride, 0), input.coords_min, list(km._cmax)
     km, request, key, tag, output_stride, coords_min, coords_max = _map_request(input, kernel_size_code, stride_code, padding_code)
     if request is not None:
         km = backend.build_kernel_map(**request)
@@ -318,12 +334,92 @@ def _chain_out_coords(input: spTensor, layers) -> dict:
     return dict(zip(idx, outs)) if outs is not None else {}
 
 
-def _prebuild(input: spTensor, layers):
+class MapPlanner:
+    """Keeps the native plans (``backend.PyramidPlan``: one allocation for all maps of a network on one cloud) a network
+    has used, one per (layer list, coordinate box, batch count); a plan is reused for every cloud of at most its
+    capacity in rows and replaced by a larger one when a cloud exceeds it.  The maps of a cloud live in the plan's
+    allocation until the next cloud is built with it: a caller that keeps maps across forwards (a prefetcher, two
+    clouds in flight) uses one planner per cloud in flight, or none."""
+
+    def __init__(self, headroom: float = 1.125):
+        self.plans = {}
+        self.headroom = headroom
+
+    def plan_for(self, key, n: int, make):
+        plan = self.plans.get(key)
+        if plan is None or plan.n_cap < n:
+            cap = -(-int(n * self.headroom) // 4096) * 4096
+            plan = self.plans[key] = make(cap)
+        return plan
+
+
+def _prebuild_planned(input: spTensor, layers, planner: MapPlanner):
+    """The maps `layers` asks for through the native planner, or None where it does not apply (a map already cached,
+    reference tags, no batch count, a strided layer whose kernel differs from its stride or that is padded, a cloud
+    that is not sorted): the caller then builds them map by map.  Same maps, same cache entries."""
+    if not input.coords.is_cuda or not input.batchsize or input.batchsize <= 0:
+        return None
+    if input.init_tag and input.init_tag[0] not in ('end', 'auto'):      # the reference's D1 / D2 tags: map by map
+        return None
+    entries, strided, requests = [], [], []
+    stride_code, cmin, cmax, level = input.stride, list(input.coords_min[:3]), list(input.coords_max[:3]), 0
+    seen = {}
+    for ks, st, pad in layers:
+        ksc, sc, pc = (conv_info_encoder(_triple(v, "layer")) for v in (ks, st, pad))
+        if ksc == _UNIT and sc == _UNIT:
+            continue
+        key = (ksc, stride_code, sc)
+        if key in input.kmaps:
+            return None
+        k3, s3, p3 = conv_info_decoder(ksc), conv_info_decoder(sc), conv_info_decoder(pc)
+        subm = sc == _UNIT
+        if subm:
+            if key not in seen:
+                seen[key] = len(requests)
+                requests.append((level, level, k3, s3, p3, cmin, cmax, True, True, False, False))
+                entries.append((key, stride_code, level, level))
+            continue
+        if k3 != s3 or any(p3) or key in seen:
+            return None
+        cmax = backend.strided_coords_max(cmax, k3, s3, p3)
+        out_stride = output_stride_compute(sc, stride_code, 0)
+        strided.append(backend.Geom.make(k3, s3, p3, cmin, cmax, False))
+        seen[key] = len(requests)
+        requests.append((level, level + 1, k3, s3, p3, cmin, cmax, False, True, True, False))
+        entries.append((key, out_stride, level, level + 1))
+        stride_code, level = out_stride, level + 1
+    if not requests:
+        return None
+    coords = input.coords if input.coords.is_contiguous() else input.coords.contiguous()
+    n = coords.shape[0]
+    pkey = (tuple(map(tuple, ((r[0], r[1]) + tuple(r[2]) + tuple(r[6]) for r in requests))), tuple(input.coords_min[:3]),
+            int(input.batchsize), coords.device)
+    try:
+        plan = planner.plan_for(pkey, n, lambda cap: backend.PyramidPlan(cap, strided, requests, input.batchsize, coords.device))
+        level_coords, maps = plan.build(coords)
+    except backend.PlanNotApplicable:
+        return None
+    level_stride = {0: input.stride}
+    for (key, out_stride, lin, lout), km in zip(entries, maps):
+        km.tag = 'auto'
+        input.kmaps[key] = km
+        level_stride[lout] = out_stride
+    input.cbook.setdefault(input.stride, input.coords)
+    for lv in range(1, len(level_coords)):
+        input.cbook[level_stride[lv]] = level_coords[lv]
+    return maps
+
+
+def _prebuild(input: spTensor, layers, planner: Optional[MapPlanner] = None):
     """Builds the maps `layers` asks for, starting at `input`.  Returns (the tensor at the coordinates the last
     entry leaves, the maps that were built now)."""
+    layers = list(layers)
+    if planner is not None:
+        built = _prebuild_planned(input, layers, planner)
+        if built is not None:
+            return input, built
     x = input
     pending, done = [], []
-    layers = list(layers)
     chained = _chain_out_coords(input, layers)
     try:
         for i, (ks, stride, pad) in enumerate(layers):
@@ -357,15 +453,16 @@ def _prebuild(input: spTensor, layers):
     return x, done
 
 
-def prebuild_maps(input: spTensor, layers) -> None:
+def prebuild_maps(input: spTensor, layers, planner: Optional[MapPlanner] = None) -> None:
     """Build, ahead of any convolution, the maps a network will ask for.  ``layers`` lists
     (kernel_size, stride, padding) in network order (ints or triples; transposed layers and 1x1
     layers need no entry); a strided entry moves on to its output coordinates, as the network does.
     The output coordinates of the strided layers are computed first, level by level (their number has
     to reach the host); then all maps are built together, every stage of the build as one launch over
     all layers, and their pair counts are read back in one copy.  The layers that follow find every
-    map in the cache."""
-    _prebuild(input, layers)
+    map in the cache.  With a ``planner`` the whole pyramid is laid out and built by the library in one allocation
+    (``MapPlanner``); where that does not apply the maps are built as described."""
+    _prebuild(input, layers, planner)
 
 
 class MapPrefetcher:
