@@ -77,15 +77,22 @@ __host__ __device__ static inline unsigned long long pce_home_slot(unsigned long
 
 // ---------------------------------------------------------------------------------------------
 // Row order of the ordered output-stationary dataflow (pce_row_order, pce_conv_fwd_oso):
-// order = perm[n_rows] | mask[n_rows] | tail[PCE_ORDER_TAIL] | rec[n_rows] (int4, 16-byte aligned).  The tail holds
-// the histogram, the cursors and the bases of the counting sort over ORDER_KEYS keys -- the offset of the rows with
-// one neighbour, then (lowest, second-lowest) offset of the rows with two, then of the rows with more -- and the counts.  rec[p], for the
-// positions p of rows that have a neighbour, repeats what a wavefront needs of the row at perm[p] in one 16-byte
-// load: {row, mask, neighbour at the lowest offset of the mask, neighbour at the second-lowest or -1}.
+// order = perm[n_rows] | mask[n_rows] | tail[PCE_ORDER_TAIL] | rec[n_rows] (int4, 16-byte aligned) | srec[PCE_ORDER_SREC_ROWS][32].
+// The tail holds the histogram, the cursors and the bases of the counting sort over ORDER_KEYS keys -- the offset of
+// the rows with one neighbour, then (lowest, second-lowest) offset of the rows with two, then of the rows with more
+// -- and the counts.  rec[p], for the positions p of rows that have a neighbour, repeats what a wavefront needs of the
+// row at perm[p] in one 16-byte load: {row, mask, neighbour at the lowest offset of the mask, neighbour at the
+// second-lowest or -1}.  srec[i], for the i-th row with two neighbours or more in the order (position n_plain +
+// n_single + i), holds {row, mask, neighbour at offset 0, 1, ... 29 (-1 where the mask has no bit)}; it is written
+// only where those rows number at most PCE_ORDER_SREC_ROWS (an eighth of the rows: the clouds the kernel that
+// reads it is meant for).
 // ---------------------------------------------------------------------------------------------
 #define PCE_ORDER_TAIL 8192
 #define PCE_ORDER_REC_OFFSET(n_rows) ((2 * (long long)(n_rows) + PCE_ORDER_TAIL + 3) & ~3ll)
-#define PCE_ORDER_ELEMS(n_rows) (PCE_ORDER_REC_OFFSET(n_rows) + 4 * (long long)(n_rows))
+#define PCE_ORDER_SREC_OFFSET(n_rows) (PCE_ORDER_REC_OFFSET(n_rows) + 4 * (long long)(n_rows))
+#define PCE_ORDER_SREC_ROWS(n_rows) ((long long)(n_rows) / 8 + 32)
+#define PCE_ORDER_SREC_KV 30
+#define PCE_ORDER_ELEMS(n_rows) (PCE_ORDER_SREC_OFFSET(n_rows) + 32 * PCE_ORDER_SREC_ROWS(n_rows))
 #define ORDER_MAX_KV 32
 #define ORDER_KEYS 2048
 #define ORDER_HIST 0

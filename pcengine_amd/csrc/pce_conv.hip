@@ -2570,6 +2570,128 @@ __global__ void __launch_bounds__(256, 4) wave_os_kernel(TileArgs a, const int *
   store_rows_via_lds<half_t, NB>(V, Pl[wave], (half_t *)a.out, orow, a, 0, lane, l32, g, a.stream);
 }
 
+// A chunk of 32 rows with two neighbours or more, NBW column blocks of it from column n0 on, by one workgroup.
+// The four wavefronts split the INPUT CHANNELS, 16 each (one K step of the MFMA), and all walk the offsets of the
+// chunk's union: a step then holds 16 bytes of a neighbour row and 16 bytes of weights per column block in a lane
+// -- 12 registers at 64 columns, 8 at 32 -- so six or ten offsets are in flight per wavefront, where a wavefront that
+// owns whole offsets (wave_os_kernel: k mod 4) has registers for one and spends one trip to memory per offset, seven
+// in a row on a dense cluster.  The four partial sums of a row meet through LDS in wavefront 0, which stores the row.
+// The rows of the chunk come as 128-byte records {row, mask, neighbour at offset 0, 1, ...} (the row order writes
+// them for the rows with two neighbours or more): thread t fetches 16 bytes of the record of row t / 8 and files
+// them by [slot][row] in LDS (33 words per slot: the eight threads of a row hit eight banks).  One trip to memory
+// stands between the start of the workgroup and its first row gather; the centre product is one more offset of
+// the walk (its neighbour is the row itself), so the workgroup copies neither centre rows nor centre weights.
+// sb, s_end: the chunk's first record and the end of its section of the records.
+template <int NBW, int KS, int REGION>
+__device__ __forceinline__ void os2_shared_chunk(const TileArgs &a, const int *__restrict__ order, int mid, long long sb,
+                                                 long long s_end, int n0, half8 (&Pl)[4][REGION]) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int l32 = lane & 31, g = lane >> 5;
+  const half_t *Wp = (const half_t *)a.Wp;
+  const half_t *A = (const half_t *)a.A;
+  const long long wstep = (long long)a.k8_total * a.n_pad * 8;
+  const long long n = a.n_rows;
+  const half8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  constexpr int IDX_LD = 33;
+  int *idxL = reinterpret_cast<int *>(&Pl[0][0]);
+  static_assert(32 * IDX_LD * 4 <= 2 * REGION * 16, "the index table fits two regions");
+  {
+    const int r = threadIdx.x >> 3, q = threadIdx.x & 7;
+    const bool have = sb + r < s_end;
+    typedef int v4i_t __attribute__((ext_vector_type(4)));
+    const v4i_t v = *reinterpret_cast<const __attribute__((address_space(1))) v4i_t *>(
+        (const __attribute__((address_space(1))) int *)(order + PCE_ORDER_SREC_OFFSET(n)) + ((have ? sb + r : sb) * 32 + q * 4));
+#pragma unroll
+    for (int j = 0; j < 4; ++j) idxL[(4 * q + j) * IDX_LD + r] = have ? v[j] : (4 * q + j == 1 ? 0 : -1);
+  }
+  __syncthreads();
+  const int orow = idxL[l32];
+  const unsigned m = (unsigned)idxL[IDX_LD + l32];
+  unsigned uu = m;
+#pragma unroll
+  for (int d = 1; d < 32; d <<= 1) uu |= (unsigned)__shfl_xor((int)uu, d, PCE_WAVE);
+  const unsigned u = (unsigned)__builtin_amdgcn_readfirstlane((int)uu) | (1u << mid);   // the chunk's offsets and the centre
+  f32x16 acc[NBW];
+#pragma unroll
+  for (int nb = 0; nb < NBW; ++nb)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[nb][j] = 0.f;
+  if (wave < KS) {
+    const int s = wave;   // this wavefront's K step: input channels [16 s, 16 s + 16)
+    // slot j holds the row fragment, the row's index and the weight fragments of one offset
+    constexpr int SLOTS = NBW == 2 ? 6 : 10;
+    half8 rf[SLOTS], wf[SLOTS][NBW];
+    int ri[SLOTS];
+    unsigned rem_issue = u;
+    const half_t *Ab = A + s * 16 + g * 8;
+    const half_t *Wb = Wp + ((long long)(2 * s + g) * a.n_pad + n0 + l32) * 8;
+    // (every step issues its loads and its MFMAs unconditionally -- a slot beyond the last offset loads from a
+    // valid address and multiplies zeros -- so that the waits in front of the MFMAs are counted exactly and leave the
+    // loads of the other slots in flight; with the loads under a condition every wait became a full one)
+#define PCE_OS2_ISSUE(J_)                                                                                          \
+  {                                                                                                                \
+    const int k_ = rem_issue ? __ffs((int)rem_issue) - 1 : 0;                                                      \
+    const int v_ = idxL[(2 + k_) * IDX_LD + l32];                                                                  \
+    ri[J_] = rem_issue ? (k_ == mid ? orow : v_) : -1;                                                             \
+    rem_issue &= rem_issue - 1u;                                                                                   \
+    rf[J_] = *reinterpret_cast<const half8 *>(Ab + (long long)(ri[J_] >= 0 ? ri[J_] : 0) * a.lda);                 \
+    _Pragma("unroll") for (int nb = 0; nb < NBW; ++nb)                                                             \
+      wf[J_][nb] = *reinterpret_cast<const half8 *>(Wb + k_ * wstep + nb * 32 * 8);                                \
+  }
+#define PCE_OS2_USE(J_)                                                                                            \
+  {                                                                                                                \
+    const half8 f_ = ri[J_] >= 0 ? rf[J_] : zero;                                                                  \
+    _Pragma("unroll") for (int nb = 0; nb < NBW; ++nb)                                                             \
+      acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[J_][nb], f_, acc[nb], 0, 0, 0);                          \
+  }
+#pragma unroll
+    for (int j = 0; j < SLOTS; ++j) PCE_OS2_ISSUE(j)
+    for (int round = (__popc(u) + SLOTS - 1) / SLOTS; round > 0; --round) {   // wavefront-uniform
+#pragma unroll
+      for (int j = 0; j < SLOTS; ++j) {
+        __builtin_amdgcn_sched_barrier(0);
+        PCE_OS2_USE(j)
+        PCE_OS2_ISSUE(j)
+      }
+    }
+#undef PCE_OS2_ISSUE
+#undef PCE_OS2_USE
+  }
+  // wavefronts 1..3 hand their accumulators to wavefront 0, one 32-column block at a time through their own regions
+  // (wavefront 1's region holds the end of the index table: the first barrier below stands behind its last reader);
+  // a lane's 16 values go as four 16-byte pieces, piece j of all lanes side by side: no bank conflicts
+  typedef float f32x4_t __attribute__((ext_vector_type(4)));
+  f32x4_t *mine = reinterpret_cast<f32x4_t *>(&Pl[wave][0]);
+#pragma unroll
+  for (int nb = 0; nb < NBW; ++nb) {
+    __syncthreads();
+    if (wave > 0 && wave < KS) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) mine[j * 64 + lane] = f32x4_t{acc[nb][4 * j], acc[nb][4 * j + 1], acc[nb][4 * j + 2], acc[nb][4 * j + 3]};
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+      for (int w2 = 1; w2 < 4; ++w2) {
+        if (w2 < KS) {
+          const f32x4_t *theirs = reinterpret_cast<const f32x4_t *>(&Pl[w2][0]);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const f32x4_t o = theirs[j * 64 + lane];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[nb][4 * j + i] += o[i];
+          }
+        }
+      }
+    }
+  }
+  if (wave > 0) return;
+  float V[NBW][2][8];
+  gather_row_pieces<NBW>(acc, V, g);
+  if (a.bias || a.res || a.act) epilogue_row_pieces<half_t, NBW, true>(V, a, orow, n0, g, a.act != PCE_ACT_NONE);
+  store_rows_via_lds<half_t, NBW>(V, Pl[0], (half_t *)a.out, orow, a, n0, lane, l32, g, a.stream);
+}
+
 // The same layer for clouds where most rows have no neighbour at all (at least half of them), in three kinds of
 // workgroup, so that every wavefront of the launch is resident from the start and none waits for more trips to
 // memory than its rows need (per-wavefront timestamps of wave_os_kernel on the 150 k-voxel scan: two rounds of
@@ -2582,16 +2704,16 @@ __global__ void __launch_bounds__(256, 4) wave_os_kernel(TileArgs a, const int *
 //   single  32 rows with exactly one neighbour, from the row order's records {row, mask, neighbour, -}: one trip for
 //           the records, one for the centre rows, the neighbour's fragments and the weights of the chunk's first
 //           offset (the order sorts these rows by their offset: a chunk has one offset, two at a boundary);
-//   shared  32 rows with two neighbours or more per workgroup (two workgroups per chunk for 33-64 output channels,
-//           32 columns each), the offsets split over the four wavefronts by k mod 4 as in wave_os_kernel; a
-//           wavefront requests the neighbour indices of all its offsets (at most seven) in one trip and keeps row
-//           fragments and weights of two offsets in flight (16 + 16 registers per offset at 32 columns).
-// Rows with three neighbours or more form their sums as in wave_os_kernel (per wavefront over its offsets in
-// ascending order, then wavefront 0 adds the others' in turn) and come out bit-identical to it; rows with two are
-// summed the same way here and in one wavefront there, so their last bits may differ between the two kernels.
+//   shared  32 rows with two neighbours or more per workgroup, from the row order's 128-byte records {row, mask,
+//           neighbour at every offset}: one trip for the records, then the four wavefronts, which split the input
+//           channels, walk the offsets of the chunk (the centre among them) with six in flight each.
+// A row's sum is formed per wavefront over its offsets in ascending order, then wavefront 0 adds the others' in
+// turn: the same for every run and every position of the row in the order, but not the order of additions of
+// wave_os_kernel, so rows with two neighbours or more may differ from that kernel's in their last bits.
 template <int NB, int KS>
 __global__ void __launch_bounds__(256, 4) wave_os2_kernel(TileArgs a, const int *__restrict__ order, int mid, long long n_plain,
-                                                          long long n_single, int shared_wgs, int single_wgs) {
+                                                          long long n_single, long long n_two, int heavy_wgs,
+                                                          int shared_wgs, int single_wgs) {
   constexpr int PPR = KS * 2;   // 16-byte pieces per input row
   constexpr int REGION0 = WaveLds<NB>::PIECES > 64 * PPR ? WaveLds<NB>::PIECES : 64 * PPR;
   constexpr int REGION = REGION0 > 256 ? REGION0 : 256;   // also one accumulator block of 64 lanes
@@ -2604,7 +2726,7 @@ __global__ void __launch_bounds__(256, 4) wave_os2_kernel(TileArgs a, const int 
   const half_t *A = (const half_t *)a.A;
   const long long wstep = (long long)a.k8_total * a.n_pad * 8;
   const long long n = a.n_rows;
-  {
+  if ((int)blockIdx.x >= shared_wgs) {   // (the shared workgroups read the centre weights as they read the others')
     constexpr int FR = KS * 2 * NB * 32;   // fragments: [k8][column]
 #pragma unroll
     for (int i = 0; i < (FR + 255) / 256; ++i) {
@@ -2755,148 +2877,51 @@ __global__ void __launch_bounds__(256, 4) wave_os2_kernel(TileArgs a, const int 
   }
 #undef PCE_OS2_FRAGS
   // ---- shared: 32 rows with two neighbours or more per workgroup ------------------------------------------------
-  // The four wavefronts split the INPUT CHANNELS, 16 each (one K step of the MFMA), and all walk the offsets of
-  // the chunk's union: a step then holds 16 bytes of a neighbour row and 16 bytes of weights per column block in a
-  // lane -- 12 registers at 64 columns -- so four offsets are in flight per wavefront, where a wavefront that owns
-  // whole offsets (wave_os_kernel: k mod 4) has registers for one and spends one trip to memory per offset, seven in
-  // a row on a dense cluster.  The neighbour indices of the chunk, [offset][row], are fetched once per workgroup
-  // (wavefront w those of the offsets k = w mod 4) into LDS.  Each wavefront adds its share of the centre product;
-  // the four partial sums of a row meet through LDS in wavefront 0, which stores the row.
-  const long long p0 = n_plain + n_single + (long long)blockIdx.x * 32;
-  const bool valid = p0 + l32 < n;
-  const int4 rc = rec[valid ? p0 + l32 : p0];
-  const int orow = valid ? rc.x : -1;
-  const unsigned m = valid ? (unsigned)rc.y : 0u;
-  unsigned uu = m;
-#pragma unroll
-  for (int d = 1; d < 32; d <<= 1) uu |= (unsigned)__shfl_xor((int)uu, d, PCE_WAVE);
-  const unsigned u = (unsigned)__builtin_amdgcn_readfirstlane((int)uu);   // offsets any of the 32 rows has
-  // the table of neighbour indices lives behind the centre rows in wavefront 0's region and runs into wavefront 1's
-  // (wavefront 0 stages the finished rows over it once every wavefront is done with it)
-  int *idxL = reinterpret_cast<int *>(&Pl[0][32 * PPR]);
-  static_assert((32 * PPR) * 16 + 27 * 32 * 4 <= 2 * REGION * 16, "centre rows and index table fit two regions");
-  if (wave == 0) {
-#pragma unroll
-    for (int it = 0; it < KS; ++it) {
-      const int e = it * 64 + lane, r = e / PPR, sl = e % PPR;
-      const int row = __shfl(rc.x, r, PCE_WAVE);
-      const half_t *gp = A + (long long)row * a.lda + ((sl ^ row_swizzle<PPR>(r)) * 8);
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
-                                       (__attribute__((address_space(3))) void *)&Pl[0][it * 64], 16, 0, 0);
-    }
+  // first the chunks of rows with three neighbours or more, the longest walks of the launch: at 33-64 output
+  // channels two workgroups each, one per block of 32 columns (ten offsets in flight instead of six); then the
+  // chunks of rows with two
+  const long long n_shared = n - n_plain - n_single;
+  if ((int)blockIdx.x < heavy_wgs) {
+    if (NB == 2)
+      os2_shared_chunk<1, KS, REGION>(a, order, mid, n_two + (long long)(blockIdx.x >> 1) * 32, n_shared, (blockIdx.x & 1) * 32, Pl);
+    else
+      os2_shared_chunk<NB, KS, REGION>(a, order, mid, n_two + (long long)blockIdx.x * 32, n_shared, 0, Pl);
+  } else {
+    os2_shared_chunk<NB, KS, REGION>(a, order, mid, ((long long)blockIdx.x - heavy_wgs) * 32, n_two, 0, Pl);
   }
-  {
-    // this wavefront's share of the index table: up to seven offsets, all requested before any is written
-    unsigned rem = u & (0x11111111u << wave);
-    rem = (unsigned)__builtin_amdgcn_readfirstlane((int)rem);
-    int kk[7], vv[7];
-#pragma unroll
-    for (int t = 0; t < 7; ++t) {
-      kk[t] = rem ? __ffs((int)rem) - 1 : -1;
-      rem &= rem - 1u;
-    }
-#pragma unroll
-    for (int t = 0; t < 7; ++t) {
-      const bool has = kk[t] >= 0 && ((m >> (kk[t] >= 0 ? kk[t] : 0)) & 1u);
-      const int v = a.nbr[has ? (long long)kk[t] * n + orow : 0];
-      vv[t] = has ? v : -1;
-    }
-#pragma unroll
-    for (int t = 0; t < 7; ++t)
-      if (kk[t] >= 0 && g == 0) idxL[kk[t] * 32 + l32] = vv[t];
+}
+
+// compute units of the current device (asked once per device)
+static int cu_count() {
+  static int cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  if (!cached[dev]) {
+    int v = 0;
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    cached[dev] = v;
   }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();   // centre weights, centre rows and the index table are in LDS
-  f32x16 acc[NB];
-#pragma unroll
-  for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-    for (int j = 0; j < 16; ++j) acc[nb][j] = 0.f;
-  if (wave < KS) {
-    const int s = wave;   // this wavefront's K step: input channels [16 s, 16 s + 16)
-    {
-      const half8 af = Pl[0][l32 * PPR + ((2 * s + g) ^ row_swizzle<PPR>(l32))];
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-        acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(Wc[(2 * s + g) * (NB * 32) + nb * 32 + l32], af, acc[nb], 0, 0, 0);
-    }
-    // six offsets in flight (eight at 32 columns): slot j holds the row fragment, the row's index and the weight fragments of one offset
-    constexpr int SLOTS = NB == 2 ? 6 : 8;
-    half8 rf[SLOTS], wf[SLOTS][NB];
-    int ri[SLOTS];
-    unsigned rem_issue = u;
-    const half_t *Ab = A + s * 16 + g * 8;
-    const half_t *Wb = Wp + ((long long)(2 * s + g) * a.n_pad + l32) * 8;
-    // (every step issues its loads and its MFMAs unconditionally -- a slot beyond the last offset loads from a
-    // valid address and multiplies zeros -- so that the waits in front of the MFMAs are counted exactly and leave the
-    // loads of the three other slots in flight; with the loads under a condition every wait became a full one)
-#define PCE_OS2_ISSUE(J_)                                                                                          \
-  {                                                                                                                \
-    const int k_ = rem_issue ? __ffs((int)rem_issue) - 1 : 0;                                                      \
-    const int v_ = idxL[k_ * 32 + l32];                                                                            \
-    ri[J_] = rem_issue ? v_ : -1;                                                                                  \
-    rem_issue &= rem_issue - 1u;                                                                                   \
-    rf[J_] = *reinterpret_cast<const half8 *>(Ab + (long long)(ri[J_] >= 0 ? ri[J_] : 0) * a.lda);                 \
-    _Pragma("unroll") for (int nb = 0; nb < NB; ++nb)                                                              \
-      wf[J_][nb] = *reinterpret_cast<const half8 *>(Wb + k_ * wstep + nb * 32 * 8);                                \
-  }
-#define PCE_OS2_USE(J_)                                                                                            \
-  {                                                                                                                \
-    const half8 f_ = ri[J_] >= 0 ? rf[J_] : zero;                                                                  \
-    _Pragma("unroll") for (int nb = 0; nb < NB; ++nb)                                                              \
-      acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[J_][nb], f_, acc[nb], 0, 0, 0);                          \
-  }
-#pragma unroll
-    for (int j = 0; j < SLOTS; ++j) PCE_OS2_ISSUE(j)
-    for (int round = (__popc(u) + SLOTS - 1) / SLOTS; round > 0; --round) {   // wavefront-uniform
-#pragma unroll
-      for (int j = 0; j < SLOTS; ++j) {
-        __builtin_amdgcn_sched_barrier(0);
-        PCE_OS2_USE(j)
-        PCE_OS2_ISSUE(j)
-      }
-    }
-#undef PCE_OS2_ISSUE
-#undef PCE_OS2_USE
-  }
-  // wavefronts 1..3 hand their accumulators to wavefront 0, one 32-column block at a time through their own regions
-  // (wavefront 1's region holds the end of the index table: the first barrier below stands behind its last reader)
-  f32x16 *mine = reinterpret_cast<f32x16 *>(&Pl[wave][0]);
-#pragma unroll
-  for (int nb = 0; nb < NB; ++nb) {
-    __syncthreads();
-    if (wave > 0 && wave < KS) mine[lane] = acc[nb];
-    __syncthreads();
-    if (wave == 0) {
-#pragma unroll
-      for (int w2 = 1; w2 < 4; ++w2) {
-        if (w2 < KS) {
-          const f32x16 other = reinterpret_cast<const f32x16 *>(&Pl[w2][0])[lane];
-#pragma unroll
-          for (int j = 0; j < 16; ++j) acc[nb][j] += other[j];
-        }
-      }
-    }
-  }
-  if (wave > 0) return;
-  float V[NB][2][8];
-  gather_row_pieces<NB>(acc, V, g);
-  if (a.bias || a.res || a.act) epilogue_row_pieces<half_t, NB, true>(V, a, orow, 0, g, a.act != PCE_ACT_NONE);
-  store_rows_via_lds<half_t, NB>(V, Pl[0], (half_t *)a.out, orow, a, 0, lane, l32, g, a.stream);
+  return cached[dev];
+}
+
+// workgroups of the three-kind kernel over a row order
+static long long os2_workgroups(long long n_out, long long n_nonzero, long long n_single, long long n_heavy, int nb) {
+  return pce_div_up(n_heavy, 32) * (nb == 2 ? 2 : 1) + pce_div_up(n_nonzero - n_single - n_heavy, 32) +
+         pce_div_up(pce_div_up(n_single, 32), 4) + pce_div_up(pce_div_up(n_out, 64), 4);
 }
 
 // the three-kind kernel over a row order, or (order == nullptr) its stream workgroups alone: a plain GEMM
 static int launch_wave_os2(const TileArgs &a, const int *order, int mid, long long n_out, long long n_nonzero, long long n_single,
-                           int nb, int ks, hipStream_t s) {
-  const long long n_plain = n_out - n_nonzero, n_shared = n_nonzero - n_single;
-  const long long shared_wgs = pce_div_up(n_shared, 32), single_wgs = pce_div_up(pce_div_up(n_single, 32), 4),
-                  stream_wgs = pce_div_up(pce_div_up(n_out, 64), 4);
+                           long long n_heavy, int nb, int ks, hipStream_t s) {
+  const long long n_plain = n_out - n_nonzero, n_two = n_nonzero - n_single - n_heavy;
+  const long long heavy_wgs = pce_div_up(n_heavy, 32) * (nb == 2 ? 2 : 1), shared_wgs = heavy_wgs + pce_div_up(n_two, 32),
+                  single_wgs = pce_div_up(pce_div_up(n_single, 32), 4), stream_wgs = pce_div_up(pce_div_up(n_out, 64), 4);
   if (shared_wgs + single_wgs + stream_wgs >= (1ll << 31) - 8) PCE_FAIL(PCE_ECAPACITY, "%lld rows exceed the grid limit", (long long)n_out);
   const unsigned grid2 = (unsigned)(shared_wgs + single_wgs + stream_wgs);
 #define PCE_WOS2_CASE(NB_, KS_)                                                                                    \
   if (nb == NB_ && ks == KS_) {                                                                                    \
     hipLaunchKernelGGL((wave_os2_kernel<NB_, KS_>), dim3(grid2), dim3(256), 0, s, a, order, mid, n_plain, n_single, \
-                       (int)shared_wgs, (int)single_wgs);                                                          \
+                       n_two, (int)heavy_wgs, (int)shared_wgs, (int)single_wgs);                                   \
     PCE_LAUNCH_CHECK("wave_os2");                                                                                  \
     return PCE_OK;                                                                                                 \
   }
@@ -3236,14 +3261,19 @@ extern "C" int pce_conv_fwd_oso(const void *in, const void *w, const void *wp, v
 #undef PCE_WOSW_CASE
     PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: unsupported shape c_in=%d c_out=%d", (int)c_in, (int)c_out);
   }
-  // Clouds whose rows mostly have no neighbour, and few of them two or more: the three-kind kernel, the bulk streamed
-  // in storage order.  Needs the counts of rows with any neighbour and with exactly one; a caller that does not state
-  // them (-1), a layer without a centre offset and other clouds take the kernel that visits every row through the
-  // order.  Measured on prefixes of the 150 k-voxel scan, this kernel / that one: 7.9 / 10.0 us on 60 k rows (0.7 % of
-  // them with two neighbours or more), 10.0 / 10.2 on 90 k (3.5 %), 12.4 / 11.9 on all (4.1 %): the workgroups of
-  // shared rows are its longest chains, so it takes clouds with at most 1/32 of such rows.
-  if (mid >= 0 && n_nonzero >= 0 && n_single >= 0 && 2 * n_nonzero <= n_out && 32 * (n_nonzero - n_single) <= n_out && stage_on(12))
-    return launch_wave_os2(a, order, (int)mid, n_out, n_nonzero, n_single, nb, ks, s);
+  // Clouds whose rows mostly have no neighbour, few of them two or more, and small enough that every workgroup of the
+  // three-kind kernel is resident at once (four per CU): that kernel, the bulk streamed in storage order.  It shortens
+  // the chains of dependent trips to memory that set the duration of a launch of one round of wavefronts; it
+  // multiplies the rows with neighbours twice, which costs more than that saves once the rows come in several rounds.
+  // Needs the counts of rows with any neighbour and with exactly one; a caller that does not state them (-1), a
+  // layer without a centre offset, 16 input channels (one wavefront of four would walk the shared rows) and other
+  // clouds take the kernel that visits every row through the order.  This kernel / that one, 64 -> 64 channels:
+  // 7.3 / 12.3 us on 60 k rows of a LiDAR scan, 9.1 / 10.5 on 90 k, 11.4 / 11.9 on all 150 k (4 % of the rows with
+  // two neighbours or more), 8.7 / 12.2 on a 100 k scan; 34.4 / 32.2 on four scans in a batch; 16 -> 32: 7.0 / 6.7.
+  if (mid >= 0 && kv <= PCE_ORDER_SREC_KV && ks >= 2 && n_nonzero >= 0 && n_single >= 0 && 2 * n_nonzero <= n_out &&
+      n_nonzero - n_single <= PCE_ORDER_SREC_ROWS(n_out) && 8 * (n_nonzero - n_single) <= n_out &&
+      os2_workgroups(n_out, n_nonzero, n_single, n_heavy, nb) <= 4ll * cu_count() && stage_on(12))
+    return launch_wave_os2(a, order, (int)mid, n_out, n_nonzero, n_single, n_heavy, nb, ks, s);
 #define PCE_WOS_CASE(NB_, KS_)                                                                              \
   if (nb == NB_ && ks == KS_) {                                                                              \
     hipLaunchKernelGGL((wave_os_kernel<NB_, KS_>), dim3(grid), dim3(256), 0, s, a, perm, rmask, (int)mid, n_main,   \
@@ -3269,7 +3299,7 @@ static int dense_impl(const void *in, const void *w, const void *wp, void *out, 
   // narrow fp16 layers: the stream workgroups of the three-kind ordered kernel alone (64 consecutive rows per
   // wavefront, weights once per workgroup through LDS): 7.1 us on 150 k rows of 64 -> 64 channels, the tile kernel 8.3
   if (sizeof(T) == 2 && wave_os_ok(a, 1, 0) && stage_on(12))
-    return launch_wave_os2(a, nullptr, 0, n, 0, 0, (c_out + 31) / 32, c_in / 16, s);
+    return launch_wave_os2(a, nullptr, 0, n, 0, 0, 0, (c_out + 31) / 32, c_in / 16, s);
   return launch_tile<T>(a, pce_div_up(n, 128), s);
 }
 

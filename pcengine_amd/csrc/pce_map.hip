@@ -1755,6 +1755,23 @@ __device__ __forceinline__ void order_scatter_block(long long n_rows, int *__res
     r.z = nbr[(long long)(mirror >= 0 ? mirror - k1 : k1) * n_rows + row];
     r.w = k2 >= 0 ? nbr[(long long)(mirror >= 0 ? mirror - k2 : k2) * n_rows + row] : -1;
     reinterpret_cast<int4 *>(order + PCE_ORDER_REC_OFFSET(n_rows))[p] = r;
+    // rows with two neighbours or more: the 128-byte record with the neighbour at every offset
+    const long long n_single = tail[ORDER_N_SINGLE];
+    const long long si = (long long)gbase[key] + rank - n_single;
+    if (key >= 32 && (long long)tail[ORDER_N_NONZERO] - n_single <= PCE_ORDER_SREC_ROWS(n_rows)) {
+      int v[32];
+      v[0] = (int)row;
+      v[1] = (int)m;
+#pragma unroll
+      for (int k = 0; k < PCE_ORDER_SREC_KV; ++k) {   // (loads from an address valid for every k, selected afterwards)
+        const bool has = (m >> k) & 1u;
+        const int x = nbr[(long long)(has ? (mirror >= 0 ? mirror - k : k) : 0) * n_rows + row];
+        v[2 + k] = has ? x : -1;
+      }
+      pce_v4i *dst = reinterpret_cast<pce_v4i *>(order + PCE_ORDER_SREC_OFFSET(n_rows) + si * 32);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) dst[q] = pce_v4i{v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]};
+    }
   }
 }
 

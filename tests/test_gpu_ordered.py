@@ -59,7 +59,8 @@ def test_row_order_built_with_the_map_and_on_its_own(cloud):
     km = _subm(coords)
     n = len(coords)
     rec_at = (2 * n + 8192 + 3) // 4 * 4
-    assert km.order is not None and km.order.numel() == rec_at + 4 * n == _lib.load().pce_row_order_elems(n)
+    srec_at, srec_rows = rec_at + 4 * n, n // 8 + 32
+    assert km.order is not None and km.order.numel() == srec_at + 32 * srec_rows == _lib.load().pce_row_order_elems(n)
     lazy = _subm(coords, want_order=False)
     assert lazy.order is None
     backend.row_order(lazy)
@@ -94,6 +95,19 @@ def test_row_order_built_with_the_map_and_on_its_own(cloud):
             bits = [k for k in range(27) if (mask >> k) & 1]
             assert nb0 == nbr_of[(row, bits[0])]
             assert nb1 == (nbr_of[(row, bits[1])] if len(bits) > 1 else -1)
+        # the 128-byte records of the rows with two neighbours or more, in the order's sequence: row, mask and the
+        # neighbour at every offset (-1 where there is none); written where those rows are at most an eighth
+        n_single = int((pc == 1).sum())
+        shared = perm[n_plain + n_single:]
+        if len(shared) <= srec_rows:
+            srec = order[srec_at:srec_at + 32 * len(shared)].reshape(len(shared), 32).astype(np.int64)
+            assert np.array_equal(srec[:, 0], shared) and np.array_equal(srec[:, 1], masks[shared])
+            want = np.full((len(shared), 30), -1, np.int64)
+            for i, row in enumerate(shared):
+                for k in range(27):
+                    if (masks[row] >> k) & 1:
+                        want[i, k] = nbr_of[(int(row), k)]
+            assert np.array_equal(srec[:, 2:], want)
 
 
 @pytest.mark.parametrize("cloud", sorted(CLOUDS))
