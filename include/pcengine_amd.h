@@ -8,10 +8,22 @@
  * State the library keeps between calls: (1) per device, a ring of eight pinned host blocks (32 KB
  * each, allocated on the first pce_kmap_build / pce_kmap_build_batch on that device, never freed)
  * from which the descriptors of a batched map build are copied to the device, guarded by one mutex,
- * so calls from several host threads are safe; (2) the thread-local text of pce_last_error().
- * Nothing else: no caches, no tables, no switches.  (The stage mask a benchmark uses to time one
- * kernel of a dataflow alone exists only in the separately built measurement library, see
- * pcengine_amd_measure.h.)
+ * so calls from several host threads are safe; (2) a static device array of 32 MiB per GPU the library
+ * runs on, the accumulator of pce_conv_fwd_fod_static, with its device address looked up once per device
+ * (pce_conv_fod_static_init, or the first call); calls of that entry point that overlap on one GPU race;
+ * (3) the number of compute units of each device, asked once; (4) the thread-local text of
+ * pce_last_error().  Nothing else: no caches, no tables, no switches.  (The stage mask a benchmark uses to
+ * time one kernel of a dataflow alone exists only in the separately built measurement library, see
+ * pcengine_amd_measure.h; that library carries a static array of its own.)
+ *
+ * Versioning: pce_version() returns PCE_ABI_VERSION of the header the library was built from.  The structs
+ * below (pce_epilogue_t, pce_kmap_problem_t, pce_pyr_*_t) have no size field: a caller compiles against the
+ * header of the library it loads, zero-initialises every struct with the sizeof of that header, and refuses to
+ * run when pce_version() differs from its PCE_ABI_VERSION.  Version 200 against 100: pce_epilogue_t grew
+ * ld_in / ld_out, pce_kmap_problem_t grew n_batch / flags / order and its status became int32[8], the row
+ * order grew records, pce_conv_fwd_oso and pce_row_order take three counts, pce_select_dataflow takes mid and
+ * transposed, pce_set_stage_mask left this library; pce_pyramid_*, pce_outcoords_chain_planned,
+ * pce_conv_oso_takes and pce_conv_fod_static_init are new.
  *
  * These entry points are what the reference's five pybind functions
  * (backend/pybind_cuda.cpp:8-14) decompose into:
@@ -78,6 +90,7 @@ typedef struct pce_geom {
   int32_t subm;       /* 1: submanifold (out coords = in coords, centre offset handled densely) */
 } pce_geom_t;
 
+#define PCE_ABI_VERSION 200
 int pce_version(void);
 const char *pce_last_error(void);
 
@@ -349,8 +362,13 @@ int pce_conv_fwd_fod(const void *in_feats, const void *weight, const void *weigh
  * has no centre offset, overwrites the accumulator rows before they are added to.  All calls on one GPU share
  * that GPU's array: calls that overlap in time on one GPU (different streams or host threads) race and
  * must be serialised by the caller.  Same results as pce_conv_fwd_fod up to the order of its fp32 atomic
- * additions. */
+ * additions.
+ * The device address of the array is looked up once per device, with hipGetSymbolAddress under a mutex, on
+ * the first call on that device: a caller that captures calls into a HIP graph runs
+ * pce_conv_fod_static_init() on the device beforehand, outside the capture (it does that look-up and nothing
+ * else; an uncaptured first call of pce_conv_fwd_fod_static serves as well). */
 int64_t pce_conv_fod_static_capacity_bytes(void);
+int pce_conv_fod_static_init(void);
 int pce_conv_fwd_fod_static(const void *in_feats, const void *weight, const void *weight_packed,
                             void *out_feats, int32_t dtype,
                             int64_t n_in, int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv,
@@ -539,9 +557,18 @@ int pce_conv_wgrad(const void *in_feats, const void *grad_out, int32_t dtype, in
                    const int32_t *imap_dev, const int32_t *omap_dev, const int32_t *kpos_dev,
                    const int32_t *qkpos_dev, int64_t qsum, float *grad_w_f32_dev, pce_stream_t stream);
 
-/* Per-layer dataflow choice from map density (pairs per output row) and channel widths. */
+/* Per-layer dataflow choice from map density (pairs per output row), channel widths and the layer's kind:
+ * `mid` as in the forward entry points (the centre offset of a submanifold layer, -1 otherwise), `transposed`
+ * 1 for a transposed layer (n_in / n_out are then the rows read and written by that layer, i.e. the map's
+ * swapped).  Returns a PCE_DATAFLOW_* code whose entry point takes the layer: PCE_DATAFLOW_OSO only where
+ * pce_conv_oso_takes() is 1 and the layer is not transposed.  (Replaces the reference's fixed choice per layer
+ * class, PCEngine/script/spconv.py:94-124: D1 or D2 by the tag the model file sets.) */
 int pce_select_dataflow(int64_t n_in, int64_t n_out, int64_t n_pairs, int32_t c_in, int32_t c_out,
-                        int32_t kv, int32_t dtype);
+                        int32_t kv, int32_t mid, int32_t transposed, int32_t dtype);
+
+/* 1 when pce_conv_fwd_oso takes a layer of this dtype, these widths, kernel volume and centre offset (it checks
+ * alignment and the packed weights besides), else 0. */
+int pce_conv_oso_takes(int32_t dtype, int32_t c_in, int32_t c_out, int32_t kv, int32_t mid);
 
 #ifdef __cplusplus
 }

@@ -19,6 +19,7 @@ DATAFLOW_FOD, DATAFLOW_GMS, DATAFLOW_OS, DATAFLOW_FDS, DATAFLOW_OSO = 0, 1, 2, 3
 QUANTUM = 128
 KMAP_NO_GRID = 1
 KMAP_TABLE_ONLY = 2
+ABI_VERSION = 200        # PCE_ABI_VERSION of include/pcengine_amd.h
 CSR_CODE = 1186111
 
 
@@ -134,6 +135,7 @@ _SIGNATURES = {
     "pce_conv_fwd_fod": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32,
                                    c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, POINTER(Epilogue), c_void_p]),
     "pce_conv_fod_static_capacity_bytes": (c_int64, []),
+    "pce_conv_fod_static_init": (c_int32, []),
     "pce_conv_fwd_fod_static": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32,
                                           c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, POINTER(Epilogue), c_void_p]),
     "pce_conv_fwd_gms": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32,
@@ -150,7 +152,8 @@ _SIGNATURES = {
     "pce_pyramid_plan_sizeof": (c_int64, []),
     "pce_pyramid_plan": (c_int32, [c_int64, c_int32, POINTER(Geom), c_int32, POINTER(PyrRequest), c_int32, POINTER(PyrPlan)]),
     "pce_pyramid_build": (c_int32, [POINTER(PyrPlan), c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
-    "pce_select_dataflow": (c_int32, [c_int64, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32]),
+    "pce_select_dataflow": (c_int32, [c_int64, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32]),
+    "pce_conv_oso_takes": (c_int32, [c_int32, c_int32, c_int32, c_int32, c_int32]),
 }
 
 # only in the measurement build (include/pcengine_amd_measure.h)
@@ -181,6 +184,10 @@ def load() -> ctypes.CDLL:
             f"{LIB_PATH} is missing: build it with `python -m pcengine_amd.build` "
             "(hipcc, --offload-arch=gfx950).  pcengine_amd has no other compute path.")
     lib = ctypes.CDLL(LIB_PATH)
+    lib.pce_version.restype = c_int32
+    if lib.pce_version() != ABI_VERSION:
+        raise PCEError(f"{LIB_PATH} has ABI version {lib.pce_version()}, this package binds version {ABI_VERSION}: "
+                       "rebuild it with `python -m pcengine_amd.build`")
     _attach(lib, _SIGNATURES)
     _lib = lib
     return lib

@@ -710,16 +710,11 @@ def row_order(km: KernelMap) -> torch.Tensor:
 
 
 def oso_takes(km: KernelMap, c_in: int, c_out: int, dtype: torch.dtype, transposed: bool = False) -> bool:
-    """Shapes the ordered output-stationary dataflow exists for."""
-    if transposed or km.kv > 31:
+    """Layers the ordered output-stationary dataflow takes (``pce_conv_oso_takes``; never a transposed layer)."""
+    if transposed or dtype not in (torch.float16, torch.float32):
         return False
-    if dtype == torch.float32:
-        return km.subm and c_in % 8 == 0 and c_in <= 32 and c_out % 8 == 0 and c_out <= 32
-    if dtype != torch.float16 or c_out % 8:
-        return False
-    if c_out <= 64:
-        return c_in % 16 == 0 and c_in <= 64
-    return (c_in in (64, 96) and c_out <= 128) or (c_in == 128 and c_out <= 96)      # the K-stepped form (wave_osw_kernel)
+    code = PCE_F16 if dtype == torch.float16 else PCE_F32
+    return bool(_lib.load().pce_conv_oso_takes(code, c_in, c_out, km.kv, _mid(km.ks) if km.subm else -1))
 
 
 def ensure_nbr(km: KernelMap, transposed: bool) -> None:
@@ -737,10 +732,8 @@ def select_dataflow(km: KernelMap, c_in: int, c_out: int, dtype: torch.dtype, tr
     lib = _lib.load()
     n_out = km.n_in if transposed else km.n_out
     n_in = km.n_out if transposed else km.n_in
-    df = lib.pce_select_dataflow(n_in, n_out, km.M, c_in, c_out, km.kv, PCE_F16 if dtype == torch.float16 else PCE_F32)
-    if df == DATAFLOW_OSO and not oso_takes(km, c_in, c_out, dtype, transposed):
-        df = DATAFLOW_FDS       # the row counts of such a layer, but transposed, or with an even kernel size at stride 1
-    return df
+    return lib.pce_select_dataflow(n_in, n_out, km.M, c_in, c_out, km.kv, _mid(km.ks) if km.subm else -1, int(bool(transposed)),
+                                   PCE_F16 if dtype == torch.float16 else PCE_F32)
 
 
 def pack_weights(weight: torch.Tensor) -> Optional[torch.Tensor]:

@@ -2021,7 +2021,7 @@ static __device__ __align__(256) unsigned char scratch[PCE_STATIC_SCRATCH_BYTES]
 static void *g_scratch_ptr[PCE_STATIC_MAX_DEVICES];
 static std::mutex g_scratch_mutex;
 
-// device address of this device's copy of `scratch` (looked up on the first call on the device)
+// device address of this device's copy of `scratch` (looked up by pce_conv_fod_static_init, or on the first call on the device)
 static int static_scratch(void **ptr) {
   int dev = 0;
   PCE_HIP(hipGetDevice(&dev));
@@ -2038,6 +2038,11 @@ static int static_scratch(void **ptr) {
 }
 
 extern "C" int64_t pce_conv_fod_static_capacity_bytes(void) { return PCE_STATIC_SCRATCH_BYTES; }
+
+extern "C" int pce_conv_fod_static_init(void) {
+  void *p = nullptr;
+  return static_scratch(&p);
+}
 
 extern "C" int pce_conv_fwd_fod_static(const void *in, const void *w, const void *wp, void *out, int32_t dtype, int64_t n_in,
                                        int64_t n_out, int32_t c_in, int32_t c_out, int32_t kv, int32_t mid,
@@ -2988,7 +2993,7 @@ __global__ void __launch_bounds__(256, 2) wave_osw_kernel(TileArgs a, const int 
 #pragma unroll
     for (int j = 0; j < 16; ++j) acc[nb][j] = 0.f;
   // the weight fragments of an offset, GB K steps at a time: all of them up to 18 (72 registers), else two batches
-  constexpr int GB = KS * NB <= 18 ? KS : KS / 2;
+  constexpr int GB = KS * NB <= 18 ? KS : (KS + 1) / 2;   // (the second batch of an odd KS is one step shorter)
   if (centre) {
     const half_t *Wk = Wp + mid * wstep + ((long long)g * a.n_pad + l32) * 8;
 #pragma unroll
@@ -2998,15 +3003,17 @@ __global__ void __launch_bounds__(256, 2) wave_osw_kernel(TileArgs a, const int 
       for (int s = 0; s < GB; ++s)
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
-          wf[s][nb] = *reinterpret_cast<const half8 *>(Wk + ((long long)(2 * (b0 + s)) * a.n_pad + nb * 32) * 8);
+          if (b0 + s < KS) wf[s][nb] = *reinterpret_cast<const half8 *>(Wk + ((long long)(2 * (b0 + s)) * a.n_pad + nb * 32) * 8);
       // the global -> LDS copies have landed once nothing is outstanding; the fragment reads stay behind this statement
       // (the first batch of weights travels with the rows)
       if (b0 == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
       for (int s = 0; s < GB; ++s) {
-        const half8 af = Pl[wave][l32 * PPR + ((2 * (b0 + s) + g) ^ row_swizzle<PPR>(l32))];
+        if (b0 + s < KS) {
+          const half8 af = Pl[wave][l32 * PPR + ((2 * (b0 + s) + g) ^ row_swizzle<PPR>(l32))];
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[s][nb], af, acc[nb], 0, 0, 0);
+          for (int nb = 0; nb < NB; ++nb) acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[s][nb], af, acc[nb], 0, 0, 0);
+        }
       }
     }
   }
@@ -3031,7 +3038,7 @@ __global__ void __launch_bounds__(256, 2) wave_osw_kernel(TileArgs a, const int 
       for (int s = 0; s < GB; ++s)
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
-          wf[s][nb] = *reinterpret_cast<const half8 *>(Wk + ((long long)(2 * (b0 + s)) * a.n_pad + nb * 32) * 8);
+          if (b0 + s < KS) wf[s][nb] = *reinterpret_cast<const half8 *>(Wk + ((long long)(2 * (b0 + s)) * a.n_pad + nb * 32) * 8);
       if (b0 == 0) {
         nb_next = a.nbr[nidx];
         __builtin_amdgcn_sched_barrier(0);
@@ -3044,7 +3051,8 @@ __global__ void __launch_bounds__(256, 2) wave_osw_kernel(TileArgs a, const int 
 #pragma unroll
       for (int s = 0; s < GB; ++s)
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[s][nb], af[b0 + s], acc[nb], 0, 0, 0);
+        for (int nb = 0; nb < NB; ++nb)
+          if (b0 + s < KS) acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[s][nb], af[b0 + s], acc[nb], 0, 0, 0);
     }
   }
   if (heavy) {
@@ -3075,9 +3083,25 @@ __global__ void __launch_bounds__(256, 2) wave_osw_kernel(TileArgs a, const int 
 
 // shapes the K-stepped form takes: fp16, 64 or 96 channels in and 65 to 128 out, or 128 in and 65 to 96 out (the shapes
 // it was measured to lead on; 128 -> 128 and 192 -> 128 ran 3 to 30 % behind deferred scatter)
+// widths the K-stepped kernel is built for: 4 to 8 K steps of 16 input channels, 3 or 4 blocks of 32 output columns,
+// at most 24 weight fragments per offset and lane (what leaves a wavefront its accumulators beside them)
+static bool osw_widths(int c_in, int c_out) {
+  const int ks = c_in / 16, nb = (c_out + 31) / 32;
+  return c_in % 16 == 0 && c_out % 8 == 0 && ks >= 4 && ks <= 8 && nb >= 3 && nb <= 4 && ks * nb <= 24;
+}
+// widths of the ordered-row kernel proper (fp16) and of its fp32 form
+static bool os_widths(int c_in, int c_out) { return c_in % 16 == 0 && c_in <= 64 && c_out % 8 == 0 && c_out <= 64; }
+static bool os_f32_widths(int c_in, int c_out) { return c_in % 8 == 0 && c_in <= 32 && c_out % 8 == 0 && c_out <= 32; }
+// layers pce_conv_fwd_oso takes, by dtype, widths, kernel volume and centre offset alone (it checks alignment and
+// the packed weights besides): what the selector may answer PCE_DATAFLOW_OSO for
+static bool oso_layer(int dtype, int c_in, int c_out, int kv, int mid) {
+  if (kv < 1 || kv >= ORDER_MAX_KV || mid >= kv || c_in <= 0 || c_out <= 0) return false;
+  if (dtype == PCE_F32) return mid >= 0 && os_f32_widths(c_in, c_out);
+  return dtype == PCE_F16 && (os_widths(c_in, c_out) || osw_widths(c_in, c_out));
+}
+
 static bool wave_osw_ok(const TileArgs &a, int kv, int mid) {
-  const bool shape = (a.c_in == 64 || a.c_in == 96) ? a.c_out <= 128 : (a.c_in == 128 && a.c_out <= 96);
-  return a.Wp && a.a_vec && a.o_vec && shape && a.c_out % 8 == 0 && a.c_out > 64 && kv < ORDER_MAX_KV && mid < kv &&
+  return a.Wp && a.a_vec && a.o_vec && osw_widths(a.c_in, a.c_out) && kv < ORDER_MAX_KV && mid < kv &&
          aligned16(a.bias) && aligned16(a.res);
 }
 
@@ -3215,8 +3239,8 @@ extern "C" int pce_conv_fwd_oso(const void *in, const void *w, const void *wp, v
   const bool wide = !f32 && wave_osw_ok(a, kv, mid);
   if (!wide && (f32 ? !wave_os_f32_ok(a, kv, mid) : !wave_os_ok(a, kv, mid)))
     PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: takes layers in fp16 of at most 64 channels (multiples of 16 in, 8 out, packed "
-                         "weights), of 64 or 96 -> 65..128 and 128 -> 65..96 channels, or submanifold layers in fp32 of at most "
-                         "32 (multiples of 8), 16-byte aligned rows, kernel volumes up to 31; got dtype %d, %d -> %d channels, "
+                         "weights), of 64..128 -> 65..128 channels with c_in / 16 * ceil(c_out / 32) <= 24, or submanifold layers in fp32 "
+                         "of at most 32 (multiples of 8), 16-byte aligned rows, kernel volumes up to 31; got dtype %d, %d -> %d channels, "
                          "kv %d, mid %d", (int)dtype, (int)c_in, (int)c_out, (int)kv, (int)mid);
   if (n_heavy < 0 || n_heavy > n_out) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: n_heavy=%lld outside [0, n_out]", (long long)n_heavy);
   if (n_nonzero >= 0 && (n_nonzero < n_heavy || n_nonzero > n_out))
@@ -3257,7 +3281,8 @@ extern "C" int pce_conv_fwd_oso(const void *in, const void *w, const void *wp, v
     PCE_LAUNCH_CHECK("wave_osw");                                                                            \
     return PCE_OK;                                                                                           \
   }
-    PCE_WOSW_CASE(3, 4) PCE_WOSW_CASE(3, 6) PCE_WOSW_CASE(3, 8) PCE_WOSW_CASE(4, 4) PCE_WOSW_CASE(4, 6)
+    PCE_WOSW_CASE(3, 4) PCE_WOSW_CASE(3, 5) PCE_WOSW_CASE(3, 6) PCE_WOSW_CASE(3, 7) PCE_WOSW_CASE(3, 8)
+    PCE_WOSW_CASE(4, 4) PCE_WOSW_CASE(4, 5) PCE_WOSW_CASE(4, 6)
 #undef PCE_WOSW_CASE
     PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: unsupported shape c_in=%d c_out=%d", (int)c_in, (int)c_out);
   }
@@ -4152,6 +4177,10 @@ extern "C" int pce_concat_cols(const void *a, int32_t c_a, const void *b, int32_
   return PCE_OK;
 }
 
+extern "C" int pce_conv_oso_takes(int32_t dtype, int32_t c_in, int32_t c_out, int32_t kv, int32_t mid) {
+  return oso_layer(dtype, c_in, c_out, kv, mid) ? 1 : 0;
+}
+
 // Map density rho = pairs per output row.  The deferred-scatter dataflow does only the useful
 // multiplications and pays M*(c_in + 2*c_out) elements of gather / partial-row traffic for them; the
 // output-stationary kernel touches no intermediate memory but multiplies every offset of every
@@ -4170,44 +4199,42 @@ extern "C" int pce_concat_cols(const void *a, int32_t c_a, const void *b, int32_
 // The atomic fetch-on-demand and the staged gather-GEMM-scatter dataflows of the reference were never
 // the fastest (gather-GEMM-scatter comes first only on a 4-channel input layer, by 10 %).
 extern "C" int pce_select_dataflow(int64_t n_in, int64_t n_out, int64_t n_pairs, int32_t c_in, int32_t c_out, int32_t kv,
-                                   int32_t dtype) {
+                                   int32_t mid, int32_t transposed, int32_t dtype) {
   if (n_out <= 0) return PCE_DATAFLOW_FDS;
   if (kv == 1) return PCE_DATAFLOW_OS;
   const double rho = (double)n_pairs / (double)n_out;
   const int64_t prod = (int64_t)c_in * c_out;
+  // The ordered dataflow, where pce_conv_fwd_oso takes the layer (never a transposed one: its rows are the inputs').
+  const bool oso = !transposed && oso_layer(dtype, c_in, c_out, kv, mid);
+  const bool subm = mid >= 0, down = mid < 0 && kv <= 8 && n_out < n_in;
   // narrow fp16 submanifold layers: one launch over rows ordered by neighbour pattern.  Measured against deferred
   // scatter with bias, residual and ReLU fused: 0.78-0.93 of its time at 0.1-0.2 pairs per row (100-150 k voxels,
   // 16-64 channels), 0.62-0.83 at 0.8, 0.64-0.83 at 3, 0.60-0.62 at 5.3 (541 k voxels, where it equals plain
   // output-stationary); beyond that the dense output-stationary tiles below take over.
-  // the fp32 form is bound by its MFMAs (v_mfma_f32_32x32x2_f32, c_in / 2 of them per offset and wavefront): measured
-  // against deferred scatter at 4.7 pairs per row 0.76 (8 channels), 0.87 (16), 1.15 (32); at 0.2 pairs per row 0.49, 0.62, 0.82
-  if (dtype == PCE_F32 && n_in == n_out && kv >= 3 && kv <= 31 && (kv & 1) && c_in % 8 == 0 && c_in <= 32 && c_out % 8 == 0 &&
-      c_out <= 32 && rho <= (c_in <= 16 ? 6.0 : 2.0))
+  // the fp32 form is bound by its MFMAs (c_in / 4 of them per offset and 16 rows): measured against deferred scatter
+  // at 4.7 pairs per row 0.76 (8 channels), 0.87 (16), 1.15 (32); at 0.2 pairs per row 0.49, 0.62, 0.82
+  if (oso && subm && dtype == PCE_F32 && rho <= (c_in <= 16 ? 6.0 : 2.0)) return PCE_DATAFLOW_OSO;
+  // (a cloud of fewer than two 128-row tiles per compute unit -- 256 of them -- leaves the dense tiles' launch short
+  // of workgroups: 24 k rows at 9.2 pairs per row, 48 -> 48 channels: ordered rows 17 us, deferred scatter 21, tiles 28)
+  if (oso && subm && dtype == PCE_F16 && os_widths(c_in, c_out) && rho <= (n_out < 2 * 256 * 128 ? 12.0 : 6.0)) return PCE_DATAFLOW_OSO;
+  // the K-stepped form of the same kernel (wave_osw_kernel): a wavefront walks c_in / 16 K steps per offset of its
+  // rows' union, so the density up to which it leads falls with the input width.  Measured on the levels of a
+  // 100 k-voxel LiDAR pyramid against the faster of deferred scatter and the dense tiles: 64 -> 96, 96 -> 96, 64 -> 128
+  // (4 to 6 K steps) at 0.8 / 3.0 / 8.9 pairs per row 0.80-0.88 / 0.71-0.79 / 0.81-0.91 of its time (equal at 0.13 and
+  // at 19.5); 128 -> 96 (8 K steps) 0.91 at 0.8 and 3.0, 1.03-1.12 elsewhere
+  if (oso && subm && dtype == PCE_F16 && osw_widths(c_in, c_out) && rho >= 0.5 && rho <= (c_in <= 96 ? 12.0 : 4.0))
     return PCE_DATAFLOW_OSO;
-  if (dtype == PCE_F16 && n_in == n_out && kv >= 3 && kv <= 31 && (kv & 1) && c_in % 16 == 0 && c_in <= 64 && c_out % 8 == 0 &&
-      c_out <= 64 && rho <= 6.0)
-    return PCE_DATAFLOW_OSO;
-  // the K-stepped form of the same kernel (wave_osw_kernel), measured on the levels of a 100 k-voxel LiDAR pyramid
-  // against the faster of deferred scatter and the dense tiles: 64 -> 96, 96 -> 96, 64 -> 128 at 0.8 / 3.0 / 8.9 pairs
-  // per row 0.80-0.88 / 0.71-0.79 / 0.81-0.91 of its time (equal at 0.13 and at 19.5); 128 -> 96 0.91 at 0.8 and 3.0,
-  // 1.03-1.12 elsewhere
-  if (dtype == PCE_F16 && n_in == n_out && kv >= 3 && kv <= 31 && (kv & 1) && c_out % 8 == 0 && c_out > 64) {
-    if ((c_in == 64 || c_in == 96) && c_out <= 128 && rho >= 0.5 && rho <= 12.0) return PCE_DATAFLOW_OSO;
-    if (c_in == 128 && c_out <= 96 && rho >= 0.5 && rho <= 4.0) return PCE_DATAFLOW_OSO;
-  }
   // narrow fp16 stride-2 layers (every input row in exactly one pair, 1-8 per output row), through the same ordered
   // rows without a centre term: 0.58-0.66 of the output-stationary tiles' time at 1.0-1.4 pairs per row (66-146 k
   // output rows, 32 and 64 channels; 680 k rows: 0.71), 0.57 at 2.4 on 27 k rows and 1.05 at 2.5 on 276 k rows of
   // indoor scenes, where half the rows have three pairs or more
-  if (dtype == PCE_F16 && kv <= 8 && n_out < n_in && c_in % 16 == 0 && c_in <= 64 && c_out % 8 == 0 && c_out <= 64 && rho <= 2.0)
-    return PCE_DATAFLOW_OSO;
+  if (oso && down && dtype == PCE_F16 && os_widths(c_in, c_out) && rho <= 2.0) return PCE_DATAFLOW_OSO;
   // ... and of the K-stepped kernel's shapes: 64 -> 128, 64 / 96 -> 96, 96 -> 128, 128 -> 96 at 1.0-2.5 pairs per row on
   // five levels of LiDAR and indoor pyramids (26 k to 541 k output rows) 0.64-0.94 of the faster of deferred scatter
-  // and the dense tiles (64 -> 128 on the 146 k-row level of the headline cloud: 21.3 vs 24.5 us); 128 -> 128, tried
-  // with a sixth instantiation, ran from 0.72 to 1.06 of it with nothing in (rows, density) to tell the cases apart
-  if (dtype == PCE_F16 && kv <= 8 && n_out < n_in && c_out % 8 == 0 && c_out > 64 && rho <= 2.6 &&
-      (((c_in == 64 || c_in == 96) && c_out <= 128) || (c_in == 128 && c_out <= 96)))
-    return PCE_DATAFLOW_OSO;
+  // and the dense tiles (64 -> 128 on the 146 k-row level of the headline cloud: 21.3 vs 24.5 us); 128 -> 128 (32
+  // weight fragments per offset: beyond what the kernel is built for) ran from 0.72 to 1.06 of it with nothing in
+  // (rows, density) to tell the cases apart
+  if (oso && down && dtype == PCE_F16 && osw_widths(c_in, c_out) && rho <= 2.6) return PCE_DATAFLOW_OSO;
   if (kv <= 8 && n_out <= n_in && rho >= 1.0 && prod <= 64 * 64 && dtype == PCE_F16) return PCE_DATAFLOW_OS;
   if (kv <= 8 && n_out <= n_in && rho >= 2.0 && prod <= 128 * 128 && dtype == PCE_F16) return PCE_DATAFLOW_OS;
   double takeover;

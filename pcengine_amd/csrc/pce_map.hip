@@ -24,7 +24,7 @@ void pce_set_error(const char *fmt, ...) {
 }
 
 extern "C" const char *pce_last_error(void) { return g_err; }
-extern "C" int pce_version(void) { return 100; }
+extern "C" int pce_version(void) { return PCE_ABI_VERSION; }
 
 // ------------------------------------------------------------------------------------------------
 // small device helpers

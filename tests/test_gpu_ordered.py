@@ -140,7 +140,8 @@ def test_map_built_without_pair_lists(cloud):
 
 @pytest.mark.parametrize("cloud", sorted(CLOUDS))
 @pytest.mark.parametrize("c_in,c_out", [(64, 64), (32, 32), (16, 32), (48, 24), (64, 8), (16, 64),
-                                        (64, 96), (96, 96), (64, 128), (96, 128), (128, 96), (96, 72)])   # the last six: the K-stepped kernel
+                                        (64, 96), (96, 96), (64, 128), (96, 128), (128, 96), (96, 72),
+                                        (80, 96), (112, 80), (80, 128)])   # from 64 -> 96 on: the K-stepped kernel
 def test_ordered_dataflow_against_the_oracle(cloud, c_in, c_out):
     coords = CLOUDS[cloud]()
     ref, _ = _oracle_masks(coords)
@@ -196,10 +197,12 @@ def test_ordered_dataflow_fp32_against_the_oracle(cloud, c_in, c_out):
     again = backend.conv_forward(fd, wd, _subm(coords), DATAFLOW_OSO, bias=bd, act=("leaky_relu", 0.1))
     assert torch.equal(out, again)
     # column slices in and out, as the skip connections use them
-    wide_in = torch.full((n, c_in + 12), 7.0, dtype=torch.float32, device=DEV)
-    wide_in[:, 4:4 + c_in] = fd
+    # (row strides of whole 32-byte groups, so that both views are read and written in place: no dense copy is made)
+    wide_in = torch.full((n, c_in + 16), 7.0, dtype=torch.float32, device=DEV)
+    wide_in[:, 8:8 + c_in] = fd
     wide_out = torch.full((n, c_out + 16), -3.0, dtype=torch.float32, device=DEV)
-    got = backend.conv_forward(wide_in[:, 4:4 + c_in], wd, km, DATAFLOW_OSO, out=wide_out[:, 8:8 + c_out], bias=bd, act=("leaky_relu", 0.1))
+    assert backend._row_stride(wide_in[:, 8:8 + c_in]) == c_in + 16 and backend._row_stride(wide_out[:, 8:8 + c_out]) == c_out + 16
+    got = backend.conv_forward(wide_in[:, 8:8 + c_in], wd, km, DATAFLOW_OSO, out=wide_out[:, 8:8 + c_out], bias=bd, act=("leaky_relu", 0.1))
     assert torch.equal(got, out) and bool((wide_out[:, :8] == -3.0).all()) and bool((wide_out[:, 8 + c_out:] == -3.0).all())
 
 
@@ -253,7 +256,7 @@ def test_row_order_of_strided_maps(cloud, geom):
 
 @pytest.mark.parametrize("cloud", sorted(CLOUDS))
 @pytest.mark.parametrize("geom", range(len(STRIDED)))
-@pytest.mark.parametrize("c_in,c_out", [(32, 32), (64, 64), (16, 64), (48, 24), (64, 96), (128, 80)])
+@pytest.mark.parametrize("c_in,c_out", [(32, 32), (64, 64), (16, 64), (48, 24), (64, 96), (128, 80), (80, 104)])
 def test_ordered_dataflow_strided_against_the_oracle(cloud, geom, c_in, c_out):
     """The ordered rows without a centre term (strided layers, fp16): the float64 oracle within 1e-3, epilogue fused,
     bit-equal from run to run, column slices on both sides."""
@@ -323,7 +326,9 @@ def test_ordered_dataflow_on_column_slices_and_the_selector():
     assert backend.select_dataflow(km, 64, 64, torch.float32) != DATAFLOW_OSO
     assert backend.select_dataflow(km, 128, 128, torch.float16) != DATAFLOW_OSO
     assert backend.oso_takes(km, 96, 96, torch.float16) and backend.oso_takes(km, 128, 96, torch.float16)
+    assert backend.oso_takes(km, 80, 96, torch.float16) and backend.oso_takes(km, 112, 72, torch.float16) and backend.oso_takes(km, 80, 128, torch.float16)
     assert not backend.oso_takes(km, 128, 128, torch.float16) and not backend.oso_takes(km, 192, 128, torch.float16)
+    assert not backend.oso_takes(km, 112, 128, torch.float16)
     # the two pair-proportional dataflows agree to fp16 rounding (they round partial sums at different places)
     fds = backend.conv_forward(f, w, km, DATAFLOW_FDS, packed=packed)
     assert float((fds.float() - want.float()).norm() / want.float().norm()) <= 1e-3

@@ -75,7 +75,7 @@ def test_argument_validation_needs_no_gpu():
 def test_selector_is_monotone_in_density():
     lib = _lib.load()
     n = 100000
-    picks = [lib.pce_select_dataflow(n, n, int(rho * n), 64, 64, 27, 0) for rho in (0.1, 0.5, 1.0, 3.0, 8.0, 20.0)]
+    picks = [lib.pce_select_dataflow(n, n, int(rho * n), 64, 64, 27, 13, 0, 0) for rho in (0.1, 0.5, 1.0, 3.0, 8.0, 20.0)]
     assert picks[0] == _lib.DATAFLOW_OSO and picks[-1] == _lib.DATAFLOW_OS
     order = {_lib.DATAFLOW_OSO: 0, _lib.DATAFLOW_FDS: 0, _lib.DATAFLOW_FOD: 0, _lib.DATAFLOW_GMS: 1, _lib.DATAFLOW_OS: 2}
     ranks = [order[p] for p in picks]
@@ -109,21 +109,38 @@ def test_selector_on_measured_layers():
         (65807, 65807, 586656, 64, 128, 27, OSO),      # 56 vs 63 us for the dense tiles
         (25916, 25916, 506646, 64, 128, 27, OS),       # rho = 19.5: 33 vs 37 us
     ]
+    mid_of = lambda kv: kv // 2 if kv == 27 else -1
     for n_in, n_out, pairs, ci, co, kv, want in cases:
-        assert lib.pce_select_dataflow(n_in, n_out, pairs, ci, co, kv, _lib.PCE_F16) == want, (n_in, n_out, ci, co, kv)
+        assert lib.pce_select_dataflow(n_in, n_out, pairs, ci, co, kv, mid_of(kv), 0, _lib.PCE_F16) == want, (n_in, n_out, ci, co, kv)
+    sel = lambda n_in, n_out, pairs, ci, co, kv, dt, transposed=0: lib.pce_select_dataflow(n_in, n_out, pairs, ci, co, kv, mid_of(kv), transposed, dt)
     # fp32: the ordered dataflow up to 32 channels (configuration 1), deferred scatter beyond
-    assert lib.pce_select_dataflow(20804, 20804, 98238, 16, 16, 27, _lib.PCE_F32) == OSO
-    assert lib.pce_select_dataflow(20804, 20804, 98238, 64, 64, 27, _lib.PCE_F32) == FDS
-    assert lib.pce_select_dataflow(20804, 20804, 98238, 32, 32, 27, _lib.PCE_F32) == FDS      # 32 channels: only on sparse clouds
-    assert lib.pce_select_dataflow(149866, 149866, 30620, 32, 32, 27, _lib.PCE_F32) == OSO
+    assert sel(20804, 20804, 98238, 16, 16, 27, _lib.PCE_F32) == OSO
+    assert sel(20804, 20804, 98238, 64, 64, 27, _lib.PCE_F32) == FDS
+    assert sel(20804, 20804, 98238, 32, 32, 27, _lib.PCE_F32) == FDS      # 32 channels: only on sparse clouds
+    assert sel(149866, 149866, 30620, 32, 32, 27, _lib.PCE_F32) == OSO
     # narrow 2x2x2 stride-2 layers in fp16: the ordered rows up to two pairs per output row, the dense tiles beyond;
-    # never in fp32, never for the transposed layer (more output rows than input rows)
-    assert lib.pce_select_dataflow(149866, 146018, 149866, 32, 32, 8, _lib.PCE_F16) == OSO
-    assert lib.pce_select_dataflow(99692, 97941, 99692, 32, 32, 8, _lib.PCE_F16) == OSO
-    assert lib.pce_select_dataflow(89469, 65807, 89469, 64, 64, 8, _lib.PCE_F16) == OSO       # 1.36 pairs per row
-    assert lib.pce_select_dataflow(679728, 276205, 679728, 64, 64, 8, _lib.PCE_F16) == OS     # 2.46 on an indoor batch
-    assert lib.pce_select_dataflow(149866, 146018, 149866, 32, 32, 8, _lib.PCE_F32) != OSO
-    assert lib.pce_select_dataflow(146018, 149866, 149866, 32, 32, 8, _lib.PCE_F16) != OSO
+    # never in fp32, never for the transposed layer
+    assert sel(149866, 146018, 149866, 32, 32, 8, _lib.PCE_F16) == OSO
+    assert sel(99692, 97941, 99692, 32, 32, 8, _lib.PCE_F16) == OSO
+    assert sel(89469, 65807, 89469, 64, 64, 8, _lib.PCE_F16) == OSO       # 1.36 pairs per row
+    assert sel(679728, 276205, 679728, 64, 64, 8, _lib.PCE_F16) == OS     # 2.46 on an indoor batch
+    assert sel(149866, 146018, 149866, 32, 32, 8, _lib.PCE_F32) != OSO
+    assert sel(146018, 149866, 149866, 32, 32, 8, _lib.PCE_F16, 1) != OSO
+    # The ordered dataflow is answered only for layers its entry point takes: over a grid of widths, kernel volumes,
+    # centre offsets, dtypes and densities every OSO answer is a layer pce_conv_oso_takes accepts, never a transposed
+    # one; an fp32 layer without a centre offset and equal row counts (a strided layer that lost no rows) is not one.
+    for dt in (_lib.PCE_F16, _lib.PCE_F32):
+        for kv, mid in ((27, 13), (27, -1), (8, -1), (125, 62), (31, 15), (33, 16), (9, 4)):
+            for ci in (4, 8, 16, 24, 32, 48, 64, 80, 96, 112, 128, 160, 192, 256):
+                for co in (8, 16, 20, 32, 48, 64, 72, 80, 96, 128, 160, 192, 256):
+                    for n_in, n_out, pairs in ((50000, 50000, 5000), (50000, 50000, 100000), (50000, 50000, 600000), (50000, 40000, 50000)):
+                        for tr in (0, 1):
+                            if lib.pce_select_dataflow(n_in, n_out, pairs, ci, co, kv, mid, tr, dt) == OSO:
+                                assert tr == 0 and lib.pce_conv_oso_takes(dt, ci, co, kv, mid) == 1, (dt, kv, mid, ci, co, n_in, n_out)
+    assert lib.pce_select_dataflow(50000, 50000, 50000, 16, 16, 27, -1, 0, _lib.PCE_F32) != OSO
+    assert lib.pce_conv_oso_takes(_lib.PCE_F16, 80, 96, 27, 13) == 1 and lib.pce_conv_oso_takes(_lib.PCE_F16, 112, 96, 27, 13) == 1
+    assert lib.pce_conv_oso_takes(_lib.PCE_F16, 128, 128, 27, 13) == 0 and lib.pce_conv_oso_takes(_lib.PCE_F16, 112, 128, 27, 13) == 0
+    assert lib.pce_conv_oso_takes(_lib.PCE_F16, 64, 64, 33, 16) == 0
 
 
 def test_codes_and_strides():

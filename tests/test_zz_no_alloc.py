@@ -90,3 +90,42 @@ def test_static_scratch_entry_point_limits_and_fp32():
                                            None, torch.cuda.current_stream().cuda_stream))
     want = orc.conv_forward(rounded(f, torch.float32), rounded(w, torch.float32), ref, (3, 3, 3))
     assert orc.rel_l2(out.double().cpu().numpy(), want) <= 1e-5
+
+
+def test_static_scratch_entry_point_under_graph_capture():
+    """Two calls of the static entry point captured into one HIP graph (the second on a smaller layer, both sharing
+    the array), after pce_conv_fod_static_init outside the capture: every replay, with eager work and
+    synchronisations in between, equals the workspace entry point's result to the bar of the eager test."""
+    lib = _lib.load()
+    assert lib.pce_conv_fod_static_init() == _lib.PCE_OK
+    dt = torch.float16
+    layers = []
+    for seed, coords, c_in, c_out in [(5, synth.random_cloud(seed=83, n=20000, extent=30, batches=2), 32, 64),
+                                      (6, synth.random_cloud(seed=84, n=3000, extent=14), 64, 32)]:
+        km = gpu_map(coords, (3, 3, 3), (1, 1, 1), (0, 0, 0))
+        fd = torch.as_tensor(synth.features(seed, km.n_in, c_in), device=DEV).to(dt)
+        wd = torch.as_tensor(synth.weights(seed, km.kv, c_in, c_out), device=DEV).to(dt)
+        out = torch.full((km.n_out, c_out), float("nan"), dtype=dt, device=DEV)
+        ws_bytes = lib.pce_conv_fod_workspace_bytes(km.n_out, c_out, _lib.PCE_F16)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=DEV)
+        want = torch.empty_like(out)
+        tail = (_lib.PCE_F16, km.n_in, km.n_out, c_in, c_out, km.kv, 13, km.imap.data_ptr(), km.omap.data_ptr(), km.kpos.data_ptr(),
+                km.qkpos.data_ptr(), km.qsum)
+        _lib.check(lib.pce_conv_fwd_fod(fd.data_ptr(), wd.data_ptr(), None, want.data_ptr(), *tail, ws.data_ptr(), ws_bytes, None,
+                                        torch.cuda.current_stream().cuda_stream))
+        layers.append((km, fd, wd, out, want, tail))
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        s = torch.cuda.current_stream().cuda_stream
+        for km, fd, wd, out, want, tail in layers:
+            _lib.check(lib.pce_conv_fwd_fod_static(fd.data_ptr(), wd.data_ptr(), None, out.data_ptr(), *tail, None, s))
+    for _ in range(3):
+        for km, fd, wd, out, want, tail in layers:
+            out.fill_(float("nan"))
+        (layers[0][1] * 2).sum().item()          # eager work and a synchronisation between replays
+        g.replay()
+        torch.cuda.synchronize()
+        for km, fd, wd, out, want, tail in layers:
+            assert bool(torch.isfinite(out).all())
+            assert orc.rel_l2(out.double().cpu().numpy(), want.double().cpu().numpy()) <= 1e-3
