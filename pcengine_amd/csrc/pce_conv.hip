@@ -3110,6 +3110,10 @@ static bool wave_osw_ok(const TileArgs &a, int kv, int mid) {
 // values the lane with g = 0 holds the first half, the lane with g = 1 the second (KQ 16-byte loads each), and MFMA
 // step (q, e) of v_mfma_f32_32x32x2_f32 contracts k = 4 q + e (lanes 0-31) with k = c_in / 2 + 4 q + e (lanes 32-63);
 // the weights of an offset are read in that order, one value per lane and step, 128 contiguous bytes per half.
+// (A form on v_mfma_f32_16x16x4_f32 -- half the MFMA time at 16 output columns -- with the offsets in a three-stage
+// software pipeline measured 10.5 us where this kernel takes 9.8 on a 21 k-voxel surface cloud at 16 -> 16 channels,
+// and 23.3 against 17.1 at 32 -> 32: the layer is bound by its gathers, not by the MFMA chain, and that form issues
+// more of them per offset.)
 template <int KQ>
 __global__ void __launch_bounds__(256, 4) wave_os_f32_kernel(TileArgs a, const int *__restrict__ perm,
                                                              const unsigned *__restrict__ rmask, int mid, long long n_main,
@@ -3250,8 +3254,15 @@ extern "C" int pce_conv_fwd_oso(const void *in, const void *w, const void *wp, v
   if ((uintptr_t)order & 15) PCE_FAIL(PCE_EINVAL, "pce_conv_fwd_oso: the order array must be 16-byte aligned");
   a.nbr = nbr;
   a.n_rows = n_out;
-  const long long n_main = n_out - n_heavy;
-  const long long heavy_wgs = pce_div_up(n_heavy, 32), main_wgs = pce_div_up(pce_div_up(n_main, 32), 4);
+  // Chunks of rows with two neighbours or more (the end of the order: rows with two, then rows with three or more)
+  // take a workgroup each, its four wavefronts splitting the offsets; the chunks before them a wavefront each.  A
+  // caller that states only the count of rows with three or more gets those split.  (Splitting the rows with two as
+  // well: 15.1 -> 10.4 us on a 21 k-voxel surface cloud in fp32 16 -> 16, 14.3 -> 11.9 in fp16 64 -> 64, where the
+  // few chunks of such rows, each with a union of eight offsets or more walked by one wavefront, ended last; 0-8 %
+  // on the levels of a LiDAR pyramid.)
+  const long long n_split = (n_nonzero >= 0 && n_single >= 0) ? n_nonzero - n_single : n_heavy;
+  const long long n_main = n_out - n_split;
+  const long long heavy_wgs = pce_div_up(n_split, 32), main_wgs = pce_div_up(pce_div_up(n_main, 32), 4);
   if (heavy_wgs + main_wgs >= (1ll << 31) - 8) PCE_FAIL(PCE_ECAPACITY, "pce_conv_fwd_oso: %lld rows exceed the grid limit", (long long)n_out);
   const unsigned grid = (unsigned)(heavy_wgs + main_wgs);
   const int *perm = order;
@@ -4220,9 +4231,10 @@ extern "C" int pce_select_dataflow(int64_t n_in, int64_t n_out, int64_t n_pairs,
   // the K-stepped form of the same kernel (wave_osw_kernel): a wavefront walks c_in / 16 K steps per offset of its
   // rows' union, so the density up to which it leads falls with the input width.  Measured on the levels of a
   // 100 k-voxel LiDAR pyramid against the faster of deferred scatter and the dense tiles: 64 -> 96, 96 -> 96, 64 -> 128
-  // (4 to 6 K steps) at 0.8 / 3.0 / 8.9 pairs per row 0.80-0.88 / 0.71-0.79 / 0.81-0.91 of its time (equal at 0.13 and
-  // at 19.5); 128 -> 96 (8 K steps) 0.91 at 0.8 and 3.0, 1.03-1.12 elsewhere
-  if (oso && subm && dtype == PCE_F16 && osw_widths(c_in, c_out) && rho >= 0.5 && rho <= (c_in <= 96 ? 12.0 : 4.0))
+  // (4 to 6 K steps) at 0.13 / 0.8 / 3.0 / 8.9 pairs per row 0.89-0.93 / 0.77-0.85 / 0.71-0.79 / 0.81-0.91 of its time
+  // (equal at 19.5; 80 -> 80 at 0.06 on 50 k rows: 0.66); 128 -> 96 (8 K steps) 0.97 at 0.13, 0.81 at 0.8, 0.91 at 3.0,
+  // 1.03-1.12 beyond
+  if (oso && subm && dtype == PCE_F16 && osw_widths(c_in, c_out) && rho <= (c_in <= 96 ? 12.0 : 4.0))
     return PCE_DATAFLOW_OSO;
   // narrow fp16 stride-2 layers (every input row in exactly one pair, 1-8 per output row), through the same ordered
   // rows without a centre term: 0.58-0.66 of the output-stationary tiles' time at 1.0-1.4 pairs per row (66-146 k

@@ -91,7 +91,7 @@ def test_selector_on_measured_layers():
         (97941, 97941, 80234, 32, 32, 27, OSO),        # narrow layers of a LiDAR network: rho 0.8 and 3.0
         (89469, 89469, 271786, 64, 64, 27, OSO),
         (541185, 541185, 2852000, 64, 64, 27, OSO),    # indoor batch, rho 5.3: equal to output-stationary, 0.6 of deferred scatter
-        (99692, 99692, 13406, 96, 96, 27, FDS),        # hardly any pairs: the centre GEMM decides, deferred scatter as fast
+        (99692, 99692, 13406, 96, 96, 27, OSO),        # hardly any pairs: 18-20 vs 20-22 us for deferred scatter
         (97941, 97941, 80234, 96, 96, 27, OSO),        # the K-stepped ordered kernel: 28 vs 32 us
         (97941, 97941, 80234, 128, 96, 27, OSO),       # 31 vs 34 us
         (89469, 89469, 271786, 128, 128, 27, FDS),     # wider than the ordered kernels take: 64 vs 67 us
