@@ -2731,7 +2731,25 @@ __global__ void __launch_bounds__(256, 4) wave_os2_kernel(TileArgs a, const int 
   const half_t *A = (const half_t *)a.A;
   const long long wstep = (long long)a.k8_total * a.n_pad * 8;
   const long long n = a.n_rows;
-  if ((int)blockIdx.x >= shared_wgs) {   // (the shared workgroups read the centre weights as they read the others')
+  // ---- shared: 32 rows with two neighbours or more per workgroup ------------------------------------------------
+  // first the chunks of rows with three neighbours or more, the longest walks of the launch: at 33-64 output
+  // channels two workgroups each, one per block of 32 columns (ten offsets in flight instead of six); then the
+  // chunks of rows with two
+  // (first in the code as well: these workgroups have the longest way to go, and what a wavefront runs before its
+  // first load it fetches from a cold instruction cache)
+  const long long n_shared = n - n_plain - n_single;
+  if ((int)blockIdx.x < heavy_wgs) {
+    if (NB == 2)
+      os2_shared_chunk<1, KS, REGION>(a, order, mid, n_two + (long long)(blockIdx.x >> 1) * 32, n_shared, (blockIdx.x & 1) * 32, Pl);
+    else
+      os2_shared_chunk<NB, KS, REGION>(a, order, mid, n_two + (long long)blockIdx.x * 32, n_shared, 0, Pl);
+    return;
+  }
+  if ((int)blockIdx.x < shared_wgs) {
+    os2_shared_chunk<NB, KS, REGION>(a, order, mid, ((long long)blockIdx.x - heavy_wgs) * 32, n_two, 0, Pl);
+    return;
+  }
+  {   // (the shared workgroups read the centre weights as they read the others')
     constexpr int FR = KS * 2 * NB * 32;   // fragments: [k8][column]
 #pragma unroll
     for (int i = 0; i < (FR + 255) / 256; ++i) {
@@ -2881,19 +2899,6 @@ __global__ void __launch_bounds__(256, 4) wave_os2_kernel(TileArgs a, const int 
     return;
   }
 #undef PCE_OS2_FRAGS
-  // ---- shared: 32 rows with two neighbours or more per workgroup ------------------------------------------------
-  // first the chunks of rows with three neighbours or more, the longest walks of the launch: at 33-64 output
-  // channels two workgroups each, one per block of 32 columns (ten offsets in flight instead of six); then the
-  // chunks of rows with two
-  const long long n_shared = n - n_plain - n_single;
-  if ((int)blockIdx.x < heavy_wgs) {
-    if (NB == 2)
-      os2_shared_chunk<1, KS, REGION>(a, order, mid, n_two + (long long)(blockIdx.x >> 1) * 32, n_shared, (blockIdx.x & 1) * 32, Pl);
-    else
-      os2_shared_chunk<NB, KS, REGION>(a, order, mid, n_two + (long long)blockIdx.x * 32, n_shared, 0, Pl);
-  } else {
-    os2_shared_chunk<NB, KS, REGION>(a, order, mid, ((long long)blockIdx.x - heavy_wgs) * 32, n_two, 0, Pl);
-  }
 }
 
 // compute units of the current device (asked once per device)
@@ -3302,11 +3307,12 @@ extern "C" int pce_conv_fwd_oso(const void *in, const void *w, const void *wp, v
   // the chains of dependent trips to memory that set the duration of a launch of one round of wavefronts; it
   // multiplies the rows with neighbours twice, which costs more than that saves once the rows come in several rounds.
   // Needs the counts of rows with any neighbour and with exactly one; a caller that does not state them (-1), a
-  // layer without a centre offset, 16 input channels (one wavefront of four would walk the shared rows) and other
-  // clouds take the kernel that visits every row through the order.  This kernel / that one, 64 -> 64 channels:
-  // 7.3 / 12.3 us on 60 k rows of a LiDAR scan, 9.1 / 10.5 on 90 k, 11.4 / 11.9 on all 150 k (4 % of the rows with
-  // two neighbours or more), 8.7 / 12.2 on a 100 k scan; 34.4 / 32.2 on four scans in a batch; 16 -> 32: 7.0 / 6.7.
-  if (mid >= 0 && kv <= PCE_ORDER_SREC_KV && ks >= 2 && n_nonzero >= 0 && n_single >= 0 && 2 * n_nonzero <= n_out &&
+  // layer without a centre offset, fewer than 48 input channels (its shared rows are walked by one wavefront per
+  // 16 input channels) and other clouds take the kernel that visits every row through the order.  This kernel /
+  // that one, 64 -> 64 channels: 11.2 / 11.8 us on a 150 k-voxel LiDAR scan (4 % of the rows with two neighbours or
+  // more), 8.5 / 10.0 on a 100 k scan; 32.4 / 32.4 on four scans in a batch (that kernel either way); 32 -> 32: 7.6 /
+  // 7.8 on the 150 k scan, 6.6 / 5.7 on the 100 k scan, 5.9 / 4.7 on half of it; 16 -> 32: 7.0 / 6.7.
+  if (mid >= 0 && kv <= PCE_ORDER_SREC_KV && ks >= 3 && n_nonzero >= 0 && n_single >= 0 && 2 * n_nonzero <= n_out &&
       n_nonzero - n_single <= PCE_ORDER_SREC_ROWS(n_out) && 8 * (n_nonzero - n_single) <= n_out &&
       os2_workgroups(n_out, n_nonzero, n_single, n_heavy, nb) <= 4ll * cu_count() && stage_on(12))
     return launch_wave_os2(a, order, (int)mid, n_out, n_nonzero, n_single, n_heavy, nb, ks, s);

@@ -342,7 +342,7 @@ SPARSE_CLOUDS = {
 
 
 @pytest.mark.parametrize("cloud", sorted(SPARSE_CLOUDS))
-@pytest.mark.parametrize("c_in,c_out", [(64, 64), (32, 32), (16, 64), (48, 24), (64, 8)])
+@pytest.mark.parametrize("c_in,c_out", [(64, 64), (32, 32), (16, 64), (48, 24), (64, 8), (48, 64)])
 def test_streamed_form_against_the_ordered_form(cloud, c_in, c_out):
     """Clouds where at most half the rows have a neighbour run as three kinds of workgroup (rows without neighbours
     streamed in storage order, rows with one by their records, the rest shared by four wavefronts): against the
