@@ -117,6 +117,51 @@ def regret_summary(records):
             "time_weighted": round(picked / best, 4), "picked_ms": round(picked, 4), "best_ms": round(best, 4)}
 
 
+def trace_net(config, forwards):
+    """Forwards of the network of configuration 4 or 5 on its synthetic cloud: two to warm up (the first builds the
+    kernel maps), `forwards` over the kept maps, `forwards` more with the maps built by the native planner."""
+    import torch
+    import pcengine_amd as pe
+    from pcengine_amd import nets, synth
+    dev = "cuda:0"
+    if config == "cfg4":
+        coords, kw, batches = synth.lidar_cloud_100k(), {}, 1
+    else:
+        coords, kw, batches = synth.indoor_batch(), dict(stem=64, enc=(64, 128, 256, 512), dec=(512, 256, 192, 192)), 8
+    feats = torch.as_tensor(synth.features(4, len(coords), 4), device=dev).half()
+    cd = torch.as_tensor(coords, device=dev)
+    torch.manual_seed(4)
+    model = nets.SparseResUNet(4, 20, **kw).to(dev).eval().fuse_bn().half()
+    cmax = coords[:, 1:].max(0).tolist()
+
+    def forward(keep=None):
+        x = pe.spTensor(feats, cd, None, [0, 0, 0], cmax, batchsize=batches)
+        if keep is not None:
+            x.kmaps, x.cbook = keep.kmaps, keep.cbook
+        with torch.no_grad():
+            return model(x)
+
+    def timed(fn):
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(forwards):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / max(forwards, 1)
+    y0 = forward()
+    forward(y0)
+    kept = timed(lambda: forward(y0))
+    model.use_planner()
+    for _ in range(3):
+        forward()
+    planned = timed(forward)
+    print(json.dumps({"config": config, "voxels": len(coords), "forwards": forwards, "forward_ms_kept_maps": round(kept, 3),
+                      "forward_ms_planned_map_build": round(planned, 3)}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -132,10 +177,17 @@ def main() -> int:
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip configurations 1 (fp32 C16 layer), 3 (k2s2 down + transposed up) and 5 (8-scene indoor "
                          "batch, widened network), whose timings go to extra.cfg1 / cfg3 / cfg5")
+    ap.add_argument("--trace-net", default=None, choices=["cfg4", "cfg5"],
+                    help="run only forwards of the configuration-4 / configuration-5 network (what a kernel trace of the "
+                         "network is taken from): --forwards of them over kept kernel maps, then as many that build their "
+                         "maps through the native planner; prints one line and exits")
+    ap.add_argument("--forwards", type=int, default=5)
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this engine has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         return 2
+    if args.trace_net:
+        return trace_net(args.trace_net, args.forwards)
 
     import numpy as np
     import torch

@@ -18,7 +18,11 @@ extern "C" {
  * sum in its epilogue), 5 = the pipelined tile kernel for wide fp16 layers (cleared: the single-stage
  * tile kernel), 6 = pair tiles and centre GEMM of a wide deferred-scatter layer in one launch (cleared:
  * two launches), 9 = the pipelined output-stationary kernel for wide fp16 layers of few tiles (cleared:
- * the single-stage tile kernel).  Default: all bits set.  Process-wide and unsynchronised: one thread,
+ * the single-stage tile kernel), 10 = output rows may leave with the non-temporal hint (cleared: never),
+ * 11 = ... only where the output tensor is 16 MiB or more (cleared, with 10 set: always), 12 = the
+ * three-kind form of the ordered dataflow on clouds it is meant for and its stream workgroups as the plain
+ * GEMM of narrow fp16 layers (cleared: the kernel that visits every row through the order; the tile
+ * kernel).  Default: all bits set.  Process-wide and unsynchronised: one thread,
  * measurement runs only. */
 void pce_set_stage_mask(uint32_t mask);
 

@@ -191,45 +191,3 @@ class SparseResUNet(nn.Module):
             x = up(x, out=buf[:, :up.conv.out_channels])
             x = dec(x._like(buf))
         return self.head(x)
-
-
-def _main() -> None:
-    """``python -m pcengine_amd.nets``: the network of configuration 4 or 5 on its synthetic cloud, a few forwards with
-    the kernel maps kept (what a kernel trace of the network is taken from)."""
-    import argparse
-    from . import synth
-    ap = argparse.ArgumentParser(description="forward passes of the configuration-4 / configuration-5 network on synthetic data")
-    ap.add_argument("--config", default="cfg4", choices=["cfg4", "cfg5"])
-    ap.add_argument("--forwards", type=int, default=5)
-    args = ap.parse_args()
-    dev = "cuda:0"
-    if args.config == "cfg4":
-        coords, kw, batches = synth.lidar_cloud_100k(), {}, 1
-    else:
-        coords, kw, batches = synth.indoor_batch(), dict(stem=64, enc=(64, 128, 256, 512), dec=(512, 256, 192, 192)), 8
-    feats = torch.as_tensor(synth.features(4, len(coords), 4), device=dev).half()
-    cd = torch.as_tensor(coords, device=dev)
-    torch.manual_seed(4)
-    model = SparseResUNet(4, 20, **kw).to(dev).eval().fuse_bn().half()
-    cmax = coords[:, 1:].max(0).tolist()
-
-    def forward(keep=None):
-        x = spTensor(feats, cd, None, [0, 0, 0], cmax, batchsize=batches)
-        if keep is not None:
-            x.kmaps, x.cbook = keep.kmaps, keep.cbook
-        with torch.no_grad():
-            return model(x)
-    y0 = forward()
-    forward(y0)
-    torch.cuda.synchronize()
-    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    a.record()
-    for _ in range(args.forwards):
-        forward(y0)
-    b.record()
-    torch.cuda.synchronize()
-    print(f"{args.config}: {len(coords)} voxels, {a.elapsed_time(b) / max(args.forwards, 1):.3f} ms per forward over kept kernel maps")
-
-
-if __name__ == "__main__":
-    _main()
