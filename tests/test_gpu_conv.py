@@ -197,6 +197,33 @@ def test_dense_1x1(dtype):
         assert orc.rel_l2(out.double().cpu().numpy(), want) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("c_in,c_out", [(192, 192), (256, 192), (192, 168)])
+def test_dense_wide_many_rows(c_in, c_out):
+    """Plain GEMMs of wide fp16 layers on enough rows for the kernel that keeps the whole weight matrix in LDS
+    (a workgroup per CU, 32-row chunks per wavefront): a row count that is no multiple of 32, with and without the
+    epilogue, against float64 on sampled rows and bit for bit against the same rows computed in a short matrix (the
+    tile kernels); (192, 168) is a width that kernel is not built for."""
+    n = 131072 + 4097
+    rng = np.random.default_rng(c_in + c_out)
+    f = (rng.standard_normal((n, c_in)) * 0.5).astype(np.float32)
+    w = (rng.standard_normal((c_in, c_out)) * 0.05).astype(np.float32)
+    bias, res = rng.standard_normal(c_out) * 0.3, rng.standard_normal((n, c_out)).astype(np.float32)
+    dt = torch.float16
+    fd, wd = torch.as_tensor(f, device=DEV).to(dt), torch.as_tensor(w, device=DEV).to(dt)
+    bd, rd = torch.as_tensor(bias, device=DEV).to(dt), torch.as_tensor(res, device=DEV).to(dt)
+    pk = backend.pack_weights(wd)
+    rows = np.concatenate([np.arange(0, 70), rng.integers(0, n, 400), np.arange(n - 70, n)])
+    plain = backend.dense_forward(fd, wd, pk)
+    want = rounded(f[rows], dt) @ rounded(w, dt)
+    assert orc.rel_l2(plain[rows].double().cpu().numpy(), want) <= 1e-3
+    fused = backend.dense_forward(fd, wd, pk, bias=bd, residual=rd, act="relu")
+    want = np.maximum(want + rounded(bias, dt) + rounded(res[rows], dt), 0)
+    assert orc.rel_l2(fused[rows].double().cpu().numpy(), want) <= 1e-3
+    assert bool(torch.isfinite(fused).all())
+    head = slice(0, 5000)
+    assert torch.equal(backend.dense_forward(fd[head].contiguous(), wd, pk, bias=bd, residual=rd[head].contiguous(), act="relu"), fused[head])
+
+
 def test_config1_fp32_c16():
     coords = synth.sphere_plane_cloud()
     fd, wd, ref_map, want = _case(coords, (3, 3, 3), (1, 1, 1), (0, 0, 0), 16, 16, torch.float32, seed=1)
