@@ -1482,13 +1482,9 @@ static void launch_tile_nb(TileArgs a, long long tiles, hipStream_t s) {
   }
 }
 
-static int launch_wres_gemm(const TileArgs &a, hipStream_t s);
-static bool wres_gemm_ok(const TileArgs &a, int elem_size);
-
 template <typename T>
 static int launch_tile(const TileArgs &a, long long tiles, hipStream_t s) {
   if (tiles <= 0) return PCE_OK;
-  if (stage_on(13) && wres_gemm_ok(a, sizeof(T))) return launch_wres_gemm(a, s);
   if (tiles * ((a.c_out + 127) / 128) >= (1ll << 31) - 8) PCE_FAIL(PCE_ECAPACITY, "tile count %lld exceeds the grid limit", tiles);
   // plain GEMMs of 96 columns and at most 128 input channels stay with the tile kernel below: 12.1 vs 13.8 us on
   // 100 k rows (128 -> 96), 75 vs 80 and 87 vs 94 us on 950 k rows (96 -> 96, 128 -> 96); from 128 columns the pipelined
@@ -2905,123 +2901,6 @@ __global__ void __launch_bounds__(256, 4) wave_os2_kernel(TileArgs a, const int 
 #undef PCE_OS2_FRAGS
 }
 
-// Plain GEMM of a wide fp16 layer (centre terms of the wide deferred-scatter layers, 1x1 shortcuts) with the WHOLE
-// packed weight matrix resident in LDS (72 KB at 192 x 192, 96 KB at 256 x 192): one workgroup per CU stays for the
-// launch, copies the weights once, and its wavefronts then work independently of one another -- no barrier after
-// the first -- each over chunks of 32 consecutive rows: rows global -> LDS in line order into the wavefront's own
-// region, KS x NB MFMAs with both operands read from LDS, epilogue, rows out through the same region as full lines.
-// The tile kernels read the weights again for every 128-row tile (72 KB per tile at 192 x 192: 534 MB of L2 traffic
-// for 365 MB of rows on 950 k rows) and the rows once per 128-column slab.
-template <int NB, int KS, int WAVES, bool DB>
-__global__ void __launch_bounds__(WAVES * 64, 1) wres_gemm_kernel(TileArgs a) {
-  constexpr int PPR = KS * 2;   // 16-byte pieces per input row
-  constexpr int REGION = WaveLds<NB>::PIECES > 32 * PPR ? WaveLds<NB>::PIECES : 32 * PPR;
-  constexpr int FR = KS * 2 * NB * 32;   // weight fragments: [k8][column]
-  constexpr int BUFS = DB ? 2 : 1;       // row regions per wavefront: with two, the next chunk's rows travel during this chunk's MFMAs
-  static_assert((FR + WAVES * BUFS * REGION) * 16 <= 160 * 1024, "weights and the row regions fit the LDS of a CU");
-  static_assert(FR % (WAVES * 64) == 0, "every thread copies the same number of weight fragments");
-  __shared__ __attribute__((aligned(16))) half8 Wc[FR];
-  __shared__ __attribute__((aligned(16))) half8 Pl[WAVES][BUFS][REGION];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int l32 = lane & 31, g = lane >> 5;
-  const half_t *Wp = (const half_t *)a.Wp + (long long)a.w_fixed * a.k8_total * a.n_pad * 8;   // the weights of the layer's one offset
-  const half_t *A = (const half_t *)a.A;
-  const long long n = a.n_rows, chunks = (n + 31) / 32, step = (long long)gridDim.x * WAVES;
-#pragma unroll
-  for (int i = 0; i < FR / (WAVES * 64); ++i) {
-    const half_t *gp = Wp + (long long)(i * (WAVES * 64) + wave * 64 + lane) * 8;
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
-                                     (__attribute__((address_space(3))) void *)&Wc[i * (WAVES * 64) + wave * 64], 16, 0, 0);
-  }
-  long long c = (long long)blockIdx.x * WAVES + wave;
-  // the 32 rows of chunk c_ -> region b_ of this wavefront, in line order (rows past the end repeat the last row)
-#define PCE_WRES_ROWS(c_, b_)                                                                                      \
-  {                                                                                                                \
-    const long long r0_ = (c_) * 32;                                                                               \
-    _Pragma("unroll") for (int it = 0; it < KS; ++it) {                                                            \
-      const int e = it * 64 + lane, r = e / PPR, sl = e % PPR;                                                     \
-      const long long row = r0_ + r < n ? r0_ + r : n - 1;                                                         \
-      const half_t *gp = A + row * a.lda + ((sl ^ row_swizzle<PPR>(r)) * 8);                                       \
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,                         \
-                                       (__attribute__((address_space(3))) void *)&Pl[wave][b_][it * 64], 16, 0, 0); \
-    }                                                                                                              \
-  }
-  if (c < chunks) PCE_WRES_ROWS(c, 0)
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();   // the weights of all wavefronts' copies are in LDS; the only barrier of the kernel
-  int b = 0;
-  while (c < chunks) {
-    const long long cn = c + step;
-    if (DB && cn < chunks) {
-      // region b ^ 1 staged the previous chunk's rows; they were read back before their stores were issued
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      if (b == 0) PCE_WRES_ROWS(cn, BUFS - 1) else PCE_WRES_ROWS(cn, 0)
-    }
-    half8 *rows = Pl[wave][b];
-    f32x16 acc[NB];
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-      for (int j = 0; j < 16; ++j) acc[nb][j] = 0.f;
-    // (the fragments of K step s + 1 are requested before the MFMAs of step s: one wavefront per SIMD has nobody
-    // else to hide the LDS latency behind)
-    half8 wf[2][NB], af[2];
-#define PCE_WRES_FRAGS(B_, S_)                                                                                     \
-  {                                                                                                                \
-    af[B_] = rows[l32 * PPR + ((2 * (S_) + g) ^ row_swizzle<PPR>(l32))];                                           \
-    _Pragma("unroll") for (int nb = 0; nb < NB; ++nb) wf[B_][nb] = Wc[(2 * (S_) + g) * (NB * 32) + nb * 32 + l32]; \
-  }
-    PCE_WRES_FRAGS(0, 0)
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      if (s + 1 < KS) PCE_WRES_FRAGS((s + 1) & 1, s + 1)
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[s & 1][nb], af[s & 1], acc[nb], 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-#undef PCE_WRES_FRAGS
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    __builtin_amdgcn_wave_barrier();   // every lane has read its fragments: the region becomes the output staging area
-    const long long row = c * 32 + l32;
-    const int orow = row < n ? (int)row : -1;
-    float V[NB][2][8];
-    gather_row_pieces<NB>(acc, V, g);
-    if (a.bias || a.res || a.act) {
-      bool with_act = a.act != PCE_ACT_NONE;
-      if (with_act && a.act_alone_only) with_act = orow >= 0 && a.ocsr[orow] == a.ocsr[orow + 1];
-      epilogue_row_pieces<half_t, NB, true>(V, a, orow, 0, g, with_act);
-    }
-    if (DB) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the next chunk's rows (and the previous chunk's stores) before this chunk's stores queue up behind them
-    store_rows_via_lds<half_t, NB>(V, rows, (half_t *)a.out, orow, a, 0, lane, l32, g, a.stream);
-    c = cn;
-    if (DB) {
-      b ^= BUFS - 1;
-    } else if (c < chunks) {
-      // the staged rows have been read back (the stores hold them in registers): the region takes the next chunk
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      PCE_WRES_ROWS(c, 0)
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    }
-  }
-#undef PCE_WRES_ROWS
-}
-
-// shapes the weights-resident GEMM takes: fp16, packed weights, 16-byte rows everywhere, widths it is built for,
-// and enough rows that a workgroup per CU amortises its copy of the weights (this kernel / pipe_gemm_kernel, us:
-// 192 -> 192 on 951 k rows 180 / 213, 541 k 108 / 125, 216 k 44 / 45, 66 k 20 / 18; 256 -> 192: 206 / 252, 123 / 150,
-// 52 / 55, 23 / 22)
-static bool wres_gemm_ok(const TileArgs &a, int elem_size) {
-  const int nb = a.n_pad / 32, ks = a.c_in / 16;
-  const bool built = (nb == 6 && (ks == 12 || ks == 16));
-  return elem_size == 2 && a.mode == MODE_DENSE && a.epi == EPI_ROWS && a.Wp && a.a_vec && a.o_vec && a.c_in % 16 == 0 &&
-         a.k8_total == 2 * ks && built && aligned16(a.bias) && aligned16(a.res) && a.n_rows >= 128 * 1024;
-}
-
 // compute units of the current device (asked once per device)
 static int cu_count() {
   static int cached[64];
@@ -3033,27 +2912,6 @@ static int cu_count() {
     cached[dev] = v;
   }
   return cached[dev];
-}
-
-static int launch_wres_gemm(const TileArgs &a, hipStream_t s) {
-  const int nb = a.n_pad / 32, ks = a.c_in / 16, cus = cu_count();
-  if (cus <= 0) PCE_FAIL(PCE_EHIP, "wres_gemm: the device reports no compute units");
-  const long long chunks = pce_div_up(a.n_rows, 32);
-#define PCE_WRES_CASE(NB_, KS_, WAVES_, DB_)                                                                       \
-  if (nb == NB_ && ks == KS_) {                                                                                    \
-    const long long wgs = pce_div_up(chunks, WAVES_);                                                              \
-    hipLaunchKernelGGL((wres_gemm_kernel<NB_, KS_, WAVES_, DB_>), dim3((unsigned)(wgs < cus ? wgs : cus)), dim3(WAVES_ * 64), 0, \
-                       s, a);                                                                                      \
-    PCE_LAUNCH_CHECK("wres_gemm");                                                                                 \
-    return PCE_OK;                                                                                                 \
-  }
-  // (two row regions per wavefront, the next chunk's rows in flight during the MFMAs, leave room for three wavefronts
-  // at 192 input channels and two at 256: 198 and 340 us on 950 k rows against 181 and 204 with four wavefronts and
-  // one region each -- a wavefront is busy with its MFMAs and its epilogue, not waiting for its rows; six wavefronts
-  // with one region each at 192 input channels: 205 us)
-  PCE_WRES_CASE(6, 12, 4, false) PCE_WRES_CASE(6, 16, 4, false)
-#undef PCE_WRES_CASE
-  PCE_FAIL(PCE_EINVAL, "wres_gemm: unsupported shape c_in=%d c_out=%d", a.c_in, a.c_out);
 }
 
 // workgroups of the three-kind kernel over a row order

@@ -199,10 +199,9 @@ def test_dense_1x1(dtype):
 
 @pytest.mark.parametrize("c_in,c_out", [(192, 192), (256, 192), (192, 168)])
 def test_dense_wide_many_rows(c_in, c_out):
-    """Plain GEMMs of wide fp16 layers on enough rows for the kernel that keeps the whole weight matrix in LDS
-    (a workgroup per CU, 32-row chunks per wavefront): a row count that is no multiple of 32, with and without the
-    epilogue, against float64 on sampled rows and bit for bit against the same rows computed in a short matrix (the
-    tile kernels); (192, 168) is a width that kernel is not built for."""
+    """Plain GEMMs of wide fp16 layers on many rows (the centre terms and 1x1 shortcuts of a network's widest levels):
+    a row count that is no multiple of the tile height, with and without the epilogue, against float64 on sampled rows
+    and bit for bit against the same rows computed in a short matrix."""
     n = 131072 + 4097
     rng = np.random.default_rng(c_in + c_out)
     f = (rng.standard_normal((n, c_in)) * 0.5).astype(np.float32)
