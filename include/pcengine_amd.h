@@ -446,33 +446,45 @@ int pce_conv_fwd_os(const void *in_feats, const void *weight, const void *weight
                     const int32_t *nbr_dev, const pce_epilogue_t *epilogue, pce_stream_t stream);
 
 /* Output-stationary over ordered rows, for narrow layers on clouds where most voxels have few
- * neighbours (surfaces: 0.2 pairs per voxel on a 64 x 2048 LiDAR scan at 0.1 m).  pce_row_order derives from the
- * output-major neighbour table, once per map, the order in which the rows are visited -- rows without neighbours
- * first, in their own order, then the rows with one or two neighbours sorted by the offsets they have them at, then
- * the rows with three or more, sorted likewise -- and every row's offset mask: order_dev = perm[n_rows] |
- * mask[n_rows] | 8192 ints of scratch | rec[n_rows] (16 bytes each, for the positions of rows with a neighbour:
- * {row, mask, neighbour at the lowest offset of the mask, neighbour at the second-lowest or -1}),
- * pce_row_order_elems ints in all, 16-byte aligned; kv <= 31; four launches and one wait for counts_host[0] =
- * n_heavy, the number of rows of the last part, counts_host[1] = n_nonzero, the number of rows with any
- * neighbour, and counts_host[2] = n_single, the number with exactly one (they come first among the rows with
- * neighbours, sorted by the offset); the positions of rows with equal keys depend on the run, the results of the
- * layer do not.  pce_conv_fwd_oso takes the three counts as order_counts_host.  With n_nonzero and n_single stated
- * (-1: not known), submanifold fp16 layers of at most 64 channels on clouds where at most half the rows have a
- * neighbour run as three kinds of workgroup: the bulk of the rows streamed in storage order, 64 per wavefront,
- * stored where their mask is empty; rows with one neighbour by their records; rows with two or more 32 to a
- * workgroup (two workgroups above 32 output channels) whose wavefronts share the offsets.  pce_conv_fwd_oso then runs the layer as one launch: a wavefront takes 32 rows
- * of that order, multiplies their centre rows, gathers for each offset any of them has the neighbours of the rows
- * that have it, and stores each finished row once (epilogue fused); the rows of the last part, whose offsets are
- * many, go 32 to a workgroup whose four wavefronts share the offsets.  PCE_F16, packed weights: c_in a multiple of
- * 16 and at most 64 with c_out a multiple of 8 and at most 64; or c_in 64 or 96 with c_out a multiple of 8 in 65..128;
- * or c_in 128 with c_out a multiple of 8 in 65..96 (these wider shapes stream an offset's weights from the packed copy
- * K step by K step); PCE_F32: c_in and c_out multiples of 8 and at most 32
+ * neighbours (surfaces: 0.2 pairs per voxel on a 64 x 2048 LiDAR scan at 0.1 m).
+ *
+ * pce_row_order derives from the output-major neighbour table, once per map, the order in which the rows are
+ * visited -- rows without neighbours first, in their own order, then the rows with one neighbour sorted by its
+ * offset, the rows with two sorted by (lowest, second-lowest) offset, the rows with three or more likewise -- and
+ * what the kernels read of every row:
+ *   order_dev = perm[n_rows] | mask[n_rows] | 8192 ints of scratch
+ *             | rec[n_rows]  (16 bytes each, at the positions of rows with a neighbour: {row, mask, neighbour at
+ *                             the lowest offset of the mask, neighbour at the second-lowest or -1})
+ *             | srec[n_rows / 8 + 32]  (128 bytes each, for the i-th row with two neighbours or more: {row, mask,
+ *                             neighbour at offset 0 ... 29, -1 where there is none}; written only where those
+ *                             rows are at most n_rows / 8 + 32)
+ * pce_row_order_elems(n_rows) ints in all, 16-byte aligned; kv <= 31; four launches and one wait for counts_host[0]
+ * = n_heavy, the number of rows with three neighbours or more, counts_host[1] = n_nonzero, the number with any
+ * neighbour, and counts_host[2] = n_single, the number with exactly one.  The positions of rows with equal keys
+ * depend on the run, the results of the layer do not.  pce_kmap_build_batch builds the same with the map (status
+ * words 4, 6, 7).
+ *
+ * pce_conv_fwd_oso runs the layer as one launch over that order and takes the three counts as
+ * order_counts_host: THE COUNTS THAT CAME WITH THIS ORDER (the kernels find a row's records by them; counts of
+ * another order make them read rows that do not exist), or -1 for n_nonzero and n_single when they are not known.
+ * A wavefront takes 32 rows of the order, multiplies their centre rows, gathers for each offset any of them has
+ * the neighbours of the rows that have it, and stores each finished row once (epilogue fused); chunks of rows with
+ * two neighbours or more (three or more when only n_heavy is stated) go to a workgroup whose four wavefronts share
+ * the offsets.  With all counts stated, a centre offset (mid >= 0), PCE_F16 with 48-64 input channels, at most half
+ * the rows with a neighbour, at most an eighth with two or more, and few enough rows that all workgroups are
+ * resident at once, the launch has three kinds of workgroup instead: the bulk of the rows streamed in storage
+ * order, 64 per wavefront, stored where their mask is empty; rows with one neighbour by their 16-byte records; rows
+ * with two or more by their 128-byte records, 32 to a workgroup whose wavefronts split the input channels.
+ *
+ * Layers taken (pce_conv_oso_takes): PCE_F16 with packed weights, c_in a multiple of 16 and c_out of 8: both at most
+ * 64; or c_in 64..128 with c_out 65..128 and (c_in / 16) * ceil(c_out / 32) <= 24 (these stream an offset's
+ * weights from the packed copy K step by K step); PCE_F32: c_in and c_out multiples of 8 and at most 32
  * (weight_packed is not read) and mid >= 0; PCE_EINVAL otherwise.  In PCE_F16 a layer without a centre offset
  * (mid = -1: a strided layer, n_in != n_out, nbr_dev = its output-major table [kv][n_out], order from pce_row_order
  * with mid = -1) runs the same way from zero sums: every output row of a 2x2x2 stride-2 layer has one to eight pairs,
- * the order groups the rows by where they have them.  Takes the row strides
- * of pce_epilogue_t.  No counterpart in the reference: it computes what the fetch-on-demand kernels compute
- * (backend/spconv.cuh:1567-1730) with the scatter-add replaced by register accumulation, as pce_conv_fwd_os. */
+ * the order groups the rows by where they have them.  Takes the row strides of pce_epilogue_t.  No counterpart in
+ * the reference: it computes what the fetch-on-demand kernels compute (backend/spconv.cuh:1567-1730) with the
+ * scatter-add replaced by register accumulation, as pce_conv_fwd_os. */
 int64_t pce_row_order_elems(int64_t n_rows);
 int pce_row_order(const int32_t *nbr_dev, int32_t kv, int64_t n_rows, int32_t mid, int32_t *order_dev,
                   int64_t order_elems, int64_t *counts_host /* [3] */, pce_stream_t stream);
