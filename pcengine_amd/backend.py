@@ -732,8 +732,14 @@ def select_dataflow(km: KernelMap, c_in: int, c_out: int, dtype: torch.dtype, tr
     lib = _lib.load()
     n_out = km.n_in if transposed else km.n_out
     n_in = km.n_out if transposed else km.n_in
-    return lib.pce_select_dataflow(n_in, n_out, km.M, c_in, c_out, km.kv, _mid(km.ks) if km.subm else -1, int(bool(transposed)),
-                                   PCE_F16 if dtype == torch.float16 else PCE_F32)
+    df = lib.pce_select_dataflow(n_in, n_out, km.M, c_in, c_out, km.kv, _mid(km.ks) if km.subm else -1, int(bool(transposed)),
+                                 PCE_F16 if dtype == torch.float16 else PCE_F32)
+    if not km.has_pairs and df not in (DATAFLOW_OSO, DATAFLOW_OS):
+        # a map built without pair lists (its layers were expected to read the neighbour table only): rather than
+        # build them now, the layer takes the table-reading dataflow that is closest (a band of densities where the
+        # ordered dataflow is within a tenth of deferred scatter)
+        df = DATAFLOW_OSO if oso_takes(km, c_in, c_out, dtype, transposed) else DATAFLOW_OS
+    return df
 
 
 def pack_weights(weight: torch.Tensor) -> Optional[torch.Tensor]:

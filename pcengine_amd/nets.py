@@ -8,6 +8,7 @@ blocks), four decoder stages (transposed k2s2 + skip concatenation + two residua
 """
 from __future__ import annotations
 
+import os
 from typing import List, Sequence
 
 import torch
@@ -115,11 +116,33 @@ class SparseResUNet(nn.Module):
         self._arena = None         # made on the first planned forward, on the device of its input
         return self
 
-    def map_plan(self):
-        """(kernel_size, stride, padding) of the layers that need a kernel map, in execution order."""
-        plan = [(3, 1, 0)]
-        for _ in self.down:
-            plan += [(2, 2, 0), (3, 1, 0)]
+    def map_plan(self, dtype=None):
+        """(kernel_size, stride, padding[, table_only]) of the layers that need a kernel map, in execution order.
+        With ``dtype`` (an inference forward in that dtype) the 3x3x3 map of a level whose layers ALL have widths the
+        ordered output-stationary dataflow takes is marked table-only: the selector gives such layers the ordered or
+        the plain output-stationary dataflow, neither of which reads pair lists, so the build skips them (a layer
+        that asks for them after all -- a forced dataflow -- gets them built then)."""
+        lean = [False] * (len(self.down) + 1)
+        if dtype in (torch.float16, torch.float32):
+            code = backend.PCE_F16 if dtype == torch.float16 else backend.PCE_F32
+            takes = backend._lib.load().pce_conv_oso_takes
+            widths = [[] for _ in lean]           # (c_in, c_out) of the 3x3x3 layers of every level
+            auto = [True]
+            def add(level, module):
+                for m in module.modules():
+                    if isinstance(m, conv3d) and m.kernel_volume == 27 and not m.transposed and list(m.stride) == [1, 1, 1]:
+                        widths[level].append((max(m.in_channels, 16), m.out_channels))
+                        auto[0] = auto[0] and m.dataflow == "auto"
+            add(0, self.stem)
+            for l, enc in enumerate(self.enc):
+                add(l + 1, enc)
+            for i, dec in enumerate(self.dec):
+                add(len(self.down) - 1 - i, dec)
+            if auto[0] and not os.environ.get("PCENGINE_DATAFLOW"):
+                lean = [bool(w) and all(takes(code, ci, co, 27, 13) for ci, co in w) for w in widths]
+        plan = [(3, 1, 0, lean[0])]
+        for l in range(len(self.down)):
+            plan += [(2, 2, 0), (3, 1, 0, lean[l + 1])]
         return plan
 
     def forward(self, x: spTensor) -> spTensor:
@@ -135,7 +158,8 @@ class SparseResUNet(nn.Module):
     def _forward(self, x: spTensor, planner) -> spTensor:
         # no host wait is left between the layers below; with a planner (see use_planner) all maps of the cloud are
         # laid out and built by the library in one allocation
-        prebuild_maps(x, self.map_plan(), planner)
+        inference = not (torch.is_grad_enabled() and (x.feats.requires_grad or any(p.requires_grad for p in self.parameters())))
+        prebuild_maps(x, self.map_plan(x.feats.dtype if inference else None), planner)
         if self._skips_in_place(x):
             return self._forward_skips_in_place(x)
         x = self.stem(x)

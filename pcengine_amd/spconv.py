@@ -317,7 +317,8 @@ def _chain_out_coords(input: spTensor, layers) -> dict:
         return {}
     geoms, idx = [], []
     stride, cmax, cmin = input.stride, list(input.coords_max[:3]), list(input.coords_min[:3])
-    for i, (ks, st, pad) in enumerate(layers):
+    for i, entry in enumerate(layers):
+        ks, st, pad, _ = _layer_entry(entry)
         ksc, sc, pc = (conv_info_encoder(_triple(v, "layer")) for v in (ks, st, pad))
         if sc == _UNIT:
             continue
@@ -332,6 +333,17 @@ def _chain_out_coords(input: spTensor, layers) -> dict:
         return {}
     outs = backend.build_out_coords_chain(input.coords.contiguous(), geoms, input.batchsize)
     return dict(zip(idx, outs)) if outs is not None else {}
+
+
+def _layer_entry(entry):
+    """(kernel_size, stride, padding, table_only) of an entry of a layer list: the fourth element is optional and
+    says that every layer that will use the map takes a dataflow that reads the neighbour table and the row order
+    only (the ordered or the plain output-stationary one), so that a 3x3x3 submanifold map may be built without its
+    pair lists (``PCE_KMAP_TABLE_ONLY``; they are built on first use should a layer ask for them after all)."""
+    if len(entry) == 4:
+        return entry[0], entry[1], entry[2], bool(entry[3])
+    ks, stride, pad = entry
+    return ks, stride, pad, False
 
 
 class MapPlanner:
@@ -364,7 +376,8 @@ def _prebuild_planned(input: spTensor, layers, planner: MapPlanner):
     entries, strided, requests = [], [], []
     stride_code, cmin, cmax, level = input.stride, list(input.coords_min[:3]), list(input.coords_max[:3]), 0
     seen = {}
-    for ks, st, pad in layers:
+    for entry in layers:
+        ks, st, pad, table_only = _layer_entry(entry)
         ksc, sc, pc = (conv_info_encoder(_triple(v, "layer")) for v in (ks, st, pad))
         if ksc == _UNIT and sc == _UNIT:
             continue
@@ -376,7 +389,8 @@ def _prebuild_planned(input: spTensor, layers, planner: MapPlanner):
         if subm:
             if key not in seen:
                 seen[key] = len(requests)
-                requests.append((level, level, k3, s3, p3, cmin, cmax, True, True, False, False))
+                lean = table_only and k3 == (3, 3, 3)
+                requests.append((level, level, k3, s3, p3, cmin, cmax, True, not lean, False, lean))
                 entries.append((key, stride_code, level, level))
             continue
         if k3 != s3 or any(p3) or key in seen:
@@ -392,7 +406,7 @@ def _prebuild_planned(input: spTensor, layers, planner: MapPlanner):
         return None
     coords = input.coords if input.coords.is_contiguous() else input.coords.contiguous()
     n = coords.shape[0]
-    pkey = (tuple(map(tuple, ((r[0], r[1]) + tuple(r[2]) + tuple(r[6]) for r in requests))), tuple(input.coords_min[:3]),
+    pkey = (tuple(map(tuple, ((r[0], r[1], r[10]) + tuple(r[2]) + tuple(r[6]) for r in requests))), tuple(input.coords_min[:3]),
             int(input.batchsize), coords.device)
     try:
         plan = planner.plan_for(pkey, n, lambda cap: backend.PyramidPlan(cap, strided, requests, input.batchsize, coords.device))
@@ -422,7 +436,8 @@ def _prebuild(input: spTensor, layers, planner: Optional[MapPlanner] = None):
     pending, done = [], []
     chained = _chain_out_coords(input, layers)
     try:
-        for i, (ks, stride, pad) in enumerate(layers):
+        for i, entry in enumerate(layers):
+            ks, stride, pad, table_only = _layer_entry(entry)
             ksc, sc, pc = (conv_info_encoder(_triple(v, "layer")) for v in (ks, stride, pad))
             if ksc == _UNIT and sc == _UNIT:
                 continue
@@ -430,6 +445,8 @@ def _prebuild(input: spTensor, layers, planner: Optional[MapPlanner] = None):
             if request is not None:
                 if i in chained:
                     request["out_coords"] = chained[i]
+                if table_only and sc == _UNIT and tag not in ('D1', 'D2') and tuple(conv_info_decoder(ksc)) == (3, 3, 3):
+                    request["want_csr"], request["want_pairs"] = False, False
                 km = backend.prepare_map(**request)
                 pending.append((x, km, key, tag, out_stride))
                 x.kmaps[key] = km          # placeholder: a later entry with the same key is the same map
@@ -456,7 +473,8 @@ def _prebuild(input: spTensor, layers, planner: Optional[MapPlanner] = None):
 def prebuild_maps(input: spTensor, layers, planner: Optional[MapPlanner] = None) -> None:
     """Build, ahead of any convolution, the maps a network will ask for.  ``layers`` lists
     (kernel_size, stride, padding) in network order (ints or triples; transposed layers and 1x1
-    layers need no entry); a strided entry moves on to its output coordinates, as the network does.
+    layers need no entry; an optional fourth element True marks a 3x3x3 submanifold map whose layers all read the
+    neighbour table only, ``_layer_entry``); a strided entry moves on to its output coordinates, as the network does.
     The output coordinates of the strided layers are computed first, level by level (their number has
     to reach the host); then all maps are built together, every stage of the build as one launch over
     all layers, and their pair counts are read back in one copy.  The layers that follow find every

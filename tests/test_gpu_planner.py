@@ -144,3 +144,41 @@ def test_planned_forward_allocates_nothing_and_matches_the_plain_forward():
         got_big = model(xb()).feats.clone()
         model.use_planner(False)
         assert torch.equal(got_big, model(xb()).feats)
+
+
+@pytest.mark.parametrize("planned", [False, True])
+def test_network_builds_maps_without_pair_lists_where_its_layers_read_the_table_only(planned, monkeypatch):
+    """The U-Net marks the 3x3x3 map of a level table-only when every layer of the level has a width the ordered
+    dataflow takes (an fp16 inference forward of the default network: its two upper levels): those maps come without
+    pair lists, the others with them, and the forward is bit-identical to one whose maps were all built in full."""
+    coords = synth.lidar_cloud_100k()[::3].copy()
+    f = torch.as_tensor(synth.features(4, len(coords), 4), device=DEV).half()
+    cd = dev_coords(coords)
+    cmax = coords[:, 1:].max(0).tolist()
+    torch.manual_seed(4)
+    model = nets.SparseResUNet(4, 20).to(DEV).eval().fuse_bn().half()
+    plan = model.map_plan(torch.float16)
+    assert [e[3] for e in plan if len(e) == 4] == [True, True, False, False, False]
+    assert not any(e[3] for e in model.map_plan() if len(e) == 4) and not any(e[3] for e in model.map_plan(torch.float32) if len(e) == 4)
+    if planned:
+        model.use_planner()
+    mk = lambda: pe.spTensor(f, cd, None, [0, 0, 0], cmax, batchsize=1)
+    with torch.no_grad():
+        x = mk()
+        lean = model(x).feats.clone()
+        subm = sorted((km.n_out, km.has_pairs) for key, km in x.kmaps.items() if km.subm)
+        assert [h for _, h in subm] == [True, True, True, False, False]          # by rows: the two largest levels are lean
+        assert all(km.has_pairs for km in x.kmaps.values() if not km.subm)
+        monkeypatch.setattr(model, "map_plan", lambda dtype=None: [e[:3] for e in plan])
+        y = mk()
+        full = model(y).feats.clone()
+        assert all(km.has_pairs for km in y.kmaps.values())
+    assert torch.equal(lean, full)
+    # a forced dataflow that reads pair lists on a lean map builds them then
+    km = max((km for km in x.kmaps.values() if km.subm), key=lambda k: k.n_out)
+    w = torch.as_tensor(synth.weights(2, 27, 32, 32), device=DEV).half()
+    g = torch.as_tensor(synth.features(3, km.n_out, 32), device=DEV).half()
+    a = backend.conv_forward(g, w, km, backend.DATAFLOW_FDS)
+    assert km.has_pairs
+    b = backend.conv_forward(g, w, km, backend.DATAFLOW_OSO)
+    assert float((a.float() - b.float()).norm() / b.float().norm()) <= 2e-3
