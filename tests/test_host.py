@@ -143,6 +143,22 @@ def test_selector_on_measured_layers():
     assert lib.pce_conv_oso_takes(_lib.PCE_F16, 64, 64, 33, 16) == 0
 
 
+def test_network_map_plan_marks_levels_whose_layers_read_the_table_only():
+    """`SparseResUNet.map_plan(dtype)`: a level is table-only when all of its 3x3x3 layers have widths
+    `pce_conv_oso_takes` accepts in that dtype -- the two upper levels of the default network in fp16, none in fp32
+    (96 channels), none without a dtype (training), none when a dataflow is forced."""
+    import torch
+    from pcengine_amd import nets
+    marks = lambda plan: [e[3] for e in plan if len(e) == 4]
+    m = nets.SparseResUNet(4, 20)
+    assert marks(m.map_plan(torch.float16)) == [True, True, False, False, False]
+    assert marks(m.map_plan(torch.float32)) == [False] * 5 and marks(m.map_plan()) == [False] * 5
+    assert [e[:3] for e in m.map_plan()] == [(3, 1, 0), (2, 2, 0), (3, 1, 0), (2, 2, 0), (3, 1, 0), (2, 2, 0), (3, 1, 0), (2, 2, 0), (3, 1, 0)]
+    narrow = nets.SparseResUNet(4, 20, stem=16, enc=(16, 32, 32, 64), dec=(64, 32, 32, 16))
+    assert marks(narrow.map_plan(torch.float16)) == [True, True, True, False, True]      # the fourth level has a 96 -> 64 layer: no ordered width
+    assert marks(nets.SparseResUNet(4, 20, dataflow="fds").map_plan(torch.float16)) == [False] * 5
+
+
 def test_codes_and_strides():
     assert pe.conv_info_encoder([1, 1, 1]) == 94585
     for v in [(1, 1, 1), (2, 2, 2), (3, 1, 5), (8, 8, 8)]:
