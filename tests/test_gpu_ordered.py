@@ -413,3 +413,50 @@ def test_ordered_dataflow_argument_errors():
     with pytest.raises(ValueError):
         backend.conv_forward(torch.zeros((n, 192), dtype=torch.float16, device=DEV), torch.zeros((27, 192, 128), dtype=torch.float16, device=DEV),
                              km, DATAFLOW_OSO)
+
+
+def _molecules(singles, dimers, trimers, blob, seed=0):
+    """A cloud with chosen numbers of rows per neighbour count: isolated voxels, pairs of adjacent voxels (one
+    neighbour each), lines of three (the middle voxel has two neighbours), and one filled blob of blob^3 voxels
+    (three neighbours or more).  Groups sit on a lattice of pitch 4 so that they do not touch."""
+    rng = np.random.default_rng(seed)
+    groups = [np.zeros((1, 3), int)] * singles + [np.array([[0, 0, 0], [0, 0, 1]])] * dimers + \
+             [np.array([[0, 0, 0], [0, 1, 0], [0, 2, 0]])] * trimers
+    side = int(np.ceil(len(groups) ** (1 / 3))) + 1
+    cells = rng.permutation(side ** 3)[:len(groups)]
+    pts = [g + 4 * np.array([c // (side * side), (c // side) % side, c % side]) for g, c in zip(groups, cells)]
+    if blob:
+        b = np.stack(np.meshgrid(*[np.arange(blob)] * 3, indexing="ij"), -1).reshape(-1, 3) + 4 * side + 4
+        pts.append(b)
+    xyz = np.concatenate(pts, 0)
+    c = np.concatenate([np.zeros((len(xyz), 1), int), xyz], 1)
+    return np.unique(c, axis=0).astype(np.int32)
+
+
+@pytest.mark.parametrize("mix", [(3000, 0, 0, 0), (3000, 400, 0, 0), (3000, 0, 300, 0), (5000, 300, 100, 0), (4000, 200, 100, 6),
+                                 (2000, 0, 0, 5), (3001, 37, 1, 0)])
+@pytest.mark.parametrize("c_in,c_out", [(64, 64), (48, 32)])
+def test_three_kind_form_on_clouds_with_chosen_neighbour_counts(mix, c_in, c_out):
+    """The three kinds of workgroup one at a time and together: clouds made of isolated voxels, pairs, lines of three
+    and a filled blob, so that the sections of the order (no neighbour / one / two / three or more) are empty, tiny or
+    ragged at will; the counts against their construction, the layer against the oracle."""
+    singles, dimers, trimers, blob = mix
+    coords = _molecules(*mix, seed=sum(mix))
+    n = len(coords)
+    assert n == singles + 2 * dimers + 3 * trimers + blob ** 3
+    ref, masks = _oracle_masks(coords)
+    pc = _popcount(masks)
+    km = _subm(coords)
+    assert km.order_single == 2 * dimers + 2 * trimers == int((pc == 1).sum())
+    assert km.order_nonzero - km.order_single - km.order_heavy == trimers == int((pc == 2).sum())
+    assert km.order_heavy == blob ** 3 == int((pc >= 3).sum())
+    assert 2 * km.order_nonzero <= n and 8 * (km.order_nonzero - km.order_single) <= n        # the three-kind form takes it
+    dt = torch.float16
+    f, w = synth.features(c_in, n, c_in), synth.weights(c_out, 27, c_in, c_out)
+    fd, wd = torch.as_tensor(f, device=DEV).to(dt), torch.as_tensor(w, device=DEV).to(dt)
+    out = backend.conv_forward(fd, wd, km, DATAFLOW_OSO, packed=backend.pack_weights(wd))
+    want = orc.conv_forward(rounded(f, dt), rounded(w, dt), ref, K3)
+    assert orc.rel_l2(out.double().cpu().numpy(), want) <= 1e-3
+    # row by row: no row of any section is left unwritten or written by the wrong kind
+    err = np.abs(out.double().cpu().numpy() - want).max(1)
+    assert err.max() <= 2e-2, (int(err.argmax()), int(pc[err.argmax()]))
