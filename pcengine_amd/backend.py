@@ -34,9 +34,14 @@ def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else t.data_ptr()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(device) -> int:
     if _arena is not None and _arena.stream_device == device:      # inside allocate_from: looked up once per forward
         return _arena.stream
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index)       # the handle of torch's current stream without a Stream object (4 us per layer)
     return torch.cuda.current_stream(device).cuda_stream
 
 
@@ -709,12 +714,19 @@ def row_order(km: KernelMap) -> torch.Tensor:
     return km.order
 
 
+_oso_takes_cache = {}
+
+
 def oso_takes(km: KernelMap, c_in: int, c_out: int, dtype: torch.dtype, transposed: bool = False) -> bool:
     """Layers the ordered output-stationary dataflow takes (``pce_conv_oso_takes``; never a transposed layer)."""
     if transposed or dtype not in (torch.float16, torch.float32):
         return False
-    code = PCE_F16 if dtype == torch.float16 else PCE_F32
-    return bool(_lib.load().pce_conv_oso_takes(code, c_in, c_out, km.kv, _mid(km.ks) if km.subm else -1))
+    key = (dtype, c_in, c_out, km.kv, km.subm, km.ks)
+    ans = _oso_takes_cache.get(key)
+    if ans is None:
+        code = PCE_F16 if dtype == torch.float16 else PCE_F32
+        ans = _oso_takes_cache[key] = bool(_lib.load().pce_conv_oso_takes(code, c_in, c_out, km.kv, _mid(km.ks) if km.subm else -1))
+    return ans
 
 
 def ensure_nbr(km: KernelMap, transposed: bool) -> None:
@@ -794,7 +806,8 @@ def _epilogue(feats: torch.Tensor, n_out: int, c_out: int, bias, residual, act, 
     e.ld_in, e.ld_out = ld_in, ld_out
     keep = []
     if bias is not None:
-        bias = bias.detach().to(device=feats.device, dtype=feats.dtype).contiguous()
+        if bias.requires_grad or bias.dtype != feats.dtype or bias.device != feats.device or not bias.is_contiguous():
+            bias = bias.detach().to(device=feats.device, dtype=feats.dtype).contiguous()
         if bias.numel() != c_out:
             raise ValueError(f"bias has {bias.numel()} elements, the layer has {c_out} output channels")
         e.bias = bias.data_ptr()
